@@ -1,0 +1,136 @@
+"""ctypes binding of libhs_attn.so: the same C ABI a Rust `-sys` crate would bind.
+
+This module is plumbing for tests, the smoke check and the benchmark: torch supplies device
+memory and the current stream, every call goes through the extern "C" entry points declared
+in include/hs_attn.h.  There is no fallback: if the shared library is missing the import of
+`lib()` raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhs_attn.so")
+
+HS_OK = 0
+HS_ERR_INVALID_ARGUMENT = 1
+HS_ERR_OVERFLOW = 2
+HS_ERR_WORKSPACE = 3
+HS_ERR_LAUNCH = 4
+HS_BF16, HS_F32, HS_F16 = 0, 1, 2
+
+EXPORTS = [
+    "hs_attn_last_error", "hs_attn_abi_version",
+    "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
+    "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8",
+]
+
+
+class KvLayout(ctypes.Structure):
+    """Mirror of `struct hs_kv_layout`."""
+    _fields_ = [
+        ("code_stride_seq", ctypes.c_int64),
+        ("code_stride_head", ctypes.c_int64),
+        ("scale_stride_seq", ctypes.c_int64),
+        ("scale_stride_head", ctypes.c_int64),
+        ("capacity_tokens", ctypes.c_int32),
+        ("block_table_stride", ctypes.c_int32),
+        ("k_block_table", ctypes.c_void_p),
+        ("v_block_table", ctypes.c_void_p),
+    ]
+
+
+class HsError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("hs_attn error %d: %s" % (code, msg))
+        self.code = code
+
+
+_lib = None
+
+
+def lib():
+    """Load libhs_attn.so (built by `python -m hyprstream_amd.build`); raises if absent."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError("libhs_attn.so not built: run `python -m hyprstream_amd.build` (%s)" % LIB_PATH)
+        L = ctypes.CDLL(LIB_PATH)
+        L.hs_attn_last_error.restype = ctypes.c_char_p
+        L.hs_decode_attn_workspace_bytes.restype = ctypes.c_size_t
+        L.hs_decode_attn_workspace_bytes.argtypes = [ctypes.c_int32] * 5
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != HS_OK:
+        raise HsError(rc, lib().hs_attn_last_error().decode())
+
+
+def contiguous_layout(Hkv, capacity_tokens, D, scale_pad=4):
+    """Head-major cache of one buffer per tensor: codes [B, Hkv, cap, D], scales [B, Hkv, cap_padded]."""
+    cap_s = (capacity_tokens + scale_pad - 1) // scale_pad * scale_pad
+    return KvLayout(Hkv * capacity_tokens * D, capacity_tokens * D, Hkv * cap_s, cap_s, capacity_tokens, 0, None, None)
+
+
+def paged_layout(Hkv, block_tokens, D, k_table, v_table):
+    """Pool of blocks [nblocks, Hkv, block_tokens, D]; tables are int32 device tensors [B, max_blocks]."""
+    assert k_table.dtype.is_signed and k_table.element_size() == 4 and k_table.is_contiguous()
+    return KvLayout(Hkv * block_tokens * D, block_tokens * D, Hkv * block_tokens, block_tokens, block_tokens,
+                    k_table.shape[1], k_table.data_ptr(), v_table.data_ptr())
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr() if t is not None else None)
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dtype_code(t):
+    import torch
+    return {torch.bfloat16: HS_BF16, torch.float32: HS_F32, torch.float16: HS_F16}[t.dtype]
+
+
+def kv_quantize_int8(k_src, v_src, k_codes, v_codes, k_scales, v_scales, layout, positions=None, start_pos=0):
+    B, S, Hkv, D = k_src.shape
+    assert k_src.is_contiguous() and v_src.is_contiguous()
+    check(lib().hs_kv_quantize_int8(_ptr(k_src), _ptr(v_src), _dtype_code(k_src), _ptr(k_codes), _ptr(v_codes),
+                                    _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout), _ptr(positions),
+                                    ctypes.c_int32(start_pos), B, S, Hkv, D, _stream()))
+
+
+def kv_fp8_calibrate(k_src, v_src, k_scales, v_scales):
+    B, S, Hkv, D = k_src.shape
+    check(lib().hs_kv_fp8_calibrate(_ptr(k_src), _ptr(v_src), _dtype_code(k_src), _ptr(k_scales), _ptr(v_scales),
+                                    B, S, Hkv, D, _stream()))
+
+
+def kv_quantize_fp8(k_src, v_src, k_codes, v_codes, k_scales, v_scales, layout, positions=None, start_pos=0):
+    B, S, Hkv, D = k_src.shape
+    assert k_src.is_contiguous() and v_src.is_contiguous()
+    check(lib().hs_kv_quantize_fp8(_ptr(k_src), _ptr(v_src), _dtype_code(k_src), _ptr(k_codes), _ptr(v_codes),
+                                   _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout), _ptr(positions),
+                                   ctypes.c_int32(start_pos), B, S, Hkv, D, _stream()))
+
+
+def kv_dequantize(codes, scales, fp8, layout, which_table, out):
+    B, T, Hkv, D = out.shape
+    check(lib().hs_kv_dequantize(_ptr(codes), _ptr(scales), int(fp8), ctypes.byref(layout), int(which_table),
+                                 _ptr(out), _dtype_code(out), B, T, Hkv, D, _stream()))
+
+
+def decode_workspace_bytes(B, Hq, Hkv, D, max_seq_len):
+    return lib().hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, max_seq_len)
+
+
+def decode_attn(q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace, Hkv, max_seq_len,
+                softmax_scale, fp8=False):
+    B, Hq, D = q.shape
+    fn = lib().hs_decode_attn_fp8 if fp8 else lib().hs_decode_attn_int8
+    check(fn(_ptr(q), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout),
+             _ptr(seq_lens), _ptr(out), _ptr(workspace),
+             ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0),
+             B, Hq, Hkv, D, ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))

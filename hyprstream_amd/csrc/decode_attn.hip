@@ -1,0 +1,428 @@
+// Dequant-fused GQA decode attention over the int8 / FP8-e4m3fn KV cache (gfx950, wave64).
+//
+// Split-K flash decoding.  Grid = (chunks, kv-heads, sequences); one 256-thread workgroup owns
+// one chunk of `chunk_tokens` cached tokens of one (sequence, kv-head) and all G = Hq/Hkv query
+// heads that read it, so every K/V byte is fetched from HBM exactly once.  Each of the four
+// wavefronts walks its own 32-token steps of the chunk with a private online-softmax state;
+// the next step's K/V/scales are already in flight (register double buffer) while the current
+// one is consumed.  The wavefronts' (m, l, o) are merged through LDS, the chunk partial goes to
+// the workspace, and a second small kernel merges the chunks.
+//
+// Arithmetic.  Both products run on the MFMA pipe (v_mfma_f32_16x16x32_f16) with the G query
+// heads on the N axis (padded to 16):
+//   S[t, g]  = sum_d K[t, d] Q[g, d]          A = K codes, 16 tokens x 32 d per issue
+//   O[d, g] += sum_t V^T[d, t] P[t, g]        A = V codes transposed in registers, B = P
+// int8 codes enter the MFMA as EXACT fp16 integers: byte b -> fp16 bits 0x6400 | (b ^ 0x80)
+// = 1152 + code.  For K the 1152 offset is cancelled by seeding the accumulator with
+// -1152 * sum_d Q[g, d]; for V it is subtracted with one packed fp16 add (exact).  Q (bf16) is
+// scaled per head by a power of two into fp16 range (exact) and the power is folded back into
+// the softmax scale.  Scores, softmax and all accumulation are fp32; the per-token K scale is
+// applied to the fp32 score, the per-token V scale is folded into P before P is rounded to fp16.
+// The score accumulator layout (lane = head + 16*q, register r -> token 4q + r) is exactly the
+// B-operand layout of the second product, so P never crosses lanes; the only cross-lane traffic
+// is the running max (two butterfly steps over the lanes that share a head).
+//
+// HBM bytes per cached token and kv-head: 2*D codes + 8 B of scales (int8) -- 264 B at D = 128.
+#include "common.hpp"
+
+namespace hs {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kD = 128;          // head_dim served by this kernel
+constexpr int kStep = 32;        // tokens per wavefront step
+constexpr int kWavesPerWg = 4;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kPScale = 64.0f;  // P is carried as 64*p*s_v in fp16 (keeps small weights normal)
+
+struct DecodeArgs {
+    const uint16_t *q;   // [B, Hq, D] bf16
+    const uint8_t *kc, *vc;
+    const float *ks, *vs;
+    KvAddr ka, va;
+    const int32_t *seq_lens;
+    float *part_o;   // [B, Hq, nchunks, D]
+    float *part_ml;  // [B, Hq, nchunks, 2]   (m in log2 units, l)
+    int32_t B, Hq, Hkv, G, chunk_tokens, nchunks, max_seq_len;
+    float scale_log2e;
+};
+
+template <bool FP8>
+struct Stage {
+    u32x4 k[2][2];  // [16-token tile][16-byte half of this lane's 32 B of the row]
+    u32x2 v[8];     // [token slot e = 4u + r] 8 bytes: d = 8*(lane%16) .. +7
+    float4v sk[2];  // K scales of tokens 16u + 4q + r   (int8 only)
+    float4v sv[2];
+};
+
+__device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    u32x4 t = {a, b, c, d};
+    return __builtin_bit_cast(half8, t);
+}
+
+// Two bytes (in the high byte of each 16-bit half of t) holding e4m3fn codes -> two fp16 whose
+// value is code_value * 2^-8 (exponent bias 15 instead of 7; the factor is folded into the scale).
+__device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t t) {
+    return (t & 0x80008000u) | ((t >> 1) & 0x3f803f80u);
+}
+
+template <bool FP8>
+__global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
+    const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int L = min(a.seq_lens[b], a.max_seq_len);
+    const int t_begin = chunk * a.chunk_tokens;
+    if (t_begin >= L) return;
+    const int t_end = min(L, t_begin + a.chunk_tokens);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int li = lane & 15, lq = lane >> 4;
+    const int G = a.G;
+
+    // ---- Q operand: lane (head li, quarter lq) holds Q[head][32*lq + 8*j + e] for MFMA j.
+    half8 qop[4];
+    float cq = 0.0f, cinit = 0.0f;
+    {
+        float qf[32];
+        float amax = 0.0f;
+        if (li < G) {
+            const uint16_t *qp = a.q + ((int64_t)b * a.Hq + h * G + li) * kD + 32 * lq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                u32x4 w = *(const u32x4 *)(qp + 8 * i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16);
+                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) qf[i] = 0.0f;
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        int ex = 0;
+        if (amax > 0.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
+        float qsum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                _Float16 hq = (_Float16)ldexpf(qf[8 * j + e], -ex);
+                qop[j][e] = hq;
+                qsum += (float)hq;
+            }
+        }
+        qsum += __shfl_xor(qsum, 16, 64);
+        qsum += __shfl_xor(qsum, 32, 64);
+        if (li < G) {
+            cq = ldexpf(a.scale_log2e, ex);
+            if (FP8) {
+                cq *= 256.0f * a.ks[(int64_t)b * a.Hkv + h];  // 2^8 rebias of the fp16 view of e4m3
+            } else {
+                cinit = -1152.0f * qsum;
+            }
+        }
+    }
+    // fp8: the V scale is one constant per (sequence, head); it multiplies the finished partial.
+    const float out_scale = (1.0f / kPScale) * (FP8 ? 256.0f * a.vs[(int64_t)b * a.Hkv + h] : 1.0f);
+
+    float4v acc[8];  // O[d = 32*lq + 8*r + bb][head li] in acc[bb][r]
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;
+
+    const int nsteps = (t_end - t_begin + kStep - 1) / kStep;
+
+    auto load_stage = [&](Stage<FP8> &st, int step) {
+        const int t0 = t_begin + step * kStep;
+        int64_t ku, vu;
+        int kslot, vslot;
+        resolve(a.ka, b, t0, ku, kslot);
+        resolve(a.va, b, t0, vu, vslot);
+        const int last = L - 1 - t0;  // last valid row offset inside this step (>= 0)
+        const uint8_t *kb = a.kc + ku * a.ka.code_stride_seq + (int64_t)h * a.ka.code_stride_head + (int64_t)kslot * kD;
+        const uint8_t *vb = a.vc + vu * a.va.code_stride_seq + (int64_t)h * a.va.code_stride_head + (int64_t)vslot * kD;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int row = min(16 * u + li, last);
+            const uint8_t *p = kb + row * kD + 32 * lq;
+            st.k[u][0] = *(const u32x4 *)p;
+            st.k[u][1] = *(const u32x4 *)(p + 16);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = min(16 * u + 4 * lq + r, last);
+                st.v[4 * u + r] = *(const u32x2 *)(vb + row * kD + 8 * li);
+            }
+        if (!FP8) {
+            const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)h * a.ka.scale_stride_head + kslot;
+            const float *vsb = a.vs + vu * a.va.scale_stride_seq + (int64_t)h * a.va.scale_stride_head + vslot;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const int tok = min(16 * u + 4 * lq, last & ~3);
+                st.sk[u] = *(const float4v *)(ksb + tok);
+                st.sv[u] = *(const float4v *)(vsb + tok);
+            }
+        }
+    };
+
+    auto compute_stage = [&](const Stage<FP8> &st, int step) {
+        const int t0 = t_begin + step * kStep;
+        // ---- scores: 2 tiles x 4 MFMAs (K of 128 split in 4 x 32)
+        float4v s[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            s[u] = (float4v){cinit, cinit, cinit, cinit};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t w0 = st.k[u][j >> 1][2 * (j & 1)], w1 = st.k[u][j >> 1][2 * (j & 1) + 1];
+                half8 ak;
+                if (FP8) {
+                    ak = as_half8(fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, w0, 0x010c000cu)),
+                                  fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, w0, 0x030c020cu)),
+                                  fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, w1, 0x010c000cu)),
+                                  fp8x2_to_f16x2(__builtin_amdgcn_perm(0u, w1, 0x030c020cu)));
+                } else {
+                    const uint32_t x0 = w0 ^ 0x80808080u, x1 = w1 ^ 0x80808080u;
+                    ak = as_half8(__builtin_amdgcn_perm(0x64646464u, x0, 0x04010400u),
+                                  __builtin_amdgcn_perm(0x64646464u, x0, 0x04030402u),
+                                  __builtin_amdgcn_perm(0x64646464u, x1, 0x04010400u),
+                                  __builtin_amdgcn_perm(0x64646464u, x1, 0x04030402u));
+                }
+                s[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak, qop[j], s[u], 0, 0, 0);
+            }
+        }
+        // ---- scale to log2 units, mask the tail
+        float sc[8], pv[8];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                sc[4 * u + r] = FP8 ? s[u][r] * cq : s[u][r] * st.sk[u][r] * cq;
+                pv[4 * u + r] = FP8 ? kPScale : st.sv[u][r] * kPScale;
+            }
+        const bool tail = t0 + kStep > L;
+        if (tail) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (t0 + 16 * u + 4 * lq + r >= L) {
+                        sc[4 * u + r] = -INFINITY;
+                        pv[4 * u + r] = 0.0f;
+                    }
+        }
+        // ---- online softmax (max shared by the 4 lanes of a head)
+        float mx = sc[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sc[i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+            m_run = m_new;
+        }
+        uint32_t pb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float p0 = __builtin_amdgcn_exp2f(sc[2 * i] - m_run);
+            const float p1 = __builtin_amdgcn_exp2f(sc[2 * i + 1] - m_run);
+            l_run += p0 + p1;
+            half2v hp = {(_Float16)(p0 * pv[2 * i]), (_Float16)(p1 * pv[2 * i + 1])};
+            pb[i] = __builtin_bit_cast(uint32_t, hp);
+        }
+        const half8 pop = as_half8(pb[0], pb[1], pb[2], pb[3]);
+        // ---- O += V^T P : 8 MFMAs, one per byte column bb of this lane's 8 d's
+#pragma unroll
+        for (int bb = 0; bb < 8; ++bb) {
+            uint32_t av[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const uint32_t lo = st.v[2 * p][bb >> 2], hi = st.v[2 * p + 1][bb >> 2];
+                if (FP8) {
+                    const uint32_t sel = 0x040c000cu + ((uint32_t)(bb & 3) << 8) + ((uint32_t)(bb & 3) << 24);
+                    av[p] = fp8x2_to_f16x2(__builtin_amdgcn_perm(hi, lo, sel));
+                } else {
+                    const uint32_t sel = 0x0c040c00u + (uint32_t)(bb & 3) + ((uint32_t)(bb & 3) << 16);
+                    const uint32_t w = __builtin_amdgcn_perm(hi, lo, sel) ^ 0x64806480u;
+                    half2v hv = __builtin_bit_cast(half2v, w) - (half2v){(_Float16)1152.0f, (_Float16)1152.0f};
+                    av[p] = __builtin_bit_cast(uint32_t, hv);
+                }
+            }
+            acc[bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av[0], av[1], av[2], av[3]), pop, acc[bb], 0, 0, 0);
+        }
+    };
+
+    // ---- software pipeline over this wavefront's steps (wave, wave+4, ...)
+    Stage<FP8> sa, sb;
+    int step = wave;
+    if (step < nsteps) load_stage(sa, step);
+    while (step < nsteps) {
+        const int n1 = step + kWavesPerWg;
+        if (n1 < nsteps) load_stage(sb, n1);
+        compute_stage(sa, step);
+        if (n1 >= nsteps) break;
+        const int n2 = n1 + kWavesPerWg;
+        if (n2 < nsteps) load_stage(sa, n2);
+        compute_stage(sb, n1);
+        step = n2;
+    }
+
+    // ---- merge the four wavefronts through LDS
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    __shared__ float sm_m[kWavesPerWg][16], sm_l[kWavesPerWg][16];
+    __shared__ float sm_o[kWavesPerWg][16][kD + 4];
+    if (lq == 0) {
+        sm_m[wave][li] = m_run;
+        sm_l[wave][li] = l_run;
+    }
+    __syncthreads();
+    float M = sm_m[0][li];
+#pragma unroll
+    for (int w = 1; w < kWavesPerWg; ++w) M = fmaxf(M, sm_m[w][li]);
+    const float f = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - M);
+    if (li < G) {
+#pragma unroll
+        for (int bb = 0; bb < 8; ++bb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sm_o[wave][li][32 * lq + 8 * r + bb] = acc[bb][r] * f;
+    }
+    __syncthreads();
+    const int64_t prow = ((int64_t)b * a.Hq + h * G) * a.nchunks + chunk;
+    for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
+        const int g = idx / kD, d = idx % kD;
+        float o = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWavesPerWg; ++w) o += sm_o[w][g][d];
+        a.part_o[(prow + (int64_t)g * a.nchunks) * kD + d] = o * out_scale;
+    }
+    if (threadIdx.x < G) {
+        const int g = threadIdx.x;
+        float Mg = sm_m[0][g];
+        for (int w = 1; w < kWavesPerWg; ++w) Mg = fmaxf(Mg, sm_m[w][g]);
+        float l = 0.0f;
+        for (int w = 0; w < kWavesPerWg; ++w)
+            l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
+        float *ml = a.part_ml + (prow + (int64_t)g * a.nchunks) * 2;
+        ml[0] = Mg;
+        ml[1] = l;
+    }
+}
+
+// Merge the chunk partials of one (sequence, query head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c.
+__global__ __launch_bounds__(128) void decode_merge_kernel(const float *part_o, const float *part_ml,
+                                                          const int32_t *seq_lens, uint16_t *out, int Hq, int nchunks,
+                                                          int chunk_tokens, int max_seq_len) {
+    const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    const int L = min(seq_lens[b], max_seq_len);
+    const int n = L <= 0 ? 0 : min(nchunks, (L + chunk_tokens - 1) / chunk_tokens);
+    const int64_t row = ((int64_t)b * Hq + hq) * nchunks;
+    float M = -INFINITY;
+    for (int c = 0; c < n; ++c) M = fmaxf(M, part_ml[(row + c) * 2]);
+    float o = 0.0f, l = 0.0f;
+    for (int c = 0; c < n; ++c) {
+        const float w = __builtin_amdgcn_exp2f(part_ml[(row + c) * 2] - M);
+        l += w * part_ml[(row + c) * 2 + 1];
+        o += w * part_o[(row + c) * kD + d];
+    }
+    out[((int64_t)b * Hq + hq) * kD + d] = (uint16_t)f32_to_bf16_bits(n > 0 ? o / l : 0.0f);
+}
+
+int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
+
+static int pick_chunk_tokens(int B, int Hkv, int max_seq_len) {
+    // Aim at >= 4 workgroups per CU over 256 CUs, chunks a multiple of 128 tokens (4 waves x 32).
+    const int64_t units = (int64_t)B * Hkv;
+    int64_t want_chunks = (1024 + units - 1) / units;
+    if (want_chunks < 1) want_chunks = 1;
+    int64_t ct = ((int64_t)max_seq_len + want_chunks - 1) / want_chunks;
+    ct = (ct + 127) / 128 * 128;
+    if (ct < 256) ct = 256;
+    return (int)ct;
+}
+
+static int launch_decode(bool fp8, const void *q, const void *kc, const void *vc, const float *ks, const float *vs,
+                         const hs_kv_layout *l, const int32_t *seq_lens, void *out, void *ws, size_t ws_bytes, int B,
+                         int Hq, int Hkv, int D, int max_seq_len, float softmax_scale, hipStream_t stream) {
+    if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
+    if (D != kD) return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 128, got %d", D);
+    if (!q || !kc || !vc || !ks || !vs || !seq_lens || !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (Hq <= 0 || Hq % Hkv != 0 || Hq / Hkv > 16)
+        return fail(HS_ERR_INVALID_ARGUMENT, "need Hq %% Hkv == 0 and Hq/Hkv <= 16 (Hq=%d Hkv=%d)", Hq, Hkv);
+    if (max_seq_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "max_seq_len must be positive");
+    if (l->k_block_table && (l->capacity_tokens % kStep) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of %d tokens", kStep);
+    if (B == 0) return HS_OK;
+    {
+        const int64_t cap = l->k_block_table ? (int64_t)l->capacity_tokens * l->block_table_stride : l->capacity_tokens;
+        if (max_seq_len > cap)
+            return fail(HS_ERR_OVERFLOW, "max_seq_len %d exceeds what the cache can hold (%lld tokens)", max_seq_len,
+                        (long long)cap);
+    }
+    const size_t need = hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, max_seq_len);
+    if (!ws || ws_bytes < need)
+        return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+    if (((uintptr_t)ws & 255) != 0) return fail(HS_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+    DecodeArgs a;
+    a.q = (const uint16_t *)q;
+    a.kc = (const uint8_t *)kc; a.vc = (const uint8_t *)vc;
+    a.ks = ks; a.vs = vs;
+    a.ka = make_addr(*l, 0); a.va = make_addr(*l, 1);
+    a.seq_lens = seq_lens;
+    a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv; a.max_seq_len = max_seq_len;
+    a.chunk_tokens = pick_chunk_tokens(B, Hkv, max_seq_len);
+    a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
+    a.part_o = (float *)ws;
+    a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * kD;
+    a.scale_log2e = softmax_scale * kLog2e;
+    dim3 grid(a.nchunks, Hkv, B);
+    if (fp8) decode_attn_kernel<true><<<grid, 256, 0, stream>>>(a);
+    else decode_attn_kernel<false><<<grid, 256, 0, stream>>>(a);
+    if (int rc = check_launch("decode_attn")) return rc;
+    decode_merge_kernel<<<dim3(Hq, B), 128, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq, a.nchunks,
+                                                         a.chunk_tokens, max_seq_len);
+    return check_launch("decode_merge");
+}
+
+}  // namespace hs
+
+extern "C" {
+
+size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || max_seq_len <= 0) return 0;
+    const int ct = hs::pick_chunk_tokens(B, Hkv, max_seq_len);
+    const size_t nchunks = (size_t)((max_seq_len + ct - 1) / ct);
+    const size_t n = (size_t)B * Hq * nchunks * ((size_t)D + 2) * sizeof(float);
+    return (n + 255) / 256 * 256;
+}
+
+int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes, const float *k_scales,
+                        const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                        void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
+                        int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
+    return hs::launch_decode(false, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+                             workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8_t *v_codes, const float *k_scales,
+                       const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                       void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
+                       int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
+    return hs::launch_decode(true, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+                             workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,287 @@
+// Quantize-on-write and dense-view kernels for the int8 / FP8-e4m3fn KV cache (gfx950).
+//
+// One 64-lane wavefront owns one (sequence, token, kv-head) row of head_dim elements,
+// E = D/64 consecutive elements per lane: the absmax is a wavefront max-reduction, the
+// row's codes leave as one coalesced store, the scale as a single dword.  HBM traffic is
+// read 2 or 4 B + write 1 B per element (+4 B per row); only the S new tokens are touched.
+//
+// Arithmetic is written to be bit-identical to the CPU oracle: IEEE fp32 division
+// (-fhip-fp32-correctly-rounded-divide-sqrt), round-half-even (v_rndne_f32), no fast-math.
+#include "common.hpp"
+
+namespace hs {
+
+struct QuantArgs {
+    const void *src[2];   // K, V  [B, S, Hkv, D]
+    void *codes[2];
+    float *scales[2];     // int8: written; fp8: read ([B, Hkv])
+    KvAddr addr[2];
+    const int32_t *positions;
+    int32_t start_pos, B, S, Hkv, D, dtype;
+};
+
+__device__ __forceinline__ uint32_t f32_to_e4m3fn_bits(float y) {
+    uint32_t u = __float_as_uint(y);
+    uint32_t sign = (u >> 24) & 0x80u;
+    u &= 0x7fffffffu;
+    if (u >= 0x43f00000u) return sign | 0x7fu;  // >= 480, inf, NaN
+    float a = __uint_as_float(u);
+    uint32_t r;
+    if (a < 0.015625f) {
+        r = (uint32_t)rintf(a * 512.0f);  // subnormal grid 2^-9; 8 == smallest normal
+    } else {
+        r = (u + 0x7ffffu + ((u >> 20) & 1u)) >> 20;  // RNE on the 3 kept mantissa bits
+        r -= (120u << 3);                              // rebias 127 -> 7
+        if (r > 0x7fu) r = 0x7fu;
+    }
+    return sign | r;
+}
+
+template <int E, bool FP8>
+__global__ __launch_bounds__(256) void kv_quantize_kernel(QuantArgs a) {
+    const int which = blockIdx.y;  // 0 = K, 1 = V
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t rows = (int64_t)a.B * a.S * a.Hkv;
+    if (row >= rows) return;
+    const int h = (int)(row % a.Hkv);
+    const int64_t bs = row / a.Hkv;
+    const int s = (int)(bs % a.S);
+    const int b = (int)(bs / a.S);
+    const int pos = (a.positions ? a.positions[b] : a.start_pos) + s;
+    const KvAddr &ad = a.addr[which];
+    int64_t unit;
+    int slot;
+    if (!resolve(ad, b, pos, unit, slot)) return;
+
+    float x[E];
+    load_src<E>(a.src[which], a.dtype, row * a.D + lane * E, x);
+
+    uint8_t *dst = (uint8_t *)a.codes[which] + unit * ad.code_stride_seq + (int64_t)h * ad.code_stride_head +
+                   (int64_t)slot * a.D + lane * E;
+    uint32_t packed = 0;
+    if (!FP8) {
+        float m = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float v = fabsf(x[e]);
+            m = v > m ? v : m;
+        }
+        m = wave_max(m);
+        float sc = 0.0f;
+        if (m > 0.0f) {
+            sc = m / 127.0f;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float q = rintf(x[e] / sc);
+                q = q > 127.0f ? 127.0f : q;
+                q = q < -127.0f ? -127.0f : q;
+                if (q != q) q = 0.0f;
+                packed |= ((uint32_t)(int)q & 0xffu) << (8 * e);
+            }
+        }
+        if (lane == 0) a.scales[which][unit * ad.scale_stride_seq + (int64_t)h * ad.scale_stride_head + slot] = sc;
+    } else {
+        const float sc = a.scales[which][(int64_t)b * a.Hkv + h];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float y = 0.0f;
+            if (sc > 0.0f) {
+                y = x[e] / sc;
+                if (y > 448.0f) y = 448.0f;
+                if (y < -448.0f) y = -448.0f;
+            }
+            packed |= f32_to_e4m3fn_bits(y) << (8 * e);
+        }
+    }
+    if (E == 4) *(uint32_t *)dst = packed;
+    else if (E == 2) *(uint16_t *)dst = (uint16_t)packed;
+    else *dst = (uint8_t)packed;
+}
+
+// scale[b, h] = max_{s, d} |x| / 448.  One workgroup per (b, h, tensor).
+__global__ __launch_bounds__(256) void fp8_calibrate_kernel(const void *k_src, const void *v_src, int dtype,
+                                                           float *k_scales, float *v_scales, int B, int S, int Hkv,
+                                                           int D) {
+    const int which = blockIdx.y;
+    const int b = blockIdx.x / Hkv, h = blockIdx.x % Hkv;
+    const void *src = which ? v_src : k_src;
+    float m = 0.0f;
+    const int per_row = D;
+    for (int64_t i = threadIdx.x; i < (int64_t)S * per_row; i += 256) {
+        int s = (int)(i / per_row), d = (int)(i % per_row);
+        float x[1];
+        load_src<1>(src, dtype, (((int64_t)b * S + s) * Hkv + h) * D + d, x);
+        float v = fabsf(x[0]);
+        m = v > m ? v : m;
+    }
+    m = wave_max(m);
+    __shared__ float red[4];
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        (which ? v_scales : k_scales)[b * Hkv + h] = m / 448.0f;
+    }
+}
+
+__device__ __forceinline__ float e4m3fn_bits_to_f32(uint32_t c) {
+    uint32_t e = (c >> 3) & 0xfu, m = c & 7u;
+    float v;
+    if (e == 0) v = (float)m * 0.001953125f;  // m * 2^-9
+    else if (e == 15 && m == 7) v = __uint_as_float(0x7fc00000u);
+    else v = __uint_as_float(((e + 120u) << 23) | (m << 20));
+    return (c & 0x80u) ? -v : v;
+}
+
+struct DequantArgs {
+    const void *codes;
+    const float *scales;
+    KvAddr addr;
+    void *out;
+    int32_t B, T, Hkv, D, out_dtype, fp8;
+};
+
+template <int E>
+__global__ __launch_bounds__(256) void kv_dequantize_kernel(DequantArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (int64_t)a.B * a.T * a.Hkv) return;
+    const int h = (int)(row % a.Hkv);
+    const int64_t bt = row / a.Hkv;
+    const int t = (int)(bt % a.T);
+    const int b = (int)(bt / a.T);
+    int64_t unit;
+    int slot;
+    float v[E];
+    if (resolve(a.addr, b, t, unit, slot)) {
+        const uint8_t *src = (const uint8_t *)a.codes + unit * a.addr.code_stride_seq +
+                             (int64_t)h * a.addr.code_stride_head + (int64_t)slot * a.D + lane * E;
+        float sc = a.fp8 ? a.scales[(int64_t)b * a.Hkv + h]
+                         : a.scales[unit * a.addr.scale_stride_seq + (int64_t)h * a.addr.scale_stride_head + slot];
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            v[e] = sc * (a.fp8 ? e4m3fn_bits_to_f32(src[e]) : (float)(int8_t)src[e]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[e] = 0.0f;
+    }
+    const int64_t o = row * a.D + lane * E;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        if (a.out_dtype == HS_F32) ((float *)a.out)[o + e] = v[e];
+        else if (a.out_dtype == HS_BF16) ((uint16_t *)a.out)[o + e] = (uint16_t)f32_to_bf16_bits(v[e]);
+        else {
+            _Float16 f = (_Float16)v[e];
+            __builtin_memcpy((uint16_t *)a.out + o + e, &f, 2);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host launchers
+
+static int check_common(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales) {
+    if (!l) return fail(HS_ERR_INVALID_ARGUMENT, "layout is NULL");
+    if (B < 0 || S < 0 || Hkv <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d Hkv=%d", B, S, Hkv);
+    if (D != 64 && D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "head_dim %d not in {64,128,256}", D);
+    if (l->capacity_tokens <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "capacity_tokens must be positive");
+    if (l->code_stride_head < (int64_t)l->capacity_tokens * D || (l->code_stride_head & 15))
+        return fail(HS_ERR_INVALID_ARGUMENT, "code_stride_head %lld too small or not a multiple of 16",
+                    (long long)l->code_stride_head);
+    if (need_scales && (l->scale_stride_head < l->capacity_tokens || (l->scale_stride_head & 3) ||
+                        (l->scale_stride_seq & 3) || (l->code_stride_seq & 15)))
+        return fail(HS_ERR_INVALID_ARGUMENT, "scale_stride_head %lld too small or not a multiple of 4",
+                    (long long)l->scale_stride_head);
+    if ((l->k_block_table == nullptr) != (l->v_block_table == nullptr))
+        return fail(HS_ERR_INVALID_ARGUMENT, "give both block tables or neither");
+    if (l->k_block_table && l->block_table_stride <= 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "block_table_stride must be positive when paged");
+    return HS_OK;
+}
+
+int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales) {
+    return check_common(l, B, S, Hkv, D, need_scales);
+}
+
+template <bool FP8>
+static int launch_quantize(const void *k_src, const void *v_src, int dtype, void *kc, void *vc, float *ks, float *vs,
+                           const hs_kv_layout *l, const int32_t *positions, int start_pos, int B, int S, int Hkv,
+                           int D, hipStream_t stream) {
+    if (int rc = check_common(l, B, S, Hkv, D, !FP8)) return rc;
+    if (!k_src || !v_src || !kc || !vc || !ks || !vs) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16)
+        return fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", dtype);
+    if (!positions) {
+        if (start_pos < 0) return fail(HS_ERR_INVALID_ARGUMENT, "negative start_pos");
+        int64_t cap = l->k_block_table ? (int64_t)l->capacity_tokens * l->block_table_stride : l->capacity_tokens;
+        if ((int64_t)start_pos + S > cap)
+            return fail(HS_ERR_OVERFLOW,
+                        "Cache overflow: trying to cache %d tokens starting at position %d, but capacity is %lld", S,
+                        start_pos, (long long)cap);
+    }
+    const int64_t rows = (int64_t)B * S * Hkv;
+    if (rows == 0) return HS_OK;
+    QuantArgs a;
+    a.src[0] = k_src; a.src[1] = v_src;
+    a.codes[0] = kc; a.codes[1] = vc;
+    a.scales[0] = ks; a.scales[1] = vs;
+    a.addr[0] = make_addr(*l, 0); a.addr[1] = make_addr(*l, 1);
+    a.positions = positions; a.start_pos = start_pos;
+    a.B = B; a.S = S; a.Hkv = Hkv; a.D = D; a.dtype = dtype;
+    dim3 grid((unsigned)((rows + 3) / 4), 2);
+    if (D == 64) kv_quantize_kernel<1, FP8><<<grid, 256, 0, stream>>>(a);
+    else if (D == 128) kv_quantize_kernel<2, FP8><<<grid, 256, 0, stream>>>(a);
+    else kv_quantize_kernel<4, FP8><<<grid, 256, 0, stream>>>(a);
+    return check_launch(FP8 ? "kv_quantize_fp8" : "kv_quantize_int8");
+}
+
+}  // namespace hs
+
+extern "C" {
+
+int hs_kv_quantize_int8(const void *k_src, const void *v_src, int src_dtype, int8_t *k_codes, int8_t *v_codes,
+                        float *k_scales, float *v_scales, const hs_kv_layout *layout, const int32_t *positions,
+                        int32_t start_pos, int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream) {
+    return hs::launch_quantize<false>(k_src, v_src, src_dtype, k_codes, v_codes, k_scales, v_scales, layout, positions,
+                                      start_pos, B, S, Hkv, D, (hipStream_t)stream);
+}
+
+int hs_kv_quantize_fp8(const void *k_src, const void *v_src, int src_dtype, uint8_t *k_codes, uint8_t *v_codes,
+                       const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                       const int32_t *positions, int32_t start_pos, int32_t B, int32_t S, int32_t Hkv, int32_t D,
+                       hs_stream_t stream) {
+    return hs::launch_quantize<true>(k_src, v_src, src_dtype, k_codes, v_codes, (float *)k_scales, (float *)v_scales,
+                                     layout, positions, start_pos, B, S, Hkv, D, (hipStream_t)stream);
+}
+
+int hs_kv_fp8_calibrate(const void *k_src, const void *v_src, int src_dtype, float *k_scales, float *v_scales,
+                        int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream) {
+    if (!k_src || !v_src || !k_scales || !v_scales) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (B <= 0 || S <= 0 || Hkv <= 0 || D <= 0)
+        return hs::fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d Hkv=%d D=%d", B, S, Hkv, D);
+    if (src_dtype != HS_BF16 && src_dtype != HS_F32 && src_dtype != HS_F16)
+        return hs::fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", src_dtype);
+    hs::fp8_calibrate_kernel<<<dim3(B * Hkv, 2), 256, 0, (hipStream_t)stream>>>(k_src, v_src, src_dtype, k_scales,
+                                                                               v_scales, B, S, Hkv, D);
+    return hs::check_launch("fp8_calibrate");
+}
+
+int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8, const hs_kv_layout *layout, int which_table,
+                     void *out, int out_dtype, int32_t B, int32_t T, int32_t Hkv, int32_t D, hs_stream_t stream) {
+    if (int rc = hs::validate_layout(layout, B, T, Hkv, D, !fmt_fp8)) return rc;
+    if (!codes || !scales || !out) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (out_dtype != HS_BF16 && out_dtype != HS_F32 && out_dtype != HS_F16)
+        return hs::fail(HS_ERR_INVALID_ARGUMENT, "unknown out_dtype %d", out_dtype);
+    const int64_t rows = (int64_t)B * T * Hkv;
+    if (rows == 0) return HS_OK;
+    hs::DequantArgs a;
+    a.codes = codes; a.scales = scales; a.addr = hs::make_addr(*layout, which_table ? 1 : 0);
+    a.out = out; a.B = B; a.T = T; a.Hkv = Hkv; a.D = D; a.out_dtype = out_dtype; a.fp8 = fmt_fp8 ? 1 : 0;
+    dim3 grid((unsigned)((rows + 3) / 4));
+    if (D == 64) hs::kv_dequantize_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    else if (D == 128) hs::kv_dequantize_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    else hs::kv_dequantize_kernel<4><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    return hs::check_launch("kv_dequantize");
+}
+
+}  // extern "C"

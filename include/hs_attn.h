@@ -1,0 +1,164 @@
+/*
+ * hs_attn.h -- C ABI of libhs_attn.so: hyprstream's attention hot path over a
+ * quantized KV cache, hand-written for AMD MI355X (gfx950).
+ *
+ * Shape of the interface.  It follows the reference's only native boundary,
+ * crates/bitsandbytes-sys (crates/bitsandbytes-sys/src/bindings.rs:15-334):
+ * extern "C", raw device pointers, integer sizes, a trailing stream handle
+ * (bindings.rs:13 `bnb_stream_t`), the CALLER allocates every buffer and the
+ * library keeps no pointer and no state between calls
+ * (crates/hyprstream/src/runtime/kv_cache.rs:797-865, 915-957).  Two deliberate
+ * differences from that precedent: every entry point returns an int status
+ * (0 = HS_OK) with the message available from hs_attn_last_error(), because
+ * the bitsandbytes symbols return void and cannot report a bad launch; and
+ * element counts that can exceed 2^31 are int64_t (bindings.rs uses c_int).
+ *
+ * Notation: B sequences, S new tokens in this call, T cached tokens,
+ * Hq query heads, Hkv key/value heads (Hq % Hkv == 0, q-head h reads kv-head
+ * h / (Hq/Hkv): architectures/llama.rs:847-872), D head_dim.
+ *
+ * Cache layout in device memory (buffers allocated by the caller):
+ *   codes   one byte per element, head-major inside a sequence:
+ *           code(b, h, t, d) at  codes + b*code_stride_seq + h*code_stride_head + t*D + d
+ *   int8 scales  fp32, one per (token, kv-head):
+ *           scale(b, h, t)   at  scales + b*scale_stride_seq + h*scale_stride_head + t
+ *   fp8 scales   fp32 [B, Hkv], one per (sequence, kv-head)
+ * With block tables (paged mode, the reference's BlockPool of fixed-size token
+ * blocks, kv_cache.rs:477-693) "b" above is replaced by the block id found at
+ * table[b*block_table_stride + t / capacity_tokens] and t by t % capacity_tokens.
+ * A dense [B, T, Hkv, D] tensor, as LayerKVCache::get returns it
+ * (kv_cache.rs:1499-1643), is produced on request by hs_kv_dequantize.
+ *
+ * Threading: every function is re-entrant; work is enqueued on `stream`
+ * (NULL = the default stream, which is what tch/libtorch uses) of the caller's
+ * current device and nothing synchronises with the host.
+ */
+#ifndef HS_ATTN_H
+#define HS_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HS_ATTN_ABI_VERSION 1
+
+typedef void *hs_stream_t; /* hipStream_t */
+
+#if defined(__GNUC__)
+#define HS_API __attribute__((visibility("default")))
+#else
+#define HS_API
+#endif
+
+enum hs_status {
+    HS_OK = 0,
+    HS_ERR_INVALID_ARGUMENT = 1, /* null pointer, bad shape, unsupported head_dim, misaligned stride */
+    HS_ERR_OVERFLOW = 2,         /* write past capacity_tokens (kv_cache.rs:1288-1294 "Cache overflow") */
+    HS_ERR_WORKSPACE = 3,        /* workspace too small */
+    HS_ERR_LAUNCH = 4            /* hipGetLastError() after the launch */
+};
+
+enum hs_dtype { HS_BF16 = 0, HS_F32 = 1, HS_F16 = 2 };
+
+typedef struct hs_kv_layout {
+    int64_t code_stride_seq;    /* bytes between sequences (or blocks when paged) */
+    int64_t code_stride_head;   /* bytes between kv-heads inside a sequence/block; >= capacity_tokens*D, multiple of 16 */
+    int64_t scale_stride_seq;   /* fp32 elements between sequences (or blocks); int8 format only */
+    int64_t scale_stride_head;  /* fp32 elements between kv-heads; >= capacity_tokens, multiple of 4 */
+    int32_t capacity_tokens;    /* tokens one sequence (or one block) can hold */
+    int32_t block_table_stride; /* entries per sequence in the block tables; 0 = not paged */
+    const int32_t *k_block_table; /* device, [B, block_table_stride]; NULL = not paged */
+    const int32_t *v_block_table; /* device, may equal k_block_table when K and V pools are separate buffers */
+} hs_kv_layout;
+
+/* Message of the last failing call on this thread ("" if none). */
+HS_API const char *hs_attn_last_error(void);
+HS_API int hs_attn_abi_version(void);
+
+/* ---- quantize-on-write (replaces the buffer + flush + requantize-everything scheme of
+ * LayerKVCache::update / flush_buffer, kv_cache.rs:1275-1432, 1204-1272, and the
+ * cquantize_blockwise_* calls at kv_cache.rs:823-840) ------------------------------------
+ * k_src, v_src: [B, S, Hkv, D] contiguous, dtype src_dtype (K already rotated: the cache
+ * holds post-RoPE keys, llama.rs:598-611).  Token s of sequence b goes to position
+ * (positions ? positions[b] : start_pos) + s.  `positions` is a device array of B ints.
+ * int8: per (token, kv-head) row  s = max|x| / 127 (fp32), code = clamp(rint(x / s), +-127),
+ * all-zero row -> s = 0, codes 0.  Only the S new tokens are touched.
+ * Errors: HS_ERR_OVERFLOW when positions == NULL and start_pos + S > capacity (not paged);
+ * rows whose device-side position falls outside the capacity/table are skipped. */
+HS_API int hs_kv_quantize_int8(const void *k_src, const void *v_src, int src_dtype,
+                        int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                        const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos,
+                        int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream);
+
+/* FP8 e4m3fn cache with one fp32 scale per (sequence, kv-head).  Calibration computes
+ * scale[b, h] = max over (s, d) |x| / 448 from the tokens given (typically the prompt);
+ * quantization stores e4m3fn(clamp(x / scale, +-448)), round-to-nearest-even. */
+HS_API int hs_kv_fp8_calibrate(const void *k_src, const void *v_src, int src_dtype,
+                        float *k_scales, float *v_scales,
+                        int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream);
+HS_API int hs_kv_quantize_fp8(const void *k_src, const void *v_src, int src_dtype,
+                       uint8_t *k_codes, uint8_t *v_codes, const float *k_scales, const float *v_scales,
+                       const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos,
+                       int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream);
+
+/* ---- dense view (what LayerKVCache::get materialises, kv_cache.rs:1517-1580; replaces
+ * cdequantize_blockwise_*, bindings.rs:47-75).  Not on the attention path: the attention
+ * kernels read codes directly.  out: [B, T, Hkv, D] in out_dtype; which_table 0 = K table,
+ * 1 = V table (paged only).  fmt_fp8 0: int8 codes + per-token scales; 1: e4m3fn + per-head. */
+HS_API int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8, const hs_kv_layout *layout,
+                     int which_table, void *out, int out_dtype,
+                     int32_t B, int32_t T, int32_t Hkv, int32_t D, hs_stream_t stream);
+
+/* ---- decode attention (replaces get() + GQA expand + compute_attention_masked for q_len == 1:
+ * llama.rs:605-636, 1023-1119; qwen3_5.rs:993-1053; ragged rows as in forward_batched,
+ * llama.rs:710-844, 2544-2572) ---------------------------------------------------------------
+ * q, out: [B, Hq, D] bf16.  seq_lens: device [B], cached tokens per sequence INCLUDING the
+ * one just written; rows with seq_len <= 0 produce zeros.  max_seq_len >= every seq_lens[b]
+ * (host-side bound used to size the grid).  out = softmax(q K^T * softmax_scale) V with
+ * fp32 accumulation, K/V dequantized on the fly.  workspace: device scratch of at least
+ * hs_decode_attn_workspace_bytes(...) bytes, 256-byte aligned, owned by the caller. */
+HS_API size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len);
+HS_API int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes,
+                        const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                        const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,
+                        int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                        float softmax_scale, hs_stream_t stream);
+HS_API int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8_t *v_codes,
+                       const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                       const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,
+                       int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                       float softmax_scale, hs_stream_t stream);
+
+/* ---- causal prefill over [int8 history] + [this call's bf16 K/V] (replaces update + get +
+ * compute_attention_masked for q_len > 1: llama.rs:1066-1112, mask rule "query row i sits at
+ * absolute position (k_len - q_len) + i", llama.rs:1074-1084) --------------------------------
+ * q: [B, S, Hq, D] bf16; k_new, v_new: [B, S, Hkv, D] bf16; out: [B, S, Hq, D] bf16.
+ * hist_len tokens per sequence are already in the int8 cache; query row i attends the whole
+ * history (dequantized) and new tokens 0..=i (exact bf16).  With quantize_on_write != 0 the S
+ * new tokens are also written to the cache at positions hist_len .. hist_len+S-1. */
+HS_API int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_new,
+                         int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                         const hs_kv_layout *layout, int32_t hist_len, void *out,
+                         int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
+                         float softmax_scale, int quantize_on_write, hs_stream_t stream);
+
+/* ---- gated delta rule (replaces the decode branch qwen3_5.rs:725-751 and
+ * chunked_delta_rule qwen3_5.rs:342-498) -------------------------------------------------------
+ * q, k: [B, T, nk, dk] bf16; v: [B, T, nv, dv] bf16; g, beta: [B, T, nv] fp32 (g = log decay <= 0);
+ * state: [B, nv, dk, dv] fp32, updated in place; out: [B, T, nv, dv] fp32.
+ * v-head j reads q/k-head j / (nv/nk) (qwen3_5.rs:704-720).  With l2norm != 0, q and k are first
+ * replaced by x / max(||x||, 1e-3) (qwen3_5.rs:331-335); q is then multiplied by q_scale.
+ * T == 1 is the decode step; T > 1 runs the same recurrence token by token with the state held
+ * on chip. */
+HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, const float *g, const float *beta,
+                        float *state, float *out,
+                        int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
+                        float q_scale, int l2norm, hs_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HS_ATTN_H */

@@ -1,0 +1,79 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header declares, and its
+host-side validation rejects bad arguments before anything touches a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from hyprstream_amd import bindings as hb
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hs_attn.h")).read()
+    return sorted(set(re.findall(r"HS_API\s+[\w\s\*]+?\b(hs_\w+)\s*\(", text)))
+
+
+def test_header_declares_what_bindings_expect():
+    decl = declared_symbols()
+    assert decl, "no HS_API declarations found"
+    for name in hb.EXPORTS:
+        assert name in decl
+
+
+def test_library_exports_every_declared_symbol():
+    L = hb.lib()
+    missing = [s for s in declared_symbols() if not hasattr(L, s)]
+    assert not missing, "declared in include/hs_attn.h but not exported: %s" % missing
+
+
+def test_abi_version_and_empty_error():
+    assert hb.lib().hs_attn_abi_version() == 1
+
+
+def test_layout_struct_matches_header_size():
+    # 4 x int64 + 2 x int32 + 2 pointers
+    assert ctypes.sizeof(hb.KvLayout) == 4 * 8 + 2 * 4 + 2 * 8
+
+
+def _call_quant(layout, B=1, S=1, Hkv=2, D=128, start_pos=0, fake=0x1000):
+    p = ctypes.c_void_p(fake)
+    return hb.lib().hs_kv_quantize_int8(p, p, hb.HS_BF16, p, p, p, p, ctypes.byref(layout), None,
+                                        ctypes.c_int32(start_pos), B, S, Hkv, D, None)
+
+
+def test_quantize_rejects_overflow_like_the_reference_cache():
+    """LayerKVCache::update fails with "Cache overflow" when start_pos + S > max_seq_len
+    (kv_cache.rs:1288-1294); the ABI reports the same condition before launching anything."""
+    lay = hb.contiguous_layout(2, 16, 128)
+    rc = _call_quant(lay, S=4, start_pos=13)
+    assert rc == hb.HS_ERR_OVERFLOW
+    assert b"Cache overflow" in hb.lib().hs_attn_last_error()
+
+
+def test_quantize_rejects_bad_head_dim_and_null():
+    lay = hb.contiguous_layout(2, 16, 96)
+    assert _call_quant(lay, D=96) == hb.HS_ERR_INVALID_ARGUMENT
+    lay = hb.contiguous_layout(2, 16, 128)
+    assert _call_quant(lay, fake=0) == hb.HS_ERR_INVALID_ARGUMENT
+    lay.code_stride_head = 16 * 128 - 16  # heads would overlap
+    assert _call_quant(lay) == hb.HS_ERR_INVALID_ARGUMENT
+
+
+def test_decode_rejects_small_workspace_and_bad_gqa():
+    L = hb.lib()
+    lay = hb.contiguous_layout(2, 512, 128)
+    p = ctypes.c_void_p(0x1000)
+    need = L.hs_decode_attn_workspace_bytes(3, 8, 2, 128, 512)
+    assert need > 0 and need % 256 == 0
+    rc = L.hs_decode_attn_int8(p, p, p, p, p, ctypes.byref(lay), p, p, p, ctypes.c_size_t(need - 256), 3, 8, 2, 128,
+                               512, ctypes.c_float(0.088), None)
+    assert rc == hb.HS_ERR_WORKSPACE
+    rc = L.hs_decode_attn_int8(p, p, p, p, p, ctypes.byref(lay), p, p, p, ctypes.c_size_t(need), 3, 7, 2, 128, 512,
+                               ctypes.c_float(0.088), None)
+    assert rc == hb.HS_ERR_INVALID_ARGUMENT
+    rc = L.hs_decode_attn_int8(p, p, p, p, p, ctypes.byref(lay), p, p, p, ctypes.c_size_t(need), 3, 8, 2, 128, 513,
+                               ctypes.c_float(0.088), None)
+    assert rc == hb.HS_ERR_OVERFLOW

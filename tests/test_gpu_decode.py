@@ -1,0 +1,213 @@
+"""GPU parity: dequant-fused GQA decode attention against the CPU oracle.
+
+Tolerance of the path (fp32 comparison of the bf16 output): max-abs 2e-2, mean-abs 2e-3."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from hyprstream_amd import bindings as hb
+from hyprstream_amd import workloads as wl
+from gpu_util import DEV, DeviceCache, bf16_from_bits, run_decode
+
+pytestmark = pytest.mark.gpu
+
+TOL_MAX, TOL_MEAN = 2e-2, 2e-3
+
+
+def build_cache(case, Hkv, D, cap=None, via_gpu_quantizer=True, fp8=False):
+    k, v = case["k"], case["v"]
+    B, T = k.shape[:2]
+    c = DeviceCache(B, Hkv, cap or T, D, fp8=fp8)
+    if via_gpu_quantizer:
+        ks, vs = torch.from_numpy(k).to(DEV), torch.from_numpy(v).to(DEV)
+        if fp8:
+            hb.kv_fp8_calibrate(ks, vs, c.k_scales, c.v_scales)
+        c.write(ks, vs, None, 0)
+    else:
+        if fp8:
+            sk, sv = oracle.fp8_calibrate(k), oracle.fp8_calibrate(v)
+            c.load_canonical(oracle.quant_fp8(k, sk), oracle.quant_fp8(v, sv), sk, sv)
+        else:
+            kc, ksc = oracle.quant_int8(k)
+            vc, vsc = oracle.quant_int8(v)
+            c.load_canonical(kc, vc, ksc, vsc)
+    torch.cuda.synchronize()
+    return c
+
+
+def check(case, Hq, Hkv, D, fp8=False, cap=None, label=""):
+    c = build_cache(case, Hkv, D, cap=cap, fp8=fp8)
+    T = case["k"].shape[1]
+    got = run_decode(c, case["q_bits"], case["seq_lens"], Hq)
+    kc, vc, ks, vs = c.canonical(T)
+    want = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), kc, vc, ks, vs,
+                              oracle.FMT_FP8 if fp8 else oracle.FMT_INT8, case["seq_lens"], 1.0 / np.sqrt(D))
+    assert np.isfinite(got).all(), label
+    d = np.abs(got - want)
+    print("%s max-abs %.3e mean-abs %.3e" % (label, d.max(), d.mean()), flush=True)
+    assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, label
+    return got, want
+
+
+def test_config1_single_sequence_fp32_source():
+    """B=1, Hq 32 / Hkv 8, D 128, T 2048, K/V fp32 N(0,1) (BASELINE config 1)."""
+    case = wl.decode_case(1, 1, 32, 8, 128, 2048, bf16_source=False)
+    got, want = check(case, 32, 8, 128, label="config1")
+    assert np.abs(got - want).max() < 4e-3  # far inside the stated tolerance
+
+
+def test_codes_written_by_gpu_equal_oracle_codes():
+    case = wl.decode_case(2, 2, 8, 2, 128, 300, outliers=True)
+    c = build_cache(case, 2, 128)
+    kc, vc, ks, vs = c.canonical(300)
+    wk, wks = oracle.quant_int8(case["k"])
+    wv, wvs = oracle.quant_int8(case["v"])
+    assert np.array_equal(kc, wk) and np.array_equal(vc, wv)
+    assert np.array_equal(ks, wks) and np.array_equal(vs, wvs)
+
+
+@pytest.mark.parametrize("lens", [[1], [31], [32], [33], [127, 128, 129], [1, 700, 64, 257, 5]])
+def test_ragged_lengths_and_step_boundaries(lens):
+    B = len(lens)
+    case = wl.decode_case(3, B, 32, 8, 128, max(lens), outliers=True)
+    case["seq_lens"] = np.array(lens, np.int32)
+    check(case, 32, 8, 128, cap=max(lens) + 3, label="ragged%s" % lens)
+
+
+def test_ragged_uniform_lengths_config2_shape_reduced():
+    case = wl.decode_case(4, 6, 32, 8, 128, 1500, ragged=True, outliers=True, min_len=100)
+    check(case, 32, 8, 128, label="ragged-uniform")
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 4), (16, 2), (16, 1), (64, 8)])
+def test_gqa_group_sizes(Hq, Hkv):
+    case = wl.decode_case(5, 2, Hq, Hkv, 128, 200)
+    check(case, Hq, Hkv, 128, label="gqa%d/%d" % (Hq, Hkv))
+
+
+def test_many_chunks_single_head():
+    """One sequence, one kv-head: the split-K path uses many chunks and the merge kernel does the work."""
+    case = wl.decode_case(6, 1, 4, 1, 128, 9000)
+    check(case, 4, 1, 128, label="many-chunks")
+
+
+def test_zero_and_invalid_lengths_give_zero_rows():
+    case = wl.decode_case(7, 3, 8, 2, 128, 64)
+    case["seq_lens"] = np.array([0, 64, -3], np.int32)
+    c = build_cache(case, 2, 128)
+    got = run_decode(c, case["q_bits"], case["seq_lens"], 8, max_seq_len=64)
+    assert not got[0].any() and not got[2].any() and np.isfinite(got).all() and got[1].any()
+
+
+def test_tail_garbage_is_never_read_as_data():
+    """Codes/scales past seq_len are poison (NaN scales, extreme codes): results must not change."""
+    case = wl.decode_case(8, 2, 8, 2, 128, 100)
+    case["seq_lens"] = np.array([70, 33], np.int32)
+    c = build_cache(case, 2, 128, cap=128)
+    clean = run_decode(c, case["q_bits"], case["seq_lens"], 8)
+    for b, n in enumerate(case["seq_lens"]):
+        c.k_codes[b, :, n:] = 127
+        c.v_codes[b, :, n:] = -127
+        c.k_scales[b, :, n:] = float("nan")
+        c.v_scales[b, :, n:] = float("inf")
+    dirty = run_decode(c, case["q_bits"], case["seq_lens"], 8)
+    assert np.array_equal(clean, dirty)
+
+
+def test_large_q_and_scale_ranges():
+    """Q far outside fp16 range and K/V with huge / tiny magnitudes: the power-of-two rescaling keeps it exact."""
+    case = wl.decode_case(9, 2, 8, 2, 128, 96)
+    q = oracle.bf16_to_f32(case["q_bits"])
+    q[0] *= 3.0e5
+    q[1] *= 2.0e-6
+    case["q_bits"] = wl.to_bf16_bits(q)
+    case["k"][0] *= 1e-5
+    case["k"][1] *= 1e5
+    c = build_cache(case, 2, 128)
+    got = run_decode(c, case["q_bits"], case["seq_lens"], 8)
+    kc, vc, ks, vs = c.canonical(96)
+    want = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), kc, vc, ks, vs, oracle.FMT_INT8, case["seq_lens"],
+                              1.0 / np.sqrt(128))
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() < TOL_MAX
+
+
+def test_batched_equals_serial():
+    """The reference's own test idea (llama.rs:3658-3711): a ragged batch must equal row-by-row runs."""
+    case = wl.decode_case(10, 4, 8, 2, 128, 300, ragged=True)
+    c = build_cache(case, 2, 128)
+    full = run_decode(c, case["q_bits"], case["seq_lens"], 8)
+    for b in range(4):
+        one = DeviceCache(1, 2, 300, 128)
+        one.k_codes.copy_(c.k_codes[b:b + 1]); one.v_codes.copy_(c.v_codes[b:b + 1])
+        one.k_scales.copy_(c.k_scales[b:b + 1]); one.v_scales.copy_(c.v_scales[b:b + 1])
+        row = run_decode(one, case["q_bits"][b:b + 1], case["seq_lens"][b:b + 1], 8)
+        assert np.abs(row[0] - full[b]).max() < 2e-3
+
+
+def test_paged_block_table_matches_contiguous():
+    """Blocks of 64 tokens scattered through a pool (the reference pool uses 256-token blocks,
+    kv_cache.rs:477; 64 keeps the test small) must give the same result as the contiguous cache."""
+    B, Hq, Hkv, D, T, BT = 3, 8, 2, 128, 200, 64
+    case = wl.decode_case(11, B, Hq, Hkv, D, T, ragged=True)
+    c = build_cache(case, Hkv, D)
+    want = run_decode(c, case["q_bits"], case["seq_lens"], Hq)
+    nblk = (T + BT - 1) // BT
+    r = wl.philox(12)
+    ids = r.permutation(2 * B * nblk + 5).astype(np.int32)
+    kt, vt = ids[: B * nblk].reshape(B, nblk), ids[B * nblk: 2 * B * nblk].reshape(B, nblk)
+    pool = len(ids)
+    pk = torch.zeros(pool, Hkv, BT, D, dtype=torch.int8, device=DEV)
+    ps = torch.zeros(pool, Hkv, BT, dtype=torch.float32, device=DEV)
+    k_tab, v_tab = torch.from_numpy(kt).to(DEV), torch.from_numpy(vt).to(DEV)
+    lay = hb.paged_layout(Hkv, BT, D, k_tab, v_tab)
+    # write through the paged quantizer (one pool for K and V, as the reference's BlockPool)
+    ksrc, vsrc = torch.from_numpy(case["k"]).to(DEV), torch.from_numpy(case["v"]).to(DEV)
+    hb.kv_quantize_int8(ksrc, vsrc, pk, pk, ps, ps, lay, None, 0)
+    torch.cuda.synchronize()
+    # block contents equal the contiguous cache's
+    for b in range(B):
+        for j in range(nblk):
+            n = min(BT, T - j * BT)
+            assert torch.equal(pk[kt[b, j], :, :n], c.k_codes[b, :, j * BT: j * BT + n])
+            assert torch.equal(pk[vt[b, j], :, :n], c.v_codes[b, :, j * BT: j * BT + n])
+    q = bf16_from_bits(case["q_bits"]).to(DEV)
+    out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_attn(q, pk, pk, ps, ps, lay, torch.from_numpy(case["seq_lens"]).to(DEV), out, ws, Hkv, T,
+                   1.0 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.float().cpu().numpy(), want)
+
+
+def test_constant_values_give_constant_output():
+    """Softmax weights sum to one: with every V element equal, the output is that value."""
+    case = wl.decode_case(13, 2, 8, 2, 128, 500)
+    c = build_cache(case, 2, 128)
+    c.v_codes.fill_(64)
+    c.v_scales.fill_(0.125)
+    got = run_decode(c, case["q_bits"], case["seq_lens"], 8)
+    assert np.abs(got - 8.0).max() <= 2 ** -5  # one bf16 ulp at 8.0 is 2^-4... round-to-nearest gives half
+
+
+# ------------------------------------------------------------------ fp8 cache
+def test_fp8_decode_parity():
+    case = wl.decode_case(14, 2, 64, 8, 128, 700, sigma=0.5)
+    check(case, 64, 8, 128, fp8=True, label="fp8")
+
+
+def test_fp8_subnormal_codes_survive():
+    """Values far below the head's amax land in e4m3 subnormals; they must not be flushed."""
+    case = wl.decode_case(15, 1, 8, 1, 128, 128, sigma=0.5)
+    case["v"] *= 2.0 ** -9      # most of V quantizes to subnormal codes ...
+    case["v"][0, 0, 0, 0] = 1.0  # ... because one element pins the scale
+    case["k"] *= 2.0 ** -9
+    case["k"][0, 0, 0, 0] = 1.0
+    c = build_cache(case, 1, 128, fp8=True)
+    kc, vc, ks, vs = c.canonical(128)
+    assert ((vc & 0x78) == 0).mean() > 0.5  # exponent field zero = subnormal
+    got = run_decode(c, case["q_bits"], case["seq_lens"], 8)
+    want = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), kc, vc, ks, vs, oracle.FMT_FP8, case["seq_lens"],
+                              1.0 / np.sqrt(128))
+    assert np.abs(got - want).max() < 1e-4  # outputs are ~1e-3 in magnitude: flushing would show
