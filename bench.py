@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-KV decode-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4]
+
+One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
+sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
+(one attention layer).  The default workload is the headline configuration: batch 64, 32 query
+heads, 8 KV heads, head_dim 128, every context 8192, int8 KV with per-token-per-head fp32 scales,
+K/V source N(0,1) with 1 % outliers at 8 sigma, seeded synthetic data generated on the device.
+
+The timed region starts with all inputs resident in HBM.  Four copies of the cache at different
+addresses are rotated through so that no launch finds its data in the last-level cache.
+
+Prints ONE JSON line.  `value` is algorithmic HBM bytes per step / step time (GB/s); the line also
+carries tokens/s, the roofline of the dominant kernel (HIP events around that kernel alone, on the
+stream it runs on) and the CPU baseline: the reference's libtorch op sequence (dequantize, GQA
+expand, fp32 matmul/softmax/matmul) timed on this machine's host cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
+
+WORKLOADS = {
+    # name: (B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers)
+    "c2": (64, 32, 8, 128, 8192, False, False, 1.0, True),
+    "c2-ragged": (64, 32, 8, 128, 8192, True, False, 1.0, True),
+    "c1": (1, 32, 8, 128, 2048, False, False, 1.0, False),
+    "c4": (32, 64, 8, 128, 32768, False, True, 0.5, False),
+}
+
+
+def make_source(torch, gen, shape, sigma, outliers, dev):
+    x = torch.randn(shape, generator=gen, device=dev, dtype=torch.float32) * sigma
+    if outliers:
+        m = torch.rand(shape, generator=gen, device=dev) < 0.01
+        x = torch.where(m, torch.sign(x) * (8.0 * sigma), x)
+    return x.to(torch.bfloat16)
+
+
+def cpu_baseline(torch, name, caches, q, lens, Hq, fp8, seconds_budget=20.0):
+    """Reference op sequence on the host cores, on the first rows of the same workload."""
+    from oracle import reference_path as ref
+    B = q.shape[0]
+    T = int(lens.max())
+    bs = min(B, 4 if T <= 8192 else 1)
+    kc, vc, ks, vs = caches
+    kc_h = kc[:bs, :, :T].permute(0, 2, 1, 3).contiguous().cpu()
+    vc_h = vc[:bs, :, :T].permute(0, 2, 1, 3).contiguous().cpu()
+    if fp8:
+        ks_h, vs_h = ks[:bs].cpu(), vs[:bs].cpu()
+    else:
+        ks_h = ks[:bs, :, :T].permute(0, 2, 1).contiguous().cpu()
+        vs_h = vs[:bs, :, :T].permute(0, 2, 1).contiguous().cpu()
+    q_h = q[:bs].cpu().unsqueeze(1)
+    lens_h = [int(x) for x in lens[:bs].cpu()]
+    ragged = len(set(lens_h)) > 1 or lens_h[0] != T
+
+    def run():
+        if fp8:
+            return ref.decode_attention_fp8(q_h, kc_h, vc_h, ks_h, vs_h)
+        return ref.decode_attention_int8(q_h, kc_h, vc_h, ks_h, vs_h, lens_h if ragged else None)
+
+    run()  # warm-up
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 10 and (time.perf_counter() - t_start < seconds_budget or len(times) < 3):
+        t0 = time.perf_counter()
+        out = run()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    from hyprstream_amd import workloads as wl
+    Hkv, D = kc.shape[1], kc.shape[3]
+    nbytes = (wl.decode_bytes_fp8 if fp8 else wl.decode_bytes_int8)(np.array(lens_h), Hq, Hkv, D)
+    return {
+        "value": nbytes / med / 1e9, "unit": "GB/s", "cores": int(torch.get_num_threads()), "kind": "port",
+        "sample": "first %d of %d sequences of workload %s (T=%d): libtorch CPU dequantize + GQA expand + fp32 "
+                  "matmul/softmax/matmul, median of %d runs, %.1f ms per call, %.1f tokens/s"
+                  % (bs, B, name, T, len(times), med * 1e3, bs / med),
+        "tokens_per_s": bs / med, "ms_per_call": med * 1e3,
+    }, out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU's share of the path; --gpus must be 1 (this build has no multi-GPU leg)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from hyprstream_amd import bindings as hb
+    from hyprstream_amd import workloads as wl
+
+    if not torch.cuda.is_available():
+        print("no GPU visible: bench.py needs an MI355X", file=sys.stderr)
+        sys.exit(1)
+    hb.lib()  # fail loudly if the HIP library is not built
+    dev = "cuda:0"
+    B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(wl.SEED)
+
+    ncopies = max(1, args.copies)
+    layout = hb.contiguous_layout(Hkv, T, D)
+    cdt = torch.uint8 if fp8 else torch.int8
+    caches = []
+    for c in range(ncopies):
+        kc = torch.empty(B, Hkv, T, D, dtype=cdt, device=dev)
+        vc = torch.empty(B, Hkv, T, D, dtype=cdt, device=dev)
+        if fp8:
+            ks = torch.empty(B, Hkv, dtype=torch.float32, device=dev)
+            vs = torch.empty(B, Hkv, dtype=torch.float32, device=dev)
+        else:
+            ks = torch.empty(B, Hkv, layout.scale_stride_head, dtype=torch.float32, device=dev)
+            vs = torch.empty(B, Hkv, layout.scale_stride_head, dtype=torch.float32, device=dev)
+        caches.append((kc, vc, ks, vs))
+    # fill copy 0 through the library's own quantize-on-write path (a prefill-sized write), sequence by sequence
+    kc0, vc0, ks0, vs0 = caches[0]
+    one = hb.contiguous_layout(Hkv, T, D)
+    tchunk = min(T, 8192)
+    for b in range(B):
+        for t0 in range(0, T, tchunk):
+            ksrc = make_source(torch, gen, (1, tchunk, Hkv, D), sigma, outliers, dev)
+            vsrc = make_source(torch, gen, (1, tchunk, Hkv, D), sigma, outliers, dev)
+            if fp8:
+                if t0 == 0:
+                    hb.kv_fp8_calibrate(ksrc, vsrc, ks0[b:b + 1], vs0[b:b + 1])
+                hb.kv_quantize_fp8(ksrc, vsrc, kc0[b:b + 1], vc0[b:b + 1], ks0[b:b + 1], vs0[b:b + 1], one, None, t0)
+            else:
+                hb.kv_quantize_int8(ksrc, vsrc, kc0[b:b + 1], vc0[b:b + 1], ks0[b:b + 1], vs0[b:b + 1], one, None, t0)
+    for c in range(1, ncopies):
+        for dst, src in zip(caches[c], caches[0]):
+            dst.copy_(src)
+    if ragged:
+        lens = torch.randint(512, T + 1, (B,), generator=gen, device=dev, dtype=torch.int32)
+    else:
+        lens = torch.full((B,), T, dtype=torch.int32, device=dev)
+    pos = (lens - 1).contiguous()
+    q = torch.randn(B, Hq, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    k_new = make_source(torch, gen, (B, 1, Hkv, D), sigma, outliers, dev)
+    v_new = make_source(torch, gen, (B, 1, Hkv, D), sigma, outliers, dev)
+    out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
+    max_len = T
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, max_len), dtype=torch.uint8, device=dev)
+    scale = 1.0 / float(np.sqrt(D))
+    quant = hb.kv_quantize_fp8 if fp8 else hb.kv_quantize_int8
+
+    def step(i, phases=3):
+        kc, vc, ks, vs = caches[i % ncopies]
+        quant(k_new, v_new, kc, vc, ks, vs, layout, pos, 0)
+        hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=phases)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+
+    lens_h = lens.cpu().numpy()
+    step_bytes = (wl.decode_bytes_fp8 if fp8 else wl.decode_bytes_int8)(lens_h, Hq, Hkv, D)
+    gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # ---- roofline of the dominant kernel (split-K decode attention) alone: HIP events on its stream
+    kern_bytes = step_bytes - (B * Hkv * D * (2 * 2 + 2 * 1) + (0 if fp8 else B * Hkv * 2 * 4))  # minus the write kernel's share
+    n_ev = min(args.steps, 100)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
+    for i in range(n_ev):
+        kc, vc, ks, vs = caches[i % ncopies]
+        quant(k_new, v_new, kc, vc, ks, vs, layout, pos, 0)
+        evs[i][0].record()
+        hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=1)
+        evs[i][1].record()
+        hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=2)
+    torch.cuda.synchronize()
+    kt = np.array([a.elapsed_time(b) for a, b in evs])  # ms
+    k_avg_ms = float(kt.mean())
+    achieved = kern_bytes / (k_avg_ms * 1e-3) / 1e9
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "decode_attn_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get(args.workload)
+        except Exception:
+            traffic = None
+
+    result = {
+        "metric": "decode-attn HBM GB/s (% peak) + tokens/s, B=64 ctx 8K int8 KV, Llama-3-8B shape",
+        "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3 codes, f16 MFMA, f32 accumulate" if fp8 else "int8 codes, f16 MFMA, f32 accumulate",
+        "data": "synthetic (seeded, generated on device)",
+        "config": {"workload": "%s: B=%d Hq=%d Hkv=%d D=%d T=%s %s KV, 1 new token/seq quantized on write, one layer"
+                               % (args.workload, B, Hq, Hkv, D, "U[512,%d]" % T if ragged else str(T),
+                                  "fp8-e4m3 per-head-scale" if fp8 else "int8 per-token-per-head-scale"),
+                   "cache_copies_rotated": ncopies, "algorithmic_bytes_per_step": int(step_bytes)},
+        "pct_of_hbm_peak": 100.0 * gbs / HBM_PEAK_GBS,
+        "tokens_per_s": B / (ms_per_step * 1e-3),
+        "roofline": {"bound": "hbm", "kernel": "decode_attn_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "avg_kernel_us": k_avg_ms * 1e3, "min_kernel_us": float(kt.min()) * 1e3,
+                     "algorithmic_bytes_per_launch": int(kern_bytes), "launches_timed": n_ev},
+    }
+    if not args.no_cpu_baseline:
+        cb, _ = cpu_baseline(torch, args.workload, caches[0], q, lens, Hq, fp8)
+        result["cpu_baseline"] = cb
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -21,7 +21,7 @@ HS_BF16, HS_F32, HS_F16 = 0, 1, 2
 EXPORTS = [
     "hs_attn_last_error", "hs_attn_abi_version",
     "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
-    "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8",
+    "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
 ]
 
 
@@ -127,9 +127,13 @@ def decode_workspace_bytes(B, Hq, Hkv, D, max_seq_len):
 
 
 def decode_attn(q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace, Hkv, max_seq_len,
-                softmax_scale, fp8=False):
+                softmax_scale, fp8=False, phases=3):
     B, Hq, D = q.shape
-    fn = lib().hs_decode_attn_fp8 if fp8 else lib().hs_decode_attn_int8
+    if phases != 3:
+        fn0 = lib().hs_decode_attn_phases
+        fn = lambda *a: fn0(int(fp8), int(phases), *a)
+    else:
+        fn = lib().hs_decode_attn_fp8 if fp8 else lib().hs_decode_attn_int8
     check(fn(_ptr(q), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout),
              _ptr(seq_lens), _ptr(out), _ptr(workspace),
              ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0),

@@ -354,7 +354,7 @@ static int pick_chunk_tokens(int B, int Hkv, int max_seq_len) {
     return (int)ct;
 }
 
-static int launch_decode(bool fp8, const void *q, const void *kc, const void *vc, const float *ks, const float *vs,
+static int launch_decode(bool fp8, int phases, const void *q, const void *kc, const void *vc, const float *ks, const float *vs,
                          const hs_kv_layout *l, const int32_t *seq_lens, void *out, void *ws, size_t ws_bytes, int B,
                          int Hq, int Hkv, int D, int max_seq_len, float softmax_scale, hipStream_t stream) {
     if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
@@ -388,13 +388,18 @@ static int launch_decode(bool fp8, const void *q, const void *kc, const void *vc
     a.part_o = (float *)ws;
     a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * kD;
     a.scale_log2e = softmax_scale * kLog2e;
-    dim3 grid(a.nchunks, Hkv, B);
-    if (fp8) decode_attn_kernel<true><<<grid, 256, 0, stream>>>(a);
-    else decode_attn_kernel<false><<<grid, 256, 0, stream>>>(a);
-    if (int rc = check_launch("decode_attn")) return rc;
-    decode_merge_kernel<<<dim3(Hq, B), 128, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq, a.nchunks,
-                                                         a.chunk_tokens, max_seq_len);
-    return check_launch("decode_merge");
+    if (phases & 1) {
+        dim3 grid(a.nchunks, Hkv, B);
+        if (fp8) decode_attn_kernel<true><<<grid, 256, 0, stream>>>(a);
+        else decode_attn_kernel<false><<<grid, 256, 0, stream>>>(a);
+        if (int rc = check_launch("decode_attn")) return rc;
+    }
+    if (phases & 2) {
+        decode_merge_kernel<<<dim3(Hq, B), 128, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
+                                                             a.nchunks, a.chunk_tokens, max_seq_len);
+        return check_launch("decode_merge");
+    }
+    return HS_OK;
 }
 
 }  // namespace hs
@@ -413,7 +418,7 @@ int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_co
                         const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
                         void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
                         int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
-    return hs::launch_decode(false, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+    return hs::launch_decode(false, 3, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
                              workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
 }
 
@@ -421,8 +426,19 @@ int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8_t *v_c
                        const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
                        void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
                        int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
-    return hs::launch_decode(true, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+    return hs::launch_decode(true, 3, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
                              workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const void *k_codes, const void *v_codes,
+                          const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                          const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes, int32_t B,
+                          int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len, float softmax_scale,
+                          hs_stream_t stream) {
+    if (phases < 1 || phases > 3) return hs::fail(HS_ERR_INVALID_ARGUMENT, "phases must be 1, 2 or 3");
+    return hs::launch_decode(fmt_fp8 != 0, phases, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out,
+                             workspace, workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale,
+                             (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -132,6 +132,17 @@ HS_API int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8
                        int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
                        float softmax_scale, hs_stream_t stream);
 
+/* The two phases of decode attention on their own: phases = 1 runs only the split-K kernel that
+ * leaves per-chunk partials (m, l, o) in the workspace, 2 only the merge of those partials into
+ * `out`, 3 both (identical to the calls above).  No counterpart in the reference; it exists so that
+ * the phases can be timed separately and so that partials produced for different token ranges
+ * (for instance on different devices) can share one merge. */
+HS_API int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const void *k_codes, const void *v_codes,
+                                 const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                                 const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,
+                                 int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                                 float softmax_scale, hs_stream_t stream);
+
 /* ---- causal prefill over [int8 history] + [this call's bf16 K/V] (replaces update + get +
  * compute_attention_masked for q_len > 1: llama.rs:1066-1112, mask rule "query row i sits at
  * absolute position (k_len - q_len) + i", llama.rs:1074-1084) --------------------------------

@@ -200,9 +200,9 @@ def test_fp8_decode_parity():
 def test_fp8_subnormal_codes_survive():
     """Values far below the head's amax land in e4m3 subnormals; they must not be flushed."""
     case = wl.decode_case(15, 1, 8, 1, 128, 128, sigma=0.5)
-    case["v"] *= 2.0 ** -9      # most of V quantizes to subnormal codes ...
+    case["v"] *= 2.0 ** -15     # most of V quantizes to subnormal codes ...
     case["v"][0, 0, 0, 0] = 1.0  # ... because one element pins the scale
-    case["k"] *= 2.0 ** -9
+    case["k"] *= 2.0 ** -15
     case["k"][0, 0, 0, 0] = 1.0
     c = build_cache(case, 1, 128, fp8=True)
     kc, vc, ks, vs = c.canonical(128)
@@ -210,4 +210,6 @@ def test_fp8_subnormal_codes_survive():
     got = run_decode(c, case["q_bits"], case["seq_lens"], 8)
     want = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), kc, vc, ks, vs, oracle.FMT_FP8, case["seq_lens"],
                               1.0 / np.sqrt(128))
-    assert np.abs(got - want).max() < 1e-4  # outputs are ~1e-3 in magnitude: flushing would show
+    scale = np.abs(want).max()
+    print("fp8 subnormal: |want| max %.3e err %.3e" % (scale, np.abs(got - want).max()), flush=True)
+    assert np.abs(got - want).max() < 0.02 * scale  # flushing subnormals to zero would lose most of the output
