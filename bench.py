@@ -98,6 +98,9 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU's share of the path; --gpus must be 1 (this build has no multi-GPU leg)",
@@ -113,6 +116,14 @@ def main():
         sys.exit(1)
     hb.lib()  # fail loudly if the HIP library is not built
     dev = "cuda:0"
+    if args.calibrate_copy:
+        src = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(max(1, args.steps)):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": max(1, args.steps)}))
+        return
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)
