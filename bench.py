@@ -173,10 +173,9 @@ def main():
     scale = 1.0 / float(np.sqrt(D))
     quant = hb.kv_quantize_fp8 if fp8 else hb.kv_quantize_int8
 
-    def step(i, phases=3):
+    def step(i):
         kc, vc, ks, vs = caches[i % ncopies]
-        quant(k_new, v_new, kc, vc, ks, vs, layout, pos, 0)
-        hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=phases)
+        hb.decode_step(q, k_new, v_new, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8)
 
     for i in range(args.warmup):
         step(i)

@@ -22,6 +22,7 @@ EXPORTS = [
     "hs_attn_last_error", "hs_attn_abi_version",
     "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
+    "hs_decode_step_int8", "hs_decode_step_fp8",
 ]
 
 
@@ -138,3 +139,15 @@ def decode_attn(q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, 
              _ptr(seq_lens), _ptr(out), _ptr(workspace),
              ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0),
              B, Hq, Hkv, D, ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
+
+
+def decode_step(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace, Hkv,
+                max_seq_len, softmax_scale, fp8=False):
+    """Quantize-on-write of one new token per sequence (at seq_lens-1) + decode attention, one call."""
+    B, Hq, D = q.shape
+    assert k_new.shape == (B, 1, Hkv, D) and k_new.is_contiguous() and v_new.is_contiguous()
+    fn = lib().hs_decode_step_fp8 if fp8 else lib().hs_decode_step_int8
+    check(fn(_ptr(q), _ptr(k_new), _ptr(v_new), _dtype_code(k_new), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales),
+             _ptr(v_scales), ctypes.byref(layout), _ptr(seq_lens), _ptr(out), _ptr(workspace),
+             ctypes.c_size_t(workspace.numel() * workspace.element_size()), B, Hq, Hkv, D,
+             ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))

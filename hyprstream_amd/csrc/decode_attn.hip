@@ -23,7 +23,7 @@
 // is the running max (two butterfly steps over the lanes that share a head).
 //
 // HBM bytes per cached token and kv-head: 2*D codes + 8 B of scales (int8) -- 264 B at D = 128.
-#include "common.hpp"
+#include "quant_device.hpp"
 
 namespace hs {
 
@@ -47,6 +47,8 @@ struct DecodeArgs {
     const int32_t *seq_lens;
     float *part_o;   // [B, Hq, nchunks, D]
     float *part_ml;  // [B, Hq, nchunks, 2]   (m in log2 units, l)
+    uint32_t *counters;  // [B, Hkv] arrival counters, zero on entry; nullptr = leave partials only
+    uint16_t *out;       // [B, Hq, D] bf16
     int32_t B, Hq, Hkv, G, chunk_tokens, nchunks, max_seq_len;
     float scale_log2e;
 };
@@ -58,6 +60,16 @@ struct Stage {
     float4v sk[2];  // K scales of tokens 16u + 4q + r   (int8 only)
     float4v sv[2];
 };
+
+// Device-coherent accesses for the split-K partials: relaxed agent-scope atomics compile to plain
+// global loads/stores that are coherent across the XCDs' L2 caches (sc1), so the hand-over from the
+// writing workgroups to the merging one needs no cache-wide write-back or invalidate.
+__device__ __forceinline__ void st_agent(float *p, float v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_agent(const float *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
     u32x4 t = {a, b, c, d};
@@ -302,12 +314,29 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     }
     __syncthreads();
     const int64_t prow = ((int64_t)b * a.Hq + h * G) * a.nchunks + chunk;
+    const int my_chunks = (L + a.chunk_tokens - 1) / a.chunk_tokens;
+    if (a.counters && my_chunks == 1) {
+        // single chunk: normalise and write the output directly, no workspace traffic
+        for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
+            const int g = idx / kD, d = idx % kD;
+            float o = 0.0f, l = 0.0f, Mg = sm_m[0][g];
+#pragma unroll
+            for (int w = 1; w < kWavesPerWg; ++w) Mg = fmaxf(Mg, sm_m[w][g]);
+#pragma unroll
+            for (int w = 0; w < kWavesPerWg; ++w) {
+                o += sm_o[w][g][d];
+                l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
+            }
+            a.out[((int64_t)b * a.Hq + h * G + g) * kD + d] = (uint16_t)f32_to_bf16_bits(o * out_scale / l);
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
         const int g = idx / kD, d = idx % kD;
         float o = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWavesPerWg; ++w) o += sm_o[w][g][d];
-        a.part_o[(prow + (int64_t)g * a.nchunks) * kD + d] = o * out_scale;
+        st_agent(&a.part_o[(prow + (int64_t)g * a.nchunks) * kD + d], o * out_scale);
     }
     if (threadIdx.x < G) {
         const int g = threadIdx.x;
@@ -317,9 +346,57 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         for (int w = 0; w < kWavesPerWg; ++w)
             l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
         float *ml = a.part_ml + (prow + (int64_t)g * a.nchunks) * 2;
-        ml[0] = Mg;
-        ml[1] = l;
+        st_agent(&ml[0], Mg);
+        st_agent(&ml[1], l);
     }
+    if (!a.counters) return;
+    // ---- the last workgroup of this (sequence, kv-head) to arrive merges all chunk partials
+    __shared__ int sm_last;
+    __syncthreads();  // every thread's coherent stores above have completed (vmcnt drained) before the count
+    if (threadIdx.x == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(&a.counters[b * a.Hkv + h], 1u, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+        sm_last = (old == (uint32_t)(my_chunks - 1));
+    }
+    __syncthreads();
+    if (!sm_last) return;
+    for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
+        const int g = idx / kD, d = idx % kD;
+        const int64_t row = ((int64_t)b * a.Hq + h * G + g) * a.nchunks;
+        float M = -INFINITY;
+        for (int c = 0; c < my_chunks; ++c) M = fmaxf(M, ld_agent(&a.part_ml[(row + c) * 2]));
+        float o = 0.0f, l = 0.0f;
+        for (int c = 0; c < my_chunks; ++c) {
+            const float w = __builtin_amdgcn_exp2f(ld_agent(&a.part_ml[(row + c) * 2]) - M);
+            l += w * ld_agent(&a.part_ml[(row + c) * 2 + 1]);
+            o += w * ld_agent(&a.part_o[(row + c) * kD + d]);
+        }
+        a.out[((int64_t)b * a.Hq + h * G + g) * kD + d] = (uint16_t)f32_to_bf16_bits(o / l);
+    }
+    if (threadIdx.x == 0) a.counters[b * a.Hkv + h] = 0u;  // leave the counter ready for the next call
+}
+
+// Prologue of a fused decode step: quantize the one new token of every sequence into the cache
+// (wavefront per (sequence, kv-head, K|V) row) and zero the arrival counters of the attention kernel.
+struct PrepareArgs {
+    QuantArgs qa;        // S == 1 when there is a new token, B == 0 when there is none
+    uint32_t *counters;
+    int32_t ncounters;
+    const int32_t *seq_lens;
+    uint16_t *out;       // rows of sequences without cached tokens are zeroed here
+    int32_t B, row_elems;
+};
+
+template <int E, bool FP8>
+__global__ __launch_bounds__(256) void decode_prepare_kernel(PrepareArgs p) {
+    const int gtid = blockIdx.x * 256 + threadIdx.x;
+    if (gtid < p.ncounters) p.counters[gtid] = 0u;
+    if ((int)blockIdx.x < p.B && p.seq_lens[blockIdx.x] <= 0)
+        for (int i = threadIdx.x; i < p.row_elems; i += 256) p.out[(int64_t)blockIdx.x * p.row_elems + i] = 0;
+    const int64_t rows = (int64_t)p.qa.B * p.qa.S * p.qa.Hkv;
+    const int64_t wrow = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // 2*rows wavefront rows: K then V
+    if (wrow >= 2 * rows) return;
+    quantize_row<E, FP8>(p.qa, wrow >= rows ? 1 : 0, wrow >= rows ? wrow - rows : wrow, threadIdx.x & 63);
 }
 
 // Merge the chunk partials of one (sequence, query head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c.
@@ -343,6 +420,8 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(const float *part_o, 
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
 
+static size_t counter_bytes(int B, int Hkv) { return ((size_t)B * Hkv * sizeof(uint32_t) + 255) / 256 * 256; }
+
 static int pick_chunk_tokens(int B, int Hkv, int max_seq_len) {
     // Aim at >= 4 workgroups per CU over 256 CUs, chunks a multiple of 128 tokens (4 waves x 32).
     const int64_t units = (int64_t)B * Hkv;
@@ -354,12 +433,21 @@ static int pick_chunk_tokens(int B, int Hkv, int max_seq_len) {
     return (int)ct;
 }
 
-static int launch_decode(bool fp8, int phases, const void *q, const void *kc, const void *vc, const float *ks, const float *vs,
-                         const hs_kv_layout *l, const int32_t *seq_lens, void *out, void *ws, size_t ws_bytes, int B,
-                         int Hq, int Hkv, int D, int max_seq_len, float softmax_scale, hipStream_t stream) {
+struct NewToken {  // optional quantize-on-write of one token per sequence inside the same call
+    const void *k_src = nullptr, *v_src = nullptr;  // [B, 1, Hkv, D]
+    int dtype = HS_BF16;
+};
+
+static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q, void *kc, void *vc, float *ks,
+                         float *vs, const hs_kv_layout *l, const int32_t *seq_lens, void *out, void *ws,
+                         size_t ws_bytes, int B, int Hq, int Hkv, int D, int max_seq_len, float softmax_scale,
+                         hipStream_t stream) {
     if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
     if (D != kD) return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 128, got %d", D);
     if (!q || !kc || !vc || !ks || !vs || !seq_lens || !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if ((nt.k_src == nullptr) != (nt.v_src == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give k_new and v_new or neither");
+    if (nt.k_src && nt.dtype != HS_BF16 && nt.dtype != HS_F32 && nt.dtype != HS_F16)
+        return fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", nt.dtype);
     if (Hq <= 0 || Hq % Hkv != 0 || Hq / Hkv > 16)
         return fail(HS_ERR_INVALID_ARGUMENT, "need Hq %% Hkv == 0 and Hq/Hkv <= 16 (Hq=%d Hkv=%d)", Hq, Hkv);
     if (max_seq_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "max_seq_len must be positive");
@@ -387,14 +475,36 @@ static int launch_decode(bool fp8, int phases, const void *q, const void *kc, co
     a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
     a.part_o = (float *)ws;
     a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * kD;
+    uint32_t *counters = (uint32_t *)((char *)ws + need - counter_bytes(B, Hkv));
+    a.counters = phases == 3 ? counters : nullptr;
+    a.out = (uint16_t *)out;
     a.scale_log2e = softmax_scale * kLog2e;
+    if (phases == 3) {
+        // prologue: new-token quantize-on-write (if any), counters <- 0, empty sequences' output <- 0
+        PrepareArgs p;
+        p.qa.src[0] = nt.k_src; p.qa.src[1] = nt.v_src;
+        p.qa.codes[0] = kc; p.qa.codes[1] = vc;
+        p.qa.scales[0] = ks; p.qa.scales[1] = vs;
+        p.qa.addr[0] = a.ka; p.qa.addr[1] = a.va;
+        p.qa.positions = seq_lens; p.qa.start_pos = -1;  // the new token is the last cached one
+        p.qa.B = nt.k_src ? B : 0; p.qa.S = 1; p.qa.Hkv = Hkv; p.qa.D = D; p.qa.dtype = nt.dtype;
+        p.counters = counters; p.ncounters = B * Hkv;
+        p.seq_lens = seq_lens; p.out = (uint16_t *)out; p.B = B; p.row_elems = Hq * D;
+        const int64_t wrows = 2 * (int64_t)p.qa.B * Hkv;
+        int64_t blocks = (wrows + 3) / 4;
+        if (blocks < (p.ncounters + 255) / 256) blocks = (p.ncounters + 255) / 256;
+        if (blocks < B) blocks = B;
+        if (fp8) decode_prepare_kernel<2, true><<<(unsigned)blocks, 256, 0, stream>>>(p);
+        else decode_prepare_kernel<2, false><<<(unsigned)blocks, 256, 0, stream>>>(p);
+        if (int rc = check_launch("decode_prepare")) return rc;
+    }
     if (phases & 1) {
         dim3 grid(a.nchunks, Hkv, B);
         if (fp8) decode_attn_kernel<true><<<grid, 256, 0, stream>>>(a);
         else decode_attn_kernel<false><<<grid, 256, 0, stream>>>(a);
         if (int rc = check_launch("decode_attn")) return rc;
     }
-    if (phases & 2) {
+    if (phases == 2) {
         decode_merge_kernel<<<dim3(Hq, B), 128, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
                                                              a.nchunks, a.chunk_tokens, max_seq_len);
         return check_launch("decode_merge");
@@ -411,23 +521,50 @@ size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_
     const int ct = hs::pick_chunk_tokens(B, Hkv, max_seq_len);
     const size_t nchunks = (size_t)((max_seq_len + ct - 1) / ct);
     const size_t n = (size_t)B * Hq * nchunks * ((size_t)D + 2) * sizeof(float);
-    return (n + 255) / 256 * 256;
+    return (n + 255) / 256 * 256 + hs::counter_bytes(B, Hkv);  // partials, then the arrival counters
 }
 
 int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes, const float *k_scales,
                         const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
                         void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
                         int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
-    return hs::launch_decode(false, 3, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
-                             workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+    return hs::launch_decode(false, 3, hs::NewToken(), q, (void *)k_codes, (void *)v_codes, (float *)k_scales,
+                             (float *)v_scales, layout, seq_lens, out, workspace, workspace_bytes, B, Hq, Hkv, D,
+                             max_seq_len, softmax_scale, (hipStream_t)stream);
 }
 
 int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8_t *v_codes, const float *k_scales,
                        const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
                        void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
                        int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
-    return hs::launch_decode(true, 3, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+    return hs::launch_decode(true, 3, hs::NewToken(), q, (void *)k_codes, (void *)v_codes, (float *)k_scales,
+                             (float *)v_scales, layout, seq_lens, out, workspace, workspace_bytes, B, Hq, Hkv, D,
+                             max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_step_int8(const void *q, const void *k_new, const void *v_new, int src_dtype, int8_t *k_codes,
+                        int8_t *v_codes, float *k_scales, float *v_scales, const hs_kv_layout *layout,
+                        const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes, int32_t B,
+                        int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len, float softmax_scale,
+                        hs_stream_t stream) {
+    if (!k_new || !v_new) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    hs::NewToken nt;
+    nt.k_src = k_new; nt.v_src = v_new; nt.dtype = src_dtype;
+    return hs::launch_decode(false, 3, nt, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
                              workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_step_fp8(const void *q, const void *k_new, const void *v_new, int src_dtype, uint8_t *k_codes,
+                       uint8_t *v_codes, const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                       const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes, int32_t B,
+                       int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len, float softmax_scale,
+                       hs_stream_t stream) {
+    if (!k_new || !v_new) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    hs::NewToken nt;
+    nt.k_src = k_new; nt.v_src = v_new; nt.dtype = src_dtype;
+    return hs::launch_decode(true, 3, nt, q, k_codes, v_codes, (float *)k_scales, (float *)v_scales, layout, seq_lens,
+                             out, workspace, workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale,
+                             (hipStream_t)stream);
 }
 
 int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const void *k_codes, const void *v_codes,
@@ -436,9 +573,9 @@ int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const void *k_
                           int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len, float softmax_scale,
                           hs_stream_t stream) {
     if (phases < 1 || phases > 3) return hs::fail(HS_ERR_INVALID_ARGUMENT, "phases must be 1, 2 or 3");
-    return hs::launch_decode(fmt_fp8 != 0, phases, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out,
-                             workspace, workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale,
-                             (hipStream_t)stream);
+    return hs::launch_decode(fmt_fp8 != 0, phases, hs::NewToken(), q, (void *)k_codes, (void *)v_codes,
+                             (float *)k_scales, (float *)v_scales, layout, seq_lens, out, workspace, workspace_bytes,
+                             B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
 }
 
 }  // extern "C"

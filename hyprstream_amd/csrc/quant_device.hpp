@@ -1,0 +1,93 @@
+// Device-side row quantizer shared by the quantize-on-write kernel and the decode-step prologue.
+#pragma once
+#include "common.hpp"
+
+namespace hs {
+
+struct QuantArgs {
+    const void *src[2];   // K, V  [B, S, Hkv, D]
+    void *codes[2];
+    float *scales[2];     // int8: written; fp8: read ([B, Hkv])
+    KvAddr addr[2];
+    const int32_t *positions;
+    int32_t start_pos, B, S, Hkv, D, dtype;
+};
+
+__device__ __forceinline__ uint32_t f32_to_e4m3fn_bits(float y) {
+#pragma clang fp contract(off)
+    uint32_t u = __float_as_uint(y);
+    uint32_t sign = (u >> 24) & 0x80u;
+    u &= 0x7fffffffu;
+    if (u >= 0x43f00000u) return sign | 0x7fu;  // >= 480, inf, NaN
+    float a = __uint_as_float(u);
+    uint32_t r;
+    if (a < 0.015625f) {
+        r = (uint32_t)rintf(a * 512.0f);  // subnormal grid 2^-9; 8 == smallest normal
+    } else {
+        r = (u + 0x7ffffu + ((u >> 20) & 1u)) >> 20;  // RNE on the 3 kept mantissa bits
+        r -= (120u << 3);                              // rebias 127 -> 7
+        if (r > 0x7fu) r = 0x7fu;
+    }
+    return sign | r;
+}
+
+// One wavefront quantizes row `row` (= (b*S + s)*Hkv + h) of tensor `which` (0 = K, 1 = V).
+template <int E, bool FP8>
+__device__ __forceinline__ void quantize_row(const QuantArgs &a, int which, int64_t row, int lane) {
+#pragma clang fp contract(off)  // exactly the fp32 operations written: bit-exact with the CPU oracle
+    const int h = (int)(row % a.Hkv);
+    const int64_t bs = row / a.Hkv;
+    const int s = (int)(bs % a.S);
+    const int b = (int)(bs / a.S);
+    const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
+    const KvAddr &ad = a.addr[which];
+    int64_t unit;
+    int slot;
+    if (!resolve(ad, b, pos, unit, slot)) return;
+
+    float x[E];
+    load_src<E>(a.src[which], a.dtype, row * a.D + lane * E, x);
+
+    uint8_t *dst = (uint8_t *)a.codes[which] + unit * ad.code_stride_seq + (int64_t)h * ad.code_stride_head +
+                   (int64_t)slot * a.D + lane * E;
+    uint32_t packed = 0;
+    if (!FP8) {
+        float m = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float v = fabsf(x[e]);
+            m = v > m ? v : m;
+        }
+        m = wave_max(m);
+        float sc = 0.0f;
+        if (m > 0.0f) {
+            sc = m / 127.0f;
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float q = rintf(x[e] / sc);
+                q = q > 127.0f ? 127.0f : q;
+                q = q < -127.0f ? -127.0f : q;
+                if (q != q) q = 0.0f;
+                packed |= ((uint32_t)(int)q & 0xffu) << (8 * e);
+            }
+        }
+        if (lane == 0) a.scales[which][unit * ad.scale_stride_seq + (int64_t)h * ad.scale_stride_head + slot] = sc;
+    } else {
+        const float sc = a.scales[which][(int64_t)b * a.Hkv + h];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float y = 0.0f;
+            if (sc > 0.0f) {
+                y = x[e] / sc;
+                if (y > 448.0f) y = 448.0f;
+                if (y < -448.0f) y = -448.0f;
+            }
+            packed |= f32_to_e4m3fn_bits(y) << (8 * e);
+        }
+    }
+    if (E == 4) *(uint32_t *)dst = packed;
+    else if (E == 2) *(uint16_t *)dst = (uint16_t)packed;
+    else *dst = (uint8_t)packed;
+}
+
+}  // namespace hs

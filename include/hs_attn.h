@@ -83,7 +83,7 @@ HS_API int hs_attn_abi_version(void);
  * cquantize_blockwise_* calls at kv_cache.rs:823-840) ------------------------------------
  * k_src, v_src: [B, S, Hkv, D] contiguous, dtype src_dtype (K already rotated: the cache
  * holds post-RoPE keys, llama.rs:598-611).  Token s of sequence b goes to position
- * (positions ? positions[b] : start_pos) + s.  `positions` is a device array of B ints.
+ * (positions ? positions[b] : 0) + start_pos + s.  `positions` is a device array of B ints.
  * int8: per (token, kv-head) row  s = max|x| / 127 (fp32), code = clamp(rint(x / s), +-127),
  * all-zero row -> s = 0, codes 0.  Only the S new tokens are touched.
  * Errors: HS_ERR_OVERFLOW when positions == NULL and start_pos + S > capacity (not paged);
@@ -132,9 +132,29 @@ HS_API int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8
                        int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
                        float softmax_scale, hs_stream_t stream);
 
+/* One decode step in a single call: quantize-on-write of ONE new token per sequence (k_new, v_new:
+ * [B, 1, Hkv, D] in src_dtype, written at position seq_lens[b] - 1, i.e. seq_lens already counts it)
+ * followed by decode attention over the seq_lens[b] cached tokens.  Same results as
+ * hs_kv_quantize_* + hs_decode_attn_*; the write rides in the attention call's prologue kernel
+ * (what LlamaAttention::forward does per layer: cache.update then cache.get then attention,
+ * llama.rs:605-636). */
+HS_API int hs_decode_step_int8(const void *q, const void *k_new, const void *v_new, int src_dtype,
+                               int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                               const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                               void *workspace, size_t workspace_bytes,
+                               int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                               float softmax_scale, hs_stream_t stream);
+HS_API int hs_decode_step_fp8(const void *q, const void *k_new, const void *v_new, int src_dtype,
+                              uint8_t *k_codes, uint8_t *v_codes, const float *k_scales, const float *v_scales,
+                              const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                              void *workspace, size_t workspace_bytes,
+                              int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                              float softmax_scale, hs_stream_t stream);
+
 /* The two phases of decode attention on their own: phases = 1 runs only the split-K kernel that
- * leaves per-chunk partials (m, l, o) in the workspace, 2 only the merge of those partials into
- * `out`, 3 both (identical to the calls above).  No counterpart in the reference; it exists so that
+ * leaves per-chunk partials (m, l, o) in the workspace, 2 only a stand-alone merge of those
+ * partials into `out`, 3 is identical to the calls above (there the last workgroup to finish a
+ * (sequence, kv-head) merges its partials itself).  No counterpart in the reference; it exists so that
  * the phases can be timed separately and so that partials produced for different token ranges
  * (for instance on different devices) can share one merge. */
 HS_API int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const void *k_codes, const void *v_codes,

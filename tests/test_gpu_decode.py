@@ -213,3 +213,71 @@ def test_fp8_subnormal_codes_survive():
     scale = np.abs(want).max()
     print("fp8 subnormal: |want| max %.3e err %.3e" % (scale, np.abs(got - want).max()), flush=True)
     assert np.abs(got - want).max() < 0.02 * scale  # flushing subnormals to zero would lose most of the output
+
+
+# ------------------------------------------------------------------ fused step and phases
+def test_decode_step_equals_write_then_attend_and_oracle():
+    """hs_decode_step = quantize-on-write of one new token per row at seq_len-1, then attention."""
+    B, Hq, Hkv, D, T = 5, 32, 8, 128, 700
+    case = wl.decode_case(16, B, Hq, Hkv, D, T, ragged=True, outliers=True)
+    case["seq_lens"][0] = 0  # an empty row: nothing written, zero output
+    r = wl.philox(17)
+    new_k = wl.bf16_bits_to_f32(wl.to_bf16_bits(r.standard_normal((B, 1, Hkv, D)).astype(np.float32)))
+    new_v = wl.bf16_bits_to_f32(wl.to_bf16_bits(r.standard_normal((B, 1, Hkv, D)).astype(np.float32)))
+    lens = case["seq_lens"]
+    # reference flow: two calls
+    c1 = build_cache(case, Hkv, D)
+    pos = torch.from_numpy((lens - 1).astype(np.int32)).to(DEV)
+    nk, nv = torch.from_numpy(new_k).to(DEV).bfloat16(), torch.from_numpy(new_v).to(DEV).bfloat16()
+    c1.write(nk, nv, pos, 0)
+    want_gpu = run_decode(c1, case["q_bits"], lens, Hq, max_seq_len=T)
+    # fused flow
+    c2 = build_cache(case, Hkv, D)
+    q = bf16_from_bits(case["q_bits"]).to(DEV)
+    out = torch.full((B, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_step(q, nk, nv, c2.k_codes, c2.v_codes, c2.k_scales, c2.v_scales, c2.layout,
+                   torch.from_numpy(lens).to(DEV), out, ws, Hkv, T, 1.0 / np.sqrt(D))
+    torch.cuda.synchronize()
+    same = [bool(torch.equal(x, y)) for x, y in ((c1.k_codes, c2.k_codes), (c1.v_codes, c2.v_codes),
+                                                 (c1.k_scales, c2.k_scales), (c1.v_scales, c2.v_scales))]
+    assert all(same), same
+    got = out.float().cpu().numpy()
+    assert np.array_equal(got, want_gpu)
+    assert not got[0].any()
+    # and against the oracle, with the new token's codes made by the oracle
+    k, v = case["k"].copy(), case["v"].copy()
+    for b in range(1, B):
+        k[b, lens[b] - 1], v[b, lens[b] - 1] = new_k[b, 0], new_v[b, 0]
+    wk, wks = oracle.quant_int8(k)
+    wv, wvs = oracle.quant_int8(v)
+    kc, vc, ks, vs = c2.canonical(T)
+    for b in range(1, B):
+        n = lens[b]
+        assert np.array_equal(kc[b, :n], wk[b, :n]) and np.array_equal(ks[b, :n], wks[b, :n])
+        assert np.array_equal(vc[b, :n], wv[b, :n]) and np.array_equal(vs[b, :n], wvs[b, :n])
+    want = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), wk, wv, wks, wvs, oracle.FMT_INT8, lens,
+                              1.0 / np.sqrt(D))
+    d = np.abs(got - want)
+    assert d.max() < TOL_MAX and d.mean() < TOL_MEAN
+
+
+@pytest.mark.parametrize("shape", [(1, 4, 1, 9000), (3, 32, 8, 3000), (64, 32, 8, 300)])
+def test_partials_plus_standalone_merge_equal_fused_call(shape):
+    """phases 1 then 2 (split-K kernel, then the stand-alone merge) == phases 3 (last workgroup merges)."""
+    B, Hq, Hkv, T = shape
+    case = wl.decode_case(18, B, Hq, Hkv, 128, T, ragged=True)
+    c = build_cache(case, Hkv, 128)
+    fused = run_decode(c, case["q_bits"], case["seq_lens"], Hq, max_seq_len=T)
+    again = run_decode(c, case["q_bits"], case["seq_lens"], Hq, max_seq_len=T)
+    assert np.array_equal(fused, again)  # arrival counters are left clean: a second call gives the same bits
+    q = bf16_from_bits(case["q_bits"]).to(DEV)
+    lens = torch.from_numpy(case["seq_lens"]).to(DEV)
+    out = torch.full((B, Hq, 128), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, 128, T), dtype=torch.uint8, device=DEV)
+    for ph in (1, 2):
+        hb.decode_attn(q, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, lens, out, ws, Hkv, T,
+                       1.0 / np.sqrt(128), phases=ph)
+    torch.cuda.synchronize()
+    two = out.float().cpu().numpy()
+    assert np.abs(two - fused).max() <= 2.0 ** -8 * max(1.0, np.abs(fused).max())  # same math, other summation order
