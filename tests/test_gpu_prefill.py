@@ -1,0 +1,145 @@
+"""GPU parity: causal prefill attention over [int8 history | bf16 new tokens] against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from hyprstream_amd import bindings as hb
+from hyprstream_amd import workloads as wl
+from gpu_util import DEV, DeviceCache, bf16_from_bits, run_decode
+
+pytestmark = pytest.mark.gpu
+
+TOL_MAX, TOL_MEAN = 2e-2, 2e-3
+
+
+def bf16r(x):
+    return wl.bf16_bits_to_f32(wl.to_bf16_bits(x))
+
+
+def make(stream, B, S, Hq, Hkv, D=128, sigma=1.0):
+    r = wl.philox(stream)
+    q = bf16r(r.standard_normal((B, S, Hq, D)).astype(np.float32))
+    k = bf16r((r.standard_normal((B, S, Hkv, D)) * sigma).astype(np.float32))
+    v = bf16r((r.standard_normal((B, S, Hkv, D)) * sigma).astype(np.float32))
+    return q, k, v
+
+
+def gpu_prefill(cache, q, k, v, hist, write=True):
+    B, S, Hq, D = q.shape
+    qt, kt, vt = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
+    out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(qt, kt, vt, cache.k_codes, cache.v_codes, cache.k_scales, cache.v_scales, cache.layout, hist, out,
+                    1.0 / np.sqrt(D), write)
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+def oracle_prefill(q, k_hist_deq, v_hist_deq, k, v):
+    """Dense fp32 K/V = [dequantized history | exact new tokens]; causal with the k_len - q_len offset."""
+    B, S = q.shape[:2]
+    kd = np.concatenate([k_hist_deq, k], 1) if k_hist_deq is not None else k
+    vd = np.concatenate([v_hist_deq, v], 1) if v_hist_deq is not None else v
+    T = kd.shape[1]
+    return oracle.prefill_attn(q, kd, vd, None, None, oracle.FMT_DENSE, np.full(B, T, np.int32),
+                               1.0 / np.sqrt(q.shape[-1]))
+
+
+def compare(got, want, label):
+    assert np.isfinite(got).all(), label
+    d = np.abs(got - want)
+    print("%s max-abs %.3e mean-abs %.3e" % (label, d.max(), d.mean()), flush=True)
+    assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, label
+
+
+@pytest.mark.parametrize("S", [1, 5, 16, 33, 100, 257])
+def test_prompt_without_history(S):
+    q, k, v = make(20 + S, 2, S, 32, 8)
+    c = DeviceCache(2, 8, S, 128)
+    got = gpu_prefill(c, q, k, v, 0)
+    compare(got, oracle_prefill(q, None, None, k, v), "prompt S=%d" % S)
+    # quantize-on-write left the whole prompt in the cache, bit-exact with the oracle
+    kc, vc, ks, vs = c.canonical(S)
+    wk, wks = oracle.quant_int8(k)
+    wv, wvs = oracle.quant_int8(v)
+    assert np.array_equal(kc, wk) and np.array_equal(vc, wv) and np.array_equal(ks, wks) and np.array_equal(vs, wvs)
+
+
+@pytest.mark.parametrize("hist,S", [(19, 5), (1, 1), (32, 64), (100, 37), (256, 256)])
+def test_cached_prefill_with_int8_history(hist, S):
+    """New rows on top of an int8 history: the reference's partial-prefill case (tril(k_len - q_len))."""
+    B, Hq, Hkv = 2, 8, 2
+    qh, kh, vh = make(40 + hist, B, hist, Hq, Hkv)
+    q, k, v = make(41 + S, B, S, Hq, Hkv)
+    c = DeviceCache(B, Hkv, hist + S, 128)
+    hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+    c.write(hk, hv, None, 0)
+    got = gpu_prefill(c, q, k, v, hist)
+    kc, vc, ks, vs = c.canonical(hist)
+    want = oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v)
+    compare(got, want, "hist=%d S=%d" % (hist, S))
+    assert c.k_codes[:, :, hist:hist + S].any()  # the new rows were cached behind the history
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (4, 2), (8, 2), (16, 2), (32, 8)])
+def test_gqa_group_sizes(Hq, Hkv):
+    hist, S = 40, 50
+    qh, kh, vh = make(60, 1, hist, Hq, Hkv)
+    q, k, v = make(61, 1, S, Hq, Hkv)
+    c = DeviceCache(1, Hkv, hist + S, 128)
+    c.write(torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16(), None, 0)
+    got = gpu_prefill(c, q, k, v, hist, write=False)
+    kc, vc, ks, vs = c.canonical(hist)
+    compare(got, oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v),
+            "gqa %d/%d" % (Hq, Hkv))
+    assert not c.k_codes[:, :, hist:].any()  # quantize_on_write = 0 leaves the cache alone
+
+
+def test_chunked_prefill_config3_reduced():
+    """Config 3 at reduced size: 4 chunks of 128 tokens; chunk c attends the dequantized int8 cache of the
+    earlier chunks plus its own bf16 K/V, and is itself quantized on write."""
+    B, Hq, Hkv, C, n = 1, 8, 2, 128, 4
+    q, k, v = make(70, B, C * n, Hq, Hkv)
+    c = DeviceCache(B, Hkv, C * n, 128)
+    for i in range(n):
+        sl = slice(i * C, (i + 1) * C)
+        got = gpu_prefill(c, q[:, sl], k[:, sl], v[:, sl], i * C)
+        if i:
+            kc, vc, ks, vs = c.canonical(i * C)
+            want = oracle_prefill(q[:, sl], oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k[:, sl], v[:, sl])
+        else:
+            want = oracle_prefill(q[:, sl], None, None, k[:, sl], v[:, sl])
+        compare(got, want, "chunk %d" % i)
+    kc, vc, ks, vs = c.canonical(C * n)
+    wk, wks = oracle.quant_int8(k)
+    assert np.array_equal(kc, wk) and np.array_equal(ks, wks)
+
+
+def test_two_token_cached_forward_equals_two_decode_steps():
+    """The reference's equivalence test (llama.rs:3746-3785) across the two kernels: a 2-token cached forward
+    vs two single-token decode steps.  The second token's view of the first differs (bf16 in the prefill call,
+    int8 in the decode steps), so agreement is to the path's tolerance."""
+    B, Hq, Hkv, hist = 2, 8, 2, 77
+    qh, kh, vh = make(80, B, hist, Hq, Hkv)
+    q, k, v = make(81, B, 2, Hq, Hkv)
+    c1 = DeviceCache(B, Hkv, hist + 2, 128)
+    c1.write(torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16(), None, 0)
+    two = gpu_prefill(c1, q, k, v, hist)
+    c2 = DeviceCache(B, Hkv, hist + 2, 128)
+    c2.write(torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16(), None, 0)
+    for t in range(2):
+        kt = torch.from_numpy(k[:, t:t + 1]).to(DEV).bfloat16().contiguous()
+        vt = torch.from_numpy(v[:, t:t + 1]).to(DEV).bfloat16().contiguous()
+        c2.write(kt, vt, None, hist + t)
+        step = run_decode(c2, wl.to_bf16_bits(q[:, t]), np.full(B, hist + t + 1, np.int32), Hq)
+        d = np.abs(step - two[:, t])
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN
+    assert torch.equal(c1.k_codes, c2.k_codes) and torch.equal(c1.v_scales, c2.v_scales)
+
+
+def test_overflow_is_an_error():
+    q, k, v = make(90, 1, 8, 8, 2)
+    c = DeviceCache(1, 2, 10, 128)
+    with pytest.raises(hb.HsError) as e:
+        gpu_prefill(c, q, k, v, 4)
+    assert e.value.code == hb.HS_ERR_OVERFLOW
