@@ -51,6 +51,26 @@ __device__ __forceinline__ uint32_t pick_halves(uint32_t lo, uint32_t hi, int hs
     return __builtin_amdgcn_perm(hi, lo, hsel ? 0x07060302u : 0x05040100u);
 }
 
+// Reductions over the four lanes that share a column (li, li+16, li+32, li+48): two gfx950 lane-swap
+// VALU instructions instead of LDS-crossbar shuffles.  v_permlane32_swap exchanges the upper half of
+// its first operand with the lower half of the second; v_permlane16_swap does the same on 16-lane rows.
+__device__ __forceinline__ float quad_max(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const float m = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    const uint32_t v = __float_as_uint(m);
+    const auto c = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    return fmaxf(__uint_as_float(c[0]), __uint_as_float(c[1]));
+}
+__device__ __forceinline__ float quad_sum(float x) {
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const float m = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const uint32_t v = __float_as_uint(m);
+    const auto c = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
+
 __device__ __forceinline__ uint32_t pack_f16x2(float a, float b) {
     half2v h = {(_Float16)a, (_Float16)b};
     return __builtin_bit_cast(uint32_t, h);

@@ -28,7 +28,7 @@ namespace hs {
 constexpr int kPD = 128;
 constexpr int kPStep = 32;
 #ifndef HS_PREFILL_NB
-#define HS_PREFILL_NB 4
+#define HS_PREFILL_NB 2
 #endif
 constexpr float kPLog2e = 1.4426950408889634f;
 constexpr float kPPScale = 64.0f;
@@ -82,22 +82,27 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
         for (int i = 0; i < 8; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
     }
 
-    // Online-softmax update of one column block from its eight fp32 scores (log2 units); returns the
-    // eight weights multiplied by pv[] (caller rounds them to the MFMA input type).
-    auto softmax_update = [&](int nb, float (&sc)[8], const float (&pv)[8], float (&p)[8]) {
-        float mx = sc[0];
+    // Online softmax in two halves so that the code between them is straight-line for all column blocks
+    // (MFMA issue of one block overlaps the VALU work of another): raise_max() takes the blocks' step
+    // maxima and rescales under ONE wave-uniform branch that is rarely taken once the maxima settle;
+    // weights() turns scores into exp2 weights times pv[].
+    auto raise_max = [&](const float (&mx)[kNB]) {
+        bool changed = false;
 #pragma unroll
-        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sc[i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[nb], mx);
-        if (__builtin_amdgcn_ballot_w64(m_new > m_run[nb]) != 0) {
-            const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
-            l_run[nb] *= alpha;
+        for (int nb = 0; nb < kNB; ++nb) changed |= mx[nb] > m_run[nb];
+        if (__builtin_amdgcn_ballot_w64(changed) != 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[nb][i] *= alpha;
-            m_run[nb] = m_new;
+            for (int nb = 0; nb < kNB; ++nb) {
+                const float m_new = fmaxf(m_run[nb], mx[nb]);
+                const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+                l_run[nb] *= alpha;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[nb][i] *= alpha;
+                m_run[nb] = m_new;
+            }
         }
+    };
+    auto weights = [&](int nb, const float (&sc)[8], const float (&pv)[8], float (&p)[8]) {
         const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -203,6 +208,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
                     pv[4 * u + r] = dead ? 0.0f : st.sv[u][r] * kPPScale;
                 }
             if (step + 1 < nsteps) load_hist(st, step + 1);
+            float sc[kNB][8], mx[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
                 float4v s[2];
@@ -212,15 +218,23 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak[u][j], qop[nb][j], s[u], 0, 0, 0);
                 }
-                float sc[8], p[8];
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        sc[4 * u + r] = s[u][r] * ksc[4 * u + r] * cq[nb];
-                        if (tail && (t0 + 16 * u + 4 * lq + r >= H)) sc[4 * u + r] = -INFINITY;
+                        sc[nb][4 * u + r] = s[u][r] * ksc[4 * u + r] * cq[nb];
+                        if (tail && (t0 + 16 * u + 4 * lq + r >= H)) sc[nb][4 * u + r] = -INFINITY;
                     }
-                softmax_update(nb, sc, pv, p);
+                float m = sc[nb][0];
+#pragma unroll
+                for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[nb][i]);
+                mx[nb] = quad_max(m);
+            }
+            raise_max(mx);
+#pragma unroll
+            for (int nb = 0; nb < kNB; ++nb) {
+                float p[8];
+                weights(nb, sc[nb], pv, p);
                 const half8 pop = pack_half8(pack_f16x2(p[0], p[1]), pack_f16x2(p[2], p[3]), pack_f16x2(p[4], p[5]),
                                              pack_f16x2(p[6], p[7]));
 #pragma unroll
@@ -275,9 +289,9 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
                 for (int j = 0; j < 4; ++j) ak[u][j] = __builtin_bit_cast(bf16x8, st.k[u][j]);
             if (step + 1 < nsteps) load_new(st, step + 1);
             const float pv[8] = {kPPScale, kPPScale, kPPScale, kPPScale, kPPScale, kPPScale, kPPScale, kPPScale};
+            float sc[kNB][8], mx[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                if (t0 > min(S - 1, qw0 + 16 * (nb / a.HW) + 15)) continue;  // every key of this step is in the future
                 float4v s[2];
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
@@ -285,14 +299,22 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[u][j], qop[nb][j], s[u], 0, 0, 0);
                 }
-                float sc[8], p[8];
                 const int qlim = min(qi[nb], S - 1);
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        sc[4 * u + r] = (t0 + 16 * u + 4 * lq + r <= qlim) ? s[u][r] * cq : -INFINITY;
-                softmax_update(nb, sc, pv, p);
+                        sc[nb][4 * u + r] = (t0 + 16 * u + 4 * lq + r <= qlim) ? s[u][r] * cq : -INFINITY;
+                float m = sc[nb][0];
+#pragma unroll
+                for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[nb][i]);
+                mx[nb] = quad_max(m);
+            }
+            raise_max(mx);
+#pragma unroll
+            for (int nb = 0; nb < kNB; ++nb) {
+                float p[8];
+                weights(nb, sc[nb], pv, p);
                 const bf16x8 pop = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
                                                pack_bf16x2(p[6], p[7]));
 #pragma unroll
@@ -305,9 +327,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
     // =============================== normalise and store ===============================
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
-        float l = l_run[nb];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
+        const float l = quad_sum(l_run[nb]);
         if (qi[nb] >= S) continue;
         const float inv = 1.0f / (l * kPPScale);
         uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kPD + 32 * lq;
