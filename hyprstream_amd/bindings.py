@@ -22,7 +22,7 @@ EXPORTS = [
     "hs_attn_last_error", "hs_attn_abi_version",
     "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
-    "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8",
+    "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_deltanet_forward",
 ]
 
 
@@ -163,3 +163,14 @@ def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, 
                                      _ptr(v_scales), ctypes.byref(layout), ctypes.c_int32(hist_len), _ptr(out),
                                      B, S, Hq, Hkv, D, ctypes.c_float(softmax_scale), int(bool(quantize_on_write)),
                                      _stream()))
+
+
+def deltanet_forward(q, k, v, g, beta, state, out, q_scale, l2norm=False):
+    """Gated delta rule over T tokens; q,k bf16 [B,T,nk,128], v bf16 [B,T,nv,128], g,beta fp32 [B,T,nv],
+    state fp32 [B,nv,128,128] (updated in place), out fp32 [B,T,nv,128]."""
+    B, T, nk, dk = q.shape
+    nv, dv = v.shape[2], v.shape[3]
+    for t in (q, k, v, g, beta, state, out):
+        assert t.is_contiguous()
+    check(lib().hs_deltanet_forward(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(out),
+                                    B, T, nk, nv, dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)), _stream()))

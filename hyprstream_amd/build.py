@@ -13,7 +13,7 @@ LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libhs_attn.so")
 
-SOURCES = ["api.hip", "kv_quantize.hip", "decode_attn.hip", "prefill_attn.hip"]
+SOURCES = ["api.hip", "kv_quantize.hip", "decode_attn.hip", "prefill_attn.hip", "deltanet.hip"]
 
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
