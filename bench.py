@@ -149,14 +149,69 @@ def bench_prefill(args, torch, hb, wl):
     print(json.dumps(res))
 
 
+def bench_deltanet(args, torch, hb, wl, prefill):
+    """Config 5: gated DeltaNet, nk 16 / nv 32, dk = dv = 128.  Decode: B = 64, one token, fp32 state read and
+    written once (HBM bound).  Prefill: B = 4 x 4096 tokens through the token-by-token recurrence."""
+    dev = "cuda:0"
+    nk, nv, d = 16, 32, 128
+    B, T = (4, 4096) if prefill else (64, 1)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(wl.SEED)
+    nrm = lambda x: (x / x.norm(dim=-1, keepdim=True).clamp_min(1e-3)).to(torch.bfloat16)
+    q = nrm(torch.randn(B, T, nk, d, generator=gen, device=dev))
+    k = nrm(torch.randn(B, T, nk, d, generator=gen, device=dev))
+    v = torch.randn(B, T, nv, d, generator=gen, device=dev).to(torch.bfloat16)
+    g = -torch.nn.functional.softplus(torch.randn(B, T, nv, generator=gen, device=dev))
+    beta = torch.sigmoid(torch.randn(B, T, nv, generator=gen, device=dev))
+    ncopies = 1 if prefill else max(1, args.copies)
+    states = [torch.randn(B, nv, d, d, generator=gen, device=dev) * 0.1 for _ in range(ncopies)]
+    out = torch.empty(B, T, nv, d, dtype=torch.float32, device=dev)
+    qs = 1.0 / float(np.sqrt(d))
+
+    def step(i):
+        hb.deltanet_forward(q, k, v, g, beta, states[i % ncopies], out, qs, False)
+
+    for i in range(args.warmup):
+        step(i)
+    n_ev = args.steps
+    e0 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
+    e1 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        e0[i].record()
+        step(i)
+        e1[i].record()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    kms = float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
+    state_bytes = 2 * B * nv * d * d * 4
+    io_bytes = B * T * (2 * nk * d * 2 + nv * d * 2 + 2 * nv * 4 + nv * d * 4)
+    nbytes = state_bytes + io_bytes
+    res = {
+        "metric": "deltanet %s HBM GB/s + tokens/s, nk=16 nv=32 dk=dv=128" % ("prefill" if prefill else "decode"),
+        "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 state and arithmetic, bf16 q/k/v", "data": "synthetic (seeded, generated on device)",
+        "config": {"workload": "c5-%s: gated delta rule B=%d T=%d nk=16 nv=32 dk=dv=128, fp32 state [B,32,128,128]"
+                               % ("prefill" if prefill else "decode", B, T), "algorithmic_bytes_per_step": int(nbytes)},
+        "tokens_per_s": B * T / (ms * 1e-3),
+        "roofline": {"bound": "hbm", "kernel": "deltanet_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "avg_kernel_us": kms * 1e3},
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c5-decode", "c5-prefill"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
                          "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -185,6 +240,8 @@ def main():
         return
     if args.workload == "c3":
         return bench_prefill(args, torch, hb, wl)
+    if args.workload.startswith("c5"):
+        return bench_deltanet(args, torch, hb, wl, args.workload.endswith("prefill"))
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)
@@ -241,9 +298,30 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
+    graph = None
+    if args.graph:
+        # one HIP graph holding `ncopies` consecutive steps (one per cache copy), replayed steps/ncopies times
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(ncopies):
+                step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for i in range(ncopies):
+                step(i)
+        graph.replay()
+        torch.cuda.synchronize()
+        args.steps = max(ncopies, args.steps // ncopies * ncopies)
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
+    if graph is not None:
+        for i in range(args.steps // ncopies):
+            graph.replay()
+    else:
+        for i in range(args.steps):
+            step(i)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt / args.steps * 1e3

@@ -5,8 +5,12 @@
 // heads that read it, so every K/V byte is fetched from HBM exactly once.  Each of the four
 // wavefronts walks its own 32-token steps of the chunk with a private online-softmax state;
 // the next step's K/V/scales are already in flight (register double buffer) while the current
-// one is consumed.  The wavefronts' (m, l, o) are merged through LDS, the chunk partial goes to
-// the workspace, and a second small kernel merges the chunks.
+// one is consumed.  The wavefronts' (m, l, o) are merged through LDS.  With one chunk per sequence
+// the workgroup normalises and writes the bf16 output itself (one launch per decode step);
+// otherwise the chunk partial goes to the workspace and a second small kernel merges the chunks.
+// Quantize-on-write of the step's new token rides in the same launch: the workgroup whose chunk
+// ends at the sequence end quantizes that token's K and V rows (one wavefront each), stores codes
+// and scales, and only then starts streaming, so the token it reads back is the one it wrote.
 //
 // Arithmetic.  Both products run on the MFMA pipe (v_mfma_f32_16x16x32_f16) with the G query
 // heads on the N axis (padded to 16):
@@ -47,8 +51,9 @@ struct DecodeArgs {
     const int32_t *seq_lens;
     float *part_o;   // [B, Hq, nchunks, D]
     float *part_ml;  // [B, Hq, nchunks, 2]   (m in log2 units, l)
-    uint32_t *counters;  // [B, Hkv] arrival counters, zero on entry; nullptr = leave partials only
     uint16_t *out;       // [B, Hq, D] bf16
+    QuantArgs nt;        // the step's new token (nt.src[0] == nullptr: none); position = seq_len - 1
+    int32_t direct;      // 1: single chunk, write `out` directly; 0: leave partials in the workspace
     int32_t B, Hq, Hkv, G, chunk_tokens, nchunks, max_seq_len;
     float scale_log2e;
 };
@@ -60,16 +65,6 @@ struct Stage {
     float4v sk[2];  // K scales of tokens 16u + 4q + r   (int8 only)
     float4v sv[2];
 };
-
-// Device-coherent accesses for the split-K partials: relaxed agent-scope atomics compile to plain
-// global loads/stores that are coherent across the XCDs' L2 caches (sc1), so the hand-over from the
-// writing workgroups to the merging one needs no cache-wide write-back or invalidate.
-__device__ __forceinline__ void st_agent(float *p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float ld_agent(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
     u32x4 t = {a, b, c, d};
@@ -87,11 +82,20 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int L = min(a.seq_lens[b], a.max_seq_len);
     const int t_begin = chunk * a.chunk_tokens;
-    if (t_begin >= L) return;
+    const int G = a.G;
+    if (t_begin >= L) {
+        if (chunk == 0 && a.direct)  // a sequence without cached tokens: its output rows are zero
+            for (int i = threadIdx.x; i < G * kD; i += 256) a.out[((int64_t)b * a.Hq + h * G) * kD + i] = 0;
+        return;
+    }
     const int t_end = min(L, t_begin + a.chunk_tokens);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lq = lane >> 4;
-    const int G = a.G;
+    if (a.nt.src[0] != nullptr && t_end == L) {
+        // This workgroup reads the newest token: write it first (K by wavefront 0, V by wavefront 1).
+        if (wave < 2) quantize_row<2, FP8>(a.nt, wave, (int64_t)b * a.Hkv + h, lane);
+        __syncthreads();  // codes and scales are visible to the whole workgroup before any load
+    }
 
     // ---- Q operand: lane (head li, quarter lq) holds Q[head][32*lq + 8*j + e] for MFMA j.
     half8 qop[4];
@@ -314,9 +318,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     }
     __syncthreads();
     const int64_t prow = ((int64_t)b * a.Hq + h * G) * a.nchunks + chunk;
-    const int my_chunks = (L + a.chunk_tokens - 1) / a.chunk_tokens;
-    if (a.counters && my_chunks == 1) {
-        // single chunk: normalise and write the output directly, no workspace traffic
+    if (a.direct) {
+        // single chunk: normalise and write the output, no workspace traffic
         for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
             const int g = idx / kD, d = idx % kD;
             float o = 0.0f, l = 0.0f, Mg = sm_m[0][g];
@@ -336,7 +339,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         float o = 0.0f;
 #pragma unroll
         for (int w = 0; w < kWavesPerWg; ++w) o += sm_o[w][g][d];
-        st_agent(&a.part_o[(prow + (int64_t)g * a.nchunks) * kD + d], o * out_scale);
+        a.part_o[(prow + (int64_t)g * a.nchunks) * kD + d] = o * out_scale;
     }
     if (threadIdx.x < G) {
         const int g = threadIdx.x;
@@ -346,57 +349,9 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         for (int w = 0; w < kWavesPerWg; ++w)
             l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
         float *ml = a.part_ml + (prow + (int64_t)g * a.nchunks) * 2;
-        st_agent(&ml[0], Mg);
-        st_agent(&ml[1], l);
+        ml[0] = Mg;
+        ml[1] = l;
     }
-    if (!a.counters) return;
-    // ---- the last workgroup of this (sequence, kv-head) to arrive merges all chunk partials
-    __shared__ int sm_last;
-    __syncthreads();  // every thread's coherent stores above have completed (vmcnt drained) before the count
-    if (threadIdx.x == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(&a.counters[b * a.Hkv + h], 1u, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
-        sm_last = (old == (uint32_t)(my_chunks - 1));
-    }
-    __syncthreads();
-    if (!sm_last) return;
-    for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
-        const int g = idx / kD, d = idx % kD;
-        const int64_t row = ((int64_t)b * a.Hq + h * G + g) * a.nchunks;
-        float M = -INFINITY;
-        for (int c = 0; c < my_chunks; ++c) M = fmaxf(M, ld_agent(&a.part_ml[(row + c) * 2]));
-        float o = 0.0f, l = 0.0f;
-        for (int c = 0; c < my_chunks; ++c) {
-            const float w = __builtin_amdgcn_exp2f(ld_agent(&a.part_ml[(row + c) * 2]) - M);
-            l += w * ld_agent(&a.part_ml[(row + c) * 2 + 1]);
-            o += w * ld_agent(&a.part_o[(row + c) * kD + d]);
-        }
-        a.out[((int64_t)b * a.Hq + h * G + g) * kD + d] = (uint16_t)f32_to_bf16_bits(o / l);
-    }
-    if (threadIdx.x == 0) a.counters[b * a.Hkv + h] = 0u;  // leave the counter ready for the next call
-}
-
-// Prologue of a fused decode step: quantize the one new token of every sequence into the cache
-// (wavefront per (sequence, kv-head, K|V) row) and zero the arrival counters of the attention kernel.
-struct PrepareArgs {
-    QuantArgs qa;        // S == 1 when there is a new token, B == 0 when there is none
-    uint32_t *counters;
-    int32_t ncounters;
-    const int32_t *seq_lens;
-    uint16_t *out;       // rows of sequences without cached tokens are zeroed here
-    int32_t B, row_elems;
-};
-
-template <int E, bool FP8>
-__global__ __launch_bounds__(256) void decode_prepare_kernel(PrepareArgs p) {
-    const int gtid = blockIdx.x * 256 + threadIdx.x;
-    if (gtid < p.ncounters) p.counters[gtid] = 0u;
-    if ((int)blockIdx.x < p.B && p.seq_lens[blockIdx.x] <= 0)
-        for (int i = threadIdx.x; i < p.row_elems; i += 256) p.out[(int64_t)blockIdx.x * p.row_elems + i] = 0;
-    const int64_t rows = (int64_t)p.qa.B * p.qa.S * p.qa.Hkv;
-    const int64_t wrow = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // 2*rows wavefront rows: K then V
-    if (wrow >= 2 * rows) return;
-    quantize_row<E, FP8>(p.qa, wrow >= rows ? 1 : 0, wrow >= rows ? wrow - rows : wrow, threadIdx.x & 63);
 }
 
 // Merge the chunk partials of one (sequence, query head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c.
@@ -420,13 +375,14 @@ __global__ __launch_bounds__(128) void decode_merge_kernel(const float *part_o, 
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
 
-static size_t counter_bytes(int B, int Hkv) { return ((size_t)B * Hkv * sizeof(uint32_t) + 255) / 256 * 256; }
-
 static int pick_chunk_tokens(int B, int Hkv, int max_seq_len) {
-    // Aim at >= 4 workgroups per CU over 256 CUs, chunks a multiple of 128 tokens (4 waves x 32).
+    // A workgroup costs about 1.5 us of prologue/epilogue, so chunks are as long as the grid allows:
+    // with >= 512 (sequence, kv-head) units (two resident workgroups on each of 256 CUs) nothing is
+    // split and the step is a single launch; below that, split until about 1024 workgroups exist.
+    // Chunks are a multiple of 128 tokens (4 wavefronts x 32).  Measured on MI355X: B=64 x 8 heads x
+    // 8192 tokens runs 193 us unsplit, 196 us in 2 chunks, 205 us in 8; B=32 x 8 x 32768 is fastest at 4.
     const int64_t units = (int64_t)B * Hkv;
-    int64_t want_chunks = (1024 + units - 1) / units;
-    if (want_chunks < 1) want_chunks = 1;
+    int64_t want_chunks = units >= 512 ? 1 : (1024 + units - 1) / units;
     int64_t ct = ((int64_t)max_seq_len + want_chunks - 1) / want_chunks;
     ct = (ct + 127) / 128 * 128;
     if (ct < 256) ct = 256;
@@ -475,36 +431,22 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
     a.part_o = (float *)ws;
     a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * kD;
-    uint32_t *counters = (uint32_t *)((char *)ws + need - counter_bytes(B, Hkv));
-    a.counters = phases == 3 ? counters : nullptr;
     a.out = (uint16_t *)out;
     a.scale_log2e = softmax_scale * kLog2e;
-    if (phases == 3) {
-        // prologue: new-token quantize-on-write (if any), counters <- 0, empty sequences' output <- 0
-        PrepareArgs p;
-        p.qa.src[0] = nt.k_src; p.qa.src[1] = nt.v_src;
-        p.qa.codes[0] = kc; p.qa.codes[1] = vc;
-        p.qa.scales[0] = ks; p.qa.scales[1] = vs;
-        p.qa.addr[0] = a.ka; p.qa.addr[1] = a.va;
-        p.qa.positions = seq_lens; p.qa.start_pos = -1;  // the new token is the last cached one
-        p.qa.B = nt.k_src ? B : 0; p.qa.S = 1; p.qa.Hkv = Hkv; p.qa.D = D; p.qa.dtype = nt.dtype;
-        p.counters = counters; p.ncounters = B * Hkv;
-        p.seq_lens = seq_lens; p.out = (uint16_t *)out; p.B = B; p.row_elems = Hq * D;
-        const int64_t wrows = 2 * (int64_t)p.qa.B * Hkv;
-        int64_t blocks = (wrows + 3) / 4;
-        if (blocks < (p.ncounters + 255) / 256) blocks = (p.ncounters + 255) / 256;
-        if (blocks < B) blocks = B;
-        if (fp8) decode_prepare_kernel<2, true><<<(unsigned)blocks, 256, 0, stream>>>(p);
-        else decode_prepare_kernel<2, false><<<(unsigned)blocks, 256, 0, stream>>>(p);
-        if (int rc = check_launch("decode_prepare")) return rc;
-    }
+    a.direct = (phases == 3 && a.nchunks == 1) ? 1 : 0;
+    a.nt.src[0] = nt.k_src; a.nt.src[1] = nt.v_src;
+    a.nt.codes[0] = kc; a.nt.codes[1] = vc;
+    a.nt.scales[0] = ks; a.nt.scales[1] = vs;
+    a.nt.addr[0] = a.ka; a.nt.addr[1] = a.va;
+    a.nt.positions = seq_lens; a.nt.start_pos = -1;  // the new token is the last cached one
+    a.nt.B = B; a.nt.S = 1; a.nt.Hkv = Hkv; a.nt.D = D; a.nt.dtype = nt.dtype;
     if (phases & 1) {
         dim3 grid(a.nchunks, Hkv, B);
         if (fp8) decode_attn_kernel<true><<<grid, 256, 0, stream>>>(a);
         else decode_attn_kernel<false><<<grid, 256, 0, stream>>>(a);
         if (int rc = check_launch("decode_attn")) return rc;
     }
-    if (phases == 2) {
+    if ((phases & 2) && !a.direct) {
         decode_merge_kernel<<<dim3(Hq, B), 128, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
                                                              a.nchunks, a.chunk_tokens, max_seq_len);
         return check_launch("decode_merge");
@@ -521,7 +463,7 @@ size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_
     const int ct = hs::pick_chunk_tokens(B, Hkv, max_seq_len);
     const size_t nchunks = (size_t)((max_seq_len + ct - 1) / ct);
     const size_t n = (size_t)B * Hq * nchunks * ((size_t)D + 2) * sizeof(float);
-    return (n + 255) / 256 * 256 + hs::counter_bytes(B, Hkv);  // partials, then the arrival counters
+    return (n + 255) / 256 * 256;
 }
 
 int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes, const float *k_scales,
