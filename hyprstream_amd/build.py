@@ -12,6 +12,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libhs_attn.so")
+HOST_LIB = os.path.join(LIBDIR, "libhs_kv_cache.so")
 
 SOURCES = ["api.hip", "kv_quantize.hip", "decode_attn.hip", "prefill_attn.hip", "deltanet.hip"]
 
@@ -46,6 +47,13 @@ def build(verbose=False):
     with ThreadPoolExecutor(max_workers=4) as ex:
         objs = list(ex.map(lambda s: _compile(s, verbose), SOURCES))
     cmd = ["hipcc", "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    # host-side LayerKVCache mirror: plain C++ over the C ABI above (it owns device memory, the kernels do not)
+    hsrc = [os.path.join(HERE, "host", f) for f in ("kv_cache.cpp", "kv_cache_capi.cpp")]
+    cmd = ["hipcc", "-shared", "-fPIC", "-O2", "-std=c++17", "-fvisibility=hidden", "-Wall", "-x", "hip", "--offload-arch=gfx950"]
+    cmd += hsrc + ["-o", HOST_LIB, "-L" + LIBDIR, "-lhs_attn", "-Wl,-rpath,$ORIGIN"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

@@ -1,0 +1,100 @@
+// Host-side mirror of hyprstream's LayerKVCache for the device-resident quantized formats.
+//
+// Same call surface as the reference type (crates/hyprstream/src/runtime/kv_cache.rs:1027-1891):
+//   new(max_seq_len, quant_type)   :1043      update(keys, values, start_pos) :1275
+//   get()                          :1499      clear()                         :1646
+//   truncate_to(pos)               :1707      is_initialized()                :1753
+//   memory_usage()                 :1767      quant_type()                    :1861
+// with the storage replaced: codes and scales live on the GPU in the library's head-major layout,
+// update() quantizes ONLY the new tokens (no 64-token buffer, no flush that re-quantizes the whole
+// history, no host copy of the codes: kv_cache.rs:1204-1272, 842-856), and attention reads the codes
+// directly, so get() hands out a view (pointers + layout + length) instead of materialising dense
+// tensors; get_dense() is the literal get() for callers that still want [B, T, Hkv, D] tensors.
+// Tensors are raw device pointers plus explicit shapes (the reference passes tch::Tensor).
+// Errors are returned, never thrown across the boundary: hs::Status carries the reference's messages
+// ("Cache overflow: ...", "Cache is empty", "Expected 4D tensor ..." becomes a shape check).
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <string>
+
+#include "../../include/hs_attn.h"
+
+namespace hs {
+
+// KVQuantType of the reference is {None, Int8, Nf4, Fp4} (hyprstream-rpc-std/schema/model.capnp:251-257).
+// This library serves two device formats: Int8 = symmetric absmax per (token, kv-head);
+// Fp8 = e4m3fn with one scale per (sequence, kv-head), calibrated on the first (prompt) update.
+enum class KVQuantType : int { None = 0, Int8 = 1, Fp8 = 2 };
+
+struct Status {
+    int code = HS_OK;
+    std::string message;
+    bool ok() const { return code == HS_OK; }
+};
+
+// What get() returns: everything the attention entry points need.
+struct KVView {
+    void *k_codes = nullptr, *v_codes = nullptr;
+    float *k_scales = nullptr, *v_scales = nullptr;
+    hs_kv_layout layout{};
+    int32_t batch = 0, seq_pos = 0, num_kv_heads = 0, head_dim = 0;
+    KVQuantType quant_type = KVQuantType::None;
+};
+
+class LayerKVCache {
+  public:
+    LayerKVCache(size_t max_seq_len, KVQuantType quant_type);
+    ~LayerKVCache();
+    LayerKVCache(const LayerKVCache &) = delete;
+    LayerKVCache &operator=(const LayerKVCache &) = delete;
+
+    // new_keys/new_values: device pointers to [batch, seq_len, num_kv_heads, head_dim] in `dtype`
+    // (HS_BF16 / HS_F32 / HS_F16).  Tokens land at start_pos .. start_pos+seq_len-1; seq_pos becomes
+    // start_pos + seq_len.  start_pos == 0 starts a fresh prompt (kv_cache.rs:1341-1349).
+    Status update(const void *new_keys, const void *new_values, int dtype, int32_t batch, int32_t seq_len,
+                  int32_t num_kv_heads, int32_t head_dim, size_t start_pos, hs_stream_t stream = nullptr);
+
+    Status get(KVView *view) const;  // "Cache is empty" when seq_pos == 0
+    // Dense [batch, seq_pos, num_kv_heads, head_dim] K and V in `dtype`, as the reference's get() returns.
+    Status get_dense(void *keys_out, void *values_out, int dtype, hs_stream_t stream = nullptr) const;
+
+    // Attention over the cached tokens: q, out are bf16 [batch, num_q_heads, head_dim] (one query token
+    // per sequence, every sequence at seq_pos tokens).  decode_step() first caches one new token.
+    Status decode_attention(const void *q, void *out, int32_t num_q_heads, float softmax_scale,
+                            hs_stream_t stream = nullptr);
+    Status decode_step(const void *q, const void *k_new, const void *v_new, int dtype, void *out, int32_t num_q_heads,
+                       float softmax_scale, hs_stream_t stream = nullptr);
+    // Causal attention of seq_len new tokens at start_pos over [cached 0..start_pos) | new tokens], then
+    // caches them (update + get + attention of LlamaAttention::forward in one call; int8 format only).
+    Status prefill(const void *q, const void *new_keys, const void *new_values, void *out, int32_t batch,
+                   int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, size_t start_pos,
+                   float softmax_scale, hs_stream_t stream = nullptr);
+
+    void clear();
+    void truncate_to(size_t pos);
+    bool is_initialized() const { return k_codes_ != nullptr && seq_pos > 0; }
+    size_t memory_usage() const;
+    KVQuantType quant_type() const { return quant_type_; }
+
+    size_t seq_pos = 0;      // number of cached tokens (public in the reference too)
+    size_t max_seq_len = 0;  // hard limit
+
+  private:
+    Status ensure_storage(int32_t batch, int32_t num_kv_heads, int32_t head_dim);
+    Status ensure_scratch(size_t bytes, int32_t batch);
+    void release();
+
+    KVQuantType quant_type_;
+    void *k_codes_ = nullptr, *v_codes_ = nullptr;
+    float *k_scales_ = nullptr, *v_scales_ = nullptr;
+    int32_t *seq_lens_dev_ = nullptr;  // [batch], every entry == seq_pos
+    size_t seq_lens_value_ = (size_t)-1;
+    void *workspace_ = nullptr;
+    size_t workspace_bytes_ = 0;
+    hs_kv_layout layout_{};
+    int32_t batch_ = 0, heads_ = 0, dim_ = 0;
+    size_t bytes_ = 0;
+};
+
+}  // namespace hs

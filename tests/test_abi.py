@@ -11,8 +11,8 @@ from hyprstream_amd import bindings as hb
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "hs_attn.h")).read()
+def declared_symbols(header="hs_attn.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     return sorted(set(re.findall(r"HS_API\s+[\w\s\*]+?\b(hs_\w+)\s*\(", text)))
 
 
@@ -77,3 +77,41 @@ def test_decode_rejects_small_workspace_and_bad_gqa():
     rc = L.hs_decode_attn_int8(p, p, p, p, p, ctypes.byref(lay), p, p, p, ctypes.c_size_t(need), 3, 8, 2, 128, 513,
                                ctypes.c_float(0.088), None)
     assert rc == hb.HS_ERR_OVERFLOW
+
+
+# ------------------------------------------------------------------ host mirror (libhs_kv_cache.so)
+def test_cache_library_exports_every_declared_symbol():
+    from hyprstream_amd import kv_cache as kc
+    L = kc.lib()
+    decl = declared_symbols("hs_kv_cache.h")
+    assert sorted(decl) == sorted(kc.EXPORTS)
+    missing = [s for s in decl if not hasattr(L, s)]
+    assert not missing, missing
+
+
+def test_cache_host_logic_without_a_gpu():
+    """Bookkeeping and error paths of LayerKVCache that return before any device work."""
+    from hyprstream_amd import kv_cache as kc
+    L = kc.lib()
+    assert not L.hs_cache_create(0, kc.INT8) and not L.hs_cache_create(16, 7)
+    c = ctypes.c_void_p(L.hs_cache_create(100, kc.INT8))
+    assert L.hs_cache_seq_pos(c) == 0 and L.hs_cache_max_seq_len(c) == 100
+    assert not L.hs_cache_is_initialized(c) and L.hs_cache_memory_usage(c) == 0
+    assert L.hs_cache_quant_type(c) == kc.INT8
+    p = ctypes.c_void_p(0x1000)
+    # get() on an empty cache: "Cache is empty" (kv_cache.rs:1500-1502)
+    assert L.hs_cache_get_dense(c, p, p, hb.HS_BF16, None) != hb.HS_OK
+    assert L.hs_cache_last_error(c) == b"Cache is empty"
+    # update past max_seq_len: "Cache overflow: ..." (kv_cache.rs:1288-1294)
+    rc = L.hs_cache_update(c, p, p, hb.HS_BF16, 1, 10, 8, 128, ctypes.c_int64(95), None)
+    assert rc == hb.HS_ERR_OVERFLOW
+    assert L.hs_cache_last_error(c) == (b"Cache overflow: trying to cache 10 tokens starting at position 95, "
+                                        b"but max_seq_len is 100")
+    assert L.hs_cache_seq_pos(c) == 0
+    L.hs_cache_truncate_to(c, ctypes.c_int64(5))  # nothing to truncate
+    L.hs_cache_clear(c)
+    assert L.hs_cache_seq_pos(c) == 0
+    L.hs_cache_destroy(c)
+    n = ctypes.c_void_p(L.hs_cache_create(10, kc.NONE))
+    assert L.hs_cache_update(n, p, p, hb.HS_BF16, 1, 1, 8, 128, ctypes.c_int64(0), None) == hb.HS_ERR_INVALID_ARGUMENT
+    L.hs_cache_destroy(n)
