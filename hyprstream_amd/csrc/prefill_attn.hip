@@ -6,20 +6,22 @@
 //   (2) new tokens 0..=i in exact bf16,
 // which is softmax(Q K^T * scale + causal mask) V over [history | this call's K/V].
 //
-// Work split.  A wavefront owns 64 (query, head) columns = 4 MFMA column blocks of 16: with
-// G = Hq/Hkv >= 4 that is 16 queries x 4 query heads of one kv-head, so every K/V tile it loads
-// and converts is used four times; smaller G trade heads for more queries.  A workgroup is four
-// such wavefronts on consecutive queries; grid = (query tiles, kv-heads x head groups, sequences).
-// Wavefronts never synchronise: each keeps its own online-softmax state per column and walks the
-// keys in 32-key steps with the next step's tile already in flight (register double buffer).
+// Work split.  A 512-thread workgroup (8 wavefronts, 2 per SIMD) owns 256 (query, head) columns of
+// one kv-head -- with G = Hq/Hkv >= 4: 64 consecutive queries x 4 query heads -- and walks the keys
+// in 32-key steps.  Every step's K and V tile is converted ONCE per workgroup into ready-to-issue
+// MFMA A operands in LDS (16 blocks of 64 lanes x 16 B: K as 2 tiles x 4 k-groups, V^T as 8 row
+// groups) by the eight wavefronts together, double-buffered, one barrier per step; each wavefront
+// then reads the operands with conflict-free ds_read_b128 and uses each one for its two 16-column
+// blocks.  Grid = (query tiles, kv-heads x head groups, sequences).
 //
 // Products (both on v_mfma_f32_16x16x32, keys on the M axis, columns on N):
 //   S^T[key, col]  = sum_d K[key, d] Q[col, d]
 //   O^T[d, col]   += sum_key V^T[d, key] P^T[key, col]
 // History part: f16 MFMA, int8 codes enter as exact fp16 integers (see decode_attn.hip); Q is scaled
-// per column by a power of two into fp16 range; per-token K scale on the fp32 score, per-token V
-// scale folded into P (fp16).  New-token part: bf16 MFMA straight from the caller's bf16 K/V, V^T
-// built with byte permutes in registers, P rounded to bf16.  Accumulation, softmax: fp32.
+// per column by a power of two into fp16 range; the per-token K scale multiplies the fp32 score, the
+// per-token V scale is folded into P (fp16).  New-token part: bf16 MFMA straight from the caller's
+// bf16 K/V, V^T built with permutes, P rounded to bf16.  Softmax and accumulation are fp32; the
+// score layout of the first product is the B-operand layout of the second, so P stays in its lanes.
 #include "mfma_common.hpp"
 #include "quant_device.hpp"
 
@@ -27,9 +29,8 @@ namespace hs {
 
 constexpr int kPD = 128;
 constexpr int kPStep = 32;
-#ifndef HS_PREFILL_NB
-#define HS_PREFILL_NB 2
-#endif
+constexpr int kPWaves = 8;
+constexpr int kNB = 2;  // 16-column blocks per wavefront
 constexpr float kPLog2e = 1.4426950408889634f;
 constexpr float kPPScale = 64.0f;
 
@@ -39,38 +40,40 @@ struct PrefillArgs {
     const float *ks, *vs;
     KvAddr ka, va;
     uint16_t *out;  // [B,S,Hq,D] bf16
-    int32_t B, S, Hq, Hkv, G, HW, QT, hist_len;
+    int32_t B, S, Hq, Hkv, G, HG, hist_len;
     float scale_log2e;
 };
 
-struct HistStage {
-    u32x4 k[2][2];
-    u32x2 v[8];
-    float4v sk[2], sv[2];
-};
-struct NewStage {
-    u32x4 k[2][4];  // tile u, MFMA j: eight bf16 (d = 32*lq + 8*j ..)
-    u32x4 v[8];     // key slot e: eight bf16 (d = 8*li ..)
+struct alignas(16) StepTile {
+    uint8_t k[8][1024];  // block 4*u + j: K tile u (16 keys), k-group j; 64 lanes x 16 B in MFMA lane order
+    uint8_t v[8][1024];  // block bb: V^T rows d = 8*li + bb, 32 keys
+    float ksc[32];       // K scale of the step's tokens (0 for tokens past the end)
+    float pv[32];        // V scale x 64 (0 past the end)
 };
 
-template <int kNB>  // column blocks (16 columns each) per wavefront
-__global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
+__global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
+    __shared__ StepTile tiles[2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lq = lane >> 4;
     const int b = blockIdx.z;
-    const int groups = a.G / a.HW;
+    const int groups = a.G / a.HG;
     const int kvh = blockIdx.y / groups, hg = blockIdx.y % groups;
     const int S = a.S, H = a.hist_len;
-    const int qw0 = (blockIdx.x * 4 + wave) * 16 * a.QT;  // first query of this wavefront
-    if (qw0 >= S) return;
-    const int qw_last = min(S - 1, qw0 + 16 * a.QT - 1);
+    const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
+    const int q0 = blockIdx.x * q_per_wg;
+    if (q0 >= S) return;
+    const int wg_qlast = min(S - 1, q0 + q_per_wg - 1);
 
     int head[kNB], qi[kNB];
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
-        head[nb] = kvh * a.G + hg * a.HW + nb % a.HW;
-        qi[nb] = qw0 + 16 * (nb / a.HW) + li;
+        const int bi = kNB * wave + nb;
+        head[nb] = kvh * a.G + hg * a.HG + bi % a.HG;
+        qi[nb] = q0 + 16 * (bi / a.HG) + li;
     }
+    const int wv_q0 = q0 + 16 * ((kNB * wave) / a.HG);  // first query of this wavefront
+    const int wv_qlast = min(S - 1, q0 + 16 * ((kNB * wave + kNB - 1) / a.HG) + 15);
+    const bool wv_active = wv_q0 < S;
 
     float4v acc[kNB][8];
     float m_run[kNB], l_run[kNB];
@@ -82,10 +85,8 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
         for (int i = 0; i < 8; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
     }
 
-    // Online softmax in two halves so that the code between them is straight-line for all column blocks
-    // (MFMA issue of one block overlaps the VALU work of another): raise_max() takes the blocks' step
-    // maxima and rescales under ONE wave-uniform branch that is rarely taken once the maxima settle;
-    // weights() turns scores into exp2 weights times pv[].
+    // Online softmax: raise_max() takes the blocks' step maxima (already reduced over the column) and
+    // rescales under one wave-uniform branch that is rarely taken once the maxima settle.
     auto raise_max = [&](const float (&mx)[kNB]) {
         bool changed = false;
 #pragma unroll
@@ -102,15 +103,8 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
             }
         }
     };
-    auto weights = [&](int nb, const float (&sc)[8], const float (&pv)[8], float (&p)[8]) {
-        const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const float e = __builtin_amdgcn_exp2f(sc[i] - mref);
-            l_run[nb] += e;
-            p[i] = e * pv[i];
-        }
-    };
+
+    const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
 
     // =============================== history: int8 cache, f16 MFMA ===============================
     if (H > 0) {
@@ -131,8 +125,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
             }
 #pragma unroll
             for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
-            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            amax = quad_max(amax);
             int ex = 0;
             if (amax > 0.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
             float qsum = 0.0f;
@@ -144,103 +137,139 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
                     qop[nb][j][e] = hq;
                     qsum += (float)hq;
                 }
-            qsum += __shfl_xor(qsum, 16, 64);
-            qsum += __shfl_xor(qsum, 32, 64);
+            qsum = quad_sum(qsum);
             cq[nb] = ldexpf(a.scale_log2e, ex);
             cinit[nb] = -1152.0f * qsum;
         }
 
         const int nsteps = (H + kPStep - 1) / kPStep;
-        auto load_hist = [&](HistStage &st, int step) {
+        // ---- producer roles: wavefronts 0-3 convert K (tile u = wave/2, k-groups 2*(wave&1) and +1);
+        //      wavefronts 4-7 convert V (token group wave-4, byte columns 2x and 2x+1 with x = lane/16);
+        //      wavefront 0 also stages the scales.
+        u32x4 rawk = {0u, 0u, 0u, 0u};
+        uint32_t rawv[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+        float raws = 0.0f;
+        auto issue = [&](int step) {
             const int t0 = step * kPStep;
-            int64_t ku, vu;
-            int kslot, vslot;
-            resolve(a.ka, b, t0, ku, kslot);
-            resolve(a.va, b, t0, vu, vslot);
             const int last = H - 1 - t0;
-            const uint8_t *kb = a.kc + ku * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)kslot * kPD;
-            const uint8_t *vb = a.vc + vu * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)vslot * kPD;
+            int64_t unit;
+            int slot;
+            if (wave < 4) {
+                resolve(a.ka, b, t0, unit, slot);
+                const uint8_t *kb = a.kc + unit * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)slot * kPD;
+                rawk = *(const u32x4 *)(kb + min(16 * (wave >> 1) + li, last) * kPD + 32 * lq + 16 * (wave & 1));
+                if (wave == 0) {
+                    const int tok = lane & 31;
+                    if (lane < 32) {
+                        raws = a.ks[unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot + min(tok, last)];
+                    } else {
+                        resolve(a.va, b, t0, unit, slot);
+                        raws = a.vs[unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot + min(tok, last)] * kPPScale;
+                    }
+                    if (tok > last) raws = 0.0f;
+                }
+            } else {
+                resolve(a.va, b, t0, unit, slot);
+                const uint8_t *vb = a.vc + unit * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)slot * kPD;
+                const int g4 = wave - 4;
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const uint8_t *p = kb + min(16 * u + li, last) * kPD + 32 * lq;
-                st.k[u][0] = *(const u32x4 *)p;
-                st.k[u][1] = *(const u32x4 *)(p + 16);
-            }
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    st.v[4 * u + r] = *(const u32x2 *)(vb + min(16 * u + 4 * lq + r, last) * kPD + 8 * li);
-            const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + kslot;
-            const float *vsb = a.vs + vu * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + vslot;
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int tok = min(16 * u + 4 * lq, last & ~3);
-                st.sk[u] = *(const float4v *)(ksb + tok);
-                st.sv[u] = *(const float4v *)(vsb + tok);
+                for (int e = 0; e < 8; ++e)
+                    rawv[e] = *(const uint32_t *)(vb + min(16 * (e >> 2) + 4 * g4 + (e & 3), last) * kPD + 8 * li + 4 * (lq >> 1));
             }
         };
-        HistStage st;
-        load_hist(st, 0);
-        for (int step = 0; step < nsteps; ++step) {
+        auto commit = [&](StepTile &t) {
+            if (wave < 4) {
+                const int blk = 4 * (wave >> 1) + 2 * (wave & 1);
+                *(half8 *)(t.k[blk] + obase) = int8x8_to_f16_biased(rawk[0], rawk[1]);
+                *(half8 *)(t.k[blk + 1] + obase) = int8x8_to_f16_biased(rawk[2], rawk[3]);
+                if (wave == 0) (lane < 32 ? t.ksc : t.pv)[lane & 31] = raws;
+            } else {
+                const int dst = (li + 16 * (wave - 4)) * 16;  // operand lane = (li, token group wave-4)
+                const int bsel = 2 * (lq & 1);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+                    *(half8 *)(t.v[2 * lq + i] + dst) =
+                        pack_half8(int8_pair_to_f16(rawv[0], rawv[1], bsel + i), int8_pair_to_f16(rawv[2], rawv[3], bsel + i),
+                                   int8_pair_to_f16(rawv[4], rawv[5], bsel + i), int8_pair_to_f16(rawv[6], rawv[7], bsel + i));
+            }
+        };
+        auto consume = [&](const StepTile &t, int step) {
             const int t0 = step * kPStep;
-            // raw tile -> MFMA operands; the raw registers are then free for the next tile's loads
-            half8 ak[2][4], av[8];
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    ak[u][j] = int8x8_to_f16_biased(st.k[u][j >> 1][2 * (j & 1)], st.k[u][j >> 1][2 * (j & 1) + 1]);
-#pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
-                av[bb] = pack_half8(int8_pair_to_f16(st.v[0][bb >> 2], st.v[1][bb >> 2], bb & 3),
-                                    int8_pair_to_f16(st.v[2][bb >> 2], st.v[3][bb >> 2], bb & 3),
-                                    int8_pair_to_f16(st.v[4][bb >> 2], st.v[5][bb >> 2], bb & 3),
-                                    int8_pair_to_f16(st.v[6][bb >> 2], st.v[7][bb >> 2], bb & 3));
-            float ksc[8], pv[8];
             const bool tail = t0 + kPStep > H;
+            float ksc[8], pv[8];
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < 2; ++u) {
+                const float4v k4 = *(const float4v *)(t.ksc + 16 * u + 4 * lq);
+                const float4v p4 = *(const float4v *)(t.pv + 16 * u + 4 * lq);
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const bool dead = tail && (t0 + 16 * u + 4 * lq + r >= H);
-                    ksc[4 * u + r] = dead ? 0.0f : st.sk[u][r];
-                    pv[4 * u + r] = dead ? 0.0f : st.sv[u][r] * kPPScale;
+                    ksc[4 * u + r] = k4[r];
+                    pv[4 * u + r] = p4[r];
                 }
-            if (step + 1 < nsteps) load_hist(st, step + 1);
+            }
+            float4v s[kNB][2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){cinit[nb], cinit[nb], cinit[nb], cinit[nb]};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const half8 ak = *(const half8 *)(t.k[4 * u + j] + obase);
+#pragma unroll
+                    for (int nb = 0; nb < kNB; ++nb)
+                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak, qop[nb][j], s[nb][u], 0, 0, 0);
+                }
+            }
             float sc[kNB][8], mx[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                float4v s[2];
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    s[u] = (float4v){cinit[nb], cinit[nb], cinit[nb], cinit[nb]};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak[u][j], qop[nb][j], s[u], 0, 0, 0);
-                }
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        sc[nb][4 * u + r] = s[u][r] * ksc[4 * u + r] * cq[nb];
-                        if (tail && (t0 + 16 * u + 4 * lq + r >= H)) sc[nb][4 * u + r] = -INFINITY;
-                    }
+                    for (int r = 0; r < 4; ++r) sc[nb][4 * u + r] = s[nb][u][r] * ksc[4 * u + r];
+                if (tail) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (t0 + 16 * u + 4 * lq + r >= H) sc[nb][4 * u + r] = -INFINITY;
+                }
                 float m = sc[nb][0];
 #pragma unroll
                 for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[nb][i]);
-                mx[nb] = quad_max(m);
+                mx[nb] = quad_max(m) * cq[nb];  // cq > 0: max(t) * cq == max(t * cq); -inf stays -inf
             }
             raise_max(mx);
+            half8 pop[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
+                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb];
                 float p[8];
-                weights(nb, sc[nb], pv, p);
-                const half8 pop = pack_half8(pack_f16x2(p[0], p[1]), pack_f16x2(p[2], p[3]), pack_f16x2(p[4], p[5]),
-                                             pack_f16x2(p[6], p[7]));
 #pragma unroll
-                for (int bb = 0; bb < 8; ++bb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[bb], pop, acc[nb][bb], 0, 0, 0);
+                for (int i = 0; i < 8; ++i) {
+                    const float e = __builtin_amdgcn_exp2f(sc[nb][i] * cq[nb] - mref);
+                    l_run[nb] += e;
+                    p[i] = e * pv[i];
+                }
+                pop[nb] = pack_half8(pack_f16x2(p[0], p[1]), pack_f16x2(p[2], p[3]), pack_f16x2(p[4], p[5]), pack_f16x2(p[6], p[7]));
             }
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb) {
+                const half8 av = *(const half8 *)(t.v[bb] + obase);
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb)
+                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, pop[nb], acc[nb][bb], 0, 0, 0);
+            }
+        };
+        issue(0);
+        commit(tiles[0]);
+        if (nsteps > 1) issue(1);
+        __syncthreads();
+        for (int step = 0; step < nsteps; ++step) {
+            if (step + 1 < nsteps) commit(tiles[(step + 1) & 1]);
+            if (step + 2 < nsteps) issue(step + 2);
+            if (wv_active) consume(tiles[step & 1], step);
+            __syncthreads();
         }
     }
 
@@ -254,73 +283,109 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
             for (int j = 0; j < 4; ++j) qop[nb][j] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(qp + 8 * j));
         }
         const float cq = a.scale_log2e;
-        const int nsteps = qw_last / kPStep + 1;
+        const int nsteps = wg_qlast / kPStep + 1;
         const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const int64_t rstride = (int64_t)a.Hkv * kPD;  // elements between consecutive tokens
-        auto load_new = [&](NewStage &st, int step) {
+        // producer roles: wavefronts 0-3: K tile u = wave/2, k-groups 2*(wave&1), +1 (bf16 rows are operands as
+        // they are); wavefronts 4-7: V^T, token group wave-4, columns 2x, 2x+1 (x = lane/16) of this lane's 8.
+        u32x4 rawk[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+        uint32_t rawv[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+        auto issue = [&](int step) {
             const int t0 = step * kPStep;
+            if (wave < 4) {
+                const uint16_t *p = knb + (int64_t)min(t0 + 16 * (wave >> 1) + li, S - 1) * rstride + 32 * lq + 16 * (wave & 1);
+                rawk[0] = *(const u32x4 *)p;
+                rawk[1] = *(const u32x4 *)(p + 8);
+            } else {
+                const int g4 = wave - 4;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    rawv[e] = *(const uint32_t *)(vnb + (int64_t)min(t0 + 16 * (e >> 2) + 4 * g4 + (e & 3), S - 1) * rstride + 8 * li + 2 * lq);
+            }
+        };
+        auto commit = [&](StepTile &t) {
+            if (wave < 4) {
+                const int blk = 4 * (wave >> 1) + 2 * (wave & 1);
+                *(u32x4 *)(t.k[blk] + obase) = rawk[0];
+                *(u32x4 *)(t.k[blk + 1] + obase) = rawk[1];
+            } else {
+                const int dst = (li + 16 * (wave - 4)) * 16;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    const u32x4 w = {pick_halves(rawv[0], rawv[1], i), pick_halves(rawv[2], rawv[3], i),
+                                     pick_halves(rawv[4], rawv[5], i), pick_halves(rawv[6], rawv[7], i)};
+                    *(u32x4 *)(t.v[2 * lq + i] + dst) = w;
+                }
+            }
+        };
+        auto consume = [&](const StepTile &t, int step) {
+            const int t0 = step * kPStep;
+            float4v s[kNB][2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
-                const uint16_t *p = knb + (int64_t)min(t0 + 16 * u + li, S - 1) * rstride + 32 * lq;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) st.k[u][j] = *(const u32x4 *)(p + 8 * j);
+                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const bf16x8 ak = *(const bf16x8 *)(t.k[4 * u + j] + obase);
+#pragma unroll
+                    for (int nb = 0; nb < kNB; ++nb)
+                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, qop[nb][j], s[nb][u], 0, 0, 0);
+                }
             }
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int r = 0; r < 4; ++r)
-                    st.v[4 * u + r] = *(const u32x4 *)(vnb + (int64_t)min(t0 + 16 * u + 4 * lq + r, S - 1) * rstride + 8 * li);
-        };
-        NewStage st;
-        load_new(st, 0);
-        for (int step = 0; step < nsteps; ++step) {
-            const int t0 = step * kPStep;
-            bf16x8 av[8], ak[2][4];
-#pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
-                av[bb] = pack_bf16x8(pick_halves(st.v[0][bb >> 1], st.v[1][bb >> 1], bb & 1),
-                                     pick_halves(st.v[2][bb >> 1], st.v[3][bb >> 1], bb & 1),
-                                     pick_halves(st.v[4][bb >> 1], st.v[5][bb >> 1], bb & 1),
-                                     pick_halves(st.v[6][bb >> 1], st.v[7][bb >> 1], bb & 1));
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) ak[u][j] = __builtin_bit_cast(bf16x8, st.k[u][j]);
-            if (step + 1 < nsteps) load_new(st, step + 1);
-            const float pv[8] = {kPPScale, kPPScale, kPPScale, kPPScale, kPPScale, kPPScale, kPPScale, kPPScale};
+            const bool diag = t0 + kPStep - 1 > wv_q0;  // some (key, query) pair of this step is in the future
             float sc[kNB][8], mx[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                float4v s[2];
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    s[u] = (float4v){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) s[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak[u][j], qop[nb][j], s[u], 0, 0, 0);
-                }
-                const int qlim = min(qi[nb], S - 1);
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        sc[nb][4 * u + r] = (t0 + 16 * u + 4 * lq + r <= qlim) ? s[u][r] * cq : -INFINITY;
+                    for (int r = 0; r < 4; ++r) sc[nb][4 * u + r] = s[nb][u][r] * cq;
+                if (diag) {
+                    const int qlim = min(qi[nb], S - 1);
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (t0 + 16 * u + 4 * lq + r > qlim) sc[nb][4 * u + r] = -INFINITY;
+                }
                 float m = sc[nb][0];
 #pragma unroll
                 for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[nb][i]);
                 mx[nb] = quad_max(m);
             }
             raise_max(mx);
+            bf16x8 pop[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
+                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb];
                 float p[8];
-                weights(nb, sc[nb], pv, p);
-                const bf16x8 pop = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]),
-                                               pack_bf16x2(p[6], p[7]));
 #pragma unroll
-                for (int bb = 0; bb < 8; ++bb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[bb], pop, acc[nb][bb], 0, 0, 0);
+                for (int i = 0; i < 8; ++i) {
+                    const float e = __builtin_amdgcn_exp2f(sc[nb][i] - mref);
+                    l_run[nb] += e;
+                    p[i] = e * kPPScale;
+                }
+                pop[nb] = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
             }
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb) {
+                const bf16x8 av = *(const bf16x8 *)(t.v[bb] + obase);
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb)
+                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pop[nb], acc[nb][bb], 0, 0, 0);
+            }
+        };
+        issue(0);
+        commit(tiles[0]);
+        if (nsteps > 1) issue(1);
+        __syncthreads();
+        for (int step = 0; step < nsteps; ++step) {
+            if (step + 1 < nsteps) commit(tiles[(step + 1) & 1]);
+            if (step + 2 < nsteps) issue(step + 2);
+            if (wv_active && step * kPStep <= wv_qlast) consume(tiles[step & 1], step);
+            __syncthreads();
         }
     }
 
@@ -335,8 +400,7 @@ __global__ __launch_bounds__(256, 1) void prefill_attn_kernel(PrefillArgs a) {
         for (int r = 0; r < 4; ++r) {
             u32x4 w;
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                w[e] = pack_bf16x2(acc[nb][2 * e][r] * inv, acc[nb][2 * e + 1][r] * inv);
+            for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(acc[nb][2 * e][r] * inv, acc[nb][2 * e + 1][r] * inv);
             *(u32x4 *)(op + 8 * r) = w;
         }
     }
@@ -376,13 +440,11 @@ extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void
     a.ka = make_addr(*layout, 0); a.va = make_addr(*layout, 1);
     a.out = (uint16_t *)out;
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
-    constexpr int NB = HS_PREFILL_NB;
-    a.HW = G >= NB ? NB : G;
-    a.QT = NB / a.HW;
+    a.HG = G >= 4 ? 4 : G;
     a.scale_log2e = softmax_scale * kPLog2e;
-    const int q_per_wg = 64 * a.QT;
-    dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * (G / a.HW), B);
-    prefill_attn_kernel<NB><<<grid, 256, 0, st>>>(a);
+    const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
+    dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * (G / a.HG), B);
+    prefill_attn_kernel<<<grid, 512, 0, st>>>(a);
     if (int rc = check_launch("prefill_attn")) return rc;
     if (quantize_on_write)
         return hs_kv_quantize_int8(k_new, v_new, HS_BF16, k_codes, v_codes, k_scales, v_scales, layout, nullptr,
