@@ -7,8 +7,9 @@
 // column c = l % NC of rows [rg*RPL, (rg+1)*RPL) with rg = l / NC, RPL = 128*NC/64 rows in registers.
 // The two contractions over dk are per-lane partial sums plus a butterfly over the 64/NC lanes that
 // share a column; nothing goes through LDS and wavefronts never synchronise with each other.
-//   T == 1 (decode): NC = 32 -> each lane streams 64 rows, 128-byte row segments; the kernel is a
-//          single read and a single write of the state: HBM bound, 2*dk*dv*4 bytes per (sequence, head).
+//   T == 1 (decode): deltanet_decode_kernel, a 32-column slice per wavefront read and written with
+//          16-byte accesses; a single read and a single write of the state: HBM bound,
+//          2*dk*dv*4 bytes per (sequence, head).
 //   T  > 1 (prefill): NC = 8 -> 16 state registers per lane and 16x more wavefronts; tokens are
 //          processed in order with the next token's q/k/v/g/beta already in flight.
 // q and k arrive in bf16; with l2norm they are normalised as x / max(||x||, 1e-3) in fp32.
@@ -124,6 +125,82 @@ __global__ __launch_bounds__(256) void deltanet_kernel(DeltaArgs a) {
     for (int r = 0; r < RPL; ++r) sp[(int64_t)r * kDV] = S[r];
 }
 
+// Decode step (T == 1), tuned for HBM streaming: one wavefront owns 32 columns x 128 rows; lane l holds
+// columns 4*(l%8) .. +3 (one 16-byte access per row) of rows [16*(l/8), +16): every load and store
+// instruction of the wavefront moves eight full 128-byte row segments.
+__global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const int lane = threadIdx.x & 63;
+    const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t nw = (int64_t)a.B * a.nv * 4;
+    if (wid >= nw) return;
+    const int slice = (int)(wid & 3);
+    const int j = (int)((wid >> 2) % a.nv);
+    const int b = (int)((wid >> 2) / a.nv);
+    const int hk = j / (a.nv / a.nk);
+    const int c4 = lane & 7, rg = lane >> 3;
+    const int col = slice * 32 + 4 * c4;
+    float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + rg * 16) * kDV + col;
+    f4 S[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) S[r] = *(const f4 *)(sp + (int64_t)r * kDV);
+
+    const int64_t bt = b;  // T == 1
+    const uint16_t *kp = a.k + (bt * a.nk + hk) * kDK + rg * 16;
+    const uint16_t *qp = a.q + (bt * a.nk + hk) * kDK + rg * 16;
+    float kf[16], qf[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t kw = ((const uint32_t *)kp)[i], qw = ((const uint32_t *)qp)[i];
+        kf[2 * i] = __uint_as_float(kw << 16);
+        kf[2 * i + 1] = __uint_as_float(kw & 0xffff0000u);
+        qf[2 * i] = __uint_as_float(qw << 16);
+        qf[2 * i + 1] = __uint_as_float(qw & 0xffff0000u);
+    }
+    const uint32_t v01 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col);
+    const uint32_t v23 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col + 2);
+    const f4 v = {__uint_as_float(v01 << 16), __uint_as_float(v01 & 0xffff0000u), __uint_as_float(v23 << 16),
+                  __uint_as_float(v23 & 0xffff0000u)};
+    const float g = a.g[bt * a.nv + j], beta = a.beta[bt * a.nv + j];
+    auto rows_sum = [](float x) {  // over the 8 row groups: lanes with equal l % 8
+        x += __shfl_xor(x, 8, 64);
+        x += __shfl_xor(x, 16, 64);
+        x += __shfl_xor(x, 32, 64);
+        return x;
+    };
+    float kmul = 1.0f, qmul = a.q_scale;
+    if (a.l2norm) {
+        float sk = 0.0f, sq = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            sk += kf[r] * kf[r];
+            sq += qf[r] * qf[r];
+        }
+        kmul = 1.0f / fmaxf(sqrtf(rows_sum(sk)), 1e-3f);
+        qmul = a.q_scale / fmaxf(sqrtf(rows_sum(sq)), 1e-3f);
+    }
+    const float decay = expf(g);
+    f4 m = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        kf[r] *= kmul;
+        m += kf[r] * S[r];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m[e] = rows_sum(m[e]) * decay;
+    const f4 delta = (v - m) * beta;
+    f4 o = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        S[r] = S[r] * decay + kf[r] * delta;
+        o += qf[r] * S[r];
+        *(f4 *)(sp + (int64_t)r * kDV) = S[r];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = rows_sum(o[e]) * qmul;
+    if (rg == 0) *(f4 *)(a.out + (bt * a.nv + j) * kDV + col) = o;
+}
+
 }  // namespace hs
 
 extern "C" int hs_deltanet_forward(const void *q, const void *k, const void *v, const float *g, const float *beta,
@@ -142,7 +219,7 @@ extern "C" int hs_deltanet_forward(const void *q, const void *k, const void *v, 
     hipStream_t st = (hipStream_t)stream;
     if (T == 1) {
         const int64_t waves = (int64_t)B * nv * (kDV / 32);
-        deltanet_kernel<32><<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(a);
+        deltanet_decode_kernel<<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(a);
     } else {
         const int64_t waves = (int64_t)B * nv * (kDV / 8);
         deltanet_kernel<8><<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(a);
