@@ -330,17 +330,28 @@ def main():
     step_bytes = (wl.decode_bytes_fp8 if fp8 else wl.decode_bytes_int8)(lens_h, Hq, Hkv, D)
     gbs = step_bytes / (ms_per_step * 1e-3) / 1e9
 
-    # ---- roofline of the dominant kernel (split-K decode attention) alone: HIP events on its stream
-    kern_bytes = step_bytes - (B * Hkv * D * (2 * 2 + 2 * 1) + (0 if fp8 else B * Hkv * 2 * 4))  # minus the write kernel's share
+    # ---- roofline of the dominant kernel alone: HIP events (torch's, recorded on the stream the library
+    # launches on) around each launch.  When every sequence is one chunk the whole step IS that one launch
+    # (new-token write + attention + output); otherwise the split-K kernel is timed without the merge.
+    per_chunk = B * Hq * (D + 2) * 4
+    nchunks = max(1, ws.numel() // per_chunk)  # the workspace is nchunks partial records, rounded up to 256 B
+    single = nchunks == 1
+    write_bytes = B * Hkv * D * (2 * 2 + 2 * 1) + (0 if fp8 else B * Hkv * 2 * 4)
+    kern_bytes = step_bytes if single else step_bytes - write_bytes
     n_ev = min(args.steps, 100)
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
     for i in range(n_ev):
         kc, vc, ks, vs = caches[i % ncopies]
-        quant(k_new, v_new, kc, vc, ks, vs, layout, pos, 0)
-        evs[i][0].record()
-        hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=1)
-        evs[i][1].record()
-        hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=2)
+        if single:
+            evs[i][0].record()
+            hb.decode_step(q, k_new, v_new, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8)
+            evs[i][1].record()
+        else:
+            quant(k_new, v_new, kc, vc, ks, vs, layout, pos, 0)
+            evs[i][0].record()
+            hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=1)
+            evs[i][1].record()
+            hb.decode_attn(q, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8, phases=2)
     torch.cuda.synchronize()
     kt = np.array([a.elapsed_time(b) for a, b in evs])  # ms
     k_avg_ms = float(kt.mean())
