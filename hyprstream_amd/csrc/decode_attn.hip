@@ -97,54 +97,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         __syncthreads();  // codes and scales are visible to the whole workgroup before any load
     }
 
-    // ---- Q operand: lane (head li, quarter lq) holds Q[head][32*lq + 8*j + e] for MFMA j.
     half8 qop[4];
     float cq = 0.0f, cinit = 0.0f;
-    {
-        float qf[32];
-        float amax = 0.0f;
-        if (li < G) {
-            const uint16_t *qp = a.q + ((int64_t)b * a.Hq + h * G + li) * kD + 32 * lq;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                u32x4 w = *(const u32x4 *)(qp + 8 * i);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16);
-                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
-        } else {
-#pragma unroll
-            for (int i = 0; i < 32; ++i) qf[i] = 0.0f;
-        }
-        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-        int ex = 0;
-        if (amax > 0.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
-        float qsum = 0.0f;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                _Float16 hq = (_Float16)ldexpf(qf[8 * j + e], -ex);
-                qop[j][e] = hq;
-                qsum += (float)hq;
-            }
-        }
-        qsum += __shfl_xor(qsum, 16, 64);
-        qsum += __shfl_xor(qsum, 32, 64);
-        if (li < G) {
-            cq = ldexpf(a.scale_log2e, ex);
-            if (FP8) {
-                cq *= 256.0f * a.ks[(int64_t)b * a.Hkv + h];  // 2^8 rebias of the fp16 view of e4m3
-            } else {
-                cinit = -1152.0f * qsum;
-            }
-        }
-    }
     // fp8: the V scale is one constant per (sequence, head); it multiplies the finished partial.
     const float out_scale = (1.0f / kPScale) * (FP8 ? 256.0f * a.vs[(int64_t)b * a.Hkv + h] : 1.0f);
 
@@ -285,6 +239,54 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     Stage<FP8> sa, sb;
     int step = wave;
     if (step < nsteps) load_stage(sa, step);
+    // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds Q[head][32*lq + 8*j + e] for MFMA j.
+    {
+        float qf[32];
+        float amax = 0.0f;
+        if (li < G) {
+            const uint16_t *qp = a.q + ((int64_t)b * a.Hq + h * G + li) * kD + 32 * lq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                u32x4 w = *(const u32x4 *)(qp + 8 * i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16);
+                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) qf[i] = 0.0f;
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        // amax = f * 2^ex with f in [0.5, 1); scaling by 2^-ex is exact (a multiplication by a power of two)
+        int ex = 0;
+        if (amax > 0.0f && amax < 3.0e38f) ex = min(126, max(-125, (int)((__float_as_uint(amax) >> 23) & 0xff) - 126));
+        const float down = __uint_as_float((uint32_t)(127 - ex) << 23), up = __uint_as_float((uint32_t)(127 + ex) << 23);
+        float qsum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                _Float16 hq = (_Float16)(qf[8 * j + e] * down);
+                qop[j][e] = hq;
+                qsum += (float)hq;
+            }
+        }
+        qsum += __shfl_xor(qsum, 16, 64);
+        qsum += __shfl_xor(qsum, 32, 64);
+        if (li < G) {
+            cq = a.scale_log2e * up;
+            if (FP8) {
+                cq *= 256.0f * a.ks[(int64_t)b * a.Hkv + h];  // 2^8 rebias of the fp16 view of e4m3
+            } else {
+                cinit = -1152.0f * qsum;
+            }
+        }
+    }
     while (step < nsteps) {
         const int n1 = step + kWavesPerWg;
         if (n1 < nsteps) load_stage(sb, n1);
