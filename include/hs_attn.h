@@ -151,12 +151,12 @@ HS_API int hs_decode_step_fp8(const void *q, const void *k_new, const void *v_ne
                               int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
                               float softmax_scale, hs_stream_t stream);
 
-/* The two phases of decode attention on their own: phases = 1 runs only the split-K kernel that
- * leaves per-chunk partials (m, l, o) in the workspace, 2 only a stand-alone merge of those
- * partials into `out`, 3 is identical to the calls above (there the last workgroup to finish a
- * (sequence, kv-head) merges its partials itself).  No counterpart in the reference; it exists so that
- * the phases can be timed separately and so that partials produced for different token ranges
- * (for instance on different devices) can share one merge. */
+/* The two phases of split-K decode attention on their own: phases = 1 runs only the attention kernel
+ * and leaves per-chunk partials (m, l, o) in the workspace, 2 only the merge of those partials into
+ * `out`, 3 is identical to the calls above (which skip the workspace altogether when a sequence is a
+ * single chunk).  No counterpart in the reference; it exists so that the phases can be timed
+ * separately and so that partials produced for different token ranges (for instance on different
+ * devices) can share one merge. */
 HS_API int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const void *k_codes, const void *v_codes,
                                  const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
                                  const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,

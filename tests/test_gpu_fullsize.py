@@ -1,0 +1,200 @@
+"""GPU parity at the benchmark configurations' FULL sizes.
+
+The oracle cannot redo these sizes in seconds, so each test checks (a) a sample of (sequence, head) units or
+query rows against the oracle, bit-exact for codes and within the path's tolerance for attention, and
+(b) size-independent properties: constant V gives constant output, split-K equals unsplit, chunked equals
+carried state.  Inputs are generated on the device from the seed."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from hyprstream_amd import bindings as hb
+from hyprstream_amd import workloads as wl
+from gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+TOL_MAX, TOL_MEAN = 2e-2, 2e-3
+
+
+def gen(seed):
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    return g
+
+
+def source(g, shape, sigma=1.0, outliers=False):
+    x = torch.randn(shape, generator=g, device=DEV) * sigma
+    if outliers:
+        m = torch.rand(shape, generator=g, device=DEV) < 0.01
+        x = torch.where(m, torch.sign(x) * 8.0 * sigma, x)
+    return x.to(torch.bfloat16)
+
+
+def fill_cache(g, B, Hkv, T, D, fp8, sigma, outliers, keep=()):
+    """Quantize-on-write of T tokens per sequence, one sequence at a time; returns buffers and the bf16
+    sources of the sequences listed in `keep`."""
+    lay = hb.contiguous_layout(Hkv, T, D)
+    cdt = torch.uint8 if fp8 else torch.int8
+    kc = torch.empty(B, Hkv, T, D, dtype=cdt, device=DEV)
+    vc = torch.empty_like(kc)
+    if fp8:
+        ks = torch.empty(B, Hkv, dtype=torch.float32, device=DEV)
+    else:
+        ks = torch.empty(B, Hkv, lay.scale_stride_head, dtype=torch.float32, device=DEV)
+    vs = torch.empty_like(ks)
+    kept = {}
+    for b in range(B):
+        k, v = source(g, (1, T, Hkv, D), sigma, outliers), source(g, (1, T, Hkv, D), sigma, outliers)
+        if fp8:
+            hb.kv_fp8_calibrate(k, v, ks[b:b + 1], vs[b:b + 1])
+            hb.kv_quantize_fp8(k, v, kc[b:b + 1], vc[b:b + 1], ks[b:b + 1], vs[b:b + 1], lay, None, 0)
+        else:
+            hb.kv_quantize_int8(k, v, kc[b:b + 1], vc[b:b + 1], ks[b:b + 1], vs[b:b + 1], lay, None, 0)
+        if b in keep:
+            kept[b] = (k.float().cpu().numpy(), v.float().cpu().numpy())
+    torch.cuda.synchronize()
+    return lay, kc, vc, ks, vs, kept
+
+
+def decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, fp8, phases=3):
+    B, Hq, D = q.shape
+    out = torch.full((B, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    for ph in ([1, 2] if phases == 12 else [3]):
+        hb.decode_attn(q, kc, vc, ks, vs, lay, lens, out, ws, Hkv, T, 1.0 / np.sqrt(D), fp8=fp8, phases=ph)
+    torch.cuda.synchronize()
+    return out
+
+
+def sample_check(out, q, kc, vc, ks, vs, lens, units, G, fp8):
+    for b, h in units:
+        n = int(lens[b])
+        kcb = kc[b, h, :n].cpu().numpy()[None, :, None, :]
+        vcb = vc[b, h, :n].cpu().numpy()[None, :, None, :]
+        if fp8:
+            ksb, vsb = ks[b, h].cpu().numpy().reshape(1, 1), vs[b, h].cpu().numpy().reshape(1, 1)
+        else:
+            ksb, vsb = ks[b, h, :n].cpu().numpy()[None, :, None], vs[b, h, :n].cpu().numpy()[None, :, None]
+        qb = q[b, h * G:(h + 1) * G].float().cpu().numpy()[None]
+        want = oracle.decode_attn(qb, kcb, vcb, ksb, vsb, oracle.FMT_FP8 if fp8 else oracle.FMT_INT8,
+                                  np.array([n], np.int32), 1.0 / np.sqrt(q.shape[-1]))[0]
+        d = np.abs(out[b, h * G:(h + 1) * G].float().cpu().numpy() - want)
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, d.max(), d.mean())
+
+
+def test_config2_full_size_int8_decode():
+    """B=64, Hq 32 / Hkv 8, D 128, T 8192 (headline) and ragged lengths U[512, 8192]."""
+    B, Hq, Hkv, D, T = 64, 32, 8, 128, 8192
+    g = gen(wl.SEED)
+    lay, kc, vc, ks, vs, kept = fill_cache(g, B, Hkv, T, D, False, 1.0, True, keep=(0, 63))
+    for b, (k, v) in kept.items():  # codes written at full size are the oracle's, bit for bit
+        wk, wks = oracle.quant_int8(k[:, :, 3])
+        assert np.array_equal(kc[b, 3].cpu().numpy(), wk[0]) and np.array_equal(ks[b, 3, :T].cpu().numpy(), wks[0])
+    q = torch.randn(B, Hq, D, generator=g, device=DEV).to(torch.bfloat16)
+    full = torch.full((B,), T, dtype=torch.int32, device=DEV)
+    out = decode(q, kc, vc, ks, vs, lay, full, Hkv, T, False)
+    assert torch.isfinite(out.float()).all()
+    sample_check(out, q, kc, vc, ks, vs, full.cpu().numpy(), [(0, 0), (17, 5), (63, 7)], 4, False)
+    two = decode(q, kc, vc, ks, vs, lay, full, Hkv, T, False, phases=12)  # partials + stand-alone merge
+    assert (two.float() - out.float()).abs().max() <= 2 ** -8 * max(1.0, float(out.float().abs().max()))
+    lens = torch.randint(512, T + 1, (B,), generator=g, device=DEV, dtype=torch.int32)
+    rag = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    sample_check(rag, q, kc, vc, ks, vs, lens.cpu().numpy(), [(1, 2), (40, 6)], 4, False)
+    vc.fill_(64)
+    vs.fill_(0.125)
+    const = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    assert (const.float() - 8.0).abs().max() <= 2 ** -5  # weights sum to one at every length
+
+
+def test_config4_full_size_fp8_decode():
+    """B=32, Hq 64 / Hkv 8, D 128, T 32768, e4m3 cache with per-(sequence, head) scales."""
+    B, Hq, Hkv, D, T = 32, 64, 8, 128, 32768
+    g = gen(wl.SEED + 4)
+    lay, kc, vc, ks, vs, kept = fill_cache(g, B, Hkv, T, D, True, 0.5, False, keep=(5,))
+    k, v = kept[5]
+    sk = oracle.fp8_calibrate(k)
+    assert np.array_equal(sk[0], ks[5].cpu().numpy())
+    assert np.array_equal(oracle.quant_fp8(k[:, :4096], sk)[0, :, 2], kc[5, 2, :4096].cpu().numpy())
+    q = torch.randn(B, Hq, D, generator=g, device=DEV).to(torch.bfloat16)
+    full = torch.full((B,), T, dtype=torch.int32, device=DEV)
+    out = decode(q, kc, vc, ks, vs, lay, full, Hkv, T, True)
+    assert torch.isfinite(out.float()).all()
+    sample_check(out, q, kc, vc, ks, vs, full.cpu().numpy(), [(0, 0), (31, 7)], 8, True)
+
+
+def test_config3_full_size_chunked_prefill():
+    """B=4 x 4096 tokens in 512-token chunks: sampled query rows of every chunk against the oracle over
+    [dequantized int8 cache of earlier chunks | own bf16 K/V]; the cache ends up equal to one-shot quantization."""
+    B, T, C, Hq, Hkv, D = 4, 4096, 512, 32, 8, 128
+    g = gen(wl.SEED + 3)
+    q, k, v = source(g, (B, T, Hq, D)), source(g, (B, T, Hkv, D)), source(g, (B, T, Hkv, D))
+    lay = hb.contiguous_layout(Hkv, T, D)
+    kc = torch.zeros(B, Hkv, T, D, dtype=torch.int8, device=DEV)
+    vc = torch.zeros_like(kc)
+    ks = torch.zeros(B, Hkv, lay.scale_stride_head, dtype=torch.float32, device=DEV)
+    vs = torch.zeros_like(ks)
+    outs = []
+    for i in range(0, T, C):
+        o = torch.empty(B, C, Hq, D, dtype=torch.bfloat16, device=DEV)
+        hb.prefill_attn(q[:, i:i + C].contiguous(), k[:, i:i + C].contiguous(), v[:, i:i + C].contiguous(), kc, vc, ks, vs,
+                        lay, i, o, 1.0 / np.sqrt(D), True)
+        outs.append(o)
+    torch.cuda.synchronize()
+    out = torch.cat(outs, 1)
+    assert torch.isfinite(out.float()).all()
+    r = wl.philox(33)
+    for _ in range(6):
+        b, h, pos = int(r.integers(B)), int(r.integers(Hkv)), int(r.integers(T))
+        c0 = pos // C * C  # start of the chunk this row belongs to
+        kd = torch.cat([kc[b, h, :c0].float() * ks[b, h, :c0, None], k[b, c0:pos + 1, h].float()]).cpu().numpy()
+        vd = torch.cat([vc[b, h, :c0].float() * vs[b, h, :c0, None], v[b, c0:pos + 1, h].float()]).cpu().numpy()
+        qb = q[b, pos, 4 * h:4 * h + 4].float().cpu().numpy()[None]
+        want = oracle.decode_attn(qb, kd[None, :, None], vd[None, :, None], None, None, oracle.FMT_DENSE,
+                                  np.array([pos + 1], np.int32), 1.0 / np.sqrt(D))[0]
+        d = np.abs(out[b, pos, 4 * h:4 * h + 4].float().cpu().numpy() - want)
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, pos, d.max(), d.mean())
+    wk, wks = oracle.quant_int8(k[1, :, 5].float().cpu().numpy())
+    assert np.array_equal(kc[1, 5].cpu().numpy(), wk) and np.array_equal(ks[1, 5, :T].cpu().numpy(), wks)
+
+
+def test_config5_full_size_deltanet():
+    """Decode at B = 64 (whole batch against the oracle) and prefill at B = 4 x 4096 (two sampled heads against
+    the oracle, and chunked calls with carried state against the single call)."""
+    nk, nv, d = 16, 32, 128
+    g = gen(wl.SEED + 5)
+    nrm = lambda x: (x / x.norm(dim=-1, keepdim=True).clamp_min(1e-3)).to(torch.bfloat16)
+    B = 64
+    q, k = nrm(torch.randn(B, 1, nk, d, generator=g, device=DEV)), nrm(torch.randn(B, 1, nk, d, generator=g, device=DEV))
+    v = torch.randn(B, 1, nv, d, generator=g, device=DEV).to(torch.bfloat16)
+    gg = -torch.nn.functional.softplus(torch.randn(B, 1, nv, generator=g, device=DEV))
+    beta = torch.sigmoid(torch.randn(B, 1, nv, generator=g, device=DEV))
+    s0 = torch.randn(B, nv, d, d, generator=g, device=DEV) * 0.1
+    st, out = s0.clone(), torch.empty(B, 1, nv, d, device=DEV)
+    hb.deltanet_forward(q, k, v, gg, beta, st, out, 1 / np.sqrt(d), False)
+    torch.cuda.synchronize()
+    wo, ws = oracle.deltanet_recurrent(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(),
+                                       gg.cpu().numpy(), beta.cpu().numpy(), s0.cpu().numpy(), 1 / np.sqrt(d), False)
+    assert np.abs(out.cpu().numpy() - wo).max() < 1e-5 and np.abs(st.cpu().numpy() - ws).max() < 1e-5
+    B, T = 4, 4096
+    q, k = nrm(torch.randn(B, T, nk, d, generator=g, device=DEV)), nrm(torch.randn(B, T, nk, d, generator=g, device=DEV))
+    v = torch.randn(B, T, nv, d, generator=g, device=DEV).to(torch.bfloat16)
+    gg = -torch.nn.functional.softplus(torch.randn(B, T, nv, generator=g, device=DEV))
+    beta = torch.sigmoid(torch.randn(B, T, nv, generator=g, device=DEV))
+    st, out = torch.zeros(B, nv, d, d, device=DEV), torch.empty(B, T, nv, d, device=DEV)
+    hb.deltanet_forward(q, k, v, gg, beta, st, out, 1 / np.sqrt(d), False)
+    st2, out2 = torch.zeros(B, nv, d, d, device=DEV), torch.empty(B, T, nv, d, device=DEV)
+    for i in range(0, T, 1024):  # four calls carrying the state
+        o = torch.empty(B, 1024, nv, d, device=DEV)
+        hb.deltanet_forward(q[:, i:i + 1024].contiguous(), k[:, i:i + 1024].contiguous(), v[:, i:i + 1024].contiguous(),
+                            gg[:, i:i + 1024].contiguous(), beta[:, i:i + 1024].contiguous(), st2, o, 1 / np.sqrt(d), False)
+        out2[:, i:i + 1024] = o
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2) and torch.equal(st, st2)
+    for b, j in ((0, 0), (3, 31)):  # v-head j reads k-head j // 2
+        hk = j // 2
+        wo, ws = oracle.deltanet_recurrent(q[b:b + 1, :, hk:hk + 1].float().cpu().numpy(), k[b:b + 1, :, hk:hk + 1].float().cpu().numpy(),
+                                           v[b:b + 1, :, j:j + 1].float().cpu().numpy(), gg[b:b + 1, :, j:j + 1].cpu().numpy(),
+                                           beta[b:b + 1, :, j:j + 1].cpu().numpy(), None, 1 / np.sqrt(d), False)
+        assert np.abs(out[b, :, j].cpu().numpy() - wo[0, :, 0]).max() < 1e-4
+        assert np.abs(st[b, j].cpu().numpy() - ws[0, 0]).max() < 1e-4

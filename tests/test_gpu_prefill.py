@@ -143,3 +143,37 @@ def test_overflow_is_an_error():
     with pytest.raises(hb.HsError) as e:
         gpu_prefill(c, q, k, v, 4)
     assert e.value.code == hb.HS_ERR_OVERFLOW
+
+
+def test_paged_history_matches_contiguous():
+    """History in 64-token blocks scattered through one pool (K and V blocks interleaved): prefill over it,
+    its quantize-on-write into the pool, and the dense view must equal the contiguous-cache results."""
+    B, Hq, Hkv, D, hist, S, BT = 2, 8, 2, 128, 150, 70, 64
+    qh, kh, vh = make(100, B, hist, Hq, Hkv)
+    q, k, v = make(101, B, S, Hq, Hkv)
+    c = DeviceCache(B, Hkv, hist + S, D)
+    hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+    c.write(hk, hv, None, 0)
+    want = gpu_prefill(c, q, k, v, hist)
+    nblk = (hist + S + BT - 1) // BT
+    ids = wl.philox(102).permutation(2 * B * nblk + 3).astype(np.int32)
+    kt, vt = ids[:B * nblk].reshape(B, nblk), ids[B * nblk:2 * B * nblk].reshape(B, nblk)
+    pool_c = torch.zeros(len(ids), Hkv, BT, D, dtype=torch.int8, device=DEV)
+    pool_s = torch.zeros(len(ids), Hkv, BT, dtype=torch.float32, device=DEV)
+    k_tab, v_tab = torch.from_numpy(kt).to(DEV), torch.from_numpy(vt).to(DEV)
+    lay = hb.paged_layout(Hkv, BT, D, k_tab, v_tab)
+    hb.kv_quantize_int8(hk, hv, pool_c, pool_c, pool_s, pool_s, lay, None, 0)
+    qt, knew, vnew = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
+    out = torch.empty(B, S, Hq, D, dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(qt, knew, vnew, pool_c, pool_c, pool_s, pool_s, lay, hist, out, 1.0 / np.sqrt(D), True)
+    dense_k = torch.empty(B, hist + S, Hkv, D, dtype=torch.float32, device=DEV)
+    dense_v = torch.empty_like(dense_k)
+    hb.kv_dequantize(pool_c, pool_s, False, lay, 0, dense_k)
+    hb.kv_dequantize(pool_c, pool_s, False, lay, 1, dense_v)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    ck, cv = torch.empty_like(dense_k), torch.empty_like(dense_v)
+    hb.kv_dequantize(c.k_codes, c.k_scales, False, c.layout, 0, ck)
+    hb.kv_dequantize(c.v_codes, c.v_scales, False, c.layout, 1, cv)
+    torch.cuda.synchronize()
+    assert torch.equal(dense_k, ck) and torch.equal(dense_v, cv)
