@@ -55,12 +55,27 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     __shared__ StepTile tiles[2];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lq = lane >> 4;
-    const int b = blockIdx.z;
+    // XCD-aware placement.  Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has
+    // its own L2.  All query tiles that read the same (sequence, kv-head) K/V stream are therefore given
+    // linear ids that are congruent mod 8, so the stream is fetched into ONE L2 and shared there instead of
+    // being pulled into all eight.
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+    {
+        const int X = gridDim.x, YZ = gridDim.y * gridDim.z;
+        if ((YZ & 7) == 0) {
+            const int p = bx + X * (by + gridDim.y * bz);  // dispatch order
+            const int grp = (p & 7) + 8 * (p / (8 * X));   // (kv-head group, sequence) unit
+            bx = (p >> 3) % X;
+            by = grp % gridDim.y;
+            bz = grp / gridDim.y;
+        }
+    }
+    const int b = bz;
     const int groups = a.G / a.HG;
-    const int kvh = blockIdx.y / groups, hg = blockIdx.y % groups;
+    const int kvh = by / groups, hg = by % groups;
     const int S = a.S, H = a.hist_len;
     const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
-    const int q0 = blockIdx.x * q_per_wg;
+    const int q0 = bx * q_per_wg;
     if (q0 >= S) return;
     const int wg_qlast = min(S - 1, q0 + q_per_wg - 1);
 
