@@ -12,6 +12,9 @@
 // ends at the sequence end quantizes that token's K and V rows (one wavefront each), stores codes
 // and scales, and only then starts streaming, so the token it reads back is the one it wrote.
 //
+// Cache codes and scales are read exactly once per launch, so they are loaded with the non-temporal
+// hint (streamed past the caches instead of displacing lines): measured 192 -> 181 us at B=64 x 8192.
+//
 // Arithmetic.  Both products run on the MFMA pipe (v_mfma_f32_16x16x32_f16) with the G query
 // heads on the N axis (padded to 16):
 //   S[t, g]  = sum_d K[t, d] Q[g, d]          A = K codes, 16 tokens x 32 d per issue
@@ -122,15 +125,15 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         for (int u = 0; u < 2; ++u) {
             const int row = min(16 * u + li, last);
             const uint8_t *p = kb + row * kD + 32 * lq;
-            st.k[u][0] = *(const u32x4 *)p;
-            st.k[u][1] = *(const u32x4 *)(p + 16);
+            st.k[u][0] = __builtin_nontemporal_load((const u32x4 *)p);
+            st.k[u][1] = __builtin_nontemporal_load((const u32x4 *)(p + 16));
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = min(16 * u + 4 * lq + r, last);
-                st.v[4 * u + r] = *(const u32x2 *)(vb + row * kD + 8 * li);
+                st.v[4 * u + r] = __builtin_nontemporal_load((const u32x2 *)(vb + row * kD + 8 * li));
             }
         if (!FP8) {
             const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)h * a.ka.scale_stride_head + kslot;
@@ -138,8 +141,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const int tok = min(16 * u + 4 * lq, last & ~3);
-                st.sk[u] = *(const float4v *)(ksb + tok);
-                st.sv[u] = *(const float4v *)(vsb + tok);
+                st.sk[u] = __builtin_nontemporal_load((const float4v *)(ksb + tok));
+                st.sv[u] = __builtin_nontemporal_load((const float4v *)(vsb + tok));
             }
         }
     };

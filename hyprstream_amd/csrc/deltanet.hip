@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
     float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + rg * 16) * kDV + col;
     f4 S[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) S[r] = *(const f4 *)(sp + (int64_t)r * kDV);
+    for (int r = 0; r < 16; ++r) S[r] = __builtin_nontemporal_load((const f4 *)(sp + (int64_t)r * kDV));  // read once
 
     const int64_t bt = b;  // T == 1
     const uint16_t *kp = a.k + (bt * a.nk + hk) * kDK + rg * 16;
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
     for (int r = 0; r < 16; ++r) {
         S[r] = S[r] * decay + kf[r] * delta;
         o += qf[r] * S[r];
-        *(f4 *)(sp + (int64_t)r * kDV) = S[r];
+        __builtin_nontemporal_store(S[r], (f4 *)(sp + (int64_t)r * kDV));
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = rows_sum(o[e]) * qmul;
