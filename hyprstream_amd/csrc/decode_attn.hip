@@ -63,7 +63,7 @@ struct DecodeArgs {
 
 template <bool FP8>
 struct Stage {
-    u32x4 k[2][2];  // [16-token tile][16-byte half of this lane's 32 B of the row]
+    u32x4 k[2][2];  // [16-token tile][half of the row]: 16 B at byte 64*half + 16*lq of row li
     u32x2 v[8];     // [token slot e = 4u + r] 8 bytes: d = 8*(lane%16) .. +7
     float4v sk[2];  // K scales of tokens 16u + 4q + r   (int8 only)
     float4v sv[2];
@@ -124,9 +124,9 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int row = min(16 * u + li, last);
-            const uint8_t *p = kb + row * kD + 32 * lq;
+            const uint8_t *p = kb + row * kD + 16 * lq;  // each load covers one 64-byte half of 16 rows
             st.k[u][0] = __builtin_nontemporal_load((const u32x4 *)p);
-            st.k[u][1] = __builtin_nontemporal_load((const u32x4 *)(p + 16));
+            st.k[u][1] = __builtin_nontemporal_load((const u32x4 *)(p + 64));
         }
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -242,15 +242,16 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     Stage<FP8> sa, sb;
     int step = wave;
     if (step < nsteps) load_stage(sa, step);
-    // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds Q[head][32*lq + 8*j + e] for MFMA j.
+    // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds
+    //      Q[head][64*(j/2) + 16*lq + 8*(j%2) + e] for MFMA j.
     {
         float qf[32];
         float amax = 0.0f;
         if (li < G) {
-            const uint16_t *qp = a.q + ((int64_t)b * a.Hq + h * G + li) * kD + 32 * lq;
+            const uint16_t *qp = a.q + ((int64_t)b * a.Hq + h * G + li) * kD + 16 * lq;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                u32x4 w = *(const u32x4 *)(qp + 8 * i);
+            for (int i = 0; i < 4; ++i) {  // MFMA i contracts d = 64*(i/2) + 16*lq + 8*(i%2) + e, as the K loads do
+                u32x4 w = *(const u32x4 *)(qp + 64 * (i >> 1) + 8 * (i & 1));
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16);
