@@ -65,8 +65,7 @@ template <bool FP8>
 struct Stage {
     u32x4 k[2][2];  // [16-token tile][half of the row]: 16 B at byte 64*half + 16*lq of row li
     u32x2 v[8];     // [token slot e = 4u + r] 8 bytes: d = 8*(lane%16) .. +7
-    float4v sk[2];  // K scales of tokens 16u + 4q + r   (int8 only)
-    float4v sv[2];
+    float sraw;     // int8 only: lanes 0-31 hold the K scale of token `lane`, lanes 32-63 the V scale of token lane-32
 };
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -111,6 +110,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     float m_run = -INFINITY, l_run = 0.0f;
 
     const int nsteps = (t_end - t_begin + kStep - 1) / kStep;
+    __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64];
 
     auto load_stage = [&](Stage<FP8> &st, int step) {
         const int t0 = t_begin + step * kStep;
@@ -128,6 +128,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             st.k[u][0] = __builtin_nontemporal_load((const u32x4 *)p);
             st.k[u][1] = __builtin_nontemporal_load((const u32x4 *)(p + 64));
         }
+        if (!FP8) {
+            // one 4-byte load per lane brings the step's 32 K scales and 32 V scales (two full 128-byte lines);
+            // compute_stage hands them to the lanes that need them through LDS
+            const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)h * a.ka.scale_stride_head + kslot;
+            const float *vsb = a.vs + vu * a.va.scale_stride_seq + (int64_t)h * a.va.scale_stride_head + vslot;
+            st.sraw = __builtin_nontemporal_load((lane < 32 ? ksb : vsb) + min(lane & 31, last));
+        }
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -135,20 +142,22 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                 const int row = min(16 * u + 4 * lq + r, last);
                 st.v[4 * u + r] = __builtin_nontemporal_load((const u32x2 *)(vb + row * kD + 8 * li));
             }
-        if (!FP8) {
-            const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)h * a.ka.scale_stride_head + kslot;
-            const float *vsb = a.vs + vu * a.va.scale_stride_seq + (int64_t)h * a.va.scale_stride_head + vslot;
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const int tok = min(16 * u + 4 * lq, last & ~3);
-                st.sk[u] = __builtin_nontemporal_load((const float4v *)(ksb + tok));
-                st.sv[u] = __builtin_nontemporal_load((const float4v *)(vsb + tok));
-            }
-        }
     };
 
     auto compute_stage = [&](const Stage<FP8> &st, int step) {
         const int t0 = t_begin + step * kStep;
+        // ---- token scales: lane (li, lq) needs those of tokens 16u + 4*lq + r, the rows of its score registers.
+        //      LDS operations of one wavefront complete in order, so the reads see the write without a barrier.
+        float4v sk[2], sv[2];
+        if (!FP8) {
+            sm_sc[wave][lane] = st.sraw;
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                sk[u] = *(const float4v *)&sm_sc[wave][16 * u + 4 * lq];
+                sv[u] = *(const float4v *)&sm_sc[wave][32 + 16 * u + 4 * lq];
+            }
+        }
         // ---- scores: 2 tiles x 4 MFMAs (K of 128 split in 4 x 32)
         float4v s[2];
 #pragma unroll
@@ -179,8 +188,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                sc[4 * u + r] = FP8 ? s[u][r] * cq : s[u][r] * st.sk[u][r] * cq;
-                pv[4 * u + r] = FP8 ? kPScale : st.sv[u][r] * kPScale;
+                sc[4 * u + r] = FP8 ? s[u][r] * cq : s[u][r] * sk[u][r] * cq;
+                pv[4 * u + r] = FP8 ? kPScale : sv[u][r] * kPScale;
             }
         const bool tail = t0 + kStep > L;
         if (tail) {
