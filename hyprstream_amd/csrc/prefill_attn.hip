@@ -33,6 +33,7 @@ constexpr int kPWaves = 8;
 constexpr int kNB = 2;  // 16-column blocks per wavefront
 constexpr float kPLog2e = 1.4426950408889634f;
 constexpr float kPPScale = 64.0f;
+constexpr float kSlack = 4.0f;  // log2 units by which the softmax reference value overshoots a new maximum
 
 struct PrefillArgs {
     const uint16_t *q, *kn, *vn;  // [B,S,Hq,D], [B,S,Hkv,D], [B,S,Hkv,D] bf16
@@ -100,8 +101,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         for (int i = 0; i < 8; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
     }
 
-    // Online softmax: raise_max() takes the blocks' step maxima (already reduced over the column) and
-    // rescales under one wave-uniform branch that is rarely taken once the maxima settle.
+    // Online softmax: raise_max() takes the blocks' step maxima (already reduced over the column).  The
+    // reference value m_run is not the running maximum itself but an upper bound of it: when a column's
+    // maximum passes m_run, m_run is set kSlack above the new maximum, so that later small increases need no
+    // rescaling of the 64 accumulator registers.  Every weight is then exp2(s - m_run) <= 1, the largest at
+    // least 2^-kSlack; numerator and denominator carry the same factor, which cancels in the final division.
     auto raise_max = [&](const float (&mx)[kNB]) {
         bool changed = false;
 #pragma unroll
@@ -109,7 +113,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         if (__builtin_amdgcn_ballot_w64(changed) != 0) {
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                const float m_new = fmaxf(m_run[nb], mx[nb]);
+                const float m_new = mx[nb] > m_run[nb] ? mx[nb] + kSlack : m_run[nb];
                 const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
                 l_run[nb] *= alpha;
 #pragma unroll
