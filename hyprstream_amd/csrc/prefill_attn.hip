@@ -32,7 +32,7 @@ constexpr int kPStep = 32;
 constexpr int kPWaves = 8;
 constexpr int kNB = 2;  // 16-column blocks per wavefront
 constexpr float kPLog2e = 1.4426950408889634f;
-constexpr float kPPScale = 64.0f;
+constexpr float kPShift = 6.0f;  // weights are carried as 2^6 * exp2(s - m_run): keeps small ones out of the fp16 subnormals
 constexpr float kSlack = 4.0f;  // log2 units by which the softmax reference value overshoots a new maximum
 
 struct PrefillArgs {
@@ -48,13 +48,44 @@ struct PrefillArgs {
 struct alignas(16) StepTile {
     uint8_t k[8][1024];  // block 4*u + j: K tile u (16 keys), k-group j; 64 lanes x 16 B in MFMA lane order
     uint8_t v[8][1024];  // block bb: V^T rows d = 8*li + bb, 32 keys
-    float ksc[32];       // K scale of the step's tokens (0 for tokens past the end)
-    float pv[32];        // V scale x 64 (0 past the end)
 };
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
+// load, i.e. for the tile prefetch that was issued a moment earlier and is not needed before the next step.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Walk `n` key steps.  A step of one wavefront is
+//   scores  : S^T = K Q^T                     -- MFMA, operands from LDS
+//   softmax : P from S, running max and sum   -- VALU only
+//   output  : O^T += V^T P^T                  -- MFMA, operands from LDS
+// with one workgroup barrier per step: while tile s is consumed every wavefront converts its share of tile s+1
+// into the other buffer and starts the global loads of tile s+2.  All LDS operand reads of a step are issued
+// before its first MFMA.  (A variant that kept the two wavefronts of a SIMD half a step apart behind a second
+// barrier, so that one did softmax while the other fed the matrix pipe, measured 6% slower: a wavefront issues
+// at most one instruction every four cycles whatever its kind, and the extra barrier cost more than it hid.)
+template <class Issue, class Commit, class LoadK, class Scores, class Softmax, class LoadV, class Output>
+__device__ __forceinline__ void walk_keys(int n, StepTile *tiles, Issue issue, Commit commit, LoadK load_k, Scores scores,
+                                          Softmax softmax, LoadV load_v, Output output) {
+    issue(0);
+    commit(tiles[0], 0);
+    if (n > 1) issue(1);
+    lds_barrier();
+    for (int s = 0; s < n; ++s) {
+        if (s + 1 < n) commit(tiles[(s + 1) & 1], s + 1);
+        if (s + 2 < n) issue(s + 2);
+        load_k(tiles[s & 1], s);
+        load_v(tiles[s & 1], s);
+        scores(s);
+        softmax(tiles[s & 1], s);
+        output(s);
+        lds_barrier();
+    }
+}
 
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     __shared__ StepTile tiles[2];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: wavefront-dependent branches stay uniform
     const int li = lane & 15, lq = lane >> 4;
     // XCD-aware placement.  Workgroups are handed to the 8 XCDs round-robin by linear id, and each XCD has
     // its own L2.  All query tiles that read the same (sequence, kv-head) K/V stream are therefore given
@@ -128,7 +159,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     // =============================== history: int8 cache, f16 MFMA ===============================
     if (H > 0) {
         half8 qop[kNB][4];
-        float cq[kNB], cinit[kNB];
+        float cq[kNB];
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
             const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 32 * lq;
@@ -147,105 +178,121 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             amax = quad_max(amax);
             int ex = 0;
             if (amax > 0.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
-            float qsum = 0.0f;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const _Float16 hq = (_Float16)ldexpf(qf[8 * j + e], -ex);
-                    qop[nb][j][e] = hq;
-                    qsum += (float)hq;
-                }
-            qsum = quad_sum(qsum);
+                for (int e = 0; e < 8; ++e) qop[nb][j][e] = (_Float16)ldexpf(qf[8 * j + e], -ex);
             cq[nb] = ldexpf(a.scale_log2e, ex);
-            cinit[nb] = -1152.0f * qsum;
         }
 
         const int nsteps = (H + kPStep - 1) / kPStep;
-        // ---- producer roles: wavefronts 0-3 convert K (tile u = wave/2, k-groups 2*(wave&1) and +1);
-        //      wavefronts 4-7 convert V (token group wave-4, byte columns 2x and 2x+1 with x = lane/16);
-        //      wavefront 0 also stages the scales.
-        u32x4 rawk = {0u, 0u, 0u, 0u};
-        uint32_t rawv[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
-        float raws = 0.0f;
+        // ---- producers: every wavefront converts one eighth of the step's K tile and of its V tile.
+        //      K: wavefront w fills operand block w (tile u = w/4, k-group j = w%4); lane (li, lq) loads the
+        //         eight codes K[16u + li][32lq + 8j ..] (the d's of Q operand j) and writes them as one half8.
+        //      V: lane = (d-quad x = lane%32, key pair kp = 2w + lane/32).  Slots 2*pe, 2*pe+1 of key group g
+        //         (kp = 4g + pe) are the adjacent keys 16*(pe/2) + 4g + 2*(pe%2), +1; one dword of each (a
+        //         row is read by 32 consecutive lanes) gives four fp16 pairs, for d = 4x + i, stored in
+        //         block 4*(x%2) + i at operand lane (x/2, g).
+        //      The per-token scales are applied here, once per workgroup, rather than to every score and weight:
+        //      the operands are fp16(code * scale) (relative rounding 2^-11, finer than a bf16 cache would keep).
+        const int vx = lane & 31, vkp = 2 * wave + (lane >> 5);
+        const int vkey = 16 * ((vkp & 3) >> 1) + 4 * (vkp >> 2) + 2 * (vkp & 1);
+        const int vdst = ((vx >> 1) + 16 * (vkp >> 2)) * 16 + 4 * (vkp & 3);
+        const int krow = 16 * (wave >> 2) + li, kcol = 32 * lq + 8 * (wave & 3);
+        const uint32_t koff = krow * kPD + kcol, voff = vkey * kPD + 4 * vx;
+        u32x2 rawk = {0u, 0u};
+        uint32_t rawv[2] = {0u, 0u};
+        float rawsk = 0.0f, rawsv[2] = {0.0f, 0.0f};
+        // issue() is called for steps 0, 1, 2, ... in order, so the (scalar) addresses of a step's codes and
+        // scales advance by a constant; a block table is consulted only when a cursor leaves its block.
+        const uint8_t *kb = a.kc, *vb = a.vc;
+        const float *ksp = a.ks, *vsp = a.vs;
+        int kleft = 0, vleft = 0;  // tokens between the cursor and the end of its storage unit
         auto issue = [&](int step) {
             const int t0 = step * kPStep;
             const int last = H - 1 - t0;
-            int64_t unit;
-            int slot;
-            if (wave < 4) {
+            if (kleft <= 0) {
+                int64_t unit;
+                int slot;
                 resolve(a.ka, b, t0, unit, slot);
-                const uint8_t *kb = a.kc + unit * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)slot * kPD;
-                rawk = *(const u32x4 *)(kb + min(16 * (wave >> 1) + li, last) * kPD + 32 * lq + 16 * (wave & 1));
-                if (wave == 0) {
-                    const int tok = lane & 31;
-                    if (lane < 32) {
-                        raws = a.ks[unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot + min(tok, last)];
-                    } else {
-                        resolve(a.va, b, t0, unit, slot);
-                        raws = a.vs[unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot + min(tok, last)] * kPPScale;
-                    }
-                    if (tok > last) raws = 0.0f;
-                }
-            } else {
+                kb = a.kc + unit * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)slot * kPD;
+                ksp = a.ks + unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot;
+                kleft = a.ka.capacity_tokens - slot;
+            }
+            if (vleft <= 0) {
+                int64_t unit;
+                int slot;
                 resolve(a.va, b, t0, unit, slot);
-                const uint8_t *vb = a.vc + unit * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)slot * kPD;
-                const int g4 = wave - 4;
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    rawv[e] = *(const uint32_t *)(vb + min(16 * (e >> 2) + 4 * g4 + (e & 3), last) * kPD + 8 * li + 4 * (lq >> 1));
+                vb = a.vc + unit * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)slot * kPD;
+                vsp = a.vs + unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot;
+                vleft = a.va.capacity_tokens - slot;
             }
-        };
-        auto commit = [&](StepTile &t) {
-            if (wave < 4) {
-                const int blk = 4 * (wave >> 1) + 2 * (wave & 1);
-                *(half8 *)(t.k[blk] + obase) = int8x8_to_f16_biased(rawk[0], rawk[1]);
-                *(half8 *)(t.k[blk + 1] + obase) = int8x8_to_f16_biased(rawk[2], rawk[3]);
-                if (wave == 0) (lane < 32 ? t.ksc : t.pv)[lane & 31] = raws;
+            // The loaded values are only touched in commit(): nothing waits for a load here.  A full step adds
+            // this lane's fixed offsets to the step's (scalar) base addresses; only the last, partial step clamps rows.
+            if (last >= kPStep - 1) {
+                rawk = *(const u32x2 *)(kb + koff);
+                rawv[0] = *(const uint32_t *)(vb + voff);
+                rawv[1] = *(const uint32_t *)(vb + voff + kPD);
+                rawsk = ksp[(uint32_t)krow];
+                rawsv[0] = vsp[(uint32_t)vkey];
+                rawsv[1] = vsp[(uint32_t)vkey + 1];
             } else {
-                const int dst = (li + 16 * (wave - 4)) * 16;  // operand lane = (li, token group wave-4)
-                const int bsel = 2 * (lq & 1);
+                rawk = *(const u32x2 *)(kb + (min(krow, last) * kPD + kcol));
+                rawv[0] = *(const uint32_t *)(vb + (min(vkey, last) * kPD + 4 * vx));
+                rawv[1] = *(const uint32_t *)(vb + (min(vkey + 1, last) * kPD + 4 * vx));
+                rawsk = ksp[min(krow, last)];
+                rawsv[0] = vsp[min(vkey, last)];
+                rawsv[1] = vsp[min(vkey + 1, last)];
+            }
+            kb += kPStep * kPD; vb += kPStep * kPD;
+            ksp += kPStep; vsp += kPStep;
+            kleft -= kPStep; vleft -= kPStep;
+        };
+        auto commit = [&](StepTile &t, int step) {
+            const int last = H - 1 - step * kPStep;  // keys past the end become zero rows
+            const _Float16 sk = (_Float16)(krow > last ? 0.0f : rawsk);
+            const _Float16 bias = (_Float16)1152.0f;
+            *(half8 *)(t.k[wave] + obase) = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
+            const half2v sv = {(_Float16)(vkey > last ? 0.0f : rawsv[0]), (_Float16)(vkey + 1 > last ? 0.0f : rawsv[1])};
 #pragma unroll
-                for (int i = 0; i < 2; ++i)
-                    *(half8 *)(t.v[2 * lq + i] + dst) =
-                        pack_half8(int8_pair_to_f16(rawv[0], rawv[1], bsel + i), int8_pair_to_f16(rawv[2], rawv[3], bsel + i),
-                                   int8_pair_to_f16(rawv[4], rawv[5], bsel + i), int8_pair_to_f16(rawv[6], rawv[7], bsel + i));
+            for (int i = 0; i < 4; ++i) {
+                const half2v hv = __builtin_bit_cast(half2v, int8_pair_to_f16(rawv[0], rawv[1], i)) * sv;
+                *(uint32_t *)(t.v[4 * (vx & 1) + i] + vdst) = __builtin_bit_cast(uint32_t, hv);
             }
         };
-        auto consume = [&](const StepTile &t, int step) {
-            const int t0 = step * kPStep;
-            const bool tail = t0 + kPStep > H;
-            float ksc[8], pv[8];
+        float4v s[kNB][2];  // scores of the step between scores() and softmax()
+        half8 pop[kNB];     // P^T operands between softmax() and output()
+        half8 kop[8], vop[8];  // the step's A operands, read from LDS ahead of use
+        auto load_k = [&](const StepTile &t, int) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const float4v k4 = *(const float4v *)(t.ksc + 16 * u + 4 * lq);
-                const float4v p4 = *(const float4v *)(t.pv + 16 * u + 4 * lq);
+            for (int i = 0; i < 8; ++i) kop[i] = *(const half8 *)(t.k[i] + obase);
+        };
+        auto load_v = [&](const StepTile &t, int) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    ksc[4 * u + r] = k4[r];
-                    pv[4 * u + r] = p4[r];
-                }
-            }
-            float4v s[kNB][2];
+            for (int i = 0; i < 8; ++i) vop[i] = *(const half8 *)(t.v[i] + obase);
+        };
+        auto scores = [&](int) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){cinit[nb], cinit[nb], cinit[nb], cinit[nb]};
+                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const half8 ak = *(const half8 *)(t.k[4 * u + j] + obase);
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb)
-                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak, qop[nb][j], s[nb][u], 0, 0, 0);
-                }
+                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[4 * u + j], qop[nb][j], s[nb][u], 0, 0, 0);
             }
+        };
+        auto softmax = [&](const StepTile &t, int step) {
+            const int t0 = step * kPStep;
+            const bool tail = t0 + kPStep > H;
             float sc[kNB][8], mx[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) sc[nb][4 * u + r] = s[nb][u][r] * ksc[4 * u + r];
+                    for (int r = 0; r < 4; ++r) sc[nb][4 * u + r] = s[nb][u][r];
                 if (tail) {
 #pragma unroll
                     for (int u = 0; u < 2; ++u)
@@ -259,37 +306,26 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 mx[nb] = quad_max(m) * cq[nb];  // cq > 0: max(t) * cq == max(t * cq); -inf stays -inf
             }
             raise_max(mx);
-            half8 pop[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb];
+                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
                 float p[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const float e = __builtin_amdgcn_exp2f(sc[nb][i] * cq[nb] - mref);
-                    l_run[nb] += e;
-                    p[i] = e * pv[i];
+                    p[i] = __builtin_amdgcn_exp2f(sc[nb][i] * cq[nb] - mref);
+                    l_run[nb] += p[i];
                 }
                 pop[nb] = pack_half8(pack_f16x2(p[0], p[1]), pack_f16x2(p[2], p[3]), pack_f16x2(p[4], p[5]), pack_f16x2(p[6], p[7]));
             }
+        };
+        auto output = [&](int) {
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb) {
-                const half8 av = *(const half8 *)(t.v[bb] + obase);
+            for (int bb = 0; bb < 8; ++bb)
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, pop[nb], acc[nb][bb], 0, 0, 0);
-            }
+                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb], acc[nb][bb], 0, 0, 0);
         };
-        issue(0);
-        commit(tiles[0]);
-        if (nsteps > 1) issue(1);
-        __syncthreads();
-        for (int step = 0; step < nsteps; ++step) {
-            if (step + 1 < nsteps) commit(tiles[(step + 1) & 1]);
-            if (step + 2 < nsteps) issue(step + 2);
-            if (wv_active) consume(tiles[step & 1], step);
-            __syncthreads();
-        }
+        walk_keys(nsteps, tiles, issue, commit, load_k, scores, softmax, load_v, output);
     }
 
     // =============================== new tokens: bf16, causal ===============================
@@ -306,53 +342,65 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const int64_t rstride = (int64_t)a.Hkv * kPD;  // elements between consecutive tokens
-        // producer roles: wavefronts 0-3: K tile u = wave/2, k-groups 2*(wave&1), +1 (bf16 rows are operands as
-        // they are); wavefronts 4-7: V^T, token group wave-4, columns 2x, 2x+1 (x = lane/16) of this lane's 8.
-        u32x4 rawk[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-        uint32_t rawv[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};
+        // producers, split as in the history phase: wavefront w copies K operand block w (bf16 rows are
+        // operands as they are); for V a lane takes the d-quad x = lane%32 of two adjacent keys (8 bytes of
+        // each) and stores the four (key, key+1) bf16 pairs of d = 4x + i.
+        const int vx = lane & 31, vkp = 2 * wave + (lane >> 5);
+        const int vkey = 16 * ((vkp & 3) >> 1) + 4 * (vkp >> 2) + 2 * (vkp & 1);
+        const int vdst = ((vx >> 1) + 16 * (vkp >> 2)) * 16 + 4 * (vkp & 3);
+        const int krow = 16 * (wave >> 2) + li, kcol = 32 * lq + 8 * (wave & 3);
+        const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + 4 * vx;  // elements
+        u32x4 rawk = {0u, 0u, 0u, 0u};
+        u32x2 rawv[2] = {{0u, 0u}, {0u, 0u}};
         auto issue = [&](int step) {
             const int t0 = step * kPStep;
-            if (wave < 4) {
-                const uint16_t *p = knb + (int64_t)min(t0 + 16 * (wave >> 1) + li, S - 1) * rstride + 32 * lq + 16 * (wave & 1);
-                rawk[0] = *(const u32x4 *)p;
-                rawk[1] = *(const u32x4 *)(p + 8);
+            if (t0 + kPStep <= S) {  // full step: scalar base + this lane's fixed offsets
+                const uint16_t *kb = knb + (int64_t)t0 * rstride, *vb = vnb + (int64_t)t0 * rstride;
+                rawk = *(const u32x4 *)(kb + koff);
+                rawv[0] = *(const u32x2 *)(vb + voff);
+                rawv[1] = *(const u32x2 *)(vb + voff + (uint32_t)rstride);
             } else {
-                const int g4 = wave - 4;
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    rawv[e] = *(const uint32_t *)(vnb + (int64_t)min(t0 + 16 * (e >> 2) + 4 * g4 + (e & 3), S - 1) * rstride + 8 * li + 2 * lq);
+                rawk = *(const u32x4 *)(knb + (int64_t)min(t0 + krow, S - 1) * rstride + kcol);
+                rawv[0] = *(const u32x2 *)(vnb + (int64_t)min(t0 + vkey, S - 1) * rstride + 4 * vx);
+                rawv[1] = *(const u32x2 *)(vnb + (int64_t)min(t0 + vkey + 1, S - 1) * rstride + 4 * vx);
             }
         };
         auto commit = [&](StepTile &t) {
-            if (wave < 4) {
-                const int blk = 4 * (wave >> 1) + 2 * (wave & 1);
-                *(u32x4 *)(t.k[blk] + obase) = rawk[0];
-                *(u32x4 *)(t.k[blk + 1] + obase) = rawk[1];
-            } else {
-                const int dst = (li + 16 * (wave - 4)) * 16;
+            *(u32x4 *)(t.k[wave] + obase) = rawk;
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    const u32x4 w = {pick_halves(rawv[0], rawv[1], i), pick_halves(rawv[2], rawv[3], i),
-                                     pick_halves(rawv[4], rawv[5], i), pick_halves(rawv[6], rawv[7], i)};
-                    *(u32x4 *)(t.v[2 * lq + i] + dst) = w;
-                }
-            }
+            for (int i = 0; i < 4; ++i)
+                *(uint32_t *)(t.v[4 * (vx & 1) + i] + vdst) = pick_halves(rawv[0][i >> 1], rawv[1][i >> 1], i & 1);
         };
-        auto consume = [&](const StepTile &t, int step) {
-            const int t0 = step * kPStep;
-            float4v s[kNB][2];
+        float4v s[kNB][2];
+        bf16x8 pop[kNB];
+        auto mine = [&](int step) { return wv_active && step * kPStep <= wv_qlast; };  // else all keys are in the future
+        bf16x8 kop[8], vop[8];
+        auto load_k = [&](const StepTile &t, int step) {
+            if (!mine(step)) return;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) kop[i] = *(const bf16x8 *)(t.k[i] + obase);
+        };
+        auto load_v = [&](const StepTile &t, int step) {
+            if (!mine(step)) return;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vop[i] = *(const bf16x8 *)(t.v[i] + obase);
+        };
+        auto scores = [&](int step) {
+            if (!mine(step)) return;
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const bf16x8 ak = *(const bf16x8 *)(t.k[4 * u + j] + obase);
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb)
-                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ak, qop[nb][j], s[nb][u], 0, 0, 0);
-                }
+                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[4 * u + j], qop[nb][j], s[nb][u], 0, 0, 0);
             }
+        };
+        auto softmax = [&](const StepTile &, int step) {
+            if (!mine(step)) return;
+            const int t0 = step * kPStep;
             const bool diag = t0 + kPStep - 1 > wv_q0;  // some (key, query) pair of this step is in the future
             float sc[kNB][8], mx[kNB];
 #pragma unroll
@@ -375,37 +423,27 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 mx[nb] = quad_max(m);
             }
             raise_max(mx);
-            bf16x8 pop[kNB];
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb];
+                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
                 float p[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    const float e = __builtin_amdgcn_exp2f(sc[nb][i] - mref);
-                    l_run[nb] += e;
-                    p[i] = e * kPPScale;
+                    p[i] = __builtin_amdgcn_exp2f(sc[nb][i] - mref);
+                    l_run[nb] += p[i];
                 }
                 pop[nb] = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
             }
+        };
+        auto output = [&](int step) {
+            if (!mine(step)) return;
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb) {
-                const bf16x8 av = *(const bf16x8 *)(t.v[bb] + obase);
+            for (int bb = 0; bb < 8; ++bb)
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pop[nb], acc[nb][bb], 0, 0, 0);
-            }
+                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb], acc[nb][bb], 0, 0, 0);
         };
-        issue(0);
-        commit(tiles[0]);
-        if (nsteps > 1) issue(1);
-        __syncthreads();
-        for (int step = 0; step < nsteps; ++step) {
-            if (step + 1 < nsteps) commit(tiles[(step + 1) & 1]);
-            if (step + 2 < nsteps) issue(step + 2);
-            if (wv_active && step * kPStep <= wv_qlast) consume(tiles[step & 1], step);
-            __syncthreads();
-        }
+        walk_keys(nsteps, tiles, issue, [&](StepTile &t, int) { commit(t); }, load_k, scores, softmax, load_v, output);
     }
 
     // =============================== normalise and store ===============================
@@ -413,7 +451,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     for (int nb = 0; nb < kNB; ++nb) {
         const float l = quad_sum(l_run[nb]);
         if (qi[nb] >= S) continue;
-        const float inv = 1.0f / (l * kPPScale);
+        const float inv = 1.0f / l;
         uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kPD + 32 * lq;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
