@@ -17,11 +17,11 @@
 // Products (both on v_mfma_f32_16x16x32, keys on the M axis, columns on N):
 //   S^T[key, col]  = sum_d K[key, d] Q[col, d]
 //   O^T[d, col]   += sum_key V^T[d, key] P^T[key, col]
-// History part: f16 MFMA, int8 codes enter as exact fp16 integers (see decode_attn.hip); Q is scaled
-// per column by a power of two into fp16 range; the per-token K scale multiplies the fp32 score, the
-// per-token V scale is folded into P (fp16).  New-token part: bf16 MFMA straight from the caller's
-// bf16 K/V, V^T built with permutes, P rounded to bf16.  Softmax and accumulation are fp32; the
-// score layout of the first product is the B-operand layout of the second, so P stays in its lanes.
+// History part: f16 MFMA.  The eight wavefronts that convert a tile apply the per-token scales while they are at
+// it, so the LDS operands are fp16(code * scale) and the consumers see plain K and V; Q is scaled per column by a
+// power of two into fp16 range.  New-token part: bf16 MFMA straight from the caller's bf16 K/V, V^T built with
+// permutes, P rounded to bf16.  Softmax and accumulation are fp32; the score layout of the first product is the
+// B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16 range (|x| > 65024) saturate.
 #include "mfma_common.hpp"
 #include "quant_device.hpp"
 
@@ -33,6 +33,7 @@ constexpr int kPWaves = 8;
 constexpr int kNB = 2;  // 16-column blocks per wavefront
 constexpr float kPLog2e = 1.4426950408889634f;
 constexpr float kPShift = 6.0f;  // weights are carried as 2^6 * exp2(s - m_run): keeps small ones out of the fp16 subnormals
+constexpr float kMaxScale = 512.0f;  // 127 * scale stays finite in fp16; larger magnitudes saturate instead of overflowing
 constexpr float kSlack = 4.0f;  // log2 units by which the softmax reference value overshoots a new maximum
 
 struct PrefillArgs {
@@ -250,10 +251,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         auto commit = [&](StepTile &t, int step) {
             const int last = H - 1 - step * kPStep;  // keys past the end become zero rows
-            const _Float16 sk = (_Float16)(krow > last ? 0.0f : rawsk);
+            const _Float16 sk = (_Float16)(krow > last ? 0.0f : fminf(rawsk, kMaxScale));
             const _Float16 bias = (_Float16)1152.0f;
             *(half8 *)(t.k[wave] + obase) = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
-            const half2v sv = {(_Float16)(vkey > last ? 0.0f : rawsv[0]), (_Float16)(vkey + 1 > last ? 0.0f : rawsv[1])};
+            const half2v sv = {(_Float16)(vkey > last ? 0.0f : fminf(rawsv[0], kMaxScale)),
+                               (_Float16)(vkey + 1 > last ? 0.0f : fminf(rawsv[1], kMaxScale))};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const half2v hv = __builtin_bit_cast(half2v, int8_pair_to_f16(rawv[0], rawv[1], i)) * sv;
