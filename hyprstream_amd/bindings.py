@@ -23,6 +23,7 @@ EXPORTS = [
     "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_deltanet_forward",
+    "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_decode_step_int8_rope",
 ]
 
 
@@ -103,6 +104,26 @@ def kv_quantize_int8(k_src, v_src, k_codes, v_codes, k_scales, v_scales, layout,
                                     ctypes.c_int32(start_pos), B, S, Hkv, D, _stream()))
 
 
+def kv_quantize_int8_rope(k_src, v_src, rope_sin, rope_cos, k_codes, v_codes, k_scales, v_scales, layout,
+                          positions=None, start_pos=0):
+    """As kv_quantize_int8 with K rotated on the way in; rope_sin/rope_cos: [rope_len, D/2] in k_src's dtype."""
+    B, S, Hkv, D = k_src.shape
+    assert k_src.is_contiguous() and v_src.is_contiguous() and rope_sin.is_contiguous() and rope_cos.is_contiguous()
+    assert rope_sin.dtype == k_src.dtype and rope_sin.shape[1] == D // 2
+    check(lib().hs_kv_quantize_int8_rope(_ptr(k_src), _ptr(v_src), _dtype_code(k_src), _ptr(rope_sin), _ptr(rope_cos),
+                                         ctypes.c_int32(rope_sin.shape[0]), _ptr(k_codes), _ptr(v_codes),
+                                         _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout), _ptr(positions),
+                                         ctypes.c_int32(start_pos), B, S, Hkv, D, _stream()))
+
+
+def rope_apply(x, rope_sin, rope_cos, out, positions=None, start_pos=0):
+    """Half-split rotary embedding of x [B, S, H, D] into out (same shape and dtype)."""
+    B, S, H, D = x.shape
+    assert x.is_contiguous() and out.is_contiguous() and out.dtype == x.dtype and rope_sin.dtype == x.dtype
+    check(lib().hs_rope_apply(_ptr(x), _dtype_code(x), _ptr(rope_sin), _ptr(rope_cos), ctypes.c_int32(rope_sin.shape[0]),
+                              _ptr(positions), ctypes.c_int32(start_pos), _ptr(out), B, S, H, D, _stream()))
+
+
 def kv_fp8_calibrate(k_src, v_src, k_scales, v_scales):
     B, S, Hkv, D = k_src.shape
     check(lib().hs_kv_fp8_calibrate(_ptr(k_src), _ptr(v_src), _dtype_code(k_src), _ptr(k_scales), _ptr(v_scales),
@@ -151,6 +172,19 @@ def decode_step(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, s
              _ptr(v_scales), ctypes.byref(layout), _ptr(seq_lens), _ptr(out), _ptr(workspace),
              ctypes.c_size_t(workspace.numel() * workspace.element_size()), B, Hq, Hkv, D,
              ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
+
+
+def decode_step_rope(q, k_new, v_new, rope_sin, rope_cos, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out,
+                     workspace, Hkv, max_seq_len, softmax_scale):
+    """decode_step (int8) with q and k_new arriving unrotated; bf16 tables [rope_len, D/2]."""
+    B, Hq, D = q.shape
+    assert k_new.shape == (B, 1, Hkv, D) and k_new.is_contiguous() and v_new.is_contiguous()
+    check(lib().hs_decode_step_int8_rope(_ptr(q), _ptr(k_new), _ptr(v_new), _ptr(rope_sin), _ptr(rope_cos),
+                                         ctypes.c_int32(rope_sin.shape[0]), _ptr(k_codes), _ptr(v_codes),
+                                         _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout), _ptr(seq_lens),
+                                         _ptr(out), _ptr(workspace),
+                                         ctypes.c_size_t(workspace.numel() * workspace.element_size()), B, Hq, Hkv, D,
+                                         ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
 
 
 def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, hist_len, out, softmax_scale,

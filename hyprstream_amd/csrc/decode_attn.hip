@@ -59,7 +59,30 @@ struct DecodeArgs {
     int32_t direct;      // 1: single chunk, write `out` directly; 0: leave partials in the workspace
     int32_t B, Hq, Hkv, G, chunk_tokens, nchunks, max_seq_len;
     float scale_log2e;
+    // optional rotary embedding of q (bf16 tables [rope_len, D/2]); the new token's K is rotated by nt.rope_*
+    const uint16_t *rope_sin, *rope_cos;
+    int32_t rope_len;
 };
+
+// Half-split rotary embedding of the 32 query elements a lane holds, in bf16 arithmetic (every product and sum
+// rounded to bf16, as the separate libtorch ops of RoPE::apply_rotary_pos_emb do, rope.rs:206-248).  Element
+// qf[8*i + e] is d = 64*(i/2) + 16*lq + 8*(i%2) + e, so a lane holds both halves of each rotated pair.
+__device__ __forceinline__ void rope_rotate_q(float (&qf)[32], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
+#pragma clang fp contract(off)
+    auto rb = [](float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); };
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const u32x4 sw = *(const u32x4 *)(sin_row + 16 * lq + 8 * i), cw = *(const u32x4 *)(cos_row + 16 * lq + 8 * i);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
+            const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
+            const float x1 = qf[8 * i + e], x2 = qf[8 * (i + 2) + e];
+            qf[8 * i + e] = rb(rb(x1 * cs) - rb(x2 * sn));
+            qf[8 * (i + 2) + e] = rb(rb(x1 * sn) + rb(x2 * cs));
+        }
+    }
+}
 
 template <bool FP8>
 struct Stage {
@@ -79,7 +102,7 @@ __device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t t) {
     return (t & 0x80008000u) | ((t >> 1) & 0x3f803f80u);
 }
 
-template <bool FP8>
+template <bool FP8, bool ROPE>
 __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int L = min(a.seq_lens[b], a.max_seq_len);
@@ -267,6 +290,10 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                     qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
                 }
             }
+            if (ROPE) {
+                const int p = min(max(a.seq_lens[b] - 1, 0), a.rope_len - 1);  // the query is the newest token
+                rope_rotate_q(qf, a.rope_sin + (int64_t)p * (kD / 2), a.rope_cos + (int64_t)p * (kD / 2), lq);
+            }
 #pragma unroll
             for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
         } else {
@@ -407,6 +434,8 @@ static int pick_chunk_tokens(int B, int Hkv, int max_seq_len) {
 struct NewToken {  // optional quantize-on-write of one token per sequence inside the same call
     const void *k_src = nullptr, *v_src = nullptr;  // [B, 1, Hkv, D]
     int dtype = HS_BF16;
+    const void *rope_sin = nullptr, *rope_cos = nullptr;  // rotate q and k_new (bf16 tables [rope_len, D/2])
+    int rope_len = 0;
 };
 
 static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q, void *kc, void *vc, float *ks,
@@ -455,10 +484,18 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.nt.addr[0] = a.ka; a.nt.addr[1] = a.va;
     a.nt.positions = seq_lens; a.nt.start_pos = -1;  // the new token is the last cached one
     a.nt.B = B; a.nt.S = 1; a.nt.Hkv = Hkv; a.nt.D = D; a.nt.dtype = nt.dtype;
+    if (nt.rope_sin) {
+        if (!nt.rope_cos || nt.rope_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "bad rotary tables");
+        if (!nt.k_src || nt.dtype != HS_BF16)
+            return fail(HS_ERR_INVALID_ARGUMENT, "the rotary decode step takes a bf16 new token");
+    }
+    a.nt.rope_sin = nt.rope_sin; a.nt.rope_cos = nt.rope_cos; a.nt.rope_len = nt.rope_len;
+    a.rope_sin = (const uint16_t *)nt.rope_sin; a.rope_cos = (const uint16_t *)nt.rope_cos; a.rope_len = nt.rope_len;
     if (phases & 1) {
         dim3 grid(a.nchunks, Hkv, B);
-        if (fp8) decode_attn_kernel<true><<<grid, 256, 0, stream>>>(a);
-        else decode_attn_kernel<false><<<grid, 256, 0, stream>>>(a);
+        if (fp8) decode_attn_kernel<true, false><<<grid, 256, 0, stream>>>(a);
+        else if (a.rope_sin) decode_attn_kernel<false, true><<<grid, 256, 0, stream>>>(a);
+        else decode_attn_kernel<false, false><<<grid, 256, 0, stream>>>(a);
         if (int rc = check_launch("decode_attn")) return rc;
     }
     if ((phases & 2) && !a.direct) {
@@ -507,6 +544,19 @@ int hs_decode_step_int8(const void *q, const void *k_new, const void *v_new, int
     if (!k_new || !v_new) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     hs::NewToken nt;
     nt.k_src = k_new; nt.v_src = v_new; nt.dtype = src_dtype;
+    return hs::launch_decode(false, 3, nt, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+                             workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_step_int8_rope(const void *q, const void *k_new, const void *v_new, const void *rope_sin,
+                             const void *rope_cos, int32_t rope_len, int8_t *k_codes, int8_t *v_codes, float *k_scales,
+                             float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                             void *workspace, size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
+                             int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
+    if (!k_new || !v_new || !rope_sin || !rope_cos) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    hs::NewToken nt;
+    nt.k_src = k_new; nt.v_src = v_new; nt.dtype = HS_BF16;
+    nt.rope_sin = rope_sin; nt.rope_cos = rope_cos; nt.rope_len = rope_len;
     return hs::launch_decode(false, 3, nt, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
                              workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
 }

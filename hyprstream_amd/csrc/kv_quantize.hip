@@ -18,6 +18,37 @@ __global__ __launch_bounds__(256) void kv_quantize_kernel(QuantArgs a) {
     quantize_row<E, FP8>(a, blockIdx.y, row, threadIdx.x & 63);
 }
 
+struct RopeArgs {
+    const void *x, *sin_t, *cos_t;
+    void *out;
+    const int32_t *positions;
+    int32_t start_pos, rope_len, B, S, H, D, dtype;
+};
+
+// Rotary embedding of a [B, S, H, D] tensor (the query side of a step; K is rotated inside the cache write).
+template <int E>
+__global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (int64_t)a.B * a.S * a.H) return;
+    const int64_t bs = row / a.H;
+    const int s = (int)(bs % a.S), b = (int)(bs / a.S);
+    const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
+    float x[E];
+    load_src<E>(a.x, a.dtype, row * a.D + lane * E, x);
+    rope_rotate<E>(a.x, a.dtype, row * a.D, a.D, a.sin_t, a.cos_t, a.rope_len, pos, lane * E, x);
+    const int64_t o = row * a.D + lane * E;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        if (a.dtype == HS_F32) ((float *)a.out)[o + e] = x[e];
+        else if (a.dtype == HS_BF16) ((uint16_t *)a.out)[o + e] = (uint16_t)f32_to_bf16_bits(x[e]);
+        else {
+            _Float16 f = (_Float16)x[e];
+            __builtin_memcpy((uint16_t *)a.out + o + e, &f, 2);
+        }
+    }
+}
+
 // scale[b, h] = max_{s, d} |x| / 448.  One workgroup per (b, h, tensor).
 __global__ __launch_bounds__(256) void fp8_calibrate_kernel(const void *k_src, const void *v_src, int dtype,
                                                            float *k_scales, float *v_scales, int B, int S, int Hkv,
@@ -125,8 +156,14 @@ int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool ne
 template <bool FP8>
 static int launch_quantize(const void *k_src, const void *v_src, int dtype, void *kc, void *vc, float *ks, float *vs,
                            const hs_kv_layout *l, const int32_t *positions, int start_pos, int B, int S, int Hkv,
-                           int D, hipStream_t stream) {
+                           int D, hipStream_t stream, const void *rope_sin = nullptr, const void *rope_cos = nullptr,
+                           int rope_len = 0) {
     if (int rc = check_common(l, B, S, Hkv, D, !FP8)) return rc;
+    if ((rope_sin == nullptr) != (rope_cos == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give sin and cos or neither");
+    if (rope_sin && rope_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "rope_len must be positive");
+    if (rope_sin && !positions && (int64_t)start_pos + S > rope_len)
+        return fail(HS_ERR_INVALID_ARGUMENT, "positions %d..%d exceed the rotary tables (%d rows)", start_pos,
+                    start_pos + S - 1, rope_len);
     if (!k_src || !v_src || !kc || !vc || !ks || !vs) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16)
         return fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", dtype);
@@ -147,6 +184,7 @@ static int launch_quantize(const void *k_src, const void *v_src, int dtype, void
     a.addr[0] = make_addr(*l, 0); a.addr[1] = make_addr(*l, 1);
     a.positions = positions; a.start_pos = start_pos;
     a.B = B; a.S = S; a.Hkv = Hkv; a.D = D; a.dtype = dtype;
+    a.rope_sin = rope_sin; a.rope_cos = rope_cos; a.rope_len = rope_len;
     dim3 grid((unsigned)((rows + 3) / 4), 2);
     if (D == 64) kv_quantize_kernel<1, FP8><<<grid, 256, 0, stream>>>(a);
     else if (D == 128) kv_quantize_kernel<2, FP8><<<grid, 256, 0, stream>>>(a);
@@ -163,6 +201,39 @@ int hs_kv_quantize_int8(const void *k_src, const void *v_src, int src_dtype, int
                         int32_t start_pos, int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream) {
     return hs::launch_quantize<false>(k_src, v_src, src_dtype, k_codes, v_codes, k_scales, v_scales, layout, positions,
                                       start_pos, B, S, Hkv, D, (hipStream_t)stream);
+}
+
+int hs_kv_quantize_int8_rope(const void *k_src, const void *v_src, int src_dtype, const void *rope_sin,
+                             const void *rope_cos, int32_t rope_len, int8_t *k_codes, int8_t *v_codes, float *k_scales,
+                             float *v_scales, const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos,
+                             int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream) {
+    if (!rope_sin || !rope_cos) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null rotary table");
+    return hs::launch_quantize<false>(k_src, v_src, src_dtype, k_codes, v_codes, k_scales, v_scales, layout, positions,
+                                      start_pos, B, S, Hkv, D, (hipStream_t)stream, rope_sin, rope_cos, rope_len);
+}
+
+int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,
+                  const int32_t *positions, int32_t start_pos, void *out, int32_t B, int32_t S, int32_t H, int32_t D,
+                  hs_stream_t stream) {
+    using namespace hs;
+    if (!x || !out || !rope_sin || !rope_cos) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16) return fail(HS_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+    if (B < 0 || S < 0 || H <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d H=%d", B, S, H);
+    if (D != 64 && D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "head_dim %d not in {64,128,256}", D);
+    if (rope_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "rope_len must be positive");
+    if (!positions && (start_pos < 0 || (int64_t)start_pos + S > rope_len))
+        return fail(HS_ERR_INVALID_ARGUMENT, "positions %d..%d exceed the rotary tables (%d rows)", start_pos,
+                    start_pos + S - 1, rope_len);
+    const int64_t rows = (int64_t)B * S * H;
+    if (rows == 0) return HS_OK;
+    RopeArgs a;
+    a.x = x; a.sin_t = rope_sin; a.cos_t = rope_cos; a.out = out; a.positions = positions; a.start_pos = start_pos;
+    a.rope_len = rope_len; a.B = B; a.S = S; a.H = H; a.D = D; a.dtype = dtype;
+    dim3 grid((unsigned)((rows + 3) / 4));
+    if (D == 64) rope_apply_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    else if (D == 128) rope_apply_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    else rope_apply_kernel<4><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    return check_launch("rope_apply");
 }
 
 int hs_kv_quantize_fp8(const void *k_src, const void *v_src, int src_dtype, uint8_t *k_codes, uint8_t *v_codes,

@@ -11,7 +11,45 @@ struct QuantArgs {
     KvAddr addr[2];
     const int32_t *positions;
     int32_t start_pos, B, S, Hkv, D, dtype;
+    // optional rotary embedding of K before it is quantized: sin/cos tables [rope_len, D/2] in the source
+    // dtype, row = the token's position; nullptr = K arrives rotated
+    const void *rope_sin = nullptr, *rope_cos = nullptr;
+    int32_t rope_len = 0;
 };
+
+// Round an fp32 value to the tensor dtype and back: libtorch's elementwise ops on bf16/fp16 tensors compute in
+// fp32 and round the result of EVERY op to the tensor dtype.
+__device__ __forceinline__ float round_to_dtype(float v, int dtype) {
+    if (dtype == HS_BF16) return bf16_bits_to_f32(f32_to_bf16_bits(v));
+    if (dtype == HS_F16) return (float)(_Float16)v;
+    return v;
+}
+
+// Half-split rotary embedding of this lane's E consecutive elements (first element d0) of one head row:
+//   d <  D/2 : x[d]*cos[d]       - x[d + D/2]*sin[d]
+//   d >= D/2 : x[d - D/2]*sin[j] + x[d]*cos[j],  j = d - D/2
+// as four products and two sums, each rounded to the tensor dtype (RoPE::apply_rotary_pos_emb,
+// crates/hyprstream/src/runtime/rope.rs:206-248, with tables cast to the dtype, rope.rs:118-119).
+// `src_row` = element index of the row's first element in `src`.
+template <int E>
+__device__ __forceinline__ void rope_rotate(const void *src, int dtype, int64_t src_row, int D, const void *sin_t,
+                                            const void *cos_t, int rope_len, int pos, int d0, float (&x)[E]) {
+#pragma clang fp contract(off)
+    const int half = D / 2;
+    const bool upper = d0 >= half;
+    const int j0 = upper ? d0 - half : d0;
+    const int p = pos < 0 ? 0 : (pos >= rope_len ? rope_len - 1 : pos);
+    float other[E], sn[E], cs[E];
+    load_src<E>(src, dtype, src_row + (upper ? d0 - half : d0 + half), other);
+    load_src<E>(sin_t, dtype, (int64_t)p * half + j0, sn);
+    load_src<E>(cos_t, dtype, (int64_t)p * half + j0, cs);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const float own_cos = round_to_dtype(x[e] * cs[e], dtype);
+        const float other_sin = round_to_dtype(other[e] * sn[e], dtype);
+        x[e] = round_to_dtype(upper ? other_sin + own_cos : own_cos - other_sin, dtype);
+    }
+}
 
 __device__ __forceinline__ uint32_t f32_to_e4m3fn_bits(float y) {
 #pragma clang fp contract(off)
@@ -47,6 +85,8 @@ __device__ __forceinline__ void quantize_row(const QuantArgs &a, int which, int6
 
     float x[E];
     load_src<E>(a.src[which], a.dtype, row * a.D + lane * E, x);
+    if (which == 0 && a.rope_sin != nullptr)
+        rope_rotate<E>(a.src[0], a.dtype, row * a.D, a.D, a.rope_sin, a.rope_cos, a.rope_len, pos, lane * E, x);
 
     uint8_t *dst = (uint8_t *)a.codes[which] + unit * ad.code_stride_seq + (int64_t)h * ad.code_stride_head +
                    (int64_t)slot * a.D + lane * E;

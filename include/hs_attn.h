@@ -93,6 +93,26 @@ HS_API int hs_kv_quantize_int8(const void *k_src, const void *v_src, int src_dty
                         const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos,
                         int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream);
 
+/* ---- rotary embedding fused into the write (RoPE::forward / apply_rotary_pos_emb, rope.rs:150-248, which
+ * the reference runs on q and k right before cache.update, llama.rs:598-611, qwen3_5.rs:977-990) ----------
+ * rope_sin, rope_cos: device tables [rope_len, D/2] in the tensor's dtype, row p = sin/cos(p * base^(-2i/D))
+ * computed in fp32 and cast (rope.rs:100-122); built and kept by the caller, as the reference caches them.
+ * Half-split convention: x1 = x[..., :D/2], x2 = x[..., D/2:];  x1' = x1*cos - x2*sin, x2' = x1*sin + x2*cos,
+ * each product and sum rounded to the dtype like the separate libtorch ops they replace, so codes and scales
+ * equal those of quantizing the reference's rotated K.  The table row of token (b, s) is its cache position
+ * (positions ? positions[b] : 0) + start_pos + s, clamped to the table.
+ * hs_kv_quantize_int8_rope: k_src arrives UNROTATED; V is written as it is.
+ * hs_rope_apply: x, out [B, S, H, D] in `dtype` (the query side; out may equal x only if no other row reads it,
+ * i.e. never: use a separate buffer). */
+HS_API int hs_kv_quantize_int8_rope(const void *k_src, const void *v_src, int src_dtype,
+                        const void *rope_sin, const void *rope_cos, int32_t rope_len,
+                        int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                        const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos,
+                        int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream);
+HS_API int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,
+                        const int32_t *positions, int32_t start_pos, void *out,
+                        int32_t B, int32_t S, int32_t H, int32_t D, hs_stream_t stream);
+
 /* FP8 e4m3fn cache with one fp32 scale per (sequence, kv-head).  Calibration computes
  * scale[b, h] = max over (s, d) |x| / 448 from the tokens given (typically the prompt);
  * quantization stores e4m3fn(clamp(x / scale, +-448)), round-to-nearest-even. */
@@ -139,6 +159,17 @@ HS_API int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8
  * (what LlamaAttention::forward does per layer: cache.update then cache.get then attention,
  * llama.rs:605-636). */
 HS_API int hs_decode_step_int8(const void *q, const void *k_new, const void *v_new, int src_dtype,
+                               int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                               const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                               void *workspace, size_t workspace_bytes,
+                               int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                               float softmax_scale, hs_stream_t stream);
+/* The same step with the rotary embedding of q and k_new done inside the kernel (the reference rotates both
+ * right before cache.update, llama.rs:598-611): q [B, Hq, D] and k_new [B, 1, Hkv, D] arrive UNROTATED in
+ * bf16, rope_sin / rope_cos are bf16 tables [rope_len, D/2] (see hs_rope_apply), the table row is the new
+ * token's position seq_lens[b] - 1.  Results equal hs_rope_apply(q) + hs_kv_quantize_int8_rope + decode. */
+HS_API int hs_decode_step_int8_rope(const void *q, const void *k_new, const void *v_new,
+                               const void *rope_sin, const void *rope_cos, int32_t rope_len,
                                int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
                                const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
                                void *workspace, size_t workspace_bytes,

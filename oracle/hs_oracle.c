@@ -46,6 +46,19 @@
  *                            (qwen3_5.rs:725-751), with the L2 normalisation
  *                            x / max(||x||, 1e-3) (qwen3_5.rs:331-335) and the
  *                            k/q-head -> v-head expansion (qwen3_5.rs:704-720).
+ *  - orc_rope_apply_*        rotary embedding in the half-split convention,
+ *                            x1' = x1*cos - x2*sin, x2' = x1*sin + x2*cos with
+ *                            x1 = x[..., :D/2], x2 = x[..., D/2:]
+ *                            (crates/hyprstream/src/runtime/rope.rs:206-248).
+ *                            The tables are fp32 values cast to the tensor dtype
+ *                            (rope.rs:100-122) and the four products and two
+ *                            sums are separate libtorch ops in that dtype, so a
+ *                            bf16 tensor is rounded to bf16 after EVERY op; the
+ *                            restatement does exactly that.  Pinned by golden
+ *                            vectors and a live comparison with libtorch CPU ops
+ *                            on bf16/fp32 tensors, identity at position 0, norm
+ *                            preservation and the relative-position property
+ *                            (tests/test_oracle_rope.py).
  *
  * parity unpinned: the reference's own int8 format (bitsandbytes 0.45.0
  * blockwise-64 codes, tie-breaking of its binary search) is not restated here
@@ -353,4 +366,48 @@ ORC_API void orc_deltanet_recurrent(const float *q, const float *k, const float 
             for (int i = 0; i < dk * dv; ++i) st[i] = (float)S[i];
         }
     free(S); free(qq); free(kk); free(m);
+}
+
+/* --------------------------------------------------------------------- RoPE */
+
+static inline float rbf(float f) { return bf16_to_f32(orc_f32_to_bf16(f)); }
+
+/* x, out: bf16 bit patterns [rows, H, D] with rows = B*S; sin/cos: bf16 bit patterns [table_len, D/2];
+ * pos[rows]: table row of each token.  Every product and every sum is rounded to bf16 (see the header). */
+ORC_API void orc_rope_apply_bf16(const uint16_t *x, const uint16_t *sin_t, const uint16_t *cos_t, const int32_t *pos,
+                                 int64_t rows, int H, int D, uint16_t *out) {
+    const int half = D / 2;
+    for (int64_t r = 0; r < rows; ++r) {
+        const uint16_t *st = sin_t + (int64_t)pos[r] * half, *ct = cos_t + (int64_t)pos[r] * half;
+        for (int h = 0; h < H; ++h) {
+            const uint16_t *xi = x + (r * H + h) * D;
+            uint16_t *oi = out + (r * H + h) * D;
+            for (int d = 0; d < half; ++d) {
+                const float x1 = bf16_to_f32(xi[d]), x2 = bf16_to_f32(xi[d + half]);
+                const float c = bf16_to_f32(ct[d]), s = bf16_to_f32(st[d]);
+                const volatile float a = rbf(x1 * c), b = rbf(x2 * s), e = rbf(x1 * s), f = rbf(x2 * c);
+                oi[d] = orc_f32_to_bf16(a - b);
+                oi[d + half] = orc_f32_to_bf16(e + f);
+            }
+        }
+    }
+}
+
+/* The same in fp32 (tables fp32, no rounding below fp32, products and sums not fused). */
+ORC_API void orc_rope_apply_f32(const float *x, const float *sin_t, const float *cos_t, const int32_t *pos, int64_t rows,
+                                int H, int D, float *out) {
+    const int half = D / 2;
+    for (int64_t r = 0; r < rows; ++r) {
+        const float *st = sin_t + (int64_t)pos[r] * half, *ct = cos_t + (int64_t)pos[r] * half;
+        for (int h = 0; h < H; ++h) {
+            const float *xi = x + (r * H + h) * D;
+            float *oi = out + (r * H + h) * D;
+            for (int d = 0; d < half; ++d) {
+                const volatile float a = xi[d] * ct[d], b = xi[d + half] * st[d];
+                const volatile float e = xi[d] * st[d], f = xi[d + half] * ct[d];
+                oi[d] = a - b;
+                oi[d + half] = e + f;
+            }
+        }
+    }
 }

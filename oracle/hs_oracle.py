@@ -190,3 +190,24 @@ def deltanet_recurrent(q, k, v, g, beta, state, q_scale, l2norm=False):
     lib().orc_deltanet_recurrent(_p(q), _p(k), _p(v), _p(g), _p(beta), _p(st), B, T, nk, nv, dk, dv,
                                  ctypes.c_float(q_scale), int(bool(l2norm)), _p(out))
     return out, st
+
+
+# ------------------------------------------------------------------------ RoPE
+def rope_apply_bf16(x_bits, sin_bits, cos_bits, pos):
+    """x_bits: uint16 [rows, H, D] bf16 patterns; sin/cos: uint16 [L, D/2]; pos: int32 [rows] -> uint16 [rows, H, D]."""
+    x = _c(x_bits, np.uint16)
+    rows, H, D = x.shape
+    out = np.empty_like(x)
+    lib().orc_rope_apply_bf16(_p(x), _p(_c(sin_bits, np.uint16)), _p(_c(cos_bits, np.uint16)), _p(_c(pos, np.int32)),
+                              ctypes.c_int64(rows), ctypes.c_int(H), ctypes.c_int(D), _p(out))
+    return out
+
+
+def rope_apply_f32(x, sin_t, cos_t, pos):
+    x = _c(x, np.float32)
+    rows, H, D = x.shape
+    out = np.empty_like(x)
+    lib().orc_rope_apply_f32(_p(x), _p(_c(sin_t, np.float32)), _p(_c(cos_t, np.float32)), _p(_c(pos, np.int32)),
+                             ctypes.c_int64(rows), ctypes.c_int(H), ctypes.c_int(D), _p(out))
+    return out
+

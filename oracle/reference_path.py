@@ -138,3 +138,30 @@ def deltanet_decode_step(q_t, k_t, v_t, g_t, b_t, state):
     state = state + k_t.unsqueeze(-1) * delta.unsqueeze(-2)
     out = q_t.reshape(B * nv, 1, dk).bmm(state.reshape(B * nv, dk, dv)).reshape(B, nv, dv)
     return out, state
+
+
+def rope_tables(dim, base, length, dtype=torch.bfloat16):
+    """sin/cos tables [length, dim/2]: fp32 throughout, cast at the end (rope.rs:100-122)."""
+    half = dim // 2
+    positions = torch.arange(half, dtype=torch.float32)
+    exponents = positions * 2.0 / float(dim)
+    inv_freq = torch.full([half], float(base), dtype=torch.float32).pow(-exponents)
+    pos = torch.arange(length, dtype=torch.float32)
+    angles = pos.unsqueeze(-1).matmul(inv_freq.unsqueeze(0))
+    return angles.sin().to(dtype), angles.cos().to(dtype)
+
+
+def rope_apply(x, sin_full, cos_full, position_ids):
+    """x [B, S, H, D] in the tables' dtype; position_ids int64 [S] (rope.rs:150-248): index_select on the
+    tables, unsqueeze the head axis, then x1*cos - x2*sin and x1*sin + x2*cos as separate tensor ops."""
+    half = x.shape[-1] // 2
+    sin = sin_full.index_select(0, position_ids).unsqueeze(1).unsqueeze(0)
+    cos = cos_full.index_select(0, position_ids).unsqueeze(1).unsqueeze(0)
+    x1 = x.narrow(-1, 0, half)
+    x2 = x.narrow(-1, half, half)
+    sin_e = sin.expand_as(x1)
+    cos_e = cos.expand_as(x1)
+    x1r = x1 * cos_e - x2 * sin_e
+    x2r = x1 * sin_e + x2 * cos_e
+    return torch.cat([x1r, x2r], -1)
+

@@ -12,6 +12,8 @@ oracle and not with anything from this repository's kernels:
                    scale, mask, softmax, matmul; llama.rs:1023-1119) on small cases
   deltanet.npz     the reference's decode-step op sequence (qwen3_5.rs:725-751) iterated
                    over a few tokens
+  rope.npz         the reference's table construction and rotation op sequence (rope.rs:100-122,
+                   206-248) on bf16 and fp32 tensors, bases 10000 and 1e6, positions up to 8191
 
 Inputs come from numpy's Philox generator so the file is reproducible.
 """
@@ -156,7 +158,34 @@ def make_deltanet():
                         state=st.numpy())
 
 
+def make_rope():
+    r = gen(6)
+    out = {}
+    for tag, base, D in (("a", 10000.0, 128), ("b", 1000000.0, 128), ("c", 10000.0, 64)):
+        L = 8192
+        pos = np.concatenate([[0, 1, 2, 255, 256, 257], r.integers(0, L, 10), [L - 1]]).astype(np.int64)
+        S, H = len(pos), 2
+        x = torch.from_numpy(r.standard_normal((1, S, H, D)).astype(np.float32))
+        x[0, 0, 0, :4] = torch.tensor([0.0, -0.0, 8.0, -3.5])
+        for dt_name, dt in (("bf16", torch.bfloat16), ("f32", torch.float32)):
+            sin, cos = ref.rope_tables(D, base, L, dt)
+            xd = x.to(dt)
+            y = ref.rope_apply(xd, sin, cos, torch.from_numpy(pos))
+            sel = torch.from_numpy(pos)
+            if dt == torch.bfloat16:
+                bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+                out[f"{tag}_{dt_name}_x"], out[f"{tag}_{dt_name}_y"] = bits(xd), bits(y)
+                out[f"{tag}_{dt_name}_sin"], out[f"{tag}_{dt_name}_cos"] = bits(sin.index_select(0, sel)), bits(cos.index_select(0, sel))
+            else:
+                out[f"{tag}_{dt_name}_x"], out[f"{tag}_{dt_name}_y"] = xd.numpy(), y.numpy()
+                out[f"{tag}_{dt_name}_sin"], out[f"{tag}_{dt_name}_cos"] = sin.index_select(0, sel).numpy(), cos.index_select(0, sel).numpy()
+        out[f"{tag}_pos"] = pos
+        out[f"{tag}_base"] = np.float64(base)
+    np.savez_compressed(os.path.join(HERE, "rope.npz"), **out)
+
+
 if __name__ == "__main__":
+    make_rope()
     make_int8()
     make_fp8()
     make_attention()
