@@ -1,0 +1,302 @@
+// Block pool, paged per-sequence cache and ragged-batch decode step (see block_pool.hpp).  Host code only.
+#include "block_pool.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <cstdio>
+
+namespace hs {
+
+namespace {
+Status err(int code, const std::string &m) { return Status{code, m}; }
+Status from_abi(int rc) { return rc == HS_OK ? Status{} : Status{rc, hs_attn_last_error()}; }
+Status hip_err(hipError_t e, const char *what) {
+    return e == hipSuccess ? Status{} : Status{HS_ERR_LAUNCH, std::string(what) + ": " + hipGetErrorString(e)};
+}
+Status overflow(int32_t n, size_t start, size_t cap) {
+    char buf[200];
+    snprintf(buf, sizeof(buf), "Cache overflow: trying to cache %d tokens starting at position %zu, but max_seq_len is %zu", n,
+             start, cap);
+    return err(HS_ERR_OVERFLOW, buf);
+}
+}  // namespace
+
+std::string CacheOwner::str() const {
+    switch (kind) {
+        case Stateless: return "Stateless(" + std::to_string(id) + ")";
+        case Session: return "Session(\"" + name + "\")";
+        default: return "Training(\"" + name + "\", " + std::to_string(id) + ")";
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ BlockPool
+
+BlockPool::BlockPool(size_t num_blocks, int32_t heads, int32_t dim) : total_(num_blocks), heads_(heads), dim_(dim) {
+    free_list_.reserve(num_blocks);
+    for (size_t id = 0; id < num_blocks; ++id) free_list_.push_back((BlockId)id);  // pop() hands out the highest id first
+    owner_.resize(num_blocks);
+}
+
+BlockPool::~BlockPool() {
+    if (codes_) (void)hipFree(codes_);
+    if (scales_) (void)hipFree(scales_);
+}
+
+Status BlockPool::allocate(const CacheOwner &owner, BlockId *id) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (free_list_.empty())
+        return err(HS_ERR_POOL_EXHAUSTED, "block pool exhausted (all " + std::to_string(total_) + " blocks in use)");
+    *id = free_list_.back();
+    free_list_.pop_back();
+    owner_[(size_t)*id] = std::make_unique<CacheOwner>(owner);
+    return {};
+}
+
+Status BlockPool::free(const CacheOwner &owner, BlockId id) {
+    std::lock_guard<std::mutex> g(mu_);
+    if (id < 0 || (size_t)id >= total_) return err(HS_ERR_INVALID_ARGUMENT, "Invalid block ID: " + std::to_string(id));
+    const auto &cur = owner_[(size_t)id];
+    if (!cur) return err(HS_ERR_INVALID_ARGUMENT, "double-free of block " + std::to_string(id) + " (already in free list)");
+    if (!(*cur == owner))
+        return err(HS_ERR_INVALID_ARGUMENT, "cross-owner block free rejected: block " + std::to_string(id) + " owned by " +
+                                                cur->str() + ", freed by " + owner.str());
+    owner_[(size_t)id].reset();
+    free_list_.push_back(id);
+    return {};
+}
+
+const CacheOwner *BlockPool::owner_of(BlockId id) const {
+    std::lock_guard<std::mutex> g(mu_);
+    if (id < 0 || (size_t)id >= total_) return nullptr;
+    return owner_[(size_t)id].get();
+}
+
+size_t BlockPool::used_blocks() const {
+    std::lock_guard<std::mutex> g(mu_);
+    return total_ - free_list_.size();
+}
+
+size_t BlockPool::free_block_count() const {
+    std::lock_guard<std::mutex> g(mu_);
+    return free_list_.size();
+}
+
+size_t BlockPool::used_memory() const { return used_blocks() * block_bytes(); }
+
+Status BlockPool::ensure_device() {
+    std::lock_guard<std::mutex> g(mu_);
+    if (codes_) return {};
+    if (total_ == 0) return err(HS_ERR_INVALID_ARGUMENT, "the pool has no blocks");
+    const size_t cb = total_ * (size_t)heads_ * kBlockSize * (size_t)dim_;
+    const size_t sb = total_ * (size_t)heads_ * kBlockSize * sizeof(float);
+    hipError_t e;
+    if ((e = hipMalloc((void **)&codes_, cb)) != hipSuccess) return hip_err(e, "allocating the block pool");
+    if ((e = hipMalloc((void **)&scales_, sb)) != hipSuccess) {
+        (void)hipFree(codes_);
+        codes_ = nullptr;
+        return hip_err(e, "allocating the block pool");
+    }
+    // all-zero blocks, as the reference's pre-zeroed pool (kv_cache.rs:551-556)
+    if ((e = hipMemset(codes_, 0, cb)) != hipSuccess || (e = hipMemset(scales_, 0, sb)) != hipSuccess)
+        return hip_err(e, "clearing the block pool");
+    return {};
+}
+
+hs_kv_layout BlockPool::layout(const int32_t *k_table, const int32_t *v_table, int32_t stride) const {
+    hs_kv_layout l{};
+    l.code_stride_head = (int64_t)kBlockSize * dim_;
+    l.code_stride_seq = l.code_stride_head * heads_;
+    l.scale_stride_head = (int64_t)kBlockSize;
+    l.scale_stride_seq = (int64_t)kBlockSize * heads_;
+    l.capacity_tokens = (int32_t)kBlockSize;
+    l.block_table_stride = stride;
+    l.k_block_table = k_table;
+    l.v_block_table = v_table;
+    return l;
+}
+
+// ---------------------------------------------------------------------------------------- PagedLayerKVCache
+
+PagedLayerKVCache::PagedLayerKVCache(size_t max_len, std::shared_ptr<BlockPool> pool, CacheOwner owner)
+    : max_seq_len(max_len), pool_(std::move(pool)), owner_(std::move(owner)) {}
+
+PagedLayerKVCache::~PagedLayerKVCache() {
+    clear();
+    for (void *p : {(void *)table_dev_, (void *)len_dev_, workspace_})
+        if (p) (void)hipFree(p);
+}
+
+Status PagedLayerKVCache::reserve(size_t end_pos) {
+    if (end_pos > max_seq_len) return overflow((int32_t)(end_pos - seq_pos), seq_pos, max_seq_len);
+    const size_t need = (end_pos + kBlockSize - 1) / kBlockSize;
+    while (key_blocks_.size() < need) {
+        BlockId kid, vid;
+        if (Status s = pool_->allocate(owner_, &kid); !s.ok()) return s;
+        if (Status s = pool_->allocate(owner_, &vid); !s.ok()) {
+            (void)pool_->free(owner_, kid);  // keep the pair balanced: the key block is not leaked
+            return s;
+        }
+        key_blocks_.push_back(kid);
+        value_blocks_.push_back(vid);
+    }
+    return {};
+}
+
+Status PagedLayerKVCache::sync_table() {
+    const size_t max_blocks = (max_seq_len + kBlockSize - 1) / kBlockSize;
+    hipError_t e;
+    if (!table_dev_) {
+        if ((e = hipMalloc((void **)&table_dev_, 2 * std::max<size_t>(max_blocks, 1) * sizeof(int32_t))) != hipSuccess)
+            return hip_err(e, "allocating the block table");
+        if ((e = hipMalloc((void **)&len_dev_, sizeof(int32_t))) != hipSuccess) return hip_err(e, "allocating the length");
+        table_synced_ = 0;
+    }
+    if (table_synced_ > key_blocks_.size()) table_synced_ = 0;  // blocks were returned: rewrite what is left
+    const size_t n = key_blocks_.size() - table_synced_;
+    if (n) {
+        if ((e = hipMemcpy(table_dev_ + table_synced_, key_blocks_.data() + table_synced_, n * sizeof(int32_t),
+                           hipMemcpyHostToDevice)) != hipSuccess ||
+            (e = hipMemcpy(table_dev_ + max_blocks + table_synced_, value_blocks_.data() + table_synced_, n * sizeof(int32_t),
+                           hipMemcpyHostToDevice)) != hipSuccess)
+            return hip_err(e, "uploading the block table");
+        table_synced_ = key_blocks_.size();
+    }
+    return {};
+}
+
+Status PagedLayerKVCache::update(const void *new_keys, const void *new_values, int dtype, int32_t seq_len, size_t start_pos,
+                                 hs_stream_t stream) {
+    if (seq_len < 0) return err(HS_ERR_INVALID_ARGUMENT, "negative seq_len");
+    const size_t end_pos = start_pos + (size_t)seq_len;
+    if (end_pos > max_seq_len) return overflow(seq_len, start_pos, max_seq_len);
+    if (Status s = reserve(end_pos); !s.ok()) return s;
+    if (seq_len > 0) {
+        if (Status s = pool_->ensure_device(); !s.ok()) return s;
+        if (Status s = sync_table(); !s.ok()) return s;
+        const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
+        const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
+        int rc = hs_kv_quantize_int8(new_keys, new_values, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(),
+                                     &l, nullptr, (int32_t)start_pos, 1, seq_len, pool_->num_kv_heads(), pool_->head_dim(), stream);
+        if (rc != HS_OK) return from_abi(rc);
+    }
+    seq_pos = end_pos;
+    return {};
+}
+
+Status PagedLayerKVCache::get_dense(void *keys_out, void *values_out, int dtype, hs_stream_t stream) {
+    if (seq_pos == 0) return err(HS_ERR_INVALID_ARGUMENT, "Cache is empty");
+    if (Status s = sync_table(); !s.ok()) return s;
+    const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
+    const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
+    int rc = hs_kv_dequantize(pool_->codes(), pool_->scales(), 0, &l, 0, keys_out, dtype, 1, (int32_t)seq_pos,
+                              pool_->num_kv_heads(), pool_->head_dim(), stream);
+    if (rc == HS_OK)
+        rc = hs_kv_dequantize(pool_->codes(), pool_->scales(), 0, &l, 1, values_out, dtype, 1, (int32_t)seq_pos,
+                              pool_->num_kv_heads(), pool_->head_dim(), stream);
+    return from_abi(rc);
+}
+
+Status PagedLayerKVCache::decode_attention(const void *q, void *out, int32_t hq, float scale, hs_stream_t stream) {
+    if (seq_pos == 0) return err(HS_ERR_INVALID_ARGUMENT, "Cache is empty");
+    if (Status s = sync_table(); !s.ok()) return s;
+    const int32_t heads = pool_->num_kv_heads(), dim = pool_->head_dim();
+    const size_t need = hs_decode_attn_workspace_bytes(1, hq, heads, dim, (int32_t)seq_pos);
+    hipError_t e;
+    if (need > workspace_bytes_) {
+        if (workspace_) (void)hipFree(workspace_);
+        workspace_ = nullptr;
+        workspace_bytes_ = 0;
+        if ((e = hipMalloc(&workspace_, need)) != hipSuccess) return hip_err(e, "allocating the workspace");
+        workspace_bytes_ = need;
+    }
+    const int32_t len = (int32_t)seq_pos;
+    if ((e = hipMemcpy(len_dev_, &len, sizeof(len), hipMemcpyHostToDevice)) != hipSuccess) return hip_err(e, "uploading the length");
+    const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
+    const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
+    return from_abi(hs_decode_attn_int8(q, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l, len_dev_, out,
+                                        workspace_, workspace_bytes_, 1, hq, heads, dim, len, scale, stream));
+}
+
+void PagedLayerKVCache::clear() {
+    for (BlockId id : key_blocks_) (void)pool_->free(owner_, id);
+    for (BlockId id : value_blocks_) (void)pool_->free(owner_, id);
+    key_blocks_.clear();
+    value_blocks_.clear();
+    table_synced_ = 0;
+    seq_pos = 0;
+}
+
+void PagedLayerKVCache::truncate_to(size_t pos) {
+    if (pos >= seq_pos) return;
+    const size_t needed = pos == 0 ? 0 : (pos - 1) / kBlockSize + 1;
+    if (key_blocks_.size() > needed) {
+        for (size_t i = needed; i < key_blocks_.size(); ++i) (void)pool_->free(owner_, key_blocks_[i]);
+        for (size_t i = needed; i < value_blocks_.size(); ++i) (void)pool_->free(owner_, value_blocks_[i]);
+        key_blocks_.resize(needed);
+        value_blocks_.resize(needed);
+        table_synced_ = std::min(table_synced_, needed);
+    }
+    seq_pos = pos;
+}
+
+// ----------------------------------------------------------------------------------------------- PagedBatch
+
+PagedBatch::PagedBatch(std::shared_ptr<BlockPool> pool) : pool_(std::move(pool)) {}
+
+PagedBatch::~PagedBatch() {
+    for (void *p : {(void *)tables_dev_, workspace_})
+        if (p) (void)hipFree(p);
+}
+
+Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const void *q, const void *k_new, const void *v_new,
+                               int dtype, void *out, int32_t hq, float scale, hs_stream_t stream) {
+    if (n <= 0) return err(HS_ERR_INVALID_ARGUMENT, "empty batch");
+    size_t max_len = 0, stride = 1;
+    for (int32_t i = 0; i < n; ++i) {
+        PagedLayerKVCache *r = rows[i];
+        if (!r || r->pool().get() != pool_.get()) return err(HS_ERR_INVALID_ARGUMENT, "row " + std::to_string(i) + " is not a cache of this pool");
+        if (r->seq_pos + 1 > r->max_seq_len) return overflow(1, r->seq_pos, r->max_seq_len);
+    }
+    for (int32_t i = 0; i < n; ++i) {  // all block pairs first: a refusal leaves every seq_pos where it was
+        if (Status s = rows[i]->reserve(rows[i]->seq_pos + 1); !s.ok()) return s;
+        max_len = std::max(max_len, rows[i]->seq_pos + 1);
+        stride = std::max(stride, rows[i]->num_blocks());
+    }
+    if (Status s = pool_->ensure_device(); !s.ok()) return s;
+    std::vector<int32_t> host((size_t)n * stride * 2 + (size_t)n, 0);
+    int32_t *kt = host.data(), *vt = kt + (size_t)n * stride, *lens = vt + (size_t)n * stride;
+    for (int32_t i = 0; i < n; ++i) {
+        std::copy(rows[i]->key_blocks().begin(), rows[i]->key_blocks().end(), kt + (size_t)i * stride);
+        std::copy(rows[i]->value_blocks().begin(), rows[i]->value_blocks().end(), vt + (size_t)i * stride);
+        lens[i] = (int32_t)(rows[i]->seq_pos + 1);
+    }
+    hipError_t e;
+    if (host.size() > tables_cap_) {
+        if (tables_dev_) (void)hipFree(tables_dev_);
+        tables_dev_ = nullptr;
+        tables_cap_ = 0;
+        if ((e = hipMalloc((void **)&tables_dev_, host.size() * 2 * sizeof(int32_t))) != hipSuccess) return hip_err(e, "allocating the block tables");
+        tables_cap_ = host.size() * 2;
+    }
+    if ((e = hipMemcpy(tables_dev_, host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice)) != hipSuccess)
+        return hip_err(e, "uploading the block tables");
+    const int32_t heads = pool_->num_kv_heads(), dim = pool_->head_dim();
+    const size_t need = hs_decode_attn_workspace_bytes(n, hq, heads, dim, (int32_t)max_len);
+    if (need > workspace_bytes_) {
+        if (workspace_) (void)hipFree(workspace_);
+        workspace_ = nullptr;
+        workspace_bytes_ = 0;
+        if ((e = hipMalloc(&workspace_, need)) != hipSuccess) return hip_err(e, "allocating the workspace");
+        workspace_bytes_ = need;
+    }
+    const hs_kv_layout l = pool_->layout(tables_dev_, tables_dev_ + (size_t)n * stride, (int32_t)stride);
+    int rc = hs_decode_step_int8(q, k_new, v_new, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
+                                 tables_dev_ + 2 * (size_t)n * stride, out, workspace_, workspace_bytes_, n, hq, heads, dim,
+                                 (int32_t)max_len, scale, stream);
+    if (rc != HS_OK) return from_abi(rc);
+    for (int32_t i = 0; i < n; ++i) rows[i]->seq_pos += 1;
+    return {};
+}
+
+}  // namespace hs

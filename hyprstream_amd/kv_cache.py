@@ -17,7 +17,14 @@ EXPORTS = [
     "hs_cache_get_view", "hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_clear", "hs_cache_truncate_to",
     "hs_cache_is_initialized", "hs_cache_memory_usage", "hs_cache_quant_type", "hs_cache_decode_attention",
     "hs_cache_decode_step", "hs_cache_prefill",
+    "hs_pool_create", "hs_pool_destroy", "hs_pool_last_error", "hs_pool_allocate", "hs_pool_free", "hs_pool_owner_of",
+    "hs_pool_used_blocks", "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory",
+    "hs_paged_cache_create", "hs_paged_cache_destroy", "hs_paged_cache_last_error", "hs_paged_cache_update",
+    "hs_paged_cache_get_dense", "hs_paged_cache_decode_attention", "hs_paged_cache_clear", "hs_paged_cache_truncate_to",
+    "hs_paged_cache_seq_pos", "hs_paged_cache_num_blocks", "hs_paged_batch_decode_step",
 ]
+BLOCK_SIZE = 256  # tokens per pool block
+STATELESS, SESSION, TRAINING = 0, 1, 2  # owner kinds
 
 _lib = None
 
@@ -32,8 +39,19 @@ def lib():
         L.hs_cache_create.restype = ctypes.c_void_p
         L.hs_cache_create.argtypes = [ctypes.c_int64, ctypes.c_int]
         L.hs_cache_last_error.restype = ctypes.c_char_p
-        for f in ("hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_memory_usage"):
+        for f in ("hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_memory_usage", "hs_pool_used_blocks",
+                  "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory", "hs_paged_cache_seq_pos",
+                  "hs_paged_cache_num_blocks"):
             getattr(L, f).restype = ctypes.c_int64
+        L.hs_pool_create.restype = ctypes.c_void_p
+        L.hs_pool_create.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+        L.hs_pool_last_error.restype = ctypes.c_char_p
+        L.hs_paged_cache_create.restype = ctypes.c_void_p
+        L.hs_paged_cache_create.argtypes = [ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_char_p]
+        L.hs_paged_cache_last_error.restype = ctypes.c_char_p
+        L.hs_pool_allocate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_char_p,
+                                       ctypes.POINTER(ctypes.c_int32)]
+        L.hs_pool_free.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_char_p, ctypes.c_int32]
         for f in EXPORTS:
             if f != "hs_cache_create":
                 fn = getattr(L, f)
@@ -131,3 +149,145 @@ class LayerKVCache:
                                            k.shape[2], D, ctypes.c_int64(start_pos), ctypes.c_float(softmax_scale),
                                            hb._stream()))
         return out
+
+
+# ------------------------------------------------------------------------------------------- paged mode
+def _owner(owner):
+    """owner: int -> Stateless(id); str -> Session(name); (name, id) -> Training."""
+    if isinstance(owner, int):
+        return STATELESS, owner, None
+    if isinstance(owner, str):
+        return SESSION, 0, owner.encode()
+    name, ident = owner
+    return TRAINING, ident, name.encode()
+
+
+class BlockPoolExhausted(CacheError):
+    """Fail-soft: the pool has no free block; retry once other sequences have released theirs."""
+
+
+class BlockPool:
+    """BlockPool of the reference (kv_cache.rs:508-676) over int8 blocks; bookkeeping works without a GPU."""
+
+    def __init__(self, num_blocks, num_kv_heads, head_dim):
+        self._h = ctypes.c_void_p(lib().hs_pool_create(num_blocks, num_kv_heads, head_dim))
+        if not self._h:
+            raise ValueError("bad pool shape")
+        self.num_kv_heads, self.head_dim = num_kv_heads, head_dim
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hs_pool_destroy(self._h)
+            self._h = None
+
+    def _check(self, rc):
+        if rc != hb.HS_OK:
+            cls = BlockPoolExhausted if rc == hb.HS_ERR_POOL_EXHAUSTED else CacheError
+            raise cls(rc, lib().hs_pool_last_error(self._h).decode())
+
+    def allocate(self, owner):
+        kind, ident, name = _owner(owner)
+        out = ctypes.c_int32(-1)
+        self._check(lib().hs_pool_allocate(self._h, kind, ident, name, ctypes.byref(out)))
+        return out.value
+
+    def free(self, owner, block_id):
+        kind, ident, name = _owner(owner)
+        self._check(lib().hs_pool_free(self._h, kind, ident, name, block_id))
+
+    def owner_of(self, block_id):
+        kind, ident = ctypes.c_int(), ctypes.c_uint64()
+        name = ctypes.create_string_buffer(256)
+        if not lib().hs_pool_owner_of(self._h, ctypes.c_int32(block_id), ctypes.byref(kind), ctypes.byref(ident), name,
+                                      ctypes.c_size_t(256)):
+            return None
+        if kind.value == STATELESS:
+            return ident.value
+        if kind.value == SESSION:
+            return name.value.decode()
+        return (name.value.decode(), ident.value)
+
+    def used_blocks(self):
+        return lib().hs_pool_used_blocks(self._h)
+
+    def free_block_count(self):
+        return lib().hs_pool_free_block_count(self._h)
+
+    def total_blocks(self):
+        return lib().hs_pool_total_blocks(self._h)
+
+    def used_memory(self):
+        return lib().hs_pool_used_memory(self._h)
+
+
+class PagedLayerKVCache:
+    """LayerKVCache::new_paged (kv_cache.rs:1100-1120): one sequence, int8 blocks from a shared pool."""
+
+    def __init__(self, max_seq_len, pool, owner):
+        kind, ident, name = _owner(owner)
+        self.pool = pool  # keeps the Python pool object alive as long as the cache
+        self._h = ctypes.c_void_p(lib().hs_paged_cache_create(max_seq_len, pool._h, kind, ident, name))
+        if not self._h:
+            raise ValueError("bad max_seq_len / pool")
+
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().hs_paged_cache_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    def _check(self, rc):
+        if rc != hb.HS_OK:
+            cls = BlockPoolExhausted if rc == hb.HS_ERR_POOL_EXHAUSTED else CacheError
+            raise cls(rc, lib().hs_paged_cache_last_error(self._h).decode())
+
+    @property
+    def seq_pos(self):
+        return lib().hs_paged_cache_seq_pos(self._h)
+
+    @property
+    def num_blocks(self):
+        return lib().hs_paged_cache_num_blocks(self._h)
+
+    def update(self, new_keys, new_values, start_pos):
+        if new_keys.dim() != 4 or new_keys.shape[0] != 1:
+            raise CacheError(hb.HS_ERR_INVALID_ARGUMENT, "Expected [1, S, H, D] keys, got %s" % list(new_keys.shape))
+        k, v = new_keys.contiguous(), new_values.contiguous()
+        self._check(lib().hs_paged_cache_update(self._h, hb._ptr(k), hb._ptr(v), hb._dtype_code(k), k.shape[1],
+                                                ctypes.c_int64(start_pos), hb._stream()))
+
+    def get(self, dtype=None):
+        import torch
+        dtype = dtype or torch.bfloat16
+        k = torch.empty(1, max(self.seq_pos, 0), self.pool.num_kv_heads, self.pool.head_dim, dtype=dtype, device="cuda")
+        v = torch.empty_like(k)
+        self._check(lib().hs_paged_cache_get_dense(self._h, hb._ptr(k), hb._ptr(v), hb._dtype_code(k), hb._stream()))
+        return k, v
+
+    def decode_attention(self, q, softmax_scale):
+        import torch
+        out = torch.empty_like(q)
+        self._check(lib().hs_paged_cache_decode_attention(self._h, hb._ptr(q), hb._ptr(out), q.shape[1],
+                                                          ctypes.c_float(softmax_scale), hb._stream()))
+        return out
+
+    def clear(self):
+        lib().hs_paged_cache_clear(self._h)
+
+    def truncate_to(self, pos):
+        lib().hs_paged_cache_truncate_to(self._h, ctypes.c_int64(pos))
+
+
+def paged_batch_decode_step(pool, rows, q, k_new, v_new, softmax_scale):
+    """One launch for all rows: each caches its new token and attends its own history.  q [n, Hq, D] bf16."""
+    import torch
+    n = len(rows)
+    arr = (ctypes.c_void_p * n)(*[r._h for r in rows])
+    out = torch.empty_like(q)
+    k, v = k_new.contiguous(), v_new.contiguous()
+    rc = lib().hs_paged_batch_decode_step(pool._h, arr, n, hb._ptr(q), hb._ptr(k), hb._ptr(v), hb._dtype_code(k),
+                                          hb._ptr(out), q.shape[1], ctypes.c_float(softmax_scale), hb._stream())
+    pool._check(rc)
+    return out
+

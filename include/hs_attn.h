@@ -58,7 +58,8 @@ enum hs_status {
     HS_ERR_INVALID_ARGUMENT = 1, /* null pointer, bad shape, unsupported head_dim, misaligned stride */
     HS_ERR_OVERFLOW = 2,         /* write past capacity_tokens (kv_cache.rs:1288-1294 "Cache overflow") */
     HS_ERR_WORKSPACE = 3,        /* workspace too small */
-    HS_ERR_LAUNCH = 4            /* hipGetLastError() after the launch */
+    HS_ERR_LAUNCH = 4,           /* hipGetLastError() after the launch */
+    HS_ERR_POOL_EXHAUSTED = 5    /* host-side block pool has no free block (fail-soft, hs_kv_cache.h) */
 };
 
 enum hs_dtype { HS_BF16 = 0, HS_F32 = 1, HS_F16 = 2 };

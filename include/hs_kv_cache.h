@@ -60,6 +60,57 @@ HS_API int hs_cache_prefill(hs_cache *c, const void *q, const void *new_keys, co
                             int32_t batch, int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                             int32_t head_dim, int64_t start_pos, float softmax_scale, hs_stream_t stream);
 
+/* ---- paged mode: shared block pool, per-sequence paged caches, ragged-batch decode step -----------------
+ * BlockPool (kv_cache.rs:508-676): 256-token blocks, LIFO free list, every block tagged with its owner.
+ * An owner is (kind, id, name) as CacheOwner (kv_cache.rs:49-82): kind 0 = Stateless(id), 1 = Session(name),
+ * 2 = Training(name, id).  Allocation on an empty pool returns HS_ERR_POOL_EXHAUSTED with the message
+ * "block pool exhausted (all N blocks in use)" (BlockPoolExhausted, kv_cache.rs:489-506): fail-soft, the
+ * caller may retry later.  Freeing someone else's block, a free block or an invalid id is refused and
+ * changes nothing (kv_cache.rs:606-637).  The bookkeeping needs no GPU; device memory (int8 codes +
+ * per-token scales for every block) is allocated at the first update. */
+typedef struct hs_pool hs_pool;
+typedef struct hs_paged_cache hs_paged_cache;
+
+HS_API hs_pool *hs_pool_create(int64_t num_blocks, int32_t num_kv_heads, int32_t head_dim);
+HS_API void hs_pool_destroy(hs_pool *p); /* the blocks live until the last cache of the pool is destroyed */
+HS_API const char *hs_pool_last_error(const hs_pool *p);
+HS_API int hs_pool_allocate(hs_pool *p, int owner_kind, uint64_t owner_id, const char *owner_name, int32_t *block_id);
+HS_API int hs_pool_free(hs_pool *p, int owner_kind, uint64_t owner_id, const char *owner_name, int32_t block_id);
+/* 1 and the owner's fields when the block is in use, 0 when it is free or invalid */
+HS_API int hs_pool_owner_of(const hs_pool *p, int32_t block_id, int *owner_kind, uint64_t *owner_id,
+                            char *owner_name, size_t owner_name_cap);
+HS_API int64_t hs_pool_used_blocks(const hs_pool *p);
+HS_API int64_t hs_pool_free_block_count(const hs_pool *p);
+HS_API int64_t hs_pool_total_blocks(const hs_pool *p);
+HS_API int64_t hs_pool_used_memory(const hs_pool *p);
+
+/* LayerKVCache::new_paged(max_seq_len, pool, owner), kv_cache.rs:1100-1120: one sequence, int8 format.
+ * update takes [1, seq_len, num_kv_heads, head_dim]; blocks are taken in (K, V) pairs and a failed pair is
+ * rolled back (kv_cache.rs:1456-1471); clear, truncate_to and destroy return blocks (kv_cache.rs:1679-1750,
+ * 1873-1891). */
+HS_API hs_paged_cache *hs_paged_cache_create(int64_t max_seq_len, hs_pool *pool, int owner_kind, uint64_t owner_id,
+                                             const char *owner_name);
+HS_API void hs_paged_cache_destroy(hs_paged_cache *c);
+HS_API const char *hs_paged_cache_last_error(const hs_paged_cache *c);
+HS_API int hs_paged_cache_update(hs_paged_cache *c, const void *new_keys, const void *new_values, int dtype,
+                                 int32_t seq_len, int64_t start_pos, hs_stream_t stream);
+HS_API int hs_paged_cache_get_dense(hs_paged_cache *c, void *keys_out, void *values_out, int dtype, hs_stream_t stream);
+HS_API int hs_paged_cache_decode_attention(hs_paged_cache *c, const void *q, void *out, int32_t num_q_heads,
+                                           float softmax_scale, hs_stream_t stream);
+HS_API void hs_paged_cache_clear(hs_paged_cache *c);
+HS_API void hs_paged_cache_truncate_to(hs_paged_cache *c, int64_t pos);
+HS_API int64_t hs_paged_cache_seq_pos(const hs_paged_cache *c);
+HS_API int64_t hs_paged_cache_num_blocks(const hs_paged_cache *c); /* K blocks held (= V blocks held) */
+
+/* One decode step over n paged caches of one pool, one kernel launch: each row caches one new token and attends
+ * all its tokens (what forward_batched does with pad + cat + additive mask, llama.rs:710-844, 2544-2572).
+ * q, out: bf16 [n, num_q_heads, head_dim]; k_new, v_new: [n, 1, num_kv_heads, head_dim] in dtype.
+ * If a row needs a block pair the pool cannot give, the call fails with HS_ERR_POOL_EXHAUSTED before any launch
+ * and no row's seq_pos moves; the message is read with hs_pool_last_error. */
+HS_API int hs_paged_batch_decode_step(hs_pool *pool, hs_paged_cache *const *rows, int32_t n, const void *q,
+                                      const void *k_new, const void *v_new, int dtype, void *out,
+                                      int32_t num_q_heads, float softmax_scale, hs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
