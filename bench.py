@@ -287,6 +287,8 @@ def main():
     v_new = make_source(torch, gen, (B, 1, Hkv, D), sigma, outliers, dev)
     out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=dev)
     max_len = T
+    if ragged:  # the host built the lengths, so it can tell the library how many tokens the batch holds
+        layout.total_tokens_hint = int(lens.sum().item())
     ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, max_len), dtype=torch.uint8, device=dev)
     scale = 1.0 / float(np.sqrt(D))
     quant = hb.kv_quantize_fp8 if fp8 else hb.kv_quantize_int8
@@ -333,8 +335,7 @@ def main():
     # ---- roofline of the dominant kernel alone: HIP events (torch's, recorded on the stream the library
     # launches on) around each launch.  When every sequence is one chunk the whole step IS that one launch
     # (new-token write + attention + output); otherwise the split-K kernel is timed without the merge.
-    per_chunk = B * Hq * (D + 2) * 4
-    nchunks = max(1, ws.numel() // per_chunk)  # the workspace is nchunks partial records, rounded up to 256 B
+    nchunks = hb.decode_num_chunks(B, Hkv, max_len, layout.total_tokens_hint)
     single = nchunks == 1
     write_bytes = B * Hkv * D * (2 * 2 + 2 * 1) + (0 if fp8 else B * Hkv * 2 * 4)
     kern_bytes = step_bytes if single else step_bytes - write_bytes

@@ -24,7 +24,7 @@ EXPORTS = [
     "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_deltanet_forward",
-    "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_decode_step_int8_rope",
+    "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
 ]
 
 
@@ -39,6 +39,7 @@ class KvLayout(ctypes.Structure):
         ("block_table_stride", ctypes.c_int32),
         ("k_block_table", ctypes.c_void_p),
         ("v_block_table", ctypes.c_void_p),
+        ("total_tokens_hint", ctypes.c_int64),
     ]
 
 
@@ -73,14 +74,14 @@ def check(rc):
 def contiguous_layout(Hkv, capacity_tokens, D, scale_pad=4):
     """Head-major cache of one buffer per tensor: codes [B, Hkv, cap, D], scales [B, Hkv, cap_padded]."""
     cap_s = (capacity_tokens + scale_pad - 1) // scale_pad * scale_pad
-    return KvLayout(Hkv * capacity_tokens * D, capacity_tokens * D, Hkv * cap_s, cap_s, capacity_tokens, 0, None, None)
+    return KvLayout(Hkv * capacity_tokens * D, capacity_tokens * D, Hkv * cap_s, cap_s, capacity_tokens, 0, None, None, 0)
 
 
 def paged_layout(Hkv, block_tokens, D, k_table, v_table):
     """Pool of blocks [nblocks, Hkv, block_tokens, D]; tables are int32 device tensors [B, max_blocks]."""
     assert k_table.dtype.is_signed and k_table.element_size() == 4 and k_table.is_contiguous()
     return KvLayout(Hkv * block_tokens * D, block_tokens * D, Hkv * block_tokens, block_tokens, block_tokens,
-                    k_table.shape[1], k_table.data_ptr(), v_table.data_ptr())
+                    k_table.shape[1], k_table.data_ptr(), v_table.data_ptr(), 0)
 
 
 def _ptr(t):
@@ -143,6 +144,10 @@ def kv_dequantize(codes, scales, fp8, layout, which_table, out):
     B, T, Hkv, D = out.shape
     check(lib().hs_kv_dequantize(_ptr(codes), _ptr(scales), int(fp8), ctypes.byref(layout), int(which_table),
                                  _ptr(out), _dtype_code(out), B, T, Hkv, D, _stream()))
+
+
+def decode_num_chunks(B, Hkv, max_seq_len, total_tokens_hint=0):
+    return lib().hs_decode_attn_num_chunks(B, Hkv, max_seq_len, ctypes.c_int64(total_tokens_hint))
 
 
 def decode_workspace_bytes(B, Hq, Hkv, D, max_seq_len):

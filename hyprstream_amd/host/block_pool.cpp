@@ -290,7 +290,8 @@ Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const 
         if ((e = hipMalloc(&workspace_, need)) != hipSuccess) return hip_err(e, "allocating the workspace");
         workspace_bytes_ = need;
     }
-    const hs_kv_layout l = pool_->layout(tables_dev_, tables_dev_ + (size_t)n * stride, (int32_t)stride);
+    hs_kv_layout l = pool_->layout(tables_dev_, tables_dev_ + (size_t)n * stride, (int32_t)stride);
+    for (int32_t i = 0; i < n; ++i) l.total_tokens_hint += lens[i];  // lets the kernel library balance a ragged batch
     int rc = hs_decode_step_int8(q, k_new, v_new, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
                                  tables_dev_ + 2 * (size_t)n * stride, out, workspace_, workspace_bytes_, n, hq, heads, dim,
                                  (int32_t)max_len, scale, stream);

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define HS_ATTN_ABI_VERSION 1
+#define HS_ATTN_ABI_VERSION 2
 
 typedef void *hs_stream_t; /* hipStream_t */
 
@@ -73,6 +73,9 @@ typedef struct hs_kv_layout {
     int32_t block_table_stride; /* entries per sequence in the block tables; 0 = not paged */
     const int32_t *k_block_table; /* device, [B, block_table_stride]; NULL = not paged */
     const int32_t *v_block_table; /* device, may equal k_block_table when K and V pools are separate buffers */
+    int64_t total_tokens_hint;  /* decode only, optional: sum of seq_lens over the batch as the host knows it
+                                   (0 = unknown).  A ragged batch is then cut into chunks of about half the mean
+                                   length so that long sequences do not set the time of the launch. */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */
@@ -142,6 +145,8 @@ HS_API int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8,
  * fp32 accumulation, K/V dequantized on the fly.  workspace: device scratch of at least
  * hs_decode_attn_workspace_bytes(...) bytes, 256-byte aligned, owned by the caller. */
 HS_API size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len);
+/* Chunks per sequence the decode entry points will use for this shape and hint (1 = a step is a single launch). */
+HS_API int32_t hs_decode_attn_num_chunks(int32_t B, int32_t Hkv, int32_t max_seq_len, int64_t total_tokens_hint);
 HS_API int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes,
                         const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
                         const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,

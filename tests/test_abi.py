@@ -30,12 +30,12 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_abi_version_and_empty_error():
-    assert hb.lib().hs_attn_abi_version() == 1
+    assert hb.lib().hs_attn_abi_version() == 2
 
 
 def test_layout_struct_matches_header_size():
     # 4 x int64 + 2 x int32 + 2 pointers
-    assert ctypes.sizeof(hb.KvLayout) == 4 * 8 + 2 * 4 + 2 * 8
+    assert ctypes.sizeof(hb.KvLayout) == 4 * 8 + 2 * 4 + 2 * 8 + 8
 
 
 def _call_quant(layout, B=1, S=1, Hkv=2, D=128, start_pos=0, fake=0x1000):
@@ -115,3 +115,17 @@ def test_cache_host_logic_without_a_gpu():
     n = ctypes.c_void_p(L.hs_cache_create(10, kc.NONE))
     assert L.hs_cache_update(n, p, p, hb.HS_BF16, 1, 1, 8, 128, ctypes.c_int64(0), None) == hb.HS_ERR_INVALID_ARGUMENT
     L.hs_cache_destroy(n)
+
+
+def test_chunk_policy_unsplit_for_uniform_and_split_for_ragged_hint():
+    """The headline shape stays one launch; a batch whose mean length is well below its maximum is cut finer,
+    and the workspace the library asks for covers the finest cut any hint can select."""
+    B, Hq, Hkv, D, T = 64, 32, 8, 128, 8192
+    assert hb.decode_num_chunks(B, Hkv, T) == 1
+    assert hb.decode_num_chunks(B, Hkv, T, B * T) == 1            # hint says uniform
+    n = hb.decode_num_chunks(B, Hkv, T, B * 4352)                 # U[512, 8192] has mean 4352
+    assert 2 <= n <= 16
+    assert hb.decode_num_chunks(2, Hkv, T) > 1                    # few sequences: split for occupancy as before
+    per_chunk = B * Hq * (D + 2) * 4
+    assert hb.decode_workspace_bytes(B, Hq, Hkv, D, T) >= 16 * per_chunk >= n * per_chunk
+

@@ -80,6 +80,26 @@ def test_ragged_uniform_lengths_config2_shape_reduced():
     check(case, 32, 8, 128, label="ragged-uniform")
 
 
+def test_ragged_batch_hint_changes_the_split_not_the_result():
+    """B*Hkv = 512 units (unsplit without a hint) with lengths U[100, 3000]: the hinted call cuts the long
+    sequences into several chunks, merges them, and must agree with the unsplit call and the oracle."""
+    B, Hq, Hkv, D, T = 64, 32, 8, 128, 3000
+    case = wl.decode_case(41, B, Hq, Hkv, D, T, ragged=True, outliers=True, min_len=100)
+    c = build_cache(case, Hkv, D)
+    lens = case["seq_lens"]
+    plain = run_decode(c, case["q_bits"], lens, Hq, max_seq_len=T)
+    lay = hb.contiguous_layout(Hkv, c.cap, D)
+    lay.total_tokens_hint = int(lens.sum())
+    assert hb.decode_num_chunks(B, Hkv, T) == 1 and hb.decode_num_chunks(B, Hkv, T, lay.total_tokens_hint) > 1
+    hinted = run_decode(c, case["q_bits"], lens, Hq, max_seq_len=T, layout=lay)
+    kc, vc, ks, vs = c.canonical(T)
+    want = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), kc, vc, ks, vs, oracle.FMT_INT8, lens, 1.0 / np.sqrt(D))
+    for got in (plain, hinted):
+        d = np.abs(got - want)
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN
+    assert np.abs(plain - hinted).max() < 1e-2  # same math, different summation order and one more bf16 rounding path
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 4), (16, 2), (16, 1), (64, 8)])
 def test_gqa_group_sizes(Hq, Hkv):
     case = wl.decode_case(5, 2, Hq, Hkv, 128, 200)
