@@ -51,7 +51,7 @@ def check(case, Hq, Hkv, D, fp8=False, cap=None, label=""):
 
 
 def test_config1_single_sequence_fp32_source():
-    """B=1, Hq 32 / Hkv 8, D 128, T 2048, K/V fp32 N(0,1) (BASELINE config 1)."""
+    """B=1, Hq 32 / Hkv 8, D 128, T 2048, K/V fp32 N(0,1): the single-sequence benchmark configuration."""
     case = wl.decode_case(1, 1, 32, 8, 128, 2048, bf16_source=False)
     got, want = check(case, 32, 8, 128, label="config1")
     assert np.abs(got - want).max() < 4e-3  # far inside the stated tolerance
