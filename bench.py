@@ -196,7 +196,7 @@ def bench_deltanet(args, torch, hb, wl, prefill):
         "config": {"workload": "c5-%s: gated delta rule B=%d T=%d nk=16 nv=32 dk=dv=128, fp32 state [B,32,128,128]"
                                % ("prefill" if prefill else "decode", B, T), "algorithmic_bytes_per_step": int(nbytes)},
         "tokens_per_s": B * T / (ms * 1e-3),
-        "roofline": {"bound": "hbm", "kernel": "deltanet_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": "deltanet_prefill_kernel" if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "avg_kernel_us": kms * 1e3},
     }

@@ -2,18 +2,17 @@
 //
 //   S <- S * exp(g);  m = k^T S;  delta = (v - m) * beta;  S <- S + k (x) delta;  o = q^T S
 //
-// The [dk, dv] = [128, 128] fp32 state of one (sequence, v-head) is independent per column, so it is
-// cut into slices of NC columns and ONE wavefront owns one slice for the whole call: lane l holds
-// column c = l % NC of rows [rg*RPL, (rg+1)*RPL) with rg = l / NC, RPL = 128*NC/64 rows in registers.
-// The two contractions over dk are per-lane partial sums plus a butterfly over the 64/NC lanes that
-// share a column; nothing goes through LDS and wavefronts never synchronise with each other.
-//   T == 1 (decode): deltanet_decode_kernel, a 32-column slice per wavefront read and written with
-//          16-byte accesses; a single read and a single write of the state: HBM bound,
-//          2*dk*dv*4 bytes per (sequence, head).
-//   T  > 1 (prefill): NC = 8 -> 16 state registers per lane and 16x more wavefronts; tokens are
-//          processed in order with the next token's q/k/v/g/beta already in flight.
+// The [dk, dv] = [128, 128] fp32 state of one (sequence, v-head) is independent per column, so it is cut into
+// column slices and ONE wavefront owns one slice for the whole call.  The two contractions over dk are per-lane
+// partial sums plus a reduction over the lanes that share a column.
+//   T == 1 (decode):  deltanet_decode_kernel, a 32-column slice per wavefront read and written with 16-byte
+//          non-temporal accesses; a single read and a single write of the state: HBM bound, 2*dk*dv*4 bytes per
+//          (sequence, head).
+//   T  > 1 (prefill): deltanet_prefill_kernel, 8-column slices (16 state registers per lane), eight wavefronts
+//          per workgroup sharing the token inputs through LDS; tokens are processed in order.  Bound by VALU
+//          issue: about 85 instructions per token and wavefront, 2 x 4096 wavefront-tokens per SIMD at B=4 x 4096.
 // q and k arrive in bf16; with l2norm they are normalised as x / max(||x||, 1e-3) in fp32.
-#include "common.hpp"
+#include "mfma_common.hpp"
 
 namespace hs {
 
@@ -29,100 +28,173 @@ struct DeltaArgs {
     int32_t l2norm;
 };
 
-template <int NC>
-__device__ __forceinline__ float column_sum(float x) {  // sum over the lanes l with equal l % NC
-#pragma unroll
-    for (int o = NC; o < 64; o <<= 1) x += __shfl_xor(x, o, 64);
-    return x;
-}
+// Prefill (T > 1) with the token inputs staged through LDS.  A 512-thread workgroup owns 64 state columns of one
+// (sequence, v-head): wavefront w the columns 8w .. 8w+7, lane l column l%8 of rows [16*(l/8), +16) -- 16 state
+// registers per lane.  The eight wavefronts together convert a chunk of kChunk tokens once (bf16 -> fp32, L2
+// normalisation folded into k and q, exp(g)) into LDS while the previous chunk is consumed, instead of every
+// wavefront unpacking and normalising the same k and q for itself.  The per-token work of a wavefront is then
+// the three passes over its state slice (k^T S, the rank-1 update, q^T S) plus two column reductions done with
+// lane-swap VALU instructions.
+constexpr int kChunk = 32;
 
-template <int NC>
-struct TokenIn {  // one token's inputs as this lane needs them
-    static constexpr int RPL = 2 * NC;
-    uint32_t kq[2][RPL / 2];  // packed bf16 pairs: k rows, q rows of this lane's row group
-    float v, g, beta;
+struct alignas(16) TokenChunk {
+    float k[kChunk][kDK];   // k * kmul
+    float q[kChunk][kDK];   // q * qmul (includes q_scale)
+    float v[kChunk][64];    // this workgroup's 64 columns
+    float4v scal[kChunk];   // {exp(g), exp(-g), beta, unused}
 };
 
-template <int NC>
-__global__ __launch_bounds__(256) void deltanet_kernel(DeltaArgs a) {
-    constexpr int RPL = 2 * NC;          // rows per lane
-    constexpr int SLICES = kDV / NC;     // column slices per head
-    const int lane = threadIdx.x & 63;
-    const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t nw = (int64_t)a.B * a.nv * SLICES;
-    if (wid >= nw) return;
-    const int slice = (int)(wid % SLICES);
-    const int j = (int)((wid / SLICES) % a.nv);
-    const int b = (int)(wid / SLICES / a.nv);
+// sum over the 8 lanes l, l+8, ..., l+56 that hold the row groups of one column
+__device__ __forceinline__ float rowgroup_sum(float x) {
+    x += __uint_as_float(__builtin_amdgcn_update_dpp(0, __float_as_uint(x), 0x128, 0xf, 0xf, false));  // row_ror:8
+    const uint32_t u = __float_as_uint(x);
+    const auto a = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const float m = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const uint32_t v = __float_as_uint(m);
+    const auto c = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    return __uint_as_float(c[0]) + __uint_as_float(c[1]);
+}
+
+__global__ __launch_bounds__(512) void deltanet_prefill_kernel(DeltaArgs a) {
+    __shared__ TokenChunk chunks[2];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = blockIdx.x & 1;
+    const int j = (int)((blockIdx.x >> 1) % a.nv);
+    const int b = (int)((blockIdx.x >> 1) / a.nv);
     const int hk = j / (a.nv / a.nk);
-    const int c = lane % NC, rg = lane / NC;
-    const int col = slice * NC + c;
-
-    float S[RPL];
-    float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + rg * RPL) * kDV + col;
+    const int c = lane & 7, rg = lane >> 3;
+    const int lcol = 8 * wave + c;          // column inside the workgroup's 64
+    const int col = 64 * half + lcol;
+    float S[16];
+    float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + rg * 16) * kDV + col;
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) S[r] = sp[(int64_t)r * kDV];
+    for (int r = 0; r < 16; ++r) S[r] = sp[(int64_t)r * kDV];
 
-    auto load_token = [&](TokenIn<NC> &x, int t) {
+    // ---- staging roles: thread -> (token tt, 8 consecutive k/q elements starting at 8*part), 4 v columns
+    const int tt = tid >> 4, part = tid & 15;
+    u32x4 rk = {0u, 0u, 0u, 0u}, rq = {0u, 0u, 0u, 0u};
+    u32x2 rv = {0u, 0u};
+    float rg_ = 0.0f, rb_ = 0.0f;
+    auto issue = [&](int t0) {
+        const int t = min(t0 + tt, a.T - 1);
         const int64_t bt = (int64_t)b * a.T + t;
-        const uint16_t *kp = a.k + (bt * a.nk + hk) * kDK + rg * RPL;
-        const uint16_t *qp = a.q + (bt * a.nk + hk) * kDK + rg * RPL;
-#pragma unroll
-        for (int i = 0; i < RPL / 2; ++i) {
-            x.kq[0][i] = ((const uint32_t *)kp)[i];
-            x.kq[1][i] = ((const uint32_t *)qp)[i];
+        rk = *(const u32x4 *)(a.k + (bt * a.nk + hk) * kDK + 8 * part);
+        rq = *(const u32x4 *)(a.q + (bt * a.nk + hk) * kDK + 8 * part);
+        rv = *(const u32x2 *)(a.v + (bt * a.nv + j) * kDV + 64 * half + 4 * part);
+        if (part == 0) {
+            rg_ = a.g[bt * a.nv + j];
+            rb_ = a.beta[bt * a.nv + j];
         }
-        x.v = bf16_bits_to_f32(a.v[(bt * a.nv + j) * kDV + col]);
-        x.g = a.g[bt * a.nv + j];
-        x.beta = a.beta[bt * a.nv + j];
     };
-
-    TokenIn<NC> cur, nxt;
-    load_token(cur, 0);
-    for (int t = 0; t < a.T; ++t) {
-        if (t + 1 < a.T) load_token(nxt, t + 1);
-        float kf[RPL], qf[RPL];
+    auto commit = [&](TokenChunk &ch) {
+        float kf[8], qf[8];
 #pragma unroll
-        for (int i = 0; i < RPL / 2; ++i) {
-            kf[2 * i] = __uint_as_float(cur.kq[0][i] << 16);
-            kf[2 * i + 1] = __uint_as_float(cur.kq[0][i] & 0xffff0000u);
-            qf[2 * i] = __uint_as_float(cur.kq[1][i] << 16);
-            qf[2 * i + 1] = __uint_as_float(cur.kq[1][i] & 0xffff0000u);
+        for (int i = 0; i < 4; ++i) {
+            kf[2 * i] = __uint_as_float(rk[i] << 16);
+            kf[2 * i + 1] = __uint_as_float(rk[i] & 0xffff0000u);
+            qf[2 * i] = __uint_as_float(rq[i] << 16);
+            qf[2 * i + 1] = __uint_as_float(rq[i] & 0xffff0000u);
         }
         float kmul = 1.0f, qmul = a.q_scale;
         if (a.l2norm) {
             float sk = 0.0f, sq = 0.0f;
 #pragma unroll
-            for (int r = 0; r < RPL; ++r) {
-                sk += kf[r] * kf[r];
-                sq += qf[r] * qf[r];
+            for (int i = 0; i < 8; ++i) {
+                sk += kf[i] * kf[i];
+                sq += qf[i] * qf[i];
             }
-            sk = column_sum<NC>(sk);
-            sq = column_sum<NC>(sq);
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) {  // the 16 threads of a token are 16 consecutive lanes
+                sk += __shfl_xor(sk, o, 64);
+                sq += __shfl_xor(sq, o, 64);
+            }
             kmul = 1.0f / fmaxf(sqrtf(sk), 1e-3f);
             qmul = a.q_scale / fmaxf(sqrtf(sq), 1e-3f);
         }
-        const float decay = expf(cur.g);
-        float m = 0.0f;
+        float4v k0 = {kf[0] * kmul, kf[1] * kmul, kf[2] * kmul, kf[3] * kmul};
+        float4v k1 = {kf[4] * kmul, kf[5] * kmul, kf[6] * kmul, kf[7] * kmul};
+        float4v q0 = {qf[0] * qmul, qf[1] * qmul, qf[2] * qmul, qf[3] * qmul};
+        float4v q1 = {qf[4] * qmul, qf[5] * qmul, qf[6] * qmul, qf[7] * qmul};
+        *(float4v *)&ch.k[tt][8 * part] = k0;
+        *(float4v *)&ch.k[tt][8 * part + 4] = k1;
+        *(float4v *)&ch.q[tt][8 * part] = q0;
+        *(float4v *)&ch.q[tt][8 * part + 4] = q1;
+        float4v vv = {__uint_as_float(rv[0] << 16), __uint_as_float(rv[0] & 0xffff0000u), __uint_as_float(rv[1] << 16),
+                      __uint_as_float(rv[1] & 0xffff0000u)};
+        *(float4v *)&ch.v[tt][4 * part] = vv;
+        if (part == 0) ch.scal[tt] = (float4v){expf(rg_), expf(-rg_), rb_, 0.0f};
+    };
+
+    const int nchunks = (a.T + kChunk - 1) / kChunk;
+    issue(0);
+    commit(chunks[0]);
+    if (nchunks > 1) issue(kChunk);
+    __syncthreads();
+    float D = 1.0f, invD = 1.0f;
+    float *op = a.out + (((int64_t)b * a.T) * a.nv + j) * kDV + col;
+    const int64_t ostride = (int64_t)a.nv * kDV;
+    for (int ci = 0; ci < nchunks; ++ci) {
+        if (ci + 1 < nchunks) commit(chunks[(ci + 1) & 1]);
+        if (ci + 2 < nchunks) issue((ci + 2) * kChunk);
+        const TokenChunk &ch = chunks[ci & 1];
+        const int nt = min(kChunk, a.T - ci * kChunk);
+        for (int t = 0; t < nt; ++t) {
+            float kf[16], qf[16];
 #pragma unroll
-        for (int r = 0; r < RPL; ++r) {
-            kf[r] *= kmul;
-            m += kf[r] * S[r];
-        }
-        m = column_sum<NC>(m) * decay;  // k^T (S * decay)
-        const float delta = (cur.v - m) * cur.beta;
-        float o = 0.0f;
+            for (int i = 0; i < 4; ++i) {
+                const float4v kk = *(const float4v *)&ch.k[t][16 * rg + 4 * i];
+                const float4v qq = *(const float4v *)&ch.q[t][16 * rg + 4 * i];
 #pragma unroll
-        for (int r = 0; r < RPL; ++r) {
-            S[r] = S[r] * decay + kf[r] * delta;
-            o += qf[r] * S[r];
+                for (int e = 0; e < 4; ++e) {
+                    kf[4 * i + e] = kk[e];
+                    qf[4 * i + e] = qq[e];
+                }
+            }
+            const float vv = ch.v[t][lcol];
+            const float4v sc = ch.scal[t];
+            const float decay = sc[0], beta = sc[2];
+            // The registers hold S / D with D the product of the decays since the last fold, so a token costs one
+            // FMA per state element instead of a multiply and an FMA.  D is folded back in before it can underflow.
+            if (D * decay < 1e-20f) {
+                const float f = D * decay;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) S[r] *= f;
+                D = 1.0f;
+                invD = 1.0f;
+            } else {
+                D *= decay;
+                invD *= sc[1];
+            }
+            float m0 = 0.0f, m1 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                m0 += kf[r] * S[r];
+                m1 += kf[r + 1] * S[r + 1];
+            }
+            const float m = rowgroup_sum(m0 + m1) * D;  // k^T (S_prev * decay)
+            const float kd = (vv - m) * beta * invD;    // delta / D
+            float o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                S[r] += kf[r] * kd;
+                S[r + 1] += kf[r + 1] * kd;
+                o0 += qf[r] * S[r];
+                o1 += qf[r + 1] * S[r + 1];
+            }
+            const float o = rowgroup_sum(o0 + o1) * D;
+            if (rg == 0) op[(int64_t)(ci * kChunk + t) * ostride] = o;
         }
-        o = column_sum<NC>(o) * qmul;
-        if (rg == 0) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kDV + col] = o;
-        cur = nxt;
+        // fold at every chunk end: a prefill split into calls of a multiple of kChunk tokens (state carried through
+        // memory) then rounds exactly like one call
+#pragma unroll
+        for (int r = 0; r < 16; ++r) S[r] *= D;
+        D = 1.0f;
+        invD = 1.0f;
+        __syncthreads();
     }
 #pragma unroll
-    for (int r = 0; r < RPL; ++r) sp[(int64_t)r * kDV] = S[r];
+    for (int r = 0; r < 16; ++r) sp[(int64_t)r * kDV] = S[r];
 }
 
 // Decode step (T == 1), tuned for HBM streaming: one wavefront owns 32 columns x 128 rows; lane l holds
@@ -221,8 +293,7 @@ extern "C" int hs_deltanet_forward(const void *q, const void *k, const void *v, 
         const int64_t waves = (int64_t)B * nv * (kDV / 32);
         deltanet_decode_kernel<<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(a);
     } else {
-        const int64_t waves = (int64_t)B * nv * (kDV / 8);
-        deltanet_kernel<8><<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(a);
+        deltanet_prefill_kernel<<<(unsigned)((int64_t)B * nv * 2), 512, 0, st>>>(a);
     }
     return check_launch("deltanet");
 }
