@@ -56,6 +56,14 @@ void hs_cache_truncate_to(hs_cache *c, int64_t pos) { if (c && pos >= 0) c->cach
 int hs_cache_is_initialized(const hs_cache *c) { return c && c->cache.is_initialized(); }
 int64_t hs_cache_memory_usage(const hs_cache *c) { return c ? (int64_t)c->cache.memory_usage() : 0; }
 int hs_cache_quant_type(const hs_cache *c) { return c ? (int)c->cache.quant_type() : 0; }
+const char *hs_kv_quant_canonical_str(int quant_type) {
+    switch (quant_type) {
+        case HS_KV_NONE: return "none";
+        case HS_KV_INT8: return "int8-token";
+        case HS_KV_FP8: return "fp8-e4m3fn-head";
+        default: return nullptr;
+    }
+}
 
 int hs_cache_decode_attention(hs_cache *c, const void *q, void *out, int32_t hq, float scale, hs_stream_t stream) {
     if (!c) return HS_ERR_INVALID_ARGUMENT;

@@ -16,7 +16,7 @@ EXPORTS = [
     "hs_cache_create", "hs_cache_destroy", "hs_cache_last_error", "hs_cache_update", "hs_cache_get_dense",
     "hs_cache_get_view", "hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_clear", "hs_cache_truncate_to",
     "hs_cache_is_initialized", "hs_cache_memory_usage", "hs_cache_quant_type", "hs_cache_decode_attention",
-    "hs_cache_decode_step", "hs_cache_prefill",
+    "hs_cache_decode_step", "hs_cache_prefill", "hs_kv_quant_canonical_str",
     "hs_pool_create", "hs_pool_destroy", "hs_pool_last_error", "hs_pool_allocate", "hs_pool_free", "hs_pool_owner_of",
     "hs_pool_used_blocks", "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory",
     "hs_paged_cache_create", "hs_paged_cache_destroy", "hs_paged_cache_last_error", "hs_paged_cache_update",
@@ -43,6 +43,7 @@ def lib():
                   "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory", "hs_paged_cache_seq_pos",
                   "hs_paged_cache_num_blocks"):
             getattr(L, f).restype = ctypes.c_int64
+        L.hs_kv_quant_canonical_str.restype = ctypes.c_char_p
         L.hs_pool_create.restype = ctypes.c_void_p
         L.hs_pool_create.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
         L.hs_pool_last_error.restype = ctypes.c_char_p

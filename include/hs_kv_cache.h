@@ -47,6 +47,12 @@ HS_API void hs_cache_truncate_to(hs_cache *c, int64_t pos); /* kv_cache.rs:1707-
 HS_API int hs_cache_is_initialized(const hs_cache *c);   /* kv_cache.rs:1753-1764 */
 HS_API int64_t hs_cache_memory_usage(const hs_cache *c); /* kv_cache.rs:1767-1831 */
 HS_API int hs_cache_quant_type(const hs_cache *c);       /* kv_cache.rs:1861 */
+/* Canonical lowercase name of a storage format, the string KvQuantMode::as_canonical_str feeds into the
+ * compatibility fingerprint (kv_compat.rs:215-237): "none", and for the two device formats served here
+ * "int8-token" (int8 codes, one fp32 absmax scale per token and kv-head) and "fp8-e4m3fn-head" (e4m3fn codes,
+ * one fp32 scale per sequence and kv-head).  They differ from the reference's "int8" (blockwise-64 codes) on
+ * purpose: a cache written in one format must never be reused as another.  NULL for an unknown value. */
+HS_API const char *hs_kv_quant_canonical_str(int quant_type);
 
 /* cache.get() + GQA expand + compute_attention for one query token per sequence
  * (llama.rs:605-636, 847-872, 1023-1119).  q, out: bf16 [batch, num_q_heads, head_dim]. */

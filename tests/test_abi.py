@@ -129,3 +129,14 @@ def test_chunk_policy_unsplit_for_uniform_and_split_for_ragged_hint():
     per_chunk = B * Hq * (D + 2) * 4
     assert hb.decode_workspace_bytes(B, Hq, Hkv, D, T) >= 16 * per_chunk >= n * per_chunk
 
+
+def test_format_names_are_distinct_and_stable():
+    """The names feed the reference's compatibility fingerprint (kv_compat.rs:215-237): the device formats must
+    not collide with each other or with the reference's own "int8" / "nf4" / "fp4"."""
+    from hyprstream_amd import kv_cache as kc
+    L = kc.lib()
+    names = [L.hs_kv_quant_canonical_str(i) for i in (kc.NONE, kc.INT8, kc.FP8)]
+    assert names == [b"none", b"int8-token", b"fp8-e4m3fn-head"]
+    assert not set(names) & {b"int8", b"nf4", b"fp4"}
+    assert L.hs_kv_quant_canonical_str(9) is None
+
