@@ -25,6 +25,7 @@ EXPORTS = [
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
+    "hs_deltanet_prepare", "hs_deltanet_gated_norm",
 ]
 
 
@@ -214,3 +215,32 @@ def deltanet_forward(q, k, v, g, beta, state, out, q_scale, l2norm=False):
         assert t.is_contiguous()
     check(lib().hs_deltanet_forward(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(out),
                                     B, T, nk, nv, dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)), _stream()))
+
+
+def deltanet_prepare(mixed_qkv, conv_weight, conv_state_in, a_in, b_in, neg_a_exp, dt_bias, nk, nv, dk, dv):
+    """conv1d(k=4)+SiLU with carried state, q/k/v split, g and beta.  Returns (q, k, v, g, beta, new_conv_state)."""
+    import torch
+    B, S, C = mixed_qkv.shape
+    assert C == 2 * nk * dk + nv * dv and mixed_qkv.is_contiguous() and conv_weight.is_contiguous()
+    dev = mixed_qkv.device
+    q = torch.empty(B, S, nk, dk, dtype=torch.bfloat16, device=dev)
+    k = torch.empty(B, S, nk, dk, dtype=torch.bfloat16, device=dev)
+    v = torch.empty(B, S, nv, dv, dtype=torch.bfloat16, device=dev)
+    g = torch.empty(B, S, nv, dtype=torch.float32, device=dev)
+    beta = torch.empty(B, S, nv, dtype=torch.float32, device=dev)
+    state_out = torch.empty(B, C, 3, dtype=torch.bfloat16, device=dev)
+    check(lib().hs_deltanet_prepare(_ptr(mixed_qkv), _ptr(conv_weight), _ptr(conv_state_in), _ptr(state_out),
+                                    _ptr(a_in.contiguous()), _ptr(b_in.contiguous()), _ptr(neg_a_exp), _ptr(dt_bias),
+                                    _ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), B, S, nk, nv, dk, dv, _stream()))
+    return q, k, v, g, beta, state_out
+
+
+def deltanet_gated_norm(x, z, weight, eps):
+    """x fp32 [..., D], z bf16 [..., D], weight fp32 [D] -> bf16 [..., D]."""
+    import torch
+    D = x.shape[-1]
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    check(lib().hs_deltanet_gated_norm(_ptr(x.contiguous()), _ptr(z.contiguous()), _ptr(weight), ctypes.c_float(eps),
+                                       _ptr(out), ctypes.c_int64(x.numel() // D), D, _stream()))
+    return out
+

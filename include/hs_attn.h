@@ -226,6 +226,27 @@ HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, cons
                         int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
                         float q_scale, int l2norm, hs_stream_t stream);
 
+/* ---- the elementwise steps of a gated-DeltaNet layer around the delta rule ("next" of hs_deltanet_forward) ----
+ * hs_deltanet_prepare (GatedDeltaNetLayer::forward between the input projection and the recurrence,
+ * qwen3_5.rs:629-686): depthwise causal conv1d with kernel 4 over [3 carried frames | the S new frames] of the
+ * mixed q|k|v channels, then SiLU, in bf16 (fp32 accumulation in tap order, one rounding after the conv, one
+ * after the SiLU); the result is split into q, k [B, S, nk, dk] and v [B, S, nv, dv], the inputs of
+ * hs_deltanet_forward (which L2-normalises q and k itself).  Gates in fp32: g = neg_a_exp * softplus(a + dt_bias)
+ * with neg_a_exp = -exp(A_log) precomputed by the caller as the reference does (qwen3_5.rs:563-568),
+ * beta = sigmoid(b).
+ *   mixed_qkv [B, S, 2*nk*dk + nv*dv] bf16;  conv_weight [C, 4] bf16 (the [C, 1, 4] conv1d weight);
+ *   conv_state_in [B, C, 3] bf16 or NULL (first call: zeros);  conv_state_out [B, C, 3] bf16, a different buffer;
+ *   a_in, b_in [B, S, nv] bf16;  neg_a_exp, dt_bias [nv] fp32;  g, beta [B, S, nv] fp32.
+ * hs_deltanet_gated_norm (RMSNormGated::forward, qwen3_5.rs:305-313): out = x * rsqrt(mean(x^2) + eps) * w *
+ * silu(z) per row of D elements; x fp32 [rows, D] (the recurrence output viewed as [B*S*nv, dv]), z bf16, w fp32 [D],
+ * out bf16. */
+HS_API int hs_deltanet_prepare(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in,
+                               void *conv_state_out, const void *a_in, const void *b_in, const float *neg_a_exp,
+                               const float *dt_bias, void *q, void *k, void *v, float *g, float *beta,
+                               int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv, hs_stream_t stream);
+HS_API int hs_deltanet_gated_norm(const float *x, const void *z, const float *weight, float eps, void *out,
+                                  int64_t rows, int32_t D, hs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

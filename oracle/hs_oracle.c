@@ -59,6 +59,18 @@
  *                            on bf16/fp32 tensors, identity at position 0, norm
  *                            preservation and the relative-position property
  *                            (tests/test_oracle_rope.py).
+ *  - orc_deltanet_prepare    what GatedDeltaNetLayer::forward does between the input
+ *                            projection and the delta rule (qwen3_5.rs:617-720):
+ *                            depthwise causal conv1d (kernel 4, the 3 frames before
+ *                            the call carried as state) + SiLU on the mixed q|k|v
+ *                            channels in the model dtype, g = -exp(A_log) *
+ *                            softplus(a + dt_bias) and beta = sigmoid(b) in fp32.
+ *                            The conv accumulates in fp32 in tap order and rounds
+ *                            once to bf16; libtorch's bf16 conv1d does not promise an
+ *                            accumulation order, so parity with it is to one bf16 ulp,
+ *                            not to the bit (tests/test_oracle_deltanet_glue.py).
+ *  - orc_gated_rmsnorm       RMSNormGated::forward (qwen3_5.rs:292-313):
+ *                            x * rsqrt(mean(x^2) + eps) * w * silu(z) in fp32.
  *
  * parity unpinned: the reference's own int8 format (bitsandbytes 0.45.0
  * blockwise-64 codes, tie-breaking of its binary search) is not restated here
@@ -408,6 +420,60 @@ ORC_API void orc_rope_apply_f32(const float *x, const float *sin_t, const float 
                 oi[d] = a - b;
                 oi[d + half] = e + f;
             }
+        }
+    }
+}
+
+/* ------------------------------------------------------- DeltaNet surroundings */
+
+static inline float silu_f(float x) { return x / (1.0f + expf(-x)); }
+
+/* x: bf16 [B, S, C] (C = conv channels), w: bf16 [C, K] (tap K-1 multiplies the current frame),
+ * state: bf16 [B, C, K-1] in/out (the K-1 frames before this call, oldest first; zeros before the first call),
+ * y: bf16 [B, S, C] = silu(conv) rounded to bf16 after the conv and after the SiLU. */
+ORC_API void orc_deltanet_conv_silu_bf16(const uint16_t *x, const uint16_t *w, uint16_t *state, int B, int S, int C, int K,
+                                         uint16_t *y) {
+    for (int b = 0; b < B; ++b)
+        for (int c = 0; c < C; ++c) {
+            float hist[16];
+            for (int i = 0; i < K - 1; ++i) hist[i] = bf16_to_f32(state[((int64_t)b * C + c) * (K - 1) + i]);
+            for (int t = 0; t < S; ++t) {
+                hist[K - 1] = bf16_to_f32(x[((int64_t)b * S + t) * C + c]);
+                float acc = 0.0f;
+                for (int i = 0; i < K; ++i) {
+                    const volatile float p = bf16_to_f32(w[(int64_t)c * K + i]) * hist[i];
+                    acc += p;
+                }
+                const float r = rbf(acc);
+                y[((int64_t)b * S + t) * C + c] = orc_f32_to_bf16(silu_f(r));
+                for (int i = 0; i < K - 1; ++i) hist[i] = hist[i + 1];
+            }
+            for (int i = 0; i < K - 1; ++i) state[((int64_t)b * C + c) * (K - 1) + i] = orc_f32_to_bf16(hist[i]);
+        }
+}
+
+/* a, bb: bf16 [rows, nv]; neg_a_exp, dt_bias: fp32 [nv];  g = neg_a_exp * softplus(a + dt_bias), beta = sigmoid(bb). */
+ORC_API void orc_deltanet_gates(const uint16_t *a, const uint16_t *bb, const float *neg_a_exp, const float *dt_bias,
+                                int64_t rows, int nv, float *g, float *beta) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int j = 0; j < nv; ++j) {
+            const float x = bf16_to_f32(a[r * nv + j]) + dt_bias[j];
+            const float sp = x > 20.0f ? x : log1pf(expf(x)); /* libtorch softplus, beta 1, threshold 20 */
+            g[r * nv + j] = neg_a_exp[j] * sp;
+            beta[r * nv + j] = 1.0f / (1.0f + expf(-bf16_to_f32(bb[r * nv + j])));
+        }
+}
+
+/* x: fp32 [rows, D]; z: bf16 [rows, D]; w: fp32 [D]; out: bf16 [rows, D]. */
+ORC_API void orc_gated_rmsnorm(const float *x, const uint16_t *z, const float *w, float eps, int64_t rows, int D,
+                               uint16_t *out) {
+    for (int64_t r = 0; r < rows; ++r) {
+        double ss = 0.0;
+        for (int d = 0; d < D; ++d) ss += (double)x[r * D + d] * x[r * D + d];
+        const float rrms = 1.0f / sqrtf((float)(ss / D) + eps);
+        for (int d = 0; d < D; ++d) {
+            const float n = x[r * D + d] * rrms;
+            out[r * D + d] = orc_f32_to_bf16(n * w[d] * silu_f(bf16_to_f32(z[r * D + d])));
         }
     }
 }

@@ -211,3 +211,35 @@ def rope_apply_f32(x, sin_t, cos_t, pos):
                              ctypes.c_int64(rows), ctypes.c_int(H), ctypes.c_int(D), _p(out))
     return out
 
+
+# ------------------------------------------------------- DeltaNet surroundings
+def deltanet_conv_silu_bf16(x_bits, w_bits, state_bits):
+    """x [B,S,C], w [C,K], state [B,C,K-1] (bf16 patterns) -> (y [B,S,C], new state)."""
+    x = _c(x_bits, np.uint16)
+    w = _c(w_bits, np.uint16)
+    st = _c(state_bits, np.uint16).copy()
+    B, S, C = x.shape
+    y = np.empty_like(x)
+    lib().orc_deltanet_conv_silu_bf16(_p(x), _p(w), _p(st), B, S, C, w.shape[1], _p(y))
+    return y, st
+
+
+def deltanet_gates(a_bits, b_bits, neg_a_exp, dt_bias):
+    a = _c(a_bits, np.uint16)
+    b = _c(b_bits, np.uint16)
+    nv = a.shape[-1]
+    g = np.empty(a.shape, np.float32)
+    beta = np.empty(a.shape, np.float32)
+    lib().orc_deltanet_gates(_p(a), _p(b), _p(_c(neg_a_exp, np.float32)), _p(_c(dt_bias, np.float32)),
+                             ctypes.c_int64(a.size // nv), nv, _p(g), _p(beta))
+    return g, beta
+
+
+def gated_rmsnorm(x, z_bits, w, eps):
+    x = _c(x, np.float32)
+    z = _c(z_bits, np.uint16)
+    D = x.shape[-1]
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_gated_rmsnorm(_p(x), _p(z), _p(_c(w, np.float32)), ctypes.c_float(eps), ctypes.c_int64(x.size // D), D, _p(out))
+    return out
+

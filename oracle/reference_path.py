@@ -165,3 +165,30 @@ def rope_apply(x, sin_full, cos_full, position_ids):
     x2r = x1 * sin_e + x2 * cos_e
     return torch.cat([x1r, x2r], -1)
 
+
+def deltanet_prepare(mixed_qkv, conv_weight, conv_state, a_in, b_in, neg_a_exp, dt_bias):
+    """GatedDeltaNetLayer::forward between the projection and the delta rule (qwen3_5.rs:629-686): depthwise
+    causal conv1d over [state | x] + SiLU in the model dtype, g and beta in fp32.  mixed_qkv [B,S,C];
+    conv_weight [C,1,K]; conv_state [B,C,K-1] or None.  Returns (conv_out [B,S,C], new_state, g, beta)."""
+    B, S, C = mixed_qkv.shape
+    ks = conv_weight.shape[-1]
+    x_t = mixed_qkv.permute(0, 2, 1)
+    if conv_state is None:
+        conv_state = torch.zeros(B, C, ks - 1, dtype=mixed_qkv.dtype)
+    padded = torch.cat([conv_state, x_t], 2)
+    new_state = padded.narrow(2, padded.shape[2] - (ks - 1), ks - 1).contiguous()
+    conv_out = torch.nn.functional.conv1d(padded, conv_weight, None, 1, 0, 1, C)
+    conv_out = torch.nn.functional.silu(conv_out).permute(0, 2, 1)
+    g = neg_a_exp * torch.nn.functional.softplus(a_in.float() + dt_bias)
+    beta = b_in.float().sigmoid()
+    return conv_out, new_state, g, beta
+
+
+def gated_rmsnorm(x, gate, weight_f32, eps):
+    """RMSNormGated::forward (qwen3_5.rs:305-313)."""
+    orig = gate.dtype
+    x_f = x.float()
+    mean_sq = (x_f * x_f).mean(-1, keepdim=True)
+    rrms = (mean_sq + eps).rsqrt()
+    return (x_f * rrms * weight_f32 * torch.nn.functional.silu(gate.float())).to(orig)
+
