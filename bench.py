@@ -385,6 +385,12 @@ def main():
     }
     if not args.no_cpu_baseline:
         cb, _ = cpu_baseline(torch, args.workload, caches[0], q, lens, Hq, fp8)
+        if args.workload == "c2":
+            # the reference's own CPU-runnable configuration (one sequence, 2048 tokens, int8), whole, same op sequence
+            T1 = 2048
+            one = tuple(t[:1, :, :T1].contiguous() for t in caches[0])
+            c1, _ = cpu_baseline(torch, "c1", one, q[:1], torch.full((1,), T1, dtype=torch.int32), Hq, False, seconds_budget=3.0)
+            cb["single_sequence_2048"] = {k: c1[k] for k in ("value", "unit", "ms_per_call", "tokens_per_s")}
         result["cpu_baseline"] = cb
     print(json.dumps(result))
 
