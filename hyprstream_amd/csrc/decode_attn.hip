@@ -120,11 +120,14 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     const int t_end = min(L, t_begin + a.chunk_tokens);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int li = lane & 15, lq = lane >> 4;
-    if (a.nt.src[0] != nullptr && t_end == L) {
-        // This workgroup reads the newest token: write it first (K by wavefront 0, V by wavefront 1).
+    // This workgroup reads the newest token if it owns the end of the sequence: it then writes it first (K by
+    // wavefront 0, V by wavefront 1).  With five or more steps the token sits beyond every wavefront's first tile,
+    // so those first loads are issued ahead of the write and its barrier instead of behind them.
+    const bool writes_new = a.nt.src[0] != nullptr && t_end == L;
+    auto write_new_token = [&]() {
         if (wave < 2) quantize_row<2, FP8>(a.nt, wave, (int64_t)b * a.Hkv + h, lane);
-        __syncthreads();  // codes and scales are visible to the whole workgroup before any load
-    }
+        __syncthreads();  // codes and scales are visible to the whole workgroup before any load that covers them
+    };
 
     half8 qop[4];
     float cq = 0.0f, cinit = 0.0f;
@@ -277,7 +280,10 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     // ---- software pipeline over this wavefront's steps (wave, wave+4, ...)
     Stage<FP8> sa, sb;
     int step = wave;
+    const bool early_loads = nsteps >= kWavesPerWg + 1;
+    if (writes_new && !early_loads) write_new_token();
     if (step < nsteps) load_stage(sa, step);
+    if (writes_new && early_loads) write_new_token();
     // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds
     //      Q[head][64*(j/2) + 16*lq + 8*(j%2) + e] for MFMA j.
     {
