@@ -206,8 +206,8 @@ def bench_deltanet(args, torch, hb, wl, prefill):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=300)
-    ap.add_argument("--warmup", type=int, default=50)  # the first ~30 launches after set-up run 3-4 % slower
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c5-decode", "c5-prefill"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
