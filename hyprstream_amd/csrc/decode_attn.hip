@@ -472,7 +472,7 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
                          hipStream_t stream) {
     if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
     if (D != kD) return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 128, got %d", D);
-    if (!q || !kc || !vc || !ks || !vs || !seq_lens || !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (B > 0 && (!q || !kc || !vc || !ks || !vs || !seq_lens || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if ((nt.k_src == nullptr) != (nt.v_src == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give k_new and v_new or neither");
     if (nt.k_src && nt.dtype != HS_BF16 && nt.dtype != HS_F32 && nt.dtype != HS_F16)
         return fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", nt.dtype);

@@ -279,7 +279,7 @@ extern "C" int hs_deltanet_forward(const void *q, const void *k, const void *v, 
                                    float *state, float *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk,
                                    int32_t dv, float q_scale, int l2norm, hs_stream_t stream) {
     using namespace hs;
-    if (!q || !k || !v || !g || !beta || !state || !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (B > 0 && T > 0 && (!q || !k || !v || !g || !beta || !state || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (dk != kDK || dv != kDV) return fail(HS_ERR_INVALID_ARGUMENT, "deltanet is built for dk = dv = 128, got %d x %d", dk, dv);
     if (B < 0 || T < 0 || nk <= 0 || nv <= 0 || nv % nk != 0)
         return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d T=%d nk=%d nv=%d (need nv %% nk == 0)", B, T, nk, nv);

@@ -105,9 +105,10 @@ int hs_deltanet_prepare(const void *mixed_qkv, const void *conv_weight, const vo
                         void *v, float *g, float *beta, int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
                         hs_stream_t stream) {
     using namespace hs;
-    if (!mixed_qkv || !conv_weight || !conv_state_out || !a_in || !b_in || !neg_a_exp || !dt_bias || !q || !k || !v || !g || !beta)
+    if (B > 0 && S > 0 &&
+        (!mixed_qkv || !conv_weight || !conv_state_out || !a_in || !b_in || !neg_a_exp || !dt_bias || !q || !k || !v || !g || !beta))
         return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
-    if (conv_state_in == conv_state_out) return fail(HS_ERR_INVALID_ARGUMENT, "conv_state_out must not alias conv_state_in");
+    if (conv_state_out && conv_state_in == conv_state_out) return fail(HS_ERR_INVALID_ARGUMENT, "conv_state_out must not alias conv_state_in");
     if (B < 0 || S < 0 || nk <= 0 || nv <= 0 || dk <= 0 || dv <= 0)
         return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d nk=%d nv=%d dk=%d dv=%d", B, S, nk, nv, dk, dv);
     if (B == 0 || S == 0) return HS_OK;
@@ -129,7 +130,7 @@ int hs_deltanet_prepare(const void *mixed_qkv, const void *conv_weight, const vo
 int hs_deltanet_gated_norm(const float *x, const void *z, const float *weight, float eps, void *out, int64_t rows, int32_t D,
                            hs_stream_t stream) {
     using namespace hs;
-    if (!x || !z || !weight || !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (rows > 0 && (!x || !z || !weight || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (rows < 0 || (D != 64 && D != 128 && D != 256)) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape rows=%lld D=%d", (long long)rows, D);
     if (rows == 0) return HS_OK;
     const unsigned blocks = (unsigned)((rows + 3) / 4);

@@ -164,7 +164,8 @@ static int launch_quantize(const void *k_src, const void *v_src, int dtype, void
     if (rope_sin && !positions && (int64_t)start_pos + S > rope_len)
         return fail(HS_ERR_INVALID_ARGUMENT, "positions %d..%d exceed the rotary tables (%d rows)", start_pos,
                     start_pos + S - 1, rope_len);
-    if (!k_src || !v_src || !kc || !vc || !ks || !vs) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    const bool empty = (int64_t)B * S == 0;  // an empty problem may come with null pointers (an empty tensor has none)
+    if (!empty && (!k_src || !v_src || !kc || !vc || !ks || !vs)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16)
         return fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", dtype);
     if (!positions) {
@@ -216,7 +217,7 @@ int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *ro
                   const int32_t *positions, int32_t start_pos, void *out, int32_t B, int32_t S, int32_t H, int32_t D,
                   hs_stream_t stream) {
     using namespace hs;
-    if (!x || !out || !rope_sin || !rope_cos) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if ((int64_t)B * S > 0 && (!x || !out || !rope_sin || !rope_cos)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16) return fail(HS_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
     if (B < 0 || S < 0 || H <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d H=%d", B, S, H);
     if (D != 64 && D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "head_dim %d not in {64,128,256}", D);
@@ -259,7 +260,7 @@ int hs_kv_fp8_calibrate(const void *k_src, const void *v_src, int src_dtype, flo
 int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8, const hs_kv_layout *layout, int which_table,
                      void *out, int out_dtype, int32_t B, int32_t T, int32_t Hkv, int32_t D, hs_stream_t stream) {
     if (int rc = hs::validate_layout(layout, B, T, Hkv, D, !fmt_fp8)) return rc;
-    if (!codes || !scales || !out) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if ((int64_t)B * T > 0 && (!codes || !scales || !out)) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (out_dtype != HS_BF16 && out_dtype != HS_F32 && out_dtype != HS_F16)
         return hs::fail(HS_ERR_INVALID_ARGUMENT, "unknown out_dtype %d", out_dtype);
     const int64_t rows = (int64_t)B * T * Hkv;

@@ -476,7 +476,8 @@ extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void
     using namespace hs;
     if (int rc = validate_layout(layout, B, S, Hkv, D, true)) return rc;
     if (D != kPD) return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 128, got %d", D);
-    if (!q || !k_new || !v_new || !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    const bool empty = B == 0 || S == 0;  // an empty problem may come with null pointers (an empty tensor has none)
+    if (!empty && (!q || !k_new || !v_new || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if ((hist_len > 0 || quantize_on_write) && (!k_codes || !v_codes || !k_scales || !v_scales))
         return fail(HS_ERR_INVALID_ARGUMENT, "null cache buffer");
     if (hist_len < 0) return fail(HS_ERR_INVALID_ARGUMENT, "negative hist_len");
