@@ -22,6 +22,9 @@
 // power of two into fp16 range.  New-token part: bf16 MFMA straight from the caller's bf16 K/V, V^T built with
 // permutes, P rounded to bf16.  Softmax and accumulation are fp32; the score layout of the first product is the
 // B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16 range (|x| > 65024) saturate.
+#include <climits>
+#include <type_traits>
+
 #include "mfma_common.hpp"
 #include "quant_device.hpp"
 
@@ -159,8 +162,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 
     // =============================== history: int8 cache, f16 MFMA ===============================
     if (H > 0) {
+        // Q operands carry the softmax scale and log2(e): qop = fp16(q * scale * log2e * 2^-ex), so the MFMA
+        // result is the score in log2 units times 2^-ex.  ex is zero unless a column's scaled |q| would leave
+        // the fp16 range (then the wavefront takes the path that multiplies the scores by cq = 2^ex).
         half8 qop[kNB][4];
         float cq[kNB];
+        bool scaled = false;
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
             const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 32 * lq;
@@ -170,21 +177,23 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16);
-                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16) * a.scale_log2e;
+                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * a.scale_log2e;
                 }
             }
 #pragma unroll
             for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
             amax = quad_max(amax);
             int ex = 0;
-            if (amax > 0.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
+            if (amax > 32768.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
+            scaled |= ex != 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qop[nb][j][e] = (_Float16)ldexpf(qf[8 * j + e], -ex);
-            cq[nb] = ldexpf(a.scale_log2e, ex);
+            cq[nb] = ldexpf(1.0f, ex);
         }
+        scaled = __builtin_amdgcn_ballot_w64(scaled) != 0;
 
         const int nsteps = (H + kPStep - 1) / kPStep;
         // ---- producers: every wavefront converts one eighth of the step's K tile and of its V tile.
@@ -228,23 +237,24 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 vsp = a.vs + unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot;
                 vleft = a.va.capacity_tokens - slot;
             }
-            // The loaded values are only touched in commit(): nothing waits for a load here.  A full step adds
-            // this lane's fixed offsets to the step's (scalar) base addresses; only the last, partial step clamps rows.
-            if (last >= kPStep - 1) {
-                rawk = *(const u32x2 *)(kb + koff);
-                rawv[0] = *(const uint32_t *)(vb + voff);
-                rawv[1] = *(const uint32_t *)(vb + voff + kPD);
-                rawsk = ksp[(uint32_t)krow];
-                rawsv[0] = vsp[(uint32_t)vkey];
-                rawsv[1] = vsp[(uint32_t)vkey + 1];
-            } else {
-                rawk = *(const u32x2 *)(kb + (min(krow, last) * kPD + kcol));
-                rawv[0] = *(const uint32_t *)(vb + (min(vkey, last) * kPD + 4 * vx));
-                rawv[1] = *(const uint32_t *)(vb + (min(vkey + 1, last) * kPD + 4 * vx));
-                rawsk = ksp[min(krow, last)];
-                rawsv[0] = vsp[min(vkey, last)];
-                rawsv[1] = vsp[min(vkey + 1, last)];
+            // The loaded values are only touched in commit(): nothing waits for a load here.  Addresses are the
+            // step's (scalar) base plus a 32-bit lane offset; only the last, partial step clamps rows.
+            uint32_t ko = koff, vo0 = voff, vo1 = voff + kPD, sk = 4u * krow, sv = 4u * vkey;
+            uint32_t sv1 = sv + 4u;
+            if (last < kPStep - 1) {
+                ko = min(krow, last) * kPD + kcol;
+                vo0 = min(vkey, last) * kPD + 4 * vx;
+                vo1 = min(vkey + 1, last) * kPD + 4 * vx;
+                sk = 4u * min(krow, last);
+                sv = 4u * min(vkey, last);
+                sv1 = 4u * min(vkey + 1, last);
             }
+            rawk = *(const u32x2 *)(kb + ko);
+            rawv[0] = *(const uint32_t *)(vb + vo0);
+            rawv[1] = *(const uint32_t *)(vb + vo1);
+            rawsk = *(const float *)((const uint8_t *)ksp + sk);
+            rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
+            rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
             kb += kPStep * kPD; vb += kPStep * kPD;
             ksp += kPStep; vsp += kPStep;
             kleft -= kPStep; vleft -= kPStep;
@@ -265,6 +275,16 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         float4v s[kNB][2];  // scores of the step between scores() and softmax()
         half8 pop[kNB];     // P^T operands between softmax() and output()
         half8 kop[8], vop[8];  // the step's A operands, read from LDS ahead of use
+        // The score accumulators start from -sref (over cq) instead of zero, sref = m_run - kPShift being the
+        // value the softmax subtracts: the MFMA result is then the exponent of the weight itself.
+        float sref[kNB];
+        float4v sinit[kNB];
+        int force = INT_MAX;  // takes the first step through the branch that sets the reference
+#pragma unroll
+        for (int nb = 0; nb < kNB; ++nb) {
+            sref[nb] = 0.0f;
+            sinit[nb] = (float4v){0.f, 0.f, 0.f, 0.f};
+        }
         auto load_k = [&](const StepTile &t, int) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) kop[i] = *(const half8 *)(t.k[i] + obase);
@@ -277,47 +297,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){0.f, 0.f, 0.f, 0.f};
+                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = sinit[nb];
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb)
                         s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[4 * u + j], qop[nb][j], s[nb][u], 0, 0, 0);
-            }
-        };
-        auto softmax = [&](const StepTile &t, int step) {
-            const int t0 = step * kPStep;
-            const bool tail = t0 + kPStep > H;
-            float sc[kNB][8], mx[kNB];
-#pragma unroll
-            for (int nb = 0; nb < kNB; ++nb) {
-#pragma unroll
-                for (int u = 0; u < 2; ++u)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) sc[nb][4 * u + r] = s[nb][u][r];
-                if (tail) {
-#pragma unroll
-                    for (int u = 0; u < 2; ++u)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (t0 + 16 * u + 4 * lq + r >= H) sc[nb][4 * u + r] = -INFINITY;
-                }
-                float m = sc[nb][0];
-#pragma unroll
-                for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[nb][i]);
-                mx[nb] = quad_max(m) * cq[nb];  // cq > 0: max(t) * cq == max(t * cq); -inf stays -inf
-            }
-            raise_max(mx);
-#pragma unroll
-            for (int nb = 0; nb < kNB; ++nb) {
-                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
-                float p[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    p[i] = __builtin_amdgcn_exp2f(sc[nb][i] * cq[nb] - mref);
-                    l_run[nb] += p[i];
-                }
-                pop[nb] = pack_half8(pack_f16x2(p[0], p[1]), pack_f16x2(p[2], p[3]), pack_f16x2(p[4], p[5]), pack_f16x2(p[6], p[7]));
             }
         };
         auto output = [&](int) {
@@ -327,7 +312,74 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 for (int nb = 0; nb < kNB; ++nb)
                     acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb], acc[nb][bb], 0, 0, 0);
         };
-        walk_keys(nsteps, tiles, issue, commit, load_k, scores, softmax, load_v, output);
+        // softmax(): e = exponent of each weight (score in log2 units minus sref).  The common step only checks,
+        // per lane and on the bit patterns (a positive float orders like its bits; a NaN reads as large), whether
+        // any exponent exceeds kPShift, i.e. whether a score passed m_run; only then, at the first step and at a
+        // partial last step does the wavefront reduce the column maxima and move the reference.
+        auto softmax_for = [&](auto scaled_tag) {
+            constexpr bool kScaled = decltype(scaled_tag)::value;
+            return [&](const StepTile &, int step) {
+                const int lim = H - step * kPStep;  // keys of this step that exist
+                float e[kNB][8];
+                int over = force;
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb) {
+#pragma unroll
+                    for (int u = 0; u < 2; ++u)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) e[nb][4 * u + r] = kScaled ? s[nb][u][r] * cq[nb] : s[nb][u][r];
+                    int mi = __float_as_int(e[nb][0]);
+#pragma unroll
+                    for (int i = 1; i < 8; ++i) mi = max(mi, __float_as_int(e[nb][i]));
+                    over = max(over, mi);
+                }
+                const bool slow = __builtin_amdgcn_ballot_w64(over > __float_as_int(kPShift)) != 0;
+                if (slow || lim < kPStep) {
+                    force = INT_MIN;
+                    float mx[kNB];
+#pragma unroll
+                    for (int nb = 0; nb < kNB; ++nb) {
+                        if (lim < kPStep) {
+#pragma unroll
+                            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                                for (int r = 0; r < 4; ++r)
+                                    if (4 * lq >= lim - (16 * u + r)) e[nb][4 * u + r] = -INFINITY;
+                        }
+                        float m = e[nb][0];
+#pragma unroll
+                        for (int i = 1; i < 8; ++i) m = fmaxf(m, e[nb][i]);
+                        mx[nb] = quad_max(m) + sref[nb];  // the column's largest score of this step, log2 units
+                    }
+                    raise_max(mx);
+#pragma unroll
+                    for (int nb = 0; nb < kNB; ++nb) {
+                        const float nref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
+                        const float d = nref - sref[nb];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) e[nb][i] -= d;
+                        sref[nb] = nref;
+                        const float c0 = kScaled ? -nref / cq[nb] : -nref;
+                        sinit[nb] = (float4v){c0, c0, c0, c0};
+                    }
+                }
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb) {
+                    uint32_t pk[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const half2v h = {(_Float16)__builtin_amdgcn_exp2f(e[nb][2 * i]), (_Float16)__builtin_amdgcn_exp2f(e[nb][2 * i + 1])};
+                        l_run[nb] = __builtin_amdgcn_fdot2(h, (half2v){(_Float16)1.0f, (_Float16)1.0f}, l_run[nb], false);
+                        pk[i] = __builtin_bit_cast(uint32_t, h);
+                    }
+                    pop[nb] = pack_half8(pk[0], pk[1], pk[2], pk[3]);
+                }
+            };
+        };
+        if (scaled)
+            walk_keys(nsteps, tiles, issue, commit, load_k, scores, softmax_for(std::true_type{}), load_v, output);
+        else
+            walk_keys(nsteps, tiles, issue, commit, load_k, scores, softmax_for(std::false_type{}), load_v, output);
     }
 
     // =============================== new tokens: bf16, causal ===============================

@@ -81,6 +81,35 @@ def test_cached_prefill_with_int8_history(hist, S):
     assert c.k_codes[:, :, hist:hist + S].any()  # the new rows were cached behind the history
 
 
+@pytest.mark.parametrize("qscale", [4.0e5, 1.0e-3])
+def test_query_magnitudes_outside_the_fp16_range(qscale):
+    """|q| * scale * log2(e) above 2^15 takes the kernel's rescaled-operand path (attention is one-hot there);
+    tiny queries give near-uniform weights.  One-hot columns whose two best scores lie within 1% of each other
+    are skipped: which of the two keys wins is decided by rounding."""
+    B, Hq, Hkv, hist, S = 1, 8, 2, 100, 37
+    qh, kh, vh = make(60, B, hist, Hq, Hkv)
+    q, k, v = make(61, B, S, Hq, Hkv)
+    q = bf16r(q * np.float32(qscale))
+    c = DeviceCache(B, Hkv, hist + S, 128)
+    c.write(torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16(), None, 0)
+    got = gpu_prefill(c, q, k, v, hist)
+    kc, vc, ks, vs = c.canonical(hist)
+    kd = np.concatenate([oracle.dequant_int8(kc, ks), k], 1)
+    want = oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v)
+    assert np.isfinite(got).all()
+    d = np.abs(got - want).max(-1)  # [B, S, Hq]
+    checked = 0
+    for si in range(S):
+        for h in range(Hq):
+            sc = kd[0, :hist + si + 1, h // (Hq // Hkv)].astype(np.float64) @ q[0, si, h].astype(np.float64)
+            top = np.sort(sc)[-2:]
+            if qscale > 1 and len(sc) > 1 and top[1] - top[0] < 1e-2 * abs(top[1]):
+                continue
+            checked += 1
+            assert d[0, si, h] < TOL_MAX, (si, h, d[0, si, h])
+    assert checked > 0.9 * S * Hq
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(4, 4), (4, 2), (8, 2), (16, 2), (32, 8)])
 def test_gqa_group_sizes(Hq, Hkv):
     hist, S = 40, 50
