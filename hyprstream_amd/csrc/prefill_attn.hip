@@ -127,11 +127,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     const bool wv_active = wv_q0 < S;
 
     float4v acc[kNB][8];
-    float m_run[kNB], l_run[kNB];
+    float m_run[kNB];
+    float4v l_run[kNB];  // row sums, kept on the matrix pipe: ones(16x32) x P^T, every register holds the column's sum
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
         m_run[nb] = -INFINITY;
-        l_run[nb] = 0.0f;
+        l_run[nb] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
     }
@@ -261,11 +262,16 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         auto commit = [&](StepTile &t, int step) {
             const int last = H - 1 - step * kPStep;  // keys past the end become zero rows
-            const _Float16 sk = (_Float16)(krow > last ? 0.0f : fminf(rawsk, kMaxScale));
+            float fk = rawsk, fv0 = rawsv[0], fv1 = rawsv[1];
+            if (last < kPStep - 1) {  // the last, partial step only
+                if (krow > last) fk = 0.0f;
+                if (vkey > last) fv0 = 0.0f;
+                if (vkey + 1 > last) fv1 = 0.0f;
+            }
+            const _Float16 sk = (_Float16)fminf(fk, kMaxScale);
             const _Float16 bias = (_Float16)1152.0f;
             *(half8 *)(t.k[wave] + obase) = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
-            const half2v sv = {(_Float16)(vkey > last ? 0.0f : fminf(rawsv[0], kMaxScale)),
-                               (_Float16)(vkey + 1 > last ? 0.0f : fminf(rawsv[1], kMaxScale))};
+            const half2v sv = {(_Float16)fminf(fv0, kMaxScale), (_Float16)fminf(fv1, kMaxScale)};
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const half2v hv = __builtin_bit_cast(half2v, int8_pair_to_f16(rawv[0], rawv[1], i)) * sv;
@@ -274,6 +280,9 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         float4v s[kNB][2];  // scores of the step between scores() and softmax()
         half8 pop[kNB];     // P^T operands between softmax() and output()
+        half8 ones;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
         half8 kop[8], vop[8];  // the step's A operands, read from LDS ahead of use
         // The score accumulators start from -sref (over cq) instead of zero, sref = m_run - kPShift being the
         // value the softmax subtracts: the MFMA result is then the exponent of the weight itself.
@@ -369,10 +378,10 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const half2v h = {(_Float16)__builtin_amdgcn_exp2f(e[nb][2 * i]), (_Float16)__builtin_amdgcn_exp2f(e[nb][2 * i + 1])};
-                        l_run[nb] = __builtin_amdgcn_fdot2(h, (half2v){(_Float16)1.0f, (_Float16)1.0f}, l_run[nb], false);
                         pk[i] = __builtin_bit_cast(uint32_t, h);
                     }
                     pop[nb] = pack_half8(pk[0], pk[1], pk[2], pk[3]);
+                    l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pop[nb], l_run[nb], 0, 0, 0);
                 }
             };
         };
@@ -384,14 +393,28 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 
     // =============================== new tokens: bf16, causal ===============================
     {
+        // Q operands carry the softmax scale and log2(e), rounded back to bf16 (2^-9 relative, the precision the
+        // weights are rounded to anyway), so that the MFMA result needs no multiplication; as in the history
+        // phase the score accumulators start from -sref and the common step only checks for an overflow.
         bf16x8 qop[kNB][4];
+        float sref[kNB];
+        float4v sinit[kNB];
+        int force = H > 0 ? INT_MIN : INT_MAX;  // nothing seen yet: the first step sets the reference
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
             const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 32 * lq;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) qop[nb][j] = __builtin_bit_cast(bf16x8, *(const u32x4 *)(qp + 8 * j));
+            for (int j = 0; j < 4; ++j) {
+                const u32x4 w = *(const u32x4 *)(qp + 8 * j);
+                uint32_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    o[e] = pack_bf16x2(__uint_as_float(w[e] << 16) * a.scale_log2e, __uint_as_float(w[e] & 0xffff0000u) * a.scale_log2e);
+                qop[nb][j] = pack_bf16x8(o[0], o[1], o[2], o[3]);
+            }
+            sref[nb] = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
+            sinit[nb] = (float4v){-sref[nb], -sref[nb], -sref[nb], -sref[nb]};
         }
-        const float cq = a.scale_log2e;
         const int nsteps = wg_qlast / kPStep + 1;
         const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
@@ -428,7 +451,9 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         float4v s[kNB][2];
         bf16x8 pop[kNB];
         auto mine = [&](int step) { return wv_active && step * kPStep <= wv_qlast; };  // else all keys are in the future
-        bf16x8 kop[8], vop[8];
+        bf16x8 kop[8], vop[8], ones;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
         auto load_k = [&](const StepTile &t, int step) {
             if (!mine(step)) return;
 #pragma unroll
@@ -444,7 +469,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = (float4v){0.f, 0.f, 0.f, 0.f};
+                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = sinit[nb];
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -456,37 +481,53 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             if (!mine(step)) return;
             const int t0 = step * kPStep;
             const bool diag = t0 + kPStep - 1 > wv_q0;  // some (key, query) pair of this step is in the future
-            float sc[kNB][8], mx[kNB];
+            float e[kNB][8];
+            int over = force;
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) sc[nb][4 * u + r] = s[nb][u][r] * cq;
+                    for (int r = 0; r < 4; ++r) e[nb][4 * u + r] = s[nb][u][r];
                 if (diag) {
-                    const int qlim = min(qi[nb], S - 1);
+                    const int qrel = min(qi[nb], S - 1) - t0 - 4 * lq;  // key offsets 16u + r beyond this are in the future
 #pragma unroll
                     for (int u = 0; u < 2; ++u)
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            if (t0 + 16 * u + 4 * lq + r > qlim) sc[nb][4 * u + r] = -INFINITY;
+                            if (16 * u + r > qrel) e[nb][4 * u + r] = -INFINITY;
                 }
-                float m = sc[nb][0];
 #pragma unroll
-                for (int i = 1; i < 8; ++i) m = fmaxf(m, sc[nb][i]);
-                mx[nb] = quad_max(m);
+                for (int i = 0; i < 8; ++i) over = max(over, __float_as_int(e[nb][i]));
             }
-            raise_max(mx);
+            if (__builtin_amdgcn_ballot_w64(over > __float_as_int(kPShift)) != 0) {
+                force = INT_MIN;
+                float mx[kNB];
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb) {
+                    float m = e[nb][0];
+#pragma unroll
+                    for (int i = 1; i < 8; ++i) m = fmaxf(m, e[nb][i]);
+                    mx[nb] = quad_max(m) + sref[nb];
+                }
+                raise_max(mx);
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb) {
+                    const float nref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
+                    const float d = nref - sref[nb];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) e[nb][i] -= d;
+                    sref[nb] = nref;
+                    sinit[nb] = (float4v){-nref, -nref, -nref, -nref};
+                }
+            }
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
-                const float mref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
                 float p[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    p[i] = __builtin_amdgcn_exp2f(sc[nb][i] - mref);
-                    l_run[nb] += p[i];
-                }
+                for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_exp2f(e[nb][i]);
                 pop[nb] = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
+                l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pop[nb], l_run[nb], 0, 0, 0);
             }
         };
         auto output = [&](int step) {
@@ -503,7 +544,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     // =============================== normalise and store ===============================
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
-        const float l = quad_sum(l_run[nb]);
+        const float l = l_run[nb][0];
         if (qi[nb] >= S) continue;
         const float inv = 1.0f / l;
         uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kPD + 32 * lq;
