@@ -54,19 +54,28 @@ struct alignas(16) StepTile {
     uint8_t v[8][1024];  // block bb: V^T rows d = 8*li + bb, 32 keys
 };
 
+struct alignas(16) HistTile {
+    StepTile h[2];  // keys 0..31 and 32..63 of a 64-key history step
+};
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
 // load, i.e. for the tile prefetch that was issued a moment earlier and is not needed before the next step.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Walk `n` key steps.  A step of one wavefront is
+// Walk `n` key steps of the new-token phase (the history phase has its own loop, same shape, 64 keys per step).
+// A step of one wavefront is
 //   scores  : S^T = K Q^T                     -- MFMA, operands from LDS
 //   softmax : P from S, running max and sum   -- VALU only
 //   output  : O^T += V^T P^T                  -- MFMA, operands from LDS
 // with one workgroup barrier per step: while tile s is consumed every wavefront converts its share of tile s+1
 // into the other buffer and starts the global loads of tile s+2.  All LDS operand reads of a step are issued
-// before its first MFMA.  (A variant that kept the two wavefronts of a SIMD half a step apart behind a second
-// barrier, so that one did softmax while the other fed the matrix pipe, measured 6% slower: a wavefront issues
-// at most one instruction every four cycles whatever its kind, and the extra barrier cost more than it hid.)
+// before its first MFMA.
+// What was measured on this loop (gfx950, two wavefronts per SIMD): an MFMA 16x16x32 occupies the SIMD's
+// vector issue port for about half of its 16 cycles, plain vector instructions run in its shadow (two per MFMA
+// are free), v_exp_f32 one per MFMA, while v_dot2_f32_f16 stalls the matrix pipe (row sums are therefore an
+// MFMA with a ones operand, not dot products or additions).  Variants that paired the matrix work of one
+// wavefront with the vector work of the other behind a second barrier per step, or that software-pipelined
+// scores(s+1) against softmax(s) inside one wavefront, were correct but not faster than this order.
 template <class Issue, class Commit, class LoadK, class Scores, class Softmax, class LoadV, class Output>
 __device__ __forceinline__ void walk_keys(int n, StepTile *tiles, Issue issue, Commit commit, LoadK load_k, Scores scores,
                                           Softmax softmax, LoadV load_v, Output output) {
@@ -87,7 +96,8 @@ __device__ __forceinline__ void walk_keys(int n, StepTile *tiles, Issue issue, C
 }
 
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
-    __shared__ StepTile tiles[2];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];
+    StepTile *tiles = (StepTile *)lds;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: wavefront-dependent branches stay uniform
     const int li = lane & 15, lq = lane >> 4;
@@ -160,6 +170,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     };
 
     const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
+    const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;  // wavefronts w and w+4 share a SIMD
 
     // =============================== history: int8 cache, f16 MFMA ===============================
     if (H > 0) {
@@ -196,23 +207,30 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         }
         scaled = __builtin_amdgcn_ballot_w64(scaled) != 0;
 
-        const int nsteps = (H + kPStep - 1) / kPStep;
-        // ---- producers: every wavefront converts one eighth of the step's K tile and of its V tile.
-        //      K: wavefront w fills operand block w (tile u = w/4, k-group j = w%4); lane (li, lq) loads the
-        //         eight codes K[16u + li][32lq + 8j ..] (the d's of Q operand j) and writes them as one half8.
-        //      V: lane = (d-quad x = lane%32, key pair kp = 2w + lane/32).  Slots 2*pe, 2*pe+1 of key group g
-        //         (kp = 4g + pe) are the adjacent keys 16*(pe/2) + 4g + 2*(pe%2), +1; one dword of each (a
-        //         row is read by 32 consecutive lanes) gives four fp16 pairs, for d = 4x + i, stored in
-        //         block 4*(x%2) + i at operand lane (x/2, g).
+        // A history step covers 64 keys: two 32-key tiles (halves) in the layout of StepTile.  The work that comes
+        // once per step whatever its size -- barrier, loop and address bookkeeping, the overflow check, waits --
+        // is shared by twice as many MFMAs as in a 32-key step.
+        constexpr int kHStep = 64;
+        const int nsteps = (H + kHStep - 1) / kHStep;
+        HistTile *htiles = (HistTile *)lds;
+        // ---- producers: every wavefront converts one eighth of the step's K tiles and of its V tiles.
+        //      K: wavefront w takes 16-key block u4 = w/2 and the d-halves jp = w%2 of every 32-d group: lane
+        //         (li, lq) loads the 16 codes K[16u4 + li][32lq + 16jp ..] and writes operand blocks j = 2jp and
+        //         2jp+1 of tile u4/2 (eight codes = the d's of Q operand j each).
+        //      V: lane = (d-octet x = lane%16, key pair pp = 4w + lane/16).  Pair pp = 16hh + 4g + pe of tile hh:
+        //         slots 2pe, 2pe+1 of key group g are the adjacent keys 16*(pe/2) + 4g + 2*(pe%2), +1; eight
+        //         bytes of each give the fp16 pairs for d = 8x + bb, stored in block bb at operand lane (x, g).
         //      The per-token scales are applied here, once per workgroup, rather than to every score and weight:
         //      the operands are fp16(code * scale) (relative rounding 2^-11, finer than a bf16 cache would keep).
-        const int vx = lane & 31, vkp = 2 * wave + (lane >> 5);
-        const int vkey = 16 * ((vkp & 3) >> 1) + 4 * (vkp >> 2) + 2 * (vkp & 1);
-        const int vdst = ((vx >> 1) + 16 * (vkp >> 2)) * 16 + 4 * (vkp & 3);
-        const int krow = 16 * (wave >> 2) + li, kcol = 32 * lq + 8 * (wave & 3);
-        const uint32_t koff = krow * kPD + kcol, voff = vkey * kPD + 4 * vx;
-        u32x2 rawk = {0u, 0u};
-        uint32_t rawv[2] = {0u, 0u};
+        const int vx = lane & 15, vpp = 4 * wave + (lane >> 4);
+        const int vhh = vpp >> 4, vg = (vpp >> 2) & 3, vpe = vpp & 3;
+        const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
+        const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
+        const int ku4 = wave >> 1, kjp = wave & 1;
+        const int krow = 16 * ku4 + li, kcol = 32 * lq + 16 * kjp;
+        const uint32_t koff = krow * kPD + kcol, voff = vkey * kPD + 8 * vx;
+        u32x4 rawk = {0u, 0u, 0u, 0u};
+        u32x2 rawv[2] = {{0u, 0u}, {0u, 0u}};
         float rawsk = 0.0f, rawsv[2] = {0.0f, 0.0f};
         // issue() is called for steps 0, 1, 2, ... in order, so the (scalar) addresses of a step's codes and
         // scales advance by a constant; a block table is consulted only when a cursor leaves its block.
@@ -220,7 +238,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const float *ksp = a.ks, *vsp = a.vs;
         int kleft = 0, vleft = 0;  // tokens between the cursor and the end of its storage unit
         auto issue = [&](int step) {
-            const int t0 = step * kPStep;
+            const int t0 = step * kHStep;
             const int last = H - 1 - t0;
             if (kleft <= 0) {
                 int64_t unit;
@@ -242,50 +260,50 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             // step's (scalar) base plus a 32-bit lane offset; only the last, partial step clamps rows.
             uint32_t ko = koff, vo0 = voff, vo1 = voff + kPD, sk = 4u * krow, sv = 4u * vkey;
             uint32_t sv1 = sv + 4u;
-            if (last < kPStep - 1) {
+            if (last < kHStep - 1) {
                 ko = min(krow, last) * kPD + kcol;
-                vo0 = min(vkey, last) * kPD + 4 * vx;
-                vo1 = min(vkey + 1, last) * kPD + 4 * vx;
+                vo0 = min(vkey, last) * kPD + 8 * vx;
+                vo1 = min(vkey + 1, last) * kPD + 8 * vx;
                 sk = 4u * min(krow, last);
                 sv = 4u * min(vkey, last);
                 sv1 = 4u * min(vkey + 1, last);
             }
-            rawk = *(const u32x2 *)(kb + ko);
-            rawv[0] = *(const uint32_t *)(vb + vo0);
-            rawv[1] = *(const uint32_t *)(vb + vo1);
+            rawk = *(const u32x4 *)(kb + ko);
+            rawv[0] = *(const u32x2 *)(vb + vo0);
+            rawv[1] = *(const u32x2 *)(vb + vo1);
             rawsk = *(const float *)((const uint8_t *)ksp + sk);
             rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
             rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
-            kb += kPStep * kPD; vb += kPStep * kPD;
-            ksp += kPStep; vsp += kPStep;
-            kleft -= kPStep; vleft -= kPStep;
+            kb += kHStep * kPD; vb += kHStep * kPD;
+            ksp += kHStep; vsp += kHStep;
+            kleft -= kHStep; vleft -= kHStep;
         };
-        auto commit = [&](StepTile &t, int step) {
-            const int last = H - 1 - step * kPStep;  // keys past the end become zero rows
+        auto commit = [&](HistTile &t, int step) {
+            const int last = H - 1 - step * kHStep;  // keys past the end become zero rows
             float fk = rawsk, fv0 = rawsv[0], fv1 = rawsv[1];
-            if (last < kPStep - 1) {  // the last, partial step only
+            if (last < kHStep - 1) {  // the last, partial step only
                 if (krow > last) fk = 0.0f;
                 if (vkey > last) fv0 = 0.0f;
                 if (vkey + 1 > last) fv1 = 0.0f;
             }
             const _Float16 sk = (_Float16)fminf(fk, kMaxScale);
             const _Float16 bias = (_Float16)1152.0f;
-            *(half8 *)(t.k[wave] + obase) = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
+            uint8_t *kd = t.h[ku4 >> 1].k[4 * (ku4 & 1) + 2 * kjp] + obase;
+            *(half8 *)kd = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
+            *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[2], rawk[3]) - bias) * sk;
             const half2v sv = {(_Float16)fminf(fv0, kMaxScale), (_Float16)fminf(fv1, kMaxScale)};
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const half2v hv = __builtin_bit_cast(half2v, int8_pair_to_f16(rawv[0], rawv[1], i)) * sv;
-                *(uint32_t *)(t.v[4 * (vx & 1) + i] + vdst) = __builtin_bit_cast(uint32_t, hv);
+            for (int bb = 0; bb < 8; ++bb) {
+                const half2v hv = __builtin_bit_cast(half2v, int8_pair_to_f16(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3)) * sv;
+                *(uint32_t *)(t.h[vhh].v[bb] + vdst) = __builtin_bit_cast(uint32_t, hv);
             }
         };
-        float4v s[kNB][2];  // scores of the step between scores() and softmax()
-        half8 pop[kNB];     // P^T operands between softmax() and output()
+        float4v s[kNB][4];    // scores of the step: key block u4 = 2*half + u
+        half8 pop[kNB][2];    // P^T operands per half
+        half8 kop[8], vop[8];
         half8 ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
-        half8 kop[8], vop[8];  // the step's A operands, read from LDS ahead of use
-        // The score accumulators start from -sref (over cq) instead of zero, sref = m_run - kPShift being the
-        // value the softmax subtracts: the MFMA result is then the exponent of the weight itself.
         float sref[kNB];
         float4v sinit[kNB];
         int force = INT_MAX;  // takes the first step through the branch that sets the reference
@@ -294,32 +312,33 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             sref[nb] = 0.0f;
             sinit[nb] = (float4v){0.f, 0.f, 0.f, 0.f};
         }
-        auto load_k = [&](const StepTile &t, int) {
+        auto scores = [&](const HistTile &t) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) kop[i] = *(const half8 *)(t.k[i] + obase);
-        };
-        auto load_v = [&](const StepTile &t, int) {
+            for (int hh = 0; hh < 2; ++hh) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vop[i] = *(const half8 *)(t.v[i] + obase);
-        };
-        auto scores = [&](int) {
+                for (int i = 0; i < 8; ++i) kop[i] = *(const half8 *)(t.h[hh].k[i] + obase);
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = sinit[nb];
+                    for (int nb = 0; nb < kNB; ++nb) s[nb][2 * hh + u] = sinit[nb];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                    for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int nb = 0; nb < kNB; ++nb)
-                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[4 * u + j], qop[nb][j], s[nb][u], 0, 0, 0);
+                        for (int nb = 0; nb < kNB; ++nb)
+                            s[nb][2 * hh + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[4 * u + j], qop[nb][j], s[nb][2 * hh + u], 0, 0, 0);
+                }
             }
         };
-        auto output = [&](int) {
+        auto load_v = [&](const HistTile &t, int hh) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vop[i] = *(const half8 *)(t.h[hh].v[i] + obase);
+        };
+        auto output = [&](int hh) {
 #pragma unroll
             for (int bb = 0; bb < 8; ++bb)
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb], acc[nb][bb], 0, 0, 0);
+                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb][hh], acc[nb][bb], 0, 0, 0);
         };
         // softmax(): e = exponent of each weight (score in log2 units minus sref).  The common step only checks,
         // per lane and on the bit patterns (a positive float orders like its bits; a NaN reads as large), whether
@@ -327,37 +346,35 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // partial last step does the wavefront reduce the column maxima and move the reference.
         auto softmax_for = [&](auto scaled_tag) {
             constexpr bool kScaled = decltype(scaled_tag)::value;
-            return [&](const StepTile &, int step) {
-                const int lim = H - step * kPStep;  // keys of this step that exist
-                float e[kNB][8];
+            return [&](int step) {
+                const int lim = H - step * kHStep;  // keys of this step that exist
+                float e[kNB][16];
                 int over = force;
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb) {
 #pragma unroll
-                    for (int u = 0; u < 2; ++u)
+                    for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
-                        for (int r = 0; r < 4; ++r) e[nb][4 * u + r] = kScaled ? s[nb][u][r] * cq[nb] : s[nb][u][r];
-                    int mi = __float_as_int(e[nb][0]);
+                        for (int r = 0; r < 4; ++r) e[nb][4 * u4 + r] = kScaled ? s[nb][u4][r] * cq[nb] : s[nb][u4][r];
 #pragma unroll
-                    for (int i = 1; i < 8; ++i) mi = max(mi, __float_as_int(e[nb][i]));
-                    over = max(over, mi);
+                    for (int i = 0; i < 16; ++i) over = max(over, __float_as_int(e[nb][i]));
                 }
                 const bool slow = __builtin_amdgcn_ballot_w64(over > __float_as_int(kPShift)) != 0;
-                if (slow || lim < kPStep) {
+                if (slow || lim < kHStep) {
                     force = INT_MIN;
                     float mx[kNB];
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb) {
-                        if (lim < kPStep) {
+                        if (lim < kHStep) {
 #pragma unroll
-                            for (int u = 0; u < 2; ++u)
+                            for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
                                 for (int r = 0; r < 4; ++r)
-                                    if (4 * lq >= lim - (16 * u + r)) e[nb][4 * u + r] = -INFINITY;
+                                    if (4 * lq >= lim - (16 * u4 + r)) e[nb][4 * u4 + r] = -INFINITY;
                         }
                         float m = e[nb][0];
 #pragma unroll
-                        for (int i = 1; i < 8; ++i) m = fmaxf(m, e[nb][i]);
+                        for (int i = 1; i < 16; ++i) m = fmaxf(m, e[nb][i]);
                         mx[nb] = quad_max(m) + sref[nb];  // the column's largest score of this step, log2 units
                     }
                     raise_max(mx);
@@ -366,29 +383,60 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                         const float nref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
                         const float d = nref - sref[nb];
 #pragma unroll
-                        for (int i = 0; i < 8; ++i) e[nb][i] -= d;
+                        for (int i = 0; i < 16; ++i) e[nb][i] -= d;
                         sref[nb] = nref;
                         const float c0 = kScaled ? -nref / cq[nb] : -nref;
                         sinit[nb] = (float4v){c0, c0, c0, c0};
                     }
                 }
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb) {
-                    uint32_t pk[4];
+                for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const half2v h = {(_Float16)__builtin_amdgcn_exp2f(e[nb][2 * i]), (_Float16)__builtin_amdgcn_exp2f(e[nb][2 * i + 1])};
-                        pk[i] = __builtin_bit_cast(uint32_t, h);
+                    for (int hh = 0; hh < 2; ++hh) {
+                        uint32_t pk[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const half2v h = {(_Float16)__builtin_amdgcn_exp2f(e[nb][8 * hh + 2 * i]),
+                                              (_Float16)__builtin_amdgcn_exp2f(e[nb][8 * hh + 2 * i + 1])};
+                            pk[i] = __builtin_bit_cast(uint32_t, h);
+                        }
+                        pop[nb][hh] = pack_half8(pk[0], pk[1], pk[2], pk[3]);
+                        l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pop[nb][hh], l_run[nb], 0, 0, 0);
                     }
-                    pop[nb] = pack_half8(pk[0], pk[1], pk[2], pk[3]);
-                    l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pop[nb], l_run[nb], 0, 0, 0);
-                }
             };
         };
+        // One barrier per step: while tile s is consumed every wavefront converts its share of tile s+1 into
+        // the other buffer and starts the global loads of tile s+2.  The second wavefront of each SIMD does its
+        // conversion at the end of the step instead of the beginning, so that its matrix phases tend to meet
+        // the other one's vector phases.
+        auto walk = [&](auto softmax) {
+            issue(0);
+            commit(htiles[0], 0);
+            if (nsteps > 1) issue(1);
+            lds_barrier();
+            for (int st = 0; st < nsteps; ++st) {
+                if (!late) {
+                    if (st + 1 < nsteps) commit(htiles[(st + 1) & 1], st + 1);
+                    if (st + 2 < nsteps) issue(st + 2);
+                }
+                const HistTile &t = htiles[st & 1];
+                scores(t);
+                load_v(t, 0);
+                softmax(st);
+                output(0);
+                load_v(t, 1);
+                output(1);
+                if (late) {
+                    if (st + 1 < nsteps) commit(htiles[(st + 1) & 1], st + 1);
+                    if (st + 2 < nsteps) issue(st + 2);
+                }
+                lds_barrier();
+            }
+        };
         if (scaled)
-            walk_keys(nsteps, tiles, issue, commit, load_k, scores, softmax_for(std::true_type{}), load_v, output);
+            walk(softmax_for(std::true_type{}));
         else
-            walk_keys(nsteps, tiles, issue, commit, load_k, scores, softmax_for(std::false_type{}), load_v, output);
+            walk(softmax_for(std::false_type{}));
     }
 
     // =============================== new tokens: bf16, causal ===============================
