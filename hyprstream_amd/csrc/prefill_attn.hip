@@ -46,6 +46,7 @@ struct PrefillArgs {
     KvAddr ka, va;
     uint16_t *out;  // [B,S,Hq,D] bf16
     int32_t B, S, Hq, Hkv, G, HG, hist_len;
+    int32_t heavy_first;  // the grid outnumbers the CUs: order the query tiles by decreasing work
     float scale_log2e;
 };
 
@@ -112,6 +113,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             const int p = bx + X * (by + gridDim.y * bz);  // dispatch order
             const int grp = (p & 7) + 8 * (p / (8 * X));   // (kv-head group, sequence) unit
             bx = (p >> 3) % X;
+            if (a.heavy_first) bx = X - 1 - bx;  // late query tiles have the most keys: start them first
             by = grp % gridDim.y;
             bz = grp / gridDim.y;
         }
@@ -608,6 +610,19 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
 
+// CUs of the current device (looked up once per device; 256 if the query fails).
+static int compute_units() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return n;
+}
+
 }  // namespace hs
 
 extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_new, int8_t *k_codes,
@@ -630,8 +645,8 @@ extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void
     if ((int64_t)hist_len + (quantize_on_write ? S : 0) > cap)
         return fail(HS_ERR_OVERFLOW, "Cache overflow: trying to cache %d tokens starting at position %d, but capacity is %lld",
                     S, hist_len, (long long)cap);
-    if (layout->k_block_table && (layout->capacity_tokens % kPStep) != 0)
-        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of %d tokens", kPStep);
+    if (layout->k_block_table && (layout->capacity_tokens % 64) != 0)  // a history step reads 64 tokens of one block
+        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of 64 tokens");
     if (B == 0 || S == 0) return HS_OK;
     hipStream_t st = (hipStream_t)stream;
     PrefillArgs a;
@@ -645,6 +660,9 @@ extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void
     a.scale_log2e = softmax_scale * kPLog2e;
     const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
     dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * (G / a.HG), B);
+    // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
+    // that the launch does not end on them; a single round keeps the plain order.
+    a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
     prefill_attn_kernel<<<grid, 512, 0, st>>>(a);
     if (int rc = check_launch("prefill_attn")) return rc;
     if (quantize_on_write)
