@@ -65,6 +65,28 @@ def test_prompt_without_history(S):
     assert np.array_equal(kc, wk) and np.array_equal(vc, wv) and np.array_equal(ks, wks) and np.array_equal(vs, wvs)
 
 
+def test_long_prompt_more_workgroups_than_cus():
+    """18 query tiles x 8 kv-heads x 2 sequences = 288 workgroups: more than the chip's CUs, which is when the
+    kernel starts the query tiles with the most keys first."""
+    q, k, v = make(33, 2, 1100, 32, 8)
+    c = DeviceCache(2, 8, 1100, 128)
+    got = gpu_prefill(c, q, k, v, 0)
+    compare(got, oracle_prefill(q, None, None, k, v), "prompt S=1100")
+
+
+def test_paged_blocks_must_hold_multiples_of_64_tokens():
+    B, Hq, Hkv, D, BT = 1, 8, 2, 128, 96
+    q, k, v = make(34, B, 8, Hq, Hkv)
+    tab = torch.zeros(B, 2, dtype=torch.int32, device=DEV)
+    pool_c = torch.zeros(4, Hkv, BT, D, dtype=torch.int8, device=DEV)
+    pool_s = torch.zeros(4, Hkv, BT, dtype=torch.float32, device=DEV)
+    lay = hb.paged_layout(Hkv, BT, D, tab, tab)
+    qt, kt, vt = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
+    out = torch.empty(B, 8, Hq, D, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(hb.HsError, match="multiple of 64"):
+        hb.prefill_attn(qt, kt, vt, pool_c, pool_c, pool_s, pool_s, lay, 0, out, 1.0 / np.sqrt(D), False)
+
+
 @pytest.mark.parametrize("hist,S", [(19, 5), (1, 1), (32, 64), (100, 37), (256, 256)])
 def test_cached_prefill_with_int8_history(hist, S):
     """New rows on top of an int8 history: the reference's partial-prefill case (tril(k_len - q_len))."""
