@@ -46,6 +46,25 @@ __device__ __forceinline__ uint32_t int8_pair_to_f16(uint32_t lo, uint32_t hi, i
     return __builtin_bit_cast(uint32_t, hv);
 }
 
+// e4m3fn codes -> fp16.  A code shifted into bits 14..7 of a half (sign kept in bit 15) is the fp16 number
+// value/256, subnormal codes included (fp16 subnormals have the same shape eight binades lower); the producer
+// multiplies by 256 * scale afterwards.  `t` holds one code in the high byte of each half.
+__device__ __forceinline__ uint32_t e4m3_high_bytes_to_f16(uint32_t t) {
+    return (t & 0x80008000u) | ((t & 0x7f007f00u) >> 1);
+}
+// Eight e4m3fn codes (two dwords, byte order = k-slot order) -> eight fp16 holding value/256.
+__device__ __forceinline__ half8 e4m3x8_to_f16_div256(uint32_t w0, uint32_t w1) {
+    return pack_half8(e4m3_high_bytes_to_f16(__builtin_amdgcn_perm(0u, w0, 0x010c000cu)),
+                      e4m3_high_bytes_to_f16(__builtin_amdgcn_perm(0u, w0, 0x030c020cu)),
+                      e4m3_high_bytes_to_f16(__builtin_amdgcn_perm(0u, w1, 0x010c000cu)),
+                      e4m3_high_bytes_to_f16(__builtin_amdgcn_perm(0u, w1, 0x030c020cu)));
+}
+// Byte `bsel` (0..3) of `lo` and of `hi` (e4m3fn codes) -> two fp16 holding value/256.
+__device__ __forceinline__ uint32_t e4m3_pair_to_f16_div256(uint32_t lo, uint32_t hi, int bsel) {
+    const uint32_t sel = ((4u + (uint32_t)bsel) << 24) | 0x000c000cu | ((uint32_t)bsel << 8);
+    return e4m3_high_bytes_to_f16(__builtin_amdgcn_perm(hi, lo, sel));
+}
+
 // 16-bit half `hsel` (0 = low, 1 = high) of `lo` and of `hi` packed into one dword (lo first).
 __device__ __forceinline__ uint32_t pick_halves(uint32_t lo, uint32_t hi, int hsel) {
     return __builtin_amdgcn_perm(hi, lo, hsel ? 0x07060302u : 0x05040100u);

@@ -96,6 +96,7 @@ __device__ __forceinline__ void walk_keys(int n, StepTile *tiles, Issue issue, C
     }
 }
 
+template <bool FP8>  // format of the history: int8 codes with token scales, or e4m3fn codes with head scales
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];
     StepTile *tiles = (StepTile *)lds;
@@ -234,6 +235,10 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         u32x4 rawk = {0u, 0u, 0u, 0u};
         u32x2 rawv[2] = {{0u, 0u}, {0u, 0u}};
         float rawsk = 0.0f, rawsv[2] = {0.0f, 0.0f};
+        if (FP8) {  // one scale per (sequence, kv-head); the codes convert to value/256 (see e4m3_high_bytes_to_f16)
+            rawsk = 256.0f * a.ks[(int64_t)b * a.Hkv + kvh];
+            rawsv[0] = rawsv[1] = 256.0f * a.vs[(int64_t)b * a.Hkv + kvh];
+        }
         // issue() is called for steps 0, 1, 2, ... in order, so the (scalar) addresses of a step's codes and
         // scales advance by a constant; a block table is consulted only when a cursor leaves its block.
         const uint8_t *kb = a.kc, *vb = a.vc;
@@ -247,7 +252,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 int slot;
                 resolve(a.ka, b, t0, unit, slot);
                 kb = a.kc + unit * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)slot * kPD;
-                ksp = a.ks + unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot;
+                if (!FP8) ksp = a.ks + unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot;
                 kleft = a.ka.capacity_tokens - slot;
             }
             if (vleft <= 0) {
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 int slot;
                 resolve(a.va, b, t0, unit, slot);
                 vb = a.vc + unit * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)slot * kPD;
-                vsp = a.vs + unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot;
+                if (!FP8) vsp = a.vs + unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot;
                 vleft = a.va.capacity_tokens - slot;
             }
             // The loaded values are only touched in commit(): nothing waits for a load here.  Addresses are the
@@ -273,9 +278,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             rawk = *(const u32x4 *)(kb + ko);
             rawv[0] = *(const u32x2 *)(vb + vo0);
             rawv[1] = *(const u32x2 *)(vb + vo1);
-            rawsk = *(const float *)((const uint8_t *)ksp + sk);
-            rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
-            rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
+            if (!FP8) {
+                rawsk = *(const float *)((const uint8_t *)ksp + sk);
+                rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
+                rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
+            }
             kb += kHStep * kPD; vb += kHStep * kPD;
             ksp += kHStep; vsp += kHStep;
             kleft -= kHStep; vleft -= kHStep;
@@ -288,15 +295,24 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 if (vkey > last) fv0 = 0.0f;
                 if (vkey + 1 > last) fv1 = 0.0f;
             }
-            const _Float16 sk = (_Float16)fminf(fk, kMaxScale);
+            // largest operand: 127 * scale (int8), 1.75 * 256 * scale (fp8); both stay finite in fp16
+            const float smax = FP8 ? 64.0f * kMaxScale : kMaxScale;
+            const _Float16 sk = (_Float16)fminf(fk, smax);
             const _Float16 bias = (_Float16)1152.0f;
             uint8_t *kd = t.h[ku4 >> 1].k[4 * (ku4 & 1) + 2 * kjp] + obase;
-            *(half8 *)kd = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
-            *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[2], rawk[3]) - bias) * sk;
-            const half2v sv = {(_Float16)fminf(fv0, kMaxScale), (_Float16)fminf(fv1, kMaxScale)};
+            if (FP8) {
+                *(half8 *)kd = e4m3x8_to_f16_div256(rawk[0], rawk[1]) * sk;
+                *(half8 *)(kd + 1024) = e4m3x8_to_f16_div256(rawk[2], rawk[3]) * sk;
+            } else {
+                *(half8 *)kd = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
+                *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[2], rawk[3]) - bias) * sk;
+            }
+            const half2v sv = {(_Float16)fminf(fv0, smax), (_Float16)fminf(fv1, smax)};
 #pragma unroll
             for (int bb = 0; bb < 8; ++bb) {
-                const half2v hv = __builtin_bit_cast(half2v, int8_pair_to_f16(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3)) * sv;
+                const uint32_t pair = FP8 ? e4m3_pair_to_f16_div256(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3)
+                                          : int8_pair_to_f16(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3);
+                const half2v hv = __builtin_bit_cast(half2v, pair) * sv;
                 *(uint32_t *)(t.h[vhh].v[bb] + vdst) = __builtin_bit_cast(uint32_t, hv);
             }
         };
@@ -623,14 +639,11 @@ static int compute_units() {
     return n;
 }
 
-}  // namespace hs
-
-extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_new, int8_t *k_codes,
-                                    int8_t *v_codes, float *k_scales, float *v_scales, const hs_kv_layout *layout,
-                                    int32_t hist_len, void *out, int32_t B, int32_t S, int32_t Hq, int32_t Hkv,
-                                    int32_t D, float softmax_scale, int quantize_on_write, hs_stream_t stream) {
-    using namespace hs;
-    if (int rc = validate_layout(layout, B, S, Hkv, D, true)) return rc;
+static int launch_prefill(bool fp8, const void *q, const void *k_new, const void *v_new, void *k_codes, void *v_codes,
+                          float *k_scales, float *v_scales, const hs_kv_layout *layout, int32_t hist_len, void *out,
+                          int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale,
+                          int quantize_on_write, hs_stream_t stream) {
+    if (int rc = validate_layout(layout, B, S, Hkv, D, !fp8)) return rc;
     if (D != kPD) return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 128, got %d", D);
     const bool empty = B == 0 || S == 0;  // an empty problem may come with null pointers (an empty tensor has none)
     if (!empty && (!q || !k_new || !v_new || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
@@ -663,10 +676,35 @@ extern "C" int hs_prefill_attn_int8(const void *q, const void *k_new, const void
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
-    prefill_attn_kernel<<<grid, 512, 0, st>>>(a);
+    if (fp8) prefill_attn_kernel<true><<<grid, 512, 0, st>>>(a);
+    else prefill_attn_kernel<false><<<grid, 512, 0, st>>>(a);
     if (int rc = check_launch("prefill_attn")) return rc;
-    if (quantize_on_write)
-        return hs_kv_quantize_int8(k_new, v_new, HS_BF16, k_codes, v_codes, k_scales, v_scales, layout, nullptr,
-                                   hist_len, B, S, Hkv, D, stream);
-    return HS_OK;
+    if (!quantize_on_write) return HS_OK;
+    if (fp8)
+        return hs_kv_quantize_fp8(k_new, v_new, HS_BF16, (uint8_t *)k_codes, (uint8_t *)v_codes, k_scales, v_scales,
+                                  layout, nullptr, hist_len, B, S, Hkv, D, stream);
+    return hs_kv_quantize_int8(k_new, v_new, HS_BF16, (int8_t *)k_codes, (int8_t *)v_codes, k_scales, v_scales, layout,
+                               nullptr, hist_len, B, S, Hkv, D, stream);
 }
+
+}  // namespace hs
+
+extern "C" {
+
+int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_new, int8_t *k_codes, int8_t *v_codes,
+                         float *k_scales, float *v_scales, const hs_kv_layout *layout, int32_t hist_len, void *out,
+                         int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale,
+                         int quantize_on_write, hs_stream_t stream) {
+    return hs::launch_prefill(false, q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, hist_len, out, B, S,
+                              Hq, Hkv, D, softmax_scale, quantize_on_write, stream);
+}
+
+int hs_prefill_attn_fp8(const void *q, const void *k_new, const void *v_new, uint8_t *k_codes, uint8_t *v_codes,
+                        const float *k_scales, const float *v_scales, const hs_kv_layout *layout, int32_t hist_len,
+                        void *out, int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale,
+                        int quantize_on_write, hs_stream_t stream) {
+    return hs::launch_prefill(true, q, k_new, v_new, k_codes, v_codes, (float *)k_scales, (float *)v_scales, layout,
+                              hist_len, out, B, S, Hq, Hkv, D, softmax_scale, quantize_on_write, stream);
+}
+
+}  // extern "C"

@@ -30,7 +30,7 @@ def gpu_prefill(cache, q, k, v, hist, write=True):
     qt, kt, vt = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
     out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
     hb.prefill_attn(qt, kt, vt, cache.k_codes, cache.v_codes, cache.k_scales, cache.v_scales, cache.layout, hist, out,
-                    1.0 / np.sqrt(D), write)
+                    1.0 / np.sqrt(D), write, fp8=cache.fp8)
     torch.cuda.synchronize()
     return out.float().cpu().numpy()
 
@@ -101,6 +101,46 @@ def test_cached_prefill_with_int8_history(hist, S):
     want = oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v)
     compare(got, want, "hist=%d S=%d" % (hist, S))
     assert c.k_codes[:, :, hist:hist + S].any()  # the new rows were cached behind the history
+
+
+@pytest.mark.parametrize("hist,S,sigma", [(19, 5, 1.0), (64, 64, 0.5), (150, 70, 0.5), (333, 200, 1.0)])
+def test_cached_prefill_with_fp8_history(hist, S, sigma):
+    """The same over an e4m3fn history with per-head scales: the new rows are encoded with the scales calibrated
+    on the history (values beyond 448 * scale clamp, as in the oracle), then join the attended history."""
+    B, Hq, Hkv = 2, 8, 2
+    qh, kh, vh = make(70 + hist, B, hist, Hq, Hkv, sigma=sigma)
+    q, k, v = make(71 + S, B, S, Hq, Hkv, sigma=sigma)
+    c = DeviceCache(B, Hkv, hist + S, 128, fp8=True)
+    hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+    hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+    c.write(hk, hv, None, 0)
+    got = gpu_prefill(c, q, k, v, hist)
+    kc, vc, ks, vs = c.canonical(hist + S)
+    want = oracle_prefill(q, oracle.dequant_fp8(kc[:, :hist], ks), oracle.dequant_fp8(vc[:, :hist], vs), k, v)
+    compare(got, want, "fp8 hist=%d S=%d" % (hist, S))
+    # the new rows were cached behind the history with the oracle's codes
+    ek, ev = oracle.quant_fp8(k, ks), oracle.quant_fp8(v, vs)
+    assert np.array_equal(kc[:, hist:], ek) and np.array_equal(vc[:, hist:], ev)
+
+
+def test_fp8_history_with_subnormal_codes_and_every_code_value():
+    """All 254 finite e4m3fn codes (subnormals included) in the history convert exactly: one key per code value
+    in V (K codes cycle too), compared with the oracle's dequantized view."""
+    B, Hq, Hkv, D, hist, S = 1, 4, 1, 128, 256, 16
+    r = wl.philox(77)
+    codes = np.arange(256, dtype=np.uint8)
+    codes[codes == 0x7f] = 0x7e
+    codes[codes == 0xff] = 0xfe
+    kc = np.stack([np.roll(codes, 3 * d) for d in range(D)], -1).reshape(1, hist, 1, D)
+    vc = np.stack([np.roll(codes, 7 * d + 1) for d in range(D)], -1).reshape(1, hist, 1, D)
+    ks = np.array([[0.004]], np.float32)
+    vs = np.array([[0.02]], np.float32)
+    c = DeviceCache(B, Hkv, hist + S, D, fp8=True)
+    c.load_canonical(kc, vc, ks, vs)
+    q, k, v = make(78, B, S, Hq, Hkv)
+    got = gpu_prefill(c, q, k, v, hist, write=False)
+    want = oracle_prefill(q, oracle.dequant_fp8(kc, ks), oracle.dequant_fp8(vc, vs), k, v)
+    compare(got, want, "fp8 all codes")
 
 
 @pytest.mark.parametrize("qscale", [4.0e5, 1.0e-3])
