@@ -176,7 +176,8 @@ Status LayerKVCache::decode_step(const void *q, const void *k_new, const void *v
 Status LayerKVCache::prefill(const void *q, const void *new_keys, const void *new_values, void *out, int32_t batch,
                              int32_t seq_len, int32_t hq, int32_t heads, int32_t dim, size_t start_pos, float scale,
                              hs_stream_t stream) {
-    if (quant_type_ != KVQuantType::Int8) return err(HS_ERR_INVALID_ARGUMENT, "prefill attention serves the Int8 format");
+    if (quant_type_ == KVQuantType::None)
+        return err(HS_ERR_INVALID_ARGUMENT, "full-precision storage is not served by this library; use Int8 or Fp8");
     const size_t end_pos = start_pos + (size_t)seq_len;
     if (end_pos > max_seq_len) {
         char buf[200];
@@ -186,8 +187,18 @@ Status LayerKVCache::prefill(const void *q, const void *new_keys, const void *ne
     }
     if (start_pos > seq_pos) return err(HS_ERR_INVALID_ARGUMENT, "start_pos is past the cached tokens");
     if (Status s = ensure_storage(batch, heads, dim); !s.ok()) return s;
-    int rc = hs_prefill_attn_int8(q, new_keys, new_values, (int8_t *)k_codes_, (int8_t *)v_codes_, k_scales_, v_scales_, &layout_,
-                                  (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
+    int rc;
+    if (quant_type_ == KVQuantType::Fp8) {
+        if (start_pos == 0) {  // fresh prompt: calibrate the per-(sequence, head) scales on it, as update() does
+            rc = hs_kv_fp8_calibrate(new_keys, new_values, HS_BF16, k_scales_, v_scales_, batch, seq_len, heads, dim, stream);
+            if (rc != HS_OK) return from_abi(rc);
+        }
+        rc = hs_prefill_attn_fp8(q, new_keys, new_values, (uint8_t *)k_codes_, (uint8_t *)v_codes_, k_scales_, v_scales_,
+                                 &layout_, (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
+    } else {
+        rc = hs_prefill_attn_int8(q, new_keys, new_values, (int8_t *)k_codes_, (int8_t *)v_codes_, k_scales_, v_scales_,
+                                  &layout_, (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
+    }
     if (rc != HS_OK) return from_abi(rc);
     seq_pos = end_pos;
     return {};

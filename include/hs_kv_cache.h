@@ -61,7 +61,8 @@ HS_API int hs_cache_decode_attention(hs_cache *c, const void *q, void *out, int3
 /* cache.update(one token) + the above, one kernel launch. k_new, v_new: [batch, 1, num_kv_heads, head_dim]. */
 HS_API int hs_cache_decode_step(hs_cache *c, const void *q, const void *k_new, const void *v_new, int dtype,
                                 void *out, int32_t num_q_heads, float softmax_scale, hs_stream_t stream);
-/* cache.update(seq_len tokens at start_pos) + causal attention of those tokens (int8 format). */
+/* cache.update(seq_len tokens at start_pos) + causal attention of those tokens (bf16 q / keys / values; an FP8
+ * cache calibrates its scales on the tokens written at start_pos 0, as update does). */
 HS_API int hs_cache_prefill(hs_cache *c, const void *q, const void *new_keys, const void *new_values, void *out,
                             int32_t batch, int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                             int32_t head_dim, int64_t start_pos, float softmax_scale, hs_stream_t stream);
