@@ -122,6 +122,58 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
     }
 }
 
+// The same for many rows of a 16-bit tensor: D/8 lanes own a row, eight consecutive elements each (16-byte loads
+// of the lane's elements, of their partners half a row away and of the sin/cos entries; one 16-byte store), so a
+// wavefront carries 64/(D/8) rows.  Per element the operations and their roundings are those of rope_rotate().
+template <int LPR>
+__global__ __launch_bounds__(256) void rope_apply_rows_kernel(RopeArgs a) {
+#pragma clang fp contract(off)
+    constexpr int kRowsPerWave = 64 / LPR;
+    const int lane = threadIdx.x & 63, sub = lane % LPR;
+    const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * kRowsPerWave + lane / LPR;
+    if (row >= (int64_t)a.B * a.S * a.H) return;
+    const int64_t bs = row / a.H;
+    const int s = (int)(bs % a.S), b = (int)(bs / a.S);
+    const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
+    const int p = pos < 0 ? 0 : (pos >= a.rope_len ? a.rope_len - 1 : pos);
+    const int half = a.D / 2, d0 = sub * 8;
+    const bool upper = d0 >= half;
+    const int j0 = upper ? d0 - half : d0;
+    const uint16_t *xr = (const uint16_t *)a.x + row * a.D;
+    const uint4 own = *(const uint4 *)(xr + d0), oth = *(const uint4 *)(xr + (upper ? d0 - half : d0 + half));
+    const uint4 sn = *(const uint4 *)((const uint16_t *)a.sin_t + (int64_t)p * half + j0);
+    const uint4 cs = *(const uint4 *)((const uint16_t *)a.cos_t + (int64_t)p * half + j0);
+    const uint32_t wo[4] = {own.x, own.y, own.z, own.w}, wp[4] = {oth.x, oth.y, oth.z, oth.w};
+    const uint32_t ws[4] = {sn.x, sn.y, sn.z, sn.w}, wc[4] = {cs.x, cs.y, cs.z, cs.w};
+    uint32_t res[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t r2[2];
+#pragma unroll
+        for (int hsel = 0; hsel < 2; ++hsel) {
+            const auto f = [&](uint32_t w) {
+                const uint16_t h16 = (uint16_t)(hsel ? w >> 16 : w & 0xffffu);
+                if (a.dtype == HS_BF16) return bf16_bits_to_f32(h16);
+                _Float16 t;
+                __builtin_memcpy(&t, &h16, 2);
+                return (float)t;
+            };
+            const float own_cos = round_to_dtype(f(wo[i]) * f(wc[i]), a.dtype);
+            const float other_sin = round_to_dtype(f(wp[i]) * f(ws[i]), a.dtype);
+            const float y = upper ? other_sin + own_cos : own_cos - other_sin;
+            if (a.dtype == HS_BF16) r2[hsel] = f32_to_bf16_bits(y);
+            else {
+                const _Float16 t = (_Float16)y;
+                uint16_t h16;
+                __builtin_memcpy(&h16, &t, 2);
+                r2[hsel] = h16;
+            }
+        }
+        res[i] = r2[0] | (r2[1] << 16);
+    }
+    *(uint4 *)((uint16_t *)a.out + row * a.D + d0) = make_uint4(res[0], res[1], res[2], res[3]);
+}
+
 // scale[b, h] = max_{s, d} |x| / 448.  One workgroup per (b, h, tensor).
 __global__ __launch_bounds__(256) void fp8_calibrate_kernel(const void *k_src, const void *v_src, int dtype,
                                                            float *k_scales, float *v_scales, int B, int S, int Hkv,
@@ -315,6 +367,15 @@ int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *ro
     RopeArgs a;
     a.x = x; a.sin_t = rope_sin; a.cos_t = rope_cos; a.out = out; a.positions = positions; a.start_pos = start_pos;
     a.rope_len = rope_len; a.B = B; a.S = S; a.H = H; a.D = D; a.dtype = dtype;
+    const bool aligned = (((uintptr_t)x | (uintptr_t)out | (uintptr_t)rope_sin | (uintptr_t)rope_cos) & 15) == 0;
+    if (dtype != HS_F32 && aligned) {  // 16-bit tensors: several rows per wavefront
+        const int rows_per_wg = 4 * (64 / (D / 8));
+        dim3 g((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
+        if (D == 64) rope_apply_rows_kernel<8><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else if (D == 128) rope_apply_rows_kernel<16><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else rope_apply_rows_kernel<32><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        return check_launch("rope_apply");
+    }
     dim3 grid((unsigned)((rows + 3) / 4));
     if (D == 64) rope_apply_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(a);
     else if (D == 128) rope_apply_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(a);
