@@ -2,26 +2,30 @@
 //
 // One call serves S new tokens per sequence (a prompt, or one chunk of a chunked prefill).  Query
 // row i sits at absolute position hist_len + i and attends
-//   (1) the hist_len tokens already in the int8 cache, dequantized on the fly, and
+//   (1) the hist_len tokens already in the cache (int8 with token scales, or e4m3fn with head scales),
+//       dequantized on the fly, and
 //   (2) new tokens 0..=i in exact bf16,
 // which is softmax(Q K^T * scale + causal mask) V over [history | this call's K/V].
 //
 // Work split.  A 512-thread workgroup (8 wavefronts, 2 per SIMD) owns 256 (query, head) columns of
-// one kv-head -- with G = Hq/Hkv >= 4: 64 consecutive queries x 4 query heads -- and walks the keys
-// in 32-key steps.  Every step's K and V tile is converted ONCE per workgroup into ready-to-issue
-// MFMA A operands in LDS (16 blocks of 64 lanes x 16 B: K as 2 tiles x 4 k-groups, V^T as 8 row
-// groups) by the eight wavefronts together, double-buffered, one barrier per step; each wavefront
-// then reads the operands with conflict-free ds_read_b128 and uses each one for its two 16-column
-// blocks.  Grid = (query tiles, kv-heads x head groups, sequences).
+// one kv-head -- with G = Hq/Hkv >= 4: 64 consecutive queries x 4 query heads -- and walks the keys,
+// 64 per step over the history and 32 per step over the new tokens.  Every step's K and V tiles are
+// converted ONCE per workgroup into ready-to-issue MFMA A operands in LDS (blocks of 64 lanes x 16 B:
+// per 32 keys K as 2 tiles x 4 k-groups, V^T as 8 row groups) by the eight wavefronts together,
+// double-buffered, one barrier per step; each wavefront then reads the operands with conflict-free
+// ds_read_b128 and uses each one for its two 16-column blocks.
+// Grid = (query tiles, kv-heads x head groups, sequences).
 //
 // Products (both on v_mfma_f32_16x16x32, keys on the M axis, columns on N):
 //   S^T[key, col]  = sum_d K[key, d] Q[col, d]
 //   O^T[d, col]   += sum_key V^T[d, key] P^T[key, col]
-// History part: f16 MFMA.  The eight wavefronts that convert a tile apply the per-token scales while they are at
-// it, so the LDS operands are fp16(code * scale) and the consumers see plain K and V; Q is scaled per column by a
-// power of two into fp16 range.  New-token part: bf16 MFMA straight from the caller's bf16 K/V, V^T built with
-// permutes, P rounded to bf16.  Softmax and accumulation are fp32; the score layout of the first product is the
-// B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16 range (|x| > 65024) saturate.
+// History part: f16 MFMA.  The eight wavefronts that convert a tile apply the scales while they are at it, so
+// the LDS operands are fp16(code * scale) and the consumers see plain K and V.  New-token part: bf16 MFMA
+// straight from the caller's bf16 K/V, V^T built with permutes, P rounded to bf16.  In both parts Q carries
+// the softmax scale and log2(e), the score accumulators start from minus the softmax reference, and the row
+// sums are one more MFMA with a ones operand.  Softmax and accumulation are fp32; the score layout of the first
+// product is the B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16
+// range (|x| > 65024) saturate.
 #include <climits>
 #include <type_traits>
 
