@@ -9,7 +9,7 @@
 //
 // Work split.  A 512-thread workgroup (8 wavefronts, 2 per SIMD) owns 256 (query, head) columns of
 // one kv-head -- with G = Hq/Hkv >= 4: 64 consecutive queries x 4 query heads -- and walks the keys,
-// 64 per step over the history and 32 per step over the new tokens.  Every step's K and V tiles are
+// 64 per step.  Every step's K and V tiles are
 // converted ONCE per workgroup into ready-to-issue MFMA A operands in LDS (blocks of 64 lanes x 16 B:
 // per 32 keys K as 2 tiles x 4 k-groups, V^T as 8 row groups) by the eight wavefronts together,
 // double-buffered, one barrier per step; each wavefront then reads the operands with conflict-free
@@ -35,7 +35,6 @@
 namespace hs {
 
 constexpr int kPD = 128;
-constexpr int kPStep = 32;
 constexpr int kPWaves = 8;
 constexpr int kNB = 2;  // 16-column blocks per wavefront
 constexpr float kPLog2e = 1.4426950408889634f;
@@ -60,50 +59,29 @@ struct alignas(16) StepTile {
 };
 
 struct alignas(16) HistTile {
-    StepTile h[2];  // keys 0..31 and 32..63 of a 64-key history step
+    StepTile h[2];  // keys 0..31 and 32..63 of a 64-key step (history or new tokens)
 };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
 // load, i.e. for the tile prefetch that was issued a moment earlier and is not needed before the next step.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Walk `n` key steps of the new-token phase (the history phase has its own loop, same shape, 64 keys per step).
-// A step of one wavefront is
+// A step of one wavefront (64 keys, as two 32-key tiles) is
 //   scores  : S^T = K Q^T                     -- MFMA, operands from LDS
 //   softmax : P from S, running max and sum   -- VALU only
 //   output  : O^T += V^T P^T                  -- MFMA, operands from LDS
 // with one workgroup barrier per step: while tile s is consumed every wavefront converts its share of tile s+1
-// into the other buffer and starts the global loads of tile s+2.  All LDS operand reads of a step are issued
-// before its first MFMA.
+// into the other buffer and starts the global loads of tile s+2.
 // What was measured on this loop (gfx950, two wavefronts per SIMD): an MFMA 16x16x32 occupies the SIMD's
 // vector issue port for about half of its 16 cycles, plain vector instructions run in its shadow (two per MFMA
 // are free), v_exp_f32 one per MFMA, while v_dot2_f32_f16 stalls the matrix pipe (row sums are therefore an
 // MFMA with a ones operand, not dot products or additions).  Variants that paired the matrix work of one
 // wavefront with the vector work of the other behind a second barrier per step, or that software-pipelined
-// scores(s+1) against softmax(s) inside one wavefront, were correct but not faster than this order.
-template <class Issue, class Commit, class LoadK, class Scores, class Softmax, class LoadV, class Output>
-__device__ __forceinline__ void walk_keys(int n, StepTile *tiles, Issue issue, Commit commit, LoadK load_k, Scores scores,
-                                          Softmax softmax, LoadV load_v, Output output) {
-    issue(0);
-    commit(tiles[0], 0);
-    if (n > 1) issue(1);
-    lds_barrier();
-    for (int s = 0; s < n; ++s) {
-        if (s + 1 < n) commit(tiles[(s + 1) & 1], s + 1);
-        if (s + 2 < n) issue(s + 2);
-        load_k(tiles[s & 1], s);
-        load_v(tiles[s & 1], s);
-        scores(s);
-        softmax(tiles[s & 1], s);
-        output(s);
-        lds_barrier();
-    }
-}
-
+// scores(s+1) against softmax(s) inside one wavefront, were correct but not faster than this order; steps of
+// 64 keys instead of 32 were (the per-step bookkeeping is shared by twice the MFMAs).
 template <bool FP8>  // format of the history: int8 codes with token scales, or e4m3fn codes with head scales
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];
-    StepTile *tiles = (StepTile *)lds;
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];  // two step buffers
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: wavefront-dependent branches stay uniform
     const int li = lane & 15, lq = lane >> 4;
@@ -485,90 +463,112 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             sref[nb] = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
             sinit[nb] = (float4v){-sref[nb], -sref[nb], -sref[nb], -sref[nb]};
         }
-        const int nsteps = wg_qlast / kPStep + 1;
+        // 64 keys per step, as two 32-key tiles in the layout of the history phase.
+        constexpr int kNStep = 64;
+        const int nsteps = wg_qlast / kNStep + 1;
+        HistTile *ntiles = (HistTile *)lds;
         const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
         const int64_t rstride = (int64_t)a.Hkv * kPD;  // elements between consecutive tokens
-        // producers, split as in the history phase: wavefront w copies K operand block w (bf16 rows are
-        // operands as they are); for V a lane takes the d-quad x = lane%32 of two adjacent keys (8 bytes of
-        // each) and stores the four (key, key+1) bf16 pairs of d = 4x + i.
-        const int vx = lane & 31, vkp = 2 * wave + (lane >> 5);
-        const int vkey = 16 * ((vkp & 3) >> 1) + 4 * (vkp >> 2) + 2 * (vkp & 1);
-        const int vdst = ((vx >> 1) + 16 * (vkp >> 2)) * 16 + 4 * (vkp & 3);
-        const int krow = 16 * (wave >> 2) + li, kcol = 32 * lq + 8 * (wave & 3);
-        const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + 4 * vx;  // elements
-        u32x4 rawk = {0u, 0u, 0u, 0u};
-        u32x2 rawv[2] = {{0u, 0u}, {0u, 0u}};
+        // producers, split as in the history phase (bf16 rows are operands as they are): wavefront w copies the
+        // 16-key block u4 = w/2, d-halves jp = w%2 (32 bytes per lane = operand blocks 2jp and 2jp+1); for V a lane
+        // takes the d-octet x = lane%16 of two adjacent keys (16 bytes of each) and stores the eight (key, key+1)
+        // bf16 pairs of d = 8x + bb into block bb.
+        const int vx = lane & 15, vpp = 4 * wave + (lane >> 4);
+        const int vhh = vpp >> 4, vg = (vpp >> 2) & 3, vpe = vpp & 3;
+        const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
+        const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
+        const int ku4 = wave >> 1, kjp = wave & 1;
+        const int krow = 16 * ku4 + li, kcol = 32 * lq + 16 * kjp;
+        const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + 8 * vx;  // elements
+        u32x4 rawk[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+        u32x4 rawv[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
         auto issue = [&](int step) {
-            const int t0 = step * kPStep;
-            if (t0 + kPStep <= S) {  // full step: scalar base + this lane's fixed offsets
+            const int t0 = step * kNStep;
+            const uint16_t *kp, *vp0, *vp1;
+            if (t0 + kNStep <= S) {  // full step: scalar base + this lane's fixed offsets
                 const uint16_t *kb = knb + (int64_t)t0 * rstride, *vb = vnb + (int64_t)t0 * rstride;
-                rawk = *(const u32x4 *)(kb + koff);
-                rawv[0] = *(const u32x2 *)(vb + voff);
-                rawv[1] = *(const u32x2 *)(vb + voff + (uint32_t)rstride);
-            } else {
-                rawk = *(const u32x4 *)(knb + (int64_t)min(t0 + krow, S - 1) * rstride + kcol);
-                rawv[0] = *(const u32x2 *)(vnb + (int64_t)min(t0 + vkey, S - 1) * rstride + 4 * vx);
-                rawv[1] = *(const u32x2 *)(vnb + (int64_t)min(t0 + vkey + 1, S - 1) * rstride + 4 * vx);
+                kp = kb + koff;
+                vp0 = vb + voff;
+                vp1 = vb + voff + (uint32_t)rstride;
+            } else {  // rows past the last token repeat it; the causal mask removes them
+                kp = knb + (int64_t)min(t0 + krow, S - 1) * rstride + kcol;
+                vp0 = vnb + (int64_t)min(t0 + vkey, S - 1) * rstride + 8 * vx;
+                vp1 = vnb + (int64_t)min(t0 + vkey + 1, S - 1) * rstride + 8 * vx;
             }
+            rawk[0] = *(const u32x4 *)kp;
+            rawk[1] = *(const u32x4 *)(kp + 8);
+            rawv[0] = *(const u32x4 *)vp0;
+            rawv[1] = *(const u32x4 *)vp1;
         };
-        auto commit = [&](StepTile &t) {
-            *(u32x4 *)(t.k[wave] + obase) = rawk;
+        auto commit = [&](HistTile &t) {
+            uint8_t *kd = t.h[ku4 >> 1].k[4 * (ku4 & 1) + 2 * kjp] + obase;
+            *(u32x4 *)kd = rawk[0];
+            *(u32x4 *)(kd + 1024) = rawk[1];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *(uint32_t *)(t.v[4 * (vx & 1) + i] + vdst) = pick_halves(rawv[0][i >> 1], rawv[1][i >> 1], i & 1);
+            for (int bb = 0; bb < 8; ++bb)
+                *(uint32_t *)(t.h[vhh].v[bb] + vdst) = pick_halves(rawv[0][bb >> 1], rawv[1][bb >> 1], bb & 1);
         };
-        float4v s[kNB][2];
-        bf16x8 pop[kNB];
-        auto mine = [&](int step) { return wv_active && step * kPStep <= wv_qlast; };  // else all keys are in the future
+        float4v s[kNB][4];
+        bf16x8 pop[kNB][2];
+        // Halves of step `step` that hold a key some query of this wavefront may see (0: the step is skipped).
+        auto halves = [&](int step) {
+            if (!wv_active || step * kNStep > wv_qlast) return 0;
+            return step * kNStep + 32 > wv_qlast ? 1 : 2;
+        };
         bf16x8 kop[8], vop[8], ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
-        auto load_k = [&](const StepTile &t, int step) {
-            if (!mine(step)) return;
+        auto scores = [&](const HistTile &t, int nh) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) kop[i] = *(const bf16x8 *)(t.k[i] + obase);
-        };
-        auto load_v = [&](const StepTile &t, int step) {
-            if (!mine(step)) return;
+            for (int hh = 0; hh < 2; ++hh) {
+                if (hh >= nh) break;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vop[i] = *(const bf16x8 *)(t.v[i] + obase);
-        };
-        auto scores = [&](int step) {
-            if (!mine(step)) return;
+                for (int i = 0; i < 8; ++i) kop[i] = *(const bf16x8 *)(t.h[hh].k[i] + obase);
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+                for (int u = 0; u < 2; ++u) {
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb) s[nb][u] = sinit[nb];
+                    for (int nb = 0; nb < kNB; ++nb) s[nb][2 * hh + u] = sinit[nb];
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                    for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int nb = 0; nb < kNB; ++nb)
-                        s[nb][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[4 * u + j], qop[nb][j], s[nb][u], 0, 0, 0);
+                        for (int nb = 0; nb < kNB; ++nb)
+                            s[nb][2 * hh + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[4 * u + j], qop[nb][j], s[nb][2 * hh + u], 0, 0, 0);
+                }
             }
         };
-        auto softmax = [&](const StepTile &, int step) {
-            if (!mine(step)) return;
-            const int t0 = step * kPStep;
-            const bool diag = t0 + kPStep - 1 > wv_q0;  // some (key, query) pair of this step is in the future
-            float e[kNB][8];
+        auto load_v = [&](const HistTile &t, int hh) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[i] + obase);
+        };
+        auto output = [&](int hh) {
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb)
+#pragma unroll
+                for (int nb = 0; nb < kNB; ++nb)
+                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb][hh], acc[nb][bb], 0, 0, 0);
+        };
+        auto softmax = [&](int step, int nh) {
+            const int t0 = step * kNStep;
+            const bool diag = t0 + kNStep - 1 > wv_q0;  // some (key, query) pair of this step is in the future
+            float e[kNB][16];
             int over = force;
 #pragma unroll
             for (int nb = 0; nb < kNB; ++nb) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u)
+                for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) e[nb][4 * u + r] = s[nb][u][r];
+                    for (int r = 0; r < 4; ++r) e[nb][4 * u4 + r] = (u4 < 2 * nh) ? s[nb][u4][r] : -INFINITY;
                 if (diag) {
-                    const int qrel = min(qi[nb], S - 1) - t0 - 4 * lq;  // key offsets 16u + r beyond this are in the future
+                    const int qrel = min(qi[nb], S - 1) - t0 - 4 * lq;  // key offsets 16u4 + r beyond this are in the future
 #pragma unroll
-                    for (int u = 0; u < 2; ++u)
+                    for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            if (16 * u + r > qrel) e[nb][4 * u + r] = -INFINITY;
+                            if (16 * u4 + r > qrel) e[nb][4 * u4 + r] = -INFINITY;
                 }
 #pragma unroll
-                for (int i = 0; i < 8; ++i) over = max(over, __float_as_int(e[nb][i]));
+                for (int i = 0; i < 16; ++i) over = max(over, __float_as_int(e[nb][i]));
             }
             if (__builtin_amdgcn_ballot_w64(over > __float_as_int(kPShift)) != 0) {
                 force = INT_MIN;
@@ -577,7 +577,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 for (int nb = 0; nb < kNB; ++nb) {
                     float m = e[nb][0];
 #pragma unroll
-                    for (int i = 1; i < 8; ++i) m = fmaxf(m, e[nb][i]);
+                    for (int i = 1; i < 16; ++i) m = fmaxf(m, e[nb][i]);
                     mx[nb] = quad_max(m) + sref[nb];
                 }
                 raise_max(mx);
@@ -586,29 +586,44 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                     const float nref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
                     const float d = nref - sref[nb];
 #pragma unroll
-                    for (int i = 0; i < 8; ++i) e[nb][i] -= d;
+                    for (int i = 0; i < 16; ++i) e[nb][i] -= d;
                     sref[nb] = nref;
                     sinit[nb] = (float4v){-nref, -nref, -nref, -nref};
                 }
             }
 #pragma unroll
-            for (int nb = 0; nb < kNB; ++nb) {
-                float p[8];
+            for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
-                for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_exp2f(e[nb][i]);
-                pop[nb] = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
-                l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pop[nb], l_run[nb], 0, 0, 0);
+                for (int hh = 0; hh < 2; ++hh) {
+                    if (hh >= nh) break;
+                    float p[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) p[i] = __builtin_amdgcn_exp2f(e[nb][8 * hh + i]);
+                    pop[nb][hh] = pack_bf16x8(pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3]), pack_bf16x2(p[4], p[5]), pack_bf16x2(p[6], p[7]));
+                    l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pop[nb][hh], l_run[nb], 0, 0, 0);
+                }
+        };
+        issue(0);
+        commit(ntiles[0]);
+        if (nsteps > 1) issue(1);
+        lds_barrier();
+        for (int st = 0; st < nsteps; ++st) {
+            if (st + 1 < nsteps) commit(ntiles[(st + 1) & 1]);
+            if (st + 2 < nsteps) issue(st + 2);
+            const int nh = halves(st);
+            if (nh > 0) {
+                const HistTile &t = ntiles[st & 1];
+                scores(t, nh);
+                load_v(t, 0);
+                softmax(st, nh);
+                output(0);
+                if (nh > 1) {
+                    load_v(t, 1);
+                    output(1);
+                }
             }
-        };
-        auto output = [&](int step) {
-            if (!mine(step)) return;
-#pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
-#pragma unroll
-                for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb], acc[nb][bb], 0, 0, 0);
-        };
-        walk_keys(nsteps, tiles, issue, [&](StepTile &t, int) { commit(t); }, load_k, scores, softmax, load_v, output);
+            lds_barrier();
+        }
     }
 
     // =============================== normalise and store ===============================
