@@ -158,6 +158,48 @@ def test_config3_full_size_chunked_prefill():
     assert np.array_equal(kc[1, 5].cpu().numpy(), wk) and np.array_equal(ks[1, 5, :T].cpu().numpy(), wks)
 
 
+def test_config3_shape_with_fp8_history():
+    """The same shape over an FP8 e4m3fn cache (per-head scales calibrated on the first chunk, N(0, 0.5^2) sources as
+    in the FP8 decode configuration): sampled query rows against the oracle over [dequantized fp8 cache of earlier
+    chunks | own bf16 K/V]; the finished cache holds the oracle's codes."""
+    B, T, C, Hq, Hkv, D = 4, 4096, 512, 32, 8, 128
+    g = gen(wl.SEED + 7)
+    q = source(g, (B, T, Hq, D))
+    k, v = source(g, (B, T, Hkv, D), 0.5), source(g, (B, T, Hkv, D), 0.5)
+    lay = hb.contiguous_layout(Hkv, T, D)
+    kc = torch.zeros(B, Hkv, T, D, dtype=torch.uint8, device=DEV)
+    vc = torch.zeros_like(kc)
+    ks = torch.zeros(B, Hkv, dtype=torch.float32, device=DEV)
+    vs = torch.zeros_like(ks)
+    hb.kv_fp8_calibrate(k[:, :C].contiguous(), v[:, :C].contiguous(), ks, vs)
+    outs = []
+    for i in range(0, T, C):
+        o = torch.empty(B, C, Hq, D, dtype=torch.bfloat16, device=DEV)
+        hb.prefill_attn(q[:, i:i + C].contiguous(), k[:, i:i + C].contiguous(), v[:, i:i + C].contiguous(), kc, vc, ks, vs,
+                        lay, i, o, 1.0 / np.sqrt(D), True, fp8=True)
+        outs.append(o)
+    torch.cuda.synchronize()
+    out = torch.cat(outs, 1)
+    assert torch.isfinite(out.float()).all()
+    ksn, vsn = ks.cpu().numpy(), vs.cpu().numpy()
+    r = wl.philox(37)
+    for _ in range(6):
+        b, h, pos = int(r.integers(B)), int(r.integers(Hkv)), int(r.integers(T))
+        c0 = pos // C * C
+        kh = oracle.dequant_fp8(kc[b, h, :c0].cpu().numpy()[None, :, None], ksn[b:b + 1, h:h + 1])[0, :, 0]
+        vh = oracle.dequant_fp8(vc[b, h, :c0].cpu().numpy()[None, :, None], vsn[b:b + 1, h:h + 1])[0, :, 0]
+        kd = np.concatenate([kh, k[b, c0:pos + 1, h].float().cpu().numpy()])
+        vd = np.concatenate([vh, v[b, c0:pos + 1, h].float().cpu().numpy()])
+        qb = q[b, pos, 4 * h:4 * h + 4].float().cpu().numpy()[None]
+        want = oracle.decode_attn(qb, kd[None, :, None], vd[None, :, None], None, None, oracle.FMT_DENSE,
+                                  np.array([pos + 1], np.int32), 1.0 / np.sqrt(D))[0]
+        d = np.abs(out[b, pos, 4 * h:4 * h + 4].float().cpu().numpy() - want)
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, pos, d.max(), d.mean())
+    # the finished cache holds the oracle's codes for a sampled (sequence, head)
+    wk = oracle.quant_fp8(k[2, :, 3].float().cpu().numpy()[None, :, None], ksn[2:3, 3:4])[0, :, 0]
+    assert np.array_equal(kc[2, 3].cpu().numpy(), wk)
+
+
 def test_config5_full_size_deltanet():
     """Decode at B = 64 (whole batch against the oracle) and prefill at B = 4 x 4096 (two sampled heads against
     the oracle, and chunked calls with carried state against the single call)."""
