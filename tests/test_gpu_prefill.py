@@ -143,6 +143,36 @@ def test_fp8_history_with_subnormal_codes_and_every_code_value():
     compare(got, want, "fp8 all codes")
 
 
+def test_paged_fp8_history_matches_contiguous():
+    """FP8 history in 64-token blocks scattered through one pool: the same bits as over the contiguous cache."""
+    B, Hq, Hkv, D, hist, S, BT = 2, 8, 2, 128, 150, 70, 64
+    qh, kh, vh = make(110, B, hist, Hq, Hkv, sigma=0.5)
+    q, k, v = make(111, B, S, Hq, Hkv, sigma=0.5)
+    c = DeviceCache(B, Hkv, hist + S, D, fp8=True)
+    hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+    hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+    c.write(hk, hv, None, 0)
+    want = gpu_prefill(c, q, k, v, hist)
+    nblk = (hist + S + BT - 1) // BT
+    ids = wl.philox(112).permutation(2 * B * nblk + 3).astype(np.int32)
+    kt, vt = ids[:B * nblk].reshape(B, nblk), ids[B * nblk:2 * B * nblk].reshape(B, nblk)
+    pool_c = torch.zeros(len(ids), Hkv, BT, D, dtype=torch.uint8, device=DEV)
+    k_tab, v_tab = torch.from_numpy(kt).to(DEV), torch.from_numpy(vt).to(DEV)
+    lay = hb.paged_layout(Hkv, BT, D, k_tab, v_tab)
+    hb.kv_quantize_fp8(hk, hv, pool_c, pool_c, c.k_scales, c.v_scales, lay, None, 0)
+    qt, knew, vnew = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
+    out = torch.empty(B, S, Hq, D, dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(qt, knew, vnew, pool_c, pool_c, c.k_scales, c.v_scales, lay, hist, out, 1.0 / np.sqrt(D), True, fp8=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    dense = torch.empty(B, hist + S, Hkv, D, dtype=torch.float32, device=DEV)
+    ref = torch.empty_like(dense)
+    hb.kv_dequantize(pool_c, c.k_scales, True, lay, 0, dense)
+    hb.kv_dequantize(c.k_codes, c.k_scales, True, c.layout, 0, ref)
+    torch.cuda.synchronize()
+    assert torch.equal(dense, ref)
+
+
 @pytest.mark.parametrize("qscale", [4.0e5, 1.0e-3])
 def test_query_magnitudes_outside_the_fp16_range(qscale):
     """|q| * scale * log2(e) above 2^15 takes the kernel's rescaled-operand path (attention is one-hot there);
