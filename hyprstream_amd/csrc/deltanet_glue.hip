@@ -61,6 +61,89 @@ __global__ __launch_bounds__(256) void deltanet_conv_kernel(PrepArgs a) {
     }
 }
 
+// SiLU through v_exp_f32 and v_rcp_f32 (a few fp32 ulp; the result is rounded to bf16 right after).
+__device__ __forceinline__ float silu_fast(float x) {
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+
+// The same for channel counts that are multiples of 8: a thread owns 8 adjacent channels (16-byte accesses) and
+// kConvFrames frames, and issues all its loads before it computes, so the kernel runs at memory speed instead of
+// at the latency of one 2-byte load per frame.  thread = (sequence, frame block, channel octet).
+constexpr int kConvFrames = 16;
+__global__ __launch_bounds__(256) void deltanet_conv8_kernel(PrepArgs a) {
+#pragma clang fp contract(off)
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (c >= a.C) return;
+    const int t0 = blockIdx.y * kConvFrames, b = blockIdx.z;
+    const int nt = min(a.S - t0, kConvFrames);
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    u32x4 fr[kConvFrames + 3];  // frames t0-3 .. t0+kConvFrames-1, 8 channels each
+#pragma unroll
+    for (int i = 0; i < kConvFrames + 3; ++i) {
+        const int t = t0 - 3 + i;
+        fr[i] = (u32x4){0u, 0u, 0u, 0u};
+        if (t >= 0) {
+            if (i < nt + 3) fr[i] = *(const u32x4 *)(a.x + ((int64_t)b * a.S + t) * a.C + c);
+        } else if (a.state_in) {  // carried state [B, C, 3]: frame -3 + j of channel c + e is element 3*e + j
+            const uint16_t *sp = a.state_in + ((int64_t)b * a.C + c) * 3 + (3 + t);
+            uint32_t h[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) h[e] = sp[3 * e];
+            fr[i] = (u32x4){h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+        }
+    }
+    u32x4 wq[4];  // w[c + e][tap] = element 4*e + tap of these 64 bytes
+#pragma unroll
+    for (int i = 0; i < 4; ++i) wq[i] = *(const u32x4 *)(a.w + (int64_t)c * kConvK + 8 * i);
+    auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
+    auto hi = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
+    float wt[8][kConvK];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const uint32_t w01 = wq[e >> 1][2 * (e & 1)], w23 = wq[e >> 1][2 * (e & 1) + 1];
+        wt[e][0] = lo(w01); wt[e][1] = hi(w01); wt[e][2] = lo(w23); wt[e][3] = hi(w23);
+    }
+    uint16_t *dst;
+    int64_t stride, off;
+    if (c < a.key_dim) { dst = a.q; stride = a.key_dim; off = c; }
+    else if (c < 2 * a.key_dim) { dst = a.k; stride = a.key_dim; off = c - a.key_dim; }
+    else { dst = a.v; stride = a.val_dim; off = c - 2 * a.key_dim; }
+    auto chan = [&](const u32x4 &f, int e) { return (e & 1) ? hi(f[e >> 1]) : lo(f[e >> 1]); };
+#pragma unroll
+    for (int i = 0; i < kConvFrames; ++i) {
+        if (i >= nt) continue;
+        float y[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float acc = wt[e][0] * chan(fr[i], e);
+            acc += wt[e][1] * chan(fr[i + 1], e);
+            acc += wt[e][2] * chan(fr[i + 2], e);
+            acc += wt[e][3] * chan(fr[i + 3], e);
+            y[e] = silu_fast((float)(__bf16)acc);  // the conv output is a bf16 tensor before the SiLU
+        }
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        uint32_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {  // hardware round-to-nearest-even conversion, two values per instruction
+            const bf16x2 p = {(__bf16)y[2 * e], (__bf16)y[2 * e + 1]};
+            o[e] = __builtin_bit_cast(uint32_t, p);
+        }
+        *(u32x4 *)(dst + ((int64_t)b * a.S + t0 + i) * stride + off) = (u32x4){o[0], o[1], o[2], o[3]};
+    }
+    if (t0 + nt == a.S) {  // this thread saw the end of the sequence: the last three frames are the new state
+        uint16_t *so = a.state_out + ((int64_t)b * a.C + c) * 3;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) {
+            u32x4 f = fr[0];
+#pragma unroll
+            for (int i = 0; i < kConvFrames + 3; ++i)
+                if (i == nt + j) f = fr[i];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) so[3 * e + j] = (uint16_t)((e & 1) ? f[e >> 1] >> 16 : f[e >> 1] & 0xffffu);
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void deltanet_gates_kernel(const uint16_t *a_in, const uint16_t *b_in, const float *neg_a_exp,
                                                             const float *dt_bias, float *g, float *beta, int64_t n, int nv) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -96,6 +179,40 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_kernel(const float *x, cons
     }
 }
 
+// The same with D/8 lanes per row (eight elements each: 16-byte accesses, 64/(D/8) rows per wavefront).
+template <int LPR>
+__global__ __launch_bounds__(256) void gated_rmsnorm_rows_kernel(const float *x, const uint16_t *z, const float *w, float eps,
+                                                                uint16_t *out, int64_t rows) {
+    constexpr int D = 8 * LPR;
+    const int lane = threadIdx.x & 63, sub = lane % LPR;
+    int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / LPR) + lane / LPR;
+    const bool live = row < rows;  // lanes past the end still take part in the shuffles
+    if (!live) row = rows - 1;
+    const int64_t e0 = row * D + sub * 8;
+    const float4 xa = *(const float4 *)(x + e0), xb = *(const float4 *)(x + e0 + 4);
+    const uint4 zz = *(const uint4 *)(z + e0);
+    const float4 wa = *(const float4 *)(w + sub * 8), wb = *(const float4 *)(w + sub * 8 + 4);
+    const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+    const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+    const uint32_t zw[4] = {zz.x, zz.y, zz.z, zz.w};
+    float ss = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += xv[e] * xv[e];
+#pragma unroll
+    for (int o = 1; o < LPR; o <<= 1) ss += __shfl_xor(ss, o, 64);
+    const float rrms = 1.0f / sqrtf(ss / (float)D + eps);
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    uint32_t o4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float z0 = __uint_as_float(zw[i] << 16), z1 = __uint_as_float(zw[i] & 0xffff0000u);
+        const bf16x2 p = {(__bf16)(xv[2 * i] * rrms * wv[2 * i] * silu_fast(z0)),
+                          (__bf16)(xv[2 * i + 1] * rrms * wv[2 * i + 1] * silu_fast(z1))};
+        o4[i] = __builtin_bit_cast(uint32_t, p);
+    }
+    if (live) *(uint4 *)(out + e0) = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+}
+
 }  // namespace hs
 
 extern "C" {
@@ -118,8 +235,15 @@ int hs_deltanet_prepare(const void *mixed_qkv, const void *conv_weight, const vo
     a.q = (uint16_t *)q; a.k = (uint16_t *)k; a.v = (uint16_t *)v;
     a.B = B; a.S = S; a.key_dim = nk * dk; a.val_dim = nv * dv; a.C = 2 * a.key_dim + a.val_dim;
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid((unsigned)((a.C + 255) / 256), (unsigned)((S + kConvTimeBlock - 1) / kConvTimeBlock), (unsigned)B);
-    deltanet_conv_kernel<<<grid, 256, 0, st>>>(a);
+    const bool wide = (a.key_dim % 8) == 0 && (a.val_dim % 8) == 0 &&
+                      (((uintptr_t)mixed_qkv | (uintptr_t)conv_weight | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) == 0;
+    if (wide) {
+        dim3 grid((unsigned)((a.C / 8 + 255) / 256), (unsigned)((S + kConvFrames - 1) / kConvFrames), (unsigned)B);
+        deltanet_conv8_kernel<<<grid, 256, 0, st>>>(a);
+    } else {
+        dim3 grid((unsigned)((a.C + 255) / 256), (unsigned)((S + kConvTimeBlock - 1) / kConvTimeBlock), (unsigned)B);
+        deltanet_conv_kernel<<<grid, 256, 0, st>>>(a);
+    }
     if (int rc = check_launch("deltanet_conv")) return rc;
     const int64_t n = (int64_t)B * S * nv;
     deltanet_gates_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const uint16_t *)a_in, (const uint16_t *)b_in, neg_a_exp,
@@ -133,8 +257,16 @@ int hs_deltanet_gated_norm(const float *x, const void *z, const float *weight, f
     if (rows > 0 && (!x || !z || !weight || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (rows < 0 || (D != 64 && D != 128 && D != 256)) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape rows=%lld D=%d", (long long)rows, D);
     if (rows == 0) return HS_OK;
-    const unsigned blocks = (unsigned)((rows + 3) / 4);
     hipStream_t st = (hipStream_t)stream;
+    if ((((uintptr_t)x | (uintptr_t)z | (uintptr_t)weight | (uintptr_t)out) & 15) == 0) {  // several rows per wavefront
+        const int rows_per_wg = 4 * (64 / (D / 8));
+        const unsigned g = (unsigned)((rows + rows_per_wg - 1) / rows_per_wg);
+        if (D == 64) gated_rmsnorm_rows_kernel<8><<<g, 256, 0, st>>>(x, (const uint16_t *)z, weight, eps, (uint16_t *)out, rows);
+        else if (D == 128) gated_rmsnorm_rows_kernel<16><<<g, 256, 0, st>>>(x, (const uint16_t *)z, weight, eps, (uint16_t *)out, rows);
+        else gated_rmsnorm_rows_kernel<32><<<g, 256, 0, st>>>(x, (const uint16_t *)z, weight, eps, (uint16_t *)out, rows);
+        return check_launch("gated_rmsnorm");
+    }
+    const unsigned blocks = (unsigned)((rows + 3) / 4);
     if (D == 64) gated_rmsnorm_kernel<1><<<blocks, 256, 0, st>>>(x, (const uint16_t *)z, weight, eps, (uint16_t *)out, rows);
     else if (D == 128) gated_rmsnorm_kernel<2><<<blocks, 256, 0, st>>>(x, (const uint16_t *)z, weight, eps, (uint16_t *)out, rows);
     else gated_rmsnorm_kernel<4><<<blocks, 256, 0, st>>>(x, (const uint16_t *)z, weight, eps, (uint16_t *)out, rows);
