@@ -253,6 +253,59 @@ __global__ __launch_bounds__(256) void kv_dequantize_kernel(DequantArgs a) {
     }
 }
 
+// The same with D/8 lanes per row: 8-byte code loads, 16- or 32-byte stores, 64/(D/8) rows per wavefront.
+template <int LPR>
+__global__ __launch_bounds__(256) void kv_dequantize_rows_kernel(DequantArgs a) {
+    const int lane = threadIdx.x & 63, sub = lane % LPR;
+    const int64_t row = ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / LPR) + lane / LPR;
+    if (row >= (int64_t)a.B * a.T * a.Hkv) return;
+    const int h = (int)(row % a.Hkv);
+    const int64_t bt = row / a.Hkv;
+    const int t = (int)(bt % a.T);
+    const int b = (int)(bt / a.T);
+    int64_t unit;
+    int slot;
+    float v[8];
+    if (resolve(a.addr, b, t, unit, slot)) {
+        const uint8_t *src = (const uint8_t *)a.codes + unit * a.addr.code_stride_seq +
+                             (int64_t)h * a.addr.code_stride_head + (int64_t)slot * a.D + sub * 8;
+        const float sc = a.fp8 ? a.scales[(int64_t)b * a.Hkv + h]
+                               : a.scales[unit * a.addr.scale_stride_seq + (int64_t)h * a.addr.scale_stride_head + slot];
+        const uint2 c8 = *(const uint2 *)src;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const uint32_t byte = ((e < 4 ? c8.x : c8.y) >> (8 * (e & 3))) & 0xffu;
+            v[e] = sc * (a.fp8 ? e4m3fn_bits_to_f32(byte) : (float)(int8_t)byte);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+    }
+    const int64_t o = row * a.D + sub * 8;
+    if (a.out_dtype == HS_F32) {
+        *(float4 *)((float *)a.out + o) = make_float4(v[0], v[1], v[2], v[3]);
+        *(float4 *)((float *)a.out + o + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            uint32_t h2[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                if (a.out_dtype == HS_BF16) h2[j] = f32_to_bf16_bits(v[2 * i + j]);
+                else {
+                    const _Float16 f = (_Float16)v[2 * i + j];
+                    uint16_t u;
+                    __builtin_memcpy(&u, &f, 2);
+                    h2[j] = u;
+                }
+            }
+            w[i] = h2[0] | (h2[1] << 16);
+        }
+        *(uint4 *)((uint16_t *)a.out + o) = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+}
+
 // ------------------------------------------------------------------ host launchers
 
 static int check_common(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales) {
@@ -414,6 +467,14 @@ int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8, const 
     hs::DequantArgs a;
     a.codes = codes; a.scales = scales; a.addr = hs::make_addr(*layout, which_table ? 1 : 0);
     a.out = out; a.B = B; a.T = T; a.Hkv = Hkv; a.D = D; a.out_dtype = out_dtype; a.fp8 = fmt_fp8 ? 1 : 0;
+    if ((((uintptr_t)codes) & 7) == 0 && (((uintptr_t)out) & 15) == 0 && (layout->code_stride_seq & 7) == 0) {
+        const int rows_per_wg = 4 * (64 / (D / 8));
+        dim3 g((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
+        if (D == 64) hs::kv_dequantize_rows_kernel<8><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else if (D == 128) hs::kv_dequantize_rows_kernel<16><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else hs::kv_dequantize_rows_kernel<32><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        return hs::check_launch("kv_dequantize");
+    }
     dim3 grid((unsigned)((rows + 3) / 4));
     if (D == 64) hs::kv_dequantize_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(a);
     else if (D == 128) hs::kv_dequantize_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(a);
