@@ -184,6 +184,27 @@ Status PagedLayerKVCache::update(const void *new_keys, const void *new_values, i
     return {};
 }
 
+Status PagedLayerKVCache::prefill(const void *q, const void *new_keys, const void *new_values, void *out, int32_t seq_len,
+                                  int32_t hq, size_t start_pos, float scale, hs_stream_t stream) {
+    if (seq_len < 0) return err(HS_ERR_INVALID_ARGUMENT, "negative seq_len");
+    const size_t end_pos = start_pos + (size_t)seq_len;
+    if (end_pos > max_seq_len) return overflow(seq_len, start_pos, max_seq_len);
+    if (start_pos > seq_pos) return err(HS_ERR_INVALID_ARGUMENT, "start_pos is past the cached tokens");
+    if (Status s = reserve(end_pos); !s.ok()) return s;
+    if (seq_len > 0) {
+        if (Status s = pool_->ensure_device(); !s.ok()) return s;
+        if (Status s = sync_table(); !s.ok()) return s;
+        const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
+        const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
+        int rc = hs_prefill_attn_int8(q, new_keys, new_values, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
+                                      (int32_t)start_pos, out, 1, seq_len, hq, pool_->num_kv_heads(), pool_->head_dim(), scale, 1,
+                                      stream);
+        if (rc != HS_OK) return from_abi(rc);
+    }
+    seq_pos = end_pos;
+    return {};
+}
+
 Status PagedLayerKVCache::get_dense(void *keys_out, void *values_out, int dtype, hs_stream_t stream) {
     if (seq_pos == 0) return err(HS_ERR_INVALID_ARGUMENT, "Cache is empty");
     if (Status s = sync_table(); !s.ok()) return s;

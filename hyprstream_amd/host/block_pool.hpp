@@ -91,6 +91,10 @@ class PagedLayerKVCache {
                   hs_stream_t stream = nullptr);
     Status get_dense(void *keys_out, void *values_out, int dtype, hs_stream_t stream = nullptr);
     Status decode_attention(const void *q, void *out, int32_t num_q_heads, float softmax_scale, hs_stream_t stream = nullptr);
+    // update(seq_len bf16 tokens at start_pos) + causal attention of those tokens over [cached history | themselves];
+    // q, out: bf16 [1, seq_len, num_q_heads, head_dim].  Blocks are taken as in update().
+    Status prefill(const void *q, const void *new_keys, const void *new_values, void *out, int32_t seq_len, int32_t num_q_heads,
+                   size_t start_pos, float softmax_scale, hs_stream_t stream = nullptr);
     void clear();
     void truncate_to(size_t pos);  // frees the blocks beyond the last needed one (kv_cache.rs:1725-1748)
     size_t num_blocks() const { return key_blocks_.size(); }

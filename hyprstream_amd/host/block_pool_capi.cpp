@@ -92,6 +92,11 @@ int hs_paged_cache_decode_attention(hs_paged_cache *c, const void *q, void *out,
     if (!c) return HS_ERR_INVALID_ARGUMENT;
     return c->done(c->cache.decode_attention(q, out, hq, scale, stream));
 }
+int hs_paged_cache_prefill(hs_paged_cache *c, const void *q, const void *new_keys, const void *new_values, void *out,
+                           int32_t seq_len, int32_t hq, int64_t start_pos, float scale, hs_stream_t stream) {
+    if (!c || start_pos < 0) return HS_ERR_INVALID_ARGUMENT;
+    return c->done(c->cache.prefill(q, new_keys, new_values, out, seq_len, hq, (size_t)start_pos, scale, stream));
+}
 void hs_paged_cache_clear(hs_paged_cache *c) { if (c) c->cache.clear(); }
 void hs_paged_cache_truncate_to(hs_paged_cache *c, int64_t pos) { if (c && pos >= 0) c->cache.truncate_to((size_t)pos); }
 int64_t hs_paged_cache_seq_pos(const hs_paged_cache *c) { return c ? (int64_t)c->cache.seq_pos : 0; }

@@ -16,7 +16,7 @@ EXPORTS = [
     "hs_cache_create", "hs_cache_destroy", "hs_cache_last_error", "hs_cache_update", "hs_cache_get_dense",
     "hs_cache_get_view", "hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_clear", "hs_cache_truncate_to",
     "hs_cache_is_initialized", "hs_cache_memory_usage", "hs_cache_quant_type", "hs_cache_decode_attention",
-    "hs_cache_decode_step", "hs_cache_prefill", "hs_kv_quant_canonical_str",
+    "hs_cache_decode_step", "hs_cache_prefill", "hs_paged_cache_prefill", "hs_kv_quant_canonical_str",
     "hs_pool_create", "hs_pool_destroy", "hs_pool_last_error", "hs_pool_allocate", "hs_pool_free", "hs_pool_owner_of",
     "hs_pool_used_blocks", "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory",
     "hs_paged_cache_create", "hs_paged_cache_destroy", "hs_paged_cache_last_error", "hs_paged_cache_update",
@@ -271,6 +271,15 @@ class PagedLayerKVCache:
         out = torch.empty_like(q)
         self._check(lib().hs_paged_cache_decode_attention(self._h, hb._ptr(q), hb._ptr(out), q.shape[1],
                                                           ctypes.c_float(softmax_scale), hb._stream()))
+        return out
+
+    def prefill(self, q, new_keys, new_values, start_pos, softmax_scale):
+        import torch
+        _, S, Hq, _ = q.shape
+        k, v = new_keys.contiguous(), new_values.contiguous()
+        out = torch.empty_like(q)
+        self._check(lib().hs_paged_cache_prefill(self._h, hb._ptr(q.contiguous()), hb._ptr(k), hb._ptr(v), hb._ptr(out), S, Hq,
+                                                 ctypes.c_int64(start_pos), ctypes.c_float(softmax_scale), hb._stream()))
         return out
 
     def clear(self):

@@ -104,6 +104,11 @@ HS_API int hs_paged_cache_update(hs_paged_cache *c, const void *new_keys, const 
 HS_API int hs_paged_cache_get_dense(hs_paged_cache *c, void *keys_out, void *values_out, int dtype, hs_stream_t stream);
 HS_API int hs_paged_cache_decode_attention(hs_paged_cache *c, const void *q, void *out, int32_t num_q_heads,
                                            float softmax_scale, hs_stream_t stream);
+/* update(seq_len bf16 tokens at start_pos) + causal attention of those tokens over [cached history | themselves];
+ * q, out: bf16 [1, seq_len, num_q_heads, head_dim]; new_keys, new_values: bf16 [1, seq_len, num_kv_heads, head_dim]. */
+HS_API int hs_paged_cache_prefill(hs_paged_cache *c, const void *q, const void *new_keys, const void *new_values, void *out,
+                                  int32_t seq_len, int32_t num_q_heads, int64_t start_pos, float softmax_scale,
+                                  hs_stream_t stream);
 HS_API void hs_paged_cache_clear(hs_paged_cache *c);
 HS_API void hs_paged_cache_truncate_to(hs_paged_cache *c, int64_t pos);
 HS_API int64_t hs_paged_cache_seq_pos(const hs_paged_cache *c);

@@ -66,6 +66,35 @@ def test_update_across_block_boundaries_and_truncate():
     assert np.array_equal(gk.cpu().numpy(), _dense_reference(k))
 
 
+def test_chunked_prefill_through_a_paged_cache():
+    """Two prompt chunks that cross block boundaries: attention of each chunk over [cached blocks | itself] against
+    the oracle, and the blocks end up holding what update() would have written."""
+    r = wl.philox(905)
+    Hq, Hkv, D, C = 8, 2, 128, 300
+    pool = kc.BlockPool(16, Hkv, D)
+    cache = kc.PagedLayerKVCache(2048, pool, 7)
+    q, k, v = _rand(r, 1, 2 * C, Hq, D), _rand(r, 1, 2 * C, Hkv, D), _rand(r, 1, 2 * C, Hkv, D)
+    o0 = cache.prefill(q[:, :C], k[:, :C], v[:, :C], 0, 1 / np.sqrt(D))
+    assert cache.seq_pos == C and cache.num_blocks == 2
+    o1 = cache.prefill(q[:, C:], k[:, C:], v[:, C:], C, 1 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert cache.seq_pos == 2 * C and cache.num_blocks == 3
+    kd, vd = cache.get(torch.float32)
+    assert np.array_equal(kd.cpu().numpy(), _dense_reference(k)) and np.array_equal(vd.cpu().numpy(), _dense_reference(v))
+    kn, vn = k.float().cpu().numpy(), v.float().cpu().numpy()
+    want0 = oracle.prefill_attn(q[:, :C].float().cpu().numpy(), kn[:, :C], vn[:, :C], None, None, oracle.FMT_DENSE,
+                                np.array([C], np.int32), 1 / np.sqrt(D))
+    k1 = np.concatenate([kd[:, :C].cpu().numpy(), kn[:, C:]], 1)
+    v1 = np.concatenate([vd[:, :C].cpu().numpy(), vn[:, C:]], 1)
+    want1 = oracle.prefill_attn(q[:, C:].float().cpu().numpy(), k1, v1, None, None, oracle.FMT_DENSE,
+                                np.array([2 * C], np.int32), 1 / np.sqrt(D))
+    for got, want in ((o0, want0), (o1, want1)):
+        d = np.abs(got.float().cpu().numpy() - want)
+        assert d.max() < 2e-2 and d.mean() < 2e-3
+    with pytest.raises(kc.CacheError, match="past the cached tokens"):
+        cache.prefill(q[:, :C], k[:, :C], v[:, :C], 1000, 1 / np.sqrt(D))
+
+
 def test_paged_cache_frees_blocks_on_drop():
     r = wl.philox(902)
     pool = kc.BlockPool(8, 2, 64)
