@@ -90,28 +90,35 @@ def cpu_baseline(torch, name, caches, q, lens, Hq, fp8, seconds_budget=20.0):
     }, out
 
 
-def bench_prefill(args, torch, hb, wl):
+def bench_prefill(args, torch, hb, wl, C=512, fp8=False):
     """Config 3: chunked causal prefill, B=4 x 4096 tokens in 512-token chunks, Hq 32 / Hkv 8, D 128.
-    One step = all eight chunk calls of one layer (attention + quantize-on-write of every chunk)."""
+    One step = all eight chunk calls of one layer (attention + quantize-on-write of every chunk).
+    Variants: C = 4096 (the whole prompt in one call), fp8 = an e4m3fn cache with per-head scales."""
     dev = "cuda:0"
-    B, T, C, Hq, Hkv, D = 4, 4096, 512, 32, 8, 128
+    B, T, Hq, Hkv, D = 4, 4096, 32, 8, 128
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)
+    sigma = 0.5 if fp8 else 1.0
     q = torch.randn(B, T, Hq, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
-    k = torch.randn(B, T, Hkv, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
-    v = torch.randn(B, T, Hkv, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+    k = (sigma * torch.randn(B, T, Hkv, D, generator=gen, device=dev, dtype=torch.float32)).to(torch.bfloat16)
+    v = (sigma * torch.randn(B, T, Hkv, D, generator=gen, device=dev, dtype=torch.float32)).to(torch.bfloat16)
     chunks = [(q[:, i:i + C].contiguous(), k[:, i:i + C].contiguous(), v[:, i:i + C].contiguous()) for i in range(0, T, C)]
     lay = hb.contiguous_layout(Hkv, T, D)
-    kc = torch.zeros(B, Hkv, T, D, dtype=torch.int8, device=dev)
+    kc = torch.zeros(B, Hkv, T, D, dtype=torch.uint8 if fp8 else torch.int8, device=dev)
     vc = torch.zeros_like(kc)
-    ks = torch.zeros(B, Hkv, lay.scale_stride_head, dtype=torch.float32, device=dev)
-    vs = torch.zeros_like(ks)
+    if fp8:
+        ks = torch.zeros(B, Hkv, dtype=torch.float32, device=dev)
+        vs = torch.zeros_like(ks)
+        hb.kv_fp8_calibrate(chunks[0][1], chunks[0][2], ks, vs)  # per-head scales from the first chunk
+    else:
+        ks = torch.zeros(B, Hkv, lay.scale_stride_head, dtype=torch.float32, device=dev)
+        vs = torch.zeros_like(ks)
     outs = [torch.empty(B, C, Hq, D, dtype=torch.bfloat16, device=dev) for _ in chunks]
     scale = 1.0 / float(np.sqrt(D))
 
     def step(write=True):
         for i, (qc, kcn, vcn) in enumerate(chunks):
-            hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write)
+            hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8)
 
     for _ in range(args.warmup):
         step()
@@ -134,15 +141,17 @@ def bench_prefill(args, torch, hb, wl):
     kms = float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
     peak = 2500.0
     res = {
-        "metric": "prefill-attn TFLOP/s (% bf16 MFMA peak) + tokens/s, B=4 x 4096 in 512-chunks, Llama-3-8B shape",
+        "metric": "prefill-attn TFLOP/s (%% bf16 MFMA peak) + tokens/s, B=4 x 4096 in %d-chunks, Llama-3-8B shape" % C,
         "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 MFMA (new tokens) + f16 MFMA over int8 codes (history), f32 accumulate",
+        "dtype": "bf16 MFMA (new tokens) + f16 MFMA over %s codes (history), f32 accumulate" % ("fp8" if fp8 else "int8"),
         "data": "synthetic (seeded, generated on device)",
-        "config": {"workload": "c3: chunked causal prefill B=4 T=4096 chunk=512 Hq=32 Hkv=8 D=128, int8 cache of earlier "
-                               "chunks + own bf16 K/V, quantize-on-write, one layer", "algorithmic_flops_per_step": int(flops)},
+        "config": {"workload": "c3%s: chunked causal prefill B=4 T=4096 chunk=%d Hq=32 Hkv=8 D=128, %s cache of earlier "
+                               "chunks + own bf16 K/V, quantize-on-write, one layer"
+                               % ("-fp8" if fp8 else "-prompt" if C == T else "", C, "fp8 e4m3fn" if fp8 else "int8"),
+                   "algorithmic_flops_per_step": int(flops)},
         "tokens_per_s": B * T / (ms * 1e-3),
-        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel (8 chunk launches)", "achieved": flops / (kms * 1e-3) / 1e12,
+        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel (%d chunk launches)" % len(chunks), "achieved": flops / (kms * 1e-3) / 1e12,
                      "peak": peak, "unit": "TFLOP/s", "frac": flops / (kms * 1e-3) / 1e12 / peak, "traffic": None,
                      "avg_us_8_launches": kms * 1e3},
     }
@@ -208,7 +217,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c5-decode", "c5-prefill"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c5-decode", "c5-prefill"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
@@ -238,8 +247,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": max(1, args.steps)}))
         return
-    if args.workload == "c3":
-        return bench_prefill(args, torch, hb, wl)
+    if args.workload.startswith("c3"):
+        return bench_prefill(args, torch, hb, wl, C=4096 if args.workload == "c3-prompt" else 512,
+                             fp8=args.workload == "c3-fp8")
     if args.workload.startswith("c5"):
         return bench_deltanet(args, torch, hb, wl, args.workload.endswith("prefill"))
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]

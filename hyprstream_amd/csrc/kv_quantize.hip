@@ -18,12 +18,12 @@ __global__ __launch_bounds__(256) void kv_quantize_kernel(QuantArgs a) {
     quantize_row<E, FP8>(a, blockIdx.y, row, threadIdx.x & 63);
 }
 
-// int8 quantize-on-write for many rows: LPR = D/8 lanes own one row (eight consecutive elements each, one 16-byte
+// Quantize-on-write for many rows: LPR = D/8 lanes own one row (eight consecutive elements each, one 16-byte
 // load for 16-bit sources and one 8-byte store of codes), so a wavefront carries 64/LPR rows and the per-row
 // bookkeeping -- index arithmetic, address resolution, the absmax reduction, the scale store -- is paid once
 // per wavefront instead of once per row.  The arithmetic per element is that of quantize_row (same IEEE
 // divisions, same rounding): the codes and scales are the same bits.  Grid: (row groups of one sequence, K/V, B).
-template <int LPR>
+template <int LPR, bool FP8>
 __global__ __launch_bounds__(256) void kv_quantize_rows_kernel(QuantArgs a) {
 #pragma clang fp contract(off)
     constexpr int kRowsPerWave = 64 / LPR;
@@ -60,35 +60,49 @@ __global__ __launch_bounds__(256) void kv_quantize_rows_kernel(QuantArgs a) {
             }
         }
     }
-    float m = 0.0f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const float v = fabsf(x[e]);
-        m = v > m ? v : m;
-    }
-#pragma unroll
-    for (int o = LPR / 2; o > 0; o >>= 1) {
-        const float w = __shfl_xor(m, o, 64);
-        m = m > w ? m : w;
-    }
     float sc = 0.0f;
     uint32_t packed[2] = {0u, 0u};
-    if (m > 0.0f) {
-        sc = m / 127.0f;
+    if (FP8) {  // one scale per (sequence, kv-head), read; the element arithmetic of quantize_row
+        sc = a.scales[which][(int64_t)b * a.Hkv + h];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            float q = rintf(x[e] / sc);
-            q = q > 127.0f ? 127.0f : q;
-            q = q < -127.0f ? -127.0f : q;
-            if (q != q) q = 0.0f;
-            packed[e >> 2] |= ((uint32_t)(int)q & 0xffu) << (8 * (e & 3));
+            float y = 0.0f;
+            if (sc > 0.0f) {
+                y = x[e] / sc;
+                if (y > 448.0f) y = 448.0f;
+                if (y < -448.0f) y = -448.0f;
+            }
+            packed[e >> 2] |= f32_to_e4m3fn_bits(y) << (8 * (e & 3));
+        }
+    } else {
+        float m = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float v = fabsf(x[e]);
+            m = v > m ? v : m;
+        }
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) {
+            const float w = __shfl_xor(m, o, 64);
+            m = m > w ? m : w;
+        }
+        if (m > 0.0f) {
+            sc = m / 127.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float q = rintf(x[e] / sc);
+                q = q > 127.0f ? 127.0f : q;
+                q = q < -127.0f ? -127.0f : q;
+                if (q != q) q = 0.0f;
+                packed[e >> 2] |= ((uint32_t)(int)q & 0xffu) << (8 * (e & 3));
+            }
         }
     }
     if (!ok) return;
     uint8_t *dst = (uint8_t *)a.codes[which] + unit * ad.code_stride_seq + (int64_t)h * ad.code_stride_head +
                    (int64_t)slot * a.D + sub * 8;
     *(uint2 *)dst = make_uint2(packed[0], packed[1]);
-    if (sub == 0) a.scales[which][unit * ad.scale_stride_seq + (int64_t)h * ad.scale_stride_head + slot] = sc;
+    if (!FP8 && sub == 0) a.scales[which][unit * ad.scale_stride_seq + (int64_t)h * ad.scale_stride_head + slot] = sc;
 }
 
 struct RopeArgs {
@@ -364,17 +378,17 @@ static int launch_quantize(const void *k_src, const void *v_src, int dtype, void
     a.positions = positions; a.start_pos = start_pos;
     a.B = B; a.S = S; a.Hkv = Hkv; a.D = D; a.dtype = dtype;
     a.rope_sin = rope_sin; a.rope_cos = rope_cos; a.rope_len = rope_len;
-    // Bulk int8 writes without rotation take the kernel that packs several rows into a wavefront; it wants
+    // Bulk writes without rotation take the kernel that packs several rows into a wavefront; it wants
     // 16-byte aligned sources and 8-byte aligned code rows and at most 65535 sequences (grid.z).
     const bool aligned = (((uintptr_t)k_src | (uintptr_t)v_src) & 15) == 0 && (((uintptr_t)kc | (uintptr_t)vc) & 7) == 0 &&
                          (l->code_stride_seq & 7) == 0;
-    if (!FP8 && !rope_sin && aligned && B <= 65535 && (int64_t)S * Hkv < (1 << 30)) {
+    if (!rope_sin && aligned && B <= 65535 && (int64_t)S * Hkv < (1 << 30)) {
         const int lpr = D / 8, rows_per_wg = 4 * (64 / lpr);
         dim3 g((unsigned)(((int64_t)S * Hkv + rows_per_wg - 1) / rows_per_wg), 2, B);
-        if (D == 64) kv_quantize_rows_kernel<8><<<g, 256, 0, stream>>>(a);
-        else if (D == 128) kv_quantize_rows_kernel<16><<<g, 256, 0, stream>>>(a);
-        else kv_quantize_rows_kernel<32><<<g, 256, 0, stream>>>(a);
-        return check_launch("kv_quantize_int8");
+        if (D == 64) kv_quantize_rows_kernel<8, FP8><<<g, 256, 0, stream>>>(a);
+        else if (D == 128) kv_quantize_rows_kernel<16, FP8><<<g, 256, 0, stream>>>(a);
+        else kv_quantize_rows_kernel<32, FP8><<<g, 256, 0, stream>>>(a);
+        return check_launch(FP8 ? "kv_quantize_fp8" : "kv_quantize_int8");
     }
     dim3 grid((unsigned)((rows + 3) / 4), 2);
     if (D == 64) kv_quantize_kernel<1, FP8><<<grid, 256, 0, stream>>>(a);
