@@ -214,6 +214,45 @@ __global__ __launch_bounds__(256) void fp8_calibrate_kernel(const void *k_src, c
     }
 }
 
+// The same for 16-bit sources: 1024 threads per (b, h, tensor), 16-byte loads (eight elements), many rows in flight.
+__global__ __launch_bounds__(1024) void fp8_calibrate16_kernel(const uint16_t *k_src, const uint16_t *v_src, int dtype,
+                                                              float *k_scales, float *v_scales, int B, int S, int Hkv, int D) {
+    const int which = blockIdx.y;
+    const int b = blockIdx.x / Hkv, h = blockIdx.x % Hkv;
+    const uint16_t *src = which ? v_src : k_src;
+    const int lpr = D / 8, sub = threadIdx.x % lpr, rows_per_pass = 1024 / lpr;
+    float m = 0.0f;
+    for (int s0 = threadIdx.x / lpr; s0 < S; s0 += rows_per_pass) {
+        const uint4 w = *(const uint4 *)(src + (((int64_t)b * S + s0) * Hkv + h) * D + sub * 8);
+        const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float x0, x1;
+            if (dtype == HS_BF16) {
+                x0 = __uint_as_float(ww[i] << 16);
+                x1 = __uint_as_float(ww[i] & 0xffff0000u);
+            } else {
+                _Float16 f[2];
+                __builtin_memcpy(f, &ww[i], 4);
+                x0 = (float)f[0];
+                x1 = (float)f[1];
+            }
+            const float a0 = fabsf(x0), a1 = fabsf(x1);
+            m = a0 > m ? a0 : m;
+            m = a1 > m ? a1 : m;
+        }
+    }
+    m = wave_max(m);
+    __shared__ float red[16];
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int i = 1; i < 16; ++i) m = fmaxf(m, red[i]);
+        (which ? v_scales : k_scales)[b * Hkv + h] = m / 448.0f;
+    }
+}
+
 __device__ __forceinline__ float e4m3fn_bits_to_f32(uint32_t c) {
     uint32_t e = (c >> 3) & 0xfu, m = c & 7u;
     float v;
@@ -465,8 +504,12 @@ int hs_kv_fp8_calibrate(const void *k_src, const void *v_src, int src_dtype, flo
         return hs::fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d Hkv=%d D=%d", B, S, Hkv, D);
     if (src_dtype != HS_BF16 && src_dtype != HS_F32 && src_dtype != HS_F16)
         return hs::fail(HS_ERR_INVALID_ARGUMENT, "unknown src_dtype %d", src_dtype);
-    hs::fp8_calibrate_kernel<<<dim3(B * Hkv, 2), 256, 0, (hipStream_t)stream>>>(k_src, v_src, src_dtype, k_scales,
-                                                                               v_scales, B, S, Hkv, D);
+    if (src_dtype != HS_F32 && (D == 64 || D == 128 || D == 256) && (((uintptr_t)k_src | (uintptr_t)v_src) & 15) == 0)
+        hs::fp8_calibrate16_kernel<<<dim3(B * Hkv, 2), 1024, 0, (hipStream_t)stream>>>(
+            (const uint16_t *)k_src, (const uint16_t *)v_src, src_dtype, k_scales, v_scales, B, S, Hkv, D);
+    else
+        hs::fp8_calibrate_kernel<<<dim3(B * Hkv, 2), 256, 0, (hipStream_t)stream>>>(k_src, v_src, src_dtype, k_scales,
+                                                                                   v_scales, B, S, Hkv, D);
     return hs::check_launch("fp8_calibrate");
 }
 
