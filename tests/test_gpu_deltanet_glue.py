@@ -124,3 +124,33 @@ def test_prepare_rejects_aliased_state_and_nulls():
     f = torch.zeros(8, device=DEV)
     rc = L.hs_deltanet_prepare(p(x), p(x), p(st), p(st), p(x), p(x), p(f), p(f), p(x), p(x), p(x), p(f), p(f), 1, 4, 1, 1, 128, 128, None)
     assert rc == hb.HS_ERR_INVALID_ARGUMENT and b"alias" in L.hs_attn_last_error()
+
+
+def test_inputs_without_16_byte_alignment_take_the_narrow_kernels():
+    """An input whose address is only element-aligned is served by the one-channel / one-row kernels, to the same bar."""
+    def misaligned(t):
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device=DEV)
+        out = buf[1:].view(t.shape)
+        out.copy_(t)
+        assert out.data_ptr() % 16 != 0
+        return out
+
+    B, S, nk, nv, dk, dv = 2, 37, 2, 4, 128, 128
+    p = _layer_inputs(1300, B, S, nk, nv, dk, dv)
+    q, k, v, g, beta, st = hb.deltanet_prepare(misaligned(p["x"]), p["w"].to(DEV), p["st"].to(DEV), p["a"].to(DEV), p["b"].to(DEV),
+                                               p["nae"].to(DEV), p["dtb"].to(DEV), nk, nv, dk, dv)
+    torch.cuda.synchronize()
+    y, want_st = orc.deltanet_conv_silu_bf16(_bits(p["x"]), _bits(p["w"]), _bits(p["st"]))
+    kd = nk * dk
+    assert _ulps(_bits(q).reshape(B, S, kd), y[..., :kd]).max() <= 1
+    assert _ulps(_bits(k).reshape(B, S, kd), y[..., kd:2 * kd]).max() <= 1
+    assert _ulps(_bits(v).reshape(B, S, nv * dv), y[..., 2 * kd:]).max() <= 1
+    assert np.array_equal(_bits(st), want_st)
+
+    r = wl.philox(1301)
+    x = torch.from_numpy((r.standard_normal((5, 3, 128)) * 2).astype(np.float32))
+    z = torch.from_numpy(r.standard_normal((5, 3, 128)).astype(np.float32)).to(torch.bfloat16)
+    w = torch.from_numpy(r.standard_normal(128).astype(np.float32))
+    got = hb.deltanet_gated_norm(misaligned(x), z.to(DEV), w.to(DEV), 1e-6)
+    torch.cuda.synchronize()
+    assert _ulps(_bits(got), orc.gated_rmsnorm(x.numpy(), _bits(z), w.numpy(), 1e-6)).max() <= 1

@@ -174,3 +174,53 @@ def test_fp8_dense_view():
     torch.cuda.synchronize()
     kc, vc, ks, vs = c.canonical(9)
     assert np.array_equal(out.cpu().numpy(), oracle.dequant_fp8(vc, vs))
+
+
+def _misaligned(t):
+    """The same values in a contiguous tensor whose address is only element-aligned (not 16-byte aligned)."""
+    buf = torch.empty(t.numel() + 1, dtype=t.dtype, device=t.device)
+    out = buf[1:].view(t.shape)
+    out.copy_(t)
+    assert out.is_contiguous() and out.data_ptr() % 16 != 0
+    return out
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_sources_without_16_byte_alignment_give_the_same_bits(fp8):
+    """Tensors that do not meet the wide kernels' alignment take the one-row-per-wavefront kernels: same cache."""
+    B, S, Hkv, D = 2, 21, 3, 128
+    r = wl.philox(31)
+    k = torch.from_numpy(r.standard_normal((B, S, Hkv, D)).astype(np.float32)).to(DEV).bfloat16()
+    v = torch.from_numpy(r.standard_normal((B, S, Hkv, D)).astype(np.float32)).to(DEV).bfloat16()
+    caches = []
+    for ks, vs in ((k, v), (_misaligned(k), _misaligned(v))):
+        c = DeviceCache(B, Hkv, S, D, fp8=fp8)
+        if fp8:
+            hb.kv_fp8_calibrate(ks, vs, c.k_scales, c.v_scales)
+        c.write(ks, vs)
+        caches.append(c)
+    torch.cuda.synchronize()
+    a, m = caches
+    for name in ("k_codes", "v_codes", "k_scales", "v_scales"):
+        assert torch.equal(getattr(a, name), getattr(m, name)), name
+    # dense view into an output that is not 16-byte aligned
+    want = torch.empty(B, S, Hkv, D, dtype=torch.bfloat16, device=DEV)
+    got = _misaligned(want)
+    hb.kv_dequantize(a.k_codes, a.k_scales, fp8, a.layout, 0, want)
+    hb.kv_dequantize(a.k_codes, a.k_scales, fp8, a.layout, 0, got)
+    torch.cuda.synchronize()
+    assert torch.equal(want, got)
+
+
+def test_rope_without_16_byte_alignment_gives_the_same_bits():
+    B, S, H, D = 2, 9, 4, 128
+    r = wl.philox(32)
+    x = torch.from_numpy(r.standard_normal((B, S, H, D)).astype(np.float32)).to(DEV).bfloat16()
+    ang = torch.from_numpy(r.random((S, D // 2)).astype(np.float32) * 6.0).to(DEV)
+    sin, cos = ang.sin().bfloat16().contiguous(), ang.cos().bfloat16().contiguous()
+    want = torch.empty_like(x)
+    hb.rope_apply(x, sin, cos, want)
+    got = _misaligned(want)
+    hb.rope_apply(_misaligned(x), sin, cos, got)
+    torch.cuda.synchronize()
+    assert torch.equal(want, got)
