@@ -81,8 +81,10 @@ def contiguous_layout(Hkv, capacity_tokens, D, scale_pad=4):
 def paged_layout(Hkv, block_tokens, D, k_table, v_table):
     """Pool of blocks [nblocks, Hkv, block_tokens, D]; tables are int32 device tensors [B, max_blocks]."""
     assert k_table.dtype.is_signed and k_table.element_size() == 4 and k_table.is_contiguous()
-    return KvLayout(Hkv * block_tokens * D, block_tokens * D, Hkv * block_tokens, block_tokens, block_tokens,
-                    k_table.shape[1], k_table.data_ptr(), v_table.data_ptr(), 0)
+    lay = KvLayout(Hkv * block_tokens * D, block_tokens * D, Hkv * block_tokens, block_tokens, block_tokens,
+                   k_table.shape[1], k_table.data_ptr(), v_table.data_ptr(), 0)
+    lay._tables = (k_table, v_table)  # the struct holds raw addresses: the tensors must live as long as it does
+    return lay
 
 
 def _ptr(t):

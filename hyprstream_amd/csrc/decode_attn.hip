@@ -38,13 +38,20 @@
 namespace hs {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kD = 128;          // head_dim served by this kernel
-constexpr int kStep = 32;        // tokens per wavefront step
+// head_dim 128 or 256.  A wavefront step always covers 8 KB of codes: 32 tokens at D = 128, 16 at D = 256 (the
+// second product then runs on v_mfma_f32_16x16x16_f16, whose operand layout matches one 16-token score tile).
+template <int D> struct Shape {
+    static constexpr int kStep = D == 256 ? 16 : 32;  // tokens per wavefront step
+    static constexpr int NT = kStep / 16;             // 16-token score tiles per step
+    static constexpr int NJ = D / 32;                 // MFMAs per score tile (32 d each)
+    static constexpr int NC = D / 128;                // 128-column groups of V / O
+};
 constexpr int kWavesPerWg = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kPScale = 64.0f;  // P is carried as 64*p*s_v in fp16 (keeps small weights normal)
@@ -69,29 +76,32 @@ struct DecodeArgs {
 
 // Half-split rotary embedding of the 32 query elements a lane holds, in bf16 arithmetic (every product and sum
 // rounded to bf16, as the separate libtorch ops of RoPE::apply_rotary_pos_emb do, rope.rs:206-248).  Element
-// qf[8*i + e] is d = 64*(i/2) + 16*lq + 8*(i%2) + e, so a lane holds both halves of each rotated pair.
-__device__ __forceinline__ void rope_rotate_q(float (&qf)[32], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
+// qf[8*i + e] is d = 64*(i/2) + 16*lq + 8*(i%2) + e (i < NJ = D/32), so a lane holds both halves of each rotated
+// pair: blocks i and i + NJ/2.
+template <int NJ>
+__device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
 #pragma clang fp contract(off)
     auto rb = [](float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); };
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const u32x4 sw = *(const u32x4 *)(sin_row + 16 * lq + 8 * i), cw = *(const u32x4 *)(cos_row + 16 * lq + 8 * i);
+    for (int i = 0; i < NJ / 2; ++i) {
+        const int j0 = 64 * (i >> 1) + 16 * lq + 8 * (i & 1);
+        const u32x4 sw = *(const u32x4 *)(sin_row + j0), cw = *(const u32x4 *)(cos_row + j0);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
             const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
-            const float x1 = qf[8 * i + e], x2 = qf[8 * (i + 2) + e];
+            const float x1 = qf[8 * i + e], x2 = qf[8 * (i + NJ / 2) + e];
             qf[8 * i + e] = rb(rb(x1 * cs) - rb(x2 * sn));
-            qf[8 * (i + 2) + e] = rb(rb(x1 * sn) + rb(x2 * cs));
+            qf[8 * (i + NJ / 2) + e] = rb(rb(x1 * sn) + rb(x2 * cs));
         }
     }
 }
 
-template <bool FP8>
+template <int D>
 struct Stage {
-    u32x4 k[2][2];  // [16-token tile][half of the row]: 16 B at byte 64*half + 16*lq of row li
-    u32x2 v[8];     // [token slot e = 4u + r] 8 bytes: d = 8*(lane%16) .. +7
-    float sraw;     // int8 only: lanes 0-31 hold the K scale of token `lane`, lanes 32-63 the V scale of token lane-32
+    u32x4 k[Shape<D>::NT][Shape<D>::NJ / 2];  // [16-token tile][64-byte piece of the row]: 16 B at byte 64*piece + 16*lq of row li
+    u32x2 v[Shape<D>::NC][4 * Shape<D>::NT];  // [column group c][token slot e = 4u + r] 8 bytes: d = 128*c + 8*(lane%16) .. +7
+    float sraw;  // int8 only: lanes [0, kStep) hold the K scale of token `lane`, lanes [kStep, 2*kStep) the V scales
 };
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -105,8 +115,9 @@ __device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t t) {
     return (t & 0x80008000u) | ((t >> 1) & 0x3f803f80u);
 }
 
-template <bool FP8, bool ROPE>
+template <int kD, bool FP8, bool ROPE>
 __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
+    constexpr int kStep = Shape<kD>::kStep, NT = Shape<kD>::NT, NJ = Shape<kD>::NJ, NC = Shape<kD>::NC;
     // Workgroups go to the 8 XCDs round-robin by linear id.  Low chunk indices always hold work, high ones only
     // for long sequences, so the chunk index is rotated by (head + sequence): every XCD then sees every index
     // equally often instead of two XCDs getting all the first chunks.
@@ -128,24 +139,24 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     // so those first loads are issued ahead of the write and its barrier instead of behind them.
     const bool writes_new = a.nt.src[0] != nullptr && t_end == L;
     auto write_new_token = [&]() {
-        if (wave < 2) quantize_row<2, FP8>(a.nt, wave, (int64_t)b * a.Hkv + h, lane);
+        if (wave < 2) quantize_row<kD / 64, FP8>(a.nt, wave, (int64_t)b * a.Hkv + h, lane);
         __syncthreads();  // codes and scales are visible to the whole workgroup before any load that covers them
     };
 
-    half8 qop[4];
+    half8 qop[NJ];
     float cq = 0.0f, cinit = 0.0f;
     // fp8: the V scale is one constant per (sequence, head); it multiplies the finished partial.
     const float out_scale = (1.0f / kPScale) * (FP8 ? 256.0f * a.vs[(int64_t)b * a.Hkv + h] : 1.0f);
 
-    float4v acc[8];  // O[d = 32*lq + 8*r + bb][head li] in acc[bb][r]
+    float4v acc[8 * NC];  // O[d = 128*c + 32*lq + 8*r + bb][head li] in acc[8*c + bb][r]
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < 8 * NC; ++i) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
 
     const int nsteps = (t_end - t_begin + kStep - 1) / kStep;
     __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64];
 
-    auto load_stage = [&](Stage<FP8> &st, int step) {
+    auto load_stage = [&](Stage<kD> &st, int step) {
         const int t0 = t_begin + step * kStep;
         int64_t ku, vu;
         int kslot, vslot;
@@ -155,49 +166,52 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         const uint8_t *kb = a.kc + ku * a.ka.code_stride_seq + (int64_t)h * a.ka.code_stride_head + (int64_t)kslot * kD;
         const uint8_t *vb = a.vc + vu * a.va.code_stride_seq + (int64_t)h * a.va.code_stride_head + (int64_t)vslot * kD;
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < NT; ++u) {
             const int row = min(16 * u + li, last);
-            const uint8_t *p = kb + row * kD + 16 * lq;  // each load covers one 64-byte half of 16 rows
-            st.k[u][0] = __builtin_nontemporal_load((const u32x4 *)p);
-            st.k[u][1] = __builtin_nontemporal_load((const u32x4 *)(p + 64));
+            const uint8_t *p = kb + row * kD + 16 * lq;  // each load covers one 64-byte piece of 16 rows
+#pragma unroll
+            for (int hf = 0; hf < NJ / 2; ++hf) st.k[u][hf] = __builtin_nontemporal_load((const u32x4 *)(p + 64 * hf));
         }
         if (!FP8) {
-            // one 4-byte load per lane brings the step's 32 K scales and 32 V scales (two full 128-byte lines);
+            // one 4-byte load per lane brings the step's K scales and V scales (two full 128-byte lines at 32 tokens);
             // compute_stage hands them to the lanes that need them through LDS
             const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)h * a.ka.scale_stride_head + kslot;
             const float *vsb = a.vs + vu * a.va.scale_stride_seq + (int64_t)h * a.va.scale_stride_head + vslot;
-            st.sraw = __builtin_nontemporal_load((lane < 32 ? ksb : vsb) + min(lane & 31, last));
+            const int sl = lane & (2 * kStep - 1);  // 16-token steps: the upper 32 lanes repeat the lower ones
+            st.sraw = __builtin_nontemporal_load((sl < kStep ? ksb : vsb) + min(sl & (kStep - 1), last));
         }
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int c = 0; c < NC; ++c)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int row = min(16 * u + 4 * lq + r, last);
-                st.v[4 * u + r] = __builtin_nontemporal_load((const u32x2 *)(vb + row * kD + 8 * li));
-            }
+            for (int u = 0; u < NT; ++u)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = min(16 * u + 4 * lq + r, last);
+                    st.v[c][4 * u + r] = __builtin_nontemporal_load((const u32x2 *)(vb + row * kD + 128 * c + 8 * li));
+                }
     };
 
-    auto compute_stage = [&](const Stage<FP8> &st, int step) {
+    auto compute_stage = [&](const Stage<kD> &st, int step) {
         const int t0 = t_begin + step * kStep;
         // ---- token scales: lane (li, lq) needs those of tokens 16u + 4*lq + r, the rows of its score registers.
         //      LDS operations of one wavefront complete in order, so the reads see the write without a barrier.
-        float4v sk[2], sv[2];
+        float4v sk[NT], sv[NT];
         if (!FP8) {
             sm_sc[wave][lane] = st.sraw;
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
+            for (int u = 0; u < NT; ++u) {
                 sk[u] = *(const float4v *)&sm_sc[wave][16 * u + 4 * lq];
-                sv[u] = *(const float4v *)&sm_sc[wave][32 + 16 * u + 4 * lq];
+                sv[u] = *(const float4v *)&sm_sc[wave][kStep + 16 * u + 4 * lq];
             }
         }
-        // ---- scores: 2 tiles x 4 MFMAs (K of 128 split in 4 x 32)
-        float4v s[2];
+        // ---- scores: NT tiles x NJ MFMAs (the head dimension in pieces of 32)
+        float4v s[NT];
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
+        for (int u = 0; u < NT; ++u) {
             s[u] = (float4v){cinit, cinit, cinit, cinit};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NJ; ++j) {
                 const uint32_t w0 = st.k[u][j >> 1][2 * (j & 1)], w1 = st.k[u][j >> 1][2 * (j & 1) + 1];
                 half8 ak;
                 if (FP8) {
@@ -216,9 +230,9 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             }
         }
         // ---- scale to log2 units, mask the tail
-        float sc[8], pv[8];
+        float sc[4 * NT], pv[4 * NT];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < NT; ++u)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 sc[4 * u + r] = FP8 ? s[u][r] * cq : s[u][r] * sk[u][r] * cq;
@@ -227,7 +241,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         const bool tail = t0 + kStep > L;
         if (tail) {
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < NT; ++u)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
                     if (t0 + 16 * u + 4 * lq + r >= L) {
@@ -238,7 +252,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         // ---- online softmax (max shared by the 4 lanes of a head)
         float mx = sc[0];
 #pragma unroll
-        for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sc[i]);
+        for (int i = 1; i < 4 * NT; ++i) mx = fmaxf(mx, sc[i]);
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run, mx);
@@ -246,26 +260,26 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= alpha;
 #pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] *= alpha;
+            for (int i = 0; i < 8 * NC; ++i) acc[i] *= alpha;
             m_run = m_new;
         }
-        uint32_t pb[4];
+        uint32_t pb[2 * NT];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < 2 * NT; ++i) {
             const float p0 = __builtin_amdgcn_exp2f(sc[2 * i] - m_run);
             const float p1 = __builtin_amdgcn_exp2f(sc[2 * i + 1] - m_run);
             l_run += p0 + p1;
             half2v hp = {(_Float16)(p0 * pv[2 * i]), (_Float16)(p1 * pv[2 * i + 1])};
             pb[i] = __builtin_bit_cast(uint32_t, hp);
         }
-        const half8 pop = as_half8(pb[0], pb[1], pb[2], pb[3]);
-        // ---- O += V^T P : 8 MFMAs, one per byte column bb of this lane's 8 d's
+        // ---- O += V^T P : 8 MFMAs per column group, one per byte column bb of this lane's 8 d's
 #pragma unroll
-        for (int bb = 0; bb < 8; ++bb) {
-            uint32_t av[4];
+        for (int cb = 0; cb < 8 * NC; ++cb) {
+            const int c = cb >> 3, bb = cb & 7;
+            uint32_t av[2 * NT];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const uint32_t lo = st.v[2 * p][bb >> 2], hi = st.v[2 * p + 1][bb >> 2];
+            for (int p = 0; p < 2 * NT; ++p) {
+                const uint32_t lo = st.v[c][2 * p][bb >> 2], hi = st.v[c][2 * p + 1][bb >> 2];
                 if (FP8) {
                     const uint32_t sel = 0x040c000cu + ((uint32_t)(bb & 3) << 8) + ((uint32_t)(bb & 3) << 24);
                     av[p] = fp8x2_to_f16x2(__builtin_amdgcn_perm(hi, lo, sel));
@@ -276,12 +290,19 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                     av[p] = __builtin_bit_cast(uint32_t, hv);
                 }
             }
-            acc[bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av[0], av[1], av[2], av[3]), pop, acc[bb], 0, 0, 0);
+            if constexpr (NT == 2) {
+                acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av[0], av[1], av[2], av[3]),
+                                                                 as_half8(pb[0], pb[1], pb[2], pb[3]), acc[cb], 0, 0, 0);
+            } else {
+                const u32x2 aw = {av[0], av[1]}, pw = {pb[0], pb[1]};
+                acc[cb] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, aw), __builtin_bit_cast(half4, pw),
+                                                                acc[cb], 0, 0, 0);
+            }
         }
     };
 
     // ---- software pipeline over this wavefront's steps (wave, wave+4, ...)
-    Stage<FP8> sa, sb;
+    Stage<kD> sa, sb;
     int step = wave;
     const bool early_loads = nsteps >= kWavesPerWg + 1;
     if (writes_new && !early_loads) write_new_token();
@@ -290,12 +311,12 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds
     //      Q[head][64*(j/2) + 16*lq + 8*(j%2) + e] for MFMA j.
     {
-        float qf[32];
+        float qf[8 * NJ];
         float amax = 0.0f;
         if (li < G) {
             const uint16_t *qp = a.q + ((int64_t)b * a.Hq + h * G + li) * kD + 16 * lq;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {  // MFMA i contracts d = 64*(i/2) + 16*lq + 8*(i%2) + e, as the K loads do
+            for (int i = 0; i < NJ; ++i) {  // MFMA i contracts d = 64*(i/2) + 16*lq + 8*(i%2) + e, as the K loads do
                 u32x4 w = *(const u32x4 *)(qp + 64 * (i >> 1) + 8 * (i & 1));
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -305,13 +326,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             }
             if (ROPE) {
                 const int p = min(max(a.seq_lens[b] - 1, 0), a.rope_len - 1);  // the query is the newest token
-                rope_rotate_q(qf, a.rope_sin + (int64_t)p * (kD / 2), a.rope_cos + (int64_t)p * (kD / 2), lq);
+                rope_rotate_q<NJ>(qf, a.rope_sin + (int64_t)p * (kD / 2), a.rope_cos + (int64_t)p * (kD / 2), lq);
             }
 #pragma unroll
-            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
+            for (int i = 0; i < 8 * NJ; ++i) amax = fmaxf(amax, fabsf(qf[i]));
         } else {
 #pragma unroll
-            for (int i = 0; i < 32; ++i) qf[i] = 0.0f;
+            for (int i = 0; i < 8 * NJ; ++i) qf[i] = 0.0f;
         }
         amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
         amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
@@ -321,7 +342,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         const float down = __uint_as_float((uint32_t)(127 - ex) << 23), up = __uint_as_float((uint32_t)(127 + ex) << 23);
         float qsum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 _Float16 hq = (_Float16)(qf[8 * j + e] * down);
@@ -355,7 +376,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
     __shared__ float sm_m[kWavesPerWg][16], sm_l[kWavesPerWg][16];
-    __shared__ float sm_o[kWavesPerWg][16][kD + 4];
+    __shared__ float sm_o[kWavesPerWg][16][128 + 4];  // one 128-column group of O at a time
     if (lq == 0) {
         sm_m[wave][li] = m_run;
         sm_l[wave][li] = l_run;
@@ -365,38 +386,42 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 #pragma unroll
     for (int w = 1; w < kWavesPerWg; ++w) M = fmaxf(M, sm_m[w][li]);
     const float f = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f(m_run - M);
-    if (li < G) {
-#pragma unroll
-        for (int bb = 0; bb < 8; ++bb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sm_o[wave][li][32 * lq + 8 * r + bb] = acc[bb][r] * f;
-    }
-    __syncthreads();
     const int64_t prow = ((int64_t)b * a.Hq + h * G) * a.nchunks + chunk;
-    if (a.direct) {
-        // single chunk: normalise and write the output, no workspace traffic
-        for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
-            const int g = idx / kD, d = idx % kD;
-            float o = 0.0f, l = 0.0f, Mg = sm_m[0][g];
 #pragma unroll
-            for (int w = 1; w < kWavesPerWg; ++w) Mg = fmaxf(Mg, sm_m[w][g]);
+    for (int c = 0; c < NC; ++c) {
+        if (c > 0) __syncthreads();  // the previous group has been read
+        if (li < G) {
 #pragma unroll
-            for (int w = 0; w < kWavesPerWg; ++w) {
-                o += sm_o[w][g][d];
-                l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
-            }
-            a.out[((int64_t)b * a.Hq + h * G + g) * kD + d] = (uint16_t)f32_to_bf16_bits(o * out_scale / l);
+            for (int bb = 0; bb < 8; ++bb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sm_o[wave][li][32 * lq + 8 * r + bb] = acc[8 * c + bb][r] * f;
         }
-        return;
-    }
-    for (int idx = threadIdx.x; idx < G * kD; idx += 256) {
-        const int g = idx / kD, d = idx % kD;
-        float o = 0.0f;
+        __syncthreads();
+        if (a.direct) {
+            // single chunk: normalise and write the output, no workspace traffic
+            for (int idx = threadIdx.x; idx < G * 128; idx += 256) {
+                const int g = idx / 128, d = idx % 128;
+                float o = 0.0f, l = 0.0f, Mg = sm_m[0][g];
 #pragma unroll
-        for (int w = 0; w < kWavesPerWg; ++w) o += sm_o[w][g][d];
-        a.part_o[(prow + (int64_t)g * a.nchunks) * kD + d] = o * out_scale;
+                for (int w = 1; w < kWavesPerWg; ++w) Mg = fmaxf(Mg, sm_m[w][g]);
+#pragma unroll
+                for (int w = 0; w < kWavesPerWg; ++w) {
+                    o += sm_o[w][g][d];
+                    l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
+                }
+                a.out[((int64_t)b * a.Hq + h * G + g) * kD + 128 * c + d] = (uint16_t)f32_to_bf16_bits(o * out_scale / l);
+            }
+        } else {
+            for (int idx = threadIdx.x; idx < G * 128; idx += 256) {
+                const int g = idx / 128, d = idx % 128;
+                float o = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kWavesPerWg; ++w) o += sm_o[w][g][d];
+                a.part_o[(prow + (int64_t)g * a.nchunks) * kD + 128 * c + d] = o * out_scale;
+            }
+        }
     }
-    if (threadIdx.x < G) {
+    if (!a.direct && threadIdx.x < G) {
         const int g = threadIdx.x;
         float Mg = sm_m[0][g];
         for (int w = 1; w < kWavesPerWg; ++w) Mg = fmaxf(Mg, sm_m[w][g]);
@@ -410,10 +435,10 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 }
 
 // Merge the chunk partials of one (sequence, query head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c.
-__global__ __launch_bounds__(128) void decode_merge_kernel(const float *part_o, const float *part_ml,
+__global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, const float *part_ml,
                                                           const int32_t *seq_lens, uint16_t *out, int Hq, int nchunks,
                                                           int chunk_tokens, int max_seq_len) {
-    const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+    const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x, kD = blockDim.x;  // one thread per output element
     const int L = min(seq_lens[b], max_seq_len);
     const int n = L <= 0 ? 0 : min(nchunks, (L + chunk_tokens - 1) / chunk_tokens);
     const int64_t row = ((int64_t)b * Hq + hq) * nchunks;
@@ -471,7 +496,7 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
                          size_t ws_bytes, int B, int Hq, int Hkv, int D, int max_seq_len, float softmax_scale,
                          hipStream_t stream) {
     if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
-    if (D != kD) return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 128, got %d", D);
+    if (D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 128 and 256, got %d", D);
     if (B > 0 && (!q || !kc || !vc || !ks || !vs || !seq_lens || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if ((nt.k_src == nullptr) != (nt.v_src == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give k_new and v_new or neither");
     if (nt.k_src && nt.dtype != HS_BF16 && nt.dtype != HS_F32 && nt.dtype != HS_F16)
@@ -479,8 +504,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     if (Hq <= 0 || Hq % Hkv != 0 || Hq / Hkv > 16)
         return fail(HS_ERR_INVALID_ARGUMENT, "need Hq %% Hkv == 0 and Hq/Hkv <= 16 (Hq=%d Hkv=%d)", Hq, Hkv);
     if (max_seq_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "max_seq_len must be positive");
-    if (l->k_block_table && (l->capacity_tokens % kStep) != 0)
-        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of %d tokens", kStep);
+    if (l->k_block_table && (l->capacity_tokens % 32) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of 32 tokens");
     if (B == 0) return HS_OK;
     {
         const int64_t cap = l->k_block_table ? (int64_t)l->capacity_tokens * l->block_table_stride : l->capacity_tokens;
@@ -502,7 +527,7 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.chunk_tokens = pick_chunk_tokens(B, Hkv, max_seq_len, l->total_tokens_hint);
     a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
     a.part_o = (float *)ws;
-    a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * kD;
+    a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * D;
     a.out = (uint16_t *)out;
     a.scale_log2e = softmax_scale * kLog2e;
     a.direct = (phases == 3 && a.nchunks == 1) ? 1 : 0;
@@ -521,13 +546,19 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.rope_sin = (const uint16_t *)nt.rope_sin; a.rope_cos = (const uint16_t *)nt.rope_cos; a.rope_len = nt.rope_len;
     if (phases & 1) {
         dim3 grid(a.nchunks, Hkv, B);
-        if (fp8) decode_attn_kernel<true, false><<<grid, 256, 0, stream>>>(a);
-        else if (a.rope_sin) decode_attn_kernel<false, true><<<grid, 256, 0, stream>>>(a);
-        else decode_attn_kernel<false, false><<<grid, 256, 0, stream>>>(a);
+        if (D == 128) {
+            if (fp8) decode_attn_kernel<128, true, false><<<grid, 256, 0, stream>>>(a);
+            else if (a.rope_sin) decode_attn_kernel<128, false, true><<<grid, 256, 0, stream>>>(a);
+            else decode_attn_kernel<128, false, false><<<grid, 256, 0, stream>>>(a);
+        } else {
+            if (fp8) decode_attn_kernel<256, true, false><<<grid, 256, 0, stream>>>(a);
+            else if (a.rope_sin) decode_attn_kernel<256, false, true><<<grid, 256, 0, stream>>>(a);
+            else decode_attn_kernel<256, false, false><<<grid, 256, 0, stream>>>(a);
+        }
         if (int rc = check_launch("decode_attn")) return rc;
     }
     if ((phases & 2) && !a.direct) {
-        decode_merge_kernel<<<dim3(Hq, B), 128, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
+        decode_merge_kernel<<<dim3(Hq, B), D, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
                                                              a.nchunks, a.chunk_tokens, max_seq_len);
         return check_launch("decode_merge");
     }

@@ -142,7 +142,8 @@ HS_API int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8,
  * q, out: [B, Hq, D] bf16.  seq_lens: device [B], cached tokens per sequence INCLUDING the
  * one just written; rows with seq_len <= 0 produce zeros.  max_seq_len >= every seq_lens[b]
  * (host-side bound used to size the grid).  out = softmax(q K^T * softmax_scale) V with
- * fp32 accumulation, K/V dequantized on the fly.  workspace: device scratch of at least
+ * fp32 accumulation, K/V dequantized on the fly.  D is 128 or 256 (Hq/Hkv <= 16); anything
+ * else is HS_ERR_INVALID_ARGUMENT.  workspace: device scratch of at least
  * hs_decode_attn_workspace_bytes(...) bytes, 256-byte aligned, owned by the caller. */
 HS_API size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len);
 /* Chunks per sequence the decode entry points will use for this shape and hint (1 = a step is a single launch). */

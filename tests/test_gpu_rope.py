@@ -85,10 +85,11 @@ def test_quantize_with_rope_bit_exact(D):
     assert not kc[:, :start].any()  # nothing before start_pos is touched
 
 
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("lens", [[300, 300, 300], [1, 129, 700]])
-def test_decode_step_with_rope_matches_unfused_and_oracle(lens):
-    r = wl.philox(740 + len(set(lens)))
-    B, Hq, Hkv, D, L = len(lens), 16, 4, 128, 1024
+def test_decode_step_with_rope_matches_unfused_and_oracle(lens, D):
+    r = wl.philox(740 + len(set(lens)) + D)
+    B, Hq, Hkv, L = len(lens), 16, 4, 1024
     T = max(lens)
     sin, cos = _tables(D, 500000.0, L, torch.bfloat16)
     sin_d, cos_d = sin.to(DEV), cos.to(DEV)
