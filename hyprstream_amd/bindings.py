@@ -24,7 +24,7 @@ EXPORTS = [
     "hs_kv_quantize_int8", "hs_kv_fp8_calibrate", "hs_kv_quantize_fp8", "hs_kv_dequantize",
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
-    "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
+    "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
     "hs_deltanet_prepare", "hs_deltanet_gated_norm",
 ]
 
@@ -121,12 +121,16 @@ def kv_quantize_int8_rope(k_src, v_src, rope_sin, rope_cos, k_codes, v_codes, k_
                                          ctypes.c_int32(start_pos), B, S, Hkv, D, _stream()))
 
 
-def rope_apply(x, rope_sin, rope_cos, out, positions=None, start_pos=0):
-    """Half-split rotary embedding of x [B, S, H, D] into out (same shape and dtype)."""
+def rope_apply(x, rope_sin, rope_cos, out, positions=None, start_pos=0, rotary_dim=None):
+    """Half-split rotary embedding of x [B, S, H, D] into out (same shape and dtype).  rotary_dim < D rotates only the
+    leading rotary_dim elements of each head (tables [rope_len, rotary_dim/2]) and copies the rest."""
     B, S, H, D = x.shape
     assert x.is_contiguous() and out.is_contiguous() and out.dtype == x.dtype and rope_sin.dtype == x.dtype
-    check(lib().hs_rope_apply(_ptr(x), _dtype_code(x), _ptr(rope_sin), _ptr(rope_cos), ctypes.c_int32(rope_sin.shape[0]),
-                              _ptr(positions), ctypes.c_int32(start_pos), _ptr(out), B, S, H, D, _stream()))
+    rd = D if rotary_dim is None else rotary_dim
+    assert rope_sin.shape[1] == rd // 2 and rope_sin.is_contiguous() and rope_cos.is_contiguous()
+    check(lib().hs_rope_apply_partial(_ptr(x), _dtype_code(x), _ptr(rope_sin), _ptr(rope_cos), ctypes.c_int32(rope_sin.shape[0]),
+                                      _ptr(positions), ctypes.c_int32(start_pos), _ptr(out), B, S, H, D, ctypes.c_int32(rd),
+                                      _stream()))
 
 
 def kv_fp8_calibrate(k_src, v_src, k_scales, v_scales):

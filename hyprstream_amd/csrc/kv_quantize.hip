@@ -110,6 +110,7 @@ struct RopeArgs {
     void *out;
     const int32_t *positions;
     int32_t start_pos, rope_len, B, S, H, D, dtype;
+    int32_t rd;  // rotated leading part of each row (pairs d, d + rd/2); elements [rd, D) pass through
 };
 
 // Rotary embedding of a [B, S, H, D] tensor (the query side of a step; K is rotated inside the cache write).
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
     const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
     float x[E];
     load_src<E>(a.x, a.dtype, row * a.D + lane * E, x);
-    rope_rotate<E>(a.x, a.dtype, row * a.D, a.D, a.sin_t, a.cos_t, a.rope_len, pos, lane * E, x);
+    if (lane * E < a.rd) rope_rotate<E>(a.x, a.dtype, row * a.D, a.rd, a.sin_t, a.cos_t, a.rope_len, pos, lane * E, x);
     const int64_t o = row * a.D + lane * E;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -150,11 +151,16 @@ __global__ __launch_bounds__(256) void rope_apply_rows_kernel(RopeArgs a) {
     const int s = (int)(bs % a.S), b = (int)(bs / a.S);
     const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
     const int p = pos < 0 ? 0 : (pos >= a.rope_len ? a.rope_len - 1 : pos);
-    const int half = a.D / 2, d0 = sub * 8;
+    const int half = a.rd / 2, d0 = sub * 8;
+    const uint16_t *xr = (const uint16_t *)a.x + row * a.D;
+    const uint4 own = *(const uint4 *)(xr + d0);
+    if (d0 >= a.rd) {  // beyond the rotated part
+        *(uint4 *)((uint16_t *)a.out + row * a.D + d0) = own;
+        return;
+    }
     const bool upper = d0 >= half;
     const int j0 = upper ? d0 - half : d0;
-    const uint16_t *xr = (const uint16_t *)a.x + row * a.D;
-    const uint4 own = *(const uint4 *)(xr + d0), oth = *(const uint4 *)(xr + (upper ? d0 - half : d0 + half));
+    const uint4 oth = *(const uint4 *)(xr + (upper ? d0 - half : d0 + half));
     const uint4 sn = *(const uint4 *)((const uint16_t *)a.sin_t + (int64_t)p * half + j0);
     const uint4 cs = *(const uint4 *)((const uint16_t *)a.cos_t + (int64_t)p * half + j0);
     const uint32_t wo[4] = {own.x, own.y, own.z, own.w}, wp[4] = {oth.x, oth.y, oth.z, oth.w};
@@ -459,7 +465,15 @@ int hs_kv_quantize_int8_rope(const void *k_src, const void *v_src, int src_dtype
 int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,
                   const int32_t *positions, int32_t start_pos, void *out, int32_t B, int32_t S, int32_t H, int32_t D,
                   hs_stream_t stream) {
+    return hs_rope_apply_partial(x, dtype, rope_sin, rope_cos, rope_len, positions, start_pos, out, B, S, H, D, D, stream);
+}
+
+int hs_rope_apply_partial(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,
+                          const int32_t *positions, int32_t start_pos, void *out, int32_t B, int32_t S, int32_t H,
+                          int32_t D, int32_t rotary_dim, hs_stream_t stream) {
     using namespace hs;
+    if (rotary_dim <= 0 || rotary_dim > D || (rotary_dim % 16) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "rotary_dim %d must be a multiple of 16 in (0, head_dim %d]", rotary_dim, D);
     if ((int64_t)B * S > 0 && (!x || !out || !rope_sin || !rope_cos)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16) return fail(HS_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
     if (B < 0 || S < 0 || H <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d H=%d", B, S, H);
@@ -472,7 +486,7 @@ int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *ro
     if (rows == 0) return HS_OK;
     RopeArgs a;
     a.x = x; a.sin_t = rope_sin; a.cos_t = rope_cos; a.out = out; a.positions = positions; a.start_pos = start_pos;
-    a.rope_len = rope_len; a.B = B; a.S = S; a.H = H; a.D = D; a.dtype = dtype;
+    a.rope_len = rope_len; a.B = B; a.S = S; a.H = H; a.D = D; a.dtype = dtype; a.rd = rotary_dim;
     const bool aligned = (((uintptr_t)x | (uintptr_t)out | (uintptr_t)rope_sin | (uintptr_t)rope_cos) & 15) == 0;
     if (dtype != HS_F32 && aligned) {  // 16-bit tensors: several rows per wavefront
         const int rows_per_wg = 4 * (64 / (D / 8));

@@ -116,6 +116,12 @@ HS_API int hs_kv_quantize_int8_rope(const void *k_src, const void *v_src, int sr
 HS_API int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,
                         const int32_t *positions, int32_t start_pos, void *out,
                         int32_t B, int32_t S, int32_t H, int32_t D, hs_stream_t stream);
+/* Partial rotary embedding (Qwen3.5: the first rotary_dim = head_dim/4 elements of each head are rotated, the
+ * rest pass through; qwen3_5.rs:977-990 does narrow + rope + cat).  Tables are [rope_len, rotary_dim/2]; the
+ * rotated pairs are (d, d + rotary_dim/2).  rotary_dim is a multiple of 16, at most D; == D is hs_rope_apply. */
+HS_API int hs_rope_apply_partial(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,
+                        const int32_t *positions, int32_t start_pos, void *out,
+                        int32_t B, int32_t S, int32_t H, int32_t D, int32_t rotary_dim, hs_stream_t stream);
 
 /* FP8 e4m3fn cache with one fp32 scale per (sequence, kv-head).  Calibration computes
  * scale[b, h] = max over (s, d) |x| / 448 from the tokens given (typically the prompt);

@@ -56,6 +56,49 @@ def test_rope_apply_f32_bit_exact():
     assert np.array_equal(out.cpu().numpy().view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("D,rd", [(256, 64), (128, 32), (128, 96), (64, 16)])
+def test_partial_rotary_equals_narrow_rope_cat(D, rd):
+    """Qwen3.5 rotates the first rotary_dim elements of every head and passes the rest through
+    (qwen3_5.rs:977-990: narrow, rope, cat); tables are built for rotary_dim."""
+    r = wl.philox(720 + D + rd)
+    B, S, H, L = 2, 11, 3, 512
+    sin, cos = _tables(rd, 10000000.0, L, torch.bfloat16)
+    x = torch.from_numpy(r.standard_normal((B, S, H, D)).astype(np.float32) * 2).to(torch.bfloat16)
+    out = torch.full_like(x, float("nan"), device=DEV)
+    hb.rope_apply(x.to(DEV), sin.to(DEV), cos.to(DEV), out, None, start_pos=100, rotary_dim=rd)
+    # the element-aligned path (one row per wavefront) gives the same bits
+    buf = torch.empty(x.numel() + 1, dtype=x.dtype, device=DEV)
+    xm = buf[1:].view(x.shape)
+    xm.copy_(x)
+    out_m = torch.empty_like(out)
+    hb.rope_apply(xm, sin.to(DEV), cos.to(DEV), out_m, None, start_pos=100, rotary_dim=rd)
+    torch.cuda.synchronize()
+    pos = np.tile(100 + np.arange(S, dtype=np.int32), B)
+    xb = _bits(x).reshape(B * S, H, D)
+    want = xb.copy()
+    want[..., :rd] = orc.rope_apply_bf16(np.ascontiguousarray(xb[..., :rd]), _bits(sin), _bits(cos), pos)
+    assert np.array_equal(_bits(out).reshape(B * S, H, D), want)
+    assert torch.equal(out, out_m)
+    # fp32 tensors
+    sin32, cos32 = _tables(rd, 10000000.0, L, torch.float32)
+    x32 = x.float()
+    out32 = torch.empty_like(x32, device=DEV)
+    hb.rope_apply(x32.to(DEV), sin32.to(DEV), cos32.to(DEV), out32, None, start_pos=100, rotary_dim=rd)
+    torch.cuda.synchronize()
+    w32 = x32.numpy().reshape(B * S, H, D).copy()
+    w32[..., :rd] = orc.rope_apply_f32(np.ascontiguousarray(w32[..., :rd]), sin32.numpy(), cos32.numpy(), pos)
+    assert np.array_equal(out32.cpu().numpy().reshape(B * S, H, D).view(np.uint32), w32.view(np.uint32))
+
+
+def test_partial_rotary_rejects_bad_rotary_dim():
+    x = torch.zeros(1, 2, 2, 128, dtype=torch.bfloat16, device=DEV)
+    for rd in (24, 144):
+        sin = torch.zeros(8, rd // 2, dtype=torch.bfloat16, device=DEV)
+        with pytest.raises(hb.HsError) as e:
+            hb.rope_apply(x, sin, sin, torch.empty_like(x), None, 0, rotary_dim=rd)
+        assert e.value.code == 1 and "rotary_dim" in str(e.value)
+
+
 def test_rope_apply_rejects_positions_beyond_the_table():
     x = torch.zeros(1, 4, 2, 128, dtype=torch.bfloat16, device=DEV)
     sin = torch.zeros(6, 64, dtype=torch.bfloat16, device=DEV)
