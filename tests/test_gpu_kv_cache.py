@@ -80,10 +80,11 @@ def test_fresh_prompt_restarts_and_truncate_keeps_prefix():
     assert cache.seq_pos == 5
 
 
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("quant", [kc.INT8, kc.FP8])
-def test_attention_through_the_cache_object(quant):
+def test_attention_through_the_cache_object(quant, D):
     """update + get + attention as LlamaAttention::forward strings them together (llama.rs:605-636)."""
-    B, T, Hq, Hkv, D = 2, 150, 8, 2, 128
+    B, T, Hq, Hkv = 2, 150, 8, 2
     sig = 1.0 if quant == kc.INT8 else 0.5
     k, v = randn(9, B, T, Hkv, D) * sig, randn(10, B, T, Hkv, D) * sig
     q = randn(11, B, Hq, D)
