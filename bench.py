@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|d256-int8|d256-fp8|c3|c3-prompt|c3-fp8|c5-decode|c5-prefill]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|d256-int8|d256-fp8|c3|c3-prompt|c3-fp8|c5-decode|c5-prefill|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -161,9 +161,10 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False):
     print(json.dumps(res))
 
 
-def bench_deltanet(args, torch, hb, wl, prefill):
+def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False):
     """Config 5: gated DeltaNet, nk 16 / nv 32, dk = dv = 128.  Decode: B = 64, one token, fp32 state read and
-    written once (HBM bound).  Prefill: B = 4 x 4096 tokens through the token-by-token recurrence."""
+    written once (HBM bound).  Prefill: B = 4 x 4096 tokens in chunks of 64 on the matrix pipe (c5-prefill), or
+    through the token-by-token fp32 recurrence (c5-prefill-recurrent)."""
     dev = "cuda:0"
     nk, nv, d = 16, 32, 128
     B, T = (4, 4096) if prefill else (64, 1)
@@ -180,8 +181,14 @@ def bench_deltanet(args, torch, hb, wl, prefill):
     out = torch.empty(B, T, nv, d, dtype=torch.float32, device=dev)
     qs = 1.0 / float(np.sqrt(d))
 
+    chunked = prefill and not recurrent
+    ws = torch.empty(hb.deltanet_chunked_workspace_bytes(B, T, nv), dtype=torch.uint8, device=dev) if chunked else None
+
     def step(i):
-        hb.deltanet_forward(q, k, v, g, beta, states[i % ncopies], out, qs, False)
+        if chunked:
+            hb.deltanet_forward_chunked(q, k, v, g, beta, states[i % ncopies], out, qs, False, workspace=ws)
+        else:
+            hb.deltanet_forward(q, k, v, g, beta, states[i % ncopies], out, qs, False)
 
     for i in range(args.warmup):
         step(i)
@@ -204,11 +211,14 @@ def bench_deltanet(args, torch, hb, wl, prefill):
         "metric": "deltanet %s HBM GB/s + tokens/s, nk=16 nv=32 dk=dv=128" % ("prefill" if prefill else "decode"),
         "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32 state and arithmetic, bf16 q/k/v", "data": "synthetic (seeded, generated on device)",
-        "config": {"workload": "c5-%s: gated delta rule B=%d T=%d nk=16 nv=32 dk=dv=128, fp32 state [B,32,128,128]"
-                               % ("prefill" if prefill else "decode", B, T), "algorithmic_bytes_per_step": int(nbytes)},
+        "dtype": "f16 MFMA operands, f32 accumulation, triangular solve and state; bf16 q/k/v" if chunked else "f32 state and arithmetic, bf16 q/k/v",
+        "data": "synthetic (seeded, generated on device)",
+        "config": {"workload": "c5-%s: gated delta rule B=%d T=%d nk=16 nv=32 dk=dv=128, fp32 state [B,32,128,128]%s"
+                               % ("prefill" if prefill else "decode", B, T,
+                                  ", chunk size 64" if chunked else (", token recurrence" if prefill else "")),
+                   "algorithmic_bytes_per_step": int(nbytes)},
         "tokens_per_s": B * T / (ms * 1e-3),
-        "roofline": {"bound": "hbm", "kernel": "deltanet_prefill_kernel" if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": ("deltanet_chunk_prepare_kernel + deltanet_chunk_scan_kernel" if chunked else "deltanet_prefill_kernel") if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "avg_kernel_us": kms * 1e3},
     }
@@ -220,7 +230,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c5-decode", "c5-prefill"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c5-decode", "c5-prefill", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
@@ -254,7 +264,7 @@ def main():
         return bench_prefill(args, torch, hb, wl, C=4096 if args.workload == "c3-prompt" else 512,
                              fp8=args.workload == "c3-fp8")
     if args.workload.startswith("c5"):
-        return bench_deltanet(args, torch, hb, wl, args.workload.endswith("prefill"))
+        return bench_deltanet(args, torch, hb, wl, "prefill" in args.workload, recurrent=args.workload.endswith("recurrent"))
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)

@@ -25,7 +25,7 @@ EXPORTS = [
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
-    "hs_deltanet_prepare", "hs_deltanet_gated_norm",
+    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_forward_chunked", "hs_deltanet_chunked_workspace_bytes",
 ]
 
 
@@ -222,6 +222,28 @@ def deltanet_forward(q, k, v, g, beta, state, out, q_scale, l2norm=False):
         assert t.is_contiguous()
     check(lib().hs_deltanet_forward(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(out),
                                     B, T, nk, nv, dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)), _stream()))
+
+
+def deltanet_chunked_workspace_bytes(B, T, nv):
+    lib().hs_deltanet_chunked_workspace_bytes.restype = ctypes.c_size_t
+    return int(lib().hs_deltanet_chunked_workspace_bytes(B, T, nv))
+
+
+def deltanet_forward_chunked(q, k, v, g, beta, state, out, q_scale, l2norm=False, workspace=None):
+    """The same over a prompt in 64-token chunks on the matrix pipe (fp16 operands, fp32 accumulation and state)."""
+    import torch
+    B, T, nk, dk = q.shape
+    nv, dv = v.shape[2], v.shape[3]
+    for t in (q, k, v, g, beta, state, out):
+        assert t.is_contiguous()
+    lib().hs_deltanet_chunked_workspace_bytes.restype = ctypes.c_size_t
+    need = lib().hs_deltanet_chunked_workspace_bytes(B, T, nv)
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    check(lib().hs_deltanet_forward_chunked(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(out),
+                                            B, T, nk, nv, dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)),
+                                            _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream()))
+    return workspace
 
 
 def deltanet_prepare(mixed_qkv, conv_weight, conv_state_in, a_in, b_in, neg_a_exp, dt_bias, nk, nv, dk, dv):

@@ -1,0 +1,518 @@
+// Gated delta rule over a prompt in chunks of 64 tokens on the MFMA pipe (gfx950, wave64).
+//
+// The reference's own prefill formulation (chunked_delta_rule, qwen3_5.rs:342-498; chunk size 64): with
+// G_t the running sum of the log-decays g inside a chunk, k and q L2-normalised (q also scaled), and
+//   L[i][j] = -beta_i (k_i . k_j) exp(G_i - G_j)  for j < i (0 otherwise),      N = (I - L)^-1,
+//   U = N (v * beta),     W = N (k * beta * exp(G)),
+// a chunk that starts from the state S (dk x dv) gives
+//   V' = U - W S
+//   O  = (q * exp(G)) S + tril(q k^T * exp(G_i - G_j)) V'
+//   S <- exp(G_63) S + (k * exp(G_63 - G))^T V'.
+// It is the token recurrence S <- S e^g; S += k (v - k^T S) beta; o = q^T S regrouped, so the results differ
+// from the recurrent kernel only by rounding.
+//
+// Two kernels.  deltanet_chunk_prepare_kernel does everything that does not involve S, for all chunks of all
+// (sequence, v-head) pairs in parallel (one 512-thread workgroup per chunk): normalisation, the two 64x64
+// products on MFMA, the triangular inverse in fp32 (16x16 blocks: diagonal blocks by repeated squaring, the
+// rest by block substitution), U and W on MFMA, and writes every matrix the second kernel needs into the
+// workspace ALREADY in MFMA operand order (fp16).  deltanet_chunk_scan_kernel walks the chunks of one
+// (sequence, v-head, 64-column half of the state) in order with the state in accumulator registers: 28 MFMAs
+// per wavefront and chunk, operands straight from the workspace, S and V' exchanged between the wavefronts
+// through LDS in operand order.
+//
+// Operands are fp16 (11-bit significands; every decay factor is <= 1, so nothing overflows and what underflows
+// is negligible in absolute terms), accumulation and the state are fp32.  Against the fp32 recurrence the
+// outputs differ by about 1e-3 relative.
+//
+// MFMA layouts (v_mfma_f32_16x16x32_f16, lane l: li = l % 16, lq = l / 16): A row li / B column li hold eight
+// k-slots of group lq; C/D column li holds rows 4*lq + r.  Where one operand of a product is the accumulator
+// of an earlier one (S, V', W^T, the masked q k^T), the k-slots stand for the rows that accumulator layout
+// holds -- slots 0-3: row 4*lq + r of the even 16-row tile of a 32-row slab, slots 4-7: the same rows of the
+// odd tile -- and the other operand is read in the same order.
+#include <climits>
+
+#include "mfma_common.hpp"
+
+namespace hs {
+
+constexpr int kC = 64;               // tokens per chunk
+constexpr int kWD = 128;             // dk = dv = 128
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+
+// Workspace of one (sequence, v-head, chunk): byte offsets.  Every matrix is a list of 64-lane blocks.
+constexpr int kOffWn = 0;        // -W      A operand [token tile 4][dk slab 4][lane] 16 B
+constexpr int kOffQp = 16384;    // q e^G   A operand [token tile 4][dk slab 4][lane] 16 B
+constexpr int kOffKd = 32768;    // (k e^(G63-G))^T  A operand [dk tile 8][token slab 2][lane] 16 B
+constexpr int kOffQK = 49152;    // masked q k^T     A operand [token tile 4][token slab 2][lane] 16 B
+constexpr int kOffU = 57344;     // U       accumulator tiles [token tile 4][dv tile 8][lane] 8 B
+constexpr int kOffDecay = 73728; // exp(G63), one float
+constexpr int kUnitBytes = 73984;
+
+struct ChunkArgs {
+    const uint16_t *q, *k, *v;  // bf16 [B,T,nk,128], [B,T,nk,128], [B,T,nv,128]
+    const float *g, *beta;      // [B,T,nv]
+    float *state;               // [B,nv,128,128]
+    float *out;                 // [B,T,nv,128]
+    uint8_t *ws;
+    int32_t B, T, nk, nv, nc;
+    float q_scale;
+    int32_t l2norm;
+};
+
+__device__ __forceinline__ half8 f32x8_to_half8(const float4v &a, const float4v &b) {
+    half8 h;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        h[e] = (_Float16)a[e];
+        h[4 + e] = (_Float16)b[e];
+    }
+    return h;
+}
+
+// ------------------------------------------------------------------------------------------------ prepare
+constexpr int kPitchH = 136;  // halves per row of the row-major k / q tiles
+constexpr int kPitchT = 72;   // halves per row of the transposed k / v tiles
+constexpr int kPitchF = 68;   // floats per row of the 64x64 fp32 matrices
+constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsKT = 34816, kLdsVT = 53248, kLdsL = 71680, kLdsN = 89088,
+              kLdsF = 106496, kLdsBytes = 108032;
+
+__global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
+    _Float16 *kh = (_Float16 *)(lds + kLdsKh), *qh = (_Float16 *)(lds + kLdsQh);
+    _Float16 *KT = (_Float16 *)(lds + kLdsKT), *VT = (_Float16 *)(lds + kLdsVT);
+    float *Lm = (float *)(lds + kLdsL), *Nm = (float *)(lds + kLdsN);
+    float *P0 = (float *)(lds + kLdsKh), *P1 = (float *)(lds + kLdsQh);  // scratch once k / q row tiles are dead
+    float *gs = (float *)(lds + kLdsF), *bs = gs + 64, *Gs = gs + 128, *eG = gs + 192, *eGl = gs + 256, *be = gs + 320;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lq = lane >> 4;
+    const int64_t unit = blockIdx.x;
+    const int c = (int)(unit % a.nc);
+    const int j = (int)((unit / a.nc) % a.nv);
+    const int b = (int)(unit / ((int64_t)a.nc * a.nv));
+    const int hk = j / (a.nv / a.nk);
+    uint8_t *wsu = a.ws + unit * kUnitBytes;
+
+    // ---- 1. load 64 tokens, normalise, stage: thread = (token tt, 16 consecutive elements)
+    {
+        const int tt = tid >> 3, part = tid & 7;
+        const int t = c * kC + tt;
+        const bool valid = t < a.T;
+        float kf[16], qf[16], vf[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) kf[e] = qf[e] = vf[e] = 0.0f;
+        if (valid) {
+            const int64_t bt = (int64_t)b * a.T + t;
+            const uint16_t *kp = a.k + (bt * a.nk + hk) * kWD + 16 * part;
+            const uint16_t *qp = a.q + (bt * a.nk + hk) * kWD + 16 * part;
+            const uint16_t *vp = a.v + (bt * a.nv + j) * kWD + 16 * part;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const u32x4 kw = *(const u32x4 *)(kp + 8 * i), qw = *(const u32x4 *)(qp + 8 * i), vw = *(const u32x4 *)(vp + 8 * i);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    kf[8 * i + 2 * e] = __uint_as_float(kw[e] << 16);
+                    kf[8 * i + 2 * e + 1] = __uint_as_float(kw[e] & 0xffff0000u);
+                    qf[8 * i + 2 * e] = __uint_as_float(qw[e] << 16);
+                    qf[8 * i + 2 * e + 1] = __uint_as_float(qw[e] & 0xffff0000u);
+                    vf[8 * i + 2 * e] = __uint_as_float(vw[e] << 16);
+                    vf[8 * i + 2 * e + 1] = __uint_as_float(vw[e] & 0xffff0000u);
+                }
+            }
+        }
+        float kmul = 1.0f, qmul = a.q_scale;
+        if (a.l2norm) {
+            float sk = 0.0f, sq = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                sk += kf[e] * kf[e];
+                sq += qf[e] * qf[e];
+            }
+#pragma unroll
+            for (int o = 1; o < 8; o <<= 1) {  // the eight threads of a token are eight consecutive lanes
+                sk += __shfl_xor(sk, o, 64);
+                sq += __shfl_xor(sq, o, 64);
+            }
+            kmul = 1.0f / fmaxf(sqrtf(sk), 1e-3f);
+            qmul = a.q_scale / fmaxf(sqrtf(sq), 1e-3f);
+        }
+        half8 k8[2], q8[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const _Float16 kk = (_Float16)(kf[e] * kmul);
+            k8[e >> 3][e & 7] = kk;
+            q8[e >> 3][e & 7] = (_Float16)(qf[e] * qmul);
+            KT[(16 * part + e) * kPitchT + tt] = kk;
+            VT[(16 * part + e) * kPitchT + tt] = (_Float16)vf[e];
+        }
+        *(half8 *)&kh[tt * kPitchH + 16 * part] = k8[0];
+        *(half8 *)&kh[tt * kPitchH + 16 * part + 8] = k8[1];
+        *(half8 *)&qh[tt * kPitchH + 16 * part] = q8[0];
+        *(half8 *)&qh[tt * kPitchH + 16 * part + 8] = q8[1];
+        if (part == 0) {
+            gs[tt] = valid ? a.g[((int64_t)b * a.T + t) * a.nv + j] : 0.0f;
+            bs[tt] = valid ? a.beta[((int64_t)b * a.T + t) * a.nv + j] : 0.0f;
+        }
+    }
+    __syncthreads();
+
+    // ---- 2. running sum of g and the decay factors (wavefront 0)
+    if (wave == 0) {
+        float x = gs[lane];
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float y = __shfl_up(x, o, 64);
+            if (lane >= o) x += y;
+        }
+        const float g63 = __shfl(x, 63, 64);
+        const float e = expf(x);
+        Gs[lane] = x;
+        eG[lane] = e;
+        eGl[lane] = expf(g63 - x);
+        be[lane] = bs[lane] * e;
+        if (lane == 63) *(float *)(wsu + kOffDecay) = e;
+    }
+
+    // ---- 3. k k^T (rows i, columns j) and k q^T (rows j, columns i): wavefront w owns row tile w/2, column tiles 2(w%2), +1
+    float4v kk[2], qk[2];
+    const int mt = wave >> 1;
+    {
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+            kk[x] = (float4v){0.f, 0.f, 0.f, 0.f};
+            qk[x] = (float4v){0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const half8 ar = *(const half8 *)&kh[(16 * mt + li) * kPitchH + 32 * s + 8 * lq];
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int nt = 2 * (wave & 1) + x;
+                const half8 bk = *(const half8 *)&kh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
+                const half8 bq = *(const half8 *)&qh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
+                kk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bk, kk[x], 0, 0, 0);
+                qk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bq, qk[x], 0, 0, 0);
+            }
+        }
+    }
+    __syncthreads();  // G and the factors are visible
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        const int nt = 2 * (wave & 1) + x;
+        const int col = 16 * nt + li;
+        const float gcol = Gs[col];
+        half4v m;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = 16 * mt + 4 * lq + r;
+            // L[i = row][j = col]
+            Lm[row * kPitchF + col] = col < row ? -bs[row] * kk[x][r] * expf(Gs[row] - gcol) : 0.0f;
+            // masked q k^T: row = key j, col = query i, kept for j <= i
+            m[r] = (_Float16)(row <= col ? qk[x][r] * expf(gcol - Gs[row]) : 0.0f);
+        }
+        *(half4v *)(wsu + kOffQK + ((nt * 2 + (mt >> 1)) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
+    }
+    // q e^G as the A operand of q S: block (token tile, dk slab), lane (token li, group lq)
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
+        const int tok = 16 * (blk >> 2) + (ln & 15), d0 = 32 * (blk & 3) + 4 * (ln >> 4);
+        const half4v lo = *(const half4v *)&qh[tok * kPitchH + d0], hi = *(const half4v *)&qh[tok * kPitchH + d0 + 16];
+        const float f = eG[tok];
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            o[e] = (_Float16)((float)lo[e] * f);
+            o[4 + e] = (_Float16)((float)hi[e] * f);
+        }
+        *(half8 *)(wsu + kOffQp + (blk * 64 + ln) * 16) = o;
+    }
+    __syncthreads();  // L complete; the row-major k / q tiles are dead from here on
+
+    // ---- 4. N = (I - L)^-1 in fp32, 16x16 blocks.  128 threads per block product: thread = (row r, columns c0, c0+1).
+    {
+        const int grp = tid >> 7, r = (tid & 127) >> 3, c0 = 2 * (tid & 7);
+        auto at = [&](float *m, int ba, int bb) { return m + (16 * ba) * kPitchF + 16 * bb; };
+        // dst[r][c0..] = (add ? add : 0) + X Y
+        auto mul16 = [&](float *dst, const float *X, const float *Y, const float *add) {
+            float s0 = add ? add[r * kPitchF + c0] : 0.0f, s1 = add ? add[r * kPitchF + c0 + 1] : 0.0f;
+#pragma unroll
+            for (int k = 0; k < 16; ++k) {
+                const float xv = X[r * kPitchF + k];
+                s0 += xv * Y[k * kPitchF + c0];
+                s1 += xv * Y[k * kPitchF + c0 + 1];
+            }
+            dst[r * kPitchF + c0] = s0;
+            dst[r * kPitchF + c0 + 1] = s1;
+        };
+        // strictly upper blocks of N are zero
+        for (int e = tid; e < 6 * 256; e += 512) {
+            const int ub = e >> 8, rr = (e >> 4) & 15, cc = e & 15;
+            const int ba = ub < 3 ? 0 : (ub < 5 ? 1 : 2), bb = ub < 3 ? ub + 1 : (ub < 5 ? ub - 1 : 3);
+            at(Nm, ba, bb)[rr * kPitchF + cc] = 0.0f;
+        }
+        // diagonal blocks: N_aa = (I + L)(I + L^2)(I + L^4)(I + L^8), block a = grp
+        float *Lb = at(Lm, grp, grp), *Nb = at(Nm, grp, grp), *Pb = at(P0, grp, grp), *Qb = at(P1, grp, grp);
+        {
+            const float l0 = Lb[r * kPitchF + c0], l1 = Lb[r * kPitchF + c0 + 1];
+            Pb[r * kPitchF + c0] = l0;
+            Pb[r * kPitchF + c0 + 1] = l1;
+            Nb[r * kPitchF + c0] = l0 + (r == c0 ? 1.0f : 0.0f);
+            Nb[r * kPitchF + c0 + 1] = l1 + (r == c0 + 1 ? 1.0f : 0.0f);
+        }
+        __syncthreads();
+#pragma unroll 1
+        for (int itn = 0; itn < 3; ++itn) {
+            mul16(Qb, Pb, Pb, nullptr);  // next power
+            __syncthreads();
+            mul16(Lb, Nb, Qb, Nb);       // N (I + P^2) = N + N P^2, into the free block
+            __syncthreads();
+            float *t0 = Pb; Pb = Qb; Qb = t0;
+            float *t1 = Nb; Nb = Lb; Lb = t1;
+        }
+        // three swaps: the result sits in L's diagonal block; move it to N
+        {
+            float *dst = at(Nm, grp, grp);
+            dst[r * kPitchF + c0] = Nb[r * kPitchF + c0];
+            dst[r * kPitchF + c0 + 1] = Nb[r * kPitchF + c0 + 1];
+        }
+        __syncthreads();
+        // blocks below the diagonal by distance d: N_ab = N_aa (sum_{m=b}^{a-1} L_am N_mb)
+#pragma unroll 1
+        for (int d = 1; d < 4; ++d) {
+            const int ba = grp + d, bb = grp;  // block (ba, bb), live for ba < 4
+            if (ba < 4) {
+                float s0 = 0.0f, s1 = 0.0f;
+                for (int m = bb; m < ba; ++m) {
+                    const float *X = at(Lm, ba, m), *Y = at(Nm, m, bb);
+#pragma unroll
+                    for (int k = 0; k < 16; ++k) {
+                        const float xv = X[r * kPitchF + k];
+                        s0 += xv * Y[k * kPitchF + c0];
+                        s1 += xv * Y[k * kPitchF + c0 + 1];
+                    }
+                }
+                float *Z = at(P0, ba, bb);
+                Z[r * kPitchF + c0] = s0;
+                Z[r * kPitchF + c0 + 1] = s1;
+            }
+            __syncthreads();
+            if (ba < 4) mul16(at(Nm, ba, bb), at(Nm, ba, ba), at(P0, ba, bb), nullptr);
+            __syncthreads();
+        }
+    }
+
+    // ---- 5. W^T = (k beta e^G)^T N^T (rows dk, columns token i) and U = N (v beta) (rows token i, columns dv)
+    auto nrow = [&](int row, int s) {  // N[row][32 s + 8 lq .. +7] as eight fp16
+        const float4v x0 = *(const float4v *)&Nm[row * kPitchF + 32 * s + 8 * lq];
+        const float4v x1 = *(const float4v *)&Nm[row * kPitchF + 32 * s + 8 * lq + 4];
+        return f32x8_to_half8(x0, x1);
+    };
+    auto scaled = [&](const _Float16 *T, int row, int s, const float *f) {  // T[row][32 s + 8 lq + e] * f[32 s + 8 lq + e]
+        const half8 x = *(const half8 *)&T[row * kPitchT + 32 * s + 8 * lq];
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = (_Float16)((float)x[e] * f[32 * s + 8 * lq + e]);
+        return o;
+    };
+    {
+        const int dt = wave;  // dk tile
+        half8 ak[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) ak[s] = scaled(KT, 16 * dt + li, s, be);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+            float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+                if (32 * s <= 16 * nt + 15) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak[s], nrow(16 * nt + li, s), acc, 0, 0, 0);
+            half4v o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = (_Float16)(-acc[r]);
+            *(half4v *)(wsu + kOffWn + ((nt * 4 + (dt >> 1)) * 64 + lane) * 16 + 8 * (dt & 1)) = o;
+        }
+        const int vt = wave;  // dv tile
+        half8 bv[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) bv[s] = scaled(VT, 16 * vt + li, s, bs);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+                if (32 * s <= 16 * tt + 15) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(nrow(16 * tt + li, s), bv[s], acc, 0, 0, 0);
+            half4v o;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[r];
+            *(half4v *)(wsu + kOffU + ((tt * 8 + vt) * 64 + lane) * 8) = o;
+        }
+    }
+    // (k e^(G63 - G))^T as the A operand of the state update: block (dk tile, token slab), lane (dk li, group lq)
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+        const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
+        const int dk = 16 * (blk >> 1) + (ln & 15), t0 = 32 * (blk & 1) + 4 * (ln >> 4);
+        const half4v lo = *(const half4v *)&KT[dk * kPitchT + t0], hi = *(const half4v *)&KT[dk * kPitchT + t0 + 16];
+        half8 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            o[e] = (_Float16)((float)lo[e] * eGl[t0 + e]);
+            o[4 + e] = (_Float16)((float)hi[e] * eGl[t0 + 16 + e]);
+        }
+        *(half8 *)(wsu + kOffKd + (blk * 64 + ln) * 16) = o;
+    }
+}
+
+// --------------------------------------------------------------------------------------------------- scan
+struct ChunkOps {  // what one wavefront reads per chunk
+    u32x4 wn[4], qp[4], qk[2], kd[2][2];
+    u32x2 uu[2];
+    float decay;
+};
+
+__global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 4 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
+    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 4 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lq = lane >> 4;
+    // the two column halves of a (sequence, head) read the same workspace: give them linear ids that are congruent
+    // mod 8, so that they run on the same XCD and share its L2
+    const int p = blockIdx.x, pairs = a.B * a.nv;
+    int pair, half;
+    if ((pairs & 7) == 0) {
+        pair = (p & 7) + 8 * (p >> 4);
+        half = (p >> 3) & 1;
+    } else {
+        pair = p >> 1;
+        half = p & 1;
+    }
+    const int b = pair / a.nv, j = pair % a.nv;
+    const int tw = wave & 3, cp = wave >> 2;  // token tile (also dk slab of the owned state), column pair
+    const uint8_t *wsp = a.ws + (int64_t)pair * a.nc * kUnitBytes;
+
+    float4v S[2][2];  // [dk tile 2*tw + x][column tile 2*cp + y]
+    float *sp = a.state + ((int64_t)pair * kWD) * kWD + 64 * half + 32 * cp + li;
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int y = 0; y < 2; ++y)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) S[x][y][r] = sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y];
+
+    auto load_ops = [&](ChunkOps &o, int ci) {
+        const uint8_t *u = wsp + (int64_t)ci * kUnitBytes;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            o.wn[s] = *(const u32x4 *)(u + kOffWn + ((tw * 4 + s) * 64 + lane) * 16);
+            o.qp[s] = *(const u32x4 *)(u + kOffQp + ((tw * 4 + s) * 64 + lane) * 16);
+        }
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            o.qk[s] = *(const u32x4 *)(u + kOffQK + ((tw * 2 + s) * 64 + lane) * 16);
+#pragma unroll
+            for (int x = 0; x < 2; ++x) o.kd[x][s] = *(const u32x4 *)(u + kOffKd + (((2 * tw + x) * 2 + s) * 64 + lane) * 16);
+        }
+#pragma unroll
+        for (int y = 0; y < 2; ++y) o.uu[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + 4 * half + 2 * cp + y) * 64 + lane) * 8);
+        o.decay = *(const float *)(u + kOffDecay);
+    };
+    auto h8 = [](const u32x4 &w) { return __builtin_bit_cast(half8, w); };
+
+    ChunkOps cur, nxt;
+    load_ops(cur, 0);
+    for (int ci = 0; ci < a.nc; ++ci) {
+        if (ci + 1 < a.nc) load_ops(nxt, ci + 1);
+        // S as the B operand of W S and q S
+#pragma unroll
+        for (int y = 0; y < 2; ++y)
+            *(half8 *)(s_lds + ((tw * 4 + 2 * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
+        __syncthreads();
+        float4v vp[2], o[2];
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+            const half4v u4 = __builtin_bit_cast(half4v, cur.uu[y]);
+            vp[y] = (float4v){(float)u4[0], (float)u4[1], (float)u4[2], (float)u4[3]};
+            o[y] = (float4v){0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int y = 0; y < 2; ++y) {
+                const half8 sb = *(const half8 *)(s_lds + ((s * 4 + 2 * cp + y) * 64 + lane) * 16);
+                vp[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.wn[s]), sb, vp[y], 0, 0, 0);
+                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.qp[s]), sb, o[y], 0, 0, 0);
+            }
+        // V' (this wavefront's 16 tokens) as half of a B operand block
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+            half4v h;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) h[r] = (_Float16)vp[y][r];
+            *(half4v *)(v_lds + (((tw >> 1) * 4 + 2 * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int y = 0; y < 2; ++y) {
+#pragma unroll
+            for (int x = 0; x < 2; ++x) S[x][y] *= cur.decay;
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const half8 vb = *(const half8 *)(v_lds + ((s * 4 + 2 * cp + y) * 64 + lane) * 16);
+                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.qk[s]), vb, o[y], 0, 0, 0);
+#pragma unroll
+                for (int x = 0; x < 2; ++x) S[x][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.kd[x][s]), vb, S[x][y], 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = ci * kC + 16 * tw + 4 * lq + r;
+                if (t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + 32 * cp + 16 * y + li] = o[y][r];
+            }
+        }
+        cur = nxt;
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int y = 0; y < 2; ++y)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y] = S[x][y][r];
+}
+
+}  // namespace hs
+
+extern "C" {
+
+size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nv) {
+    if (B <= 0 || T <= 0 || nv <= 0) return 0;
+    return (size_t)B * nv * ((T + hs::kC - 1) / hs::kC) * hs::kUnitBytes;
+}
+
+int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
+                                float *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
+                                float q_scale, int l2norm, void *workspace, size_t workspace_bytes, hs_stream_t stream) {
+    using namespace hs;
+    if (B > 0 && T > 0 && (!q || !k || !v || !g || !beta || !state || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (dk != kWD || dv != kWD) return fail(HS_ERR_INVALID_ARGUMENT, "deltanet is built for dk = dv = 128, got %d x %d", dk, dv);
+    if (B < 0 || T < 0 || nk <= 0 || nv <= 0 || nv % nk != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d T=%d nk=%d nv=%d (need nv %% nk == 0)", B, T, nk, nv);
+    if (B == 0 || T == 0) return HS_OK;
+    const int64_t units = (int64_t)B * nv * ((T + kC - 1) / kC);
+    if (units > INT32_MAX || (int64_t)B * nv > (1 << 29)) return fail(HS_ERR_INVALID_ARGUMENT, "too many chunks (%lld)", (long long)units);
+    const size_t need = hs_deltanet_chunked_workspace_bytes(B, T, nv);
+    if (!workspace || workspace_bytes < need) return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if ((((uintptr_t)workspace | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "q, k, v and the workspace must be 16-byte aligned");
+    ChunkArgs a;
+    a.q = (const uint16_t *)q; a.k = (const uint16_t *)k; a.v = (const uint16_t *)v;
+    a.g = g; a.beta = beta; a.state = state; a.out = out; a.ws = (uint8_t *)workspace;
+    a.B = B; a.T = T; a.nk = nk; a.nv = nv; a.nc = (T + kC - 1) / kC; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
+    hipStream_t st = (hipStream_t)stream;
+    deltanet_chunk_prepare_kernel<<<(unsigned)units, 512, 0, st>>>(a);
+    if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
+    deltanet_chunk_scan_kernel<<<(unsigned)(2 * B * nv), 512, 0, st>>>(a);
+    return check_launch("deltanet_chunk_scan");
+}
+
+}  // extern "C"
