@@ -16,7 +16,7 @@
 // products on MFMA, the triangular inverse in fp32 (16x16 blocks: diagonal blocks by repeated squaring, the
 // rest by block substitution), U and W on MFMA, and writes every matrix the second kernel needs into the
 // workspace ALREADY in MFMA operand order (fp16).  deltanet_chunk_scan_kernel walks the chunks of one
-// (sequence, v-head, 64-column half of the state) in order with the state in accumulator registers: 28 MFMAs
+// (sequence, v-head) in order with the state in accumulator registers: 56 MFMAs
 // per wavefront and chunk, operands straight from the workspace, S and V' exchanged between the wavefronts
 // through LDS in operand order.
 //
@@ -92,7 +92,10 @@ __global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a
     const int j = (int)((unit / a.nc) % a.nv);
     const int b = (int)(unit / ((int64_t)a.nc * a.nv));
     const int hk = j / (a.nv / a.nk);
-    uint8_t *wsu = a.ws + unit * kUnitBytes;
+    // chunk-major workspace: the workgroups of the scan kernel walk the chunks in step, so what they read at one
+    // moment is one contiguous region spread over all memory channels (sequence-major, they would all sit at the
+    // same offset of regions a fixed stride apart and queue up on a few channels)
+    uint8_t *wsu = a.ws + ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kUnitBytes;
 
     // ---- 1. load 64 tokens, normalise, stage: thread = (token tt, 16 consecutive elements)
     {
@@ -365,44 +368,43 @@ __global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a
 }
 
 // --------------------------------------------------------------------------------------------------- scan
+// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for the operand prefetch of the
+// next chunk, which is issued at the top of the loop and not needed before the next iteration.
+__device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+constexpr int kYT = 4;  // 16-column tiles of the state per wavefront
+
 struct ChunkOps {  // what one wavefront reads per chunk
     u32x4 wn[4], qp[4], qk[2], kd[2][2];
-    u32x2 uu[2];
+    u32x2 uu[kYT];
     float decay;
 };
 
+// One workgroup per (sequence, v-head): every workspace byte is read once.  Wavefront w: token tile w % 4 (also the
+// 32-row dk slab of the state it owns) x column tiles 4*(w / 4) .. +3.
 __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 4 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 4 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
+    __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 8 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
+    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 8 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
-    // the two column halves of a (sequence, head) read the same workspace: give them linear ids that are congruent
-    // mod 8, so that they run on the same XCD and share its L2
-    const int p = blockIdx.x, pairs = a.B * a.nv;
-    int pair, half;
-    if ((pairs & 7) == 0) {
-        pair = (p & 7) + 8 * (p >> 4);
-        half = (p >> 3) & 1;
-    } else {
-        pair = p >> 1;
-        half = p & 1;
-    }
+    const int pair = blockIdx.x;
     const int b = pair / a.nv, j = pair % a.nv;
-    const int tw = wave & 3, cp = wave >> 2;  // token tile (also dk slab of the owned state), column pair
-    const uint8_t *wsp = a.ws + (int64_t)pair * a.nc * kUnitBytes;
+    const int tw = wave & 3, cp = wave >> 2;
+    const uint8_t *wsp = a.ws + (int64_t)pair * kUnitBytes;
+    const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
 
-    float4v S[2][2];  // [dk tile 2*tw + x][column tile 2*cp + y]
-    float *sp = a.state + ((int64_t)pair * kWD) * kWD + 64 * half + 32 * cp + li;
+    float4v S[2][kYT];  // [dk tile 2*tw + x][column tile kYT*cp + y]
+    float *sp = a.state + ((int64_t)pair * kWD) * kWD + 16 * kYT * cp + li;
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
-        for (int y = 0; y < 2; ++y)
+        for (int y = 0; y < kYT; ++y)
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[x][y][r] = sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y];
 
     auto load_ops = [&](ChunkOps &o, int ci) {
-        const uint8_t *u = wsp + (int64_t)ci * kUnitBytes;
+        const uint8_t *u = wsp + ci * chunk_stride;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             o.wn[s] = *(const u32x4 *)(u + kOffWn + ((tw * 4 + s) * 64 + lane) * 16);
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
             for (int x = 0; x < 2; ++x) o.kd[x][s] = *(const u32x4 *)(u + kOffKd + (((2 * tw + x) * 2 + s) * 64 + lane) * 16);
         }
 #pragma unroll
-        for (int y = 0; y < 2; ++y) o.uu[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + 4 * half + 2 * cp + y) * 64 + lane) * 8);
+        for (int y = 0; y < kYT; ++y) o.uu[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + kYT * cp + y) * 64 + lane) * 8);
         o.decay = *(const float *)(u + kOffDecay);
     };
     auto h8 = [](const u32x4 &w) { return __builtin_bit_cast(half8, w); };
@@ -423,15 +425,17 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
     ChunkOps cur, nxt;
     load_ops(cur, 0);
     for (int ci = 0; ci < a.nc; ++ci) {
-        if (ci + 1 < a.nc) load_ops(nxt, ci + 1);
+        // next chunk's operands (the last iteration re-reads its own: one path through the loop keeps the
+        // compiler's wait counters exact, a skipped prefetch made it wait for everything in flight)
+        load_ops(nxt, min(ci + 1, a.nc - 1));
         // S as the B operand of W S and q S
 #pragma unroll
-        for (int y = 0; y < 2; ++y)
-            *(half8 *)(s_lds + ((tw * 4 + 2 * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
-        __syncthreads();
-        float4v vp[2], o[2];
+        for (int y = 0; y < kYT; ++y)
+            *(half8 *)(s_lds + ((tw * 8 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
+        lds_sync();
+        float4v vp[kYT], o[kYT];
 #pragma unroll
-        for (int y = 0; y < 2; ++y) {
+        for (int y = 0; y < kYT; ++y) {
             const half4v u4 = __builtin_bit_cast(half4v, cur.uu[y]);
             vp[y] = (float4v){(float)u4[0], (float)u4[1], (float)u4[2], (float)u4[3]};
             o[y] = (float4v){0.f, 0.f, 0.f, 0.f};
@@ -439,27 +443,27 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int y = 0; y < 2; ++y) {
-                const half8 sb = *(const half8 *)(s_lds + ((s * 4 + 2 * cp + y) * 64 + lane) * 16);
+            for (int y = 0; y < kYT; ++y) {
+                const half8 sb = *(const half8 *)(s_lds + ((s * 8 + kYT * cp + y) * 64 + lane) * 16);
                 vp[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.wn[s]), sb, vp[y], 0, 0, 0);
                 o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.qp[s]), sb, o[y], 0, 0, 0);
             }
         // V' (this wavefront's 16 tokens) as half of a B operand block
 #pragma unroll
-        for (int y = 0; y < 2; ++y) {
+        for (int y = 0; y < kYT; ++y) {
             half4v h;
 #pragma unroll
             for (int r = 0; r < 4; ++r) h[r] = (_Float16)vp[y][r];
-            *(half4v *)(v_lds + (((tw >> 1) * 4 + 2 * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
+            *(half4v *)(v_lds + (((tw >> 1) * 8 + kYT * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
         }
-        __syncthreads();
+        lds_sync();
 #pragma unroll
-        for (int y = 0; y < 2; ++y) {
+        for (int y = 0; y < kYT; ++y) {
 #pragma unroll
             for (int x = 0; x < 2; ++x) S[x][y] *= cur.decay;
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
-                const half8 vb = *(const half8 *)(v_lds + ((s * 4 + 2 * cp + y) * 64 + lane) * 16);
+                const half8 vb = *(const half8 *)(v_lds + ((s * 8 + kYT * cp + y) * 64 + lane) * 16);
                 o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.qk[s]), vb, o[y], 0, 0, 0);
 #pragma unroll
                 for (int x = 0; x < 2; ++x) S[x][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.kd[x][s]), vb, S[x][y], 0, 0, 0);
@@ -467,7 +471,7 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = ci * kC + 16 * tw + 4 * lq + r;
-                if (t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + 32 * cp + 16 * y + li] = o[y][r];
+                if (t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 16 * (kYT * cp + y) + li] = o[y][r];
             }
         }
         cur = nxt;
@@ -475,7 +479,7 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
-        for (int y = 0; y < 2; ++y)
+        for (int y = 0; y < kYT; ++y)
 #pragma unroll
             for (int r = 0; r < 4; ++r) sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y] = S[x][y][r];
 }
@@ -511,7 +515,7 @@ int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, con
     hipStream_t st = (hipStream_t)stream;
     deltanet_chunk_prepare_kernel<<<(unsigned)units, 512, 0, st>>>(a);
     if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
-    deltanet_chunk_scan_kernel<<<(unsigned)(2 * B * nv), 512, 0, st>>>(a);
+    deltanet_chunk_scan_kernel<<<(unsigned)(B * nv), 512, 0, st>>>(a);
     return check_launch("deltanet_chunk_scan");
 }
 
