@@ -73,10 +73,16 @@ __device__ __forceinline__ half8 f32x8_to_half8(const float4v &a, const float4v 
 constexpr int kPitchH = 136;  // halves per row of the row-major k / q tiles
 constexpr int kPitchT = 72;   // halves per row of the transposed k / v tiles
 constexpr int kPitchF = 68;   // floats per row of the 64x64 fp32 matrices
-constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsKT = 34816, kLdsVT = 53248, kLdsL = 71680, kLdsN = 89088,
-              kLdsF = 106496, kLdsBytes = 108032;
+// 71 KB, two workgroups per CU.  The transposed tiles are written after the inverse, over what is dead by then
+// (the row-major tiles, their scratch aliases and L).
+constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsL = 34816, kLdsN = 52224, kLdsF = 69632, kLdsBytes = 71168;
+constexpr int kLdsKT = 0, kLdsVT = 18432;  // 2 x 18432 <= 52224
 
-__global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
+// Transposed tiles [feature d][token]: the eight-token (16-byte) pieces of a row are permuted by d / 16, so that the
+// threads of a wavefront, which write one token each for features 16 apart, hit different banks.
+__device__ __forceinline__ int tpos(int d, int tok) { return d * kPitchT + ((((tok >> 3) ^ (d >> 4)) & 7) << 3) + (tok & 7); }
+
+__global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
     _Float16 *kh = (_Float16 *)(lds + kLdsKh), *qh = (_Float16 *)(lds + kLdsQh);
     _Float16 *KT = (_Float16 *)(lds + kLdsKT), *VT = (_Float16 *)(lds + kLdsVT);
@@ -98,8 +104,9 @@ __global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a
     uint8_t *wsu = a.ws + ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kUnitBytes;
 
     // ---- 1. load 64 tokens, normalise, stage: thread = (token tt, 16 consecutive elements)
+    half8 kreg[2], vreg[2];  // this thread's k-hat and v, written transposed once the inverse is done
+    const int tt = tid >> 3, part = tid & 7;
     {
-        const int tt = tid >> 3, part = tid & 7;
         const int t = c * kC + tt;
         const bool valid = t < a.T;
         float kf[16], qf[16], vf[16];
@@ -146,9 +153,10 @@ __global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a
             const _Float16 kk = (_Float16)(kf[e] * kmul);
             k8[e >> 3][e & 7] = kk;
             q8[e >> 3][e & 7] = (_Float16)(qf[e] * qmul);
-            KT[(16 * part + e) * kPitchT + tt] = kk;
-            VT[(16 * part + e) * kPitchT + tt] = (_Float16)vf[e];
+            vreg[e >> 3][e & 7] = (_Float16)vf[e];
         }
+        kreg[0] = k8[0];
+        kreg[1] = k8[1];
         *(half8 *)&kh[tt * kPitchH + 16 * part] = k8[0];
         *(half8 *)&kh[tt * kPitchH + 16 * part + 8] = k8[1];
         *(half8 *)&qh[tt * kPitchH + 16 * part] = q8[0];
@@ -307,13 +315,19 @@ __global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a
     }
 
     // ---- 5. W^T = (k beta e^G)^T N^T (rows dk, columns token i) and U = N (v beta) (rows token i, columns dv)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        KT[tpos(16 * part + e, tt)] = kreg[e >> 3][e & 7];
+        VT[tpos(16 * part + e, tt)] = vreg[e >> 3][e & 7];
+    }
+    __syncthreads();
     auto nrow = [&](int row, int s) {  // N[row][32 s + 8 lq .. +7] as eight fp16
         const float4v x0 = *(const float4v *)&Nm[row * kPitchF + 32 * s + 8 * lq];
         const float4v x1 = *(const float4v *)&Nm[row * kPitchF + 32 * s + 8 * lq + 4];
         return f32x8_to_half8(x0, x1);
     };
     auto scaled = [&](const _Float16 *T, int row, int s, const float *f) {  // T[row][32 s + 8 lq + e] * f[32 s + 8 lq + e]
-        const half8 x = *(const half8 *)&T[row * kPitchT + 32 * s + 8 * lq];
+        const half8 x = *(const half8 *)&T[tpos(row, 32 * s + 8 * lq)];
         half8 o;
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = (_Float16)((float)x[e] * f[32 * s + 8 * lq + e]);
@@ -356,7 +370,7 @@ __global__ __launch_bounds__(512) void deltanet_chunk_prepare_kernel(ChunkArgs a
     for (int it = 0; it < 2; ++it) {
         const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
         const int dk = 16 * (blk >> 1) + (ln & 15), t0 = 32 * (blk & 1) + 4 * (ln >> 4);
-        const half4v lo = *(const half4v *)&KT[dk * kPitchT + t0], hi = *(const half4v *)&KT[dk * kPitchT + t0 + 16];
+        const half4v lo = *(const half4v *)&KT[tpos(dk, t0)], hi = *(const half4v *)&KT[tpos(dk, t0 + 16)];
         half8 o;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
