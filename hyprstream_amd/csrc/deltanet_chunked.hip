@@ -30,6 +30,7 @@
 // holds -- slots 0-3: row 4*lq + r of the even 16-row tile of a 32-row slab, slots 4-7: the same rows of the
 // odd tile -- and the other operand is read in the same order.
 #include <climits>
+#include <type_traits>
 
 #include "mfma_common.hpp"
 
@@ -387,16 +388,15 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
 __device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 constexpr int kYT = 4;  // 16-column tiles of the state per wavefront
+constexpr int kSharedBytes = kOffU;  // -W, q e^G, (k e^(G63-G))^T and the masked q k^T: what every wavefront of the workgroup reads
+static_assert(kSharedBytes == 7 * 512 * 16, "seven 16-byte pieces per thread");
 
-struct ChunkOps {  // what one wavefront reads per chunk
-    u32x4 wn[4], qp[4], qk[2], kd[2][2];
-    u32x2 uu[kYT];
-    float decay;
-};
-
-// One workgroup per (sequence, v-head): every workspace byte is read once.  Wavefront w: token tile w % 4 (also the
-// 32-row dk slab of the state it owns) x column tiles 4*(w / 4) .. +3.
+// One workgroup per (sequence, v-head): every workspace byte is requested once.  Wavefront w: token tile w % 4 (also
+// the 32-row dk slab of the state it owns) x column tiles 4*(w / 4) .. +3.  The A operands are common to the
+// wavefronts of a token tile, so the workgroup fetches them once (seven 16-byte loads per thread, one chunk
+// ahead, parked in registers) and hands them round through LDS; only U is read by the wavefront that uses it.
 __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t ops[kSharedBytes];       // this chunk's shared A operands
     __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 8 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
     __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 8 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
     const int tid = threadIdx.x, lane = tid & 63;
@@ -417,51 +417,54 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[x][y][r] = sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y];
 
-    auto load_ops = [&](ChunkOps &o, int ci) {
+    u32x4 stg[7];        // the next chunk's shared operands, in flight
+    u32x2 uu[kYT], un[kYT];
+    float decay, decay_n;
+    auto fetch = [&](int ci) {
         const uint8_t *u = wsp + ci * chunk_stride;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            o.wn[s] = *(const u32x4 *)(u + kOffWn + ((tw * 4 + s) * 64 + lane) * 16);
-            o.qp[s] = *(const u32x4 *)(u + kOffQp + ((tw * 4 + s) * 64 + lane) * 16);
-        }
+        for (int i = 0; i < 7; ++i) stg[i] = *(const u32x4 *)(u + (tid + 512 * i) * 16);
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            o.qk[s] = *(const u32x4 *)(u + kOffQK + ((tw * 2 + s) * 64 + lane) * 16);
-#pragma unroll
-            for (int x = 0; x < 2; ++x) o.kd[x][s] = *(const u32x4 *)(u + kOffKd + (((2 * tw + x) * 2 + s) * 64 + lane) * 16);
-        }
-#pragma unroll
-        for (int y = 0; y < kYT; ++y) o.uu[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + kYT * cp + y) * 64 + lane) * 8);
-        o.decay = *(const float *)(u + kOffDecay);
+        for (int y = 0; y < kYT; ++y) un[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + kYT * cp + y) * 64 + lane) * 8);
+        decay_n = *(const float *)(u + kOffDecay);
     };
-    auto h8 = [](const u32x4 &w) { return __builtin_bit_cast(half8, w); };
+    auto park = [&]() {  // registers -> LDS; the caller orders it against the readers
+#pragma unroll
+        for (int i = 0; i < 7; ++i) *(u32x4 *)(ops + (tid + 512 * i) * 16) = stg[i];
+#pragma unroll
+        for (int y = 0; y < kYT; ++y) uu[y] = un[y];
+        decay = decay_n;
+    };
+    auto opA = [&](int off, int blk) { return *(const half8 *)(ops + off + (blk * 64 + lane) * 16); };
 
-    ChunkOps cur, nxt;
-    load_ops(cur, 0);
-    for (int ci = 0; ci < a.nc; ++ci) {
-        // next chunk's operands (the last iteration re-reads its own: one path through the loop keeps the
-        // compiler's wait counters exact, a skipped prefetch made it wait for everything in flight)
-        load_ops(nxt, min(ci + 1, a.nc - 1));
+    fetch(0);
+    park();
+    // One chunk.  `guard`: the chunk may reach past T (only the last one can); full chunks store without a predicate.
+    auto step = [&](int ci, auto guard_tag) {
+        constexpr bool guard = decltype(guard_tag)::value;
+        fetch(min(ci + 1, a.nc - 1));  // the last iteration re-reads its own chunk: one path through the loop
         // S as the B operand of W S and q S
 #pragma unroll
         for (int y = 0; y < kYT; ++y)
             *(half8 *)(s_lds + ((tw * 8 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
-        lds_sync();
+        lds_sync();  // also: this chunk's operands are parked
         float4v vp[kYT], o[kYT];
 #pragma unroll
         for (int y = 0; y < kYT; ++y) {
-            const half4v u4 = __builtin_bit_cast(half4v, cur.uu[y]);
+            const half4v u4 = __builtin_bit_cast(half4v, uu[y]);
             vp[y] = (float4v){(float)u4[0], (float)u4[1], (float)u4[2], (float)u4[3]};
             o[y] = (float4v){0.f, 0.f, 0.f, 0.f};
         }
 #pragma unroll
-        for (int s = 0; s < 4; ++s)
+        for (int s = 0; s < 4; ++s) {
+            const half8 wn = opA(kOffWn, tw * 4 + s), qp = opA(kOffQp, tw * 4 + s);
 #pragma unroll
             for (int y = 0; y < kYT; ++y) {
                 const half8 sb = *(const half8 *)(s_lds + ((s * 8 + kYT * cp + y) * 64 + lane) * 16);
-                vp[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.wn[s]), sb, vp[y], 0, 0, 0);
-                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.qp[s]), sb, o[y], 0, 0, 0);
+                vp[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wn, sb, vp[y], 0, 0, 0);
+                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qp, sb, o[y], 0, 0, 0);
             }
+        }
         // V' (this wavefront's 16 tokens) as half of a B operand block
 #pragma unroll
         for (int y = 0; y < kYT; ++y) {
@@ -471,25 +474,35 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
             *(half4v *)(v_lds + (((tw >> 1) * 8 + kYT * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
         }
         lds_sync();
+        const float dec = decay;
 #pragma unroll
-        for (int y = 0; y < kYT; ++y) {
+        for (int s = 0; s < 2; ++s) {
+            const half8 qk = opA(kOffQK, tw * 2 + s), kd0 = opA(kOffKd, (2 * tw) * 2 + s), kd1 = opA(kOffKd, (2 * tw + 1) * 2 + s);
 #pragma unroll
-            for (int x = 0; x < 2; ++x) S[x][y] *= cur.decay;
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
+            for (int y = 0; y < kYT; ++y) {
+                if (s == 0) {
+                    S[0][y] *= dec;
+                    S[1][y] *= dec;
+                }
                 const half8 vb = *(const half8 *)(v_lds + ((s * 8 + kYT * cp + y) * 64 + lane) * 16);
-                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.qk[s]), vb, o[y], 0, 0, 0);
-#pragma unroll
-                for (int x = 0; x < 2; ++x) S[x][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h8(cur.kd[x][s]), vb, S[x][y], 0, 0, 0);
+                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qk, vb, o[y], 0, 0, 0);
+                S[0][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd0, vb, S[0][y], 0, 0, 0);
+                S[1][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd1, vb, S[1][y], 0, 0, 0);
             }
+        }
+#pragma unroll
+        for (int y = 0; y < kYT; ++y)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = ci * kC + 16 * tw + 4 * lq + r;
-                if (t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 16 * (kYT * cp + y) + li] = o[y][r];
+                if (!guard || t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 16 * (kYT * cp + y) + li] = o[y][r];
             }
-        }
-        cur = nxt;
-    }
+        lds_sync();  // every wavefront is done with this chunk's operands
+        park();
+    };
+    const int nfull = a.T / kC;
+    for (int ci = 0; ci < nfull; ++ci) step(ci, std::false_type());
+    if (nfull < a.nc) step(nfull, std::true_type());
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
