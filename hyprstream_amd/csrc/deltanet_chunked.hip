@@ -389,13 +389,16 @@ __device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\
 
 constexpr int kYT = 4;  // 16-column tiles of the state per wavefront
 constexpr int kSharedBytes = kOffU;  // -W, q e^G, (k e^(G63-G))^T and the masked q k^T: what every wavefront of the workgroup reads
-static_assert(kSharedBytes == 7 * 512 * 16, "seven 16-byte pieces per thread");
+constexpr int kScanThreads = 640;  // eight computing wavefronts and two that only move operands
+static_assert(kSharedBytes == 28 * 128 * 16, "28 16-byte pieces per loader thread");
 
-// One workgroup per (sequence, v-head): every workspace byte is requested once.  Wavefront w: token tile w % 4 (also
-// the 32-row dk slab of the state it owns) x column tiles 4*(w / 4) .. +3.  The A operands are common to the
-// wavefronts of a token tile, so the workgroup fetches them once (seven 16-byte loads per thread, one chunk
-// ahead, parked in registers) and hands them round through LDS; only U is read by the wavefront that uses it.
-__global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
+// One workgroup per (sequence, v-head): every workspace byte is requested once.  Wavefront w < 8: token tile w % 4
+// (also the 32-row dk slab of the state it owns) x column tiles 4*(w / 4) .. +3.  The A operands are common to the
+// wavefronts of a token tile, so they are fetched once per workgroup, one chunk ahead, and handed round through
+// LDS -- by wavefronts 8 and 9, which do nothing else: a wavefront that issues 1-KB loads waits behind the CU's
+// address unit (measured: ~2500 cycles per chunk for the 72 KB), and a computing wavefront that waits there holds
+// up every barrier of the chunk.  Only U is read by the wavefront that uses it.
+__global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(ChunkArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t ops[kSharedBytes];       // this chunk's shared A operands
     __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 8 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
     __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 8 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
@@ -408,6 +411,30 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
     const uint8_t *wsp = a.ws + (int64_t)pair * kUnitBytes;
     const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
 
+    if (wave >= 8) {  // ---- the two loader wavefronts
+        const int lt = tid - 512;
+        u32x4 stg[28];
+        auto fetch = [&](int ci) {
+            const uint8_t *u = wsp + ci * chunk_stride;
+#pragma unroll
+            for (int i = 0; i < 28; ++i) stg[i] = *(const u32x4 *)(u + (lt + 128 * i) * 16);
+        };
+        auto park = [&]() {
+#pragma unroll
+            for (int i = 0; i < 28; ++i) *(u32x4 *)(ops + (lt + 128 * i) * 16) = stg[i];
+        };
+        fetch(0);
+        park();
+        for (int ci = 0; ci < a.nc; ++ci) {
+            fetch(min(ci + 1, a.nc - 1));
+            lds_sync();  // chunk ci's operands are visible
+            lds_sync();
+            lds_sync();  // every computing wavefront is done with them
+            park();
+        }
+        return;
+    }
+
     float4v S[2][kYT];  // [dk tile 2*tw + x][column tile kYT*cp + y]
     float *sp = a.state + ((int64_t)pair * kWD) * kWD + 16 * kYT * cp + li;
 #pragma unroll
@@ -417,20 +444,15 @@ __global__ __launch_bounds__(512) void deltanet_chunk_scan_kernel(ChunkArgs a) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[x][y][r] = sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y];
 
-    u32x4 stg[7];        // the next chunk's shared operands, in flight
     u32x2 uu[kYT], un[kYT];
     float decay, decay_n;
     auto fetch = [&](int ci) {
         const uint8_t *u = wsp + ci * chunk_stride;
 #pragma unroll
-        for (int i = 0; i < 7; ++i) stg[i] = *(const u32x4 *)(u + (tid + 512 * i) * 16);
-#pragma unroll
         for (int y = 0; y < kYT; ++y) un[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + kYT * cp + y) * 64 + lane) * 8);
         decay_n = *(const float *)(u + kOffDecay);
     };
-    auto park = [&]() {  // registers -> LDS; the caller orders it against the readers
-#pragma unroll
-        for (int i = 0; i < 7; ++i) *(u32x4 *)(ops + (tid + 512 * i) * 16) = stg[i];
+    auto park = [&]() {
 #pragma unroll
         for (int y = 0; y < kYT; ++y) uu[y] = un[y];
         decay = decay_n;
@@ -542,7 +564,7 @@ int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, con
     hipStream_t st = (hipStream_t)stream;
     deltanet_chunk_prepare_kernel<<<(unsigned)units, 512, 0, st>>>(a);
     if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
-    deltanet_chunk_scan_kernel<<<(unsigned)(B * nv), 512, 0, st>>>(a);
+    deltanet_chunk_scan_kernel<<<(unsigned)(B * nv), kScanThreads, 0, st>>>(a);
     return check_launch("deltanet_chunk_scan");
 }
 
