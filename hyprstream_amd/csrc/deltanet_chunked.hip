@@ -412,25 +412,41 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
     const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
 
     if (wave >= 8) {  // ---- the two loader wavefronts
+        // Region A of `ops` (-W, q e^G: 32 KB) is read between the two barriers of a chunk, region B (the rest:
+        // 24 KB) after the second one.  So A of the next chunk is written after the second barrier, B of a chunk
+        // after its first barrier -- neither write holds anybody up -- and each is fetched a whole chunk earlier.
         const int lt = tid - 512;
-        u32x4 stg[28];
-        auto fetch = [&](int ci) {
-            const uint8_t *u = wsp + ci * chunk_stride;
+        constexpr int kA = kOffKd / (128 * 16), kB = (kSharedBytes - kOffKd) / (128 * 16);  // 16 and 12 pieces per thread
+        u32x4 sa[kA], sb[kB];
+        auto fetch_a = [&](int ci) {
+            const uint8_t *u = wsp + min(ci, a.nc - 1) * chunk_stride;
 #pragma unroll
-            for (int i = 0; i < 28; ++i) stg[i] = *(const u32x4 *)(u + (lt + 128 * i) * 16);
+            for (int i = 0; i < kA; ++i) sa[i] = *(const u32x4 *)(u + (lt + 128 * i) * 16);
         };
-        auto park = [&]() {
+        auto fetch_b = [&](int ci) {
+            const uint8_t *u = wsp + min(ci, a.nc - 1) * chunk_stride + kOffKd;
 #pragma unroll
-            for (int i = 0; i < 28; ++i) *(u32x4 *)(ops + (lt + 128 * i) * 16) = stg[i];
+            for (int i = 0; i < kB; ++i) sb[i] = *(const u32x4 *)(u + (lt + 128 * i) * 16);
         };
-        fetch(0);
-        park();
+        auto park_a = [&]() {
+#pragma unroll
+            for (int i = 0; i < kA; ++i) *(u32x4 *)(ops + (lt + 128 * i) * 16) = sa[i];
+        };
+        auto park_b = [&]() {
+#pragma unroll
+            for (int i = 0; i < kB; ++i) *(u32x4 *)(ops + kOffKd + (lt + 128 * i) * 16) = sb[i];
+        };
+        fetch_a(0);
+        fetch_b(0);
+        park_a();
+        fetch_a(1);
         for (int ci = 0; ci < a.nc; ++ci) {
-            fetch(min(ci + 1, a.nc - 1));
-            lds_sync();  // chunk ci's operands are visible
-            lds_sync();
-            lds_sync();  // every computing wavefront is done with them
-            park();
+            lds_sync();  // A of chunk ci is visible; nobody reads B of chunk ci - 1 any more
+            park_b();
+            fetch_b(ci + 1);
+            lds_sync();  // B of chunk ci is visible; nobody reads A of chunk ci any more
+            park_a();
+            fetch_a(ci + 2);
         }
         return;
     }
@@ -469,7 +485,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
 #pragma unroll
         for (int y = 0; y < kYT; ++y)
             *(half8 *)(s_lds + ((tw * 8 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
-        lds_sync();  // also: this chunk's operands are parked
+        lds_sync();  // also: the loaders have parked this chunk's -W and q e^G
         float4v vp[kYT], o[kYT];
 #pragma unroll
         for (int y = 0; y < kYT; ++y) {
@@ -519,7 +535,6 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
                 const int t = ci * kC + 16 * tw + 4 * lq + r;
                 if (!guard || t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 16 * (kYT * cp + y) + li] = o[y][r];
             }
-        lds_sync();  // every wavefront is done with this chunk's operands
         park();
     };
     const int nfull = a.T / kC;
