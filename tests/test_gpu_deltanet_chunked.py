@@ -125,3 +125,20 @@ def test_workspace_and_shape_errors():
         hb.deltanet_forward_chunked(q.repeat(1, 1, 3, 1), k.repeat(1, 1, 3, 1), v, g, beta, st, out, 1.0, True)
     assert e.value.code == hb.HS_ERR_INVALID_ARGUMENT
     torch.cuda.synchronize()
+
+
+def test_against_the_numpy_restatement_of_the_reference_chunked_form():
+    """oracle/deltanet_chunked.py follows chunked_delta_rule (qwen3_5.rs:342-498) statement by statement."""
+    from oracle import deltanet_chunked as dc
+    B, T, nk, nv = 1, 200, 2, 4
+    case = wl.deltanet_case(77, B, T, nk, nv, 128, 128)
+    s0 = (wl.philox(78).standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)
+    o, s = run(case, s0, 1 / np.sqrt(128.0), True)
+    f = wl.bf16_bits_to_f32
+    rep = nv // nk
+    qn = dc.l2_normalize(f(case["q_bits"])) / np.sqrt(128.0)
+    kn = dc.l2_normalize(f(case["k_bits"]))
+    hm = lambda x: np.repeat(x, rep, axis=2).transpose(0, 2, 1, 3)  # [B,T,nk,d] -> [B,nv,T,d]
+    wo, ws = dc.chunked_delta_rule(hm(qn), hm(kn), f(case["v_bits"]).transpose(0, 2, 1, 3), case["g"].transpose(0, 2, 1),
+                                   case["beta"].transpose(0, 2, 1), s0, dtype=np.float64)
+    check(o, s, np.asarray(wo, np.float32).transpose(0, 2, 1, 3), np.asarray(ws, np.float32), "numpy chunked form")
