@@ -290,82 +290,18 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
             dst[r * kPitchF + c0 + 1] = Nb[r * kPitchF + c0 + 1];
         }
         __syncthreads();
-        // blocks below the diagonal by distance d: N_ab = N_aa (sum_{m=b}^{a-1} L_am N_mb)
-#pragma unroll 1
-        for (int d = 1; d < 4; ++d) {
-            const int ba = grp + d, bb = grp;  // block (ba, bb), live for ba < 4
-            if (ba < 4) {
-                float s0 = 0.0f, s1 = 0.0f;
-                for (int m = bb; m < ba; ++m) {
-                    const float *X = at(Lm, ba, m), *Y = at(Nm, m, bb);
-#pragma unroll
-                    for (int k = 0; k < 16; ++k) {
-                        const float xv = X[r * kPitchF + k];
-                        s0 += xv * Y[k * kPitchF + c0];
-                        s1 += xv * Y[k * kPitchF + c0 + 1];
-                    }
-                }
-                float *Z = at(P0, ba, bb);
-                Z[r * kPitchF + c0] = s0;
-                Z[r * kPitchF + c0 + 1] = s1;
-            }
-            __syncthreads();
-            if (ba < 4) mul16(at(Nm, ba, bb), at(Nm, ba, ba), at(P0, ba, bb), nullptr);
-            __syncthreads();
-        }
     }
 
-    // ---- 5. W^T = (k beta e^G)^T N^T (rows dk, columns token i) and U = N (v beta) (rows token i, columns dv)
+    // ---- 5. X = N [v beta | k beta e^G] by block forward substitution, X_a = N_aa (R_a + sum_{m<a} L_am X_m), on
+    //         v_mfma_f32_16x16x16_f16.  A wavefront owns 32 columns (wavefronts 0-3: U, two dv tiles each; 4-7: W, the
+    //         two dk tiles of one slab) and walks the four row blocks with X_m in registers: the accumulator layout
+    //         of X_m (column li, rows 4 lq + r) is the B operand layout of the next level, so nothing is exchanged.
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
         KT[tpos(16 * part + e, tt)] = kreg[e >> 3][e & 7];
         VT[tpos(16 * part + e, tt)] = vreg[e >> 3][e & 7];
     }
     __syncthreads();
-    auto nrow = [&](int row, int s) {  // N[row][32 s + 8 lq .. +7] as eight fp16
-        const float4v x0 = *(const float4v *)&Nm[row * kPitchF + 32 * s + 8 * lq];
-        const float4v x1 = *(const float4v *)&Nm[row * kPitchF + 32 * s + 8 * lq + 4];
-        return f32x8_to_half8(x0, x1);
-    };
-    auto scaled = [&](const _Float16 *T, int row, int s, const float *f) {  // T[row][32 s + 8 lq + e] * f[32 s + 8 lq + e]
-        const half8 x = *(const half8 *)&T[tpos(row, 32 * s + 8 * lq)];
-        half8 o;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = (_Float16)((float)x[e] * f[32 * s + 8 * lq + e]);
-        return o;
-    };
-    {
-        const int dt = wave;  // dk tile
-        half8 ak[2];
-#pragma unroll
-        for (int s = 0; s < 2; ++s) ak[s] = scaled(KT, 16 * dt + li, s, be);
-#pragma unroll
-        for (int nt = 0; nt < 4; ++nt) {
-            float4v acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-                if (32 * s <= 16 * nt + 15) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ak[s], nrow(16 * nt + li, s), acc, 0, 0, 0);
-            half4v o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[r] = (_Float16)(-acc[r]);
-            *(half4v *)(wsu + kOffWn + ((nt * 4 + (dt >> 1)) * 64 + lane) * 16 + 8 * (dt & 1)) = o;
-        }
-        const int vt = wave;  // dv tile
-        half8 bv[2];
-#pragma unroll
-        for (int s = 0; s < 2; ++s) bv[s] = scaled(VT, 16 * vt + li, s, bs);
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-            float4v acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < 2; ++s)
-                if (32 * s <= 16 * tt + 15) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(nrow(16 * tt + li, s), bv[s], acc, 0, 0, 0);
-            half4v o;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) o[r] = (_Float16)acc[r];
-            *(half4v *)(wsu + kOffU + ((tt * 8 + vt) * 64 + lane) * 8) = o;
-        }
-    }
     // (k e^(G63 - G))^T as the A operand of the state update: block (dk tile, token slab), lane (dk li, group lq)
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
@@ -379,6 +315,52 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
             o[4 + e] = (_Float16)((float)hi[e] * eGl[t0 + 16 + e]);
         }
         *(half8 *)(wsu + kOffKd + (blk * 64 + ln) * 16) = o;
+    }
+    __syncthreads();  // the transposed k tile has been read for the output above: its rows may be reused below
+    {
+        const bool is_w = wave >= 4;
+        const _Float16 *T = is_w ? KT : VT;
+        const float *fac = is_w ? be : bs;
+        const int tile0 = 2 * (wave & 3);
+        auto f4h = [](const float4v &x) { return (half4v){(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]}; };
+        half4v xh[2][4];
+#pragma unroll
+        for (int ra = 0; ra < 4; ++ra) {
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int col = 16 * (tile0 + x) + li;
+                const half4v rr = *(const half4v *)&T[tpos(col, 16 * ra + 4 * lq)];
+                float4v acc;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[r] = (float)rr[r] * fac[16 * ra + 4 * lq + r];
+#pragma unroll
+                for (int m = 0; m < ra; ++m) {
+                    const half4v la = f4h(*(const float4v *)&Lm[(16 * ra + li) * kPitchF + 16 * m + 4 * lq]);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x16f16(la, xh[x][m], acc, 0, 0, 0);
+                }
+                const half4v na = f4h(*(const float4v *)&Nm[(16 * ra + li) * kPitchF + 16 * ra + 4 * lq]);
+                const float4v xa = __builtin_amdgcn_mfma_f32_16x16x16f16(na, f4h(acc), (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                xh[x][ra] = f4h(xa);
+                if (!is_w) *(half4v *)(wsu + kOffU + ((ra * 8 + tile0 + x) * 64 + lane) * 8) = xh[x][ra];
+            }
+        }
+        if (is_w) {
+            // -W as the A operand of the scan (row = token, k-slots = the slab's dk in accumulator order): element
+            // (token 4 lq + r, dk li of tile x) belongs to lane (4 lq + r) + 16 (li / 4), slot li % 4 + 4 x.  Shuffled
+            // through this wavefront's own 32 rows of the transposed k tile, which nobody reads any more.
+            uint8_t *stg = (uint8_t *)(KT + (32 * (wave & 3)) * kPitchT);
+#pragma unroll
+            for (int ra = 0; ra < 4; ++ra)
+#pragma unroll
+                for (int x = 0; x < 2; ++x)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        *(_Float16 *)(stg + (ra * 64 + 4 * lq + r + 16 * (li >> 2)) * 16 + 2 * ((li & 3) + 4 * x)) = -xh[x][ra][r];
+            __builtin_amdgcn_wave_barrier();  // LDS operations of one wavefront complete in order
+#pragma unroll
+            for (int ra = 0; ra < 4; ++ra)
+                *(u32x4 *)(wsu + kOffWn + ((ra * 4 + (wave & 3)) * 64 + lane) * 16) = *(const u32x4 *)(stg + (ra * 64 + lane) * 16);
+        }
     }
 }
 
