@@ -38,6 +38,7 @@ namespace hs {
 
 constexpr int kC = 64;               // tokens per chunk
 constexpr int kWD = 128;             // dk = dv = 128
+constexpr float kLog2eC = 1.4426950408889634f;
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
 // Workspace of one (sequence, v-head, chunk): byte offsets.  Every matrix is a list of 64-lane blocks.
@@ -219,9 +220,9 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
         for (int r = 0; r < 4; ++r) {
             const int row = 16 * mt + 4 * lq + r;
             // L[i = row][j = col]
-            Lm[row * kPitchF + col] = col < row ? -bs[row] * kk[x][r] * expf(Gs[row] - gcol) : 0.0f;
+            Lm[row * kPitchF + col] = col < row ? -bs[row] * kk[x][r] * __builtin_amdgcn_exp2f((Gs[row] - gcol) * kLog2eC) : 0.0f;
             // masked q k^T: row = key j, col = query i, kept for j <= i
-            m[r] = (_Float16)(row <= col ? qk[x][r] * expf(gcol - Gs[row]) : 0.0f);
+            m[r] = (_Float16)(row <= col ? qk[x][r] * __builtin_amdgcn_exp2f((gcol - Gs[row]) * kLog2eC) : 0.0f);
         }
         *(half4v *)(wsu + kOffQK + ((nt * 2 + (mt >> 1)) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
     }
@@ -248,22 +249,16 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
         auto at = [&](float *m, int ba, int bb) { return m + (16 * ba) * kPitchF + 16 * bb; };
         // dst[r][c0..] = (add ? add : 0) + X Y
         auto mul16 = [&](float *dst, const float *X, const float *Y, const float *add) {
-            float s0 = add ? add[r * kPitchF + c0] : 0.0f, s1 = add ? add[r * kPitchF + c0 + 1] : 0.0f;
+            typedef float float2v __attribute__((ext_vector_type(2)));
+            float2v acc = add ? *(const float2v *)&add[r * kPitchF + c0] : (float2v){0.0f, 0.0f};
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
-                const float xv = X[r * kPitchF + k];
-                s0 += xv * Y[k * kPitchF + c0];
-                s1 += xv * Y[k * kPitchF + c0 + 1];
+            for (int k4 = 0; k4 < 4; ++k4) {  // 16-byte reads of the row, 8-byte reads of the two columns
+                const float4v xv = *(const float4v *)&X[r * kPitchF + 4 * k4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc += xv[e] * *(const float2v *)&Y[(4 * k4 + e) * kPitchF + c0];
             }
-            dst[r * kPitchF + c0] = s0;
-            dst[r * kPitchF + c0 + 1] = s1;
+            *(float2v *)&dst[r * kPitchF + c0] = acc;
         };
-        // strictly upper blocks of N are zero
-        for (int e = tid; e < 6 * 256; e += 512) {
-            const int ub = e >> 8, rr = (e >> 4) & 15, cc = e & 15;
-            const int ba = ub < 3 ? 0 : (ub < 5 ? 1 : 2), bb = ub < 3 ? ub + 1 : (ub < 5 ? ub - 1 : 3);
-            at(Nm, ba, bb)[rr * kPitchF + cc] = 0.0f;
-        }
         // diagonal blocks: N_aa = (I + L)(I + L^2)(I + L^4)(I + L^8), block a = grp
         float *Lb = at(Lm, grp, grp), *Nb = at(Nm, grp, grp), *Pb = at(P0, grp, grp), *Qb = at(P1, grp, grp);
         {
