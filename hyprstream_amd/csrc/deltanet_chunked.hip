@@ -13,12 +13,12 @@
 //
 // Two kernels.  deltanet_chunk_prepare_kernel does everything that does not involve S, for all chunks of all
 // (sequence, v-head) pairs in parallel (one 512-thread workgroup per chunk): normalisation, the two 64x64
-// products on MFMA, the triangular inverse in fp32 (16x16 blocks: diagonal blocks by repeated squaring, the
-// rest by block substitution), U and W on MFMA, and writes every matrix the second kernel needs into the
-// workspace ALREADY in MFMA operand order (fp16).  deltanet_chunk_scan_kernel walks the chunks of one
-// (sequence, v-head) in order with the state in accumulator registers: 56 MFMAs
-// per wavefront and chunk, operands straight from the workspace, S and V' exchanged between the wavefronts
-// through LDS in operand order.
+// products on MFMA, the inverses of the four diagonal 16x16 blocks of I - L in fp32 (repeated squaring), then
+// [U | W] = N [v beta | k beta e^G] by block forward substitution on MFMA (the rest of N is never formed), and
+// writes every matrix the second kernel needs into the workspace ALREADY in MFMA operand order (fp16).
+// deltanet_chunk_scan_kernel walks the chunks of one (sequence, v-head) in order with the state in accumulator
+// registers: 56 MFMAs per computing wavefront and chunk, S and V' exchanged between the wavefronts through LDS
+// in operand order, the chunk's operands brought in by two wavefronts that do nothing else.
 //
 // Operands are fp16 (11-bit significands; every decay factor is <= 1, so nothing overflows and what underflows
 // is negligible in absolute terms), accumulation and the state are fp32.  Against the fp32 recurrence the
@@ -26,7 +26,7 @@
 //
 // MFMA layouts (v_mfma_f32_16x16x32_f16, lane l: li = l % 16, lq = l / 16): A row li / B column li hold eight
 // k-slots of group lq; C/D column li holds rows 4*lq + r.  Where one operand of a product is the accumulator
-// of an earlier one (S, V', W^T, the masked q k^T), the k-slots stand for the rows that accumulator layout
+// of an earlier one (S, V', the masked q k^T), the k-slots stand for the rows that accumulator layout
 // holds -- slots 0-3: row 4*lq + r of the even 16-row tile of a 32-row slab, slots 4-7: the same rows of the
 // odd tile -- and the other operand is read in the same order.
 #include <climits>
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
     }
     __syncthreads();  // L complete; the row-major k / q tiles are dead from here on
 
-    // ---- 4. N = (I - L)^-1 in fp32, 16x16 blocks.  128 threads per block product: thread = (row r, columns c0, c0+1).
+    // ---- 4. the diagonal 16x16 blocks of N = (I - L)^-1 in fp32.  128 threads per block: thread = (row r, columns c0, c0+1).
     {
         const int grp = tid >> 7, r = (tid & 127) >> 3, c0 = 2 * (tid & 7);
         auto at = [&](float *m, int ba, int bb) { return m + (16 * ba) * kPitchF + 16 * bb; };
