@@ -240,3 +240,64 @@ def test_config5_full_size_deltanet():
                                            beta[b:b + 1, :, j:j + 1].cpu().numpy(), None, 1 / np.sqrt(d), False)
         assert np.abs(out[b, :, j].cpu().numpy() - wo[0, :, 0]).max() < 1e-4
         assert np.abs(st[b, j].cpu().numpy() - ws[0, 0]).max() < 1e-4
+
+
+def test_config5_full_size_chunked_deltanet():
+    """B = 4 x 4096 tokens, chunk size 64, on the matrix pipe: sampled (sequence, head) pairs against the oracle of
+    the recurrence, the whole output against the fp32 recurrent kernel, and four calls carrying the state
+    (cut at multiples of 64) against the single call, bit for bit."""
+    nk, nv, d = 16, 32, 128
+    g = gen(wl.SEED + 55)
+    nrm = lambda x: (x / x.norm(dim=-1, keepdim=True).clamp_min(1e-3)).to(torch.bfloat16)
+    B, T = 4, 4096
+    q, k = nrm(torch.randn(B, T, nk, d, generator=g, device=DEV)), nrm(torch.randn(B, T, nk, d, generator=g, device=DEV))
+    v = torch.randn(B, T, nv, d, generator=g, device=DEV).to(torch.bfloat16)
+    gg = -torch.nn.functional.softplus(torch.randn(B, T, nv, generator=g, device=DEV))
+    beta = torch.sigmoid(torch.randn(B, T, nv, generator=g, device=DEV))
+    qs = 1 / np.sqrt(d)
+    st, out = torch.zeros(B, nv, d, d, device=DEV), torch.full((B, T, nv, d), float("nan"), device=DEV)
+    ws = hb.deltanet_forward_chunked(q, k, v, gg, beta, st, out, qs, False)
+    st2, out2 = torch.zeros(B, nv, d, d, device=DEV), torch.empty(B, T, nv, d, device=DEV)
+    for i in range(0, T, 1024):
+        o = torch.empty(B, 1024, nv, d, device=DEV)
+        hb.deltanet_forward_chunked(q[:, i:i + 1024].contiguous(), k[:, i:i + 1024].contiguous(), v[:, i:i + 1024].contiguous(),
+                                    gg[:, i:i + 1024].contiguous(), beta[:, i:i + 1024].contiguous(), st2, o, qs, False, workspace=ws)
+        out2[:, i:i + 1024] = o
+    st3, out3 = torch.zeros(B, nv, d, d, device=DEV), torch.empty(B, T, nv, d, device=DEV)
+    hb.deltanet_forward(q, k, v, gg, beta, st3, out3, qs, False)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all() and torch.equal(out, out2) and torch.equal(st, st2)
+    rel = 3e-3
+    assert float((out - out3).abs().max()) <= rel * float(out3.abs().max())
+    assert float((st - st3).abs().max()) <= rel * float(st3.abs().max())
+    for b, j in ((0, 1), (3, 30)):
+        hk = j // 2
+        wo, wst = oracle.deltanet_recurrent(q[b:b + 1, :, hk:hk + 1].float().cpu().numpy(), k[b:b + 1, :, hk:hk + 1].float().cpu().numpy(),
+                                            v[b:b + 1, :, j:j + 1].float().cpu().numpy(), gg[b:b + 1, :, j:j + 1].cpu().numpy(),
+                                            beta[b:b + 1, :, j:j + 1].cpu().numpy(), None, qs, False)
+        eo = np.abs(out[b, :, j].cpu().numpy() - wo[0, :, 0]).max()
+        es = np.abs(st[b, j].cpu().numpy() - wst[0, 0]).max()
+        assert eo <= rel * np.abs(wo).max() and es <= rel * np.abs(wst).max(), (b, j, eo, es)
+        assert eo < TOL_MAX
+
+
+def test_head_dim_256_full_size_decode():
+    """The Qwen3.5 full-attention head shape at the size of config 2: B=64, Hq 16 / Hkv 4, D 256, T 8192, int8."""
+    B, Hq, Hkv, D, T = 64, 16, 4, 256, 8192
+    g = gen(wl.SEED + 256)
+    lay, kc, vc, ks, vs, kept = fill_cache(g, B, Hkv, T, D, False, 1.0, True, keep=(7,))
+    kk, _ = kept[7]
+    wk, wks = oracle.quant_int8(kk[:, :, 1])
+    assert np.array_equal(kc[7, 1].cpu().numpy(), wk[0]) and np.array_equal(ks[7, 1, :T].cpu().numpy(), wks[0])
+    q = torch.randn(B, Hq, D, generator=g, device=DEV).to(torch.bfloat16)
+    lens = torch.randint(512, T + 1, (B,), generator=g, device=DEV, dtype=torch.int32)
+    lens[0] = T
+    out = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    assert torch.isfinite(out.float()).all()
+    sample_check(out, q, kc, vc, ks, vs, lens.cpu().numpy(), [(0, 0), (33, 3)], 4, False)
+    two = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False, phases=12)
+    assert (two.float() - out.float()).abs().max() <= 2 ** -8 * max(1.0, float(out.float().abs().max()))
+    vc.fill_(64)
+    vs.fill_(0.125)
+    const = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    assert (const.float() - 8.0).abs().max() <= 2 ** -5
