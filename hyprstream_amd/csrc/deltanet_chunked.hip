@@ -13,7 +13,7 @@
 //
 // Two kernels.  deltanet_chunk_prepare_kernel does everything that does not involve S, for all chunks of all
 // (sequence, v-head) pairs in parallel (one 512-thread workgroup per chunk): normalisation, the two 64x64
-// products on MFMA, the inverses of the four diagonal 16x16 blocks of I - L in fp32 (repeated squaring), then
+// products on MFMA, the inverses of the four diagonal 16x16 blocks of I - L (repeated squaring, one wavefront per block), then
 // [U | W] = N [v beta | k beta e^G] by block forward substitution on MFMA (the rest of N is never formed), and
 // writes every matrix the second kernel needs into the workspace ALREADY in MFMA operand order (fp16).
 // deltanet_chunk_scan_kernel walks the chunks of one (sequence, v-head) in order with the state in accumulator
@@ -243,49 +243,41 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
     }
     __syncthreads();  // L complete; the row-major k / q tiles are dead from here on
 
-    // ---- 4. the diagonal 16x16 blocks of N = (I - L)^-1 in fp32.  128 threads per block: thread = (row r, columns c0, c0+1).
-    {
-        const int grp = tid >> 7, r = (tid & 127) >> 3, c0 = 2 * (tid & 7);
-        auto at = [&](float *m, int ba, int bb) { return m + (16 * ba) * kPitchF + 16 * bb; };
-        // dst[r][c0..] = (add ? add : 0) + X Y
-        auto mul16 = [&](float *dst, const float *X, const float *Y, const float *add) {
-            typedef float float2v __attribute__((ext_vector_type(2)));
-            float2v acc = add ? *(const float2v *)&add[r * kPitchF + c0] : (float2v){0.0f, 0.0f};
+    // ---- 4. the diagonal 16x16 blocks of N = (I - L)^-1: N_aa = (I + L)(I + L^2)(I + L^4)(I + L^8) with L = L_aa.
+    //         Wavefront a < 4 does block a by itself -- six 16x16x16 products on MFMA (fp16 operands, fp32
+    //         accumulation), the matrices passing through its own LDS blocks between products (the operations of
+    //         one wavefront on LDS complete in order, so no workgroup barrier is needed until all four are done).
+    if (wave < 4) {
+        auto at = [&](float *m, int blk) { return m + (16 * blk) * kPitchF + 16 * blk; };
+        auto f4h = [](const float4v &x) { return (half4v){(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]}; };
+        // dst = (add ? add : 0) + X Y; lane (li, lq) holds rows 4 lq + r of column li of the result
+        auto mm = [&](float *dst, const float *X, const float *Y, const float *add) {
+            const half4v xa = f4h(*(const float4v *)&X[li * kPitchF + 4 * lq]);
+            float4v yb, c;
 #pragma unroll
-            for (int k4 = 0; k4 < 4; ++k4) {  // 16-byte reads of the row, 8-byte reads of the two columns
-                const float4v xv = *(const float4v *)&X[r * kPitchF + 4 * k4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc += xv[e] * *(const float2v *)&Y[(4 * k4 + e) * kPitchF + c0];
+            for (int r = 0; r < 4; ++r) {
+                yb[r] = Y[(4 * lq + r) * kPitchF + li];
+                c[r] = add ? add[(4 * lq + r) * kPitchF + li] : 0.0f;
             }
-            *(float2v *)&dst[r * kPitchF + c0] = acc;
+            c = __builtin_amdgcn_mfma_f32_16x16x16f16(xa, f4h(yb), c, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[(4 * lq + r) * kPitchF + li] = c[r];
+            __builtin_amdgcn_wave_barrier();
         };
-        // diagonal blocks: N_aa = (I + L)(I + L^2)(I + L^4)(I + L^8), block a = grp
-        float *Lb = at(Lm, grp, grp), *Nb = at(Nm, grp, grp), *Pb = at(P0, grp, grp), *Qb = at(P1, grp, grp);
-        {
-            const float l0 = Lb[r * kPitchF + c0], l1 = Lb[r * kPitchF + c0 + 1];
-            Pb[r * kPitchF + c0] = l0;
-            Pb[r * kPitchF + c0 + 1] = l1;
-            Nb[r * kPitchF + c0] = l0 + (r == c0 ? 1.0f : 0.0f);
-            Nb[r * kPitchF + c0 + 1] = l1 + (r == c0 + 1 ? 1.0f : 0.0f);
-        }
-        __syncthreads();
-#pragma unroll 1
-        for (int itn = 0; itn < 3; ++itn) {
-            mul16(Qb, Pb, Pb, nullptr);  // next power
-            __syncthreads();
-            mul16(Lb, Nb, Qb, Nb);       // N (I + P^2) = N + N P^2, into the free block
-            __syncthreads();
-            float *t0 = Pb; Pb = Qb; Qb = t0;
-            float *t1 = Nb; Nb = Lb; Lb = t1;
-        }
-        // three swaps: the result sits in L's diagonal block; move it to N
-        {
-            float *dst = at(Nm, grp, grp);
-            dst[r * kPitchF + c0] = Nb[r * kPitchF + c0];
-            dst[r * kPitchF + c0 + 1] = Nb[r * kPitchF + c0 + 1];
-        }
-        __syncthreads();
+        float *Lb = at(Lm, wave), *Nb = at(Nm, wave), *Pb = at(P0, wave), *Qb = at(P1, wave);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchF + li] = Lb[(4 * lq + r) * kPitchF + li] + (4 * lq + r == li ? 1.0f : 0.0f);
+        __builtin_amdgcn_wave_barrier();
+        mm(Qb, Lb, Lb, nullptr);  // L^2
+        mm(Lb, Nb, Qb, Nb);       // (I + L)(I + L^2), into L's block (L itself is not needed any more)
+        mm(Pb, Qb, Qb, nullptr);  // L^4
+        mm(Nb, Lb, Pb, Lb);       // ... (I + L^4)
+        mm(Qb, Pb, Pb, nullptr);  // L^8
+        mm(Lb, Nb, Qb, Nb);       // ... (I + L^8): the inverse, in L's diagonal block
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchF + li] = Lb[(4 * lq + r) * kPitchF + li];
     }
+    __syncthreads();
 
     // ---- 5. X = N [v beta | k beta e^G] by block forward substitution, X_a = N_aa (R_a + sum_{m<a} L_am X_m), on
     //         v_mfma_f32_16x16x16_f16.  A wavefront owns 32 columns (wavefronts 0-3: U, two dv tiles each; 4-7: W, the
