@@ -16,8 +16,8 @@
 // products on MFMA, the inverses of the four diagonal 16x16 blocks of I - L (repeated squaring, one wavefront per block), then
 // [U | W] = N [v beta | k beta e^G] by block forward substitution on MFMA (the rest of N is never formed), and
 // writes every matrix the second kernel needs into the workspace ALREADY in MFMA operand order (fp16).
-// deltanet_chunk_scan_kernel walks the chunks of one (sequence, v-head) in order with the state in accumulator
-// registers: 56 MFMAs per computing wavefront and chunk, S and V' exchanged between the wavefronts through LDS
+// deltanet_chunk_scan_kernel walks the chunks of one (sequence, v-head, half of the state columns) in order with
+// the state in accumulator registers: 28 MFMAs per computing wavefront and chunk, S and V' exchanged between the wavefronts through LDS
 // in operand order, the chunk's operands brought in by two wavefronts that do nothing else.
 //
 // Operands are fp16 (11-bit significands; every decay factor is <= 1, so nothing overflows and what underflows
@@ -356,25 +356,37 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
 // next chunk, which is issued at the top of the loop and not needed before the next iteration.
 __device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-constexpr int kYT = 4;  // 16-column tiles of the state per wavefront
+constexpr int kYT = 2;  // 16-column tiles of the state per wavefront (a workgroup owns 64 of the 128 columns)
 constexpr int kSharedBytes = kOffU;  // -W, q e^G, (k e^(G63-G))^T and the masked q k^T: what every wavefront of the workgroup reads
 constexpr int kScanThreads = 640;  // eight computing wavefronts and two that only move operands
 static_assert(kSharedBytes == 28 * 128 * 16, "28 16-byte pieces per loader thread");
 
-// One workgroup per (sequence, v-head): every workspace byte is requested once.  Wavefront w < 8: token tile w % 4
-// (also the 32-row dk slab of the state it owns) x column tiles 4*(w / 4) .. +3.  The A operands are common to the
+// Two workgroups per (sequence, v-head), 64 of the 128 state columns each (with one, half the CUs stay idle at
+// B x nv = 128; the second reader of the common operands finds them in the L2 it shares with the first).
+// Wavefront w < 8: token tile w % 4 (also the 32-row dk slab of the state it owns) x column tiles 2*(w / 4), +1.
+// The A operands are common to the
 // wavefronts of a token tile, so they are fetched once per workgroup, one chunk ahead, and handed round through
 // LDS -- by wavefronts 8 and 9, which do nothing else: a wavefront that issues 1-KB loads waits behind the CU's
 // address unit (measured: ~2500 cycles per chunk for the 72 KB), and a computing wavefront that waits there holds
 // up every barrier of the chunk.  Only U is read by the wavefront that uses it.
 __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(ChunkArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t ops[kSharedBytes];       // this chunk's shared A operands
-    __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 8 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 8 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
+    __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 4 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
+    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 4 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
-    const int pair = blockIdx.x;
+    // the two column halves of a (sequence, head) read the same operands: linear ids congruent mod 8 put them on
+    // the same XCD, where the second reader finds them in L2
+    const int p = blockIdx.x, pairs = a.B * a.nv;
+    int pair, half;
+    if ((pairs & 7) == 0) {
+        pair = (p & 7) + 8 * (p >> 4);
+        half = (p >> 3) & 1;
+    } else {
+        pair = p >> 1;
+        half = p & 1;
+    }
     const int b = pair / a.nv, j = pair % a.nv;
     const int tw = wave & 3, cp = wave >> 2;
     const uint8_t *wsp = a.ws + (int64_t)pair * kUnitBytes;
@@ -421,7 +433,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
     }
 
     float4v S[2][kYT];  // [dk tile 2*tw + x][column tile kYT*cp + y]
-    float *sp = a.state + ((int64_t)pair * kWD) * kWD + 16 * kYT * cp + li;
+    float *sp = a.state + ((int64_t)pair * kWD) * kWD + 64 * half + 16 * kYT * cp + li;
 #pragma unroll
     for (int x = 0; x < 2; ++x)
 #pragma unroll
@@ -434,7 +446,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
     auto fetch = [&](int ci) {
         const uint8_t *u = wsp + ci * chunk_stride;
 #pragma unroll
-        for (int y = 0; y < kYT; ++y) un[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + kYT * cp + y) * 64 + lane) * 8);
+        for (int y = 0; y < kYT; ++y) un[y] = *(const u32x2 *)(u + kOffU + ((tw * 8 + 4 * half + kYT * cp + y) * 64 + lane) * 8);
         decay_n = *(const float *)(u + kOffDecay);
     };
     auto park = [&]() {
@@ -453,7 +465,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
         // S as the B operand of W S and q S
 #pragma unroll
         for (int y = 0; y < kYT; ++y)
-            *(half8 *)(s_lds + ((tw * 8 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
+            *(half8 *)(s_lds + ((tw * 4 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
         lds_sync();  // also: the loaders have parked this chunk's -W and q e^G
         float4v vp[kYT], o[kYT];
 #pragma unroll
@@ -467,7 +479,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
             const half8 wn = opA(kOffWn, tw * 4 + s), qp = opA(kOffQp, tw * 4 + s);
 #pragma unroll
             for (int y = 0; y < kYT; ++y) {
-                const half8 sb = *(const half8 *)(s_lds + ((s * 8 + kYT * cp + y) * 64 + lane) * 16);
+                const half8 sb = *(const half8 *)(s_lds + ((s * 4 + kYT * cp + y) * 64 + lane) * 16);
                 vp[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wn, sb, vp[y], 0, 0, 0);
                 o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qp, sb, o[y], 0, 0, 0);
             }
@@ -478,7 +490,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
             half4v h;
 #pragma unroll
             for (int r = 0; r < 4; ++r) h[r] = (_Float16)vp[y][r];
-            *(half4v *)(v_lds + (((tw >> 1) * 8 + kYT * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
+            *(half4v *)(v_lds + (((tw >> 1) * 4 + kYT * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
         }
         lds_sync();
         const float dec = decay;
@@ -491,7 +503,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
                     S[0][y] *= dec;
                     S[1][y] *= dec;
                 }
-                const half8 vb = *(const half8 *)(v_lds + ((s * 8 + kYT * cp + y) * 64 + lane) * 16);
+                const half8 vb = *(const half8 *)(v_lds + ((s * 4 + kYT * cp + y) * 64 + lane) * 16);
                 o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qk, vb, o[y], 0, 0, 0);
                 S[0][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd0, vb, S[0][y], 0, 0, 0);
                 S[1][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd1, vb, S[1][y], 0, 0, 0);
@@ -502,7 +514,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = ci * kC + 16 * tw + 4 * lq + r;
-                if (!guard || t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 16 * (kYT * cp + y) + li] = o[y][r];
+                if (!guard || t < a.T) a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + 16 * (kYT * cp + y) + li] = o[y][r];
             }
         park();
     };
@@ -548,7 +560,7 @@ int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, con
     hipStream_t st = (hipStream_t)stream;
     deltanet_chunk_prepare_kernel<<<(unsigned)units, 512, 0, st>>>(a);
     if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
-    deltanet_chunk_scan_kernel<<<(unsigned)(B * nv), kScanThreads, 0, st>>>(a);
+    deltanet_chunk_scan_kernel<<<(unsigned)(2 * B * nv), kScanThreads, 0, st>>>(a);
     return check_launch("deltanet_chunk_scan");
 }
 
