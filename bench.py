@@ -182,7 +182,7 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False):
     qs = 1.0 / float(np.sqrt(d))
 
     chunked = prefill and not recurrent
-    ws = torch.empty(hb.deltanet_chunked_workspace_bytes(B, T, nv), dtype=torch.uint8, device=dev) if chunked else None
+    ws = torch.empty(hb.deltanet_chunked_workspace_bytes(B, T, nk, nv), dtype=torch.uint8, device=dev) if chunked else None
 
     def step(i):
         if chunked:

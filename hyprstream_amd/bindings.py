@@ -224,9 +224,9 @@ def deltanet_forward(q, k, v, g, beta, state, out, q_scale, l2norm=False):
                                     B, T, nk, nv, dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)), _stream()))
 
 
-def deltanet_chunked_workspace_bytes(B, T, nv):
+def deltanet_chunked_workspace_bytes(B, T, nk, nv):
     lib().hs_deltanet_chunked_workspace_bytes.restype = ctypes.c_size_t
-    return int(lib().hs_deltanet_chunked_workspace_bytes(B, T, nv))
+    return int(lib().hs_deltanet_chunked_workspace_bytes(B, T, nk, nv))
 
 
 def deltanet_forward_chunked(q, k, v, g, beta, state, out, q_scale, l2norm=False, workspace=None):
@@ -237,7 +237,7 @@ def deltanet_forward_chunked(q, k, v, g, beta, state, out, q_scale, l2norm=False
     for t in (q, k, v, g, beta, state, out):
         assert t.is_contiguous()
     lib().hs_deltanet_chunked_workspace_bytes.restype = ctypes.c_size_t
-    need = lib().hs_deltanet_chunked_workspace_bytes(B, T, nv)
+    need = lib().hs_deltanet_chunked_workspace_bytes(B, T, nk, nv)
     if workspace is None:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     check(lib().hs_deltanet_forward_chunked(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(out),

@@ -41,14 +41,22 @@ constexpr int kWD = 128;             // dk = dv = 128
 constexpr float kLog2eC = 1.4426950408889634f;
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
-// Workspace of one (sequence, v-head, chunk): byte offsets.  Every matrix is a list of 64-lane blocks.
+// Workspace, chunk-major; every matrix is a list of 64-lane blocks in MFMA operand order.
+// Per (sequence, k-head, chunk) -- the normalised q and k do not depend on the v-head, so the v-heads of a k-head
+// share them and the decays that make them "q e^G" and "(k e^(G63-G))^T" travel as two vectors per v-head:
+constexpr int kOffQh = 0;        // q (normalised, scaled)  A operand [token tile 4][dk slab 4][lane] 16 B
+constexpr int kOffKt = 16384;    // k^T (normalised)        A operand [dk tile 8][token slab 2][lane] 16 B
+constexpr int kHeadBytes = 32768;
+// Per (sequence, v-head, chunk):
 constexpr int kOffWn = 0;        // -W      A operand [token tile 4][dk slab 4][lane] 16 B
-constexpr int kOffQp = 16384;    // q e^G   A operand [token tile 4][dk slab 4][lane] 16 B
-constexpr int kOffKd = 32768;    // (k e^(G63-G))^T  A operand [dk tile 8][token slab 2][lane] 16 B
-constexpr int kOffQK = 49152;    // masked q k^T     A operand [token tile 4][token slab 2][lane] 16 B
-constexpr int kOffU = 57344;     // U       accumulator tiles [token tile 4][dv tile 8][lane] 8 B
-constexpr int kOffDecay = 73728; // exp(G63), one float
-constexpr int kUnitBytes = 73984;
+constexpr int kOffQK = 16384;    // masked q k^T     A operand [token tile 4][token slab 2][lane] 16 B
+constexpr int kOffU = 24576;     // U       accumulator tiles [token tile 4][dv tile 8][lane] 8 B
+constexpr int kOffEG = 40960;    // exp(G_t), 64 floats
+constexpr int kOffEGl = 41216;   // exp(G_63 - G_t), 64 floats
+constexpr int kOffDecay = 41472; // exp(G63), one float
+constexpr int kUnitBytes = 41728;
+// The same matrices inside the scan kernel's LDS operand buffer:
+constexpr int kOpsWn = 0, kOpsQh = 16384, kOpsKt = 32768, kOpsQK = 49152, kOpsFac = 57344, kOpsBytes = 57856;
 
 struct ChunkArgs {
     const uint16_t *q, *k, *v;  // bf16 [B,T,nk,128], [B,T,nk,128], [B,T,nv,128]
@@ -103,7 +111,11 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
     // chunk-major workspace: the workgroups of the scan kernel walk the chunks in step, so what they read at one
     // moment is one contiguous region spread over all memory channels (sequence-major, they would all sit at the
     // same offset of regions a fixed stride apart and queue up on a few channels)
-    uint8_t *wsu = a.ws + ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kUnitBytes;
+    const int rep = a.nv / a.nk;
+    uint8_t *wsc = a.ws + (int64_t)c * ((int64_t)a.B * a.nk * kHeadBytes + (int64_t)a.B * a.nv * kUnitBytes);
+    uint8_t *wsh = wsc + ((int64_t)b * a.nk + hk) * kHeadBytes;  // written by the first v-head of the k-head
+    uint8_t *wsu = wsc + (int64_t)a.B * a.nk * kHeadBytes + ((int64_t)b * a.nv + j) * kUnitBytes;
+    const bool first_of_head = j % rep == 0;
 
     // ---- 1. load 64 tokens, normalise, stage: thread = (token tt, 16 consecutive elements)
     half8 kreg[2], vreg[2];  // this thread's k-hat and v, written transposed once the inverse is done
@@ -226,20 +238,25 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
         }
         *(half4v *)(wsu + kOffQK + ((nt * 2 + (mt >> 1)) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
     }
-    // q e^G as the A operand of q S: block (token tile, dk slab), lane (token li, group lq)
+    // q as the A operand of q S: block (token tile, dk slab), lane (token li, group lq); the scan applies e^G
+    if (first_of_head) {
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
-        const int tok = 16 * (blk >> 2) + (ln & 15), d0 = 32 * (blk & 3) + 4 * (ln >> 4);
-        const half4v lo = *(const half4v *)&qh[tok * kPitchH + d0], hi = *(const half4v *)&qh[tok * kPitchH + d0 + 16];
-        const float f = eG[tok];
-        half8 o;
+        for (int it = 0; it < 2; ++it) {
+            const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
+            const int tok = 16 * (blk >> 2) + (ln & 15), d0 = 32 * (blk & 3) + 4 * (ln >> 4);
+            const half4v lo = *(const half4v *)&qh[tok * kPitchH + d0], hi = *(const half4v *)&qh[tok * kPitchH + d0 + 16];
+            half8 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            o[e] = (_Float16)((float)lo[e] * f);
-            o[4 + e] = (_Float16)((float)hi[e] * f);
+            for (int e = 0; e < 4; ++e) {
+                o[e] = lo[e];
+                o[4 + e] = hi[e];
+            }
+            *(half8 *)(wsh + kOffQh + (blk * 64 + ln) * 16) = o;
         }
-        *(half8 *)(wsu + kOffQp + (blk * 64 + ln) * 16) = o;
+    }
+    if (tid < 64) {
+        *(float *)(wsu + kOffEG + 4 * tid) = eG[tid];
+        *(float *)(wsu + kOffEGl + 4 * tid) = eGl[tid];
     }
     __syncthreads();  // L complete; the row-major k / q tiles are dead from here on
 
@@ -289,19 +306,22 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
         VT[tpos(16 * part + e, tt)] = vreg[e >> 3][e & 7];
     }
     __syncthreads();
-    // (k e^(G63 - G))^T as the A operand of the state update: block (dk tile, token slab), lane (dk li, group lq)
+    // k^T as the A operand of the state update: block (dk tile, token slab), lane (dk li, group lq); the scan
+    // applies e^(G63 - G)
+    if (first_of_head) {
 #pragma unroll
-    for (int it = 0; it < 2; ++it) {
-        const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
-        const int dk = 16 * (blk >> 1) + (ln & 15), t0 = 32 * (blk & 1) + 4 * (ln >> 4);
-        const half4v lo = *(const half4v *)&KT[tpos(dk, t0)], hi = *(const half4v *)&KT[tpos(dk, t0 + 16)];
-        half8 o;
+        for (int it = 0; it < 2; ++it) {
+            const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
+            const int dk = 16 * (blk >> 1) + (ln & 15), t0 = 32 * (blk & 1) + 4 * (ln >> 4);
+            const half4v lo = *(const half4v *)&KT[tpos(dk, t0)], hi = *(const half4v *)&KT[tpos(dk, t0 + 16)];
+            half8 o;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            o[e] = (_Float16)((float)lo[e] * eGl[t0 + e]);
-            o[4 + e] = (_Float16)((float)hi[e] * eGl[t0 + 16 + e]);
+            for (int e = 0; e < 4; ++e) {
+                o[e] = lo[e];
+                o[4 + e] = hi[e];
+            }
+            *(half8 *)(wsh + kOffKt + (blk * 64 + ln) * 16) = o;
         }
-        *(half8 *)(wsu + kOffKd + (blk * 64 + ln) * 16) = o;
     }
     __syncthreads();  // the transposed k tile has been read for the output above: its rows may be reused below
     {
@@ -357,9 +377,8 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
 __device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 constexpr int kYT = 2;  // 16-column tiles of the state per wavefront (a workgroup owns 64 of the 128 columns)
-constexpr int kSharedBytes = kOffU;  // -W, q e^G, (k e^(G63-G))^T and the masked q k^T: what every wavefront of the workgroup reads
 constexpr int kScanThreads = 640;  // eight computing wavefronts and two that only move operands
-static_assert(kSharedBytes == 28 * 128 * 16, "28 16-byte pieces per loader thread");
+static_assert(kOpsFac == 28 * 128 * 16, "28 16-byte pieces per loader thread");
 
 // Two workgroups per (sequence, v-head), 64 of the 128 state columns each (with one, half the CUs stay idle at
 // B x nv = 128; the second reader of the common operands finds them in the L2 it shares with the first).
@@ -370,7 +389,7 @@ static_assert(kSharedBytes == 28 * 128 * 16, "28 16-byte pieces per loader threa
 // address unit (measured: ~2500 cycles per chunk for the 72 KB), and a computing wavefront that waits there holds
 // up every barrier of the chunk.  Only U is read by the wavefront that uses it.
 __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(ChunkArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t ops[kSharedBytes];       // this chunk's shared A operands
+    __shared__ __attribute__((aligned(16))) uint8_t ops[kOpsBytes];          // this chunk's A operands and decay vectors
     __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 4 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
     __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 4 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
     const int tid = threadIdx.x, lane = tid & 63;
@@ -389,33 +408,41 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
     }
     const int b = pair / a.nv, j = pair % a.nv;
     const int tw = wave & 3, cp = wave >> 2;
-    const uint8_t *wsp = a.ws + (int64_t)pair * kUnitBytes;
-    const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
+    const int64_t chunk_stride = (int64_t)a.B * a.nk * kHeadBytes + (int64_t)a.B * a.nv * kUnitBytes;
+    const uint8_t *wsh = a.ws + ((int64_t)b * a.nk + j / (a.nv / a.nk)) * kHeadBytes;        // + ci * chunk_stride
+    const uint8_t *wsp = a.ws + (int64_t)a.B * a.nk * kHeadBytes + (int64_t)pair * kUnitBytes;  // + ci * chunk_stride
 
     if (wave >= 8) {  // ---- the two loader wavefronts
-        // Region A of `ops` (-W, q e^G: 32 KB) is read between the two barriers of a chunk, region B (the rest:
-        // 24 KB) after the second one.  So A of the next chunk is written after the second barrier, B of a chunk
+        // Region A of `ops` (-W, q and the decay vectors: 32.5 KB) is read between the two barriers of a chunk, region
+        // B (k^T and the masked q k^T: 24 KB) after the second one.  So A of the next chunk is written after the second barrier, B of a chunk
         // after its first barrier -- neither write holds anybody up -- and each is fetched a whole chunk earlier.
         const int lt = tid - 512;
-        constexpr int kA = kOffKd / (128 * 16), kB = (kSharedBytes - kOffKd) / (128 * 16);  // 16 and 12 pieces per thread
-        u32x4 sa[kA], sb[kB];
+        u32x4 sa[16], sb[12];
+        float fac = 0.0f;  // one of the 128 decay factors per loader thread
         auto fetch_a = [&](int ci) {
-            const uint8_t *u = wsp + min(ci, a.nc - 1) * chunk_stride;
+            const int64_t o = min(ci, a.nc - 1) * chunk_stride;
 #pragma unroll
-            for (int i = 0; i < kA; ++i) sa[i] = *(const u32x4 *)(u + (lt + 128 * i) * 16);
+            for (int i = 0; i < 8; ++i) {
+                sa[i] = *(const u32x4 *)(wsp + o + kOffWn + (lt + 128 * i) * 16);
+                sa[8 + i] = *(const u32x4 *)(wsh + o + kOffQh + (lt + 128 * i) * 16);
+            }
+            fac = *(const float *)(wsp + o + kOffEG + 4 * lt);  // e^G (64 floats) then e^(G63-G) (64 floats)
         };
         auto fetch_b = [&](int ci) {
-            const uint8_t *u = wsp + min(ci, a.nc - 1) * chunk_stride + kOffKd;
+            const int64_t o = min(ci, a.nc - 1) * chunk_stride;
 #pragma unroll
-            for (int i = 0; i < kB; ++i) sb[i] = *(const u32x4 *)(u + (lt + 128 * i) * 16);
+            for (int i = 0; i < 8; ++i) sb[i] = *(const u32x4 *)(wsh + o + kOffKt + (lt + 128 * i) * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sb[8 + i] = *(const u32x4 *)(wsp + o + kOffQK + (lt + 128 * i) * 16);
         };
         auto park_a = [&]() {
 #pragma unroll
-            for (int i = 0; i < kA; ++i) *(u32x4 *)(ops + (lt + 128 * i) * 16) = sa[i];
+            for (int i = 0; i < 16; ++i) *(u32x4 *)(ops + (lt + 128 * i) * 16) = sa[i];
+            *(float *)(ops + kOpsFac + 4 * lt) = fac;
         };
         auto park_b = [&]() {
 #pragma unroll
-            for (int i = 0; i < kB; ++i) *(u32x4 *)(ops + kOffKd + (lt + 128 * i) * 16) = sb[i];
+            for (int i = 0; i < 12; ++i) *(u32x4 *)(ops + kOpsKt + (lt + 128 * i) * 16) = sb[i];
         };
         fetch_a(0);
         fetch_b(0);
@@ -467,6 +494,14 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
         for (int y = 0; y < kYT; ++y)
             *(half8 *)(s_lds + ((tw * 4 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
         lds_sync();  // also: the loaders have parked this chunk's -W and q e^G
+        // decay vectors (region A of the buffer: read them before the second barrier).  e^G of this lane's token row;
+        // e^(G63-G) of the tokens that are the k-slots of the state update: 32 s + 4 lq + e and 32 s + 16 + 4 lq + e
+        const _Float16 eg_row = (_Float16)*(const float *)(ops + kOpsFac + 4 * (16 * tw + li));
+        half8 egl[2];
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            egl[s] = f32x8_to_half8(*(const float4v *)(ops + kOpsFac + 256 + 4 * (32 * s + 4 * lq)),
+                                    *(const float4v *)(ops + kOpsFac + 256 + 4 * (32 * s + 16 + 4 * lq)));
         float4v vp[kYT], o[kYT];
 #pragma unroll
         for (int y = 0; y < kYT; ++y) {
@@ -476,7 +511,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
         }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const half8 wn = opA(kOffWn, tw * 4 + s), qp = opA(kOffQp, tw * 4 + s);
+            const half8 wn = opA(kOpsWn, tw * 4 + s), qp = opA(kOpsQh, tw * 4 + s) * eg_row;
 #pragma unroll
             for (int y = 0; y < kYT; ++y) {
                 const half8 sb = *(const half8 *)(s_lds + ((s * 4 + kYT * cp + y) * 64 + lane) * 16);
@@ -496,7 +531,7 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
         const float dec = decay;
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            const half8 qk = opA(kOffQK, tw * 2 + s), kd0 = opA(kOffKd, (2 * tw) * 2 + s), kd1 = opA(kOffKd, (2 * tw + 1) * 2 + s);
+            const half8 qk = opA(kOpsQK, tw * 2 + s), kd0 = opA(kOpsKt, (2 * tw) * 2 + s) * egl[s], kd1 = opA(kOpsKt, (2 * tw + 1) * 2 + s) * egl[s];
 #pragma unroll
             for (int y = 0; y < kYT; ++y) {
                 if (s == 0) {
@@ -533,9 +568,9 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
 
 extern "C" {
 
-size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nv) {
-    if (B <= 0 || T <= 0 || nv <= 0) return 0;
-    return (size_t)B * nv * ((T + hs::kC - 1) / hs::kC) * hs::kUnitBytes;
+size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv) {
+    if (B <= 0 || T <= 0 || nk <= 0 || nv <= 0) return 0;
+    return (size_t)((T + hs::kC - 1) / hs::kC) * ((size_t)B * nk * hs::kHeadBytes + (size_t)B * nv * hs::kUnitBytes);
 }
 
 int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
@@ -549,7 +584,7 @@ int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, con
     if (B == 0 || T == 0) return HS_OK;
     const int64_t units = (int64_t)B * nv * ((T + kC - 1) / kC);
     if (units > INT32_MAX || (int64_t)B * nv > (1 << 29)) return fail(HS_ERR_INVALID_ARGUMENT, "too many chunks (%lld)", (long long)units);
-    const size_t need = hs_deltanet_chunked_workspace_bytes(B, T, nv);
+    const size_t need = hs_deltanet_chunked_workspace_bytes(B, T, nk, nv);
     if (!workspace || workspace_bytes < need) return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
     if ((((uintptr_t)workspace | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) != 0)
         return fail(HS_ERR_INVALID_ARGUMENT, "q, k, v and the workspace must be 16-byte aligned");

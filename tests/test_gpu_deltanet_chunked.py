@@ -115,8 +115,8 @@ def test_workspace_and_shape_errors():
     q, k, v, g, beta = _dev(case)
     st = torch.zeros(1, 2, 128, 128, device=DEV)
     out = torch.empty(1, 70, 2, 128, device=DEV)
-    need = hb.deltanet_chunked_workspace_bytes(1, 70, 2)
-    assert need == 2 * 2 * 73984
+    need = hb.deltanet_chunked_workspace_bytes(1, 70, 1, 2)
+    assert need == 2 * (1 * 32768 + 2 * 41728)  # per chunk: one k-head block and two v-head blocks
     small = torch.empty(need - 1, dtype=torch.uint8, device=DEV)
     with pytest.raises(hb.HsError) as e:
         hb.deltanet_forward_chunked(q, k, v, g, beta, st, out, 1.0, True, workspace=small)
