@@ -142,3 +142,14 @@ def test_against_the_numpy_restatement_of_the_reference_chunked_form():
     wo, ws = dc.chunked_delta_rule(hm(qn), hm(kn), f(case["v_bits"]).transpose(0, 2, 1, 3), case["g"].transpose(0, 2, 1),
                                    case["beta"].transpose(0, 2, 1), s0, dtype=np.float64)
     check(o, s, np.asarray(wo, np.float32).transpose(0, 2, 1, 3), np.asarray(ws, np.float32), "numpy chunked form")
+
+
+@pytest.mark.parametrize("nk,nv", [(2, 2), (1, 4), (3, 3)])
+def test_head_groupings(nk, nv):
+    """One, several or all v-heads per k-head (the normalised q / k operands are written once per k-head)."""
+    B, T = 3, 130
+    case = wl.deltanet_case(80 + nk + nv, B, T, nk, nv, 128, 128)
+    s0 = (wl.philox(81).standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)
+    o, s = run(case, s0, 1 / np.sqrt(128.0), True)
+    wo, ws = want(case, s0, 1 / np.sqrt(128.0), True)
+    check(o, s, wo, ws, "nk=%d nv=%d" % (nk, nv))
