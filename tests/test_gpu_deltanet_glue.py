@@ -84,16 +84,18 @@ def test_gated_norm_matches_oracle(D):
     assert _ulps(_bits(got), want).max() <= 1
 
 
-def test_layer_core_matches_the_reference_op_sequence():
+@pytest.mark.parametrize("chunked,S", [(False, 48), (True, 48), (True, 150)])
+def test_layer_core_matches_the_reference_op_sequence(chunked, S):
     """prepare -> delta rule (L2-normalised q, k; q scaled) -> gated norm, against libtorch: conv/SiLU/gates as the
-    layer does them, the decode-step recurrence iterated (qwen3_5.rs:725-751), RMSNormGated."""
-    B, S, nk, nv, dk, dv = 2, 48, 2, 4, 128, 128
+    layer does them, the decode-step recurrence iterated (qwen3_5.rs:725-751), RMSNormGated.  `chunked`: the delta
+    rule in its chunk-64 form on the matrix pipe, as the layer runs a prompt (qwen3_5.rs:753-769)."""
+    B, nk, nv, dk, dv = 2, 2, 4, 128, 128
     p = _layer_inputs(1300, B, S, nk, nv, dk, dv)
     d = {k_: v_.to(DEV) for k_, v_ in p.items()}
     q, k, v, g, beta, _ = hb.deltanet_prepare(d["x"], d["w"], d["st"], d["a"], d["b"], d["nae"], d["dtb"], nk, nv, dk, dv)
     state = torch.zeros(B, nv, dk, dv, device=DEV)
     o = torch.empty(B, S, nv, dv, device=DEV)
-    hb.deltanet_forward(q, k, v, g, beta, state, o, 1.0 / np.sqrt(dk), True)
+    (hb.deltanet_forward_chunked if chunked else hb.deltanet_forward)(q, k, v, g, beta, state, o, 1.0 / np.sqrt(dk), True)
     y = hb.deltanet_gated_norm(o, d["z"], d["nw"], 1e-6)
     torch.cuda.synchronize()
     # reference op sequence on the CPU
@@ -112,8 +114,10 @@ def test_layer_core_matches_the_reference_op_sequence():
     ro = torch.stack(outs, 1)
     want = ref.gated_rmsnorm(ro, p["z"], p["nw"], 1e-6)
     err = (y.float().cpu() - want.float()).abs()
-    assert err.max() < 3e-2 and err.mean() < 2e-3  # bf16 outputs of O(1..4): a couple of ulps where the SiLU ulp differs
-    assert (state.cpu() - st).abs().max() < 1e-3
+    # bf16 outputs of O(1..16): a couple of ulps where the SiLU ulp differs, and one ulp of the value itself (2^-7
+    # relative) where a difference far below it flips the final rounding
+    assert (err - 2.0 ** -7 * want.float().abs()).max() < 3e-2 and err.mean() < 2e-3
+    assert (state.cpu() - st).abs().max() < (3e-3 * float(st.abs().max()) if chunked else 1e-3)
 
 
 def test_prepare_rejects_aliased_state_and_nulls():
