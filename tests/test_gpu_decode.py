@@ -378,3 +378,22 @@ def test_unsupported_head_dim_is_rejected():
         hb.decode_attn(q, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, torch.tensor([64], dtype=torch.int32, device=DEV),
                        out, ws, 2, 64, 0.125)
     assert e.value.code == hb.HS_ERR_INVALID_ARGUMENT and "head_dim" in str(e.value)
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_random_shapes(seed):
+    """Seeded random batch sizes, head groupings, head_dim, lengths and cache formats against the oracle."""
+    r = np.random.default_rng(1000 + seed)
+    B = int(r.integers(1, 6))
+    Hkv = int(r.choice([1, 2, 3, 4, 8]))
+    G = int(r.choice([1, 2, 4, 5, 8, 16]))
+    D = int(r.choice([128, 256]))
+    T = int(r.integers(1, 1400))
+    fp8 = bool(r.integers(0, 2))
+    case = wl.decode_case(200 + seed, B, Hkv * G, Hkv, D, T, ragged=True, outliers=not fp8, sigma=0.5 if fp8 else 1.0)
+    if seed % 3 == 0:
+        case["seq_lens"][0] = 0  # an empty row
+    got, _ = check(case, Hkv * G, Hkv, D, fp8=fp8, cap=T + int(r.integers(0, 70)),
+                   label="random B=%d Hkv=%d G=%d D=%d T=%d fp8=%s" % (B, Hkv, G, D, T, fp8))
+    if seed % 3 == 0:
+        assert not got[0].any()
