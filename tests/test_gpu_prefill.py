@@ -298,3 +298,31 @@ def test_paged_history_matches_contiguous():
     hb.kv_dequantize(c.v_codes, c.v_scales, False, c.layout, 1, cv)
     torch.cuda.synchronize()
     assert torch.equal(dense_k, ck) and torch.equal(dense_v, cv)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_shapes(seed):
+    """Seeded random batch sizes, head groupings, history and prompt lengths and history formats against the oracle."""
+    r = np.random.default_rng(2000 + seed)
+    B = int(r.integers(1, 4))
+    Hkv = int(r.choice([1, 2, 4]))
+    G = int(r.choice([1, 2, 4, 8]))
+    hist = int(r.choice([0, 1, 63, 64, 65, 200, 333]))
+    S = int(r.integers(1, 300))
+    fp8 = bool(r.integers(0, 2)) and hist > 0
+    sigma = 0.5 if fp8 else 1.0
+    Hq = Hkv * G
+    q, k, v = make(300 + seed, B, S, Hq, Hkv, sigma=sigma)
+    c = DeviceCache(B, Hkv, hist + S + int(r.integers(0, 50)), 128, fp8=fp8)
+    kd = vd = None
+    if hist > 0:
+        _, kh, vh = make(400 + seed, B, hist, Hq, Hkv, sigma=sigma)
+        hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+        if fp8:
+            hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+        c.write(hk, hv, None, 0)
+        kc, vc, ks, vs = c.canonical(hist)
+        deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
+        kd, vd = deq(kc, ks), deq(vc, vs)
+    got = gpu_prefill(c, q, k, v, hist)
+    compare(got, oracle_prefill(q, kd, vd, k, v), "random B=%d Hkv=%d G=%d hist=%d S=%d fp8=%s" % (B, Hkv, G, hist, S, fp8))
