@@ -7,7 +7,9 @@
 //   (2) new tokens 0..=i in exact bf16,
 // which is softmax(Q K^T * scale + causal mask) V over [history | this call's K/V].
 //
-// Work split.  A 512-thread workgroup (8 wavefronts, 2 per SIMD) owns 256 (query, head) columns of
+// Work split (numbers for head_dim 128; head_dim 256 is the same template with half the columns per wavefront
+// and twice the operand blocks per key step, see PShape).  A 512-thread workgroup (8 wavefronts, 2 per SIMD)
+// owns 256 (query, head) columns of
 // one kv-head -- with G = Hq/Hkv >= 4: 64 consecutive queries x 4 query heads -- and walks the keys,
 // 64 per step.  Every step's K and V tiles are
 // converted ONCE per workgroup into ready-to-issue MFMA A operands in LDS (blocks of 64 lanes x 16 B:
@@ -34,9 +36,16 @@
 
 namespace hs {
 
-constexpr int kPD = 128;
 constexpr int kPWaves = 8;
-constexpr int kNB = 2;  // 16-column blocks per wavefront
+// head_dim 128 or 256.  What a wavefront holds is the same for both: its output tile is (16 kNB columns) x D, so
+// D = 256 halves the columns of a wavefront (and of a workgroup: 128 instead of 256) and doubles the operand
+// blocks of a key step.
+template <int D> struct PShape {
+    static constexpr int kNB = 256 / D;  // 16-column blocks per wavefront
+    static constexpr int KG = D / 32;    // K operand blocks per 16-key tile (32 d each)
+    static constexpr int VB = D / 16;    // V^T operand blocks per 32 keys (16 rows of d each)
+    static constexpr int NC = D / 128;   // 128-wide groups of d
+};
 constexpr float kPLog2e = 1.4426950408889634f;
 constexpr float kPShift = 6.0f;  // weights are carried as 2^6 * exp2(s - m_run): keeps small ones out of the fp16 subnormals
 constexpr float kMaxScale = 512.0f;  // 127 * scale stays finite in fp16; larger magnitudes saturate instead of overflowing
@@ -53,13 +62,13 @@ struct PrefillArgs {
     float scale_log2e;
 };
 
-struct alignas(16) StepTile {
-    uint8_t k[8][1024];  // block 4*u + j: K tile u (16 keys), k-group j; 64 lanes x 16 B in MFMA lane order
-    uint8_t v[8][1024];  // block bb: V^T rows d = 8*li + bb, 32 keys
+template <int D> struct alignas(16) StepTile {
+    uint8_t k[2 * PShape<D>::KG][1024];  // block KG*u + j: K tile u (16 keys), k-group j; 64 lanes x 16 B in MFMA lane order
+    uint8_t v[PShape<D>::VB][1024];      // block 8*c + bb: V^T rows d = 128*c + 8*li + bb, 32 keys
 };
 
-struct alignas(16) HistTile {
-    StepTile h[2];  // keys 0..31 and 32..63 of a 64-key step (history or new tokens)
+template <int D> struct alignas(16) HistTile {
+    StepTile<D> h[2];  // keys 0..31 and 32..63 of a 64-key step (history or new tokens)
 };
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
@@ -79,8 +88,10 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // wavefront with the vector work of the other behind a second barrier per step, or that software-pipelined
 // scores(s+1) against softmax(s) inside one wavefront, were correct but not faster than this order; steps of
 // 64 keys instead of 32 were (the per-step bookkeeping is shared by twice the MFMAs).
-template <bool FP8>  // format of the history: int8 codes with token scales, or e4m3fn codes with head scales
+template <int kPD, bool FP8>  // head_dim; format of the history: int8 codes with token scales, or e4m3fn codes with head scales
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
+    constexpr int kNB = PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
+    typedef HistTile<kPD> HistTile;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];  // two step buffers
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: wavefront-dependent branches stay uniform
@@ -121,7 +132,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     const int wv_qlast = min(S - 1, q0 + 16 * ((kNB * wave + kNB - 1) / a.HG) + 15);
     const bool wv_active = wv_q0 < S;
 
-    float4v acc[kNB][8];
+    float4v acc[kNB][VB];
     float m_run[kNB];
     float4v l_run[kNB];  // row sums, kept on the matrix pipe: ones(16x32) x P^T, every register holds the column's sum
 #pragma unroll
@@ -129,7 +140,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         m_run[nb] = -INFINITY;
         l_run[nb] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
+        for (int i = 0; i < VB; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
     }
 
     // Online softmax: raise_max() takes the blocks' step maxima (already reduced over the column).  The
@@ -148,7 +159,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
                 l_run[nb] *= alpha;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) acc[nb][i] *= alpha;
+                for (int i = 0; i < VB; ++i) acc[nb][i] *= alpha;
                 m_run[nb] = m_new;
             }
         }
@@ -162,15 +173,15 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // Q operands carry the softmax scale and log2(e): qop = fp16(q * scale * log2e * 2^-ex), so the MFMA
         // result is the score in log2 units times 2^-ex.  ex is zero unless a column's scaled |q| would leave
         // the fp16 range (then the wavefront takes the path that multiplies the scores by cq = 2^ex).
-        half8 qop[kNB][4];
+        half8 qop[kNB][KG];
         float cq[kNB];
         bool scaled = false;
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 32 * lq;
-            float qf[32], amax = 0.0f;
+            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 8 * KG * lq;
+            float qf[8 * KG], amax = 0.0f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < KG; ++i) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -179,13 +190,13 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 }
             }
 #pragma unroll
-            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qf[i]));
+            for (int i = 0; i < 8 * KG; ++i) amax = fmaxf(amax, fabsf(qf[i]));
             amax = quad_max(amax);
             int ex = 0;
             if (amax > 32768.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
             scaled |= ex != 0;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < KG; ++j)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) qop[nb][j][e] = (_Float16)ldexpf(qf[8 * j + e], -ex);
             cq[nb] = ldexpf(1.0f, ex);
@@ -212,10 +223,16 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
         const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
         const int ku4 = wave >> 1, kjp = wave & 1;
-        const int krow = 16 * ku4 + li, kcol = 32 * lq + 16 * kjp;
+        const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp;
         const uint32_t koff = krow * kPD + kcol, voff = vkey * kPD + 8 * vx;
-        u32x4 rawk = {0u, 0u, 0u, 0u};
-        u32x2 rawv[2] = {{0u, 0u}, {0u, 0u}};
+        // head_dim 256: the same lane also takes the d-halves jp + 2 (32 codes further) and the d-octet x + 16
+        u32x4 rawk[NC];
+        u32x2 rawv[NC][2];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            rawk[c] = (u32x4){0u, 0u, 0u, 0u};
+            rawv[c][0] = rawv[c][1] = (u32x2){0u, 0u};
+        }
         float rawsk = 0.0f, rawsv[2] = {0.0f, 0.0f};
         if (FP8) {  // one scale per (sequence, kv-head); the codes convert to value/256 (see e4m3_high_bytes_to_f16)
             rawsk = 256.0f * a.ks[(int64_t)b * a.Hkv + kvh];
@@ -257,9 +274,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 sv = 4u * min(vkey, last);
                 sv1 = 4u * min(vkey + 1, last);
             }
-            rawk = *(const u32x4 *)(kb + ko);
-            rawv[0] = *(const u32x2 *)(vb + vo0);
-            rawv[1] = *(const u32x2 *)(vb + vo1);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                rawk[c] = *(const u32x4 *)(kb + ko + 32 * c);
+                rawv[c][0] = *(const u32x2 *)(vb + vo0 + 128 * c);
+                rawv[c][1] = *(const u32x2 *)(vb + vo1 + 128 * c);
+            }
             if (!FP8) {
                 rawsk = *(const float *)((const uint8_t *)ksp + sk);
                 rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
@@ -281,26 +301,30 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             const float smax = FP8 ? 64.0f * kMaxScale : kMaxScale;
             const _Float16 sk = (_Float16)fminf(fk, smax);
             const _Float16 bias = (_Float16)1152.0f;
-            uint8_t *kd = t.h[ku4 >> 1].k[4 * (ku4 & 1) + 2 * kjp] + obase;
-            if (FP8) {
-                *(half8 *)kd = e4m3x8_to_f16_div256(rawk[0], rawk[1]) * sk;
-                *(half8 *)(kd + 1024) = e4m3x8_to_f16_div256(rawk[2], rawk[3]) * sk;
-            } else {
-                *(half8 *)kd = (int8x8_to_f16_biased(rawk[0], rawk[1]) - bias) * sk;
-                *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[2], rawk[3]) - bias) * sk;
-            }
             const half2v sv = {(_Float16)fminf(fv0, smax), (_Float16)fminf(fv1, smax)};
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb) {
-                const uint32_t pair = FP8 ? e4m3_pair_to_f16_div256(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3)
-                                          : int8_pair_to_f16(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3);
-                const half2v hv = __builtin_bit_cast(half2v, pair) * sv;
-                *(uint32_t *)(t.h[vhh].v[bb] + vdst) = __builtin_bit_cast(uint32_t, hv);
+            for (int c = 0; c < NC; ++c) {
+                uint8_t *kd = t.h[ku4 >> 1].k[KG * (ku4 & 1) + 2 * kjp + 4 * c] + obase;
+                if (FP8) {
+                    *(half8 *)kd = e4m3x8_to_f16_div256(rawk[c][0], rawk[c][1]) * sk;
+                    *(half8 *)(kd + 1024) = e4m3x8_to_f16_div256(rawk[c][2], rawk[c][3]) * sk;
+                } else {
+                    *(half8 *)kd = (int8x8_to_f16_biased(rawk[c][0], rawk[c][1]) - bias) * sk;
+                    *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[c][2], rawk[c][3]) - bias) * sk;
+                }
+#pragma unroll
+                for (int bb = 0; bb < 8; ++bb) {
+                    const uint32_t pair = FP8 ? e4m3_pair_to_f16_div256(rawv[c][0][bb >> 2], rawv[c][1][bb >> 2], bb & 3)
+                                              : int8_pair_to_f16(rawv[c][0][bb >> 2], rawv[c][1][bb >> 2], bb & 3);
+                    const half2v hv = __builtin_bit_cast(half2v, pair) * sv;
+                    *(uint32_t *)(t.h[vhh].v[8 * c + bb] + vdst) = __builtin_bit_cast(uint32_t, hv);
+                }
             }
         };
         float4v s[kNB][4];    // scores of the step: key block u4 = 2*half + u
         half8 pop[kNB][2];    // P^T operands per half
-        half8 kop[8], vop[8];
+        constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
+        half8 kop[KU * KG], vop[8];
         half8 ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
@@ -316,29 +340,38 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
             for (int hh = 0; hh < 2; ++hh) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) kop[i] = *(const half8 *)(t.h[hh].k[i] + obase);
+                for (int u0 = 0; u0 < 2; u0 += KU) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                    for (int i = 0; i < KU * KG; ++i) kop[i] = *(const half8 *)(t.h[hh].k[KG * u0 + i] + obase);
 #pragma unroll
-                    for (int nb = 0; nb < kNB; ++nb) s[nb][2 * hh + u] = sinit[nb];
+                    for (int u = u0; u < u0 + KU; ++u) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                        for (int nb = 0; nb < kNB; ++nb) s[nb][2 * hh + u] = sinit[nb];
 #pragma unroll
-                        for (int nb = 0; nb < kNB; ++nb)
-                            s[nb][2 * hh + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[4 * u + j], qop[nb][j], s[nb][2 * hh + u], 0, 0, 0);
+                        for (int j = 0; j < KG; ++j)
+#pragma unroll
+                            for (int nb = 0; nb < kNB; ++nb)
+                                s[nb][2 * hh + u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop[KG * (u - u0) + j], qop[nb][j], s[nb][2 * hh + u], 0, 0, 0);
+                    }
                 }
             }
         };
-        auto load_v = [&](const HistTile &t, int hh) {
+        // V^T operands of half hh, 128-wide group c of d; output() consumes them and, for head_dim 256, goes on to
+        // the second group by itself
+        auto load_v = [&](const HistTile &t, int hh, int c = 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vop[i] = *(const half8 *)(t.h[hh].v[i] + obase);
+            for (int i = 0; i < 8; ++i) vop[i] = *(const half8 *)(t.h[hh].v[8 * c + i] + obase);
         };
-        auto output = [&](int hh) {
+        auto output = [&](const HistTile &t, int hh) {
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
+            for (int c = 0; c < NC; ++c) {
+                if (c > 0) load_v(t, hh, c);
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb][hh], acc[nb][bb], 0, 0, 0);
+                for (int bb = 0; bb < 8; ++bb)
+#pragma unroll
+                    for (int nb = 0; nb < kNB; ++nb)
+                        acc[nb][8 * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb][hh], acc[nb][8 * c + bb], 0, 0, 0);
+            }
         };
         // softmax(): e = exponent of each weight (score in log2 units minus sref).  The common step only checks,
         // per lane and on the bit patterns (a positive float orders like its bits; a NaN reads as large), whether
@@ -423,9 +456,9 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 scores(t);
                 load_v(t, 0);
                 softmax(st);
-                output(0);
+                output(t, 0);
                 load_v(t, 1);
-                output(1);
+                output(t, 1);
                 if (late) {
                     if (st + 1 < nsteps) commit(htiles[(st + 1) & 1], st + 1);
                     if (st + 2 < nsteps) issue(st + 2);
@@ -444,15 +477,15 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // Q operands carry the softmax scale and log2(e), rounded back to bf16 (2^-9 relative, the precision the
         // weights are rounded to anyway), so that the MFMA result needs no multiplication; as in the history
         // phase the score accumulators start from -sref and the common step only checks for an overflow.
-        bf16x8 qop[kNB][4];
+        bf16x8 qop[kNB][KG];
         float sref[kNB];
         float4v sinit[kNB];
         int force = H > 0 ? INT_MIN : INT_MAX;  // nothing seen yet: the first step sets the reference
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 32 * lq;
+            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 8 * KG * lq;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < KG; ++j) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * j);
                 uint32_t o[4];
 #pragma unroll
@@ -479,10 +512,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
         const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
         const int ku4 = wave >> 1, kjp = wave & 1;
-        const int krow = 16 * ku4 + li, kcol = 32 * lq + 16 * kjp;
+        const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp;
         const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + 8 * vx;  // elements
-        u32x4 rawk[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-        u32x4 rawv[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+        u32x4 rawk[NC][2], rawv[NC][2];  // head_dim 256: also the d-halves jp + 2 (32 elements on) and the d-octet x + 16
+#pragma unroll
+        for (int c = 0; c < NC; ++c) rawk[c][0] = rawk[c][1] = rawv[c][0] = rawv[c][1] = (u32x4){0u, 0u, 0u, 0u};
         auto issue = [&](int step) {
             const int t0 = step * kNStep;
             const uint16_t *kp, *vp0, *vp1;
@@ -496,18 +530,24 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 vp0 = vnb + (int64_t)min(t0 + vkey, S - 1) * rstride + 8 * vx;
                 vp1 = vnb + (int64_t)min(t0 + vkey + 1, S - 1) * rstride + 8 * vx;
             }
-            rawk[0] = *(const u32x4 *)kp;
-            rawk[1] = *(const u32x4 *)(kp + 8);
-            rawv[0] = *(const u32x4 *)vp0;
-            rawv[1] = *(const u32x4 *)vp1;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                rawk[c][0] = *(const u32x4 *)(kp + 32 * c);
+                rawk[c][1] = *(const u32x4 *)(kp + 32 * c + 8);
+                rawv[c][0] = *(const u32x4 *)(vp0 + 128 * c);
+                rawv[c][1] = *(const u32x4 *)(vp1 + 128 * c);
+            }
         };
         auto commit = [&](HistTile &t) {
-            uint8_t *kd = t.h[ku4 >> 1].k[4 * (ku4 & 1) + 2 * kjp] + obase;
-            *(u32x4 *)kd = rawk[0];
-            *(u32x4 *)(kd + 1024) = rawk[1];
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
-                *(uint32_t *)(t.h[vhh].v[bb] + vdst) = pick_halves(rawv[0][bb >> 1], rawv[1][bb >> 1], bb & 1);
+            for (int c = 0; c < NC; ++c) {
+                uint8_t *kd = t.h[ku4 >> 1].k[KG * (ku4 & 1) + 2 * kjp + 4 * c] + obase;
+                *(u32x4 *)kd = rawk[c][0];
+                *(u32x4 *)(kd + 1024) = rawk[c][1];
+#pragma unroll
+                for (int bb = 0; bb < 8; ++bb)
+                    *(uint32_t *)(t.h[vhh].v[8 * c + bb] + vdst) = pick_halves(rawv[c][0][bb >> 1], rawv[c][1][bb >> 1], bb & 1);
+            }
         };
         float4v s[kNB][4];
         bf16x8 pop[kNB][2];
@@ -516,7 +556,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             if (!wv_active || step * kNStep > wv_qlast) return 0;
             return step * kNStep + 32 > wv_qlast ? 1 : 2;
         };
-        bf16x8 kop[8], vop[8], ones;
+        constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
+        bf16x8 kop[KU * KG], vop[8], ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
         auto scores = [&](const HistTile &t, int nh) {
@@ -524,29 +565,36 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             for (int hh = 0; hh < 2; ++hh) {
                 if (hh >= nh) break;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) kop[i] = *(const bf16x8 *)(t.h[hh].k[i] + obase);
+                for (int u0 = 0; u0 < 2; u0 += KU) {
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
+                    for (int i = 0; i < KU * KG; ++i) kop[i] = *(const bf16x8 *)(t.h[hh].k[KG * u0 + i] + obase);
 #pragma unroll
-                    for (int nb = 0; nb < kNB; ++nb) s[nb][2 * hh + u] = sinit[nb];
+                    for (int u = u0; u < u0 + KU; ++u) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                        for (int nb = 0; nb < kNB; ++nb) s[nb][2 * hh + u] = sinit[nb];
 #pragma unroll
-                        for (int nb = 0; nb < kNB; ++nb)
-                            s[nb][2 * hh + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[4 * u + j], qop[nb][j], s[nb][2 * hh + u], 0, 0, 0);
+                        for (int j = 0; j < KG; ++j)
+#pragma unroll
+                            for (int nb = 0; nb < kNB; ++nb)
+                                s[nb][2 * hh + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[KG * (u - u0) + j], qop[nb][j], s[nb][2 * hh + u], 0, 0, 0);
+                    }
                 }
             }
         };
-        auto load_v = [&](const HistTile &t, int hh) {
+        auto load_v = [&](const HistTile &t, int hh, int c = 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[i] + obase);
+            for (int i = 0; i < 8; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[8 * c + i] + obase);
         };
-        auto output = [&](int hh) {
+        auto output = [&](const HistTile &t, int hh) {
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
+            for (int c = 0; c < NC; ++c) {
+                if (c > 0) load_v(t, hh, c);
 #pragma unroll
-                for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb][hh], acc[nb][bb], 0, 0, 0);
+                for (int bb = 0; bb < 8; ++bb)
+#pragma unroll
+                    for (int nb = 0; nb < kNB; ++nb)
+                        acc[nb][8 * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb][hh], acc[nb][8 * c + bb], 0, 0, 0);
+            }
         };
         auto softmax = [&](int step, int nh) {
             const int t0 = step * kNStep;
@@ -616,10 +664,10 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 scores(t, nh);
                 load_v(t, 0);
                 softmax(st, nh);
-                output(0);
+                output(t, 0);
                 if (nh > 1) {
                     load_v(t, 1);
-                    output(1);
+                    output(t, 1);
                 }
             }
             lds_barrier();
@@ -634,12 +682,14 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const float inv = 1.0f / l;
         uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kPD + 32 * lq;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            u32x4 w;
+        for (int c = 0; c < NC; ++c)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(acc[nb][2 * e][r] * inv, acc[nb][2 * e + 1][r] * inv);
-            *(u32x4 *)(op + 8 * r) = w;
-        }
+            for (int r = 0; r < 4; ++r) {  // acc[8c + bb][r] is d = 128 c + 32 lq + 8 r + bb
+                u32x4 w;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(acc[nb][8 * c + 2 * e][r] * inv, acc[nb][8 * c + 2 * e + 1][r] * inv);
+                *(u32x4 *)(op + 128 * c + 8 * r) = w;
+            }
     }
 }
 
@@ -663,7 +713,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
                           int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale,
                           int quantize_on_write, hs_stream_t stream) {
     if (int rc = validate_layout(layout, B, S, Hkv, D, !fp8)) return rc;
-    if (D != kPD) return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 128, got %d", D);
+    if (D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 128 and 256, got %d", D);
     const bool empty = B == 0 || S == 0;  // an empty problem may come with null pointers (an empty tensor has none)
     if (!empty && (!q || !k_new || !v_new || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if ((hist_len > 0 || quantize_on_write) && (!k_codes || !v_codes || !k_scales || !v_scales))
@@ -690,13 +740,18 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
     a.HG = G >= 4 ? 4 : G;
     a.scale_log2e = softmax_scale * kPLog2e;
-    const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
+    const int q_per_wg = 16 * ((256 / D) * kPWaves / a.HG);
     dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * (G / a.HG), B);
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
-    if (fp8) prefill_attn_kernel<true><<<grid, 512, 0, st>>>(a);
-    else prefill_attn_kernel<false><<<grid, 512, 0, st>>>(a);
+    if (D == 128) {
+        if (fp8) prefill_attn_kernel<128, true><<<grid, 512, 0, st>>>(a);
+        else prefill_attn_kernel<128, false><<<grid, 512, 0, st>>>(a);
+    } else {
+        if (fp8) prefill_attn_kernel<256, true><<<grid, 512, 0, st>>>(a);
+        else prefill_attn_kernel<256, false><<<grid, 512, 0, st>>>(a);
+    }
     if (int rc = check_launch("prefill_attn")) return rc;
     if (!quantize_on_write) return HS_OK;
     if (fp8)

@@ -110,9 +110,10 @@ def test_attention_through_the_cache_object(quant, D):
     assert d.max() < 2e-2 and d.mean() < 2e-3
 
 
+@pytest.mark.parametrize("D", [128, 256])
 @pytest.mark.parametrize("fmt", ["int8", "fp8"])
-def test_chunked_prefill_then_decode_through_the_cache_object(fmt):
-    B, Hq, Hkv, D, C = 1, 8, 2, 128, 96
+def test_chunked_prefill_then_decode_through_the_cache_object(fmt, D):
+    B, Hq, Hkv, C = 1, 8, 2, 96
     cache = kc.LayerKVCache(512, kc.INT8 if fmt == "int8" else kc.FP8)
     q, k, v = randn(12, B, 2 * C, Hq, D), randn(13, B, 2 * C, Hkv, D), randn(14, B, 2 * C, Hkv, D)
     o0 = cache.prefill(q[:, :C], k[:, :C], v[:, :C], 0, 1 / np.sqrt(D))

@@ -66,11 +66,12 @@ def test_update_across_block_boundaries_and_truncate():
     assert np.array_equal(gk.cpu().numpy(), _dense_reference(k))
 
 
-def test_chunked_prefill_through_a_paged_cache():
+@pytest.mark.parametrize("D", [128, 256])
+def test_chunked_prefill_through_a_paged_cache(D):
     """Two prompt chunks that cross block boundaries: attention of each chunk over [cached blocks | itself] against
     the oracle, and the blocks end up holding what update() would have written."""
-    r = wl.philox(905)
-    Hq, Hkv, D, C = 8, 2, 128, 300
+    r = wl.philox(905 + D)
+    Hq, Hkv, C = 8, 2, 300
     pool = kc.BlockPool(16, Hkv, D)
     cache = kc.PagedLayerKVCache(2048, pool, 7)
     q, k, v = _rand(r, 1, 2 * C, Hq, D), _rand(r, 1, 2 * C, Hkv, D), _rand(r, 1, 2 * C, Hkv, D)

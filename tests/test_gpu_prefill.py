@@ -326,3 +326,41 @@ def test_random_shapes(seed):
         kd, vd = deq(kc, ks), deq(vc, vs)
     got = gpu_prefill(c, q, k, v, hist)
     compare(got, oracle_prefill(q, kd, vd, k, v), "random B=%d Hkv=%d G=%d hist=%d S=%d fp8=%s" % (B, Hkv, G, hist, S, fp8))
+
+
+# ------------------------------------------------------------------ head_dim 256 (128 query columns per workgroup)
+@pytest.mark.parametrize("hist,S,fp8", [(0, 1, False), (0, 33, False), (0, 257, False), (19, 5, False), (64, 64, False),
+                                        (200, 130, False), (333, 200, True), (65, 31, True)])
+def test_head_dim_256(hist, S, fp8):
+    B, Hq, Hkv, D = 2, 8, 2, 256
+    sigma = 0.5 if fp8 else 1.0
+    q, k, v = make(500 + hist + S, B, S, Hq, Hkv, D=D, sigma=sigma)
+    c = DeviceCache(B, Hkv, hist + S, D, fp8=fp8)
+    kd = vd = None
+    if hist > 0:
+        _, kh, vh = make(600 + hist, B, hist, Hq, Hkv, D=D, sigma=sigma)
+        hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+        if fp8:
+            hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+        c.write(hk, hv, None, 0)
+        kc, vc, ks, vs = c.canonical(hist)
+        deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
+        kd, vd = deq(kc, ks), deq(vc, vs)
+    got = gpu_prefill(c, q, k, v, hist)
+    compare(got, oracle_prefill(q, kd, vd, k, v), "d256 hist=%d S=%d fp8=%s" % (hist, S, fp8))
+    if not fp8:  # the new rows were cached behind the history with the oracle's codes
+        kc, vc, ks, vs = c.canonical(hist + S)
+        wk, wks = oracle.quant_int8(k)
+        assert np.array_equal(kc[:, hist:], wk) and np.array_equal(ks[:, hist:], wks)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(2, 2), (4, 2), (16, 4), (16, 2)])
+def test_head_dim_256_group_sizes(Hq, Hkv):
+    B, S, hist, D = 1, 70, 100, 256
+    q, k, v = make(700 + Hq, B, S, Hq, Hkv, D=D)
+    _, kh, vh = make(701 + Hq, B, hist, Hq, Hkv, D=D)
+    c = DeviceCache(B, Hkv, hist + S, D)
+    c.write(torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16(), None, 0)
+    kc, vc, ks, vs = c.canonical(hist)
+    got = gpu_prefill(c, q, k, v, hist)
+    compare(got, oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v), "d256 gqa %d/%d" % (Hq, Hkv))
