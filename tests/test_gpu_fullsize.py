@@ -123,11 +123,13 @@ def test_config4_full_size_fp8_decode():
     sample_check(out, q, kc, vc, ks, vs, full.cpu().numpy(), [(0, 0), (31, 7)], 8, True)
 
 
-def test_config3_full_size_chunked_prefill():
+@pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (16, 4, 256)])
+def test_config3_full_size_chunked_prefill(Hq, Hkv, D):
     """B=4 x 4096 tokens in 512-token chunks: sampled query rows of every chunk against the oracle over
-    [dequantized int8 cache of earlier chunks | own bf16 K/V]; the cache ends up equal to one-shot quantization."""
-    B, T, C, Hq, Hkv, D = 4, 4096, 512, 32, 8, 128
-    g = gen(wl.SEED + 3)
+    [dequantized int8 cache of earlier chunks | own bf16 K/V]; the cache ends up equal to one-shot quantization.
+    Also at the head shape of Qwen3.5's full-attention layers (head_dim 256, the same flops and bytes)."""
+    B, T, C = 4, 4096, 512
+    g = gen(wl.SEED + 3 + D)
     q, k, v = source(g, (B, T, Hq, D)), source(g, (B, T, Hkv, D)), source(g, (B, T, Hkv, D))
     lay = hb.contiguous_layout(Hkv, T, D)
     kc = torch.zeros(B, Hkv, T, D, dtype=torch.int8, device=DEV)
@@ -154,8 +156,8 @@ def test_config3_full_size_chunked_prefill():
                                   np.array([pos + 1], np.int32), 1.0 / np.sqrt(D))[0]
         d = np.abs(out[b, pos, 4 * h:4 * h + 4].float().cpu().numpy() - want)
         assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, pos, d.max(), d.mean())
-    wk, wks = oracle.quant_int8(k[1, :, 5].float().cpu().numpy())
-    assert np.array_equal(kc[1, 5].cpu().numpy(), wk) and np.array_equal(ks[1, 5, :T].cpu().numpy(), wks)
+    wk, wks = oracle.quant_int8(k[1, :, Hkv - 3].float().cpu().numpy())
+    assert np.array_equal(kc[1, Hkv - 3].cpu().numpy(), wk) and np.array_equal(ks[1, Hkv - 3, :T].cpu().numpy(), wks)
 
 
 def test_config3_shape_with_fp8_history():
