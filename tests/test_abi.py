@@ -140,3 +140,28 @@ def test_format_names_are_distinct_and_stable():
     assert not set(names) & {b"int8", b"nf4", b"fp4"}
     assert L.hs_kv_quant_canonical_str(9) is None
 
+
+
+def test_workspace_sizes_are_host_arithmetic():
+    """The workspace functions need no GPU: sizes a caller can plan with."""
+    # chunked delta rule: per 64-token chunk 32,768 B per (sequence, k-head) and 41,728 B per (sequence, v-head)
+    assert hb.deltanet_chunked_workspace_bytes(4, 4096, 16, 32) == 64 * (4 * 16 * 32768 + 4 * 32 * 41728)
+    assert hb.deltanet_chunked_workspace_bytes(1, 1, 1, 1) == 32768 + 41728
+    assert hb.deltanet_chunked_workspace_bytes(1, 65, 2, 4) == 2 * (2 * 32768 + 4 * 41728)
+    assert hb.deltanet_chunked_workspace_bytes(0, 64, 1, 1) == 0
+    # decode: room for (D + 2) floats per (sequence, query head, chunk), a multiple of 256 bytes, growing with head_dim
+    small, big = hb.decode_workspace_bytes(64, 32, 8, 128, 8192), hb.decode_workspace_bytes(64, 32, 8, 256, 8192)
+    assert small % 256 == 0 and big % 256 == 0 and big > small >= 64 * 32 * 130 * 4
+
+
+def test_chunked_delta_rule_rejects_bad_arguments_before_launching():
+    p = ctypes.c_void_p(0x1000)
+    L = hb.lib()
+    call = lambda nk, nv, dk, ws, nbytes: L.hs_deltanet_forward_chunked(p, p, p, p, p, p, p, 1, 64, nk, nv, dk, 128, ctypes.c_float(1.0), 1,
+                                                                      ws, ctypes.c_size_t(nbytes), None)
+    assert call(3, 4, 128, p, 1 << 30) == hb.HS_ERR_INVALID_ARGUMENT      # nv not a multiple of nk
+    assert call(2, 4, 64, p, 1 << 30) == hb.HS_ERR_INVALID_ARGUMENT       # dk must be 128
+    assert call(2, 4, 128, p, 100) == hb.HS_ERR_WORKSPACE                 # too small
+    assert b"workspace" in L.hs_attn_last_error()
+    assert call(2, 4, 128, None, 0) == hb.HS_ERR_WORKSPACE                # none at all
+    assert call(2, 4, 128, ctypes.c_void_p(0x1004), 1 << 30) == hb.HS_ERR_INVALID_ARGUMENT  # misaligned
