@@ -44,14 +44,22 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-// head_dim 128 or 256.  A wavefront step always covers 8 KB of codes: 32 tokens at D = 128, 16 at D = 256 (the
-// second product then runs on v_mfma_f32_16x16x16_f16, whose operand layout matches one 16-token score tile).
+// head_dim 64, 128 or 256.  A wavefront step always covers 8 KB of codes: 64 tokens at D = 64, 32 at D = 128, 16 at
+// D = 256 (the second product then runs on v_mfma_f32_16x16x16_f16, whose operand layout matches one 16-token tile).
 template <int D> struct Shape {
-    static constexpr int kStep = D == 256 ? 16 : 32;  // tokens per wavefront step
+    static constexpr int kStep = 4096 / D;            // tokens per wavefront step
     static constexpr int NT = kStep / 16;             // 16-token score tiles per step
     static constexpr int NJ = D / 32;                 // MFMAs per score tile (32 d each)
-    static constexpr int NC = D / 128;                // 128-column groups of V / O
+    static constexpr int VW = D >= 128 ? 2 : 1;       // dwords of V codes a lane takes per token (d = 4*VW*li ..)
+    static constexpr int NBB = 4 * VW;                // V^T row blocks (MFMAs) per column group
+    static constexpr int CW = 16 * NBB;               // columns of a group: 128, or the whole head at D = 64
+    static constexpr int NC = D / CW;                 // column groups of V / O
+    static constexpr int NS = kStep > 32 ? 2 : 1;     // scale loads per lane and step
 };
+template <int VW> struct VCodes { typedef u32x2 type; };
+template <> struct VCodes<1> { typedef uint32_t type; };
+__device__ __forceinline__ uint32_t vword(const u32x2 &x, int i) { return x[i]; }
+__device__ __forceinline__ uint32_t vword(uint32_t x, int) { return x; }
 constexpr int kWavesPerWg = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kPScale = 64.0f;  // P is carried as 64*p*s_v in fp16 (keeps small weights normal)
@@ -77,11 +85,28 @@ struct DecodeArgs {
 // Half-split rotary embedding of the 32 query elements a lane holds, in bf16 arithmetic (every product and sum
 // rounded to bf16, as the separate libtorch ops of RoPE::apply_rotary_pos_emb do, rope.rs:206-248).  Element
 // qf[8*i + e] is d = 64*(i/2) + 16*lq + 8*(i%2) + e (i < NJ = D/32), so a lane holds both halves of each rotated
-// pair: blocks i and i + NJ/2.
+// pair: blocks i and i + NJ/2.  At D = 64 the lane holds d = 16*lq + 8*i + e only, and the other half of each pair sits
+// in the lane 32 further on (or back): the two exchange their elements and each computes its own half.
 template <int NJ>
 __device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
 #pragma clang fp contract(off)
     auto rb = [](float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); };
+    if constexpr (NJ == 2) {
+        const bool upper = lq >= 2;  // this lane holds x2 (d >= 32) of its pairs
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int j0 = 16 * (lq & 1) + 8 * i;
+            const u32x4 sw = *(const u32x4 *)(sin_row + j0), cw = *(const u32x4 *)(cos_row + j0);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
+                const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
+                const float mine = qf[8 * i + e], other = __shfl_xor(mine, 32, 64);
+                qf[8 * i + e] = upper ? rb(rb(other * sn) + rb(mine * cs)) : rb(rb(mine * cs) - rb(other * sn));
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NJ / 2; ++i) {
         const int j0 = 64 * (i >> 1) + 16 * lq + 8 * (i & 1);
@@ -100,8 +125,10 @@ __device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_
 template <int D>
 struct Stage {
     u32x4 k[Shape<D>::NT][Shape<D>::NJ / 2];  // [16-token tile][64-byte piece of the row]: 16 B at byte 64*piece + 16*lq of row li
-    u32x2 v[Shape<D>::NC][4 * Shape<D>::NT];  // [column group c][token slot e = 4u + r] 8 bytes: d = 128*c + 8*(lane%16) .. +7
-    float sraw;  // int8 only: lanes [0, kStep) hold the K scale of token `lane`, lanes [kStep, 2*kStep) the V scales
+    typename VCodes<Shape<D>::VW>::type v[Shape<D>::NC][4 * Shape<D>::NT];  // [column group c][token slot e = 4u + r]: d = CW*c + 4*VW*(lane%16) ..
+    // int8 only.  Steps of up to 32 tokens: lanes [0, kStep) hold the K scale of token `lane`, lanes [kStep, 2*kStep)
+    // the V scales; 64-token steps: [0] the K scale and [1] the V scale of token `lane`
+    float sraw[Shape<D>::NS];
 };
 
 __device__ __forceinline__ half8 as_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -118,6 +145,7 @@ __device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t t) {
 template <int kD, bool FP8, bool ROPE>
 __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     constexpr int kStep = Shape<kD>::kStep, NT = Shape<kD>::NT, NJ = Shape<kD>::NJ, NC = Shape<kD>::NC;
+    constexpr int VW = Shape<kD>::VW, NBB = Shape<kD>::NBB, CW = Shape<kD>::CW, NS = Shape<kD>::NS;
     // Workgroups go to the 8 XCDs round-robin by linear id.  Low chunk indices always hold work, high ones only
     // for long sequences, so the chunk index is rotated by (head + sequence): every XCD then sees every index
     // equally often instead of two XCDs getting all the first chunks.
@@ -148,13 +176,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     // fp8: the V scale is one constant per (sequence, head); it multiplies the finished partial.
     const float out_scale = (1.0f / kPScale) * (FP8 ? 256.0f * a.vs[(int64_t)b * a.Hkv + h] : 1.0f);
 
-    float4v acc[8 * NC];  // O[d = 128*c + 32*lq + 8*r + bb][head li] in acc[8*c + bb][r]
+    float4v acc[NBB * NC];  // O[d = CW*c + 4*NBB*lq + NBB*r + bb][head li] in acc[NBB*c + bb][r]
 #pragma unroll
-    for (int i = 0; i < 8 * NC; ++i) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < NBB * NC; ++i) acc[i] = (float4v){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.0f;
 
     const int nsteps = (t_end - t_begin + kStep - 1) / kStep;
-    __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64];
+    __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64 * NS];
 
     auto load_stage = [&](Stage<kD> &st, int step) {
         const int t0 = t_begin + step * kStep;
@@ -177,8 +205,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             // compute_stage hands them to the lanes that need them through LDS
             const float *ksb = a.ks + ku * a.ka.scale_stride_seq + (int64_t)h * a.ka.scale_stride_head + kslot;
             const float *vsb = a.vs + vu * a.va.scale_stride_seq + (int64_t)h * a.va.scale_stride_head + vslot;
-            const int sl = lane & (2 * kStep - 1);  // 16-token steps: the upper 32 lanes repeat the lower ones
-            st.sraw = __builtin_nontemporal_load((sl < kStep ? ksb : vsb) + min(sl & (kStep - 1), last));
+            if constexpr (NS == 1) {
+                const int sl = lane & (2 * kStep - 1);  // 16-token steps: the upper 32 lanes repeat the lower ones
+                st.sraw[0] = __builtin_nontemporal_load((sl < kStep ? ksb : vsb) + min(sl & (kStep - 1), last));
+            } else {
+                st.sraw[0] = __builtin_nontemporal_load(ksb + min(lane, last));
+                st.sraw[1] = __builtin_nontemporal_load(vsb + min(lane, last));
+            }
         }
 #pragma unroll
         for (int c = 0; c < NC; ++c)
@@ -187,7 +220,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int row = min(16 * u + 4 * lq + r, last);
-                    st.v[c][4 * u + r] = __builtin_nontemporal_load((const u32x2 *)(vb + row * kD + 128 * c + 8 * li));
+                    st.v[c][4 * u + r] = __builtin_nontemporal_load((const typename VCodes<VW>::type *)(vb + row * kD + CW * c + 4 * VW * li));
                 }
     };
 
@@ -197,7 +230,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         //      LDS operations of one wavefront complete in order, so the reads see the write without a barrier.
         float4v sk[NT], sv[NT];
         if (!FP8) {
-            sm_sc[wave][lane] = st.sraw;
+            sm_sc[wave][lane] = st.sraw[0];
+            if constexpr (NS == 2) sm_sc[wave][64 + lane] = st.sraw[1];
             __builtin_amdgcn_wave_barrier();
 #pragma unroll
             for (int u = 0; u < NT; ++u) {
@@ -260,7 +294,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             l_run *= alpha;
 #pragma unroll
-            for (int i = 0; i < 8 * NC; ++i) acc[i] *= alpha;
+            for (int i = 0; i < NBB * NC; ++i) acc[i] *= alpha;
             m_run = m_new;
         }
         uint32_t pb[2 * NT];
@@ -272,14 +306,14 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             half2v hp = {(_Float16)(p0 * pv[2 * i]), (_Float16)(p1 * pv[2 * i + 1])};
             pb[i] = __builtin_bit_cast(uint32_t, hp);
         }
-        // ---- O += V^T P : 8 MFMAs per column group, one per byte column bb of this lane's 8 d's
+        // ---- O += V^T P : one MFMA per 32 tokens and byte column bb of this lane's d's
 #pragma unroll
-        for (int cb = 0; cb < 8 * NC; ++cb) {
-            const int c = cb >> 3, bb = cb & 7;
+        for (int cb = 0; cb < NBB * NC; ++cb) {
+            const int c = cb / NBB, bb = cb % NBB;
             uint32_t av[2 * NT];
 #pragma unroll
             for (int p = 0; p < 2 * NT; ++p) {
-                const uint32_t lo = st.v[c][2 * p][bb >> 2], hi = st.v[c][2 * p + 1][bb >> 2];
+                const uint32_t lo = vword(st.v[c][2 * p], bb >> 2), hi = vword(st.v[c][2 * p + 1], bb >> 2);
                 if (FP8) {
                     const uint32_t sel = 0x040c000cu + ((uint32_t)(bb & 3) << 8) + ((uint32_t)(bb & 3) << 24);
                     av[p] = fp8x2_to_f16x2(__builtin_amdgcn_perm(hi, lo, sel));
@@ -290,9 +324,12 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                     av[p] = __builtin_bit_cast(uint32_t, hv);
                 }
             }
-            if constexpr (NT == 2) {
-                acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av[0], av[1], av[2], av[3]),
-                                                                 as_half8(pb[0], pb[1], pb[2], pb[3]), acc[cb], 0, 0, 0);
+            if constexpr (NT >= 2) {
+#pragma unroll
+                for (int tg = 0; tg < NT / 2; ++tg)  // 32 tokens (two score tiles) per MFMA
+                    acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as_half8(av[4 * tg], av[4 * tg + 1], av[4 * tg + 2], av[4 * tg + 3]),
+                                                                     as_half8(pb[4 * tg], pb[4 * tg + 1], pb[4 * tg + 2], pb[4 * tg + 3]),
+                                                                     acc[cb], 0, 0, 0);
             } else {
                 const u32x2 aw = {av[0], av[1]}, pw = {pb[0], pb[1]};
                 acc[cb] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(half4, aw), __builtin_bit_cast(half4, pw),
@@ -376,7 +413,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
     __shared__ float sm_m[kWavesPerWg][16], sm_l[kWavesPerWg][16];
-    __shared__ float sm_o[kWavesPerWg][16][128 + 4];  // one 128-column group of O at a time
+    __shared__ float sm_o[kWavesPerWg][16][CW + 4];  // one column group of O at a time
     if (lq == 0) {
         sm_m[wave][li] = m_run;
         sm_l[wave][li] = l_run;
@@ -392,15 +429,15 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         if (c > 0) __syncthreads();  // the previous group has been read
         if (li < G) {
 #pragma unroll
-            for (int bb = 0; bb < 8; ++bb)
+            for (int bb = 0; bb < NBB; ++bb)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) sm_o[wave][li][32 * lq + 8 * r + bb] = acc[8 * c + bb][r] * f;
+                for (int r = 0; r < 4; ++r) sm_o[wave][li][4 * NBB * lq + NBB * r + bb] = acc[NBB * c + bb][r] * f;
         }
         __syncthreads();
         if (a.direct) {
             // single chunk: normalise and write the output, no workspace traffic
-            for (int idx = threadIdx.x; idx < G * 128; idx += 256) {
-                const int g = idx / 128, d = idx % 128;
+            for (int idx = threadIdx.x; idx < G * CW; idx += 256) {
+                const int g = idx / CW, d = idx % CW;
                 float o = 0.0f, l = 0.0f, Mg = sm_m[0][g];
 #pragma unroll
                 for (int w = 1; w < kWavesPerWg; ++w) Mg = fmaxf(Mg, sm_m[w][g]);
@@ -409,15 +446,15 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                     o += sm_o[w][g][d];
                     l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
                 }
-                a.out[((int64_t)b * a.Hq + h * G + g) * kD + 128 * c + d] = (uint16_t)f32_to_bf16_bits(o * out_scale / l);
+                a.out[((int64_t)b * a.Hq + h * G + g) * kD + CW * c + d] = (uint16_t)f32_to_bf16_bits(o * out_scale / l);
             }
         } else {
-            for (int idx = threadIdx.x; idx < G * 128; idx += 256) {
-                const int g = idx / 128, d = idx % 128;
+            for (int idx = threadIdx.x; idx < G * CW; idx += 256) {
+                const int g = idx / CW, d = idx % CW;
                 float o = 0.0f;
 #pragma unroll
                 for (int w = 0; w < kWavesPerWg; ++w) o += sm_o[w][g][d];
-                a.part_o[(prow + (int64_t)g * a.nchunks) * kD + 128 * c + d] = o * out_scale;
+                a.part_o[(prow + (int64_t)g * a.nchunks) * kD + CW * c + d] = o * out_scale;
             }
         }
     }
@@ -461,7 +498,7 @@ static int pick_chunk_tokens(int B, int Hkv, int max_seq_len, int64_t total_toke
     // A workgroup costs about 1.5 us of prologue/epilogue, so chunks are as long as the grid allows:
     // with >= 512 (sequence, kv-head) units (two resident workgroups on each of 256 CUs) nothing is
     // split and the step is a single launch; below that, split until about 1024 workgroups exist.
-    // Chunks are a multiple of 128 tokens (4 wavefronts x 32).  Measured on MI355X: B=64 x 8 heads x
+    // Chunks are a multiple of 128 tokens (a whole number of wavefront steps at every head_dim).  Measured on MI355X: B=64 x 8 heads x
     // 8192 tokens runs 193 us unsplit, 196 us in 2 chunks, 205 us in 8; B=32 x 8 x 32768 is fastest at 4.
     const int64_t units = (int64_t)B * Hkv;
     int64_t want_chunks = units >= 512 ? 1 : (1024 + units - 1) / units;
@@ -496,7 +533,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
                          size_t ws_bytes, int B, int Hq, int Hkv, int D, int max_seq_len, float softmax_scale,
                          hipStream_t stream) {
     if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
-    if (D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 128 and 256, got %d", D);
+    if (D != 64 && D != 128 && D != 256)
+        return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 64, 128 and 256, got %d", D);
     if (B > 0 && (!q || !kc || !vc || !ks || !vs || !seq_lens || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if ((nt.k_src == nullptr) != (nt.v_src == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give k_new and v_new or neither");
     if (nt.k_src && nt.dtype != HS_BF16 && nt.dtype != HS_F32 && nt.dtype != HS_F16)
@@ -504,8 +542,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     if (Hq <= 0 || Hq % Hkv != 0 || Hq / Hkv > 16)
         return fail(HS_ERR_INVALID_ARGUMENT, "need Hq %% Hkv == 0 and Hq/Hkv <= 16 (Hq=%d Hkv=%d)", Hq, Hkv);
     if (max_seq_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "max_seq_len must be positive");
-    if (l->k_block_table && (l->capacity_tokens % 32) != 0)
-        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of 32 tokens");
+    if (l->k_block_table && (l->capacity_tokens % (D == 64 ? 64 : 32)) != 0)  // a wavefront step stays inside one block
+        return fail(HS_ERR_INVALID_ARGUMENT, "paged blocks must hold a multiple of %d tokens", D == 64 ? 64 : 32);
     if (B == 0) return HS_OK;
     {
         const int64_t cap = l->k_block_table ? (int64_t)l->capacity_tokens * l->block_table_stride : l->capacity_tokens;
@@ -546,7 +584,11 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.rope_sin = (const uint16_t *)nt.rope_sin; a.rope_cos = (const uint16_t *)nt.rope_cos; a.rope_len = nt.rope_len;
     if (phases & 1) {
         dim3 grid(a.nchunks, Hkv, B);
-        if (D == 128) {
+        if (D == 64) {
+            if (fp8) decode_attn_kernel<64, true, false><<<grid, 256, 0, stream>>>(a);
+            else if (a.rope_sin) decode_attn_kernel<64, false, true><<<grid, 256, 0, stream>>>(a);
+            else decode_attn_kernel<64, false, false><<<grid, 256, 0, stream>>>(a);
+        } else if (D == 128) {
             if (fp8) decode_attn_kernel<128, true, false><<<grid, 256, 0, stream>>>(a);
             else if (a.rope_sin) decode_attn_kernel<128, false, true><<<grid, 256, 0, stream>>>(a);
             else decode_attn_kernel<128, false, false><<<grid, 256, 0, stream>>>(a);

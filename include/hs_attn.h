@@ -26,6 +26,8 @@
  * With block tables (paged mode, the reference's BlockPool of fixed-size token
  * blocks, kv_cache.rs:477-693) "b" above is replaced by the block id found at
  * table[b*block_table_stride + t / capacity_tokens] and t by t % capacity_tokens.
+ * Decode attention reads a block in whole wavefront steps: capacity_tokens of a paged layout is a
+ * multiple of 32 there (of 64 at D = 64); the reference's 256-token blocks satisfy both.
  * A dense [B, T, Hkv, D] tensor, as LayerKVCache::get returns it
  * (kv_cache.rs:1499-1643), is produced on request by hs_kv_dequantize.
  *
@@ -148,7 +150,7 @@ HS_API int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8,
  * q, out: [B, Hq, D] bf16.  seq_lens: device [B], cached tokens per sequence INCLUDING the
  * one just written; rows with seq_len <= 0 produce zeros.  max_seq_len >= every seq_lens[b]
  * (host-side bound used to size the grid).  out = softmax(q K^T * softmax_scale) V with
- * fp32 accumulation, K/V dequantized on the fly.  D is 128 or 256 (Hq/Hkv <= 16); anything
+ * fp32 accumulation, K/V dequantized on the fly.  D is 64, 128 or 256 (Hq/Hkv <= 16); anything
  * else is HS_ERR_INVALID_ARGUMENT.  workspace: device scratch of at least
  * hs_decode_attn_workspace_bytes(...) bytes, 256-byte aligned, owned by the caller. */
 HS_API size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len);

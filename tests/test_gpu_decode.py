@@ -369,9 +369,79 @@ def test_head_dim_256_paged_block_table():
     assert np.array_equal(out.float().cpu().numpy(), want)
 
 
+# ------------------------------------------------------------------ head_dim 64 (64-token wavefront steps)
+@pytest.mark.parametrize("lens", [[1], [63], [64], [65], [255, 256, 257], [1, 700, 64, 513, 5]])
+def test_head_dim_64_ragged_lengths_and_step_boundaries(lens):
+    B = len(lens)
+    case = wl.decode_case(40, B, 16, 4, 64, max(lens), outliers=True)
+    case["seq_lens"] = np.array(lens, np.int32)
+    check(case, 16, 4, 64, cap=max(lens) + 3, label="d64-ragged%s" % lens)
+
+
+@pytest.mark.parametrize("Hq,Hkv,T", [(16, 4, 3000), (4, 1, 9000), (32, 2, 500), (5, 5, 300)])
+def test_head_dim_64_split_and_group_sizes(Hq, Hkv, T):
+    case = wl.decode_case(41, 2, Hq, Hkv, 64, T, ragged=True, outliers=True, min_len=T // 2)
+    check(case, Hq, Hkv, 64, label="d64-%d/%d-%d" % (Hq, Hkv, T))
+
+
+def test_head_dim_64_fp8():
+    case = wl.decode_case(42, 2, 16, 4, 64, 700, sigma=0.5)
+    check(case, 16, 4, 64, fp8=True, label="d64-fp8")
+
+
+def test_head_dim_64_fused_step_equals_write_then_attend():
+    B, Hq, Hkv, D, T = 4, 16, 4, 64, 600
+    case = wl.decode_case(43, B, Hq, Hkv, D, T, ragged=True, outliers=True)
+    r = wl.philox(44)
+    nk = torch.from_numpy(r.standard_normal((B, 1, Hkv, D)).astype(np.float32)).to(DEV).bfloat16()
+    nv = torch.from_numpy(r.standard_normal((B, 1, Hkv, D)).astype(np.float32)).to(DEV).bfloat16()
+    lens = case["seq_lens"]
+    c1 = build_cache(case, Hkv, D)
+    c1.write(nk, nv, torch.from_numpy((lens - 1).astype(np.int32)).to(DEV), 0)
+    want = run_decode(c1, case["q_bits"], lens, Hq, max_seq_len=T)
+    c2 = build_cache(case, Hkv, D)
+    out = torch.full((B, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_step(bf16_from_bits(case["q_bits"]).to(DEV), nk, nv, c2.k_codes, c2.v_codes, c2.k_scales, c2.v_scales,
+                   c2.layout, torch.from_numpy(lens).to(DEV), out, ws, Hkv, T, 1.0 / np.sqrt(D))
+    torch.cuda.synchronize()
+    for name in ("k_codes", "v_codes", "k_scales", "v_scales"):
+        assert torch.equal(getattr(c1, name), getattr(c2, name)), name
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    kc, vc, ks, vs = c2.canonical(T)
+    ref = oracle.decode_attn(oracle.bf16_to_f32(case["q_bits"]), kc, vc, ks, vs, oracle.FMT_INT8, lens, 1.0 / np.sqrt(D))
+    d = np.abs(want - ref)
+    assert d.max() < TOL_MAX and d.mean() < TOL_MEAN
+
+
+def test_head_dim_64_paged_block_table():
+    B, Hq, Hkv, D, T, BT = 2, 8, 2, 64, 300, 64
+    case = wl.decode_case(45, B, Hq, Hkv, D, T, ragged=True)
+    c = build_cache(case, Hkv, D)
+    want = run_decode(c, case["q_bits"], case["seq_lens"], Hq)
+    nblk = (T + BT - 1) // BT
+    ids = wl.philox(46).permutation(2 * B * nblk + 3).astype(np.int32)
+    kt, vt = ids[: B * nblk].reshape(B, nblk), ids[B * nblk: 2 * B * nblk].reshape(B, nblk)
+    pk = torch.zeros(len(ids), Hkv, BT, D, dtype=torch.int8, device=DEV)
+    ps = torch.zeros(len(ids), Hkv, BT, dtype=torch.float32, device=DEV)
+    k_tab, v_tab = torch.from_numpy(kt).to(DEV), torch.from_numpy(vt).to(DEV)  # the layout holds their addresses: keep them alive
+    lay = hb.paged_layout(Hkv, BT, D, k_tab, v_tab)
+    hb.kv_quantize_int8(torch.from_numpy(case["k"]).to(DEV), torch.from_numpy(case["v"]).to(DEV), pk, pk, ps, ps, lay, None, 0)
+    out = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_attn(bf16_from_bits(case["q_bits"]).to(DEV), pk, pk, ps, ps, lay, torch.from_numpy(case["seq_lens"]).to(DEV),
+                   out, ws, Hkv, T, 1.0 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert np.array_equal(out.float().cpu().numpy(), want)
+    lay32 = hb.paged_layout(Hkv, 32, D, k_tab, v_tab)  # a 64-token wavefront step would straddle two 32-token blocks
+    with pytest.raises(hb.HsError, match="multiple of 64"):
+        hb.decode_attn(bf16_from_bits(case["q_bits"]).to(DEV), pk, pk, ps, ps, lay32, torch.from_numpy(case["seq_lens"]).to(DEV),
+                       out, ws, Hkv, 32, 1.0 / np.sqrt(D))
+
+
 def test_unsupported_head_dim_is_rejected():
-    c = DeviceCache(1, 2, 64, 64)
-    q = torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=DEV)
+    c = DeviceCache(1, 2, 64, 192)
+    q = torch.zeros(1, 4, 192, dtype=torch.bfloat16, device=DEV)
     out = torch.empty_like(q)
     ws = torch.empty(1 << 16, dtype=torch.uint8, device=DEV)
     with pytest.raises(hb.HsError) as e:
@@ -387,7 +457,7 @@ def test_random_shapes(seed):
     B = int(r.integers(1, 6))
     Hkv = int(r.choice([1, 2, 3, 4, 8]))
     G = int(r.choice([1, 2, 4, 5, 8, 16]))
-    D = int(r.choice([128, 256]))
+    D = int(r.choice([64, 128, 256]))
     T = int(r.integers(1, 1400))
     fp8 = bool(r.integers(0, 2))
     case = wl.decode_case(200 + seed, B, Hkv * G, Hkv, D, T, ragged=True, outliers=not fp8, sigma=0.5 if fp8 else 1.0)

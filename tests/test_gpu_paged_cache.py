@@ -120,7 +120,7 @@ def test_exhaustion_midway_keeps_earlier_pairs_and_is_retryable():
     assert cache.seq_pos == 256
 
 
-@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("lens", [[5, 255, 256, 700], [1, 1, 1]])
 def test_ragged_batch_decode_step_matches_oracle(lens, D):
     r = wl.philox(910 + len(lens) + D)

@@ -128,7 +128,7 @@ def test_quantize_with_rope_bit_exact(D):
     assert not kc[:, :start].any()  # nothing before start_pos is touched
 
 
-@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("D", [64, 128, 256])
 @pytest.mark.parametrize("lens", [[300, 300, 300], [1, 129, 700]])
 def test_decode_step_with_rope_matches_unfused_and_oracle(lens, D):
     r = wl.philox(740 + len(set(lens)) + D)
