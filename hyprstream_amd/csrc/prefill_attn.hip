@@ -113,7 +113,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         }
     }
     const int b = bz;
-    const int groups = a.G / a.HG;
+    const int groups = (a.G + a.HG - 1) / a.HG;  // the last group of a kv-head may be partly padding (G = 3, 5, 6, 7 ...)
     const int kvh = by / groups, hg = by % groups;
     const int S = a.S, H = a.hist_len;
     const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
         const int bi = kNB * wave + nb;
-        head[nb] = kvh * a.G + hg * a.HG + bi % a.HG;
+        head[nb] = kvh * a.G + min(hg * a.HG + bi % a.HG, a.G - 1);  // a padding column repeats the group's last head
         qi[nb] = q0 + 16 * (bi / a.HG) + li;
     }
     const int wv_q0 = q0 + 16 * ((kNB * wave) / a.HG);  // first query of this wavefront
@@ -678,7 +678,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
         const float l = l_run[nb][0];
-        if (qi[nb] >= S) continue;
+        if (qi[nb] >= S || hg * a.HG + (kNB * wave + nb) % a.HG >= a.G) continue;  // padding columns write nothing
         const float inv = 1.0f / l;
         uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kPD + 32 * lq;
 #pragma unroll
@@ -720,8 +720,8 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
         return fail(HS_ERR_INVALID_ARGUMENT, "null cache buffer");
     if (hist_len < 0) return fail(HS_ERR_INVALID_ARGUMENT, "negative hist_len");
     const int G = Hq > 0 && Hkv > 0 ? Hq / Hkv : 0;
-    if (Hq <= 0 || Hq % Hkv != 0 || (G != 1 && G != 2 && G % 4 != 0))
-        return fail(HS_ERR_INVALID_ARGUMENT, "need Hq/Hkv in {1, 2, 4k} (Hq=%d Hkv=%d)", Hq, Hkv);
+    if (Hq <= 0 || Hq % Hkv != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "need Hq %% Hkv == 0 (Hq=%d Hkv=%d)", Hq, Hkv);
     const int64_t cap = layout->k_block_table ? (int64_t)layout->capacity_tokens * layout->block_table_stride
                                               : layout->capacity_tokens;
     if ((int64_t)hist_len + (quantize_on_write ? S : 0) > cap)
@@ -738,10 +738,10 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.ka = make_addr(*layout, 0); a.va = make_addr(*layout, 1);
     a.out = (uint16_t *)out;
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
-    a.HG = G >= 4 ? 4 : G;
+    a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
     const int q_per_wg = 16 * ((256 / D) * kPWaves / a.HG);
-    dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * (G / a.HG), B);
+    dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * ((G + a.HG - 1) / a.HG), B);
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();

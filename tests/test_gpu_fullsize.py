@@ -303,3 +303,25 @@ def test_head_dim_256_full_size_decode():
     vs.fill_(0.125)
     const = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
     assert (const.float() - 8.0).abs().max() <= 2 ** -5
+
+
+def test_head_dim_64_full_size_decode():
+    """64-wide heads at the cache size of config 2: B=64, Hq 32 / Hkv 16, D 64, T 8192, int8 (64-token wavefront steps)."""
+    B, Hq, Hkv, D, T = 64, 32, 16, 64, 8192
+    g = gen(wl.SEED + 64)
+    lay, kc, vc, ks, vs, kept = fill_cache(g, B, Hkv, T, D, False, 1.0, True, keep=(7,))
+    kk, _ = kept[7]
+    wk, wks = oracle.quant_int8(kk[:, :, 1])
+    assert np.array_equal(kc[7, 1].cpu().numpy(), wk[0]) and np.array_equal(ks[7, 1, :T].cpu().numpy(), wks[0])
+    q = torch.randn(B, Hq, D, generator=g, device=DEV).to(torch.bfloat16)
+    lens = torch.randint(512, T + 1, (B,), generator=g, device=DEV, dtype=torch.int32)
+    lens[0] = T
+    out = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    assert torch.isfinite(out.float()).all()
+    sample_check(out, q, kc, vc, ks, vs, lens.cpu().numpy(), [(0, 0), (33, 11)], 2, False)
+    two = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False, phases=12)
+    assert (two.float() - out.float()).abs().max() <= 2 ** -8 * max(1.0, float(out.float().abs().max()))
+    vc.fill_(64)
+    vs.fill_(0.125)
+    const = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    assert (const.float() - 8.0).abs().max() <= 2 ** -5

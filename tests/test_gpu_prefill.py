@@ -202,7 +202,7 @@ def test_query_magnitudes_outside_the_fp16_range(qscale):
     assert checked > 0.9 * S * Hq
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (4, 2), (8, 2), (16, 2), (32, 8)])
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (4, 2), (8, 2), (16, 2), (32, 8), (3, 1), (10, 2), (12, 2), (28, 4), (14, 2), (9, 1)])
 def test_gqa_group_sizes(Hq, Hkv):
     hist, S = 40, 50
     qh, kh, vh = make(60, 1, hist, Hq, Hkv)
@@ -306,7 +306,7 @@ def test_random_shapes(seed):
     r = np.random.default_rng(2000 + seed)
     B = int(r.integers(1, 4))
     Hkv = int(r.choice([1, 2, 4]))
-    G = int(r.choice([1, 2, 4, 8]))
+    G = int(r.choice([1, 2, 3, 4, 6, 7, 8]))
     hist = int(r.choice([0, 1, 63, 64, 65, 200, 333]))
     S = int(r.integers(1, 300))
     fp8 = bool(r.integers(0, 2)) and hist > 0
@@ -354,7 +354,7 @@ def test_head_dim_256(hist, S, fp8):
         assert np.array_equal(kc[:, hist:], wk) and np.array_equal(ks[:, hist:], wks)
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(2, 2), (4, 2), (16, 4), (16, 2)])
+@pytest.mark.parametrize("Hq,Hkv", [(2, 2), (4, 2), (16, 4), (16, 2), (6, 2), (7, 1)])
 def test_head_dim_256_group_sizes(Hq, Hkv):
     B, S, hist, D = 1, 70, 100, 256
     q, k, v = make(700 + Hq, B, S, Hq, Hkv, D=D)
