@@ -59,6 +59,7 @@ struct PrefillArgs {
     uint16_t *out;  // [B,S,Hq,D] bf16
     int32_t B, S, Hq, Hkv, G, HG, hist_len;
     int32_t heavy_first;  // the grid outnumbers the CUs: order the query tiles by decreasing work
+    int32_t write_new;    // quantize-on-write of the call's K/V rows by the workgroups that finish early
     float scale_log2e;
 };
 
@@ -691,6 +692,89 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 *(u32x4 *)(op + 128 * c + 8 * r) = w;
             }
     }
+
+    // =============================== quantize-on-write of the call's own K/V ===============================
+    // The query tiles at the front of the prompt walk the fewest keys and finish first: the first half of them
+    // (head group 0 of each kv-head) write the rows of two tiles each into the cache while the late tiles still
+    // compute.  Nothing in this launch reads those rows (the history ends below them).  D/8 lanes own a row, as in
+    // the stand-alone bulk writer, and the arithmetic per element is the same: the same codes and scales.
+    if (a.write_new && hg == 0) {
+#pragma clang fp contract(off)
+        constexpr int LPR = kPD / 8, RPW = 64 / LPR;
+        const int tile = q0 / q_per_wg, tiles = (S + q_per_wg - 1) / q_per_wg;
+        if (tile < (tiles + 1) / 2) {
+            const int t_lo = 2 * tile * q_per_wg, t_hi = min(S, t_lo + 2 * q_per_wg);
+            const int sub = lane % LPR;
+#pragma unroll 2
+            for (int tb = t_lo + wave * RPW; tb < t_hi; tb += kPWaves * RPW) {
+                const int t = tb + lane / LPR;
+                const bool live = t < t_hi;  // lanes of rows past the end still take part in the shuffles
+                const int tt = live ? t : t_hi - 1;
+                const int64_t e0 = (((int64_t)b * S + tt) * a.Hkv + kvh) * kPD + sub * 8;
+                const u32x4 wk = *(const u32x4 *)(a.kn + e0), wv = *(const u32x4 *)(a.vn + e0);
+#pragma unroll
+                for (int which = 0; which < 2; ++which) {
+                    const KvAddr &ad = which ? a.va : a.ka;
+                    const u32x4 w = which ? wv : wk;
+                    float *scales = const_cast<float *>(which ? a.vs : a.ks);
+                    int64_t unit;
+                    int slot;
+                    const bool ok = resolve(ad, b, H + tt, unit, slot) && live;
+                    float x[8];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        x[2 * i] = __uint_as_float(w[i] << 16);
+                        x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+                    }
+                    float sc = 0.0f;
+                    uint32_t packed[2] = {0u, 0u};
+                    if (FP8) {
+                        sc = scales[(int64_t)b * a.Hkv + kvh];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            float y = 0.0f;
+                            if (sc > 0.0f) {
+                                y = x[e] / sc;
+                                if (y > 448.0f) y = 448.0f;
+                                if (y < -448.0f) y = -448.0f;
+                            }
+                            packed[e >> 2] |= f32_to_e4m3fn_bits(y) << (8 * (e & 3));
+                        }
+                    } else {
+                        float m = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float v = fabsf(x[e]);
+                            m = v > m ? v : m;
+                        }
+#pragma unroll
+                        for (int o = LPR / 2; o > 0; o >>= 1) {
+                            const float w2 = __shfl_xor(m, o, 64);
+                            m = m > w2 ? m : w2;
+                        }
+                        if (m > 0.0f) {
+                            sc = m / 127.0f;
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                float qv = rintf(x[e] / sc);
+                                qv = qv > 127.0f ? 127.0f : qv;
+                                qv = qv < -127.0f ? -127.0f : qv;
+                                if (qv != qv) qv = 0.0f;
+                                packed[e >> 2] |= ((uint32_t)(int)qv & 0xffu) << (8 * (e & 3));
+                            }
+                        }
+                    }
+                    if (ok) {
+                        uint8_t *dst = const_cast<uint8_t *>(which ? a.vc : a.kc) + unit * ad.code_stride_seq +
+                                       (int64_t)kvh * ad.code_stride_head + (int64_t)slot * kPD + sub * 8;
+                        *(u32x2 *)dst = (u32x2){packed[0], packed[1]};
+                        if (!FP8 && sub == 0)
+                            scales[unit * ad.scale_stride_seq + (int64_t)kvh * ad.scale_stride_head + slot] = sc;
+                    }
+                }
+            }
+        }
+    }
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
@@ -738,6 +822,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.ka = make_addr(*layout, 0); a.va = make_addr(*layout, 1);
     a.out = (uint16_t *)out;
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
+    a.write_new = quantize_on_write ? 1 : 0;
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
     const int q_per_wg = 16 * ((256 / D) * kPWaves / a.HG);
@@ -753,12 +838,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
         else prefill_attn_kernel<256, false><<<grid, 512, 0, st>>>(a);
     }
     if (int rc = check_launch("prefill_attn")) return rc;
-    if (!quantize_on_write) return HS_OK;
-    if (fp8)
-        return hs_kv_quantize_fp8(k_new, v_new, HS_BF16, (uint8_t *)k_codes, (uint8_t *)v_codes, k_scales, v_scales,
-                                  layout, nullptr, hist_len, B, S, Hkv, D, stream);
-    return hs_kv_quantize_int8(k_new, v_new, HS_BF16, (int8_t *)k_codes, (int8_t *)v_codes, k_scales, v_scales, layout,
-                               nullptr, hist_len, B, S, Hkv, D, stream);
+    return HS_OK;
 }
 
 }  // namespace hs

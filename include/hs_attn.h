@@ -225,7 +225,7 @@ HS_API int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_
                          int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
                          float softmax_scale, int quantize_on_write, hs_stream_t stream);
 /* The same over an FP8 e4m3fn history with per-(sequence, kv-head) scales [B, Hkv] (read, never written: they
- * come from hs_kv_fp8_calibrate or from the model); quantize_on_write uses hs_kv_quantize_fp8. */
+ * come from hs_kv_fp8_calibrate or from the model); quantize_on_write writes the codes hs_kv_quantize_fp8 would. */
 HS_API int hs_prefill_attn_fp8(const void *q, const void *k_new, const void *v_new,
                         uint8_t *k_codes, uint8_t *v_codes, const float *k_scales, const float *v_scales,
                         const hs_kv_layout *layout, int32_t hist_len, void *out,
