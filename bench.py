@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c5-decode|c5-prefill|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c5-decode|c5-prefill|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -36,6 +36,9 @@ WORKLOADS = {
     "c2-ragged": (64, 32, 8, 128, 8192, True, False, 1.0, True),
     "c1": (1, 32, 8, 128, 2048, False, False, 1.0, False),
     "c4": (32, 64, 8, 128, 32768, False, True, 0.5, False),
+    # one sequence with a long context: the reference's usual serving shape (a single stream), split-K over 1024 workgroups
+    "b1-32k": (1, 32, 8, 128, 32768, False, False, 1.0, True),
+    "b4-16k": (4, 32, 8, 128, 16384, False, False, 1.0, True),
     # the head shape of Qwen3.5's full-attention layers (16 query / 4 KV heads of 256), same cache bytes as c2 / half of c4
     "d256-int8": (64, 16, 4, 256, 8192, False, False, 1.0, True),
     "d256-fp8": (32, 16, 4, 256, 32768, False, True, 0.5, False),

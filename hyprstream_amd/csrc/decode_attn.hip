@@ -472,22 +472,47 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 }
 
 // Merge the chunk partials of one (sequence, query head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c.
+// 256 threads: D/4 column lanes (four output elements each) x 1024/D chunk lanes, so the partials of a long
+// sequence (up to 128 chunks) are read by many lanes at once instead of one after the other; the chunk lanes meet
+// in LDS.  D is 64, 128 or 256.
 __global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, const float *part_ml,
                                                           const int32_t *seq_lens, uint16_t *out, int Hq, int nchunks,
-                                                          int chunk_tokens, int max_seq_len) {
-    const int hq = blockIdx.x, b = blockIdx.y, d = threadIdx.x, kD = blockDim.x;  // one thread per output element
+                                                          int chunk_tokens, int max_seq_len, int kD) {
+    const int hq = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
     const int L = min(seq_lens[b], max_seq_len);
     const int n = L <= 0 ? 0 : min(nchunks, (L + chunk_tokens - 1) / chunk_tokens);
     const int64_t row = ((int64_t)b * Hq + hq) * nchunks;
+    __shared__ float sm_max[4], sm_l[16];
+    __shared__ __attribute__((aligned(16))) float sm_o[1024];
     float M = -INFINITY;
-    for (int c = 0; c < n; ++c) M = fmaxf(M, part_ml[(row + c) * 2]);
-    float o = 0.0f, l = 0.0f;
-    for (int c = 0; c < n; ++c) {
-        const float w = __builtin_amdgcn_exp2f(part_ml[(row + c) * 2] - M);
-        l += w * part_ml[(row + c) * 2 + 1];
-        o += w * part_o[(row + c) * kD + d];
+    for (int c = tid; c < n; c += 256) M = fmaxf(M, part_ml[(row + c) * 2]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+    if ((tid & 63) == 0) sm_max[tid >> 6] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(sm_max[0], sm_max[1]), fmaxf(sm_max[2], sm_max[3]));
+    const int cx = kD >> 2, tx = tid % cx, ty = tid / cx, ny = 256 / cx;
+    float4v o = {0.f, 0.f, 0.f, 0.f};
+    float l = 0.0f;
+#pragma unroll 4
+    for (int c = ty; c < n; c += ny) {
+        const float m = part_ml[(row + c) * 2], lc = part_ml[(row + c) * 2 + 1];
+        const float4v v = *(const float4v *)(part_o + (row + c) * kD + 4 * tx);
+        const float w = __builtin_amdgcn_exp2f(m - M);
+        l += w * lc;
+        o += w * v;
     }
-    out[((int64_t)b * Hq + hq) * kD + d] = (uint16_t)f32_to_bf16_bits(n > 0 ? o / l : 0.0f);
+    *(float4v *)&sm_o[ty * kD + 4 * tx] = o;
+    if (tx == 0) sm_l[ty] = l;
+    __syncthreads();
+    if (tid < kD) {
+        float os = 0.0f, ls = 0.0f;
+        for (int y = 0; y < ny; ++y) {
+            os += sm_o[y * kD + tid];
+            ls += sm_l[y];
+        }
+        out[((int64_t)b * Hq + hq) * kD + tid] = (uint16_t)f32_to_bf16_bits(n > 0 ? os / ls : 0.0f);
+    }
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
@@ -497,11 +522,14 @@ constexpr int kMaxHintedChunks = 16;  // most chunks a sequence is cut into on t
 static int pick_chunk_tokens(int B, int Hkv, int max_seq_len, int64_t total_tokens_hint) {
     // A workgroup costs about 1.5 us of prologue/epilogue, so chunks are as long as the grid allows:
     // with >= 512 (sequence, kv-head) units (two resident workgroups on each of 256 CUs) nothing is
-    // split and the step is a single launch; below that, split until about 1024 workgroups exist.
-    // Chunks are a multiple of 128 tokens (a whole number of wavefront steps at every head_dim).  Measured on MI355X: B=64 x 8 heads x
-    // 8192 tokens runs 193 us unsplit, 196 us in 2 chunks, 205 us in 8; B=32 x 8 x 32768 is fastest at 4.
+    // split and the step is a single launch; below that, split until about 512 workgroups exist -- one round of
+    // resident workgroups.  Chunks are a multiple of 128 tokens (a whole number of wavefront steps at every
+    // head_dim).  Measured on MI355X, whole step in us by chunks per sequence: 1 x 8 heads x 32768 tokens: 25.1 at
+    // 128, 20.5 at 64, 20.8 at 32, 29.8 at 16; 4 x 8 x 16384: 39.7 at 64, 33.7 at 32, 30.7 at 16, 31.2 at 8;
+    // 8 x 8 x 16384: 54.5 at 16, 52.9 at 8; 16 x 8 x 8192: 54.3 at 8, 53.8 at 4; 32 x 8 x 32768: the same at 2, 3 and 4;
+    // 64 x 8 x 8192 (unsplit by the rule above): 193 unsplit, 196 in 2, 205 in 8.
     const int64_t units = (int64_t)B * Hkv;
-    int64_t want_chunks = units >= 512 ? 1 : (1024 + units - 1) / units;
+    int64_t want_chunks = units >= 512 ? 1 : (512 + units - 1) / units;
     // Ragged batch (the caller says how many tokens the batch holds in total): unsplit, the longest sequence sets
     // the time of the whole launch while the workgroups of short ones idle.  Cutting at about half the mean length
     // gives every workgroup a similar share and leaves enough of them to refill the CUs as short ones finish.
@@ -600,8 +628,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
         if (int rc = check_launch("decode_attn")) return rc;
     }
     if ((phases & 2) && !a.direct) {
-        decode_merge_kernel<<<dim3(Hq, B), D, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
-                                                             a.nchunks, a.chunk_tokens, max_seq_len);
+        decode_merge_kernel<<<dim3(Hq, B), 256, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
+                                                               a.nchunks, a.chunk_tokens, max_seq_len, D);
         return check_launch("decode_merge");
     }
     return HS_OK;
