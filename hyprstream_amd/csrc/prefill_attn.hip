@@ -89,7 +89,12 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // wavefront with the vector work of the other behind a second barrier per step, or that software-pipelined
 // scores(s+1) against softmax(s) inside one wavefront, were correct but not faster than this order; steps of
 // 64 keys instead of 32 were (the per-step bookkeeping is shared by twice the MFMAs).
-template <int kPD, bool FP8>  // head_dim; format of the history: int8 codes with token scales, or e4m3fn codes with head scales
+// kPD: head_dim the products are laid out for; FP8: the history holds e4m3fn codes with head scales instead of int8
+// codes with token scales; kRow: head_dim of the tensors in memory.  kRow = 64 runs in the kPD = 128 layout with
+// the upper half of every Q operand zero: rows are 64 wide in memory, lanes whose d would be >= 64 re-read the
+// row's first columns (finite values that meet zeros of Q, or feed output rows that are never stored), and half
+// of the matrix work is padding.
+template <int kPD, bool FP8, int kRow = kPD>
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     constexpr int kNB = PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
     typedef HistTile<kPD> HistTile;
@@ -167,6 +172,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     };
 
     const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
+    const float qscale = (kRow < kPD && 8 * KG * lq >= kRow) ? 0.0f : a.scale_log2e;  // padding columns of Q are zero
     const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;  // wavefronts w and w+4 share a SIMD
 
     // =============================== history: int8 cache, f16 MFMA ===============================
@@ -179,15 +185,15 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         bool scaled = false;
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 8 * KG * lq;
+            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + ((8 * KG * lq) & (kRow - 1));
             float qf[8 * KG], amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < KG; ++i) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16) * a.scale_log2e;
-                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * a.scale_log2e;
+                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16) * qscale;
+                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * qscale;
                 }
             }
 #pragma unroll
@@ -224,8 +230,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
         const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
         const int ku4 = wave >> 1, kjp = wave & 1;
-        const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp;
-        const uint32_t koff = krow * kPD + kcol, voff = vkey * kPD + 8 * vx;
+        const int krow = 16 * ku4 + li, kcol = (8 * KG * lq + 16 * kjp) & (kRow - 1), vcol = (8 * vx) & (kRow - 1);
+        const uint32_t koff = krow * kRow + kcol, voff = vkey * kRow + vcol;
         // head_dim 256: the same lane also takes the d-halves jp + 2 (32 codes further) and the d-octet x + 16
         u32x4 rawk[NC];
         u32x2 rawv[NC][2];
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 int64_t unit;
                 int slot;
                 resolve(a.ka, b, t0, unit, slot);
-                kb = a.kc + unit * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)slot * kPD;
+                kb = a.kc + unit * a.ka.code_stride_seq + (int64_t)kvh * a.ka.code_stride_head + (int64_t)slot * kRow;
                 if (!FP8) ksp = a.ks + unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot;
                 kleft = a.ka.capacity_tokens - slot;
             }
@@ -259,18 +265,18 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 int64_t unit;
                 int slot;
                 resolve(a.va, b, t0, unit, slot);
-                vb = a.vc + unit * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)slot * kPD;
+                vb = a.vc + unit * a.va.code_stride_seq + (int64_t)kvh * a.va.code_stride_head + (int64_t)slot * kRow;
                 if (!FP8) vsp = a.vs + unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot;
                 vleft = a.va.capacity_tokens - slot;
             }
             // The loaded values are only touched in commit(): nothing waits for a load here.  Addresses are the
             // step's (scalar) base plus a 32-bit lane offset; only the last, partial step clamps rows.
-            uint32_t ko = koff, vo0 = voff, vo1 = voff + kPD, sk = 4u * krow, sv = 4u * vkey;
+            uint32_t ko = koff, vo0 = voff, vo1 = voff + kRow, sk = 4u * krow, sv = 4u * vkey;
             uint32_t sv1 = sv + 4u;
             if (last < kHStep - 1) {
-                ko = min(krow, last) * kPD + kcol;
-                vo0 = min(vkey, last) * kPD + 8 * vx;
-                vo1 = min(vkey + 1, last) * kPD + 8 * vx;
+                ko = min(krow, last) * kRow + kcol;
+                vo0 = min(vkey, last) * kRow + vcol;
+                vo1 = min(vkey + 1, last) * kRow + vcol;
                 sk = 4u * min(krow, last);
                 sv = 4u * min(vkey, last);
                 sv1 = 4u * min(vkey + 1, last);
@@ -286,7 +292,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
                 rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
             }
-            kb += kHStep * kPD; vb += kHStep * kPD;
+            kb += kHStep * kRow; vb += kHStep * kRow;
             ksp += kHStep; vsp += kHStep;
             kleft -= kHStep; vleft -= kHStep;
         };
@@ -484,14 +490,14 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         int force = H > 0 ? INT_MIN : INT_MAX;  // nothing seen yet: the first step sets the reference
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kPD + 8 * KG * lq;
+            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + ((8 * KG * lq) & (kRow - 1));
 #pragma unroll
             for (int j = 0; j < KG; ++j) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * j);
                 uint32_t o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    o[e] = pack_bf16x2(__uint_as_float(w[e] << 16) * a.scale_log2e, __uint_as_float(w[e] & 0xffff0000u) * a.scale_log2e);
+                    o[e] = pack_bf16x2(__uint_as_float(w[e] << 16) * qscale, __uint_as_float(w[e] & 0xffff0000u) * qscale);
                 qop[nb][j] = pack_bf16x8(o[0], o[1], o[2], o[3]);
             }
             sref[nb] = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
@@ -501,9 +507,9 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         constexpr int kNStep = 64;
         const int nsteps = wg_qlast / kNStep + 1;
         HistTile *ntiles = (HistTile *)lds;
-        const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
-        const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kPD;
-        const int64_t rstride = (int64_t)a.Hkv * kPD;  // elements between consecutive tokens
+        const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kRow;
+        const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kRow;
+        const int64_t rstride = (int64_t)a.Hkv * kRow;  // elements between consecutive tokens
         // producers, split as in the history phase (bf16 rows are operands as they are): wavefront w copies the
         // 16-key block u4 = w/2, d-halves jp = w%2 (32 bytes per lane = operand blocks 2jp and 2jp+1); for V a lane
         // takes the d-octet x = lane%16 of two adjacent keys (16 bytes of each) and stores the eight (key, key+1)
@@ -513,8 +519,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
         const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
         const int ku4 = wave >> 1, kjp = wave & 1;
-        const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp;
-        const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + 8 * vx;  // elements
+        const int krow = 16 * ku4 + li, kcol = (8 * KG * lq + 16 * kjp) & (kRow - 1), vcol = (8 * vx) & (kRow - 1);
+        const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + vcol;  // elements
         u32x4 rawk[NC][2], rawv[NC][2];  // head_dim 256: also the d-halves jp + 2 (32 elements on) and the d-octet x + 16
 #pragma unroll
         for (int c = 0; c < NC; ++c) rawk[c][0] = rawk[c][1] = rawv[c][0] = rawv[c][1] = (u32x4){0u, 0u, 0u, 0u};
@@ -528,8 +534,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 vp1 = vb + voff + (uint32_t)rstride;
             } else {  // rows past the last token repeat it; the causal mask removes them
                 kp = knb + (int64_t)min(t0 + krow, S - 1) * rstride + kcol;
-                vp0 = vnb + (int64_t)min(t0 + vkey, S - 1) * rstride + 8 * vx;
-                vp1 = vnb + (int64_t)min(t0 + vkey + 1, S - 1) * rstride + 8 * vx;
+                vp0 = vnb + (int64_t)min(t0 + vkey, S - 1) * rstride + vcol;
+                vp1 = vnb + (int64_t)min(t0 + vkey + 1, S - 1) * rstride + vcol;
             }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
@@ -680,8 +686,9 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     for (int nb = 0; nb < kNB; ++nb) {
         const float l = l_run[nb][0];
         if (qi[nb] >= S || hg * a.HG + (kNB * wave + nb) % a.HG >= a.G) continue;  // padding columns write nothing
+        if (kRow < kPD && 32 * lq >= kRow) continue;                                  // nor do padding rows of d
         const float inv = 1.0f / l;
-        uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kPD + 32 * lq;
+        uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kRow + 32 * lq;
 #pragma unroll
         for (int c = 0; c < NC; ++c)
 #pragma unroll
@@ -700,7 +707,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     // the stand-alone bulk writer, and the arithmetic per element is the same: the same codes and scales.
     if (a.write_new && hg == 0) {
 #pragma clang fp contract(off)
-        constexpr int LPR = kPD / 8, RPW = 64 / LPR;
+        constexpr int LPR = kRow / 8, RPW = 64 / LPR;
         const int tile = q0 / q_per_wg, tiles = (S + q_per_wg - 1) / q_per_wg;
         if (tile < (tiles + 1) / 2) {
             const int t_lo = 2 * tile * q_per_wg, t_hi = min(S, t_lo + 2 * q_per_wg);
@@ -710,7 +717,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 const int t = tb + lane / LPR;
                 const bool live = t < t_hi;  // lanes of rows past the end still take part in the shuffles
                 const int tt = live ? t : t_hi - 1;
-                const int64_t e0 = (((int64_t)b * S + tt) * a.Hkv + kvh) * kPD + sub * 8;
+                const int64_t e0 = (((int64_t)b * S + tt) * a.Hkv + kvh) * kRow + sub * 8;
                 const u32x4 wk = *(const u32x4 *)(a.kn + e0), wv = *(const u32x4 *)(a.vn + e0);
 #pragma unroll
                 for (int which = 0; which < 2; ++which) {
@@ -766,7 +773,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                     }
                     if (ok) {
                         uint8_t *dst = const_cast<uint8_t *>(which ? a.vc : a.kc) + unit * ad.code_stride_seq +
-                                       (int64_t)kvh * ad.code_stride_head + (int64_t)slot * kPD + sub * 8;
+                                       (int64_t)kvh * ad.code_stride_head + (int64_t)slot * kRow + sub * 8;
                         *(u32x2 *)dst = (u32x2){packed[0], packed[1]};
                         if (!FP8 && sub == 0)
                             scales[unit * ad.scale_stride_seq + (int64_t)kvh * ad.scale_stride_head + slot] = sc;
@@ -797,7 +804,8 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
                           int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale,
                           int quantize_on_write, hs_stream_t stream) {
     if (int rc = validate_layout(layout, B, S, Hkv, D, !fp8)) return rc;
-    if (D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 128 and 256, got %d", D);
+    if (D != 64 && D != 128 && D != 256)
+        return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 64, 128 and 256, got %d", D);
     const bool empty = B == 0 || S == 0;  // an empty problem may come with null pointers (an empty tensor has none)
     if (!empty && (!q || !k_new || !v_new || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if ((hist_len > 0 || quantize_on_write) && (!k_codes || !v_codes || !k_scales || !v_scales))
@@ -825,12 +833,15 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.write_new = quantize_on_write ? 1 : 0;
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
-    const int q_per_wg = 16 * ((256 / D) * kPWaves / a.HG);
+    const int q_per_wg = 16 * ((256 / (D == 64 ? 128 : D)) * kPWaves / a.HG);  // head_dim 64 runs in the 128 layout
     dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * ((G + a.HG - 1) / a.HG), B);
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
-    if (D == 128) {
+    if (D == 64) {
+        if (fp8) prefill_attn_kernel<128, true, 64><<<grid, 512, 0, st>>>(a);
+        else prefill_attn_kernel<128, false, 64><<<grid, 512, 0, st>>>(a);
+    } else if (D == 128) {
         if (fp8) prefill_attn_kernel<128, true><<<grid, 512, 0, st>>>(a);
         else prefill_attn_kernel<128, false><<<grid, 512, 0, st>>>(a);
     } else {

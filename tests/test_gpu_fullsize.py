@@ -123,7 +123,7 @@ def test_config4_full_size_fp8_decode():
     sample_check(out, q, kc, vc, ks, vs, full.cpu().numpy(), [(0, 0), (31, 7)], 8, True)
 
 
-@pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (16, 4, 256)])
+@pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (16, 4, 256), (32, 8, 64)])
 def test_config3_full_size_chunked_prefill(Hq, Hkv, D):
     """B=4 x 4096 tokens in 512-token chunks: sampled query rows of every chunk against the oracle over
     [dequantized int8 cache of earlier chunks | own bf16 K/V]; the cache ends up equal to one-shot quantization.

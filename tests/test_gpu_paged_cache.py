@@ -66,7 +66,7 @@ def test_update_across_block_boundaries_and_truncate():
     assert np.array_equal(gk.cpu().numpy(), _dense_reference(k))
 
 
-@pytest.mark.parametrize("D", [128, 256])
+@pytest.mark.parametrize("D", [64, 128, 256])
 def test_chunked_prefill_through_a_paged_cache(D):
     """Two prompt chunks that cross block boundaries: attention of each chunk over [cached blocks | itself] against
     the oracle, and the blocks end up holding what update() would have written."""

@@ -312,11 +312,13 @@ def test_random_shapes(seed):
     fp8 = bool(r.integers(0, 2)) and hist > 0
     sigma = 0.5 if fp8 else 1.0
     Hq = Hkv * G
-    q, k, v = make(300 + seed, B, S, Hq, Hkv, sigma=sigma)
-    c = DeviceCache(B, Hkv, hist + S + int(r.integers(0, 50)), 128, fp8=fp8)
+    pad = int(r.integers(0, 50))
+    D = int(r.choice([64, 128]))
+    q, k, v = make(300 + seed, B, S, Hq, Hkv, D=D, sigma=sigma)
+    c = DeviceCache(B, Hkv, hist + S + pad, D, fp8=fp8)
     kd = vd = None
     if hist > 0:
-        _, kh, vh = make(400 + seed, B, hist, Hq, Hkv, sigma=sigma)
+        _, kh, vh = make(400 + seed, B, hist, Hq, Hkv, D=D, sigma=sigma)
         hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
         if fp8:
             hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
@@ -325,14 +327,16 @@ def test_random_shapes(seed):
         deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
         kd, vd = deq(kc, ks), deq(vc, vs)
     got = gpu_prefill(c, q, k, v, hist)
-    compare(got, oracle_prefill(q, kd, vd, k, v), "random B=%d Hkv=%d G=%d hist=%d S=%d fp8=%s" % (B, Hkv, G, hist, S, fp8))
+    compare(got, oracle_prefill(q, kd, vd, k, v), "random B=%d Hkv=%d G=%d D=%d hist=%d S=%d fp8=%s" % (B, Hkv, G, D, hist, S, fp8))
 
 
 # ------------------------------------------------------------------ head_dim 256 (128 query columns per workgroup)
 @pytest.mark.parametrize("hist,S,fp8", [(0, 1, False), (0, 33, False), (0, 257, False), (19, 5, False), (64, 64, False),
                                         (200, 130, False), (333, 200, True), (65, 31, True)])
-def test_head_dim_256(hist, S, fp8):
-    B, Hq, Hkv, D = 2, 8, 2, 256
+@pytest.mark.parametrize("D", [256, 64])
+def test_head_dim_256_and_64(hist, S, fp8, D):
+    """head_dim 256 is an instance of its own; head_dim 64 runs in the 128 layout with zero padding of Q."""
+    B, Hq, Hkv = 2, 8, 2
     sigma = 0.5 if fp8 else 1.0
     q, k, v = make(500 + hist + S, B, S, Hq, Hkv, D=D, sigma=sigma)
     c = DeviceCache(B, Hkv, hist + S, D, fp8=fp8)
@@ -347,20 +351,21 @@ def test_head_dim_256(hist, S, fp8):
         deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
         kd, vd = deq(kc, ks), deq(vc, vs)
     got = gpu_prefill(c, q, k, v, hist)
-    compare(got, oracle_prefill(q, kd, vd, k, v), "d256 hist=%d S=%d fp8=%s" % (hist, S, fp8))
+    compare(got, oracle_prefill(q, kd, vd, k, v), "d%d hist=%d S=%d fp8=%s" % (D, hist, S, fp8))
     if not fp8:  # the new rows were cached behind the history with the oracle's codes
         kc, vc, ks, vs = c.canonical(hist + S)
         wk, wks = oracle.quant_int8(k)
         assert np.array_equal(kc[:, hist:], wk) and np.array_equal(ks[:, hist:], wks)
 
 
+@pytest.mark.parametrize("D", [256, 64])
 @pytest.mark.parametrize("Hq,Hkv", [(2, 2), (4, 2), (16, 4), (16, 2), (6, 2), (7, 1)])
-def test_head_dim_256_group_sizes(Hq, Hkv):
-    B, S, hist, D = 1, 70, 100, 256
+def test_head_dim_256_and_64_group_sizes(Hq, Hkv, D):
+    B, S, hist = 1, 70, 100
     q, k, v = make(700 + Hq, B, S, Hq, Hkv, D=D)
     _, kh, vh = make(701 + Hq, B, hist, Hq, Hkv, D=D)
     c = DeviceCache(B, Hkv, hist + S, D)
     c.write(torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16(), None, 0)
     kc, vc, ks, vs = c.canonical(hist)
     got = gpu_prefill(c, q, k, v, hist)
-    compare(got, oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v), "d256 gqa %d/%d" % (Hq, Hkv))
+    compare(got, oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v), "d%d gqa %d/%d" % (D, Hq, Hkv))
