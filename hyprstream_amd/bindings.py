@@ -25,7 +25,7 @@ EXPORTS = [
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
-    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_forward_chunked", "hs_deltanet_chunked_workspace_bytes",
+    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_forward_chunked", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
 
@@ -201,11 +201,19 @@ def decode_step_rope(q, k_new, v_new, rope_sin, rope_cos, k_codes, v_codes, k_sc
 
 
 def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, hist_len, out, softmax_scale,
-                 quantize_on_write=True, fp8=False):
-    """Causal attention of S new tokens over [int8 or fp8 history | their own bf16 K/V]; optionally caches them."""
+                 quantize_on_write=True, fp8=False, hist_lens=None):
+    """Causal attention of S new tokens over [int8 or fp8 history | their own bf16 K/V]; optionally caches them.
+    hist_lens (int32 device tensor [B]): rows at different positions; hist_len is then their upper bound."""
     B, S, Hq, D = q.shape
     Hkv = k_new.shape[2]
     assert q.is_contiguous() and k_new.is_contiguous() and v_new.is_contiguous() and out.is_contiguous()
+    if hist_lens is not None:
+        assert str(hist_lens.dtype) == "torch.int32" and hist_lens.numel() == B and hist_lens.is_contiguous()
+        fn = lib().hs_prefill_attn_fp8_ragged if fp8 else lib().hs_prefill_attn_int8_ragged
+        check(fn(_ptr(q), _ptr(k_new), _ptr(v_new), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales), _ptr(v_scales),
+                 ctypes.byref(layout), _ptr(hist_lens), ctypes.c_int32(hist_len), _ptr(out), B, S, Hq, Hkv, D,
+                 ctypes.c_float(softmax_scale), int(bool(quantize_on_write)), _stream()))
+        return
     fn = lib().hs_prefill_attn_fp8 if fp8 else lib().hs_prefill_attn_int8
     check(fn(_ptr(q), _ptr(k_new), _ptr(v_new), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales),
                                      _ptr(v_scales), ctypes.byref(layout), ctypes.c_int32(hist_len), _ptr(out),

@@ -58,6 +58,7 @@ struct PrefillArgs {
     KvAddr ka, va;
     uint16_t *out;  // [B,S,Hq,D] bf16
     int32_t B, S, Hq, Hkv, G, HG, hist_len;
+    const int32_t *hist_lens;  // optional, device [B]: cached tokens per sequence (then hist_len is their upper bound)
     int32_t heavy_first;  // the grid outnumbers the CUs: order the query tiles by decreasing work
     int32_t write_new;    // quantize-on-write of the call's K/V rows by the workgroups that finish early
     float scale_log2e;
@@ -121,7 +122,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     const int b = bz;
     const int groups = (a.G + a.HG - 1) / a.HG;  // the last group of a kv-head may be partly padding (G = 3, 5, 6, 7 ...)
     const int kvh = by / groups, hg = by % groups;
-    const int S = a.S, H = a.hist_len;
+    const int S = a.S, H = a.hist_lens ? min(max(a.hist_lens[b], 0), a.hist_len) : a.hist_len;
     const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
     const int q0 = bx * q_per_wg;
     if (q0 >= S) return;
@@ -802,7 +803,7 @@ static int compute_units() {
 static int launch_prefill(bool fp8, const void *q, const void *k_new, const void *v_new, void *k_codes, void *v_codes,
                           float *k_scales, float *v_scales, const hs_kv_layout *layout, int32_t hist_len, void *out,
                           int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale,
-                          int quantize_on_write, hs_stream_t stream) {
+                          int quantize_on_write, hs_stream_t stream, const int32_t *hist_lens = nullptr) {
     if (int rc = validate_layout(layout, B, S, Hkv, D, !fp8)) return rc;
     if (D != 64 && D != 128 && D != 256)
         return fail(HS_ERR_INVALID_ARGUMENT, "prefill attention is built for head_dim 64, 128 and 256, got %d", D);
@@ -830,6 +831,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.ka = make_addr(*layout, 0); a.va = make_addr(*layout, 1);
     a.out = (uint16_t *)out;
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
+    a.hist_lens = hist_lens;
     a.write_new = quantize_on_write ? 1 : 0;
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
@@ -870,6 +872,25 @@ int hs_prefill_attn_fp8(const void *q, const void *k_new, const void *v_new, uin
                         int quantize_on_write, hs_stream_t stream) {
     return hs::launch_prefill(true, q, k_new, v_new, k_codes, v_codes, (float *)k_scales, (float *)v_scales, layout,
                               hist_len, out, B, S, Hq, Hkv, D, softmax_scale, quantize_on_write, stream);
+}
+
+int hs_prefill_attn_int8_ragged(const void *q, const void *k_new, const void *v_new, int8_t *k_codes, int8_t *v_codes,
+                                float *k_scales, float *v_scales, const hs_kv_layout *layout, const int32_t *hist_lens,
+                                int32_t max_hist_len, void *out, int32_t B, int32_t S, int32_t Hq, int32_t Hkv,
+                                int32_t D, float softmax_scale, int quantize_on_write, hs_stream_t stream) {
+    if (B > 0 && !hist_lens) return hs::fail(HS_ERR_INVALID_ARGUMENT, "hist_lens is NULL");
+    return hs::launch_prefill(false, q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, max_hist_len, out, B,
+                              S, Hq, Hkv, D, softmax_scale, quantize_on_write, stream, hist_lens);
+}
+
+int hs_prefill_attn_fp8_ragged(const void *q, const void *k_new, const void *v_new, uint8_t *k_codes, uint8_t *v_codes,
+                               const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                               const int32_t *hist_lens, int32_t max_hist_len, void *out, int32_t B, int32_t S,
+                               int32_t Hq, int32_t Hkv, int32_t D, float softmax_scale, int quantize_on_write,
+                               hs_stream_t stream) {
+    if (B > 0 && !hist_lens) return hs::fail(HS_ERR_INVALID_ARGUMENT, "hist_lens is NULL");
+    return hs::launch_prefill(true, q, k_new, v_new, k_codes, v_codes, (float *)k_scales, (float *)v_scales, layout,
+                              max_hist_len, out, B, S, Hq, Hkv, D, softmax_scale, quantize_on_write, stream, hist_lens);
 }
 
 }  // extern "C"

@@ -232,6 +232,22 @@ HS_API int hs_prefill_attn_fp8(const void *q, const void *k_new, const void *v_n
                         int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
                         float softmax_scale, int quantize_on_write, hs_stream_t stream);
 
+/* The same for a batch whose rows sit at different positions (forward_batched with q_len > 1: every row brings
+ * S new tokens at its own start position, llama.rs:710-844, mask rule llama.rs:2544-2572).  hist_lens: device [B],
+ * cached tokens per sequence, each clamped to [0, max_hist_len]; max_hist_len is the host-side bound the capacity
+ * check uses (max_hist_len + S must fit the cache when quantize_on_write != 0).  Row b attends its hist_lens[b]
+ * cached tokens and its own new tokens causally, and writes them at hist_lens[b] .. hist_lens[b] + S - 1. */
+HS_API int hs_prefill_attn_int8_ragged(const void *q, const void *k_new, const void *v_new,
+                                int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                                const hs_kv_layout *layout, const int32_t *hist_lens, int32_t max_hist_len,
+                                void *out, int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
+                                float softmax_scale, int quantize_on_write, hs_stream_t stream);
+HS_API int hs_prefill_attn_fp8_ragged(const void *q, const void *k_new, const void *v_new,
+                               uint8_t *k_codes, uint8_t *v_codes, const float *k_scales, const float *v_scales,
+                               const hs_kv_layout *layout, const int32_t *hist_lens, int32_t max_hist_len,
+                               void *out, int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
+                               float softmax_scale, int quantize_on_write, hs_stream_t stream);
+
 /* ---- gated delta rule (replaces the decode branch qwen3_5.rs:725-751 and
  * chunked_delta_rule qwen3_5.rs:342-498) -------------------------------------------------------
  * q, k: [B, T, nk, dk] bf16; v: [B, T, nv, dv] bf16; g, beta: [B, T, nv] fp32 (g = log decay <= 0);

@@ -369,3 +369,38 @@ def test_head_dim_256_and_64_group_sizes(Hq, Hkv, D):
     kc, vc, ks, vs = c.canonical(hist)
     got = gpu_prefill(c, q, k, v, hist)
     compare(got, oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v), "d%d gqa %d/%d" % (D, Hq, Hkv))
+
+
+@pytest.mark.parametrize("D,fp8", [(128, False), (128, True), (64, False), (256, False)])
+def test_ragged_history_lengths(D, fp8):
+    """Rows at different positions (the reference's forward_batched with q_len > 1): every row attends its own
+    history length and its new tokens, and caches them behind its own history."""
+    hists, S, Hq, Hkv = [0, 70, 333, 64], 90, 8, 2
+    B, Hmax = len(hists), max(hists)
+    sigma = 0.5 if fp8 else 1.0
+    q, k, v = make(900 + D, B, S, Hq, Hkv, D=D, sigma=sigma)
+    _, kh, vh = make(901 + D, B, Hmax, Hq, Hkv, D=D, sigma=sigma)
+    c = DeviceCache(B, Hkv, Hmax + S + 5, D, fp8=fp8)
+    hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+    if fp8:
+        hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+    c.write(hk, hv, None, 0)  # every row gets Hmax tokens; a row's own history is the first hists[b] of them
+    kc, vc, ks, vs = c.canonical(Hmax)
+    deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
+    kd, vd = deq(kc, ks), deq(vc, vs)
+    qt, kt, vt = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
+    out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(qt, kt, vt, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, Hmax, out, 1.0 / np.sqrt(D),
+                    True, fp8=fp8, hist_lens=torch.tensor(hists, dtype=torch.int32, device=DEV))
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    kc2, vc2, ks2, vs2 = c.canonical(Hmax + S)
+    for b, h in enumerate(hists):
+        want = oracle_prefill(q[b:b + 1], kd[b:b + 1, :h] if h else None, vd[b:b + 1, :h] if h else None, k[b:b + 1], v[b:b + 1])
+        compare(got[b:b + 1], want, "ragged D=%d fp8=%s row %d hist=%d" % (D, fp8, b, h))
+        if not fp8:  # the row's new tokens sit behind its own history with the oracle's codes
+            wk, wks = oracle.quant_int8(k[b:b + 1])
+            wv, wvs = oracle.quant_int8(v[b:b + 1])
+            assert np.array_equal(kc2[b, h:h + S], wk[0]) and np.array_equal(ks2[b, h:h + S], wks[0])
+            assert np.array_equal(vc2[b, h:h + S], wv[0]) and np.array_equal(vs2[b, h:h + S], wvs[0])
+            assert np.array_equal(kc2[b, :h], kc[b, :h])  # and the history below is untouched
