@@ -36,7 +36,7 @@ WORKLOADS = {
     "c2-ragged": (64, 32, 8, 128, 8192, True, False, 1.0, True),
     "c1": (1, 32, 8, 128, 2048, False, False, 1.0, False),
     "c4": (32, 64, 8, 128, 32768, False, True, 0.5, False),
-    # one sequence with a long context: the reference's usual serving shape (a single stream), split-K over 1024 workgroups
+    # one sequence with a long context: the reference's usual serving shape (a single stream), split-K over 512 workgroups
     "b1-32k": (1, 32, 8, 128, 32768, False, False, 1.0, True),
     "b4-16k": (4, 32, 8, 128, 16384, False, False, 1.0, True),
     # the head shape of Qwen3.5's full-attention layers (16 query / 4 KV heads of 256), same cache bytes as c2 / half of c4
