@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c5-decode|c5-prefill|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c5-decode|c5-prefill|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -98,13 +98,13 @@ def cpu_baseline(torch, name, caches, q, lens, Hq, fp8, seconds_budget=20.0):
     }, out
 
 
-def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False):
+def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, b1=False):
     """Config 3: chunked causal prefill, B=4 x 4096 tokens in 512-token chunks, Hq 32 / Hkv 8, D 128.
     One step = all eight chunk calls of one layer (attention + quantize-on-write of every chunk).
     Variants: C = 4096 (the whole prompt in one call), fp8 = an e4m3fn cache with per-head scales, d256 = the head
     shape of Qwen3.5's full-attention layers (Hq 16 / Hkv 4, D 256: the same flops and bytes)."""
     dev = "cuda:0"
-    B, T, Hq, Hkv, D = (4, 4096, 16, 4, 256) if d256 else (4, 4096, 32, 8, 64) if d64 else (4, 4096, 32, 8, 128)
+    B, T, Hq, Hkv, D = (4, 4096, 16, 4, 256) if d256 else (4, 4096, 32, 8, 64) if d64 else (1 if b1 else 4, 4096, 32, 8, 128)
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)
     sigma = 0.5 if fp8 else 1.0
@@ -150,14 +150,14 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False):
     kms = float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
     peak = 2500.0
     res = {
-        "metric": "prefill-attn TFLOP/s (%% bf16 MFMA peak) + tokens/s, B=4 x 4096 in %d-chunks, Llama-3-8B shape" % C,
+        "metric": "prefill-attn TFLOP/s (%% bf16 MFMA peak) + tokens/s, B=%d x 4096 in %d-chunks, Llama-3-8B shape" % (B, C),
         "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 MFMA (new tokens) + f16 MFMA over %s codes (history), f32 accumulate" % ("fp8" if fp8 else "int8"),
         "data": "synthetic (seeded, generated on device)",
-        "config": {"workload": "c3%s: chunked causal prefill B=4 T=4096 chunk=%d Hq=%d Hkv=%d D=%d, %s cache of earlier "
+        "config": {"workload": "c3%s: chunked causal prefill B=%d T=4096 chunk=%d Hq=%d Hkv=%d D=%d, %s cache of earlier "
                                "chunks + own bf16 K/V, quantize-on-write, one layer"
-                               % ("-d256" if d256 else "-d64" if d64 else "-fp8" if fp8 else "-prompt" if C == T else "", C, Hq, Hkv, D,
+                               % ("-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
                                   "fp8 e4m3fn" if fp8 else "int8"),
                    "algorithmic_flops_per_step": int(flops)},
         "tokens_per_s": B * T / (ms * 1e-3),
@@ -237,7 +237,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c5-decode", "c5-prefill", "c5-prefill-recurrent"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c5-decode", "c5-prefill", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
@@ -269,7 +269,7 @@ def main():
         return
     if args.workload.startswith("c3"):
         return bench_prefill(args, torch, hb, wl, C=4096 if args.workload == "c3-prompt" else 512,
-                             fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64")
+                             fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload == "c3-b1")
     if args.workload.startswith("c5"):
         return bench_deltanet(args, torch, hb, wl, "prefill" in args.workload, recurrent=args.workload.endswith("recurrent"))
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]

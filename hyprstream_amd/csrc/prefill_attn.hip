@@ -29,6 +29,7 @@
 // product is the B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16
 // range (|x| > 65024) saturate.
 #include <climits>
+#include <cstdlib>
 #include <type_traits>
 
 #include "mfma_common.hpp"
@@ -95,9 +96,11 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // the upper half of every Q operand zero: rows are 64 wide in memory, lanes whose d would be >= 64 re-read the
 // row's first columns (finite values that meet zeros of Q, or feed output rows that are never stored), and half
 // of the matrix work is padding.
-template <int kPD, bool FP8, int kRow = kPD>
+// kCols: 16-column blocks per wavefront if not PShape's (1 at head_dim 128: half the columns per workgroup, for grids
+// that would leave most CUs without a workgroup).
+template <int kPD, bool FP8, int kRow = kPD, int kCols = 0>
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
-    constexpr int kNB = PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
+    constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
     typedef HistTile<kPD> HistTile;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];  // two step buffers
     const int lane = threadIdx.x & 63;
@@ -835,14 +838,30 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.write_new = quantize_on_write ? 1 : 0;
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
-    const int q_per_wg = 16 * ((256 / (D == 64 ? 128 : D)) * kPWaves / a.HG);  // head_dim 64 runs in the 128 layout
+    int q_per_wg = 16 * ((256 / (D == 64 ? 128 : D)) * kPWaves / a.HG);  // head_dim 64 runs in the 128 layout
     dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * ((G + a.HG - 1) / a.HG), B);
+    // A small problem (one short sequence, a chunk of a single prompt) would occupy a fraction of the CUs with 256
+    // columns per workgroup: with half the columns there are twice the workgroups, each with half the matrix work
+    // per step and the same conversion work.
+    bool narrow = D <= 128 && q_per_wg >= 32 && 2 * (int64_t)grid.x * grid.y * grid.z <= compute_units();
+    if (const char *e = getenv("HS_PREFILL_COLUMNS"))  // tuning knob: 256 or 128 columns per workgroup whatever the grid
+        narrow = D <= 128 && q_per_wg >= 32 && atoi(e) == 128;
+    if (narrow) {
+        q_per_wg /= 2;
+        grid.x = (S + q_per_wg - 1) / q_per_wg;
+    }
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
-    if (D == 64) {
+    if (D == 64 && narrow) {
+        if (fp8) prefill_attn_kernel<128, true, 64, 1><<<grid, 512, 0, st>>>(a);
+        else prefill_attn_kernel<128, false, 64, 1><<<grid, 512, 0, st>>>(a);
+    } else if (D == 64) {
         if (fp8) prefill_attn_kernel<128, true, 64><<<grid, 512, 0, st>>>(a);
         else prefill_attn_kernel<128, false, 64><<<grid, 512, 0, st>>>(a);
+    } else if (D == 128 && narrow) {
+        if (fp8) prefill_attn_kernel<128, true, 128, 1><<<grid, 512, 0, st>>>(a);
+        else prefill_attn_kernel<128, false, 128, 1><<<grid, 512, 0, st>>>(a);
     } else if (D == 128) {
         if (fp8) prefill_attn_kernel<128, true><<<grid, 512, 0, st>>>(a);
         else prefill_attn_kernel<128, false><<<grid, 512, 0, st>>>(a);

@@ -10,6 +10,16 @@ from gpu_util import DEV, DeviceCache, bf16_from_bits, run_decode
 
 pytestmark = pytest.mark.gpu
 
+
+@pytest.fixture(autouse=True, params=["auto", "256", "128"])
+def columns_per_workgroup(request, monkeypatch):
+    """Every test runs with the library's own choice of workgroup width (half-width workgroups for small grids) and
+    with each width forced, so that small shapes exercise both instances of the kernel."""
+    if request.param == "auto":
+        monkeypatch.delenv("HS_PREFILL_COLUMNS", raising=False)
+    else:
+        monkeypatch.setenv("HS_PREFILL_COLUMNS", request.param)
+
 TOL_MAX, TOL_MEAN = 2e-2, 2e-3
 
 
