@@ -165,3 +165,26 @@ def test_chunked_delta_rule_rejects_bad_arguments_before_launching():
     assert b"workspace" in L.hs_attn_last_error()
     assert call(2, 4, 128, None, 0) == hb.HS_ERR_WORKSPACE                # none at all
     assert call(2, 4, 128, ctypes.c_void_p(0x1004), 1 << 30) == hb.HS_ERR_INVALID_ARGUMENT  # misaligned
+
+
+def test_prefill_rejects_bad_arguments_before_launching():
+    """Argument checks of the prefill entry points are host code: head_dim, head grouping, capacity (with the
+    reference's overflow message), and the per-sequence history array of the ragged form."""
+    L = hb.lib()
+    p = ctypes.c_void_p(0x1000)
+    f = ctypes.c_float(0.088)
+
+    def call(lay, hist, B=2, S=8, Hq=8, Hkv=2, D=128, q=p):
+        return L.hs_prefill_attn_int8(q, p, p, p, p, p, p, ctypes.byref(lay), hist, p, B, S, Hq, Hkv, D, f, 1, None)
+
+    assert call(hb.contiguous_layout(2, 64, 96), 0, D=96) == hb.HS_ERR_INVALID_ARGUMENT
+    lay = hb.contiguous_layout(2, 64, 128)
+    assert call(lay, 0, Hq=7) == hb.HS_ERR_INVALID_ARGUMENT          # Hq is not a multiple of Hkv
+    assert call(lay, -1) == hb.HS_ERR_INVALID_ARGUMENT
+    assert call(lay, 0, q=None) == hb.HS_ERR_INVALID_ARGUMENT
+    assert call(lay, 60) == hb.HS_ERR_OVERFLOW and b"Cache overflow" in L.hs_attn_last_error()
+    rc = L.hs_prefill_attn_int8_ragged(p, p, p, p, p, p, p, ctypes.byref(lay), None, 16, p, 2, 8, 8, 2, 128, f, 1, None)
+    assert rc == hb.HS_ERR_INVALID_ARGUMENT and b"hist_lens" in L.hs_attn_last_error()
+    rc = L.hs_prefill_attn_int8_ragged(p, p, p, p, p, p, p, ctypes.byref(lay), p, 60, p, 2, 8, 8, 2, 128, f, 1, None)
+    assert rc == hb.HS_ERR_OVERFLOW                                   # the bound, not the array, is what the host checks
+    assert call(lay, 0, B=0) == hb.HS_OK and call(lay, 0, S=0) == hb.HS_OK  # empty problems are not an error
