@@ -30,6 +30,28 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E peak
 
+
+def settle(torch, step, window=20, min_launches=300, max_launches=4000, tol=0.01):
+    """Untimed settling phase, independent of --warmup: the first few hundred launches after set-up run a few per
+    cent slower (clocks and memory settle).  Runs `step(i)` in windows of `window` launches, each window timed with
+    a pair of events on the launch stream, until at least `min_launches` have run and three consecutive windows
+    agree within `tol` (or `max_launches` is reached).  Returns (launches run, last window's us per launch)."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    hist, n = [], 0
+    while n < max_launches:
+        e0.record()
+        for i in range(window):
+            step(n + i)
+        e1.record()
+        e1.synchronize()
+        n += window
+        hist.append(e0.elapsed_time(e1) / window * 1e3)
+        if n >= min_launches and len(hist) >= 3:
+            last = hist[-3:]
+            if max(last) - min(last) <= tol * min(last):
+                break
+    return n, hist[-1]
+
 WORKLOADS = {
     # name: (B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers)
     "c2": (64, 32, 8, 128, 8192, False, False, 1.0, True),
@@ -129,6 +151,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         for i, (qc, kcn, vcn) in enumerate(chunks):
             hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8)
 
+    settle(torch, lambda i: step(), window=10, min_launches=100, max_launches=1000)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -139,7 +162,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
     ms = (time.perf_counter() - t0) / args.steps * 1e3
     flops = 4 * B * Hq * D * T * (T + 1) // 2  # causal half, QK^T + PV
     # attention kernel alone (no quantize-on-write), HIP events on its stream
-    n_ev = min(args.steps, 50)
+    n_ev = 50
     e0 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
     e1 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
     for i in range(n_ev):
@@ -197,19 +220,23 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False):
         else:
             hb.deltanet_forward(q, k, v, g, beta, states[i % ncopies], out, qs, False)
 
+    settle(torch, step, window=10 if prefill else 20, min_launches=100 if prefill else 300, max_launches=2000)
     for i in range(args.warmup):
         step(i)
-    n_ev = args.steps
-    e0 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
-    e1 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    n_ev = 100
+    e0 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
+    e1 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
+    for i in range(n_ev):
         e0[i].record()
         step(i)
         e1[i].record()
     torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) / args.steps * 1e3
     kms = float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
     state_bytes = 2 * B * nv * d * d * 4
     io_bytes = B * T * (2 * nk * d * 2 + nv * d * 2 + 2 * nv * 4 + nv * d * 4)
@@ -327,6 +354,7 @@ def main():
         kc, vc, ks, vs = caches[i % ncopies]
         hb.decode_step(q, k_new, v_new, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8)
 
+    settled, settled_us = settle(torch, step)
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -369,7 +397,7 @@ def main():
     single = nchunks == 1
     write_bytes = B * Hkv * D * (2 * 2 + 2 * 1) + (0 if fp8 else B * Hkv * 2 * 4)
     kern_bytes = step_bytes if single else step_bytes - write_bytes
-    n_ev = min(args.steps, 100)
+    n_ev = 200  # independent of --steps: a short timed region must not shorten the kernel statistics
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n_ev)]
     for i in range(n_ev):
         kc, vc, ks, vs = caches[i % ncopies]
@@ -388,11 +416,15 @@ def main():
     k_avg_ms = float(kt.mean())
     achieved = kern_bytes / (k_avg_ms * 1e-3) / 1e9
 
-    traffic = None
+    # HBM bytes per launch are a recorded counter figure (two rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE, scaled
+    # by a plain copy of known size), not something this run measures: the source file is named beside the number.
+    traffic, traffic_source = None, None
     tpath = os.path.join(ROOT, "profiles", "decode_attn_traffic.json")
     if os.path.exists(tpath):
         try:
             traffic = json.load(open(tpath)).get(args.workload)
+            if traffic is not None:
+                traffic_source = "recorded rocprofv3 counters: profiles/decode_attn_traffic.json (not measured in this run)"
         except Exception:
             traffic = None
 
@@ -410,6 +442,7 @@ def main():
         "tokens_per_s": B / (ms_per_step * 1e-3),
         "roofline": {"bound": "hbm", "kernel": "decode_attn_kernel", "achieved": achieved, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
+                     "traffic_source": traffic_source, "settle_launches": settled, "settled_us_per_launch": settled_us,
                      "avg_kernel_us": k_avg_ms * 1e3, "min_kernel_us": float(kt.min()) * 1e3,
                      "algorithmic_bytes_per_launch": int(kern_bytes), "launches_timed": n_ev},
     }

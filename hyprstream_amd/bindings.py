@@ -41,6 +41,8 @@ class KvLayout(ctypes.Structure):
         ("k_block_table", ctypes.c_void_p),
         ("v_block_table", ctypes.c_void_p),
         ("total_tokens_hint", ctypes.c_int64),
+        ("prefill_columns_hint", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 
@@ -75,14 +77,14 @@ def check(rc):
 def contiguous_layout(Hkv, capacity_tokens, D, scale_pad=4):
     """Head-major cache of one buffer per tensor: codes [B, Hkv, cap, D], scales [B, Hkv, cap_padded]."""
     cap_s = (capacity_tokens + scale_pad - 1) // scale_pad * scale_pad
-    return KvLayout(Hkv * capacity_tokens * D, capacity_tokens * D, Hkv * cap_s, cap_s, capacity_tokens, 0, None, None, 0)
+    return KvLayout(Hkv * capacity_tokens * D, capacity_tokens * D, Hkv * cap_s, cap_s, capacity_tokens, 0, None, None, 0, 0, 0)
 
 
 def paged_layout(Hkv, block_tokens, D, k_table, v_table):
     """Pool of blocks [nblocks, Hkv, block_tokens, D]; tables are int32 device tensors [B, max_blocks]."""
     assert k_table.dtype.is_signed and k_table.element_size() == 4 and k_table.is_contiguous()
     lay = KvLayout(Hkv * block_tokens * D, block_tokens * D, Hkv * block_tokens, block_tokens, block_tokens,
-                   k_table.shape[1], k_table.data_ptr(), v_table.data_ptr(), 0)
+                   k_table.shape[1], k_table.data_ptr(), v_table.data_ptr(), 0, 0, 0)
     lay._tables = (k_table, v_table)  # the struct holds raw addresses: the tensors must live as long as it does
     return lay
 
@@ -200,11 +202,16 @@ def decode_step_rope(q, k_new, v_new, rope_sin, rope_cos, k_codes, v_codes, k_sc
                                          ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
 
 
+PREFILL_COLUMNS = 0  # default for prefill_attn's `columns` (tests set it to run every case at each workgroup width)
+
+
 def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, hist_len, out, softmax_scale,
-                 quantize_on_write=True, fp8=False, hist_lens=None):
+                 quantize_on_write=True, fp8=False, hist_lens=None, columns=None):
     """Causal attention of S new tokens over [int8 or fp8 history | their own bf16 K/V]; optionally caches them.
-    hist_lens (int32 device tensor [B]): rows at different positions; hist_len is then their upper bound."""
+    hist_lens (int32 device tensor [B]): rows at different positions; hist_len is then their upper bound.
+    columns: 0 = the library's choice of workgroup width, 256 or 128 fixes it (layout.prefill_columns_hint)."""
     B, S, Hq, D = q.shape
+    layout.prefill_columns_hint = PREFILL_COLUMNS if columns is None else columns
     Hkv = k_new.shape[2]
     assert q.is_contiguous() and k_new.is_contiguous() and v_new.is_contiguous() and out.is_contiguous()
     if hist_lens is not None:

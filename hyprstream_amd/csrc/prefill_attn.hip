@@ -29,7 +29,6 @@
 // product is the B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16
 // range (|x| > 65024) saturate.
 #include <climits>
-#include <cstdlib>
 #include <type_traits>
 
 #include "mfma_common.hpp"
@@ -844,8 +843,8 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     // columns per workgroup: with half the columns there are twice the workgroups, each with half the matrix work
     // per step and the same conversion work.
     bool narrow = D <= 128 && q_per_wg >= 32 && 2 * (int64_t)grid.x * grid.y * grid.z <= compute_units();
-    if (const char *e = getenv("HS_PREFILL_COLUMNS"))  // tuning knob: 256 or 128 columns per workgroup whatever the grid
-        narrow = D <= 128 && q_per_wg >= 32 && atoi(e) == 128;
+    if (layout->prefill_columns_hint == 256 || layout->prefill_columns_hint == 128)  // the caller fixes the width
+        narrow = D <= 128 && q_per_wg >= 32 && layout->prefill_columns_hint == 128;
     if (narrow) {
         q_per_wg /= 2;
         grid.x = (S + q_per_wg - 1) / q_per_wg;

@@ -45,7 +45,7 @@
 extern "C" {
 #endif
 
-#define HS_ATTN_ABI_VERSION 2
+#define HS_ATTN_ABI_VERSION 3
 
 typedef void *hs_stream_t; /* hipStream_t */
 
@@ -78,6 +78,10 @@ typedef struct hs_kv_layout {
     int64_t total_tokens_hint;  /* decode only, optional: sum of seq_lens over the batch as the host knows it
                                    (0 = unknown).  A ragged batch is then cut into chunks of about half the mean
                                    length so that long sequences do not set the time of the launch. */
+    int32_t prefill_columns_hint; /* prefill only, optional: 0 = the library picks the (query, head) columns a
+                                   workgroup owns from the size of the grid; 256 or 128 fixes them (results are the
+                                   same within rounding either way; head_dim 256 always uses its one width). */
+    int32_t reserved;           /* set to 0 */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */

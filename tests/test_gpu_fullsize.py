@@ -81,6 +81,45 @@ def sample_check(out, q, kc, vc, ks, vs, lens, units, G, fp8):
                                   np.array([n], np.int32), 1.0 / np.sqrt(q.shape[-1]))[0]
         d = np.abs(out[b, h * G:(h + 1) * G].float().cpu().numpy() - want)
         assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, d.max(), d.mean())
+        # at these lengths the outputs themselves are about the size of the absolute tolerance (an average of thousands
+        # of N(0,1) values), so the check that bites is relative: 2^-7 of the unit's largest output
+        assert d.max() <= 2.0 ** -7 * np.abs(want).max(), (b, h, d.max(), np.abs(want).max())
+
+
+def decode_step_check(g, q, kc, vc, ks, vs, lay, lens, Hkv, T, fp8, sigma, outliers, units):
+    """The fused step (new-token write in the attention launch) at full size against (a) the oracle's quantizer for
+    the written rows, bit for bit, (b) the unfused flow -- the stand-alone writer then attention -- bit for bit,
+    (c) the oracle's attention for sampled units.  Restores nothing: the caches hold the new token afterwards."""
+    B, Hq, D = q.shape
+    G = Hq // Hkv
+    k_new, v_new = source(g, (B, 1, Hkv, D), sigma, outliers), source(g, (B, 1, Hkv, D), sigma, outliers)
+    kc2, vc2, ks2, vs2 = kc.clone(), vc.clone(), ks.clone(), vs.clone()
+    pos = (lens - 1).contiguous()
+    # unfused: writer, then attention
+    (hb.kv_quantize_fp8 if fp8 else hb.kv_quantize_int8)(k_new, v_new, kc2, vc2, ks2, vs2, lay, pos, 0)
+    want = decode(q, kc2, vc2, ks2, vs2, lay, lens, Hkv, T, fp8)
+    # fused
+    out = torch.full((B, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_step(q, k_new, v_new, kc, vc, ks, vs, lay, lens, out, ws, Hkv, T, 1.0 / np.sqrt(D), fp8=fp8)
+    torch.cuda.synchronize()
+    assert torch.equal(kc, kc2) and torch.equal(vc, vc2), "fused write differs from the stand-alone writer"
+    assert torch.equal(ks, ks2) and torch.equal(vs, vs2)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16)), "fused step differs from write-then-attend"
+    lens_h = lens.cpu().numpy()
+    kn, vn = k_new.float().cpu().numpy(), v_new.float().cpu().numpy()
+    for b in sorted({0, B - 1} | {u[0] for u in units}):
+        p = int(lens_h[b]) - 1
+        if fp8:
+            sk, sv = ks[b].cpu().numpy()[None], vs[b].cpu().numpy()[None]
+            assert np.array_equal(oracle.quant_fp8(kn[b:b + 1], sk)[0, 0], kc[b, :, p].cpu().numpy()), b
+            assert np.array_equal(oracle.quant_fp8(vn[b:b + 1], sv)[0, 0], vc[b, :, p].cpu().numpy()), b
+        else:
+            wk, wks = oracle.quant_int8(kn[b:b + 1])
+            wv, wvs = oracle.quant_int8(vn[b:b + 1])
+            assert np.array_equal(wk[0, 0], kc[b, :, p].cpu().numpy()) and np.array_equal(wks[0, 0], ks[b, :, p].cpu().numpy()), b
+            assert np.array_equal(wv[0, 0], vc[b, :, p].cpu().numpy()) and np.array_equal(wvs[0, 0], vs[b, :, p].cpu().numpy()), b
+    sample_check(out, q, kc, vc, ks, vs, lens_h, units, G, fp8)
 
 
 def test_config2_full_size_int8_decode():
@@ -98,6 +137,9 @@ def test_config2_full_size_int8_decode():
     sample_check(out, q, kc, vc, ks, vs, full.cpu().numpy(), [(0, 0), (17, 5), (63, 7)], 4, False)
     two = decode(q, kc, vc, ks, vs, lay, full, Hkv, T, False, phases=12)  # partials + stand-alone merge
     assert (two.float() - out.float()).abs().max() <= 2 ** -8 * max(1.0, float(out.float().abs().max()))
+    # the launch the benchmark times: one fused step (new token per sequence quantized on write, single launch)
+    assert hb.decode_num_chunks(B, Hkv, T) == 1
+    decode_step_check(g, q, kc, vc, ks, vs, lay, full, Hkv, T, False, 1.0, True, [(0, 3), (29, 0), (63, 7)])
     lens = torch.randint(512, T + 1, (B,), generator=g, device=DEV, dtype=torch.int32)
     rag = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
     sample_check(rag, q, kc, vc, ks, vs, lens.cpu().numpy(), [(1, 2), (40, 6)], 4, False)
@@ -121,6 +163,8 @@ def test_config4_full_size_fp8_decode():
     out = decode(q, kc, vc, ks, vs, lay, full, Hkv, T, True)
     assert torch.isfinite(out.float()).all()
     sample_check(out, q, kc, vc, ks, vs, full.cpu().numpy(), [(0, 0), (31, 7)], 8, True)
+    # the fused step at this size: two chunks per sequence, the chunk that owns the sequence end writes the token
+    decode_step_check(g, q, kc, vc, ks, vs, lay, full, Hkv, T, True, 0.5, False, [(3, 1), (31, 6)])
 
 
 @pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (16, 4, 256), (32, 8, 64)])

@@ -15,10 +15,7 @@ pytestmark = pytest.mark.gpu
 def columns_per_workgroup(request, monkeypatch):
     """Every test runs with the library's own choice of workgroup width (half-width workgroups for small grids) and
     with each width forced, so that small shapes exercise both instances of the kernel."""
-    if request.param == "auto":
-        monkeypatch.delenv("HS_PREFILL_COLUMNS", raising=False)
-    else:
-        monkeypatch.setenv("HS_PREFILL_COLUMNS", request.param)
+    monkeypatch.setattr(hb, "PREFILL_COLUMNS", 0 if request.param == "auto" else int(request.param))
 
 TOL_MAX, TOL_MEAN = 2e-2, 2e-3
 
