@@ -25,6 +25,7 @@ EXPORTS = [
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
+    "hs_decode_attn_int8_static",
     "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_forward_chunked", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
@@ -175,6 +176,14 @@ def decode_attn(q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, 
              _ptr(seq_lens), _ptr(out), _ptr(workspace),
              ctypes.c_size_t(workspace.numel() * workspace.element_size() if workspace is not None else 0),
              B, Hq, Hkv, D, ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
+
+
+def decode_attn_static(q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, Hkv, max_seq_len, softmax_scale):
+    """hs_decode_attn_int8 without a workspace argument: the split-K partials use the library's built-in scratch."""
+    B, Hq, D = q.shape
+    check(lib().hs_decode_attn_int8_static(_ptr(q), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales), _ptr(v_scales),
+                                           ctypes.byref(layout), _ptr(seq_lens), _ptr(out), B, Hq, Hkv, D,
+                                           ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
 
 
 def decode_step(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace, Hkv,

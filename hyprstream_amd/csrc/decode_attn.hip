@@ -33,9 +33,38 @@
 // is the running max (two butterfly steps over the lanes that share a head).
 //
 // HBM bytes per cached token and kv-head: 2*D codes + 8 B of scales (int8) -- 264 B at D = 128.
+#include <atomic>
+
 #include "quant_device.hpp"
 
 namespace hs {
+
+// Split-K scratch of the one entry point that takes no workspace (hs_decode_attn_int8_static): callers that cannot
+// allocate (code under graph capture, serving loops or harnesses that forbid hipMalloc) get the chunk partials'
+// memory from this array instead of a workspace argument.  Every device the library runs on holds its own copy at its
+// own address for the life of the process.  In host code the NAME below is only a handle for hipGetSymbolAddress, never
+// a device address: host code uses the per-device pointer kept in g_scratch_ptr.
+constexpr size_t kScratchBytes = (size_t)32 << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+static std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the caller's current device; looked up once per device (first call there).
+static int scratch_of_current_device(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(HS_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(HS_ERR_INVALID_ARGUMENT, "device ordinal %d out of range", dev);
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(HS_ERR_LAUNCH, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing first calls store the same address
+    }
+    *out = p;
+    return HS_OK;
+}
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
@@ -556,10 +585,12 @@ struct NewToken {  // optional quantize-on-write of one token per sequence insid
     int rope_len = 0;
 };
 
+// static_scratch: the partials go to this device's copy of `scratch` (ws / ws_bytes ignored) and the size check is
+// against what THIS call's split needs, not the worst case a caller-sized workspace has to cover.
 static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q, void *kc, void *vc, float *ks,
                          float *vs, const hs_kv_layout *l, const int32_t *seq_lens, void *out, void *ws,
                          size_t ws_bytes, int B, int Hq, int Hkv, int D, int max_seq_len, float softmax_scale,
-                         hipStream_t stream) {
+                         hipStream_t stream, bool static_scratch = false) {
     if (int rc = validate_layout(l, B, 0, Hkv, D, !fp8)) return rc;
     if (D != 64 && D != 128 && D != 256)
         return fail(HS_ERR_INVALID_ARGUMENT, "decode attention is built for head_dim 64, 128 and 256, got %d", D);
@@ -579,19 +610,28 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
             return fail(HS_ERR_OVERFLOW, "max_seq_len %d exceeds what the cache can hold (%lld tokens)", max_seq_len,
                         (long long)cap);
     }
-    const size_t need = hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, max_seq_len);
-    if (!ws || ws_bytes < need)
-        return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
-    if (((uintptr_t)ws & 255) != 0) return fail(HS_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
     DecodeArgs a;
+    a.chunk_tokens = pick_chunk_tokens(B, Hkv, max_seq_len, l->total_tokens_hint);
+    a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
+    if (static_scratch) {
+        const size_t need = a.nchunks == 1 ? 0 : (size_t)B * Hq * a.nchunks * ((size_t)D + 2) * sizeof(float);
+        if (need > kScratchBytes)
+            return fail(HS_ERR_WORKSPACE,
+                        "this shape needs %zu bytes of split-K scratch (%d chunks per sequence), the built-in scratch "
+                        "holds %zu: use hs_decode_attn_int8 with a caller workspace", need, a.nchunks, kScratchBytes);
+        if (int rc = scratch_of_current_device(&ws)) return rc;
+    } else {
+        const size_t need = hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, max_seq_len);
+        if (!ws || ws_bytes < need)
+            return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", ws_bytes, need);
+        if (((uintptr_t)ws & 255) != 0) return fail(HS_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+    }
     a.q = (const uint16_t *)q;
     a.kc = (const uint8_t *)kc; a.vc = (const uint8_t *)vc;
     a.ks = ks; a.vs = vs;
     a.ka = make_addr(*l, 0); a.va = make_addr(*l, 1);
     a.seq_lens = seq_lens;
     a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.G = Hq / Hkv; a.max_seq_len = max_seq_len;
-    a.chunk_tokens = pick_chunk_tokens(B, Hkv, max_seq_len, l->total_tokens_hint);
-    a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
     a.part_o = (float *)ws;
     a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * D;
     a.out = (uint16_t *)out;
@@ -662,6 +702,15 @@ int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_co
     return hs::launch_decode(false, 3, hs::NewToken(), q, (void *)k_codes, (void *)v_codes, (float *)k_scales,
                              (float *)v_scales, layout, seq_lens, out, workspace, workspace_bytes, B, Hq, Hkv, D,
                              max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_attn_int8_static(const void *q, const int8_t *k_codes, const int8_t *v_codes, const float *k_scales,
+                               const float *v_scales, const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                               int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len, float softmax_scale,
+                               hs_stream_t stream) {
+    return hs::launch_decode(false, 3, hs::NewToken(), q, (void *)k_codes, (void *)v_codes, (float *)k_scales,
+                             (float *)v_scales, layout, seq_lens, out, nullptr, 0, B, Hq, Hkv, D, max_seq_len,
+                             softmax_scale, (hipStream_t)stream, /*static_scratch=*/true);
 }
 
 int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8_t *v_codes, const float *k_scales,

@@ -7,7 +7,8 @@
  * extern "C", raw device pointers, integer sizes, a trailing stream handle
  * (bindings.rs:13 `bnb_stream_t`), the CALLER allocates every buffer and the
  * library keeps no pointer and no state between calls
- * (crates/hyprstream/src/runtime/kv_cache.rs:797-865, 915-957).  Two deliberate
+ * (crates/hyprstream/src/runtime/kv_cache.rs:797-865, 915-957); the one exception
+ * is hs_decode_attn_int8_static, whose split-K scratch is an array inside the library.  Two deliberate
  * differences from that precedent: every entry point returns an int status
  * (0 = HS_OK) with the message available from hs_attn_last_error(), because
  * the bitsandbytes symbols return void and cannot report a bad launch; and
@@ -163,6 +164,21 @@ HS_API int32_t hs_decode_attn_num_chunks(int32_t B, int32_t Hkv, int32_t max_seq
 HS_API int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes,
                         const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
                         const int32_t *seq_lens, void *out, void *workspace, size_t workspace_bytes,
+                        int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                        float softmax_scale, hs_stream_t stream);
+/* hs_decode_attn_int8 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no workspace argument.  It has no counterpart in the reference.  The
+ * split-K partials live in a 32 MiB array inside the library's device image (one copy per GPU the library runs on,
+ * held until the process ends); the call allocates and frees nothing.  Same kernels and same results as
+ * hs_decode_attn_int8.  A shape whose split needs more than 32 MiB of partials
+ * (B * Hq * chunks * (D + 2) * 4 bytes, chunks = hs_decode_attn_num_chunks(...); nothing when chunks == 1) is refused
+ * with HS_ERR_WORKSPACE.  The array keeps the previous call's partials; nothing in it has to start at zero, because the
+ * merge reads only what the same call wrote.  All calls on one GPU share that GPU's array: calls that overlap on one
+ * GPU (different streams or threads) race.  The array's address is looked up on the first call on each device
+ * (hipGetSymbolAddress, no allocation); make that first call outside graph capture. */
+HS_API int hs_decode_attn_int8_static(const void *q, const int8_t *k_codes, const int8_t *v_codes,
+                        const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
+                        const int32_t *seq_lens, void *out,
                         int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
                         float softmax_scale, hs_stream_t stream);
 HS_API int hs_decode_attn_fp8(const void *q, const uint8_t *k_codes, const uint8_t *v_codes,
