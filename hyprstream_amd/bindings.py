@@ -25,7 +25,7 @@ EXPORTS = [
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
-    "hs_decode_attn_int8_static",
+    "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue",
     "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_forward_chunked", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
@@ -45,6 +45,44 @@ class KvLayout(ctypes.Structure):
         ("prefill_columns_hint", ctypes.c_int32),
         ("reserved", ctypes.c_int32),
     ]
+
+
+QKNORM_NONE, QKNORM_LLAMA, QKNORM_QWEN35 = 0, 1, 2
+
+
+class QkPrologue(ctypes.Structure):
+    """Mirror of `struct hs_qk_prologue`."""
+    _fields_ = [
+        ("norm_kind", ctypes.c_int32),
+        ("norm_eps", ctypes.c_float),
+        ("q_norm_weight", ctypes.c_void_p),
+        ("k_norm_weight", ctypes.c_void_p),
+        ("q_norm_head_stride", ctypes.c_int32),
+        ("k_norm_head_stride", ctypes.c_int32),
+        ("rope_sin", ctypes.c_void_p),
+        ("rope_cos", ctypes.c_void_p),
+        ("rope_len", ctypes.c_int32),
+        ("rotary_dim", ctypes.c_int32),
+    ]
+
+
+def qk_prologue(norm_kind=QKNORM_NONE, eps=0.0, q_weight=None, k_weight=None, rope_sin=None, rope_cos=None, rotary_dim=0):
+    """Build an hs_qk_prologue from torch tensors (weights [H, D] or [D]; tables [rope_len, rotary_dim/2])."""
+    p = QkPrologue()
+    p.norm_kind, p.norm_eps = norm_kind, eps
+    keep = [q_weight, k_weight, rope_sin, rope_cos]
+    if q_weight is not None:
+        assert q_weight.is_contiguous()
+        p.q_norm_weight, p.q_norm_head_stride = q_weight.data_ptr(), (q_weight.shape[-1] if q_weight.dim() == 2 else 0)
+    if k_weight is not None:
+        assert k_weight.is_contiguous()
+        p.k_norm_weight, p.k_norm_head_stride = k_weight.data_ptr(), (k_weight.shape[-1] if k_weight.dim() == 2 else 0)
+    if rope_sin is not None:
+        assert rope_sin.is_contiguous() and rope_cos.is_contiguous() and rope_sin.shape == rope_cos.shape
+        p.rope_sin, p.rope_cos, p.rope_len = rope_sin.data_ptr(), rope_cos.data_ptr(), rope_sin.shape[0]
+    p.rotary_dim = rotary_dim
+    p._keep = keep  # the struct holds raw addresses
+    return p
 
 
 class HsError(RuntimeError):
@@ -134,6 +172,41 @@ def rope_apply(x, rope_sin, rope_cos, out, positions=None, start_pos=0, rotary_d
     check(lib().hs_rope_apply_partial(_ptr(x), _dtype_code(x), _ptr(rope_sin), _ptr(rope_cos), ctypes.c_int32(rope_sin.shape[0]),
                                       _ptr(positions), ctypes.c_int32(start_pos), _ptr(out), B, S, H, D, ctypes.c_int32(rd),
                                       _stream()))
+
+
+def qk_prologue_apply(q, k, prologue, q_out, k_out, positions=None, start_pos=0):
+    """QK-norm + rotary embedding of q [B,S,Hq,D] and k [B,S,Hkv,D] in one launch (either pair may be None)."""
+    ref_t = q if q is not None else k
+    B, S, _, D = ref_t.shape
+    Hq = q.shape[2] if q is not None else 0
+    Hkv = k.shape[2] if k is not None else 0
+    for t in (q, k, q_out, k_out):
+        assert t is None or t.is_contiguous()
+    check(lib().hs_qk_prologue_apply(_ptr(q), _ptr(k), _dtype_code(ref_t), ctypes.byref(prologue), _ptr(positions),
+                                     ctypes.c_int32(start_pos), _ptr(q_out), _ptr(k_out), B, S, Hq, Hkv, D, _stream()))
+
+
+def kv_quantize_int8_prologue(k_src, v_src, prologue, k_codes, v_codes, k_scales, v_scales, layout, positions=None,
+                              start_pos=0):
+    """kv_quantize_int8 with K normalised and rotated on the way in."""
+    B, S, Hkv, D = k_src.shape
+    assert k_src.is_contiguous() and v_src.is_contiguous()
+    check(lib().hs_kv_quantize_int8_prologue(_ptr(k_src), _ptr(v_src), _dtype_code(k_src), ctypes.byref(prologue),
+                                             _ptr(k_codes), _ptr(v_codes), _ptr(k_scales), _ptr(v_scales),
+                                             ctypes.byref(layout), _ptr(positions), ctypes.c_int32(start_pos), B, S,
+                                             Hkv, D, _stream()))
+
+
+def decode_step_prologue(q, k_new, v_new, prologue, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out,
+                         workspace, Hkv, max_seq_len, softmax_scale):
+    """decode_step (int8) with the QK-norm and the rotation of q and k_new inside the launch."""
+    B, Hq, D = q.shape
+    assert k_new.shape == (B, 1, Hkv, D) and k_new.is_contiguous() and v_new.is_contiguous()
+    check(lib().hs_decode_step_int8_prologue(_ptr(q), _ptr(k_new), _ptr(v_new), ctypes.byref(prologue), _ptr(k_codes),
+                                             _ptr(v_codes), _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout),
+                                             _ptr(seq_lens), _ptr(out), _ptr(workspace),
+                                             ctypes.c_size_t(workspace.numel() * workspace.element_size()), B, Hq, Hkv,
+                                             D, ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
 
 
 def kv_fp8_calibrate(k_src, v_src, k_scales, v_scales):

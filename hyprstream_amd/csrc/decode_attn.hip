@@ -108,46 +108,100 @@ struct DecodeArgs {
     float scale_log2e;
     // optional rotary embedding of q (bf16 tables [rope_len, D/2]); the new token's K is rotated by nt.rope_*
     const uint16_t *rope_sin, *rope_cos;
-    int32_t rope_len;
+    int32_t rope_len, rotary_dim;
+    NormSpec qnorm;  // optional QK-norm of q ahead of the rotation (the new token's K: nt.norm)
 };
 
-// Half-split rotary embedding of the 32 query elements a lane holds, in bf16 arithmetic (every product and sum
-// rounded to bf16, as the separate libtorch ops of RoPE::apply_rotary_pos_emb do, rope.rs:206-248).  Element
-// qf[8*i + e] is d = 64*(i/2) + 16*lq + 8*(i%2) + e (i < NJ = D/32), so a lane holds both halves of each rotated
-// pair: blocks i and i + NJ/2.  At D = 64 the lane holds d = 16*lq + 8*i + e only, and the other half of each pair sits
-// in the lane 32 further on (or back): the two exchange their elements and each computes its own half.
-template <int NJ>
-__device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
+// Half-split rotary embedding of the query elements a lane holds, in bf16 arithmetic (every product and sum rounded
+// to bf16, as the separate libtorch ops of RoPE::apply_rotary_pos_emb do, rope.rs:206-248).  Element qf[8*i + e] is
+// d = 64*(i/2) + 16*lq + 8*(i%2) + e (i < NJ = D/32; at D = 64: d = 16*lq + 8*i + e).  The first `rd` elements of the
+// head are rotated in pairs (d, d + rd/2), tables [.., rd/2]:
+//   rd >= 128  a lane holds both halves of each pair (register blocks i and i + rd/64);
+//   rd = 64    the halves sit 32 lanes apart (blocks 0 and 1 of lanes lq and lq ^ 2);
+//   rd = 32    16 lanes apart (blocks 0 and 1 of lanes lq = 0 and 1).
+// Cross-lane pairs exchange their elements and each lane computes its own half.
+template <int NJ, int NJR>
+__device__ __forceinline__ void rope_q_inlane(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
 #pragma clang fp contract(off)
     auto rb = [](float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); };
-    if constexpr (NJ == 2) {
-        const bool upper = lq >= 2;  // this lane holds x2 (d >= 32) of its pairs
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int j0 = 16 * (lq & 1) + 8 * i;
-            const u32x4 sw = *(const u32x4 *)(sin_row + j0), cw = *(const u32x4 *)(cos_row + j0);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
-                const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
-                const float mine = qf[8 * i + e], other = __shfl_xor(mine, 32, 64);
-                qf[8 * i + e] = upper ? rb(rb(other * sn) + rb(mine * cs)) : rb(rb(mine * cs) - rb(other * sn));
-            }
-        }
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < NJ / 2; ++i) {
+    for (int i = 0; i < NJR / 2; ++i) {
         const int j0 = 64 * (i >> 1) + 16 * lq + 8 * (i & 1);
         const u32x4 sw = *(const u32x4 *)(sin_row + j0), cw = *(const u32x4 *)(cos_row + j0);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
             const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
-            const float x1 = qf[8 * i + e], x2 = qf[8 * (i + NJ / 2) + e];
+            const float x1 = qf[8 * i + e], x2 = qf[8 * (i + NJR / 2) + e];
             qf[8 * i + e] = rb(rb(x1 * cs) - rb(x2 * sn));
-            qf[8 * (i + NJ / 2) + e] = rb(rb(x1 * sn) + rb(x2 * cs));
+            qf[8 * (i + NJR / 2) + e] = rb(rb(x1 * sn) + rb(x2 * cs));
         }
+    }
+}
+template <int NJ, int XOR>  // rd = 2 * XOR: 64 or 32
+__device__ __forceinline__ void rope_q_crosslane(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq) {
+#pragma clang fp contract(off)
+    auto rb = [](float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); };
+    if (16 * lq >= 2 * XOR) return;  // this lane's elements of blocks 0 and 1 lie beyond the rotated part
+    const bool upper = 16 * lq >= XOR;  // this lane holds x2 of its pairs
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int j0 = ((16 * lq) & (XOR - 1)) + 8 * i;
+        const u32x4 sw = *(const u32x4 *)(sin_row + j0), cw = *(const u32x4 *)(cos_row + j0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
+            const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
+            const float mine = qf[8 * i + e], other = __shfl_xor(mine, XOR, 64);
+            qf[8 * i + e] = upper ? rb(rb(other * sn) + rb(mine * cs)) : rb(rb(mine * cs) - rb(other * sn));
+        }
+    }
+}
+template <int NJ>
+__device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq, int rd) {
+    if constexpr (NJ >= 4) {
+        if (rd == 32 * NJ) return rope_q_inlane<NJ, NJ>(qf, sin_row, cos_row, lq);
+    }
+    if constexpr (NJ == 8) {
+        if (rd == 128) return rope_q_inlane<NJ, 4>(qf, sin_row, cos_row, lq);
+    }
+    if (rd == 64) return rope_q_crosslane<NJ, 32>(qf, sin_row, cos_row, lq);
+    if (rd == 32) return rope_q_crosslane<NJ, 16>(qf, sin_row, cos_row, lq);
+}
+
+// Per-head QK-norm of the query elements a lane holds (bf16 tensor; NormSpec in quant_device.hpp).  The four lanes
+// lq = 0..3 of a head share its sum of squares.
+template <int NJ>
+__device__ __forceinline__ void norm_q(float (&qf)[8 * NJ], const NormSpec &n, int head, int lq, int D) {
+#pragma clang fp contract(off)
+    double ss = 0.0;
+#pragma unroll
+    for (int i = 0; i < 8 * NJ; ++i) ss += (double)norm_square(qf[i], HS_BF16, n.kind);
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    const float rrms = norm_rrms(ss, D, HS_BF16, n.kind, n.eps);
+#pragma unroll
+    for (int i = 0; i < NJ; ++i) {
+        const int d0 = NJ == 2 ? 16 * lq + 8 * i : 64 * (i >> 1) + 16 * lq + 8 * (i & 1);
+        float w[8];
+        if (n.kind == 1) {
+            const u32x4 ww = *(const u32x4 *)((const uint16_t *)n.weight + (int64_t)head * n.head_stride + d0);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[2 * e] = __uint_as_float(ww[e] << 16);
+                w[2 * e + 1] = __uint_as_float(ww[e] & 0xffff0000u);
+            }
+        } else {
+            const float *wp = (const float *)n.weight + (int64_t)head * n.head_stride + d0;
+            const float4v w0 = *(const float4v *)wp, w1 = *(const float4v *)(wp + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[e] = w0[e];
+                w[4 + e] = w1[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qf[8 * i + e] = norm_apply(qf[8 * i + e], w[e], rrms, HS_BF16, n.kind);
     }
 }
 
@@ -390,9 +444,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                     qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
                 }
             }
-            if (ROPE) {
-                const int p = min(max(a.seq_lens[b] - 1, 0), a.rope_len - 1);  // the query is the newest token
-                rope_rotate_q<NJ>(qf, a.rope_sin + (int64_t)p * (kD / 2), a.rope_cos + (int64_t)p * (kD / 2), lq);
+            if (ROPE) {  // the step's prologue on q: QK-norm, then the rotation
+                if (a.qnorm.kind != 0) norm_q<NJ>(qf, a.qnorm, h * G + li, lq, kD);
+                if (a.rope_sin != nullptr) {
+                    const int p = min(max(a.seq_lens[b] - 1, 0), a.rope_len - 1);  // the query is the newest token
+                    const int half = a.rotary_dim / 2;
+                    rope_rotate_q<NJ>(qf, a.rope_sin + (int64_t)p * half, a.rope_cos + (int64_t)p * half, lq, a.rotary_dim);
+                }
             }
 #pragma unroll
             for (int i = 0; i < 8 * NJ; ++i) amax = fmaxf(amax, fabsf(qf[i]));
@@ -545,6 +603,8 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, 
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
+int check_prologue(const hs_qk_prologue *p, int dtype, int D, bool need_q, bool need_k);
+NormSpec norm_spec(const hs_qk_prologue *p, int which);
 
 constexpr int kMaxHintedChunks = 16;  // most chunks a sequence is cut into on the strength of the ragged-batch hint
 
@@ -581,8 +641,10 @@ static int pick_chunk_tokens(int B, int Hkv, int max_seq_len, int64_t total_toke
 struct NewToken {  // optional quantize-on-write of one token per sequence inside the same call
     const void *k_src = nullptr, *v_src = nullptr;  // [B, 1, Hkv, D]
     int dtype = HS_BF16;
-    const void *rope_sin = nullptr, *rope_cos = nullptr;  // rotate q and k_new (bf16 tables [rope_len, D/2])
-    int rope_len = 0;
+    const void *rope_sin = nullptr, *rope_cos = nullptr;  // rotate q and k_new (bf16 tables [rope_len, rotary_dim/2])
+    int rope_len = 0, rotary_dim = 0;                     // 0 = head_dim
+    NormSpec qnorm, knorm;                                // QK-norm of q and k_new ahead of the rotation
+    bool prologue = false;                                // the kernel instance with the q-side prologue
 };
 
 // static_scratch: the partials go to this device's copy of `scratch` (ws / ws_bytes ignored) and the size check is
@@ -648,21 +710,32 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
         if (!nt.k_src || nt.dtype != HS_BF16)
             return fail(HS_ERR_INVALID_ARGUMENT, "the rotary decode step takes a bf16 new token");
     }
-    a.nt.rope_sin = nt.rope_sin; a.nt.rope_cos = nt.rope_cos; a.nt.rope_len = nt.rope_len;
+    const int rd = nt.rotary_dim > 0 ? nt.rotary_dim : D;
+    if (nt.rope_sin && !(rd == D || ((rd == 32 || rd == 64 || rd == 128) && rd < D)))
+        return fail(HS_ERR_INVALID_ARGUMENT,
+                    "the fused decode step rotates head_dim, 128, 64 or 32 leading elements, not %d: run "
+                    "hs_qk_prologue_apply and hs_decode_step_int8 instead", rd);
+    if ((nt.qnorm.kind != 0 || nt.knorm.kind != 0) && (!nt.k_src || nt.dtype != HS_BF16))
+        return fail(HS_ERR_INVALID_ARGUMENT, "the decode step with a QK-norm takes a bf16 new token");
+    a.nt.rope_sin = nt.rope_sin; a.nt.rope_cos = nt.rope_cos; a.nt.rope_len = nt.rope_len; a.nt.rotary_dim = rd;
+    a.nt.norm = nt.knorm;
     a.rope_sin = (const uint16_t *)nt.rope_sin; a.rope_cos = (const uint16_t *)nt.rope_cos; a.rope_len = nt.rope_len;
+    a.rotary_dim = rd;
+    a.qnorm = nt.qnorm;
+    const bool pro = nt.prologue || a.rope_sin != nullptr;
     if (phases & 1) {
         dim3 grid(a.nchunks, Hkv, B);
         if (D == 64) {
             if (fp8) decode_attn_kernel<64, true, false><<<grid, 256, 0, stream>>>(a);
-            else if (a.rope_sin) decode_attn_kernel<64, false, true><<<grid, 256, 0, stream>>>(a);
+            else if (pro) decode_attn_kernel<64, false, true><<<grid, 256, 0, stream>>>(a);
             else decode_attn_kernel<64, false, false><<<grid, 256, 0, stream>>>(a);
         } else if (D == 128) {
             if (fp8) decode_attn_kernel<128, true, false><<<grid, 256, 0, stream>>>(a);
-            else if (a.rope_sin) decode_attn_kernel<128, false, true><<<grid, 256, 0, stream>>>(a);
+            else if (pro) decode_attn_kernel<128, false, true><<<grid, 256, 0, stream>>>(a);
             else decode_attn_kernel<128, false, false><<<grid, 256, 0, stream>>>(a);
         } else {
             if (fp8) decode_attn_kernel<256, true, false><<<grid, 256, 0, stream>>>(a);
-            else if (a.rope_sin) decode_attn_kernel<256, false, true><<<grid, 256, 0, stream>>>(a);
+            else if (pro) decode_attn_kernel<256, false, true><<<grid, 256, 0, stream>>>(a);
             else decode_attn_kernel<256, false, false><<<grid, 256, 0, stream>>>(a);
         }
         if (int rc = check_launch("decode_attn")) return rc;
@@ -743,6 +816,23 @@ int hs_decode_step_int8_rope(const void *q, const void *k_new, const void *v_new
     hs::NewToken nt;
     nt.k_src = k_new; nt.v_src = v_new; nt.dtype = HS_BF16;
     nt.rope_sin = rope_sin; nt.rope_cos = rope_cos; nt.rope_len = rope_len;
+    return hs::launch_decode(false, 3, nt, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
+                             workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_step_int8_prologue(const void *q, const void *k_new, const void *v_new, const hs_qk_prologue *prologue,
+                                 int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                                 const hs_kv_layout *layout, const int32_t *seq_lens, void *out, void *workspace,
+                                 size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
+                                 int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
+    if (!k_new || !v_new) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (int rc = hs::check_prologue(prologue, HS_BF16, D, true, true)) return rc;
+    hs::NewToken nt;
+    nt.k_src = k_new; nt.v_src = v_new; nt.dtype = HS_BF16;
+    nt.rope_sin = prologue->rope_sin; nt.rope_cos = prologue->rope_cos; nt.rope_len = prologue->rope_len;
+    nt.rotary_dim = prologue->rotary_dim;
+    nt.qnorm = hs::norm_spec(prologue, 0); nt.knorm = hs::norm_spec(prologue, 1);
+    nt.prologue = true;
     return hs::launch_decode(false, 3, nt, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
                              workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
 }

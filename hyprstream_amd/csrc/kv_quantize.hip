@@ -137,6 +137,61 @@ __global__ __launch_bounds__(256) void rope_apply_kernel(RopeArgs a) {
     }
 }
 
+struct PrologueArgs {
+    const void *x[2];   // q [B, S, Hq, D], k [B, S, Hkv, D] (either may be null)
+    void *out[2];
+    NormSpec norm[2];
+    const void *sin_t, *cos_t;  // null: no rotation
+    const int32_t *positions;
+    int32_t start_pos, rope_len, B, S, H[2], D, dtype, rd;
+};
+
+// What runs on q and k between the projections and cache.update / attention, in one launch over both tensors:
+// per-head QK-norm (NormSpec) and the (partial) rotary embedding of the normalised rows.  One wavefront per
+// (token, head) row, E = D/64 consecutive elements per lane; row r of the launch is head r % (Hq + Hkv) of token
+// r / (Hq + Hkv), the q heads first.
+template <int E>
+__global__ __launch_bounds__(256) void qk_prologue_kernel(PrologueArgs a) {
+#pragma clang fp contract(off)
+    const int lane = threadIdx.x & 63;
+    const int HH = a.H[0] + a.H[1];
+    const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= (int64_t)a.B * a.S * HH) return;
+    const int64_t bs = r / HH;
+    const int hh = (int)(r - bs * HH);
+    const int which = hh >= a.H[0] ? 1 : 0, h = which ? hh - a.H[0] : hh;
+    const int s = (int)(bs % a.S), b = (int)(bs / a.S);
+    const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
+    const int64_t row = bs * a.H[which] + h;
+    const NormSpec &n = a.norm[which];
+    float x[E];
+    load_src<E>(a.x[which], a.dtype, row * a.D + lane * E, x);
+    float rrms = 0.0f;
+    if (n.kind != 0) {
+        double ss = 0.0;
+#pragma unroll
+        for (int e = 0; e < E; ++e) ss += (double)norm_square(x[e], a.dtype, n.kind);
+        rrms = norm_rrms(wave_sum_f64(ss), a.D, a.dtype, n.kind, n.eps);
+        float w[E];
+        norm_weights<E>(n, a.dtype, h, lane * E, w);
+#pragma unroll
+        for (int e = 0; e < E; ++e) x[e] = norm_apply(x[e], w[e], rrms, a.dtype, n.kind);
+    }
+    if (a.sin_t != nullptr && lane * E < a.rd)
+        rope_rotate<E>(a.x[which], a.dtype, row * a.D, a.rd, a.sin_t, a.cos_t, a.rope_len, pos, lane * E, x, &n, rrms, h);
+    const int64_t o = row * a.D + lane * E;
+    void *out = a.out[which];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        if (a.dtype == HS_F32) ((float *)out)[o + e] = x[e];
+        else if (a.dtype == HS_BF16) ((uint16_t *)out)[o + e] = (uint16_t)f32_to_bf16_bits(x[e]);
+        else {
+            _Float16 f = (_Float16)x[e];
+            __builtin_memcpy((uint16_t *)out + o + e, &f, 2);
+        }
+    }
+}
+
 // The same for many rows of a 16-bit tensor: D/8 lanes own a row, eight consecutive elements each (16-byte loads
 // of the lane's elements, of their partners half a row away and of the sin/cos entries; one 16-byte store), so a
 // wavefront carries 64/(D/8) rows.  Per element the operations and their roundings are those of rope_rotate().
@@ -394,7 +449,7 @@ template <bool FP8>
 static int launch_quantize(const void *k_src, const void *v_src, int dtype, void *kc, void *vc, float *ks, float *vs,
                            const hs_kv_layout *l, const int32_t *positions, int start_pos, int B, int S, int Hkv,
                            int D, hipStream_t stream, const void *rope_sin = nullptr, const void *rope_cos = nullptr,
-                           int rope_len = 0) {
+                           int rope_len = 0, int rotary_dim = 0, const NormSpec *norm = nullptr) {
     if (int rc = check_common(l, B, S, Hkv, D, !FP8)) return rc;
     if ((rope_sin == nullptr) != (rope_cos == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give sin and cos or neither");
     if (rope_sin && rope_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "rope_len must be positive");
@@ -422,12 +477,13 @@ static int launch_quantize(const void *k_src, const void *v_src, int dtype, void
     a.addr[0] = make_addr(*l, 0); a.addr[1] = make_addr(*l, 1);
     a.positions = positions; a.start_pos = start_pos;
     a.B = B; a.S = S; a.Hkv = Hkv; a.D = D; a.dtype = dtype;
-    a.rope_sin = rope_sin; a.rope_cos = rope_cos; a.rope_len = rope_len;
+    a.rope_sin = rope_sin; a.rope_cos = rope_cos; a.rope_len = rope_len; a.rotary_dim = rotary_dim;
+    if (norm) a.norm = *norm;
     // Bulk writes without rotation take the kernel that packs several rows into a wavefront; it wants
     // 16-byte aligned sources and 8-byte aligned code rows and at most 65535 sequences (grid.z).
     const bool aligned = (((uintptr_t)k_src | (uintptr_t)v_src) & 15) == 0 && (((uintptr_t)kc | (uintptr_t)vc) & 7) == 0 &&
                          (l->code_stride_seq & 7) == 0;
-    if (!rope_sin && aligned && B <= 65535 && (int64_t)S * Hkv < (1 << 30)) {
+    if (!rope_sin && a.norm.kind == 0 && aligned && B <= 65535 && (int64_t)S * Hkv < (1 << 30)) {
         const int lpr = D / 8, rows_per_wg = 4 * (64 / lpr);
         dim3 g((unsigned)(((int64_t)S * Hkv + rows_per_wg - 1) / rows_per_wg), 2, B);
         if (D == 64) kv_quantize_rows_kernel<8, FP8><<<g, 256, 0, stream>>>(a);
@@ -460,6 +516,87 @@ int hs_kv_quantize_int8_rope(const void *k_src, const void *v_src, int src_dtype
     if (!rope_sin || !rope_cos) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null rotary table");
     return hs::launch_quantize<false>(k_src, v_src, src_dtype, k_codes, v_codes, k_scales, v_scales, layout, positions,
                                       start_pos, B, S, Hkv, D, (hipStream_t)stream, rope_sin, rope_cos, rope_len);
+}
+
+}  // extern "C"
+
+namespace hs {
+
+// Checks of an hs_qk_prologue shared by the entry points that take one; fills the K-side NormSpec / rotary_dim.
+int check_prologue(const hs_qk_prologue *p, int dtype, int D, bool need_q, bool need_k) {
+    if (!p) return fail(HS_ERR_INVALID_ARGUMENT, "null hs_qk_prologue");
+    if (p->norm_kind < HS_QKNORM_NONE || p->norm_kind > HS_QKNORM_QWEN35)
+        return fail(HS_ERR_INVALID_ARGUMENT, "unknown norm_kind %d", p->norm_kind);
+    if (p->norm_kind != HS_QKNORM_NONE) {
+        if ((need_q && !p->q_norm_weight) || (need_k && !p->k_norm_weight))
+            return fail(HS_ERR_INVALID_ARGUMENT, "QK-norm without a weight vector");
+        if ((p->q_norm_head_stride != 0 && p->q_norm_head_stride != D) || (p->k_norm_head_stride != 0 && p->k_norm_head_stride != D))
+            return fail(HS_ERR_INVALID_ARGUMENT, "norm weight head stride must be 0 (one [D] vector) or D (per-head rows)");
+        if (!(p->norm_eps >= 0.0f)) return fail(HS_ERR_INVALID_ARGUMENT, "negative norm_eps");
+    }
+    if ((p->rope_sin == nullptr) != (p->rope_cos == nullptr)) return fail(HS_ERR_INVALID_ARGUMENT, "give sin and cos or neither");
+    if (p->rope_sin) {
+        if (p->rope_len <= 0) return fail(HS_ERR_INVALID_ARGUMENT, "rope_len must be positive");
+        const int rd = p->rotary_dim > 0 ? p->rotary_dim : D;
+        if (rd > D || (rd % 16) != 0)
+            return fail(HS_ERR_INVALID_ARGUMENT, "rotary_dim %d must be a multiple of 16 in (0, head_dim %d]", rd, D);
+    }
+    (void)dtype;
+    return HS_OK;
+}
+
+NormSpec norm_spec(const hs_qk_prologue *p, int which) {
+    NormSpec n;
+    n.kind = p->norm_kind;
+    n.eps = p->norm_eps;
+    n.weight = which ? p->k_norm_weight : p->q_norm_weight;
+    n.head_stride = which ? p->k_norm_head_stride : p->q_norm_head_stride;
+    return n;
+}
+
+}  // namespace hs
+
+extern "C" {
+
+int hs_qk_prologue_apply(const void *q, const void *k, int dtype, const hs_qk_prologue *prologue,
+                         const int32_t *positions, int32_t start_pos, void *q_out, void *k_out, int32_t B, int32_t S,
+                         int32_t Hq, int32_t Hkv, int32_t D, hs_stream_t stream) {
+    using namespace hs;
+    if (dtype != HS_BF16 && dtype != HS_F32 && dtype != HS_F16) return fail(HS_ERR_INVALID_ARGUMENT, "unknown dtype %d", dtype);
+    if (D != 64 && D != 128 && D != 256) return fail(HS_ERR_INVALID_ARGUMENT, "head_dim %d not in {64,128,256}", D);
+    if (B < 0 || S < 0 || Hq < 0 || Hkv < 0) return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d Hq=%d Hkv=%d", B, S, Hq, Hkv);
+    const int hq = q ? Hq : 0, hk = k ? Hkv : 0;
+    if (int rc = check_prologue(prologue, dtype, D, hq > 0, hk > 0)) return rc;
+    if ((q && !q_out) || (k && !k_out)) return fail(HS_ERR_INVALID_ARGUMENT, "null output buffer");
+    if (q && q == q_out && prologue->rope_sin) return fail(HS_ERR_INVALID_ARGUMENT, "the rotation cannot run in place: give q_out its own buffer");
+    if (k && k == k_out && prologue->rope_sin) return fail(HS_ERR_INVALID_ARGUMENT, "the rotation cannot run in place: give k_out its own buffer");
+    if (prologue->rope_sin && !positions && (start_pos < 0 || (int64_t)start_pos + S > prologue->rope_len))
+        return fail(HS_ERR_INVALID_ARGUMENT, "positions %d..%d exceed the rotary tables (%d rows)", start_pos,
+                    start_pos + S - 1, prologue->rope_len);
+    const int64_t rows = (int64_t)B * S * (hq + hk);
+    if (rows == 0) return HS_OK;
+    PrologueArgs a;
+    a.x[0] = q; a.x[1] = k; a.out[0] = q_out; a.out[1] = k_out;
+    a.norm[0] = norm_spec(prologue, 0); a.norm[1] = norm_spec(prologue, 1);
+    a.sin_t = prologue->rope_sin; a.cos_t = prologue->rope_cos; a.positions = positions; a.start_pos = start_pos;
+    a.rope_len = prologue->rope_len; a.B = B; a.S = S; a.H[0] = hq; a.H[1] = hk; a.D = D; a.dtype = dtype;
+    a.rd = prologue->rotary_dim > 0 ? prologue->rotary_dim : D;
+    dim3 grid((unsigned)((rows + 3) / 4));
+    if (D == 64) qk_prologue_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    else if (D == 128) qk_prologue_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    else qk_prologue_kernel<4><<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    return check_launch("qk_prologue");
+}
+
+int hs_kv_quantize_int8_prologue(const void *k_src, const void *v_src, int src_dtype, const hs_qk_prologue *prologue,
+                                 int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                                 const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos, int32_t B,
+                                 int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream) {
+    if (int rc = hs::check_prologue(prologue, src_dtype, D, false, true)) return rc;
+    const hs::NormSpec n = hs::norm_spec(prologue, 1);
+    return hs::launch_quantize<false>(k_src, v_src, src_dtype, k_codes, v_codes, k_scales, v_scales, layout, positions,
+                                      start_pos, B, S, Hkv, D, (hipStream_t)stream, prologue->rope_sin,
+                                      prologue->rope_cos, prologue->rope_len, prologue->rotary_dim, &n);
 }
 
 int hs_rope_apply(const void *x, int dtype, const void *rope_sin, const void *rope_cos, int32_t rope_len,

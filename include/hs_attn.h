@@ -130,6 +130,42 @@ HS_API int hs_rope_apply_partial(const void *x, int dtype, const void *rope_sin,
                         const int32_t *positions, int32_t start_pos, void *out,
                         int32_t B, int32_t S, int32_t H, int32_t D, int32_t rotary_dim, hs_stream_t stream);
 
+/* ---- everything the reference runs on q and k between the projections and cache.update: per-head QK-norm, then the
+ * rotary embedding (llama.rs:589-611: apply_qk_norm llama.rs:929-991, then apply_rope; qwen3_5.rs:973-990: apply_qknorm
+ * qwen3_5.rs:1077-1091, then the partial rotary embedding) ----------------------------------------------------------
+ * HS_QKNORM_LLAMA (Gemma3 and other Llama-architecture models with q_norm / k_norm): square, mean, + eps, reciprocal,
+ *   sqrt, x * rrms, * weight as separate ops in the tensor dtype, each result rounded to it (the reference hard-codes
+ *   eps = 1e-6 there); weights in the tensor dtype, [H, D] (head stride D) or one [D] vector (head stride 0).
+ * HS_QKNORM_QWEN35: in fp32, rrms = 1 / sqrt(mean(x^2) + eps), out = (x * rrms) * (1 + weight), one cast back; fp32 weights.
+ * The sum of squares is the correctly rounded fp32 sum of the row (libtorch's own summation order depends on the host).
+ * rope_sin / rope_cos: tables [rope_len, rotary_dim / 2] in the tensor dtype as for hs_rope_apply_partial, NULL = no
+ * rotation; rotary_dim 0 means head_dim.  Results equal those of the separate ops: the rotated rows are bit-exact
+ * functions of the normalised rows, and codes written from them are those of hs_kv_quantize_int8. */
+enum hs_qk_norm_kind { HS_QKNORM_NONE = 0, HS_QKNORM_LLAMA = 1, HS_QKNORM_QWEN35 = 2 };
+typedef struct hs_qk_prologue {
+    int32_t norm_kind;            /* enum hs_qk_norm_kind */
+    float norm_eps;
+    const void *q_norm_weight;    /* device; HS_QKNORM_LLAMA: tensor dtype, HS_QKNORM_QWEN35: fp32 */
+    const void *k_norm_weight;
+    int32_t q_norm_head_stride;   /* elements between the weight rows of consecutive heads: D, or 0 for one shared [D] */
+    int32_t k_norm_head_stride;
+    const void *rope_sin;         /* device, [rope_len, rotary_dim / 2]; NULL: no rotation */
+    const void *rope_cos;
+    int32_t rope_len;
+    int32_t rotary_dim;           /* leading elements of each head that are rotated; 0 = head_dim */
+} hs_qk_prologue;
+/* q [B, S, Hq, D] -> q_out, k [B, S, Hkv, D] -> k_out in one launch (either pair may be NULL); token (b, s) takes table
+ * row (positions ? positions[b] : 0) + start_pos + s.  The pre-pass of a prefill call: q_out and k_out are what
+ * hs_prefill_attn_* expects (rotated q, rotated K for its own bf16 part and for quantize_on_write). */
+HS_API int hs_qk_prologue_apply(const void *q, const void *k, int dtype, const hs_qk_prologue *prologue,
+                        const int32_t *positions, int32_t start_pos, void *q_out, void *k_out,
+                        int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, hs_stream_t stream);
+/* hs_kv_quantize_int8 with K normalised and rotated on the way in (k_src arrives as projected); V as it is. */
+HS_API int hs_kv_quantize_int8_prologue(const void *k_src, const void *v_src, int src_dtype, const hs_qk_prologue *prologue,
+                        int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                        const hs_kv_layout *layout, const int32_t *positions, int32_t start_pos,
+                        int32_t B, int32_t S, int32_t Hkv, int32_t D, hs_stream_t stream);
+
 /* FP8 e4m3fn cache with one fp32 scale per (sequence, kv-head).  Calibration computes
  * scale[b, h] = max over (s, d) |x| / 448 from the tokens given (typically the prompt);
  * quantization stores e4m3fn(clamp(x / scale, +-448)), round-to-nearest-even. */
@@ -205,6 +241,16 @@ HS_API int hs_decode_step_int8(const void *q, const void *k_new, const void *v_n
  * token's position seq_lens[b] - 1.  Results equal hs_rope_apply(q) + hs_kv_quantize_int8_rope + decode. */
 HS_API int hs_decode_step_int8_rope(const void *q, const void *k_new, const void *v_new,
                                const void *rope_sin, const void *rope_cos, int32_t rope_len,
+                               int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
+                               const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                               void *workspace, size_t workspace_bytes,
+                               int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                               float softmax_scale, hs_stream_t stream);
+/* The step with the whole prologue inside the launch: QK-norm of q and k_new, then their rotation (hs_qk_prologue above;
+ * q [B, Hq, D], k_new [B, 1, Hkv, D], v_new in bf16 as projected; table row = seq_lens[b] - 1).  Rotated parts the
+ * kernel serves: rotary_dim = head_dim, or 128, 64, 32 leading elements (Qwen3.5: 64 of 256); anything else is
+ * HS_ERR_INVALID_ARGUMENT (run hs_qk_prologue_apply + hs_decode_step_int8).  Results equal those calls' bit for bit. */
+HS_API int hs_decode_step_int8_prologue(const void *q, const void *k_new, const void *v_new, const hs_qk_prologue *prologue,
                                int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
                                const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
                                void *workspace, size_t workspace_bytes,

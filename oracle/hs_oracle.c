@@ -424,6 +424,65 @@ ORC_API void orc_rope_apply_f32(const float *x, const float *sin_t, const float 
     }
 }
 
+/* ------------------------------------------------------------------ QK-norm */
+
+/* Per-head RMS normalisation of q / k right before the rotary embedding, bf16 tensors [rows, H, D].
+ *
+ * kind 1 -- LlamaAttention::apply_qk_norm (architectures/llama.rs:929-991, Gemma3): every op in the tensor dtype,
+ *   i.e. computed in fp32 and rounded to bf16 after EACH libtorch op:
+ *     x2 = square(x); mean = mean_dim(x2, -1, dtype = bf16)  [fp32 sum, divided by D, rounded once];
+ *     rrms = sqrt(reciprocal(mean + eps))  [eps is a scalar operand of a bf16 tensor op: it is cast to bf16 first];
+ *     out = (x * rrms) * weight, weight bf16 [H, D] (head_stride = D) or [D] (head_stride = 0).
+ * kind 2 -- Qwen3_5Model::apply_qknorm (architectures/qwen3_5.rs:1077-1091): fp32 throughout, one rounding to bf16 at
+ *   the end:  xf = float(x); mean_sq = mean(xf * xf); rrms = rsqrt(mean_sq + eps) = 1 / sqrt(.);
+ *     out = bf16((xf * rrms) * (weight + 1)), weight fp32 [D] (head_stride 0) or [H, D].
+ * The sum of the squares is accumulated in double and rounded to fp32 once (the squares of bf16 values are exact in
+ * fp32, so this is the correctly rounded fp32 sum); libtorch's own fp32 summation order depends on the host's vector
+ * width and can differ from it in the last fp32 bit, which moves a bf16 result in a few rows per million. */
+ORC_API void orc_qk_norm_bf16(const uint16_t *x, int64_t rows, int H, int D, int kind, const void *weight, int head_stride,
+                              float eps, uint16_t *out) {
+    for (int64_t r = 0; r < rows; ++r)
+        for (int h = 0; h < H; ++h) {
+            const uint16_t *xi = x + (r * H + h) * D;
+            uint16_t *oi = out + (r * H + h) * D;
+            double acc = 0.0;
+            if (kind == 1) {
+                const uint16_t *w = (const uint16_t *)weight + (int64_t)h * head_stride;
+                for (int d = 0; d < D; ++d) {
+                    const float v = bf16_to_f32(xi[d]);
+                    const volatile float sq = rbf(v * v);
+                    acc += (double)sq;
+                }
+                const volatile float sum = (float)acc;
+                const volatile float mean = rbf(sum / (float)D);
+                const volatile float t = rbf(mean + rbf(eps));
+                const volatile float rc = rbf(1.0f / t);
+                const volatile float rrms = rbf(sqrtf(rc));
+                for (int d = 0; d < D; ++d) {
+                    const volatile float y = rbf(bf16_to_f32(xi[d]) * rrms);
+                    oi[d] = orc_f32_to_bf16(y * bf16_to_f32(w[d]));
+                }
+            } else {
+                const float *w = (const float *)weight + (int64_t)h * head_stride;
+                for (int d = 0; d < D; ++d) {
+                    const float v = bf16_to_f32(xi[d]);
+                    const volatile float sq = v * v;
+                    acc += (double)sq;
+                }
+                const volatile float sum = (float)acc;
+                const volatile float mean = sum / (float)D;
+                const volatile float t = mean + eps;
+                const volatile float sr = sqrtf(t);
+                const volatile float rrms = 1.0f / sr;
+                for (int d = 0; d < D; ++d) {
+                    const volatile float y = bf16_to_f32(xi[d]) * rrms;
+                    const volatile float w1 = w[d] + 1.0f;
+                    oi[d] = orc_f32_to_bf16(y * w1);
+                }
+            }
+        }
+}
+
 /* ------------------------------------------------------- DeltaNet surroundings */
 
 static inline float silu_f(float x) { return x / (1.0f + expf(-x)); }

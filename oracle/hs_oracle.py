@@ -212,6 +212,19 @@ def rope_apply_f32(x, sin_t, cos_t, pos):
     return out
 
 
+def qk_norm_bf16(x_bits, kind, weight, eps):
+    """x_bits: uint16 [rows, H, D] bf16 patterns.  kind 1 (Llama/Gemma3, bf16 op by op): weight uint16 bf16 [H, D] or [D];
+    kind 2 (Qwen3.5, fp32, (1 + w)): weight fp32 [D] or [H, D].  Returns uint16 [rows, H, D]."""
+    x = _c(x_bits, np.uint16)
+    rows, H, D = x.shape
+    w = _c(weight, np.uint16 if kind == 1 else np.float32)
+    assert w.shape in ((D,), (H, D))
+    out = np.empty_like(x)
+    lib().orc_qk_norm_bf16(_p(x), ctypes.c_int64(rows), ctypes.c_int(H), ctypes.c_int(D), ctypes.c_int(kind), _p(w),
+                           ctypes.c_int(D if w.ndim == 2 else 0), ctypes.c_float(eps), _p(out))
+    return out
+
+
 # ------------------------------------------------------- DeltaNet surroundings
 def deltanet_conv_silu_bf16(x_bits, w_bits, state_bits):
     """x [B,S,C], w [C,K], state [B,C,K-1] (bf16 patterns) -> (y [B,S,C], new state)."""

@@ -166,6 +166,29 @@ def rope_apply(x, sin_full, cos_full, position_ids):
     return torch.cat([x1r, x2r], -1)
 
 
+def qk_norm_llama(x, weight, eps=1e-6):
+    """LlamaAttention::apply_qk_norm (llama.rs:929-991, Gemma3): per-head RMS norm in the tensor dtype, every op a
+    separate libtorch op.  x [B, S, H, D]; weight [H * D] (reshaped to [1, 1, H, D]) or [D]."""
+    H, D = x.shape[-2], x.shape[-1]
+    w = weight.reshape(H, D).unsqueeze(0).unsqueeze(0) if weight.numel() == H * D else weight.reshape(1, 1, 1, D)
+    x2 = x.square()
+    mean = x2.mean(dim=-1, keepdim=True, dtype=x.dtype)
+    rrms = (mean + eps).reciprocal().sqrt()
+    return (x * rrms) * w
+
+
+def qk_norm_qwen35(x, weight_f32, eps):
+    """Qwen3_5Model::apply_qknorm (qwen3_5.rs:1077-1091): fp32, (1 + w), one cast back.  x [B, S, H, D]; weight fp32 [D]."""
+    shp = x.shape
+    D = shp[-1]
+    flat = x.reshape(-1, D)
+    f = flat.float()
+    mean_sq = (f * f).mean(dim=-1, keepdim=True, dtype=torch.float32)
+    rrms = (mean_sq + eps).rsqrt()
+    normed = f * rrms
+    return (normed * (weight_f32.reshape(1, D) + 1.0)).to(x.dtype).reshape(shp)
+
+
 def deltanet_prepare(mixed_qkv, conv_weight, conv_state, a_in, b_in, neg_a_exp, dt_bias):
     """GatedDeltaNetLayer::forward between the projection and the delta rule (qwen3_5.rs:629-686): depthwise
     causal conv1d over [state | x] + SiLU in the model dtype, g and beta in fp32.  mixed_qkv [B,S,C];

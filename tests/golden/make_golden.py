@@ -15,6 +15,10 @@ oracle and not with anything from this repository's kernels:
   rope.npz         the reference's table construction and rotation op sequence (rope.rs:100-122,
                    206-248) on bf16 and fp32 tensors, bases 10000 and 1e6, positions up to 8191
 
+  qknorm.npz       the two per-head RMS norms that run on q and k before the rotary embedding: Llama/Gemma3's
+                   bf16 op chain (llama.rs:929-991) and Qwen3.5's fp32 (1 + w) form (qwen3_5.rs:1077-1091),
+                   head_dim 64 / 128 / 256, per-head and shared weights
+
 Inputs come from numpy's Philox generator so the file is reproducible.
 """
 import os
@@ -184,12 +188,34 @@ def make_rope():
     np.savez_compressed(os.path.join(HERE, "rope.npz"), **out)
 
 
+def make_qknorm():
+    r = gen(9)
+    out = {}
+    for D in (64, 128, 256):
+        H, rows = 3, 24
+        x = torch.from_numpy((r.standard_normal((1, rows, H, D)) * r.random((1, rows, H, 1)) * 3).astype(np.float32)).to(torch.bfloat16)
+        x[0, 0, 0] = 0  # an all-zero head: rrms = 1/sqrt(eps), output zero
+        x[0, 1, 1] *= 1e-4
+        w1 = torch.from_numpy((1.0 + 0.2 * r.standard_normal((H, D))).astype(np.float32)).to(torch.bfloat16)
+        w1s = w1[0].clone()
+        w2 = torch.from_numpy((0.05 * r.standard_normal(D)).astype(np.float32))
+        bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+        out["x_%d" % D] = bits(x[0])
+        out["w1_%d" % D] = bits(w1)
+        out["w2_%d" % D] = w2.numpy()
+        out["llama_%d" % D] = bits(ref.qk_norm_llama(x, w1.reshape(-1))[0])
+        out["llama_shared_%d" % D] = bits(ref.qk_norm_llama(x, w1s)[0])
+        out["qwen_%d" % D] = bits(ref.qk_norm_qwen35(x, w2, 1e-6)[0])
+    np.savez_compressed(os.path.join(HERE, "qknorm.npz"), **out)
+
+
 if __name__ == "__main__":
     make_rope()
     make_int8()
     make_fp8()
     make_attention()
     make_deltanet()
+    make_qknorm()
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)))
