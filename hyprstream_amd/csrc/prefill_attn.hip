@@ -26,8 +26,9 @@
 // straight from the caller's bf16 K/V, V^T built with permutes, P rounded to bf16.  In both parts Q carries
 // the softmax scale and log2(e), the score accumulators start from minus the softmax reference, and the row
 // sums are one more MFMA with a ones operand.  Softmax and accumulation are fp32; the score layout of the first
-// product is the B-operand layout of the second, so P stays in its lanes.  Cached magnitudes beyond the fp16
-// range (|x| > 65024) saturate.
+// product is the B-operand layout of the second, so P stays in its lanes.  The fp16 operands are taken
+// relative to a power-of-two reference per (sequence, kv-head) (see the history phase), so the absolute magnitude of
+// the cache does not matter; a row whose scale is more than 2^11 times that head's reference saturates.
 #include <climits>
 #include <type_traits>
 
@@ -177,12 +178,52 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
     const float qscale = (kRow < kPD && 8 * KG * lq >= kRow) ? 0.0f : a.scale_log2e;  // padding columns of Q are zero
     const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;  // wavefronts w and w+4 share a SIMD
+    float vup = 1.0f;  // 2^E of the history's V operands, folded back into the accumulators when the history ends
 
     // =============================== history: int8 cache, f16 MFMA ===============================
     if (H > 0) {
-        // Q operands carry the softmax scale and log2(e): qop = fp16(q * scale * log2e * 2^-ex), so the MFMA
-        // result is the score in log2 units times 2^-ex.  ex is zero unless a column's scaled |q| would leave
-        // the fp16 range (then the wavefront takes the path that multiplies the scores by cq = 2^ex).
+        // The history operands are fp16(code * scale), and fp16 spans 2^-14 .. 65504 only.  Each (sequence, kv-head)
+        // therefore gets a power-of-two reference for K and one for V, taken from the largest scale among its first
+        // cached tokens (int8; up to 64 of them, inside one block) or from its head scale (fp8): operands are
+        // fp16(code * scale * 2^-E), with that reference scale landing in [1/8, 1/4).  K's 2^E goes into the Q
+        // operands, V's into the accumulators when the history ends -- both exact.  What matters is then a scale's
+        // size RELATIVE to the head's own: rows up to 2^11 above the reference and down to 2^-11 below it keep full
+        // precision, whatever the absolute magnitude of the cache.
+        float kdown = 1.0f, kup = 1.0f, vdown = 1.0f;
+        {
+            float rk, rv;
+            if (FP8) {
+                rk = a.ks[(int64_t)b * a.Hkv + kvh];
+                rv = a.vs[(int64_t)b * a.Hkv + kvh];
+            } else {
+                int64_t unit;
+                int slot;
+                resolve(a.ka, b, 0, unit, slot);
+                int n = min(min(H, 64), a.ka.capacity_tokens - slot);
+                rk = a.ks[unit * a.ka.scale_stride_seq + (int64_t)kvh * a.ka.scale_stride_head + slot + min(lane, n - 1)];
+                resolve(a.va, b, 0, unit, slot);
+                n = min(min(H, 64), a.va.capacity_tokens - slot);
+                rv = a.vs[unit * a.va.scale_stride_seq + (int64_t)kvh * a.va.scale_stride_head + slot + min(lane, n - 1)];
+                rk = wave_max(rk);
+                rv = wave_max(rv);
+            }
+            auto ref_exp = [](float r) {  // E with r * 2^-E in [1/8, 1/4); 0 for a zero or non-finite reference
+                int e = 0;
+                if (r > 0.0f && r < 3.0e38f) {
+                    (void)frexpf(r, &e);
+                    e = min(max(e + 2, -100), 100);
+                }
+                return __builtin_amdgcn_readfirstlane(e);
+            };
+            const int ek = ref_exp(rk), ev = ref_exp(rv);
+            kdown = ldexpf(1.0f, -ek);
+            kup = ldexpf(1.0f, ek);
+            vdown = ldexpf(1.0f, -ev);
+            vup = ldexpf(1.0f, ev);
+        }
+        // Q operands carry the softmax scale and log2(e) and K's reference: qop = fp16(q * scale * log2e * 2^E * 2^-ex),
+        // so the MFMA result is the score in log2 units times 2^-ex.  ex is zero unless a column's scaled |q| would
+        // leave the range fp16 holds well (then the wavefront takes the path that multiplies the scores by cq = 2^ex).
         half8 qop[kNB][KG];
         float cq[kNB];
         bool scaled = false;
@@ -195,15 +236,15 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16) * qscale;
-                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * qscale;
+                    qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16) * qscale * kup;
+                    qf[8 * i + 2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u) * qscale * kup;
                 }
             }
 #pragma unroll
             for (int i = 0; i < 8 * KG; ++i) amax = fmaxf(amax, fabsf(qf[i]));
             amax = quad_max(amax);
             int ex = 0;
-            if (amax > 32768.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
+            if ((amax > 32768.0f || amax < 0.0009765625f) && amax > 0.0f && amax < 3.0e38f) (void)frexpf(amax, &ex);
             scaled |= ex != 0;
 #pragma unroll
             for (int j = 0; j < KG; ++j)
@@ -248,6 +289,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             rawsk = 256.0f * a.ks[(int64_t)b * a.Hkv + kvh];
             rawsv[0] = rawsv[1] = 256.0f * a.vs[(int64_t)b * a.Hkv + kvh];
         }
+        const float kdn = kdown, vdn = vdown;
         // issue() is called for steps 0, 1, 2, ... in order, so the (scalar) addresses of a step's codes and
         // scales advance by a constant; a block table is consulted only when a cursor leaves its block.
         const uint8_t *kb = a.kc, *vb = a.vc;
@@ -301,13 +343,14 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         auto commit = [&](HistTile &t, int step) {
             const int last = H - 1 - step * kHStep;  // keys past the end become zero rows
-            float fk = rawsk, fv0 = rawsv[0], fv1 = rawsv[1];
+            float fk = rawsk * kdn, fv0 = rawsv[0] * vdn, fv1 = rawsv[1] * vdn;
             if (last < kHStep - 1) {  // the last, partial step only
                 if (krow > last) fk = 0.0f;
                 if (vkey > last) fv0 = 0.0f;
                 if (vkey + 1 > last) fv1 = 0.0f;
             }
-            // largest operand: 127 * scale (int8), 1.75 * 256 * scale (fp8); both stay finite in fp16
+            // largest operand: 127 * scale (int8), 1.75 * 256 * scale (fp8), scale relative to the head's reference:
+            // rows more than 2^11 above it saturate here instead of overflowing
             const float smax = FP8 ? 64.0f * kMaxScale : kMaxScale;
             const _Float16 sk = (_Float16)fminf(fk, smax);
             const _Float16 bias = (_Float16)1152.0f;
@@ -480,6 +523,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             walk(softmax_for(std::true_type{}));
         else
             walk(softmax_for(std::false_type{}));
+        if (vup != 1.0f) {
+#pragma unroll
+            for (int nb = 0; nb < kNB; ++nb)
+#pragma unroll
+                for (int i = 0; i < VB; ++i) acc[nb][i] *= vup;
+        }
     }
 
     // =============================== new tokens: bf16, causal ===============================

@@ -284,7 +284,13 @@ HS_API int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const v
  * new tokens are also written to the cache at positions hist_len .. hist_len+S-1.
  * D is 64, 128 or 256 (64 runs in the layout of 128 with half of the matrix work as padding); Hq a multiple of Hkv (groups of 1, 2 or 4k query heads fill the workgroups, any
  * other group size pads its last group of four).  A paged layout needs capacity_tokens (tokens per block)
- * to be a multiple of 64 here. */
+ * to be a multiple of 64 here.
+ * Magnitudes: the cached history enters the matrix products as fp16(code * scale * 2^-E), E a power-of-two reference
+ * per (sequence, kv-head) taken from the largest token scale among the first min(hist_len, 64) cached tokens (their
+ * first block when paged; fp8: from the head scale), 2^E re-applied exactly.  Any overall magnitude of K and V is
+ * therefore served with the same relative precision (2^-11 per operand).  Inside one (sequence, kv-head), a token
+ * whose scale exceeds 2^11 times that reference saturates at 65024 * 2^E, and one below 2^-11 times it loses bits in
+ * proportion (its contribution is then below 2^-22 of the head's typical row anyway).  Decode has no such window. */
 HS_API int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_new,
                          int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
                          const hs_kv_layout *layout, int32_t hist_len, void *out,

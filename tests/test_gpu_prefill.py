@@ -110,6 +110,67 @@ def test_cached_prefill_with_int8_history(hist, S):
     assert c.k_codes[:, :, hist:hist + S].any()  # the new rows were cached behind the history
 
 
+@pytest.mark.parametrize("kmag,vmag", [(1e-5, 1e5), (1e5, 1e-5), (3e-7, 3e-7), (1.0, 1e9)])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_history_magnitude_ranges(kmag, vmag, fp8):
+    """The prefill twin of the decode test of large and tiny magnitudes.  The history enters the products as fp16, which
+    holds 2^-14 .. 65504 only; operands are taken relative to a power-of-two reference per (sequence, kv-head), so a
+    cache that is tiny or huge as a whole (a model with small or large K/V projections) keeps the relative accuracy of
+    an N(0,1) one.  Sequence 1 carries the opposite magnitudes of sequence 0.  The comparison is relative to the
+    largest output, because the outputs themselves scale with vmag."""
+    B, Hq, Hkv, hist, S = 2, 8, 2, 150, 70
+    qh, kh, vh = make(90, B, hist, Hq, Hkv)
+    q, k, v = make(91, B, S, Hq, Hkv)
+    mags = np.array([[kmag, vmag], [vmag, kmag]], np.float32)
+    kh, vh = bf16r(kh * mags[:, 0, None, None, None]), bf16r(vh * mags[:, 1, None, None, None])
+    k, v = bf16r(k * mags[:, 0, None, None, None]), bf16r(v * mags[:, 1, None, None, None])
+    q = bf16r(q / np.maximum(mags[:, 0, None, None, None], 1e-3))  # keeps the scores of a size where several keys matter
+    c = DeviceCache(B, Hkv, hist + S, 128, fp8=fp8)
+    hk, hv = torch.from_numpy(kh).to(DEV).bfloat16(), torch.from_numpy(vh).to(DEV).bfloat16()
+    if fp8:
+        hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+    c.write(hk, hv, None, 0)
+    got = gpu_prefill(c, q, k, v, hist, write=False)
+    kc, vc, ks, vs = c.canonical(hist)
+    deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
+    want = oracle_prefill(q, deq(kc, ks), deq(vc, vs), k, v)
+    assert np.isfinite(got).all()
+    for b in range(B):
+        top = np.abs(want[b]).max()
+        d = np.abs(got[b] - want[b])
+        assert d.max() < 2e-2 * top and d.mean() < 2e-3 * top, (b, d.max() / top, d.mean() / top)
+
+
+def test_history_row_far_above_its_heads_reference_saturates():
+    """Inside one (sequence, kv-head) the fp16 window is relative: a cached token whose scale is more than 2^11 times
+    the largest scale among the head's first 64 tokens saturates (pinned here: finite output, and equal to attention
+    over the history with that row's scale clamped to 512 * 2^E), while one 2^10 times the reference is still exact."""
+    B, Hq, Hkv, hist, S = 1, 4, 1, 128, 16
+    qh, kh, vh = make(92, B, hist, Hq, Hkv)
+    q, k, v = make(93, B, S, Hq, Hkv)
+    vh[0, 100] *= 2.0 ** 10   # inside the window
+    c = DeviceCache(B, Hkv, hist + S, 128)
+    c.write(torch.from_numpy(bf16r(vh * 0 + kh)).to(DEV).bfloat16(), torch.from_numpy(bf16r(vh)).to(DEV).bfloat16(), None, 0)
+    got = gpu_prefill(c, q, k, v, hist, write=False)
+    kc, vc, ks, vs = c.canonical(hist)
+    want = oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v)
+    top = np.abs(want).max()
+    assert np.abs(got - want).max() < 2e-2 * top
+    # far outside: V row 100 at 2^14 times the typical scale
+    vh[0, 100] *= 2.0 ** 4
+    c.write(torch.from_numpy(bf16r(kh)).to(DEV).bfloat16(), torch.from_numpy(bf16r(vh)).to(DEV).bfloat16(), None, 0)
+    got = gpu_prefill(c, q, k, v, hist, write=False)
+    assert np.isfinite(got).all()
+    kc, vc, ks, vs = c.canonical(hist)
+    ref_scale = vs[0, :64, 0].max()
+    E = np.frexp(ref_scale)[1] + 2                       # reference * 2^-E in [1/8, 1/4)
+    vd = oracle.dequant_int8(vc, vs)
+    assert vs[0, 100, 0] * 2.0 ** -E > 512.0
+    vd[0, 100] = vc[0, 100].astype(np.float32) * np.float32(512.0 * 2.0 ** E)  # the relative scale clamps at 512
+    sat = oracle_prefill(q, oracle.dequant_int8(kc, ks), vd, k, v)
+    assert np.abs(got - sat).max() < 2e-2 * np.abs(sat).max()
+
+
 @pytest.mark.parametrize("hist,S,sigma", [(19, 5, 1.0), (64, 64, 0.5), (150, 70, 0.5), (333, 200, 1.0)])
 def test_cached_prefill_with_fp8_history(hist, S, sigma):
     """The same over an e4m3fn history with per-head scales: the new rows are encoded with the scales calibrated
