@@ -51,7 +51,7 @@ def build(verbose=False):
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
     # host-side LayerKVCache mirror: plain C++ over the C ABI above (it owns device memory, the kernels do not)
-    hsrc = [os.path.join(HERE, "host", f) for f in ("kv_cache.cpp", "kv_cache_capi.cpp", "block_pool.cpp", "block_pool_capi.cpp")]
+    hsrc = [os.path.join(HERE, "host", f) for f in ("kv_cache.cpp", "kv_cache_capi.cpp", "block_pool.cpp", "block_pool_capi.cpp", "kv_compat.cpp", "kv_compat_capi.cpp")]
     cmd = ["hipcc", "-shared", "-fPIC", "-O2", "-std=c++17", "-fvisibility=hidden", "-Wall", "-x", "hip", "--offload-arch=gfx950"]
     cmd += hsrc + ["-o", HOST_LIB, "-L" + LIBDIR, "-lhs_attn", "-Wl,-rpath,$ORIGIN"]
     if verbose:

@@ -22,6 +22,10 @@ EXPORTS = [
     "hs_paged_cache_create", "hs_paged_cache_destroy", "hs_paged_cache_last_error", "hs_paged_cache_update",
     "hs_paged_cache_get_dense", "hs_paged_cache_decode_attention", "hs_paged_cache_clear", "hs_paged_cache_truncate_to",
     "hs_paged_cache_seq_pos", "hs_paged_cache_num_blocks", "hs_paged_batch_decode_step",
+    "hs_compat_create", "hs_compat_destroy", "hs_compat_set_uint", "hs_compat_set_opt_uint", "hs_compat_set_str",
+    "hs_compat_add_layer_type", "hs_compat_set_rope_scaling", "hs_compat_set_kv_quant",
+    "hs_compat_is_authoritatively_complete", "hs_compat_fingerprint", "hs_compat_check", "hs_compat_decide_reuse",
+    "hs_kv_quant_mode_str", "hs_kv_quant_mode_of",
 ]
 BLOCK_SIZE = 256  # tokens per pool block
 STATELESS, SESSION, TRAINING = 0, 1, 2  # owner kinds
@@ -53,6 +57,19 @@ def lib():
         L.hs_pool_allocate.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_char_p,
                                        ctypes.POINTER(ctypes.c_int32)]
         L.hs_pool_free.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_char_p, ctypes.c_int32]
+        L.hs_compat_create.restype = ctypes.c_void_p
+        L.hs_compat_destroy.argtypes = [ctypes.c_void_p]
+        L.hs_compat_set_uint.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_uint64]
+        L.hs_compat_set_opt_uint.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_uint64]
+        L.hs_compat_set_str.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_char_p]
+        L.hs_compat_add_layer_type.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        L.hs_compat_set_rope_scaling.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.c_float]
+        L.hs_compat_set_kv_quant.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        L.hs_compat_is_authoritatively_complete.argtypes = [ctypes.c_void_p]
+        L.hs_compat_fingerprint.argtypes = [ctypes.c_void_p, ctypes.c_char_p]
+        L.hs_compat_check.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_char_p, ctypes.c_size_t]
+        L.hs_compat_decide_reuse.argtypes = [ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int]
+        L.hs_kv_quant_mode_str.restype = ctypes.c_char_p
         for f in EXPORTS:
             if f != "hs_cache_create":
                 fn = getattr(L, f)
@@ -301,3 +318,67 @@ def paged_batch_decode_step(pool, rows, q, k_new, v_new, softmax_scale):
     pool._check(rc)
     return out
 
+
+
+# ---------------------------------------------------------------- cache identity (kv_compat.rs)
+KVQ_NONE, KVQ_INT8, KVQ_NF4, KVQ_FP4, KVQ_INT8_TOKEN, KVQ_FP8_E4M3FN_HEAD = range(6)
+REUSE, STAMP_FRESH, DISCARD_AND_RECOMPUTE = 0, 1, 2
+
+
+def f32_bits(x):
+    import struct
+    return struct.unpack("<I", struct.pack("<f", x))[0]
+
+
+class KvCompatDescriptor:
+    """ctypes handle on hs_compat; fields are set by the names of the reference's struct."""
+
+    def __init__(self, **fields):
+        self._h = ctypes.c_void_p(lib().hs_compat_create())
+        self.set(**fields)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().hs_compat_destroy(self._h)
+            self._h = None
+
+    def set(self, **fields):
+        L = lib()
+        for name, v in fields.items():
+            key = name.replace("__", ".").encode()
+            if name == "kv_quant":
+                rc = L.hs_compat_set_kv_quant(self._h, v)
+            elif name == "layer_types":
+                rc = 0
+                for t in v:
+                    rc |= L.hs_compat_add_layer_type(self._h, t.encode())
+            elif name == "rope_scaling":
+                rc = L.hs_compat_set_rope_scaling(self._h, None if v is None else v[0].encode(), 0.0 if v is None else v[1])
+            elif isinstance(v, str) or (v is None and name == "tokenizer_hash"):
+                rc = L.hs_compat_set_str(self._h, key, None if v is None else v.encode())
+            elif isinstance(v, tuple):  # ("opt", value-or-None)
+                rc = L.hs_compat_set_opt_uint(self._h, key, int(v[1] is not None), 0 if v[1] is None else v[1])
+            else:
+                rc = L.hs_compat_set_uint(self._h, key, int(v))
+            if rc != 0:
+                raise ValueError("bad field %s=%r" % (name, v))
+        return self
+
+    def fingerprint(self):
+        buf = ctypes.create_string_buffer(32)
+        assert lib().hs_compat_fingerprint(self._h, buf) == 0
+        return buf.raw
+
+    def is_authoritatively_complete(self):
+        return bool(lib().hs_compat_is_authoritatively_complete(self._h))
+
+    def check_against(self, observed):
+        """None if compatible, else the first differing field."""
+        buf = ctypes.create_string_buffer(64)
+        rc = lib().hs_compat_check(self._h, observed._h, buf, 64)
+        assert rc in (0, 1)
+        return None if rc == 0 else buf.value.decode()
+
+
+def decide_cache_reuse(expected, stored, cache_is_empty):
+    return lib().hs_compat_decide_reuse(expected, stored, int(cache_is_empty))

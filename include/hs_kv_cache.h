@@ -54,6 +54,39 @@ HS_API int hs_cache_quant_type(const hs_cache *c);       /* kv_cache.rs:1861 */
  * purpose: a cache written in one format must never be reused as another.  NULL for an unknown value. */
 HS_API const char *hs_kv_quant_canonical_str(int quant_type);
 
+/* ---- cache identity: which cached K/V may be reused (kv_compat.rs:84-560, 836-1130) ---------------------------------
+ * hs_compat is a KvCompatDescriptor (kv_compat.rs:285-378): an ordered set of named fields whose SHA-256 over the
+ * reference's canonical byte framing (kv_compat.rs:458-520) is the fingerprint stamped on a cache; a fingerprint
+ * computed here equals the Rust side's for the same values (the reference's own pinned digest is a test vector).
+ * Fields are set by the names of the Rust struct ("head_dim", "rope_theta_bits", "weights.base_revision",
+ * "moe.num_experts", "tokenizer_hash", ...): hs_compat_set_uint for integers, bools and f32 bit patterns,
+ * hs_compat_set_opt_uint for Option<u32> / Option<usize>, hs_compat_set_str for strings ("dtype" takes a dtype name,
+ * NULL clears "tokenizer_hash").  An unknown field or a value of the wrong kind is HS_ERR_INVALID_ARGUMENT.
+ * KvQuantMode (kv_compat.rs:215-237) has two variants more than the reference, one per device format of this library,
+ * so that a cache written in one format is never reused as another or as the reference's blockwise "int8". */
+typedef struct hs_compat hs_compat;
+enum hs_kv_quant_mode { HS_KVQ_NONE = 0, HS_KVQ_INT8 = 1, HS_KVQ_NF4 = 2, HS_KVQ_FP4 = 3,
+                        HS_KVQ_INT8_TOKEN = 4,        /* "int8-token": int8 codes + fp32 scale per (token, kv-head) */
+                        HS_KVQ_FP8_E4M3FN_HEAD = 5 }; /* "fp8-e4m3fn-head": e4m3fn codes + fp32 scale per (sequence, kv-head) */
+enum hs_cache_reuse { HS_REUSE = 0, HS_STAMP_FRESH = 1, HS_DISCARD_AND_RECOMPUTE = 2 }; /* CacheReuseDecision, kv_compat.rs:1087-1101 */
+HS_API hs_compat *hs_compat_create(void);  /* format_version = 3, dtype bfloat16, everything else zero / empty / None */
+HS_API void hs_compat_destroy(hs_compat *c);
+HS_API int hs_compat_set_uint(hs_compat *c, const char *field, uint64_t value);
+HS_API int hs_compat_set_opt_uint(hs_compat *c, const char *field, int has_value, uint64_t value);
+HS_API int hs_compat_set_str(hs_compat *c, const char *field, const char *value);
+HS_API int hs_compat_add_layer_type(hs_compat *c, const char *value);
+HS_API int hs_compat_set_rope_scaling(hs_compat *c, const char *rope_type, float factor); /* NULL type = None */
+HS_API int hs_compat_set_kv_quant(hs_compat *c, int mode);                                 /* enum hs_kv_quant_mode */
+HS_API int hs_compat_is_authoritatively_complete(const hs_compat *c);                      /* kv_compat.rs:426-428 */
+HS_API int hs_compat_fingerprint(const hs_compat *c, uint8_t out32[32]);                   /* kv_compat.rs:440-442 */
+/* check_compatibility (kv_compat.rs:836-1080): 0 = compatible; 1 = not, and `field` receives the first differing
+ * field in the reference's fixed order ("weights" and "moe_routing" for the nested structs); -1 = null argument. */
+HS_API int hs_compat_check(const hs_compat *expected, const hs_compat *observed, char *field, size_t field_cap);
+/* decide_cache_reuse (kv_compat.rs:1118-1128), fail-closed; fingerprints are 32 bytes or NULL (= None). */
+HS_API int hs_compat_decide_reuse(const uint8_t *expected32, const uint8_t *stored32, int cache_is_empty);
+HS_API const char *hs_kv_quant_mode_str(int mode); /* KvQuantMode::as_canonical_str; NULL for an unknown value */
+HS_API int hs_kv_quant_mode_of(int quant_type);    /* the mode of a cache's storage format (enum hs_kv_quant); -1 unknown */
+
 /* cache.get() + GQA expand + compute_attention for one query token per sequence
  * (llama.rs:605-636, 847-872, 1023-1119).  q, out: bf16 [batch, num_q_heads, head_dim]. */
 HS_API int hs_cache_decode_attention(hs_cache *c, const void *q, void *out, int32_t num_q_heads,
