@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include "device_fill.hpp"
+
 #include <algorithm>
 #include <cstdio>
 
@@ -143,7 +145,9 @@ Status PagedLayerKVCache::reserve(size_t end_pos) {
     return {};
 }
 
-Status PagedLayerKVCache::sync_table() {
+// New table entries (a block pair every 256 tokens) go to the device with a copy ordered on the caller's stream, so
+// a kernel of an earlier step on that stream never sees a table that changes under it.
+Status PagedLayerKVCache::sync_table(hs_stream_t stream) {
     const size_t max_blocks = (max_seq_len + kBlockSize - 1) / kBlockSize;
     hipError_t e;
     if (!table_dev_) {
@@ -155,10 +159,10 @@ Status PagedLayerKVCache::sync_table() {
     if (table_synced_ > key_blocks_.size()) table_synced_ = 0;  // blocks were returned: rewrite what is left
     const size_t n = key_blocks_.size() - table_synced_;
     if (n) {
-        if ((e = hipMemcpy(table_dev_ + table_synced_, key_blocks_.data() + table_synced_, n * sizeof(int32_t),
-                           hipMemcpyHostToDevice)) != hipSuccess ||
-            (e = hipMemcpy(table_dev_ + max_blocks + table_synced_, value_blocks_.data() + table_synced_, n * sizeof(int32_t),
-                           hipMemcpyHostToDevice)) != hipSuccess)
+        if ((e = hipMemcpyAsync(table_dev_ + table_synced_, key_blocks_.data() + table_synced_, n * sizeof(int32_t),
+                                hipMemcpyHostToDevice, (hipStream_t)stream)) != hipSuccess ||
+            (e = hipMemcpyAsync(table_dev_ + max_blocks + table_synced_, value_blocks_.data() + table_synced_,
+                                n * sizeof(int32_t), hipMemcpyHostToDevice, (hipStream_t)stream)) != hipSuccess)
             return hip_err(e, "uploading the block table");
         table_synced_ = key_blocks_.size();
     }
@@ -173,7 +177,7 @@ Status PagedLayerKVCache::update(const void *new_keys, const void *new_values, i
     if (Status s = reserve(end_pos); !s.ok()) return s;
     if (seq_len > 0) {
         if (Status s = pool_->ensure_device(); !s.ok()) return s;
-        if (Status s = sync_table(); !s.ok()) return s;
+        if (Status s = sync_table(stream); !s.ok()) return s;
         const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
         const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
         int rc = hs_kv_quantize_int8(new_keys, new_values, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(),
@@ -193,7 +197,7 @@ Status PagedLayerKVCache::prefill(const void *q, const void *new_keys, const voi
     if (Status s = reserve(end_pos); !s.ok()) return s;
     if (seq_len > 0) {
         if (Status s = pool_->ensure_device(); !s.ok()) return s;
-        if (Status s = sync_table(); !s.ok()) return s;
+        if (Status s = sync_table(stream); !s.ok()) return s;
         const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
         const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
         int rc = hs_prefill_attn_int8(q, new_keys, new_values, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
@@ -207,7 +211,7 @@ Status PagedLayerKVCache::prefill(const void *q, const void *new_keys, const voi
 
 Status PagedLayerKVCache::get_dense(void *keys_out, void *values_out, int dtype, hs_stream_t stream) {
     if (seq_pos == 0) return err(HS_ERR_INVALID_ARGUMENT, "Cache is empty");
-    if (Status s = sync_table(); !s.ok()) return s;
+    if (Status s = sync_table(stream); !s.ok()) return s;
     const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
     const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
     int rc = hs_kv_dequantize(pool_->codes(), pool_->scales(), 0, &l, 0, keys_out, dtype, 1, (int32_t)seq_pos,
@@ -220,19 +224,22 @@ Status PagedLayerKVCache::get_dense(void *keys_out, void *values_out, int dtype,
 
 Status PagedLayerKVCache::decode_attention(const void *q, void *out, int32_t hq, float scale, hs_stream_t stream) {
     if (seq_pos == 0) return err(HS_ERR_INVALID_ARGUMENT, "Cache is empty");
-    if (Status s = sync_table(); !s.ok()) return s;
+    if (Status s = sync_table(stream); !s.ok()) return s;
     const int32_t heads = pool_->num_kv_heads(), dim = pool_->head_dim();
-    const size_t need = hs_decode_attn_workspace_bytes(1, hq, heads, dim, (int32_t)seq_pos);
+    const size_t need = hs_decode_attn_workspace_bytes(1, hq, heads, dim, (int32_t)max_seq_len);  // sized once
     hipError_t e;
     if (need > workspace_bytes_) {
-        if (workspace_) (void)hipFree(workspace_);
+        if (workspace_) {
+            if ((e = hipDeviceSynchronize()) != hipSuccess) return hip_err(e, "waiting before the workspace grows");
+            (void)hipFree(workspace_);
+        }
         workspace_ = nullptr;
         workspace_bytes_ = 0;
         if ((e = hipMalloc(&workspace_, need)) != hipSuccess) return hip_err(e, "allocating the workspace");
         workspace_bytes_ = need;
     }
     const int32_t len = (int32_t)seq_pos;
-    if ((e = hipMemcpy(len_dev_, &len, sizeof(len), hipMemcpyHostToDevice)) != hipSuccess) return hip_err(e, "uploading the length");
+    if ((e = fill_i32(len_dev_, 1, len, (hipStream_t)stream)) != hipSuccess) return hip_err(e, "setting the length");
     const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
     const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
     return from_abi(hs_decode_attn_int8(q, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l, len_dev_, out,
@@ -266,8 +273,37 @@ void PagedLayerKVCache::truncate_to(size_t pos) {
 PagedBatch::PagedBatch(std::shared_ptr<BlockPool> pool) : pool_(std::move(pool)) {}
 
 PagedBatch::~PagedBatch() {
-    for (void *p : {(void *)tables_dev_, workspace_})
-        if (p) (void)hipFree(p);
+    for (Slot &sl : slots_) {
+        if (sl.dev) (void)hipFree(sl.dev);
+        if (sl.host) (void)hipHostFree(sl.host);
+        if (sl.done) (void)hipEventDestroy(sl.done);
+    }
+    if (workspace_) (void)hipFree(workspace_);
+}
+
+// A step's tables and lengths travel through one of kSlots (pinned host buffer, device buffer) pairs with a copy
+// ordered on the caller's stream; a pair is reused only after the step that last used it has finished on the GPU
+// (an event per pair; in steady state it has long fired, so nothing blocks).
+Status PagedBatch::slot_for(size_t ints, Slot **out) {
+    Slot &sl = slots_[next_slot_++ % kSlots];
+    hipError_t e;
+    if (sl.done && sl.in_use) {
+        if ((e = hipEventSynchronize(sl.done)) != hipSuccess) return hip_err(e, "waiting for a table slot");
+        sl.in_use = false;
+    }
+    if (!sl.done && (e = hipEventCreateWithFlags(&sl.done, hipEventDisableTiming)) != hipSuccess) return hip_err(e, "creating an event");
+    if (ints > sl.cap) {
+        if (sl.dev) (void)hipFree(sl.dev);
+        if (sl.host) (void)hipHostFree(sl.host);
+        sl.dev = nullptr; sl.host = nullptr; sl.cap = 0;
+        const size_t cap = ints * 2;
+        if ((e = hipMalloc((void **)&sl.dev, cap * sizeof(int32_t))) != hipSuccess) return hip_err(e, "allocating the block tables");
+        if ((e = hipHostMalloc((void **)&sl.host, cap * sizeof(int32_t), hipHostMallocDefault)) != hipSuccess)
+            return hip_err(e, "allocating the pinned block tables");
+        sl.cap = cap;
+    }
+    *out = &sl;
+    return {};
 }
 
 Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const void *q, const void *k_new, const void *v_new,
@@ -285,27 +321,29 @@ Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const 
         stride = std::max(stride, rows[i]->num_blocks());
     }
     if (Status s = pool_->ensure_device(); !s.ok()) return s;
-    std::vector<int32_t> host((size_t)n * stride * 2 + (size_t)n, 0);
-    int32_t *kt = host.data(), *vt = kt + (size_t)n * stride, *lens = vt + (size_t)n * stride;
+    const size_t ints = (size_t)n * stride * 2 + (size_t)n;
+    Slot *sl = nullptr;
+    if (Status s = slot_for(ints, &sl); !s.ok()) return s;
+    std::fill(sl->host, sl->host + ints, 0);
+    int32_t *kt = sl->host, *vt = kt + (size_t)n * stride, *lens = vt + (size_t)n * stride;
+    size_t max_cap = 0;
+    for (int32_t i = 0; i < n; ++i) max_cap = std::max(max_cap, rows[i]->max_seq_len);
     for (int32_t i = 0; i < n; ++i) {
         std::copy(rows[i]->key_blocks().begin(), rows[i]->key_blocks().end(), kt + (size_t)i * stride);
         std::copy(rows[i]->value_blocks().begin(), rows[i]->value_blocks().end(), vt + (size_t)i * stride);
         lens[i] = (int32_t)(rows[i]->seq_pos + 1);
     }
     hipError_t e;
-    if (host.size() > tables_cap_) {
-        if (tables_dev_) (void)hipFree(tables_dev_);
-        tables_dev_ = nullptr;
-        tables_cap_ = 0;
-        if ((e = hipMalloc((void **)&tables_dev_, host.size() * 2 * sizeof(int32_t))) != hipSuccess) return hip_err(e, "allocating the block tables");
-        tables_cap_ = host.size() * 2;
-    }
-    if ((e = hipMemcpy(tables_dev_, host.data(), host.size() * sizeof(int32_t), hipMemcpyHostToDevice)) != hipSuccess)
+    if ((e = hipMemcpyAsync(sl->dev, sl->host, ints * sizeof(int32_t), hipMemcpyHostToDevice, (hipStream_t)stream)) != hipSuccess)
         return hip_err(e, "uploading the block tables");
+    int32_t *tables_dev_ = sl->dev;
     const int32_t heads = pool_->num_kv_heads(), dim = pool_->head_dim();
-    const size_t need = hs_decode_attn_workspace_bytes(n, hq, heads, dim, (int32_t)max_len);
+    const size_t need = hs_decode_attn_workspace_bytes(n, hq, heads, dim, (int32_t)max_cap);  // for the rows' capacity: grows rarely
     if (need > workspace_bytes_) {
-        if (workspace_) (void)hipFree(workspace_);
+        if (workspace_) {
+            if ((e = hipDeviceSynchronize()) != hipSuccess) return hip_err(e, "waiting before the workspace grows");
+            (void)hipFree(workspace_);
+        }
         workspace_ = nullptr;
         workspace_bytes_ = 0;
         if ((e = hipMalloc(&workspace_, need)) != hipSuccess) return hip_err(e, "allocating the workspace");
@@ -317,6 +355,8 @@ Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const 
                                  tables_dev_ + 2 * (size_t)n * stride, out, workspace_, workspace_bytes_, n, hq, heads, dim,
                                  (int32_t)max_len, scale, stream);
     if (rc != HS_OK) return from_abi(rc);
+    if ((e = hipEventRecord(sl->done, (hipStream_t)stream)) != hipSuccess) return hip_err(e, "recording the slot event");
+    sl->in_use = true;
     for (int32_t i = 0; i < n; ++i) rows[i]->seq_pos += 1;
     return {};
 }

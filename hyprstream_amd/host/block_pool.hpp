@@ -18,6 +18,8 @@
 #include <string>
 #include <vector>
 
+#include <hip/hip_runtime_api.h>
+
 #include "kv_cache.hpp"
 
 namespace hs {
@@ -109,7 +111,7 @@ class PagedLayerKVCache {
     size_t max_seq_len = 0;
 
   private:
-    Status sync_table();
+    Status sync_table(hs_stream_t stream);
     std::shared_ptr<BlockPool> pool_;
     CacheOwner owner_;
     std::vector<BlockId> key_blocks_, value_blocks_;
@@ -134,9 +136,17 @@ class PagedBatch {
                        int dtype, void *out, int32_t num_q_heads, float softmax_scale, hs_stream_t stream = nullptr);
 
   private:
+    static constexpr int kSlots = 4;
+    struct Slot {  // K tables, V tables and lengths of one step: pinned host copy, device copy, "step finished" event
+        int32_t *host = nullptr, *dev = nullptr;
+        size_t cap = 0;
+        hipEvent_t done = nullptr;
+        bool in_use = false;
+    };
+    Status slot_for(size_t ints, Slot **out);
     std::shared_ptr<BlockPool> pool_;
-    int32_t *tables_dev_ = nullptr;  // K tables, V tables, lengths of the current step
-    size_t tables_cap_ = 0;
+    Slot slots_[kSlots];
+    unsigned next_slot_ = 0;
     void *workspace_ = nullptr;
     size_t workspace_bytes_ = 0;
 };

@@ -4,6 +4,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include "device_fill.hpp"
+
 #include <cstdio>
 #include <vector>
 
@@ -28,7 +30,6 @@ void LayerKVCache::release() {
     k_scales_ = v_scales_ = nullptr;
     seq_lens_dev_ = nullptr;
     workspace_bytes_ = 0;
-    seq_lens_value_ = (size_t)-1;
     batch_ = heads_ = dim_ = 0;
     bytes_ = 0;
 }
@@ -66,21 +67,23 @@ Status LayerKVCache::ensure_storage(int32_t batch, int32_t heads, int32_t dim) {
     return {};
 }
 
-Status LayerKVCache::ensure_scratch(size_t bytes, int32_t batch) {
+// The split-K workspace is sized ONCE for max_seq_len (it only ever grows if a later call brings more query heads),
+// so steady-state steps neither allocate nor free.  The sequence lengths reach the device through a fill launch on
+// the caller's stream, ordered with the attention launch that reads them.
+Status LayerKVCache::ensure_scratch(int32_t hq, int32_t batch, hs_stream_t stream) {
+    const size_t bytes = hs_decode_attn_workspace_bytes(batch, hq, heads_, dim_, (int32_t)max_seq_len);
     if (bytes > workspace_bytes_) {
-        if (workspace_) (void)hipFree(workspace_);
+        if (workspace_) {
+            // an earlier step on some stream may still use the old buffer
+            if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) return hip_err(e, "waiting before the workspace grows");
+            (void)hipFree(workspace_);
+        }
         workspace_ = nullptr;
         workspace_bytes_ = 0;
         if (hipError_t e = hipMalloc(&workspace_, bytes); e != hipSuccess) return hip_err(e, "allocating the workspace");
         workspace_bytes_ = bytes;
     }
-    if (seq_lens_value_ != seq_pos) {
-        std::vector<int32_t> lens((size_t)batch, (int32_t)seq_pos);
-        if (hipError_t e = hipMemcpy(seq_lens_dev_, lens.data(), sizeof(int32_t) * batch, hipMemcpyHostToDevice); e != hipSuccess)
-            return hip_err(e, "uploading sequence lengths");
-        seq_lens_value_ = seq_pos;
-    }
-    return {};
+    return hip_err(fill_i32(seq_lens_dev_, batch, (int32_t)seq_pos, (hipStream_t)stream), "setting the sequence lengths");
 }
 
 Status LayerKVCache::update(const void *new_keys, const void *new_values, int dtype, int32_t batch, int32_t seq_len,
@@ -139,8 +142,7 @@ Status LayerKVCache::get_dense(void *keys_out, void *values_out, int dtype, hs_s
 Status LayerKVCache::decode_attention(const void *q, void *out, int32_t hq, float scale, hs_stream_t stream) {
     KVView v;
     if (Status s = get(&v); !s.ok()) return s;
-    const size_t need = hs_decode_attn_workspace_bytes(batch_, hq, heads_, dim_, (int32_t)seq_pos);
-    if (Status s = ensure_scratch(need, batch_); !s.ok()) return s;
+    if (Status s = ensure_scratch(hq, batch_, stream); !s.ok()) return s;
     int rc = quant_type_ == KVQuantType::Fp8
                  ? hs_decode_attn_fp8(q, (const uint8_t *)k_codes_, (const uint8_t *)v_codes_, k_scales_, v_scales_, &layout_,
                                       seq_lens_dev_, out, workspace_, workspace_bytes_, batch_, hq, heads_, dim_, (int32_t)seq_pos, scale, stream)
@@ -158,8 +160,7 @@ Status LayerKVCache::decode_step(const void *q, const void *k_new, const void *v
         return err(HS_ERR_OVERFLOW, buf);
     }
     seq_pos += 1;  // the entry point writes the new token at seq_pos - 1 and attends seq_pos tokens
-    const size_t need = hs_decode_attn_workspace_bytes(batch_, hq, heads_, dim_, (int32_t)seq_pos);
-    Status s = ensure_scratch(need, batch_);
+    Status s = ensure_scratch(hq, batch_, stream);
     int rc = HS_OK;
     if (s.ok()) {
         rc = quant_type_ == KVQuantType::Fp8

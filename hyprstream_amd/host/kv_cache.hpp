@@ -82,14 +82,13 @@ class LayerKVCache {
 
   private:
     Status ensure_storage(int32_t batch, int32_t num_kv_heads, int32_t head_dim);
-    Status ensure_scratch(size_t bytes, int32_t batch);
+    Status ensure_scratch(int32_t num_q_heads, int32_t batch, hs_stream_t stream);
     void release();
 
     KVQuantType quant_type_;
     void *k_codes_ = nullptr, *v_codes_ = nullptr;
     float *k_scales_ = nullptr, *v_scales_ = nullptr;
-    int32_t *seq_lens_dev_ = nullptr;  // [batch], every entry == seq_pos
-    size_t seq_lens_value_ = (size_t)-1;
+    int32_t *seq_lens_dev_ = nullptr;  // [batch]; set to seq_pos by a fill launch on the step's stream
     void *workspace_ = nullptr;
     size_t workspace_bytes_ = 0;
     hs_kv_layout layout_{};

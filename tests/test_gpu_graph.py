@@ -71,3 +71,78 @@ def test_chunked_prefill_in_a_graph():
         g.replay()
         torch.cuda.synchronize()
         assert bool(torch.equal(out, want)) and bool(torch.equal(c.k_codes, want_codes)), "replay %d" % i
+
+
+def _cache_with_history(B, T0, cap, Hkv, D, seed, quant):
+    from hyprstream_amd import kv_cache as kc
+    r = wl.philox(seed)
+    rnd = lambda *s: torch.from_numpy(r.standard_normal(s).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    c = kc.LayerKVCache(cap, quant)
+    c.update(rnd(B, T0, Hkv, D), rnd(B, T0, Hkv, D), 0)
+    return c, rnd
+
+
+@pytest.mark.parametrize("B,T0", [(64, 300), (2, 2500)])
+def test_cache_object_decode_step_in_a_graph(B, T0):
+    """A decode step through the LayerKVCache mirror (hs_cache_decode_step) is launches only -- the sequence lengths
+    reach the device through a fill launch on the step's stream, the workspace is sized once for max_seq_len -- so it
+    can be captured.  A captured step replays at the position it was captured at: the host rewinds with truncate_to."""
+    from hyprstream_amd import kv_cache as kc
+    Hq, Hkv, D = 32, 8, 128
+    c, rnd = _cache_with_history(B, T0, T0 + 8, Hkv, D, 1520 + B, kc.INT8)
+    q, kn, vn = rnd(B, Hq, D), rnd(B, 1, Hkv, D), rnd(B, 1, Hkv, D)
+    want = c.decode_step(q, kn, vn, 0.0884)  # eager: also sizes the workspace, outside any capture
+    torch.cuda.synchronize()
+    assert c.seq_pos == T0 + 1
+    kw, vw = c.get()
+    out = torch.empty_like(q)
+    L = kc.lib()
+    import ctypes
+
+    def step():
+        rc = L.hs_cache_decode_step(c._h, hb._ptr(q), hb._ptr(kn), hb._ptr(vn), hb.HS_BF16, hb._ptr(out), Hq,
+                                    ctypes.c_float(0.0884), hb._stream())
+        assert rc == 0, L.hs_cache_last_error(c._h)
+
+    c.truncate_to(T0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    c.truncate_to(T0)
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    assert c.seq_pos == T0 + 1
+    for i in range(4):
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert bool(torch.equal(out, want)), "replay %d differs from the eager step" % i
+        (q.float().reshape(B, -1) @ q.float().reshape(B, -1).T).sum().item()
+    k2, v2 = c.get()
+    assert bool(torch.equal(k2, kw)) and bool(torch.equal(v2, vw))
+
+
+def test_cache_object_steps_on_a_side_stream_match_the_default_stream():
+    """Steps enqueued back to back on a non-blocking side stream, with no host synchronisation in between: each step's
+    lengths are ordered behind the previous step's kernel on that stream, so no step reads another step's length."""
+    from hyprstream_amd import kv_cache as kc
+    B, Hq, Hkv, D, T0, n = 3, 16, 4, 128, 500, 12
+    outs = []
+    for use_side in (False, True):
+        c, rnd = _cache_with_history(B, T0, T0 + n, Hkv, D, 1530, kc.INT8)
+        toks = [(rnd(B, Hq, D), rnd(B, 1, Hkv, D), rnd(B, 1, Hkv, D)) for _ in range(n)]
+        torch.cuda.synchronize()
+        stream = torch.cuda.Stream() if use_side else torch.cuda.current_stream()
+        with torch.cuda.stream(stream):
+            res = [c.decode_step(q, k, v, 0.0884) for q, k, v in toks]
+        stream.synchronize()
+        torch.cuda.synchronize()
+        assert c.seq_pos == T0 + n
+        outs.append((torch.stack(res), c.get()))
+    assert bool(torch.equal(outs[0][0], outs[1][0]))
+    assert bool(torch.equal(outs[0][1][0], outs[1][1][0])) and bool(torch.equal(outs[0][1][1], outs[1][1][1]))
