@@ -23,6 +23,48 @@ def test_header_declares_what_bindings_expect():
         assert name in decl
 
 
+def _c_arity(header):
+    """name -> number of parameters, from the header text."""
+    text = re.sub(r"/\*.*?\*/", " ", open(os.path.join(ROOT, "include", header)).read(), flags=re.S)
+    out = {}
+    for m in re.finditer(r"HS_API\s+[^;{]*?\b(hs_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = " ".join(m.group(2).split())
+        out[m.group(1)] = 0 if args in ("void", "") else args.count(",") + 1
+    return out
+
+
+def _rust_arity():
+    text = open(os.path.join(ROOT, "hs-attn-sys", "src", "bindings.rs")).read()
+    out = {}
+    for m in re.finditer(r"pub fn (hs_\w+)\(([^)]*)\)", text):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if not args else args.count(":")
+    return out
+
+
+def test_rust_bindings_match_the_headers_name_for_name_and_in_arity():
+    """hs-attn-sys/src/bindings.rs is what a maintainer compiles in hyprstream's tree (no rustc here): every entry point
+    of both headers must be declared there with the same number of parameters, and nothing else."""
+    want = dict(_c_arity("hs_attn.h"))
+    want.update(_c_arity("hs_kv_cache.h"))
+    got = _rust_arity()
+    assert len(want) > 70
+    assert sorted(got) == sorted(want), (sorted(set(want) - set(got)), sorted(set(got) - set(want)))
+    assert {n: a for n, a in got.items() if want[n] != a} == {}
+    text = open(os.path.join(ROOT, "hs-attn-sys", "src", "bindings.rs")).read()
+    assert "pub const HS_ATTN_ABI_VERSION: c_int = %d;" % hb.lib().hs_attn_abi_version() in text
+    # the structs carry every field of the C structs, in order
+    for struct, cls in (("hs_kv_layout", hb.KvLayout), ("hs_qk_prologue", hb.QkPrologue)):
+        body = re.search(r"pub struct %s \{(.*?)\}" % struct, text, flags=re.S).group(1)
+        assert re.findall(r"pub (\w+):", body) == [f[0] for f in cls._fields_]
+
+
+def test_rust_wrappers_call_only_declared_bindings():
+    lib_rs = open(os.path.join(ROOT, "hs-attn-sys", "src", "lib.rs")).read()
+    used = set(re.findall(r"bindings::(hs_\w+)\(", lib_rs))
+    assert used and used <= set(_rust_arity())
+
+
 def test_library_exports_every_declared_symbol():
     L = hb.lib()
     missing = [s for s in declared_symbols() if not hasattr(L, s)]
