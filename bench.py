@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c5-decode|c5-prefill|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c5-decode|c5-prefill|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -66,6 +66,9 @@ WORKLOADS = {
     "d256-fp8": (32, 16, 4, 256, 32768, False, True, 0.5, False),
     # 64-wide heads (the reference's paged-cache tests use them), same cache bytes as c2
     "d64-int8": (64, 32, 16, 64, 8192, False, False, 1.0, True),
+    # c2 with the cache in 256-token blocks scattered through a pool (the reference's BlockPool geometry,
+    # kv_cache.rs:477): the same bytes, every wavefront step resolved through the block table
+    "c2-paged": (64, 32, 8, 128, 8192, False, False, 1.0, True),
 }
 
 
@@ -267,6 +270,7 @@ def main():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c5-decode", "c5-prefill", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
@@ -334,6 +338,26 @@ def main():
     for c in range(1, ncopies):
         for dst, src in zip(caches[c], caches[0]):
             dst.copy_(src)
+    paged = args.workload == "c2-paged"
+    if paged:
+        # every cache copy becomes a pool of 256-token blocks in a random order; K and V blocks of a sequence come from
+        # one pool (ids 0..n-1 for K, n..2n-1 for V before the shuffle), as PagedLayerKVCache takes them
+        BT = args.block_tokens
+        nb = T // BT
+        perm = torch.randperm(2 * B * nb, generator=torch.Generator().manual_seed(wl.SEED)).to(torch.int32)
+        k_tab = perm[: B * nb].reshape(B, nb).contiguous().to(dev)
+        v_tab = perm[B * nb:].reshape(B, nb).contiguous().to(dev)
+        pools = []
+        for kc, vc, ks, vs in caches:
+            pc = torch.empty(2 * B * nb, Hkv, BT, D, dtype=cdt, device=dev)
+            ps = torch.empty(2 * B * nb, Hkv, BT, dtype=torch.float32, device=dev)
+            pc[k_tab.long().reshape(-1)] = kc.reshape(B, Hkv, nb, BT, D).permute(0, 2, 1, 3, 4).reshape(B * nb, Hkv, BT, D)
+            pc[v_tab.long().reshape(-1)] = vc.reshape(B, Hkv, nb, BT, D).permute(0, 2, 1, 3, 4).reshape(B * nb, Hkv, BT, D)
+            ps[k_tab.long().reshape(-1)] = ks[:, :, :T].reshape(B, Hkv, nb, BT).permute(0, 2, 1, 3).reshape(B * nb, Hkv, BT)
+            ps[v_tab.long().reshape(-1)] = vs[:, :, :T].reshape(B, Hkv, nb, BT).permute(0, 2, 1, 3).reshape(B * nb, Hkv, BT)
+            pools.append((pc, pc, ps, ps))
+        flat_caches, caches = caches, pools
+        layout = hb.paged_layout(Hkv, BT, D, k_tab, v_tab)
     if ragged:
         lens = torch.randint(512, T + 1, (B,), generator=gen, device=dev, dtype=torch.int32)
     else:
@@ -447,11 +471,11 @@ def main():
                      "algorithmic_bytes_per_launch": int(kern_bytes), "launches_timed": n_ev},
     }
     if not args.no_cpu_baseline:
-        cb, _ = cpu_baseline(torch, args.workload, caches[0], q, lens, Hq, fp8)
+        cb, _ = cpu_baseline(torch, args.workload, (flat_caches if paged else caches)[0], q, lens, Hq, fp8)
         if args.workload == "c2":
             # the reference's own CPU-runnable configuration (one sequence, 2048 tokens, int8), whole, same op sequence
             T1 = 2048
-            one = tuple(t[:1, :, :T1].contiguous() for t in caches[0])
+            one = tuple(t[:1, :, :T1].contiguous() for t in (flat_caches if paged else caches)[0])
             c1, _ = cpu_baseline(torch, "c1", one, q[:1], torch.full((1,), T1, dtype=torch.int32), Hq, False, seconds_budget=3.0)
             cb["single_sequence_2048"] = {k: c1[k] for k in ("value", "unit", "ms_per_call", "tokens_per_s")}
         result["cpu_baseline"] = cb

@@ -17,6 +17,7 @@ int check_launch(const char *what);
 struct KvAddr {
     int64_t code_stride_seq, code_stride_head, scale_stride_seq, scale_stride_head;
     int32_t capacity_tokens, block_table_stride;
+    int32_t cap_shift;     // log2(capacity_tokens) when that is a power of two (the usual 256-token blocks), else -1
     const int32_t *table;  // K or V table already chosen; nullptr = not paged
 };
 
@@ -28,6 +29,10 @@ inline KvAddr make_addr(const hs_kv_layout &l, int which_table) {
     a.scale_stride_head = l.scale_stride_head;
     a.capacity_tokens = l.capacity_tokens;
     a.block_table_stride = l.block_table_stride;
+    a.cap_shift = -1;
+    if (l.capacity_tokens > 0 && (l.capacity_tokens & (l.capacity_tokens - 1)) == 0)
+        for (int s = 0; s < 31; ++s)
+            if ((1 << s) == l.capacity_tokens) a.cap_shift = s;
     a.table = which_table ? l.v_block_table : l.k_block_table;
     return a;
 }
@@ -39,7 +44,7 @@ __device__ __forceinline__ bool resolve(const KvAddr &a, int b, int t, int64_t &
     slot = 0;
     if (t < 0) return false;
     if (a.table) {
-        int blk = t / a.capacity_tokens;
+        int blk = a.cap_shift >= 0 ? t >> a.cap_shift : t / a.capacity_tokens;
         if (blk >= a.block_table_stride) return false;
         int id = a.table[(int64_t)b * a.block_table_stride + blk];
         if (id < 0) return false;

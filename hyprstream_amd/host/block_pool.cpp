@@ -7,6 +7,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <cstring>
 
 namespace hs {
 
@@ -34,7 +35,8 @@ std::string CacheOwner::str() const {
 
 // ------------------------------------------------------------------------------------------------ BlockPool
 
-BlockPool::BlockPool(size_t num_blocks, int32_t heads, int32_t dim) : total_(num_blocks), heads_(heads), dim_(dim) {
+BlockPool::BlockPool(size_t num_blocks, int32_t heads, int32_t dim, KVQuantType format)
+    : total_(num_blocks), heads_(heads), dim_(dim), format_(format) {
     free_list_.reserve(num_blocks);
     for (size_t id = 0; id < num_blocks; ++id) free_list_.push_back((BlockId)id);  // pop() hands out the highest id first
     owner_.resize(num_blocks);
@@ -91,7 +93,8 @@ Status BlockPool::ensure_device() {
     if (codes_) return {};
     if (total_ == 0) return err(HS_ERR_INVALID_ARGUMENT, "the pool has no blocks");
     const size_t cb = total_ * (size_t)heads_ * kBlockSize * (size_t)dim_;
-    const size_t sb = total_ * (size_t)heads_ * kBlockSize * sizeof(float);
+    // fp8 blocks carry no scales; a token array of the smallest size keeps the pointer non-null for the kernel ABI
+    const size_t sb = fp8() ? 256 : total_ * (size_t)heads_ * kBlockSize * sizeof(float);
     hipError_t e;
     if ((e = hipMalloc((void **)&codes_, cb)) != hipSuccess) return hip_err(e, "allocating the block pool");
     if ((e = hipMalloc((void **)&scales_, sb)) != hipSuccess) {
@@ -125,7 +128,7 @@ PagedLayerKVCache::PagedLayerKVCache(size_t max_len, std::shared_ptr<BlockPool> 
 
 PagedLayerKVCache::~PagedLayerKVCache() {
     clear();
-    for (void *p : {(void *)table_dev_, (void *)len_dev_, workspace_})
+    for (void *p : {(void *)table_dev_, (void *)len_dev_, (void *)head_scales_dev_, workspace_})
         if (p) (void)hipFree(p);
 }
 
@@ -154,6 +157,8 @@ Status PagedLayerKVCache::sync_table(hs_stream_t stream) {
         if ((e = hipMalloc((void **)&table_dev_, 2 * std::max<size_t>(max_blocks, 1) * sizeof(int32_t))) != hipSuccess)
             return hip_err(e, "allocating the block table");
         if ((e = hipMalloc((void **)&len_dev_, sizeof(int32_t))) != hipSuccess) return hip_err(e, "allocating the length");
+        if (pool_->fp8() && (e = hipMalloc((void **)&head_scales_dev_, 2 * sizeof(float) * pool_->num_kv_heads())) != hipSuccess)
+            return hip_err(e, "allocating the head scales");
         table_synced_ = 0;
     }
     if (table_synced_ > key_blocks_.size()) table_synced_ = 0;  // blocks were returned: rewrite what is left
@@ -180,8 +185,19 @@ Status PagedLayerKVCache::update(const void *new_keys, const void *new_values, i
         if (Status s = sync_table(stream); !s.ok()) return s;
         const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
         const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
-        int rc = hs_kv_quantize_int8(new_keys, new_values, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(),
+        int rc;
+        if (pool_->fp8()) {
+            float *ks = head_scales_dev_, *vs = head_scales_dev_ + pool_->num_kv_heads();
+            if (start_pos == 0) {  // fresh prompt: calibrate the per-head scales on it, as the contiguous cache does
+                rc = hs_kv_fp8_calibrate(new_keys, new_values, dtype, ks, vs, 1, seq_len, pool_->num_kv_heads(), pool_->head_dim(), stream);
+                if (rc != HS_OK) return from_abi(rc);
+            }
+            rc = hs_kv_quantize_fp8(new_keys, new_values, dtype, (uint8_t *)pool_->codes(), (uint8_t *)pool_->codes(), ks, vs, &l,
+                                    nullptr, (int32_t)start_pos, 1, seq_len, pool_->num_kv_heads(), pool_->head_dim(), stream);
+        } else {
+            rc = hs_kv_quantize_int8(new_keys, new_values, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(),
                                      &l, nullptr, (int32_t)start_pos, 1, seq_len, pool_->num_kv_heads(), pool_->head_dim(), stream);
+        }
         if (rc != HS_OK) return from_abi(rc);
     }
     seq_pos = end_pos;
@@ -200,9 +216,20 @@ Status PagedLayerKVCache::prefill(const void *q, const void *new_keys, const voi
         if (Status s = sync_table(stream); !s.ok()) return s;
         const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
         const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
-        int rc = hs_prefill_attn_int8(q, new_keys, new_values, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
+        int rc;
+        if (pool_->fp8()) {
+            float *ks = head_scales_dev_, *vs = head_scales_dev_ + pool_->num_kv_heads();
+            if (start_pos == 0) {
+                rc = hs_kv_fp8_calibrate(new_keys, new_values, HS_BF16, ks, vs, 1, seq_len, pool_->num_kv_heads(), pool_->head_dim(), stream);
+                if (rc != HS_OK) return from_abi(rc);
+            }
+            rc = hs_prefill_attn_fp8(q, new_keys, new_values, (uint8_t *)pool_->codes(), (uint8_t *)pool_->codes(), ks, vs, &l,
+                                     (int32_t)start_pos, out, 1, seq_len, hq, pool_->num_kv_heads(), pool_->head_dim(), scale, 1, stream);
+        } else {
+            rc = hs_prefill_attn_int8(q, new_keys, new_values, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
                                       (int32_t)start_pos, out, 1, seq_len, hq, pool_->num_kv_heads(), pool_->head_dim(), scale, 1,
                                       stream);
+        }
         if (rc != HS_OK) return from_abi(rc);
     }
     seq_pos = end_pos;
@@ -214,10 +241,12 @@ Status PagedLayerKVCache::get_dense(void *keys_out, void *values_out, int dtype,
     if (Status s = sync_table(stream); !s.ok()) return s;
     const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
     const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
-    int rc = hs_kv_dequantize(pool_->codes(), pool_->scales(), 0, &l, 0, keys_out, dtype, 1, (int32_t)seq_pos,
+    const int fp8 = pool_->fp8();
+    const float *ks = fp8 ? head_scales_dev_ : pool_->scales(), *vs = fp8 ? head_scales_dev_ + pool_->num_kv_heads() : pool_->scales();
+    int rc = hs_kv_dequantize(pool_->codes(), ks, fp8, &l, 0, keys_out, dtype, 1, (int32_t)seq_pos,
                               pool_->num_kv_heads(), pool_->head_dim(), stream);
     if (rc == HS_OK)
-        rc = hs_kv_dequantize(pool_->codes(), pool_->scales(), 0, &l, 1, values_out, dtype, 1, (int32_t)seq_pos,
+        rc = hs_kv_dequantize(pool_->codes(), vs, fp8, &l, 1, values_out, dtype, 1, (int32_t)seq_pos,
                               pool_->num_kv_heads(), pool_->head_dim(), stream);
     return from_abi(rc);
 }
@@ -242,6 +271,10 @@ Status PagedLayerKVCache::decode_attention(const void *q, void *out, int32_t hq,
     if ((e = fill_i32(len_dev_, 1, len, (hipStream_t)stream)) != hipSuccess) return hip_err(e, "setting the length");
     const int32_t stride = (int32_t)((max_seq_len + kBlockSize - 1) / kBlockSize);
     const hs_kv_layout l = pool_->layout(table_dev_, table_dev_ + stride, stride);
+    if (pool_->fp8())
+        return from_abi(hs_decode_attn_fp8(q, (const uint8_t *)pool_->codes(), (const uint8_t *)pool_->codes(), head_scales_dev_,
+                                           head_scales_dev_ + heads, &l, len_dev_, out, workspace_, workspace_bytes_, 1, hq, heads,
+                                           dim, len, scale, stream));
     return from_abi(hs_decode_attn_int8(q, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l, len_dev_, out,
                                         workspace_, workspace_bytes_, 1, hq, heads, dim, len, scale, stream));
 }
@@ -321,7 +354,17 @@ Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const 
         stride = std::max(stride, rows[i]->num_blocks());
     }
     if (Status s = pool_->ensure_device(); !s.ok()) return s;
-    const size_t ints = (size_t)n * stride * 2 + (size_t)n;
+    // int32 units of the slot: K tables, V tables, lengths; an fp8 step adds (8-byte aligned) the rows' scale pointers
+    // and the gathered [2][n][Hkv] scales
+    const bool fp8 = pool_->fp8();
+    const int32_t hk = pool_->num_kv_heads();
+    const size_t base_ints = (size_t)n * stride * 2 + (size_t)n;
+    const size_t ptr_off = (base_ints + 1) / 2 * 2;
+    const size_t gath_off = ptr_off + 2 * (size_t)n;
+    const size_t ints = fp8 ? gath_off + 2 * (size_t)n * hk : base_ints;
+    if (fp8)
+        for (int32_t i = 0; i < n; ++i)
+            if (!rows[i]->head_scales()) return err(HS_ERR_INVALID_ARGUMENT, "row " + std::to_string(i) + " has no calibrated scales yet (cache is empty)");
     Slot *sl = nullptr;
     if (Status s = slot_for(ints, &sl); !s.ok()) return s;
     std::fill(sl->host, sl->host + ints, 0);
@@ -332,10 +375,18 @@ Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const 
         std::copy(rows[i]->key_blocks().begin(), rows[i]->key_blocks().end(), kt + (size_t)i * stride);
         std::copy(rows[i]->value_blocks().begin(), rows[i]->value_blocks().end(), vt + (size_t)i * stride);
         lens[i] = (int32_t)(rows[i]->seq_pos + 1);
+        if (fp8) {
+            const float *src = rows[i]->head_scales();
+            std::memcpy(sl->host + ptr_off + 2 * (size_t)i, &src, sizeof(src));
+        }
     }
     hipError_t e;
-    if ((e = hipMemcpyAsync(sl->dev, sl->host, ints * sizeof(int32_t), hipMemcpyHostToDevice, (hipStream_t)stream)) != hipSuccess)
+    if ((e = hipMemcpyAsync(sl->dev, sl->host, (fp8 ? gath_off : base_ints) * sizeof(int32_t), hipMemcpyHostToDevice,
+                            (hipStream_t)stream)) != hipSuccess)
         return hip_err(e, "uploading the block tables");
+    float *gk = (float *)(sl->dev + gath_off), *gv = gk + (size_t)n * hk;
+    if (fp8 && (e = gather_head_scales((const float *const *)(sl->dev + ptr_off), gk, gv, n, hk, (hipStream_t)stream)) != hipSuccess)
+        return hip_err(e, "gathering the head scales");
     int32_t *tables_dev_ = sl->dev;
     const int32_t heads = pool_->num_kv_heads(), dim = pool_->head_dim();
     const size_t need = hs_decode_attn_workspace_bytes(n, hq, heads, dim, (int32_t)max_cap);  // for the rows' capacity: grows rarely
@@ -351,9 +402,12 @@ Status PagedBatch::decode_step(PagedLayerKVCache *const *rows, int32_t n, const 
     }
     hs_kv_layout l = pool_->layout(tables_dev_, tables_dev_ + (size_t)n * stride, (int32_t)stride);
     for (int32_t i = 0; i < n; ++i) l.total_tokens_hint += lens[i];  // lets the kernel library balance a ragged batch
-    int rc = hs_decode_step_int8(q, k_new, v_new, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
-                                 tables_dev_ + 2 * (size_t)n * stride, out, workspace_, workspace_bytes_, n, hq, heads, dim,
-                                 (int32_t)max_len, scale, stream);
+    int rc = fp8 ? hs_decode_step_fp8(q, k_new, v_new, dtype, (uint8_t *)pool_->codes(), (uint8_t *)pool_->codes(), gk, gv, &l,
+                                      tables_dev_ + 2 * (size_t)n * stride, out, workspace_, workspace_bytes_, n, hq, heads, dim,
+                                      (int32_t)max_len, scale, stream)
+                 : hs_decode_step_int8(q, k_new, v_new, dtype, pool_->codes(), pool_->codes(), pool_->scales(), pool_->scales(), &l,
+                                       tables_dev_ + 2 * (size_t)n * stride, out, workspace_, workspace_bytes_, n, hq, heads, dim,
+                                       (int32_t)max_len, scale, stream);
     if (rc != HS_OK) return from_abi(rc);
     if ((e = hipEventRecord(sl->done, (hipStream_t)stream)) != hipSuccess) return hip_err(e, "recording the slot event");
     sl->in_use = true;

@@ -41,7 +41,9 @@ struct CacheOwner {
 
 class BlockPool {
   public:
-    BlockPool(size_t num_blocks, int32_t num_kv_heads, int32_t head_dim);
+    // format: Int8 (codes + per-token scales in every block) or Fp8 (e4m3fn codes only; the per-(sequence, kv-head)
+    // scales belong to the caches, not to the blocks)
+    BlockPool(size_t num_blocks, int32_t num_kv_heads, int32_t head_dim, KVQuantType format = KVQuantType::Int8);
     ~BlockPool();
     BlockPool(const BlockPool &) = delete;
     BlockPool &operator=(const BlockPool &) = delete;
@@ -57,7 +59,9 @@ class BlockPool {
     size_t free_block_count() const;
     size_t total_blocks() const { return total_; }
     size_t used_memory() const;  // bytes of the blocks in use
-    size_t block_bytes() const { return (size_t)heads_ * kBlockSize * ((size_t)dim_ + 4); }
+    size_t block_bytes() const { return (size_t)heads_ * kBlockSize * ((size_t)dim_ + (fp8() ? 0 : 4)); }
+    KVQuantType format() const { return format_; }
+    bool fp8() const { return format_ == KVQuantType::Fp8; }
     int32_t num_kv_heads() const { return heads_; }
     int32_t head_dim() const { return dim_; }
 
@@ -72,6 +76,7 @@ class BlockPool {
     mutable std::mutex mu_;
     size_t total_;
     int32_t heads_, dim_;
+    KVQuantType format_;
     std::vector<BlockId> free_list_;
     std::vector<std::unique_ptr<CacheOwner>> owner_;
     int8_t *codes_ = nullptr;
@@ -105,6 +110,7 @@ class PagedLayerKVCache {
     // Makes sure blocks exist for positions < end_pos (host bookkeeping only; used by the batch step).
     Status reserve(size_t end_pos);
     const CacheOwner &owner() const { return owner_; }
+    const float *head_scales() const { return head_scales_dev_; }
     const std::shared_ptr<BlockPool> &pool() const { return pool_; }
 
     size_t seq_pos = 0;
@@ -117,6 +123,7 @@ class PagedLayerKVCache {
     std::vector<BlockId> key_blocks_, value_blocks_;
     int32_t *table_dev_ = nullptr;  // [2][max_blocks]: row 0 = K blocks, row 1 = V blocks
     int32_t *len_dev_ = nullptr;
+    float *head_scales_dev_ = nullptr;  // fp8 pools: [2][Hkv], K then V, calibrated by the update at start_pos 0
     size_t table_synced_ = 0;       // number of blocks the device table already holds
     void *workspace_ = nullptr;
     size_t workspace_bytes_ = 0;
@@ -139,7 +146,7 @@ class PagedBatch {
     static constexpr int kSlots = 4;
     struct Slot {  // K tables, V tables and lengths of one step: pinned host copy, device copy, "step finished" event
         int32_t *host = nullptr, *dev = nullptr;
-        size_t cap = 0;
+        size_t cap = 0;  // in int32 units; an fp8 step also carries the rows' scale pointers and the gathered scales
         hipEvent_t done = nullptr;
         bool in_use = false;
     };

@@ -12,7 +12,7 @@ struct hs_pool {
     std::shared_ptr<hs::BlockPool> pool;
     hs::PagedBatch batch;
     std::string last_error;
-    hs_pool(size_t n, int32_t h, int32_t d) : pool(std::make_shared<hs::BlockPool>(n, h, d)), batch(pool) {}
+    hs_pool(size_t n, int32_t h, int32_t d, hs::KVQuantType f) : pool(std::make_shared<hs::BlockPool>(n, h, d, f)), batch(pool) {}
     int done(const hs::Status &s) {
         if (!s.ok()) last_error = s.message;
         return s.code;
@@ -41,10 +41,13 @@ hs::CacheOwner owner(int kind, uint64_t id, const char *name) {
 
 extern "C" {
 
-hs_pool *hs_pool_create(int64_t num_blocks, int32_t heads, int32_t dim) {
+hs_pool *hs_pool_create_format(int64_t num_blocks, int32_t heads, int32_t dim, int quant_type) {
     if (num_blocks < 0 || heads <= 0 || (dim != 64 && dim != 128 && dim != 256)) return nullptr;
-    return new (std::nothrow) hs_pool((size_t)num_blocks, heads, dim);
+    if (quant_type != HS_KV_INT8 && quant_type != HS_KV_FP8) return nullptr;
+    return new (std::nothrow) hs_pool((size_t)num_blocks, heads, dim, quant_type == HS_KV_FP8 ? hs::KVQuantType::Fp8 : hs::KVQuantType::Int8);
 }
+hs_pool *hs_pool_create(int64_t num_blocks, int32_t heads, int32_t dim) { return hs_pool_create_format(num_blocks, heads, dim, HS_KV_INT8); }
+int hs_pool_quant_type(const hs_pool *p) { return p ? (int)p->pool->format() : 0; }
 void hs_pool_destroy(hs_pool *p) { delete p; }
 const char *hs_pool_last_error(const hs_pool *p) { return p ? p->last_error.c_str() : "null pool"; }
 

@@ -17,7 +17,7 @@ EXPORTS = [
     "hs_cache_get_view", "hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_clear", "hs_cache_truncate_to",
     "hs_cache_is_initialized", "hs_cache_memory_usage", "hs_cache_quant_type", "hs_cache_decode_attention",
     "hs_cache_decode_step", "hs_cache_prefill", "hs_paged_cache_prefill", "hs_kv_quant_canonical_str",
-    "hs_pool_create", "hs_pool_destroy", "hs_pool_last_error", "hs_pool_allocate", "hs_pool_free", "hs_pool_owner_of",
+    "hs_pool_create", "hs_pool_create_format", "hs_pool_quant_type", "hs_pool_destroy", "hs_pool_last_error", "hs_pool_allocate", "hs_pool_free", "hs_pool_owner_of",
     "hs_pool_used_blocks", "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory",
     "hs_paged_cache_create", "hs_paged_cache_destroy", "hs_paged_cache_last_error", "hs_paged_cache_update",
     "hs_paged_cache_get_dense", "hs_paged_cache_decode_attention", "hs_paged_cache_clear", "hs_paged_cache_truncate_to",
@@ -50,6 +50,8 @@ def lib():
         L.hs_kv_quant_canonical_str.restype = ctypes.c_char_p
         L.hs_pool_create.restype = ctypes.c_void_p
         L.hs_pool_create.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32]
+        L.hs_pool_create_format.restype = ctypes.c_void_p
+        L.hs_pool_create_format.argtypes = [ctypes.c_int64, ctypes.c_int32, ctypes.c_int32, ctypes.c_int]
         L.hs_pool_last_error.restype = ctypes.c_char_p
         L.hs_paged_cache_create.restype = ctypes.c_void_p
         L.hs_paged_cache_create.argtypes = [ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_uint64, ctypes.c_char_p]
@@ -187,8 +189,8 @@ class BlockPoolExhausted(CacheError):
 class BlockPool:
     """BlockPool of the reference (kv_cache.rs:508-676) over int8 blocks; bookkeeping works without a GPU."""
 
-    def __init__(self, num_blocks, num_kv_heads, head_dim):
-        self._h = ctypes.c_void_p(lib().hs_pool_create(num_blocks, num_kv_heads, head_dim))
+    def __init__(self, num_blocks, num_kv_heads, head_dim, quant_type=INT8):
+        self._h = ctypes.c_void_p(lib().hs_pool_create_format(num_blocks, num_kv_heads, head_dim, quant_type))
         if not self._h:
             raise ValueError("bad pool shape")
         self.num_kv_heads, self.head_dim = num_kv_heads, head_dim

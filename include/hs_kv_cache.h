@@ -111,7 +111,12 @@ HS_API int hs_cache_prefill(hs_cache *c, const void *q, const void *new_keys, co
 typedef struct hs_pool hs_pool;
 typedef struct hs_paged_cache hs_paged_cache;
 
-HS_API hs_pool *hs_pool_create(int64_t num_blocks, int32_t num_kv_heads, int32_t head_dim);
+HS_API hs_pool *hs_pool_create(int64_t num_blocks, int32_t num_kv_heads, int32_t head_dim); /* int8 blocks */
+/* The same with the block format chosen: HS_KV_INT8 (codes + per-token scales in every block) or HS_KV_FP8 (e4m3fn
+ * codes only: the per-(sequence, kv-head) scales belong to each paged cache, which calibrates them on the tokens
+ * written at start_pos 0 exactly as the contiguous FP8 cache does).  NULL for any other format. */
+HS_API hs_pool *hs_pool_create_format(int64_t num_blocks, int32_t num_kv_heads, int32_t head_dim, int quant_type);
+HS_API int hs_pool_quant_type(const hs_pool *p);
 HS_API void hs_pool_destroy(hs_pool *p); /* the blocks live until the last cache of the pool is destroyed */
 HS_API const char *hs_pool_last_error(const hs_pool *p);
 HS_API int hs_pool_allocate(hs_pool *p, int owner_kind, uint64_t owner_id, const char *owner_name, int32_t *block_id);
@@ -124,7 +129,7 @@ HS_API int64_t hs_pool_free_block_count(const hs_pool *p);
 HS_API int64_t hs_pool_total_blocks(const hs_pool *p);
 HS_API int64_t hs_pool_used_memory(const hs_pool *p);
 
-/* LayerKVCache::new_paged(max_seq_len, pool, owner), kv_cache.rs:1100-1120: one sequence, int8 format.
+/* LayerKVCache::new_paged(max_seq_len, pool, owner), kv_cache.rs:1100-1120: one sequence, in the pool's format.
  * update takes [1, seq_len, num_kv_heads, head_dim]; blocks are taken in (K, V) pairs and a failed pair is
  * rolled back (kv_cache.rs:1456-1471); clear, truncate_to and destroy return blocks (kv_cache.rs:1679-1750,
  * 1873-1891). */

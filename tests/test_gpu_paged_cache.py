@@ -180,3 +180,96 @@ def test_batch_step_refuses_before_launch_when_the_pool_is_empty():
     out = kc.paged_batch_decode_step(pool, [a], _rand(r, 1, Hq, D), _rand(r, 1, 1, Hkv, D), _rand(r, 1, 1, Hkv, D), 0.1)
     torch.cuda.synchronize()
     assert a.seq_pos == 257 and a.num_blocks == 2 and bool(torch.isfinite(out.float()).all())
+
+
+# ---------------------------------------------------------------------------------------------- FP8 blocks
+def _fp8_reference(k_all, calib_tokens):
+    """Dense view of an FP8 cache: scales calibrated on the first `calib_tokens` tokens, codes of every token."""
+    x = k_all.float().cpu().numpy()
+    sc = oracle.fp8_calibrate(x[:, :calib_tokens])
+    return oracle.dequant_fp8(oracle.quant_fp8(x, sc), sc), sc
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp8_paged_cache_equals_the_contiguous_fp8_cache(D):
+    """The FP8 block format: update (calibration at start_pos 0), get, truncate, chunked prefill and decode through a
+    paged cache give what the contiguous FP8 LayerKVCache gives, and the oracle's codes."""
+    r = wl.philox(930 + D)
+    Hq, Hkv, T = 8, 2, 600
+    pool = kc.BlockPool(16, Hkv, D, kc.FP8)
+    assert kc.lib().hs_pool_quant_type(pool._h) == kc.FP8
+    paged = kc.PagedLayerKVCache(2048, pool, "fp8")
+    flat = kc.LayerKVCache(2048, kc.FP8)
+    k, v = _rand(r, 1, T, Hkv, D) * 0.5, _rand(r, 1, T, Hkv, D) * 0.5
+    for c in (paged, flat):
+        c.update(k[:, :250], v[:, :250], 0)
+        c.update(k[:, 250:], v[:, 250:], 250)
+    assert paged.num_blocks == 3 and pool.used_blocks() == 6
+    gk, gv = paged.get(torch.float32)
+    fk, fv = flat.get(torch.float32)
+    assert bool(torch.equal(gk, fk)) and bool(torch.equal(gv, fv))
+    wk, _ = _fp8_reference(k, 250)
+    wv, _ = _fp8_reference(v, 250)
+    assert np.array_equal(gk.cpu().numpy(), wk) and np.array_equal(gv.cpu().numpy(), wv)
+    q = _rand(r, 1, Hq, D)
+    scale = 1.0 / np.sqrt(D)
+    op, of = paged.decode_attention(q, scale), flat.decode_attention(q, scale)
+    torch.cuda.synchronize()
+    assert np.abs(op.float().cpu().numpy() - of.float().cpu().numpy()).max() < 2e-3
+    want = oracle.decode_attn(q.float().cpu().numpy(), wk, wv, None, None, oracle.FMT_DENSE, np.array([T], np.int32), scale)
+    assert np.abs(op.float().cpu().numpy() - want).max() < 2e-2
+    paged.truncate_to(300)
+    assert paged.num_blocks == 2 and pool.used_blocks() == 4
+    gk, _ = paged.get(torch.float32)
+    assert np.array_equal(gk.cpu().numpy(), wk[:, :300])
+    # chunked prefill on top of what is left: the scales stay those of the first update
+    S = 100
+    qn, kn, vn = _rand(r, 1, S, Hq, D), _rand(r, 1, S, Hkv, D) * 0.5, _rand(r, 1, S, Hkv, D) * 0.5
+    flat.truncate_to(300)
+    o1, o2 = paged.prefill(qn, kn, vn, 300, scale), flat.prefill(qn, kn, vn, 300, scale)
+    torch.cuda.synchronize()
+    assert paged.seq_pos == 400 and np.abs(o1.float().cpu().numpy() - o2.float().cpu().numpy()).max() < 4e-3
+    gk, gv = paged.get(torch.float32)
+    fk, fv = flat.get(torch.float32)
+    assert bool(torch.equal(gk, fk)) and bool(torch.equal(gv, fv))
+
+
+@pytest.mark.parametrize("lens", [[5, 255, 256, 700], [2, 2]])
+def test_fp8_ragged_batch_decode_step_matches_oracle(lens):
+    """One launch over paged FP8 caches with their own per-head scales (gathered on the device for the step)."""
+    r = wl.philox(940 + len(lens))
+    Hq, Hkv, D = 8, 2, 128
+    n = len(lens)
+    pool = kc.BlockPool(64, Hkv, D, kc.FP8)
+    rows, hist = [], []
+    for i, L in enumerate(lens):
+        c = kc.PagedLayerKVCache(2048, pool, i)
+        k, v = _rand(r, 1, L - 1, Hkv, D) * (0.3 + 0.2 * i), _rand(r, 1, L - 1, Hkv, D) * (0.3 + 0.2 * i)
+        c.update(k, v, 0)
+        rows.append(c)
+        hist.append((k, v))
+    q = _rand(r, n, Hq, D)
+    k_new, v_new = _rand(r, n, 1, Hkv, D) * 0.4, _rand(r, n, 1, Hkv, D) * 0.4
+    scale = 1.0 / np.sqrt(D)
+    out = kc.paged_batch_decode_step(pool, rows, q, k_new, v_new, scale)
+    torch.cuda.synchronize()
+    assert [c.seq_pos for c in rows] == lens
+    T = max(lens)
+    kd, vd = np.zeros((n, T, Hkv, D), np.float32), np.zeros((n, T, Hkv, D), np.float32)
+    for i, L in enumerate(lens):
+        kd[i, :L], _ = _fp8_reference(torch.cat([hist[i][0], k_new[i:i + 1]], 1), L - 1)
+        vd[i, :L], _ = _fp8_reference(torch.cat([hist[i][1], v_new[i:i + 1]], 1), L - 1)
+        gk, gv = rows[i].get(torch.float32)
+        assert np.array_equal(gk.cpu().numpy()[0], kd[i, :L]) and np.array_equal(gv.cpu().numpy()[0], vd[i, :L])
+    want = oracle.decode_attn(q.float().cpu().numpy(), kd, vd, None, None, oracle.FMT_DENSE, np.array(lens, np.int32), scale)
+    err = np.abs(out.float().cpu().numpy() - want)
+    assert err.max() < 2e-2 and err.mean() < 2e-3
+
+
+def test_fp8_batch_step_refuses_a_row_without_scales():
+    pool = kc.BlockPool(8, 2, 128, kc.FP8)
+    empty = kc.PagedLayerKVCache(512, pool, 1)
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(kc.CacheError, match="no calibrated scales"):
+        kc.paged_batch_decode_step(pool, [empty], z(1, 8, 128), z(1, 1, 2, 128), z(1, 1, 2, 128), 0.1)
+    assert empty.seq_pos == 0
