@@ -243,7 +243,9 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         return;
     }
     const int t_end = min(L, t_begin + a.chunk_tokens);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // the wavefront index as a scalar: everything derived from it (the steps this wavefront walks, block-table lookups,
+    // base addresses) then stays in scalar registers and scalar loads
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int li = lane & 15, lq = lane >> 4;
     // This workgroup reads the newest token if it owns the end of the sequence: it then writes it first (K by
     // wavefront 0, V by wavefront 1).  With five or more steps the token sits beyond every wavefront's first tile,
@@ -267,12 +269,23 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     const int nsteps = (t_end - t_begin + kStep - 1) / kStep;
     __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64 * NS];
 
+    // Where the step this wavefront loads next lives (sequence or block, slot).  With block tables the lookup is a
+    // dependent (scalar) load in front of every address, so it is issued one stage ahead: load_stage() uses the
+    // location found while the previous stage was loaded and starts the lookup for the one after.
+    int64_t nku = 0, nvu = 0;
+    int nks = 0, nvs = 0;
+    auto locate = [&](int step) {
+        const int t0 = t_begin + step * kStep;
+        if (t0 < t_end) {
+            resolve(a.ka, b, t0, nku, nks);
+            resolve(a.va, b, t0, nvu, nvs);
+        }
+    };
     auto load_stage = [&](Stage<kD> &st, int step) {
         const int t0 = t_begin + step * kStep;
-        int64_t ku, vu;
-        int kslot, vslot;
-        resolve(a.ka, b, t0, ku, kslot);
-        resolve(a.va, b, t0, vu, vslot);
+        const int64_t ku = nku, vu = nvu;
+        const int kslot = nks, vslot = nvs;
+        locate(step + kWavesPerWg);
         const int last = L - 1 - t0;  // last valid row offset inside this step (>= 0)
         const uint8_t *kb = a.kc + ku * a.ka.code_stride_seq + (int64_t)h * a.ka.code_stride_head + (int64_t)kslot * kD;
         const uint8_t *vb = a.vc + vu * a.va.code_stride_seq + (int64_t)h * a.va.code_stride_head + (int64_t)vslot * kD;
@@ -426,6 +439,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     int step = wave;
     const bool early_loads = nsteps >= kWavesPerWg + 1;
     if (writes_new && !early_loads) write_new_token();
+    locate(step);
     if (step < nsteps) load_stage(sa, step);
     if (writes_new && early_loads) write_new_token();
     // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds
