@@ -90,6 +90,7 @@ template <> struct VCodes<1> { typedef uint32_t type; };
 __device__ __forceinline__ uint32_t vword(const u32x2 &x, int i) { return x[i]; }
 __device__ __forceinline__ uint32_t vword(uint32_t x, int) { return x; }
 constexpr int kWavesPerWg = 4;
+constexpr int kMaxBalancedB = 1024;  // most sequences a batch may have for the balanced (token-range) split
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kPScale = 64.0f;  // P is carried as 64*p*s_v in fp16 (keeps small weights normal)
 
@@ -105,6 +106,10 @@ struct DecodeArgs {
     QuantArgs nt;        // the step's new token (nt.src[0] == nullptr: none); position = seq_len - 1
     int32_t direct;      // 1: single chunk, write `out` directly; 0: leave partials in the workspace
     int32_t B, Hq, Hkv, G, chunk_tokens, nchunks, max_seq_len;
+    // balanced mode (ragged batches): the cached tokens of a kv-head over the whole batch, counted in 64-token
+    // granules, are cut into `pieces` equal ranges, one per workgroup; min_granules bounds how small a range may get
+    // (and with it the partial slots a sequence can need: nchunks)
+    int32_t balanced, pieces, min_granules;
     float scale_log2e;
     // optional rotary embedding of q (bf16 tables [rope_len, D/2]); the new token's K is rotated by nt.rope_*
     const uint16_t *rope_sin, *rope_cos;
@@ -225,28 +230,21 @@ __device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t t) {
     return (t & 0x80008000u) | ((t >> 1) & 0x3f803f80u);
 }
 
-template <int kD, bool FP8, bool ROPE>
+template <int kD, bool FP8, bool ROPE, bool BAL>
 __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     constexpr int kStep = Shape<kD>::kStep, NT = Shape<kD>::NT, NJ = Shape<kD>::NJ, NC = Shape<kD>::NC;
     constexpr int VW = Shape<kD>::VW, NBB = Shape<kD>::NBB, CW = Shape<kD>::CW, NS = Shape<kD>::NS;
-    // Workgroups go to the 8 XCDs round-robin by linear id.  Low chunk indices always hold work, high ones only
-    // for long sequences, so the chunk index is rotated by (head + sequence): every XCD then sees every index
-    // equally often instead of two XCDs getting all the first chunks.
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int chunk = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
-    const int L = min(a.seq_lens[b], a.max_seq_len);
-    const int t_begin = chunk * a.chunk_tokens;
+    const int h = blockIdx.y;
     const int G = a.G;
-    if (t_begin >= L) {
-        if (chunk == 0 && a.direct)  // a sequence without cached tokens: its output rows are zero
-            for (int i = threadIdx.x; i < G * kD; i += 256) a.out[((int64_t)b * a.Hq + h * G) * kD + i] = 0;
-        return;
-    }
-    const int t_end = min(L, t_begin + a.chunk_tokens);
     // the wavefront index as a scalar: everything derived from it (the steps this wavefront walks, block-table lookups,
     // base addresses) then stays in scalar registers and scalar loads
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int li = lane & 15, lq = lane >> 4;
+    __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64 * NS];
+    __shared__ float sm_m[kWavesPerWg][16], sm_l[kWavesPerWg][16];
+    __shared__ float sm_o[kWavesPerWg][16][CW + 4];  // one column group of O at a time
+    // One work item: tokens [t_begin, t_end) of sequence b (L cached tokens), partial slot `chunk`.
+    auto run_item = [&](const int b, const int L, const int t_begin, const int t_end, const int chunk) {
     // This workgroup reads the newest token if it owns the end of the sequence: it then writes it first (K by
     // wavefront 0, V by wavefront 1).  With five or more steps the token sits beyond every wavefront's first tile,
     // so those first loads are issued ahead of the write and its barrier instead of behind them.
@@ -267,7 +265,6 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     float m_run = -INFINITY, l_run = 0.0f;
 
     const int nsteps = (t_end - t_begin + kStep - 1) / kStep;
-    __shared__ __attribute__((aligned(16))) float sm_sc[kWavesPerWg][64 * NS];
 
     // Where the step this wavefront loads next lives (sequence or block, slot).  With block tables the lookup is a
     // dependent (scalar) load in front of every address, so it is issued one stage ahead: load_stage() uses the
@@ -513,8 +510,6 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     // ---- merge the four wavefronts through LDS
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
-    __shared__ float sm_m[kWavesPerWg][16], sm_l[kWavesPerWg][16];
-    __shared__ float sm_o[kWavesPerWg][16][CW + 4];  // one column group of O at a time
     if (lq == 0) {
         sm_m[wave][li] = m_run;
         sm_l[wave][li] = l_run;
@@ -570,7 +565,70 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
         ml[0] = Mg;
         ml[1] = l;
     }
+    };  // run_item
+
+    // Fixed chunks, grid (chunks, kv-heads, sequences): one item.  Workgroups go to the 8 XCDs round-robin by linear
+    // id.  Low chunk indices always hold work, high ones only for long sequences, so the chunk index is rotated by
+    // (head + sequence): every XCD then sees every index equally often instead of two XCDs getting all the first chunks.
+    // Balanced, grid (pieces, kv-heads): the sequences of the batch are laid end to end in units of 64-token
+    // granules; workgroup p owns granules [p W, (p+1) W) of that line, W = ceil(total / pieces), so every workgroup
+    // streams the same number of bytes whatever the lengths are.  A range that crosses sequence ends holds several
+    // items; a sequence cut by range ends leaves one partial per range, in slots counted from its first range.
+    if constexpr (!BAL) {
+        const int b = blockIdx.z;
+        const int slot = (int)((blockIdx.x + blockIdx.y + blockIdx.z) % gridDim.x);
+        const int L = min(a.seq_lens[b], a.max_seq_len);
+        const int t_begin = slot * a.chunk_tokens;
+        if (t_begin >= L) {
+            if (slot == 0 && a.direct)  // a sequence without cached tokens: its output rows are zero
+                for (int i = threadIdx.x; i < G * kD; i += 256) a.out[((int64_t)b * a.Hq + h * G) * kD + i] = 0;
+            return;
+        }
+        run_item(b, L, t_begin, min(L, t_begin + a.chunk_tokens), slot);
+    } else {
+        __shared__ int sm_pref[kMaxBalancedB + 1];  // granules before sequence b
+        if (wave == 0) {
+            int running = 0;
+            for (int b0 = 0; b0 < a.B; b0 += 64) {
+                const int bb = b0 + lane;
+                int g = bb < a.B ? (min(max(a.seq_lens[bb], 0), a.max_seq_len) + 63) >> 6 : 0;
+#pragma unroll
+                for (int o = 1; o < 64; o <<= 1) {  // inclusive scan over the lanes
+                    const int up = __shfl_up(g, o, 64);
+                    if (lane >= o) g += up;
+                }
+                if (bb < a.B) sm_pref[bb + 1] = running + g;
+                running += __shfl(g, 63, 64);
+            }
+            if (lane == 0) sm_pref[0] = 0;
+        }
+        __syncthreads();
+        // values read from LDS are the same in every lane; saying so keeps all that follows from them (addresses,
+        // trip counts, block-table lookups) in scalar registers, as in the fixed-chunk instance
+        auto uni = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+        const int total = uni(sm_pref[a.B]);
+        const int W = max((total + a.pieces - 1) / a.pieces, a.min_granules);
+        const int g_lo = blockIdx.x * W, g_hi = min(total, g_lo + W);
+        if (g_lo >= g_hi) return;
+        int lo = 0, hi = a.B - 1;  // first sequence that reaches into the range: smallest b with pref[b + 1] > g_lo
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (uni(sm_pref[mid + 1]) > g_lo) hi = mid; else lo = mid + 1;
+        }
+        bool first = true;
+        for (int b = lo; b < a.B; ++b) {
+            const int pb = uni(sm_pref[b]);
+            if (pb >= g_hi) break;
+            if (uni(sm_pref[b + 1]) == pb) continue;  // an empty sequence: the merge kernel writes its zeros
+            const int L = min(a.seq_lens[b], a.max_seq_len);
+            if (!first) __syncthreads();  // the previous item's merge buffers have been read
+            first = false;
+            run_item(b, L, max(g_lo - pb, 0) * 64, min(L, (g_hi - pb) * 64), (int)blockIdx.x - pb / W);
+        }
+    }
 }
+
+
 
 // Merge the chunk partials of one (sequence, query head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c.
 // 256 threads: D/4 column lanes (four output elements each) x 1024/D chunk lanes, so the partials of a long
@@ -578,13 +636,42 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
 // in LDS.  D is 64, 128 or 256.
 __global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, const float *part_ml,
                                                           const int32_t *seq_lens, uint16_t *out, int Hq, int nchunks,
-                                                          int chunk_tokens, int max_seq_len, int kD) {
+                                                          int chunk_tokens, int max_seq_len, int kD, int B, int pieces,
+                                                          int min_granules) {
     const int hq = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
     const int L = min(seq_lens[b], max_seq_len);
-    const int n = L <= 0 ? 0 : min(nchunks, (L + chunk_tokens - 1) / chunk_tokens);
-    const int64_t row = ((int64_t)b * Hq + hq) * nchunks;
     __shared__ float sm_max[4], sm_l[16];
     __shared__ __attribute__((aligned(16))) float sm_o[1024];
+    __shared__ int sm_cnt[2][4];
+    int n;
+    if (pieces > 0) {
+        // balanced split: recompute where this sequence starts on the granule line and how wide a range is; its
+        // partials sit in slots 0 .. (last range - first range)
+        int before = 0, total = 0;
+        for (int i = tid; i < B; i += 256) {
+            const int g = (min(max(seq_lens[i], 0), max_seq_len) + 63) >> 6;
+            total += g;
+            if (i < b) before += g;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            total += __shfl_xor(total, o, 64);
+            before += __shfl_xor(before, o, 64);
+        }
+        if ((tid & 63) == 0) {
+            sm_cnt[0][tid >> 6] = total;
+            sm_cnt[1][tid >> 6] = before;
+        }
+        __syncthreads();
+        total = sm_cnt[0][0] + sm_cnt[0][1] + sm_cnt[0][2] + sm_cnt[0][3];
+        before = sm_cnt[1][0] + sm_cnt[1][1] + sm_cnt[1][2] + sm_cnt[1][3];
+        const int W = max((total + pieces - 1) / pieces, min_granules);
+        const int g = (max(L, 0) + 63) >> 6;
+        n = g == 0 ? 0 : min(nchunks, (before + g - 1) / W - before / W + 1);
+    } else {
+        n = L <= 0 ? 0 : min(nchunks, (L + chunk_tokens - 1) / chunk_tokens);
+    }
+    const int64_t row = ((int64_t)b * Hq + hq) * nchunks;
     float M = -INFINITY;
     for (int c = tid; c < n; c += 256) M = fmaxf(M, part_ml[(row + c) * 2]);
 #pragma unroll
@@ -620,9 +707,18 @@ int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool ne
 int check_prologue(const hs_qk_prologue *p, int dtype, int D, bool need_q, bool need_k);
 NormSpec norm_spec(const hs_qk_prologue *p, int which);
 
-constexpr int kMaxHintedChunks = 16;  // most chunks a sequence is cut into on the strength of the ragged-batch hint
+// Workgroups of a balanced launch: two resident on each of 256 CUs, one round.  Measured at B=64, lengths U[512, 8192]
+// (us per step): 116 with 512, 139 with 640 and 768, 125 with 1024, 129 with 1536, 136 with 2048 -- a second, partial
+// round costs more than the finer balance gains.
+constexpr int kBalancedWorkgroups = 512;
 
-static int pick_chunk_tokens(int B, int Hkv, int max_seq_len, int64_t total_tokens_hint) {
+struct Split {
+    int chunk_tokens, nchunks;            // fixed-length chunks: grid (nchunks, Hkv, B)
+    int balanced, pieces, min_granules;   // balanced token ranges: grid (pieces, Hkv), nchunks = partial slots per sequence
+};
+
+static Split pick_split(int B, int Hkv, int max_seq_len, int64_t total_tokens_hint) {
+    Split s{};
     // A workgroup costs about 1.5 us of prologue/epilogue, so chunks are as long as the grid allows:
     // with >= 512 (sequence, kv-head) units (two resident workgroups on each of 256 CUs) nothing is
     // split and the step is a single launch; below that, split until about 512 workgroups exist -- one round of
@@ -632,24 +728,35 @@ static int pick_chunk_tokens(int B, int Hkv, int max_seq_len, int64_t total_toke
     // 8 x 8 x 16384: 54.5 at 16, 52.9 at 8; 16 x 8 x 8192: 54.3 at 8, 53.8 at 4; 32 x 8 x 32768: the same at 2, 3 and 4;
     // 64 x 8 x 8192 (unsplit by the rule above): 193 unsplit, 196 in 2, 205 in 8.
     const int64_t units = (int64_t)B * Hkv;
-    int64_t want_chunks = units >= 512 ? 1 : (512 + units - 1) / units;
-    // Ragged batch (the caller says how many tokens the batch holds in total): unsplit, the longest sequence sets
-    // the time of the whole launch while the workgroups of short ones idle.  Cutting at about half the mean length
-    // gives every workgroup a similar share and leaves enough of them to refill the CUs as short ones finish.
-    // Measured at B=64, lengths U[512, 8192]: 145 us unsplit, 151 us cut at the mean, 125 us at mean/2, /3 and /4
-    // (shorter chunks shorten the tail of the launch but pay the ~4 us start-up of a workgroup more often).
-    if (total_tokens_hint > 0 && B > 0) {
-        const int64_t mean = std::max<int64_t>(1, (total_tokens_hint + B - 1) / B);
-        if (mean * 5 < (int64_t)max_seq_len * 4) {
-            const int64_t cut = std::max<int64_t>(512, mean / 2);
-            const int64_t rc = std::min<int64_t>(kMaxHintedChunks, ((int64_t)max_seq_len + cut - 1) / cut);
-            want_chunks = std::max(want_chunks, rc);
-        }
-    }
+    const int64_t want_chunks = units >= 512 ? 1 : (512 + units - 1) / units;
     int64_t ct = ((int64_t)max_seq_len + want_chunks - 1) / want_chunks;
     ct = (ct + 127) / 128 * 128;
     if (ct < 256) ct = 256;
-    return (int)ct;
+    s.chunk_tokens = (int)ct;
+    s.nchunks = (max_seq_len + s.chunk_tokens - 1) / s.chunk_tokens;
+    // Ragged batch (the caller says how many tokens the batch holds in total, and the mean length is under 4/5 of
+    // the longest): with fixed chunks the longest sequence sets the time of the launch while the workgroups of short
+    // ones idle, and cutting finer pays a workgroup's start-up more often.  Instead every workgroup gets the same
+    // number of 64-token granules of the batch laid end to end, whatever sequences they belong to.  A range is at
+    // least 512 tokens and at least 1/16 of the longest sequence, which bounds the partials of one sequence at 17.
+    if (total_tokens_hint > 0 && B > 0 && B <= kMaxBalancedB) {
+        const int64_t mean = std::max<int64_t>(1, (total_tokens_hint + B - 1) / B);
+        if (mean * 5 < (int64_t)max_seq_len * 4) {
+            const int gmax = (max_seq_len + 63) / 64;
+            s.balanced = 1;
+            s.pieces = std::max(1, kBalancedWorkgroups / Hkv);
+            s.min_granules = std::max(8, (gmax + 15) / 16);
+            s.nchunks = (gmax + s.min_granules - 1) / s.min_granules + 1;
+        }
+    }
+    return s;
+}
+
+// most partial slots per sequence any call can use, for sizing a workspace without knowing the hint
+static int max_slots(int B, int Hkv, int max_seq_len) {
+    const int gmax = (max_seq_len + 63) / 64;
+    const int mg = std::max(8, (gmax + 15) / 16);
+    return std::max(pick_split(B, Hkv, max_seq_len, 0).nchunks, (gmax + mg - 1) / mg + 1);
 }
 
 struct NewToken {  // optional quantize-on-write of one token per sequence inside the same call
@@ -687,8 +794,9 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
                         (long long)cap);
     }
     DecodeArgs a;
-    a.chunk_tokens = pick_chunk_tokens(B, Hkv, max_seq_len, l->total_tokens_hint);
-    a.nchunks = (max_seq_len + a.chunk_tokens - 1) / a.chunk_tokens;
+    const Split sp = pick_split(B, Hkv, max_seq_len, l->total_tokens_hint);
+    a.chunk_tokens = sp.chunk_tokens; a.nchunks = sp.nchunks;
+    a.balanced = sp.balanced; a.pieces = sp.pieces; a.min_granules = sp.min_granules;
     if (static_scratch) {
         const size_t need = a.nchunks == 1 ? 0 : (size_t)B * Hq * a.nchunks * ((size_t)D + 2) * sizeof(float);
         if (need > kScratchBytes)
@@ -738,25 +846,29 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.qnorm = nt.qnorm;
     const bool pro = nt.prologue || a.rope_sin != nullptr;
     if (phases & 1) {
-        dim3 grid(a.nchunks, Hkv, B);
-        if (D == 64) {
-            if (fp8) decode_attn_kernel<64, true, false><<<grid, 256, 0, stream>>>(a);
-            else if (pro) decode_attn_kernel<64, false, true><<<grid, 256, 0, stream>>>(a);
-            else decode_attn_kernel<64, false, false><<<grid, 256, 0, stream>>>(a);
-        } else if (D == 128) {
-            if (fp8) decode_attn_kernel<128, true, false><<<grid, 256, 0, stream>>>(a);
-            else if (pro) decode_attn_kernel<128, false, true><<<grid, 256, 0, stream>>>(a);
-            else decode_attn_kernel<128, false, false><<<grid, 256, 0, stream>>>(a);
+        const dim3 grid = a.balanced ? dim3(a.pieces, Hkv, 1) : dim3(a.nchunks, Hkv, B);
+#define HS_DECODE_LAUNCH(DD, BAL)                                                                      \
+    do {                                                                                               \
+        if (fp8) decode_attn_kernel<DD, true, false, BAL><<<grid, 256, 0, stream>>>(a);                \
+        else if (pro) decode_attn_kernel<DD, false, true, BAL><<<grid, 256, 0, stream>>>(a);           \
+        else decode_attn_kernel<DD, false, false, BAL><<<grid, 256, 0, stream>>>(a);                   \
+    } while (0)
+        if (a.balanced) {
+            if (D == 64) HS_DECODE_LAUNCH(64, true);
+            else if (D == 128) HS_DECODE_LAUNCH(128, true);
+            else HS_DECODE_LAUNCH(256, true);
         } else {
-            if (fp8) decode_attn_kernel<256, true, false><<<grid, 256, 0, stream>>>(a);
-            else if (pro) decode_attn_kernel<256, false, true><<<grid, 256, 0, stream>>>(a);
-            else decode_attn_kernel<256, false, false><<<grid, 256, 0, stream>>>(a);
+            if (D == 64) HS_DECODE_LAUNCH(64, false);
+            else if (D == 128) HS_DECODE_LAUNCH(128, false);
+            else HS_DECODE_LAUNCH(256, false);
         }
+#undef HS_DECODE_LAUNCH
         if (int rc = check_launch("decode_attn")) return rc;
     }
     if ((phases & 2) && !a.direct) {
         decode_merge_kernel<<<dim3(Hq, B), 256, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
-                                                               a.nchunks, a.chunk_tokens, max_seq_len, D);
+                                                               a.nchunks, a.chunk_tokens, max_seq_len, D, B,
+                                                               a.balanced ? a.pieces : 0, a.min_granules);
         return check_launch("decode_merge");
     }
     return HS_OK;
@@ -768,18 +880,15 @@ extern "C" {
 
 size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len) {
     if (B <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || max_seq_len <= 0) return 0;
-    // room for the finest split any hint can ask for
-    const int ct = hs::pick_chunk_tokens(B, Hkv, max_seq_len, 0);
-    const size_t nchunks = std::max<size_t>((size_t)((max_seq_len + ct - 1) / ct),
-                                            (size_t)std::min<int64_t>(hs::kMaxHintedChunks, ((int64_t)max_seq_len + 255) / 256));
+    // room for the most partial slots per sequence any hint can lead to
+    const size_t nchunks = (size_t)hs::max_slots(B, Hkv, max_seq_len);
     const size_t n = (size_t)B * Hq * nchunks * ((size_t)D + 2) * sizeof(float);
     return (n + 255) / 256 * 256;
 }
 
 int32_t hs_decode_attn_num_chunks(int32_t B, int32_t Hkv, int32_t max_seq_len, int64_t total_tokens_hint) {
     if (B <= 0 || Hkv <= 0 || max_seq_len <= 0) return 0;
-    const int ct = hs::pick_chunk_tokens(B, Hkv, max_seq_len, total_tokens_hint);
-    return (max_seq_len + ct - 1) / ct;
+    return hs::pick_split(B, Hkv, max_seq_len, total_tokens_hint).nchunks;
 }
 
 int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes, const float *k_scales,

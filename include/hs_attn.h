@@ -77,8 +77,9 @@ typedef struct hs_kv_layout {
     const int32_t *k_block_table; /* device, [B, block_table_stride]; NULL = not paged */
     const int32_t *v_block_table; /* device, may equal k_block_table when K and V pools are separate buffers */
     int64_t total_tokens_hint;  /* decode only, optional: sum of seq_lens over the batch as the host knows it
-                                   (0 = unknown).  A ragged batch is then cut into chunks of about half the mean
-                                   length so that long sequences do not set the time of the launch. */
+                                   (0 = unknown).  A ragged batch is then cut into equal token ranges over all
+                                   sequences (the lengths themselves are read on the device), so that long
+                                   sequences do not set the time of the launch. */
     int32_t prefill_columns_hint; /* prefill only, optional: 0 = the library picks the (query, head) columns a
                                    workgroup owns from the size of the grid; 256 or 128 fixes them (results are the
                                    same within rounding either way; head_dim 256 always uses its one width). */
@@ -195,7 +196,10 @@ HS_API int hs_kv_dequantize(const void *codes, const float *scales, int fmt_fp8,
  * else is HS_ERR_INVALID_ARGUMENT.  workspace: device scratch of at least
  * hs_decode_attn_workspace_bytes(...) bytes, 256-byte aligned, owned by the caller. */
 HS_API size_t hs_decode_attn_workspace_bytes(int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len);
-/* Chunks per sequence the decode entry points will use for this shape and hint (1 = a step is a single launch). */
+/* Partials per sequence the decode entry points will keep for this shape and hint (1 = a step is a single launch
+ * and no workspace is touched).  Without a hint: fixed-length chunks.  With a hint that marks the batch ragged
+ * (mean length under 4/5 of max_seq_len, B <= 1024): the batch is cut into equal token ranges over all sequences and
+ * the value is the most ranges one sequence can span (at most 17). */
 HS_API int32_t hs_decode_attn_num_chunks(int32_t B, int32_t Hkv, int32_t max_seq_len, int64_t total_tokens_hint);
 HS_API int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_t *v_codes,
                         const float *k_scales, const float *v_scales, const hs_kv_layout *layout,

@@ -99,11 +99,11 @@ def test_single_chunk_shape_needs_no_scratch_and_matches():
 
 
 def test_refuses_what_the_scratch_cannot_hold():
-    # B * Hq * chunks * (D + 2) * 4 bytes > 32 MiB: 48 sequences x 64 heads x 16 hinted chunks x 258 x 4 = 50.7 MB
+    # B * Hq * slots * (D + 2) * 4 bytes > 32 MiB: 48 sequences x 64 heads x 17 partial slots x 258 x 4 = 53.9 MB
     B, Hq, Hkv, D, T = 48, 64, 8, 256, 8192
     lay = hb.contiguous_layout(Hkv, T, D)
-    lay.total_tokens_hint = B * 1024  # ragged hint -> the finest split
-    assert hb.decode_num_chunks(B, Hkv, T, lay.total_tokens_hint) == 16
+    lay.total_tokens_hint = B * 1024  # ragged hint -> balanced token ranges, up to 17 partials per sequence
+    assert hb.decode_num_chunks(B, Hkv, T, lay.total_tokens_hint) == 17
     p = ctypes.c_void_p(0x1000)
     rc = hb.lib().hs_decode_attn_int8_static(p, p, p, p, p, ctypes.byref(lay), p, p, B, Hq, Hkv, D, ctypes.c_int32(T),
                                              ctypes.c_float(0.0625), None)
