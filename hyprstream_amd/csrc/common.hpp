@@ -37,6 +37,15 @@ inline KvAddr make_addr(const hs_kv_layout &l, int which_table) {
     return a;
 }
 
+// A read of memory that no kernel writes while this one runs (block tables, lengths), through the constant address
+// space: with a wavefront-uniform address it is a scalar load even in a kernel that also stores to global memory.
+// (An ordinary uniform load there becomes a vector load, whose result waits in line behind every K/V tile load the
+// wavefront has in flight.)
+__device__ __forceinline__ int32_t load_invariant(const int32_t *p, int64_t i) {
+    typedef const int32_t __attribute__((address_space(4))) *cptr;
+    return ((cptr)(uintptr_t)p)[i];
+}
+
 // Resolve (sequence b, token t) -> (storage unit, slot).  Returns false when t is outside
 // what the sequence can hold (unit/slot are then 0/0, a valid but meaningless location).
 __device__ __forceinline__ bool resolve(const KvAddr &a, int b, int t, int64_t &unit, int &slot) {
@@ -46,7 +55,7 @@ __device__ __forceinline__ bool resolve(const KvAddr &a, int b, int t, int64_t &
     if (a.table) {
         int blk = a.cap_shift >= 0 ? t >> a.cap_shift : t / a.capacity_tokens;
         if (blk >= a.block_table_stride) return false;
-        int id = a.table[(int64_t)b * a.block_table_stride + blk];
+        int id = load_invariant(a.table, (int64_t)b * a.block_table_stride + blk);
         if (id < 0) return false;
         unit = id;
         slot = t - blk * a.capacity_tokens;
