@@ -63,7 +63,7 @@ pub fn contiguous_layout(hkv: i32, capacity_tokens: i32, d: i32) -> hs_kv_layout
         v_block_table: std::ptr::null(),
         total_tokens_hint: 0,
         prefill_columns_hint: 0,
-        reserved: 0,
+        prefill_window: 0,
     }
 }
 

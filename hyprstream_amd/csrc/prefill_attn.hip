@@ -62,6 +62,7 @@ struct PrefillArgs {
     const int32_t *hist_lens;  // optional, device [B]: cached tokens per sequence (then hist_len is their upper bound)
     int32_t heavy_first;  // the grid outnumbers the CUs: order the query tiles by decreasing work
     int32_t write_new;    // quantize-on-write of the call's K/V rows by the workgroups that finish early
+    int32_t window;       // sliding window of local layers: a query at position p attends keys in (p - window, p]; 0 = none
     float scale_log2e;
 };
 
@@ -98,7 +99,9 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // of the matrix work is padding.
 // kCols: 16-column blocks per wavefront if not PShape's (1 at head_dim 128: half the columns per workgroup, for grids
 // that would leave most CUs without a workgroup).
-template <int kPD, bool FP8, int kRow = kPD, int kCols = 0>
+// kWin: the instance with a sliding window (the checks it adds to every step cost the plain instance 2 % at 4 x 4096
+// tokens, so they are compiled in only where a window is asked for).
+template <int kPD, bool FP8, int kRow = kPD, int kCols = 0, bool kWin = false>
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
     typedef HistTile<kPD> HistTile;
@@ -141,6 +144,13 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     const int wv_q0 = q0 + 16 * ((kNB * wave) / a.HG);  // first query of this wavefront
     const int wv_qlast = min(S - 1, q0 + 16 * ((kNB * wave + kNB - 1) / a.HG) + 15);
     const bool wv_active = wv_q0 < S;
+    // Sliding window: the query in-call index i sees the keys whose distance to it is below W.  The first visible key
+    // of the workgroup's (wavefront's) first query bounds where the walks start; steps below a wavefront's bound are
+    // skipped by that wavefront, steps that a bound cuts through take the masking path of the softmax.
+    const int W = kWin && a.window > 0 ? a.window : (1 << 30);
+    // in-call index of the first key column nb sees (negative: that many history tokens back)
+    auto qlo = [&](int nb) { return min(qi[nb], S - 1) - W + 1; };
+    const int wg_lo = q0 - W + 1, wv_lo = wv_q0 - W + 1, wv_lo_last = wv_qlast - W + 1;
 
     float4v acc[kNB][VB];
     float m_run[kNB];
@@ -175,6 +185,16 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         }
     };
 
+    // A column that has seen no key yet (everything so far masked) has no reference: its lanes keep sending the
+    // wavefront through the branch that sets one, because the common path would accumulate weights that the first
+    // real reference then scales by exp2(-inf).
+    auto pending = [&]() {
+        int f = INT_MIN;
+#pragma unroll
+        for (int nb = 0; nb < kNB; ++nb)
+            if (m_run[nb] == -INFINITY) f = INT_MAX;
+        return f;
+    };
     const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
     const float qscale = (kRow < kPD && 8 * KG * lq >= kRow) ? 0.0f : a.scale_log2e;  // padding columns of Q are zero
     const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;  // wavefronts w and w+4 share a SIMD
@@ -259,6 +279,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // is shared by twice as many MFMAs as in a 32-key step.
         constexpr int kHStep = 64;
         const int nsteps = (H + kHStep - 1) / kHStep;
+        const int st0 = kWin ? min(max(H + wg_lo, 0) / kHStep, nsteps) : 0;  // first step that holds a key some query of the workgroup sees
         HistTile *htiles = (HistTile *)lds;
         // ---- producers: every wavefront converts one eighth of the step's K tiles and of its V tiles.
         //      K: wavefront w takes 16-key block u4 = w/2 and the d-halves jp = w%2 of every 32-d group: lane
@@ -434,6 +455,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             constexpr bool kScaled = decltype(scaled_tag)::value;
             return [&](int step) {
                 const int lim = H - step * kHStep;  // keys of this step that exist
+                const bool edge = kWin && step * kHStep < H + wv_lo_last;  // the window of some query starts inside or after this step
                 float e[kNB][16];
                 int over = force;
 #pragma unroll
@@ -446,8 +468,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                     for (int i = 0; i < 16; ++i) over = max(over, __float_as_int(e[nb][i]));
                 }
                 const bool slow = __builtin_amdgcn_ballot_w64(over > __float_as_int(kPShift)) != 0;
-                if (slow || lim < kHStep) {
-                    force = INT_MIN;
+                if (slow || lim < kHStep || edge) {
                     float mx[kNB];
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb) {
@@ -458,12 +479,21 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                                 for (int r = 0; r < 4; ++r)
                                     if (4 * lq >= lim - (16 * u4 + r)) e[nb][4 * u4 + r] = -INFINITY;
                         }
+                        if (edge) {
+                            const int first = H + qlo(nb) - step * kHStep - 4 * lq;  // key offsets 16u4 + r below this are out of the window
+#pragma unroll
+                            for (int u4 = 0; u4 < 4; ++u4)
+#pragma unroll
+                                for (int r = 0; r < 4; ++r)
+                                    if (16 * u4 + r < first) e[nb][4 * u4 + r] = -INFINITY;
+                        }
                         float m = e[nb][0];
 #pragma unroll
                         for (int i = 1; i < 16; ++i) m = fmaxf(m, e[nb][i]);
                         mx[nb] = quad_max(m) + sref[nb];  // the column's largest score of this step, log2 units
                     }
                     raise_max(mx);
+                    force = pending();
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb) {
                         const float nref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
@@ -496,22 +526,25 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // conversion at the end of the step instead of the beginning, so that its matrix phases tend to meet
         // the other one's vector phases.
         auto walk = [&](auto softmax) {
-            issue(0);
-            commit(htiles[0], 0);
-            if (nsteps > 1) issue(1);
+            if (st0 >= nsteps) return;  // the window of every query of the workgroup starts after the history
+            issue(st0);
+            commit(htiles[st0 & 1], st0);
+            if (st0 + 1 < nsteps) issue(st0 + 1);
             lds_barrier();
-            for (int st = 0; st < nsteps; ++st) {
+            for (int st = st0; st < nsteps; ++st) {
                 if (!late) {
                     if (st + 1 < nsteps) commit(htiles[(st + 1) & 1], st + 1);
                     if (st + 2 < nsteps) issue(st + 2);
                 }
                 const HistTile &t = htiles[st & 1];
-                scores(t);
-                load_v(t, 0);
-                softmax(st);
-                output(t, 0);
-                load_v(t, 1);
-                output(t, 1);
+                if (!kWin || st * kHStep + kHStep > H + wv_lo) {  // else: no query of this wavefront sees a key of the step
+                    scores(t);
+                    load_v(t, 0);
+                    softmax(st);
+                    output(t, 0);
+                    load_v(t, 1);
+                    output(t, 1);
+                }
                 if (late) {
                     if (st + 1 < nsteps) commit(htiles[(st + 1) & 1], st + 1);
                     if (st + 2 < nsteps) issue(st + 2);
@@ -539,7 +572,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         bf16x8 qop[kNB][KG];
         float sref[kNB];
         float4v sinit[kNB];
-        int force = H > 0 ? INT_MIN : INT_MAX;  // nothing seen yet: the first step sets the reference
+        int force = pending();  // columns that have seen nothing yet: their first step sets the reference
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
             const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + ((8 * KG * lq) & (kRow - 1));
@@ -558,6 +591,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // 64 keys per step, as two 32-key tiles in the layout of the history phase.
         constexpr int kNStep = 64;
         const int nsteps = wg_qlast / kNStep + 1;
+        const int st0 = kWin ? max(wg_lo, 0) / kNStep : 0;  // first step with a key inside the window of the workgroup's first query
         HistTile *ntiles = (HistTile *)lds;
         const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kRow;
         const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kRow;
@@ -612,7 +646,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         bf16x8 pop[kNB][2];
         // Halves of step `step` that hold a key some query of this wavefront may see (0: the step is skipped).
         auto halves = [&](int step) {
-            if (!wv_active || step * kNStep > wv_qlast) return 0;
+            if (!wv_active || step * kNStep > wv_qlast || (kWin && step * kNStep + kNStep <= wv_lo)) return 0;
             return step * kNStep + 32 > wv_qlast ? 1 : 2;
         };
         constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
@@ -657,7 +691,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         auto softmax = [&](int step, int nh) {
             const int t0 = step * kNStep;
-            const bool diag = t0 + kNStep - 1 > wv_q0;  // some (key, query) pair of this step is in the future
+            // some (key, query) pair of this step is in the future, or out of the query's window
+            const bool diag = t0 + kNStep - 1 > wv_q0 || (kWin && t0 < wv_lo_last);
             float e[kNB][16];
             int over = force;
 #pragma unroll
@@ -672,13 +707,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                     for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
                         for (int r = 0; r < 4; ++r)
-                            if (16 * u4 + r > qrel) e[nb][4 * u4 + r] = -INFINITY;
+                            if (16 * u4 + r > qrel || (kWin && 16 * u4 + r < qrel - W + 1)) e[nb][4 * u4 + r] = -INFINITY;
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) over = max(over, __float_as_int(e[nb][i]));
             }
             if (__builtin_amdgcn_ballot_w64(over > __float_as_int(kPShift)) != 0) {
-                force = INT_MIN;
                 float mx[kNB];
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb) {
@@ -688,6 +722,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                     mx[nb] = quad_max(m) + sref[nb];
                 }
                 raise_max(mx);
+                force = pending();
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb) {
                     const float nref = (m_run[nb] == -INFINITY) ? 0.0f : m_run[nb] - kPShift;
@@ -710,11 +745,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                     l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pop[nb][hh], l_run[nb], 0, 0, 0);
                 }
         };
-        issue(0);
-        commit(ntiles[0]);
-        if (nsteps > 1) issue(1);
+        issue(st0);
+        commit(ntiles[st0 & 1]);
+        if (st0 + 1 < nsteps) issue(st0 + 1);
         lds_barrier();
-        for (int st = 0; st < nsteps; ++st) {
+        for (int st = st0; st < nsteps; ++st) {
             if (st + 1 < nsteps) commit(ntiles[(st + 1) & 1]);
             if (st + 2 < nsteps) issue(st + 2);
             const int nh = halves(st);
@@ -863,6 +898,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     if ((hist_len > 0 || quantize_on_write) && (!k_codes || !v_codes || !k_scales || !v_scales))
         return fail(HS_ERR_INVALID_ARGUMENT, "null cache buffer");
     if (hist_len < 0) return fail(HS_ERR_INVALID_ARGUMENT, "negative hist_len");
+    if (layout->prefill_window < 0) return fail(HS_ERR_INVALID_ARGUMENT, "negative prefill_window");
     const int G = Hq > 0 && Hkv > 0 ? Hq / Hkv : 0;
     if (Hq <= 0 || Hq % Hkv != 0)
         return fail(HS_ERR_INVALID_ARGUMENT, "need Hq %% Hkv == 0 (Hq=%d Hkv=%d)", Hq, Hkv);
@@ -884,6 +920,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
     a.hist_lens = hist_lens;
     a.write_new = quantize_on_write ? 1 : 0;
+    a.window = layout->prefill_window;
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
     int q_per_wg = 16 * ((256 / (D == 64 ? 128 : D)) * kPWaves / a.HG);  // head_dim 64 runs in the 128 layout
@@ -901,22 +938,28 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
-    if (D == 64 && narrow) {
-        if (fp8) prefill_attn_kernel<128, true, 64, 1><<<grid, 512, 0, st>>>(a);
-        else prefill_attn_kernel<128, false, 64, 1><<<grid, 512, 0, st>>>(a);
-    } else if (D == 64) {
-        if (fp8) prefill_attn_kernel<128, true, 64><<<grid, 512, 0, st>>>(a);
-        else prefill_attn_kernel<128, false, 64><<<grid, 512, 0, st>>>(a);
-    } else if (D == 128 && narrow) {
-        if (fp8) prefill_attn_kernel<128, true, 128, 1><<<grid, 512, 0, st>>>(a);
-        else prefill_attn_kernel<128, false, 128, 1><<<grid, 512, 0, st>>>(a);
-    } else if (D == 128) {
-        if (fp8) prefill_attn_kernel<128, true><<<grid, 512, 0, st>>>(a);
-        else prefill_attn_kernel<128, false><<<grid, 512, 0, st>>>(a);
-    } else {
-        if (fp8) prefill_attn_kernel<256, true><<<grid, 512, 0, st>>>(a);
-        else prefill_attn_kernel<256, false><<<grid, 512, 0, st>>>(a);
-    }
+#define HS_PREFILL_LAUNCH(WIN)                                                                              \
+    do {                                                                                                    \
+        if (D == 64 && narrow) {                                                                            \
+            if (fp8) prefill_attn_kernel<128, true, 64, 1, WIN><<<grid, 512, 0, st>>>(a);                   \
+            else prefill_attn_kernel<128, false, 64, 1, WIN><<<grid, 512, 0, st>>>(a);                      \
+        } else if (D == 64) {                                                                               \
+            if (fp8) prefill_attn_kernel<128, true, 64, 0, WIN><<<grid, 512, 0, st>>>(a);                   \
+            else prefill_attn_kernel<128, false, 64, 0, WIN><<<grid, 512, 0, st>>>(a);                      \
+        } else if (D == 128 && narrow) {                                                                    \
+            if (fp8) prefill_attn_kernel<128, true, 128, 1, WIN><<<grid, 512, 0, st>>>(a);                  \
+            else prefill_attn_kernel<128, false, 128, 1, WIN><<<grid, 512, 0, st>>>(a);                     \
+        } else if (D == 128) {                                                                              \
+            if (fp8) prefill_attn_kernel<128, true, 128, 0, WIN><<<grid, 512, 0, st>>>(a);                  \
+            else prefill_attn_kernel<128, false, 128, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
+        } else {                                                                                            \
+            if (fp8) prefill_attn_kernel<256, true, 256, 0, WIN><<<grid, 512, 0, st>>>(a);                  \
+            else prefill_attn_kernel<256, false, 256, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
+        }                                                                                                   \
+    } while (0)
+    if (a.window > 0) HS_PREFILL_LAUNCH(true);
+    else HS_PREFILL_LAUNCH(false);
+#undef HS_PREFILL_LAUNCH
     if (int rc = check_launch("prefill_attn")) return rc;
     return HS_OK;
 }

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define HS_ATTN_ABI_VERSION 3
+#define HS_ATTN_ABI_VERSION 4
 
 typedef void *hs_stream_t; /* hipStream_t */
 
@@ -83,7 +83,12 @@ typedef struct hs_kv_layout {
     int32_t prefill_columns_hint; /* prefill only, optional: 0 = the library picks the (query, head) columns a
                                    workgroup owns from the size of the grid; 256 or 128 fixes them (results are the
                                    same within rounding either way; head_dim 256 always uses its one width). */
-    int32_t reserved;           /* set to 0 */
+    int32_t prefill_window;     /* prefill only, optional: sliding window of local-attention layers (Gemma3 / Mistral;
+                                   apply_sliding_window_mask, llama.rs:1086-1091, 1123-1155): a query at absolute
+                                   position p attends the keys in (p - window, p].  0 = no window.  For a prompt on an
+                                   empty cache this is the reference's mask; with history it is the same rule on
+                                   absolute positions (the reference's [q_len, q_len] mask has no meaning there).
+                                   Decode entry points ignore it, as the reference applies no window at q_len == 1. */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */

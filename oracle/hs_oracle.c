@@ -42,6 +42,20 @@
  *  - orc_prefill_attn        the same with S query rows and the causal rule
  *                            "query row i sits at absolute position
  *                            (k_len - q_len) + i" (llama.rs:1074-1084).
+ *  - orc_prefill_attn_window the same with the sliding window of local layers
+ *                            (apply_sliding_window_mask, llama.rs:1086-1091,
+ *                            1123-1155): valid = causal AND i - j < window.  The
+ *                            reference builds that mask as [q_len, q_len] and adds it
+ *                            to the [q_len, k_len] scores, which has a meaning only
+ *                            for a prompt on an empty cache (k_len == q_len; at
+ *                            q_len == 1 the mask is a single zero, i.e. decode is
+ *                            NOT windowed there).  With history the restatement
+ *                            uses absolute positions: query p attends keys in
+ *                            (p - window, p].  Pinned by golden vectors of the
+ *                            libtorch op sequence for the empty-cache case, by
+ *                            window >= length == no window, window 1 == own V row,
+ *                            and by a brute-force restriction of the keys
+ *                            (tests/test_oracle_attention.py).
  *  - orc_deltanet_recurrent  the gated delta rule, one token at a time
  *                            (qwen3_5.rs:725-751), with the L2 normalisation
  *                            x / max(||x||, 1e-3) (qwen3_5.rs:331-335) and the
@@ -268,9 +282,9 @@ static inline double kv_at(const void *codes, const float *scales, int fmt, int 
  * attends keys 0..=that position.  out: [B, S, Hq, D] fp32.
  * A row whose kv_len is 0 (or < S) yields zeros.
  */
-ORC_API void orc_prefill_attn(const float *q, const void *kc, const void *vc, const float *ks, const float *vs,
-                              int fmt, const int32_t *kv_lens, int B, int S, int Hq, int Hkv, int D, int Tcap,
-                              float softmax_scale, float *out) {
+ORC_API void orc_prefill_attn_window(const float *q, const void *kc, const void *vc, const float *ks, const float *vs,
+                                     int fmt, const int32_t *kv_lens, int B, int S, int Hq, int Hkv, int D, int Tcap,
+                                     float softmax_scale, int window, float *out) {
     int G = Hq / Hkv;
     double *p = (double *)malloc(sizeof(double) * (size_t)(Tcap > 0 ? Tcap : 1));
     double *acc = (double *)malloc(sizeof(double) * (size_t)D);
@@ -287,7 +301,9 @@ ORC_API void orc_prefill_attn(const float *q, const void *kc, const void *vc, co
                 int h = hq / G;
                 const float *qr = q + (((int64_t)b * S + i) * Hq + hq) * D;
                 double mx = -INFINITY;
-                for (int t = 0; t <= last; ++t) {
+                /* window > 0: keys at distance >= window from the query's position are masked out */
+                int first = (window > 0 && last - window + 1 > 0) ? last - window + 1 : 0;
+                for (int t = first; t <= last; ++t) {
                     double s = 0.0;
                     for (int d = 0; d < D; ++d) s += (double)qr[d] * kv_at(kc, ks, fmt, Tcap, Hkv, D, b, t, h, d);
                     s *= (double)softmax_scale;
@@ -295,12 +311,12 @@ ORC_API void orc_prefill_attn(const float *q, const void *kc, const void *vc, co
                     if (s > mx) mx = s;
                 }
                 double l = 0.0;
-                for (int t = 0; t <= last; ++t) {
+                for (int t = first; t <= last; ++t) {
                     p[t] = exp(p[t] - mx);
                     l += p[t];
                 }
                 for (int d = 0; d < D; ++d) acc[d] = 0.0;
-                for (int t = 0; t <= last; ++t) {
+                for (int t = first; t <= last; ++t) {
                     double w = p[t];
                     for (int d = 0; d < D; ++d) acc[d] += w * kv_at(vc, vs, fmt, Tcap, Hkv, D, b, t, h, d);
                 }
@@ -309,6 +325,12 @@ ORC_API void orc_prefill_attn(const float *q, const void *kc, const void *vc, co
     }
     free(p);
     free(acc);
+}
+
+ORC_API void orc_prefill_attn(const float *q, const void *kc, const void *vc, const float *ks, const float *vs,
+                              int fmt, const int32_t *kv_lens, int B, int S, int Hq, int Hkv, int D, int Tcap,
+                              float softmax_scale, float *out) {
+    orc_prefill_attn_window(q, kc, vc, ks, vs, fmt, kv_lens, B, S, Hq, Hkv, D, Tcap, softmax_scale, 0, out);
 }
 
 /* Decode = prefill with one query row per sequence. q, out: [B, Hq, D]. */

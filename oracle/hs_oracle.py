@@ -149,10 +149,11 @@ def _kv_args(kc, vc, ks, vs, fmt):
     return kc, vc, ks, vs
 
 
-def prefill_attn(q, kc, vc, ks, vs, fmt, kv_lens, softmax_scale):
+def prefill_attn(q, kc, vc, ks, vs, fmt, kv_lens, softmax_scale, window=0):
     """q [B, S, Hq, D] fp32; cache canonical [B, Tcap, Hkv, D]; kv_lens [B].
 
     Query row i of sequence b sits at absolute position kv_lens[b]-S+i.
+    window > 0: sliding window of local layers, a query at position p attends keys in (p - window, p].
     Returns fp32 [B, S, Hq, D] (double accumulation inside).
     """
     q = _c(q, np.float32)
@@ -163,8 +164,8 @@ def prefill_attn(q, kc, vc, ks, vs, fmt, kv_lens, softmax_scale):
     kv_lens = _c(kv_lens, np.int32)
     assert kv_lens.shape == (B,) and (kv_lens <= Tcap).all()
     out = np.empty(q.shape, np.float32)
-    lib().orc_prefill_attn(_p(q), _p(kc), _p(vc), _p(ks), _p(vs), fmt, _p(kv_lens), B, S, Hq, Hkv, D, Tcap,
-                           ctypes.c_float(softmax_scale), _p(out))
+    lib().orc_prefill_attn_window(_p(q), _p(kc), _p(vc), _p(ks), _p(vs), fmt, _p(kv_lens), B, S, Hq, Hkv, D, Tcap,
+                                  ctypes.c_float(softmax_scale), int(window), _p(out))
     return out
 
 

@@ -40,8 +40,18 @@ def expand_kv_for_gqa(kv, num_heads):
     return kv.unsqueeze(3).expand(B, T, Hkv, rep, D).reshape(B, T, num_heads, D)
 
 
-def compute_attention(q, k, v, attn_mask=None):
-    """q [B,S,Hq,D], k/v [B,T,Hq,D] (already GQA-expanded) -> [B,Hq,S,D] in q.dtype."""
+def sliding_window_mask(seq_len, window, dtype=torch.float32):
+    """apply_sliding_window_mask (llama.rs:1123-1155): additive [seq_len, seq_len] mask, 0 where j <= i and
+    i - j < window, -10000 elsewhere, built as tril(0) * triu(1 - window)."""
+    causal = torch.ones(seq_len, seq_len, dtype=dtype).tril(0)
+    win = torch.ones(seq_len, seq_len, dtype=dtype).triu(1 - window)
+    return (torch.ones(seq_len, seq_len, dtype=dtype) - causal * win) * (-10000.0)
+
+
+def compute_attention(q, k, v, attn_mask=None, sliding_window=None):
+    """q [B,S,Hq,D], k/v [B,T,Hq,D] (already GQA-expanded) -> [B,Hq,S,D] in q.dtype.
+    sliding_window: the local-layer window (llama.rs:1086-1091); like the reference, single-shot and only
+    meaningful for q_len == k_len (the mask is [q_len, q_len]) or q_len == 1 (where it is a single zero)."""
     D = q.shape[-1]
     scale = 1.0 / (float(D) ** 0.5)
     kind = q.dtype
@@ -59,9 +69,11 @@ def compute_attention(q, k, v, attn_mask=None):
         elif q_len > 1:
             m = torch.ones(qc.shape[2], k_len).tril(k_len - q_len + start)
             scores = scores.masked_fill(m.eq(0.0), -10000.0)
+        if sliding_window is not None:
+            scores = scores + sliding_window_mask(q_len, sliding_window, scores.dtype)  # broadcast_add
         return scores.softmax(-1, dtype=torch.float32).matmul(v)
 
-    if attn_mask is not None or q_len <= ATTN_CHUNK:
+    if attn_mask is not None or sliding_window is not None or q_len <= ATTN_CHUNK:
         out = one(q, 0)
     else:
         out = torch.cat([one(q[:, :, s:s + ATTN_CHUNK], s) for s in range(0, q_len, ATTN_CHUNK)], 2)

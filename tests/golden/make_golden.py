@@ -10,6 +10,9 @@ oracle and not with anything from this repository's kernels:
   fp8_quant.npz    per-(sequence, head) scale amax/448, clamp, convert
   attention.npz    the reference's op sequence (transpose/contiguous, fp32 upcast, matmul,
                    scale, mask, softmax, matmul; llama.rs:1023-1119) on small cases
+  attention_window.npz  the same with the sliding-window mask of local layers (tril(0) * triu(1 - window) turned into
+                   an additive -10000 mask and added to the scores; llama.rs:1086-1091, 1123-1155) for prompts on an
+                   empty cache, windows 1, 4, 7, 16 and larger than the prompt
   deltanet.npz     the reference's decode-step op sequence (qwen3_5.rs:725-751) iterated
                    over a few tokens
   rope.npz         the reference's table construction and rotation op sequence (rope.rs:100-122,
@@ -138,6 +141,20 @@ def make_attention():
     np.savez_compressed(os.path.join(HERE, "attention.npz"), **out)
 
 
+def make_attention_window():
+    r = gen(40)
+    out = {}
+    for tag, (B, S, Hq, Hkv, D, W) in {"a": (1, 23, 2, 1, 64, 4), "b": (1, 40, 2, 1, 64, 16), "c": (2, 9, 2, 2, 64, 1),
+                                          "d": (1, 20, 2, 1, 128, 7), "e": (1, 12, 2, 1, 64, 50)}.items():
+        q = torch.from_numpy(r.standard_normal((B, S, Hq, D)).astype(np.float32))
+        k = torch.from_numpy(r.standard_normal((B, S, Hkv, D)).astype(np.float32))
+        v = torch.from_numpy(r.standard_normal((B, S, Hkv, D)).astype(np.float32))
+        o = ref.compute_attention(q, ref.expand_kv_for_gqa(k, Hq), ref.expand_kv_for_gqa(v, Hq), sliding_window=W)
+        out.update({tag + "_q": q.numpy(), tag + "_k": k.numpy(), tag + "_v": v.numpy(), tag + "_window": np.int32(W),
+                    tag + "_out": o.transpose(1, 2).contiguous().numpy()})
+    np.savez_compressed(os.path.join(HERE, "attention_window.npz"), **out)
+
+
 def make_deltanet():
     r = gen(5)
     B, T, nk, nv, dk, dv = 2, 6, 2, 4, 32, 16
@@ -214,6 +231,7 @@ if __name__ == "__main__":
     make_int8()
     make_fp8()
     make_attention()
+    make_attention_window()
     make_deltanet()
     make_qknorm()
     for f in sorted(os.listdir(HERE)):

@@ -72,7 +72,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_abi_version_and_empty_error():
-    assert hb.lib().hs_attn_abi_version() == 3
+    assert hb.lib().hs_attn_abi_version() == 4
 
 
 def test_layout_struct_matches_header_size():

@@ -1,4 +1,6 @@
 """GPU parity: causal prefill attention over [int8 history | bf16 new tokens] against the CPU oracle."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -472,3 +474,101 @@ def test_ragged_history_lengths(D, fp8):
             assert np.array_equal(kc2[b, h:h + S], wk[0]) and np.array_equal(ks2[b, h:h + S], wks[0])
             assert np.array_equal(vc2[b, h:h + S], wv[0]) and np.array_equal(vs2[b, h:h + S], wvs[0])
             assert np.array_equal(kc2[b, :h], kc[b, :h])  # and the history below is untouched
+
+
+# ---------------------------------------------------------------- sliding window (local layers)
+def gpu_prefill_window(cache, q, k, v, hist, window, hist_lens=None, write=True):
+    B, S, Hq, D = q.shape
+    qt, kt, vt = (torch.from_numpy(x).to(DEV).bfloat16().contiguous() for x in (q, k, v))
+    out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hl = None if hist_lens is None else torch.from_numpy(np.asarray(hist_lens, np.int32)).to(DEV)
+    hb.prefill_attn(qt, kt, vt, cache.k_codes, cache.v_codes, cache.k_scales, cache.v_scales, cache.layout, hist, out,
+                    1.0 / np.sqrt(D), write, fp8=cache.fp8, hist_lens=hl, window=window)
+    cache.layout.prefill_window = 0
+    torch.cuda.synchronize()
+    return out.float().cpu().numpy()
+
+
+def test_windowed_prompt_matches_the_reference_golden():
+    """The libtorch op sequence of apply_sliding_window_mask on prompts over an empty cache (llama.rs:1086-1091,
+    1123-1155), fp32 inputs rounded to bf16 for the kernel: same tolerance as every prefill test."""
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "attention_window.npz"))
+    for tag in "abde":  # head_dim 64 and 128
+        q, k, v, W = bf16r(g[tag + "_q"]), bf16r(g[tag + "_k"]), bf16r(g[tag + "_v"]), int(g[tag + "_window"])
+        B, S, Hq, D = q.shape
+        c = DeviceCache(B, k.shape[2], S, D)
+        got = gpu_prefill_window(c, q, k, v, 0, W)
+        want = oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, np.full(B, S, np.int32), 1.0 / np.sqrt(D), window=W)
+        compare(got, want, "window golden " + tag)
+        assert np.abs(got - g[tag + "_out"]).max() < 3e-2  # the golden output comes from unrounded fp32 inputs
+
+
+@pytest.mark.parametrize("D,Hq,Hkv", [(128, 32, 8), (64, 8, 4), (256, 8, 2), (128, 7, 1)])
+@pytest.mark.parametrize("W", [1, 17, 64, 100, 300, 4096])
+def test_windowed_prompt_without_history(D, Hq, Hkv, W):
+    B, S = 2, 333
+    q, k, v = make(900 + D + W, B, S, Hq, Hkv, D)
+    c = DeviceCache(B, Hkv, S, D)
+    got = gpu_prefill_window(c, q, k, v, 0, W)
+    want = oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, np.full(B, S, np.int32), 1.0 / np.sqrt(D), window=W)
+    compare(got, want, "window %d D=%d" % (W, D))
+    if W >= S:
+        assert np.array_equal(got, gpu_prefill(DeviceCache(B, Hkv, S, D), q, k, v, 0))
+    kc, vc, ks, vs = c.canonical(S)  # the cache write does not depend on the window
+    wk, wks = oracle.quant_int8(k)
+    assert np.array_equal(kc, wk) and np.array_equal(ks, wks)
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+@pytest.mark.parametrize("H,S,W", [(700, 130, 64), (700, 130, 200), (700, 130, 701), (1000, 64, 1), (129, 200, 150),
+                                   (2000, 512, 1024), (640, 512, 100)])
+def test_windowed_chunk_over_a_history(fp8, H, S, W):
+    """With cached tokens the window runs over absolute positions: query p attends keys in (p - W, p], of which some,
+    all or none are history.  Steps wholly before a workgroup's window are never loaded."""
+    B, Hq, Hkv, D = 2, 16, 4, 128
+    r = wl.philox(7000 + H + S + W)
+    kh = bf16r(r.standard_normal((B, H, Hkv, D)).astype(np.float32))
+    vh = bf16r(r.standard_normal((B, H, Hkv, D)).astype(np.float32))
+    q, k, v = make(7100 + H + W, B, S, Hq, Hkv, D)
+    c = DeviceCache(B, Hkv, H + S, D, fp8=fp8)
+    kt, vt = torch.from_numpy(kh).to(DEV), torch.from_numpy(vh).to(DEV)
+    if fp8:
+        hb.kv_fp8_calibrate(kt, vt, c.k_scales, c.v_scales)
+    c.write(kt, vt, None, 0)
+    kc, vc, ks, vs = c.canonical(H)
+    deq = oracle.dequant_fp8 if fp8 else oracle.dequant_int8
+    kd, vd = deq(kc, ks), deq(vc, vs)
+    got = gpu_prefill_window(c, q, k, v, H, W)
+    want = oracle.prefill_attn(q, np.concatenate([kd, k], 1), np.concatenate([vd, v], 1), None, None, oracle.FMT_DENSE,
+                               np.full(B, H + S, np.int32), 1.0 / np.sqrt(D), window=W)
+    compare(got, want, "window %d over H=%d S=%d fp8=%s" % (W, H, S, fp8))
+
+
+def test_windowed_ragged_rows():
+    """Rows at different positions (hist_lens): each row's window is cut at its own history length."""
+    B, S, Hq, Hkv, D, W = 3, 96, 8, 2, 128, 80
+    hist = [300, 0, 77]
+    Hmax = max(hist)
+    r = wl.philox(7300)
+    kh = bf16r(r.standard_normal((B, Hmax, Hkv, D)).astype(np.float32))
+    vh = bf16r(r.standard_normal((B, Hmax, Hkv, D)).astype(np.float32))
+    q, k, v = make(7301, B, S, Hq, Hkv, D)
+    c = DeviceCache(B, Hkv, Hmax + S, D)
+    c.write(torch.from_numpy(kh).to(DEV), torch.from_numpy(vh).to(DEV), None, 0)
+    kc, vc, ks, vs = c.canonical(Hmax)
+    kd, vd = oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs)
+    got = gpu_prefill_window(c, q, k, v, Hmax, W, hist_lens=hist, write=False)
+    for b in range(B):
+        h = hist[b]
+        want = oracle.prefill_attn(q[b:b + 1], np.concatenate([kd[b:b + 1, :h], k[b:b + 1]], 1),
+                                   np.concatenate([vd[b:b + 1, :h], v[b:b + 1]], 1), None, None, oracle.FMT_DENSE,
+                                   np.array([h + S], np.int32), 1.0 / np.sqrt(D), window=W)
+        compare(got[b:b + 1], want, "ragged window row %d" % b)
+
+
+def test_negative_window_is_refused():
+    c = DeviceCache(1, 2, 16, 128)
+    q, k, v = make(7400, 1, 4, 4, 2)
+    with pytest.raises(hb.HsError):
+        gpu_prefill_window(c, q, k, v, 0, -1)
+    c.layout.prefill_window = 0

@@ -156,3 +156,46 @@ def test_fp8_decode_vs_live_qwen35_op_sequence():
                                       torch.from_numpy(vc), torch.from_numpy(ks), torch.from_numpy(vs))
     d = np.abs(mine - theirs.float().numpy()[:, 0])
     assert d.max() < TOL_MAX and d.mean() < TOL_MEAN
+
+
+# ---------------------------------------------------------------- sliding window (local layers)
+def test_windowed_prompt_matches_reference_op_sequence_golden():
+    """apply_sliding_window_mask on a prompt over an empty cache (llama.rs:1086-1091, 1123-1155), libtorch ops."""
+    g = np.load(os.path.join(GOLDEN, "attention_window.npz"))
+    for tag in "abcde":
+        q, k, v, W = g[tag + "_q"], g[tag + "_k"], g[tag + "_v"], int(g[tag + "_window"])
+        B, S = q.shape[:2]
+        out = oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, np.full(B, S, np.int32),
+                                  1.0 / np.sqrt(q.shape[-1]), window=W)
+        assert np.abs(out - g[tag + "_out"]).max() < 2e-6, tag
+
+
+def test_window_at_least_the_length_is_no_window_and_window_one_is_the_own_value_row():
+    r = np.random.default_rng(31)
+    B, T, S, Hq, Hkv, D = 2, 29, 11, 4, 2, 64
+    q = r.standard_normal((B, S, Hq, D)).astype(np.float32)
+    k = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    v = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    lens = np.full(B, T, np.int32)
+    plain = oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, lens, 0.125)
+    for W in (T, T + 1, 10 ** 6):
+        assert np.array_equal(oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, lens, 0.125, window=W), plain)
+    one = oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, lens, 0.125, window=1)
+    own = np.repeat(v[:, T - S:], Hq // Hkv, axis=2)  # query i sees only the key at its own position
+    assert np.abs(one - own).max() < 1e-6
+
+
+def test_window_with_history_is_attention_over_the_last_window_keys():
+    """Brute force: for every query, cut the keys to (p - W, p] and run the unwindowed oracle on that slice."""
+    r = np.random.default_rng(32)
+    B, T, S, Hq, Hkv, D, W = 1, 37, 6, 2, 1, 64, 9
+    q = r.standard_normal((B, S, Hq, D)).astype(np.float32)
+    k = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    v = r.standard_normal((B, T, Hkv, D)).astype(np.float32)
+    got = oracle.prefill_attn(q, k, v, None, None, oracle.FMT_DENSE, np.array([T], np.int32), 0.125, window=W)
+    for i in range(S):
+        p = T - S + i
+        lo = max(0, p - W + 1)
+        want = oracle.prefill_attn(q[:, i:i + 1], k[:, lo:p + 1], v[:, lo:p + 1], None, None, oracle.FMT_DENSE,
+                                   np.array([p + 1 - lo], np.int32), 0.125)
+        assert np.abs(got[:, i] - want[:, 0]).max() < 1e-6
