@@ -336,7 +336,8 @@ HS_API int hs_prefill_attn_fp8_ragged(const void *q, const void *k_new, const vo
  * v-head j reads q/k-head j / (nv/nk) (qwen3_5.rs:704-720).  With l2norm != 0, q and k are first
  * replaced by x / max(||x||, 1e-3) (qwen3_5.rs:331-335); q is then multiplied by q_scale.
  * T == 1 is the decode step; T > 1 runs the same recurrence token by token with the state held
- * on chip. */
+ * on chip.  Both entry points are built for dk = dv = 128 (the Qwen3.5 head size); any other size is
+ * HS_ERR_INVALID_ARGUMENT, nothing is padded. */
 HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, const float *g, const float *beta,
                         float *state, float *out,
                         int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
