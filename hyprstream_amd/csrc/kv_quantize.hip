@@ -192,6 +192,119 @@ __global__ __launch_bounds__(256) void qk_prologue_kernel(PrologueArgs a) {
     }
 }
 
+// qk_prologue_kernel for 16-bit tensors with 16-byte-aligned buffers: D/8 lanes own a row, eight consecutive
+// elements each (one 16-byte load, one 16-byte store; 16-byte loads of the weights and of the sin/cos entries), so a
+// wavefront carries 64/(D/8) rows.  The sum of squares is reduced over the lanes of the row; the rotation takes a
+// partner's NORMALISED value from the lane that holds it instead of reading and normalising the partner again.  Per
+// element the operations and their roundings are those of the one-row-per-wavefront kernel: the same bits.
+// DT: the tensor dtype (HS_BF16 or HS_F16) as a compile-time constant, so that the per-operation rounding is one
+// instruction and not a three-way choice.
+template <int LPR, int DT>
+__global__ __launch_bounds__(256) void qk_prologue_rows_kernel(PrologueArgs a) {
+#pragma clang fp contract(off)
+    constexpr int kRowsPerWave = 64 / LPR;
+    const int lane = threadIdx.x & 63, sub = lane % LPR;
+    const int HH = a.H[0] + a.H[1];
+    const int total = a.B * a.S * HH;  // the host sends larger problems to the one-row-per-wavefront kernel
+    // Row -> (token, head) and token -> (sequence, position) with the divisions done once per wavefront on scalars:
+    // a lane's row is at most kRowsPerWave - 1 past the wavefront's first one, so it only steps forward from there.
+    const int wave_row = (blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * kRowsPerWave;
+    const int r_raw = wave_row + lane / LPR;
+    const bool live = r_raw < total;  // lanes of rows past the end still take part in the shuffles
+    const int first = min(wave_row, total - 1);
+    int bs = first / HH, hh = first - bs * HH + (min(r_raw, total - 1) - first);
+    while (hh >= HH) {
+        hh -= HH;
+        ++bs;
+    }
+    const int bs0 = first / HH;
+    int b = bs0 / a.S, s = bs0 - b * a.S + (bs - bs0);
+    while (s >= a.S) {
+        s -= a.S;
+        ++b;
+    }
+    const int which = hh >= a.H[0] ? 1 : 0, h = which ? hh - a.H[0] : hh;
+    const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
+    const int64_t row = (int64_t)bs * a.H[which] + h;
+    const NormSpec &n = a.norm[which];
+    const int d0 = sub * 8;
+    const auto unpack = [&](const uint4 v, float (&f)[8]) {
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint16_t h16 = (uint16_t)((i & 1) ? w[i >> 1] >> 16 : w[i >> 1] & 0xffffu);
+            if (DT == HS_BF16) f[i] = bf16_bits_to_f32(h16);
+            else {
+                _Float16 t;
+                __builtin_memcpy(&t, &h16, 2);
+                f[i] = (float)t;
+            }
+        }
+    };
+    float x[8];
+    unpack(*(const uint4 *)((const uint16_t *)a.x[which] + row * a.D + d0), x);
+    if (n.kind != 0) {
+        double ss = 0.0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += (double)norm_square(x[e], DT, n.kind);
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float rrms = norm_rrms(ss, a.D, DT, n.kind, n.eps);
+        float w[8];
+        if (n.kind == 1) {
+            unpack(*(const uint4 *)((const uint16_t *)n.weight + (int64_t)h * n.head_stride + d0), w);
+        } else {
+            const float4 w0 = *(const float4 *)((const float *)n.weight + (int64_t)h * n.head_stride + d0);
+            const float4 w1 = *(const float4 *)((const float *)n.weight + (int64_t)h * n.head_stride + d0 + 4);
+            w[0] = w0.x; w[1] = w0.y; w[2] = w0.z; w[3] = w0.w;
+            w[4] = w1.x; w[5] = w1.y; w[6] = w1.z; w[7] = w1.w;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] = norm_apply(x[e], w[e], rrms, DT, n.kind);
+    }
+    if (a.sin_t != nullptr) {
+        const int half = a.rd / 2;
+        const bool rotated = d0 < a.rd, upper = d0 >= half;
+        // the partner's eight elements sit half/8 lanes away in the same row
+        const int src_lane = rotated ? (upper ? lane - half / 8 : lane + half / 8) : lane;
+        float other[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) other[e] = __shfl(x[e], src_lane, 64);
+        if (rotated) {
+            const int p = pos < 0 ? 0 : (pos >= a.rope_len ? a.rope_len - 1 : pos);
+            const int j0 = upper ? d0 - half : d0;
+            float sn[8], cs[8];
+            unpack(*(const uint4 *)((const uint16_t *)a.sin_t + (int64_t)p * half + j0), sn);
+            unpack(*(const uint4 *)((const uint16_t *)a.cos_t + (int64_t)p * half + j0), cs);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float own_cos = round_to_dtype(x[e] * cs[e], DT);
+                const float other_sin = round_to_dtype(other[e] * sn[e], DT);
+                x[e] = round_to_dtype(upper ? other_sin + own_cos : own_cos - other_sin, DT);
+            }
+        }
+    }
+    if (!live) return;
+    uint32_t res[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        uint32_t r2[2];
+#pragma unroll
+        for (int hsel = 0; hsel < 2; ++hsel) {
+            const float y = x[2 * i + hsel];
+            if (DT == HS_BF16) r2[hsel] = f32_to_bf16_bits(y);
+            else {
+                const _Float16 t = (_Float16)y;
+                uint16_t h16;
+                __builtin_memcpy(&h16, &t, 2);
+                r2[hsel] = h16;
+            }
+        }
+        res[i] = r2[0] | (r2[1] << 16);
+    }
+    *(uint4 *)((uint16_t *)a.out[which] + row * a.D + d0) = make_uint4(res[0], res[1], res[2], res[3]);
+}
+
 // The same for many rows of a 16-bit tensor: D/8 lanes own a row, eight consecutive elements each (16-byte loads
 // of the lane's elements, of their partners half a row away and of the sin/cos entries; one 16-byte store), so a
 // wavefront carries 64/(D/8) rows.  Per element the operations and their roundings are those of rope_rotate().
@@ -581,6 +694,17 @@ int hs_qk_prologue_apply(const void *q, const void *k, int dtype, const hs_qk_pr
     a.sin_t = prologue->rope_sin; a.cos_t = prologue->rope_cos; a.positions = positions; a.start_pos = start_pos;
     a.rope_len = prologue->rope_len; a.B = B; a.S = S; a.H[0] = hq; a.H[1] = hk; a.D = D; a.dtype = dtype;
     a.rd = prologue->rotary_dim > 0 ? prologue->rotary_dim : D;
+    uintptr_t bits = (uintptr_t)q | (uintptr_t)k | (uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)a.sin_t | (uintptr_t)a.cos_t;
+    if (prologue->norm_kind != HS_QKNORM_NONE) bits |= (uintptr_t)a.norm[0].weight | (uintptr_t)a.norm[1].weight;
+    if (dtype != HS_F32 && (bits & 15) == 0 && rows < (1ll << 30)) {  // 16-bit tensors, 16-byte accesses: several rows per wavefront
+        const int rows_per_wg = 4 * (64 / (D / 8));
+        dim3 g((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
+        const bool bf = dtype == HS_BF16;
+        if (D == 64) bf ? qk_prologue_rows_kernel<8, HS_BF16><<<g, 256, 0, (hipStream_t)stream>>>(a) : qk_prologue_rows_kernel<8, HS_F16><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else if (D == 128) bf ? qk_prologue_rows_kernel<16, HS_BF16><<<g, 256, 0, (hipStream_t)stream>>>(a) : qk_prologue_rows_kernel<16, HS_F16><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else bf ? qk_prologue_rows_kernel<32, HS_BF16><<<g, 256, 0, (hipStream_t)stream>>>(a) : qk_prologue_rows_kernel<32, HS_F16><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        return check_launch("qk_prologue");
+    }
     dim3 grid((unsigned)((rows + 3) / 4));
     if (D == 64) qk_prologue_kernel<1><<<grid, 256, 0, (hipStream_t)stream>>>(a);
     else if (D == 128) qk_prologue_kernel<2><<<grid, 256, 0, (hipStream_t)stream>>>(a);

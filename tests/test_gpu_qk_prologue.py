@@ -58,7 +58,7 @@ def oracle_prologue(x_bits, kind, w, eps, sin, cos, pos, rd):
 
 
 @pytest.mark.parametrize("kind", [hb.QKNORM_NONE, hb.QKNORM_LLAMA, hb.QKNORM_QWEN35])
-@pytest.mark.parametrize("D,rd", [(64, 64), (128, 128), (256, 64), (256, 256), (128, 32)])
+@pytest.mark.parametrize("D,rd", [(64, 64), (128, 128), (256, 64), (256, 256), (128, 32), (128, 96), (256, 160), (64, 16)])
 def test_prologue_apply_bit_exact(kind, D, rd):
     r = wl.philox(1000 + 10 * D + rd + kind)
     B, S, Hq, Hkv, L = 2, 13, 6, 2, 512
@@ -85,6 +85,36 @@ def test_prologue_apply_bit_exact(kind, D, rd):
         hb.qk_prologue_apply(None, k.to(DEV), pro2, None, k2)
         torch.cuda.synchronize()
         assert np.array_equal(_bits(k2).reshape(B * S, Hkv, D), orc.qk_norm_bf16(_bits(k).reshape(B * S, Hkv, D), kind, _w_np(wk, kind), 1e-6))
+
+
+@pytest.mark.parametrize("kind", [hb.QKNORM_NONE, hb.QKNORM_LLAMA, hb.QKNORM_QWEN35])
+@pytest.mark.parametrize("D,rd", [(64, 32), (128, 128), (256, 96)])
+def test_prologue_kernels_for_aligned_and_unaligned_buffers_agree(kind, D, rd):
+    """16-byte-aligned 16-bit tensors take the kernel that packs several rows into a wavefront, anything else the
+    one-row-per-wavefront kernel: the same bits from both (here the same data at an address that is 2 mod 16)."""
+    r = wl.philox(1500 + D + rd + kind)
+    B, S, Hq, Hkv, L = 3, 7, 5, 3, 64
+    sin, cos = _tables(rd, 10000.0, L)
+    q = _bf(r.standard_normal((B, S, Hq, D)) * 2).to(DEV)
+    k = _bf(r.standard_normal((B, S, Hkv, D))).to(DEV)
+    wq = _weights(r, kind, Hq, D, per_head=True).to(DEV) if kind else None
+    wk = _weights(r, kind, Hkv, D, per_head=False).to(DEV) if kind else None
+    pro = hb.qk_prologue(kind, 1e-5, wq, wk, sin.to(DEV), cos.to(DEV), rd)
+
+    def shifted(t):  # the same values in a buffer whose address is 2 bytes past a 16-byte boundary
+        flat = torch.empty(t.numel() + 8, dtype=t.dtype, device=DEV)
+        v = flat[1:1 + t.numel()].view(t.shape)
+        v.copy_(t)
+        assert v.data_ptr() % 16 == 2 and v.is_contiguous()
+        return v
+
+    qa, ka = torch.empty_like(q), torch.empty_like(k)
+    hb.qk_prologue_apply(q, k, pro, qa, ka, None, 3)
+    qu, ku = shifted(torch.zeros_like(q)), shifted(torch.zeros_like(k))
+    hb.qk_prologue_apply(shifted(q), shifted(k), pro, qu, ku, None, 3)
+    torch.cuda.synchronize()
+    assert torch.equal(qa.view(torch.int16), qu.view(torch.int16)) and torch.equal(ka.view(torch.int16), ku.view(torch.int16))
+    assert qa.float().abs().sum() > 0
 
 
 def test_prologue_against_libtorch_op_sequences():
