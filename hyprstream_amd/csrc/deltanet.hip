@@ -5,7 +5,7 @@
 // The [dk, dv] = [128, 128] fp32 state of one (sequence, v-head) is independent per column, so it is cut into
 // column slices and ONE wavefront owns one slice for the whole call.  The two contractions over dk are per-lane
 // partial sums plus a reduction over the lanes that share a column.
-//   T == 1 (decode):  deltanet_decode_kernel, a 32-column slice per wavefront read and written with 16-byte
+//   T == 1 (decode):  deltanet_decode_kernel, a 32-column x 64-row piece per wavefront read and written with 16-byte
 //          non-temporal accesses; a single read and a single write of the state: HBM bound, 2*dk*dv*4 bytes per
 //          (sequence, head).
 //   T  > 1 (prefill): deltanet_prefill_kernel, 8-column slices (16 state registers per lane), eight wavefronts
@@ -197,37 +197,41 @@ __global__ __launch_bounds__(512) void deltanet_prefill_kernel(DeltaArgs a) {
     for (int r = 0; r < 16; ++r) sp[(int64_t)r * kDV] = S[r];
 }
 
-// Decode step (T == 1), tuned for HBM streaming: one wavefront owns 32 columns x 128 rows; lane l holds
-// columns 4*(l%8) .. +3 (one 16-byte access per row) of rows [16*(l/8), +16): every load and store
-// instruction of the wavefront moves eight full 128-byte row segments.
+// Decode step (T == 1), tuned for HBM streaming.  A 256-thread workgroup owns 64 columns of one (sequence, v-head);
+// wavefront w the 32-column slice w % 2 of the row half w / 2: 8 KB of state per wavefront, lane l columns
+// 4*(l%8) .. +3 (one 16-byte access per row) of rows [64*(w/2) + 8*(l/8), +8), so every load and store instruction of
+// the wavefront moves eight full 128-byte row segments.  The two contractions over dk meet between the two row halves
+// through LDS (32 floats each way).  With 16 KB per wavefront (all 128 rows, no exchange) the step took 47.9 us at
+// B = 64 x 32 heads; a plain read-scale-write kernel of the same shape takes 46.2 us with 16 KB per wavefront and
+// 43.1 us with 8 KB (more wavefronts in flight, shorter ones).
 __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
     typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ f4 sm_m[4][8], sm_o[4][8];  // [wavefront][column quad]
     const int lane = threadIdx.x & 63;
-    const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int64_t nw = (int64_t)a.B * a.nv * 4;
-    if (wid >= nw) return;
-    const int slice = (int)(wid & 3);
-    const int j = (int)((wid >> 2) % a.nv);
-    const int b = (int)((wid >> 2) / a.nv);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int sl = wave & 1, rh = wave >> 1;
+    const int chalf = (int)(blockIdx.x & 1);
+    const int j = (int)((blockIdx.x >> 1) % a.nv);
+    const int b = (int)((blockIdx.x >> 1) / a.nv);
     const int hk = j / (a.nv / a.nk);
     const int c4 = lane & 7, rg = lane >> 3;
-    const int col = slice * 32 + 4 * c4;
-    float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + rg * 16) * kDV + col;
-    f4 S[16];
+    const int col = chalf * 64 + sl * 32 + 4 * c4;
+    const int row0 = rh * 64 + rg * 8;
+    float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + row0) * kDV + col;
+    f4 S[8];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) S[r] = __builtin_nontemporal_load((const f4 *)(sp + (int64_t)r * kDV));  // read once
+    for (int r = 0; r < 8; ++r) S[r] = __builtin_nontemporal_load((const f4 *)(sp + (int64_t)r * kDV));  // read once
 
     const int64_t bt = b;  // T == 1
-    const uint16_t *kp = a.k + (bt * a.nk + hk) * kDK + rg * 16;
-    const uint16_t *qp = a.q + (bt * a.nk + hk) * kDK + rg * 16;
-    float kf[16], qf[16];
+    const uint16_t *kfull = a.k + (bt * a.nk + hk) * kDK, *qfull = a.q + (bt * a.nk + hk) * kDK;
+    const u32x4 kw = *(const u32x4 *)(kfull + row0), qw = *(const u32x4 *)(qfull + row0);
+    float kf[8], qf[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const uint32_t kw = ((const uint32_t *)kp)[i], qw = ((const uint32_t *)qp)[i];
-        kf[2 * i] = __uint_as_float(kw << 16);
-        kf[2 * i + 1] = __uint_as_float(kw & 0xffff0000u);
-        qf[2 * i] = __uint_as_float(qw << 16);
-        qf[2 * i + 1] = __uint_as_float(qw & 0xffff0000u);
+    for (int i = 0; i < 4; ++i) {
+        kf[2 * i] = __uint_as_float(kw[i] << 16);
+        kf[2 * i + 1] = __uint_as_float(kw[i] & 0xffff0000u);
+        qf[2 * i] = __uint_as_float(qw[i] << 16);
+        qf[2 * i + 1] = __uint_as_float(qw[i] & 0xffff0000u);
     }
     const uint32_t v01 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col);
     const uint32_t v23 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col + 2);
@@ -241,36 +245,44 @@ __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
         return x;
     };
     float kmul = 1.0f, qmul = a.q_scale;
-    if (a.l2norm) {
-        float sk = 0.0f, sq = 0.0f;
+    if (a.l2norm) {  // the norms run over all 128 elements: lane l takes elements 2l and 2l + 1 of each vector
+        const uint32_t k2 = ((const uint32_t *)kfull)[lane], q2 = ((const uint32_t *)qfull)[lane];
+        const float k0 = __uint_as_float(k2 << 16), k1 = __uint_as_float(k2 & 0xffff0000u);
+        const float q0 = __uint_as_float(q2 << 16), q1 = __uint_as_float(q2 & 0xffff0000u);
+        float sk = k0 * k0 + k1 * k1, sq = q0 * q0 + q1 * q1;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            sk += kf[r] * kf[r];
-            sq += qf[r] * qf[r];
+        for (int o = 1; o < 64; o <<= 1) {
+            sk += __shfl_xor(sk, o, 64);
+            sq += __shfl_xor(sq, o, 64);
         }
-        kmul = 1.0f / fmaxf(sqrtf(rows_sum(sk)), 1e-3f);
-        qmul = a.q_scale / fmaxf(sqrtf(rows_sum(sq)), 1e-3f);
+        kmul = 1.0f / fmaxf(sqrtf(sk), 1e-3f);
+        qmul = a.q_scale / fmaxf(sqrtf(sq), 1e-3f);
     }
     const float decay = expf(g);
     f4 m = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 8; ++r) {
         kf[r] *= kmul;
         m += kf[r] * S[r];
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) m[e] = rows_sum(m[e]) * decay;
+    for (int e = 0; e < 4; ++e) m[e] = rows_sum(m[e]);
+    if (rg == 0) sm_m[wave][c4] = m;
+    __syncthreads();
+    m = (sm_m[sl][c4] + sm_m[sl + 2][c4]) * decay;  // both row halves form the same sum in the same order
     const f4 delta = (v - m) * beta;
     f4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 8; ++r) {
         S[r] = S[r] * decay + kf[r] * delta;
         o += qf[r] * S[r];
         __builtin_nontemporal_store(S[r], (f4 *)(sp + (int64_t)r * kDV));
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = rows_sum(o[e]) * qmul;
-    if (rg == 0) *(f4 *)(a.out + (bt * a.nv + j) * kDV + col) = o;
+    for (int e = 0; e < 4; ++e) o[e] = rows_sum(o[e]);
+    if (rg == 0) sm_o[wave][c4] = o;
+    __syncthreads();
+    if (rh == 0 && rg == 0) *(f4 *)(a.out + (bt * a.nv + j) * kDV + col) = (sm_o[sl][c4] + sm_o[sl + 2][c4]) * qmul;
 }
 
 }  // namespace hs
@@ -290,8 +302,7 @@ extern "C" int hs_deltanet_forward(const void *q, const void *k, const void *v, 
     a.B = B; a.T = T; a.nk = nk; a.nv = nv; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     if (T == 1) {
-        const int64_t waves = (int64_t)B * nv * (kDV / 32);
-        deltanet_decode_kernel<<<(unsigned)((waves + 3) / 4), 256, 0, st>>>(a);
+        deltanet_decode_kernel<<<(unsigned)((int64_t)B * nv * 2), 256, 0, st>>>(a);
     } else {
         deltanet_prefill_kernel<<<(unsigned)((int64_t)B * nv * 2), 512, 0, st>>>(a);
     }
