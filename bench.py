@@ -284,6 +284,8 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
+    ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 128, 256],
+                    help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
@@ -297,6 +299,7 @@ def main():
     import torch
     from hyprstream_amd import bindings as hb
     from hyprstream_amd import workloads as wl
+    hb.PREFILL_COLUMNS = args.prefill_columns
 
     if not torch.cuda.is_available():
         print("no GPU visible: bench.py needs an MI355X", file=sys.stderr)

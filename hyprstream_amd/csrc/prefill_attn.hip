@@ -8,7 +8,8 @@
 // which is softmax(Q K^T * scale + causal mask) V over [history | this call's K/V].
 //
 // Work split (numbers for head_dim 128; head_dim 256 is the same template with half the columns per wavefront
-// and twice the operand blocks per key step, see PShape).  A 512-thread workgroup (8 wavefronts, 2 per SIMD)
+// and twice the operand blocks per key step, head_dim 64 with the same columns and half the operand blocks, see
+// PShape).  A 512-thread workgroup (8 wavefronts, 2 per SIMD)
 // owns 256 (query, head) columns of
 // one kv-head -- with G = Hq/Hkv >= 4: 64 consecutive queries x 4 query heads -- and walks the keys,
 // 64 per step.  Every step's K and V tiles are
@@ -42,10 +43,12 @@ constexpr int kPWaves = 8;
 // D = 256 halves the columns of a wavefront (and of a workgroup: 128 instead of 256) and doubles the operand
 // blocks of a key step.
 template <int D> struct PShape {
-    static constexpr int kNB = 256 / D;  // 16-column blocks per wavefront
-    static constexpr int KG = D / 32;    // K operand blocks per 16-key tile (32 d each)
-    static constexpr int VB = D / 16;    // V^T operand blocks per 32 keys (16 rows of d each)
-    static constexpr int NC = D / 128;   // 128-wide groups of d
+    static constexpr int kNB = D == 256 ? 1 : 2;  // 16-column blocks per wavefront
+    static constexpr int KG = D / 32;             // K operand blocks per 16-key tile (32 d each)
+    static constexpr int VB = D / 16;             // V^T operand blocks per 32 keys (16 rows of d each)
+    static constexpr int DW = D < 128 ? D : 128;  // width of a group of d: what one pass of the producers and of the output loop covers
+    static constexpr int NC = D / DW;             // groups of d
+    static constexpr int VBG = DW / 16;           // V^T operand blocks of a group: block bb holds rows d = VBG * li + bb
 };
 constexpr float kPLog2e = 1.4426950408889634f;
 constexpr float kPShift = 6.0f;  // weights are carried as 2^6 * exp2(s - m_run): keeps small ones out of the fp16 subnormals
@@ -92,18 +95,21 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // wavefront with the vector work of the other behind a second barrier per step, or that software-pipelined
 // scores(s+1) against softmax(s) inside one wavefront, were correct but not faster than this order; steps of
 // 64 keys instead of 32 were (the per-step bookkeeping is shared by twice the MFMAs).
-// kPD: head_dim the products are laid out for; FP8: the history holds e4m3fn codes with head scales instead of int8
-// codes with token scales; kRow: head_dim of the tensors in memory.  kRow = 64 runs in the kPD = 128 layout with
-// the upper half of every Q operand zero: rows are 64 wide in memory, lanes whose d would be >= 64 re-read the
-// row's first columns (finite values that meet zeros of Q, or feed output rows that are never stored), and half
-// of the matrix work is padding.
+// kPD: head_dim (64, 128 or 256; PShape); FP8: the history holds e4m3fn codes with head scales instead of int8 codes
+// with token scales.
 // kCols: 16-column blocks per wavefront if not PShape's (1 at head_dim 128: half the columns per workgroup, for grids
 // that would leave most CUs without a workgroup).
 // kWin: the instance with a sliding window (the checks it adds to every step cost the plain instance 2 % at 4 x 4096
 // tokens, so they are compiled in only where a window is asked for).
-template <int kPD, bool FP8, int kRow = kPD, int kCols = 0, bool kWin = false>
+template <int kPD, bool FP8, int kCols = 0, bool kWin = false>
 __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
+    constexpr int DW = PShape<kPD>::DW, VBG = PShape<kPD>::VBG;
+    constexpr int kRow = kPD;  // elements per row of q, k, v, out and of the cache
+    // head_dim 64: a 16-key K tile is 1 KB, one load instruction of a wavefront, and a step's V rows are half as many
+    // 8-byte pieces -- wavefronts 0-3 convert K (a tile each), wavefronts 4-7 convert V.  Otherwise every wavefront
+    // converts an eighth of both.
+    constexpr bool kSplitRoles = kPD == 64;
     typedef HistTile<kPD> HistTile;
     __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];  // two step buffers
     const int lane = threadIdx.x & 63;
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         return f;
     };
     const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
-    const float qscale = (kRow < kPD && 8 * KG * lq >= kRow) ? 0.0f : a.scale_log2e;  // padding columns of Q are zero
+    const float qscale = a.scale_log2e;
     const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;  // wavefronts w and w+4 share a SIMD
     float vup = 1.0f;  // 2^E of the history's V operands, folded back into the accumulators when the history ends
 
@@ -249,7 +255,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         bool scaled = false;
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + ((8 * KG * lq) & (kRow - 1));
+            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
             float qf[8 * KG], amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < KG; ++i) {
@@ -290,12 +296,16 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         //         bytes of each give the fp16 pairs for d = 8x + bb, stored in block bb at operand lane (x, g).
         //      The per-token scales are applied here, once per workgroup, rather than to every score and weight:
         //      the operands are fp16(code * scale) (relative rounding 2^-11, finer than a bf16 cache would keep).
-        const int vx = lane & 15, vpp = 4 * wave + (lane >> 4);
+        // (head_dim 64: eight d-octets per row, so a wavefront covers eight key pairs and wavefronts 4-7 the 32 of a
+        //  step; d = 8x + bb lives in block bb % 4 at operand lane 2x + bb / 4.  K: wavefront w < 4 takes tile w whole.)
+        const int vx = kSplitRoles ? lane & 7 : lane & 15;
+        const int vpp = kSplitRoles ? 8 * (wave & 3) + (lane >> 3) : 4 * wave + (lane >> 4);
         const int vhh = vpp >> 4, vg = (vpp >> 2) & 3, vpe = vpp & 3;
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
-        const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
-        const int ku4 = wave >> 1, kjp = wave & 1;
-        const int krow = 16 * ku4 + li, kcol = (8 * KG * lq + 16 * kjp) & (kRow - 1), vcol = (8 * vx) & (kRow - 1);
+        const int vdst = ((kSplitRoles ? 2 * vx : vx) + 16 * vg) * 16 + 4 * vpe;
+        const int ku4 = kSplitRoles ? wave & 3 : wave >> 1, kjp = kSplitRoles ? 0 : wave & 1;
+        const bool does_k = !kSplitRoles || wave < 4, does_v = !kSplitRoles || wave >= 4;
+        const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp, vcol = 8 * vx;
         const uint32_t koff = krow * kRow + kcol, voff = vkey * kRow + vcol;
         // head_dim 256: the same lane also takes the d-halves jp + 2 (32 codes further) and the d-octet x + 16
         u32x4 rawk[NC];
@@ -349,14 +359,18 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                rawk[c] = *(const u32x4 *)(kb + ko + 32 * c);
-                rawv[c][0] = *(const u32x2 *)(vb + vo0 + 128 * c);
-                rawv[c][1] = *(const u32x2 *)(vb + vo1 + 128 * c);
+                if (does_k) rawk[c] = *(const u32x4 *)(kb + ko + 32 * c);
+                if (does_v) {
+                    rawv[c][0] = *(const u32x2 *)(vb + vo0 + 128 * c);
+                    rawv[c][1] = *(const u32x2 *)(vb + vo1 + 128 * c);
+                }
             }
             if (!FP8) {
-                rawsk = *(const float *)((const uint8_t *)ksp + sk);
-                rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
-                rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
+                if (does_k) rawsk = *(const float *)((const uint8_t *)ksp + sk);
+                if (does_v) {
+                    rawsv[0] = *(const float *)((const uint8_t *)vsp + sv);
+                    rawsv[1] = *(const float *)((const uint8_t *)vsp + sv1);
+                }
             }
             kb += kHStep * kRow; vb += kHStep * kRow;
             ksp += kHStep; vsp += kHStep;
@@ -378,27 +392,31 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             const half2v sv = {(_Float16)fminf(fv0, smax), (_Float16)fminf(fv1, smax)};
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                uint8_t *kd = t.h[ku4 >> 1].k[KG * (ku4 & 1) + 2 * kjp + 4 * c] + obase;
-                if (FP8) {
-                    *(half8 *)kd = e4m3x8_to_f16_div256(rawk[c][0], rawk[c][1]) * sk;
-                    *(half8 *)(kd + 1024) = e4m3x8_to_f16_div256(rawk[c][2], rawk[c][3]) * sk;
-                } else {
-                    *(half8 *)kd = (int8x8_to_f16_biased(rawk[c][0], rawk[c][1]) - bias) * sk;
-                    *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[c][2], rawk[c][3]) - bias) * sk;
+                if (does_k) {
+                    uint8_t *kd = t.h[ku4 >> 1].k[KG * (ku4 & 1) + 2 * kjp + 4 * c] + obase;
+                    if (FP8) {
+                        *(half8 *)kd = e4m3x8_to_f16_div256(rawk[c][0], rawk[c][1]) * sk;
+                        *(half8 *)(kd + 1024) = e4m3x8_to_f16_div256(rawk[c][2], rawk[c][3]) * sk;
+                    } else {
+                        *(half8 *)kd = (int8x8_to_f16_biased(rawk[c][0], rawk[c][1]) - bias) * sk;
+                        *(half8 *)(kd + 1024) = (int8x8_to_f16_biased(rawk[c][2], rawk[c][3]) - bias) * sk;
+                    }
                 }
+                if (does_v) {
 #pragma unroll
-                for (int bb = 0; bb < 8; ++bb) {
-                    const uint32_t pair = FP8 ? e4m3_pair_to_f16_div256(rawv[c][0][bb >> 2], rawv[c][1][bb >> 2], bb & 3)
-                                              : int8_pair_to_f16(rawv[c][0][bb >> 2], rawv[c][1][bb >> 2], bb & 3);
-                    const half2v hv = __builtin_bit_cast(half2v, pair) * sv;
-                    *(uint32_t *)(t.h[vhh].v[8 * c + bb] + vdst) = __builtin_bit_cast(uint32_t, hv);
+                    for (int bb = 0; bb < 8; ++bb) {
+                        const uint32_t pair = FP8 ? e4m3_pair_to_f16_div256(rawv[c][0][bb >> 2], rawv[c][1][bb >> 2], bb & 3)
+                                                  : int8_pair_to_f16(rawv[c][0][bb >> 2], rawv[c][1][bb >> 2], bb & 3);
+                        const half2v hv = __builtin_bit_cast(half2v, pair) * sv;
+                        *(uint32_t *)(t.h[vhh].v[VBG * c + bb % VBG] + vdst + 16 * (bb / VBG)) = __builtin_bit_cast(uint32_t, hv);
+                    }
                 }
             }
         };
         float4v s[kNB][4];    // scores of the step: key block u4 = 2*half + u
         half8 pop[kNB][2];    // P^T operands per half
         constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
-        half8 kop[KU * KG], vop[8];
+        half8 kop[KU * KG], vop[VBG];
         half8 ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (_Float16)1.0f;
@@ -434,17 +452,17 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // the second group by itself
         auto load_v = [&](const HistTile &t, int hh, int c = 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vop[i] = *(const half8 *)(t.h[hh].v[8 * c + i] + obase);
+            for (int i = 0; i < VBG; ++i) vop[i] = *(const half8 *)(t.h[hh].v[VBG * c + i] + obase);
         };
         auto output = [&](const HistTile &t, int hh) {
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 if (c > 0) load_v(t, hh, c);
 #pragma unroll
-                for (int bb = 0; bb < 8; ++bb)
+                for (int bb = 0; bb < VBG; ++bb)
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb)
-                        acc[nb][8 * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb][hh], acc[nb][8 * c + bb], 0, 0, 0);
+                        acc[nb][VBG * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[bb], pop[nb][hh], acc[nb][VBG * c + bb], 0, 0, 0);
             }
         };
         // softmax(): e = exponent of each weight (score in log2 units minus sref).  The common step only checks,
@@ -575,7 +593,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         int force = pending();  // columns that have seen nothing yet: their first step sets the reference
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + ((8 * KG * lq) & (kRow - 1));
+            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
 #pragma unroll
             for (int j = 0; j < KG; ++j) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * j);
@@ -600,12 +618,16 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // 16-key block u4 = w/2, d-halves jp = w%2 (32 bytes per lane = operand blocks 2jp and 2jp+1); for V a lane
         // takes the d-octet x = lane%16 of two adjacent keys (16 bytes of each) and stores the eight (key, key+1)
         // bf16 pairs of d = 8x + bb into block bb.
-        const int vx = lane & 15, vpp = 4 * wave + (lane >> 4);
+        // (head_dim 64: eight d-octets per row, so a wavefront covers eight key pairs and wavefronts 4-7 the 32 of a
+        //  step; d = 8x + bb lives in block bb % 4 at operand lane 2x + bb / 4.  K: wavefront w < 4 takes tile w whole.)
+        const int vx = kSplitRoles ? lane & 7 : lane & 15;
+        const int vpp = kSplitRoles ? 8 * (wave & 3) + (lane >> 3) : 4 * wave + (lane >> 4);
         const int vhh = vpp >> 4, vg = (vpp >> 2) & 3, vpe = vpp & 3;
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
-        const int vdst = (vx + 16 * vg) * 16 + 4 * vpe;
-        const int ku4 = wave >> 1, kjp = wave & 1;
-        const int krow = 16 * ku4 + li, kcol = (8 * KG * lq + 16 * kjp) & (kRow - 1), vcol = (8 * vx) & (kRow - 1);
+        const int vdst = ((kSplitRoles ? 2 * vx : vx) + 16 * vg) * 16 + 4 * vpe;
+        const int ku4 = kSplitRoles ? wave & 3 : wave >> 1, kjp = kSplitRoles ? 0 : wave & 1;
+        const bool does_k = !kSplitRoles || wave < 4, does_v = !kSplitRoles || wave >= 4;
+        const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp, vcol = 8 * vx;
         const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + vcol;  // elements
         u32x4 rawk[NC][2], rawv[NC][2];  // head_dim 256: also the d-halves jp + 2 (32 elements on) and the d-octet x + 16
 #pragma unroll
@@ -625,21 +647,29 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                rawk[c][0] = *(const u32x4 *)(kp + 32 * c);
-                rawk[c][1] = *(const u32x4 *)(kp + 32 * c + 8);
-                rawv[c][0] = *(const u32x4 *)(vp0 + 128 * c);
-                rawv[c][1] = *(const u32x4 *)(vp1 + 128 * c);
+                if (does_k) {
+                    rawk[c][0] = *(const u32x4 *)(kp + 32 * c);
+                    rawk[c][1] = *(const u32x4 *)(kp + 32 * c + 8);
+                }
+                if (does_v) {
+                    rawv[c][0] = *(const u32x4 *)(vp0 + 128 * c);
+                    rawv[c][1] = *(const u32x4 *)(vp1 + 128 * c);
+                }
             }
         };
         auto commit = [&](HistTile &t) {
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                uint8_t *kd = t.h[ku4 >> 1].k[KG * (ku4 & 1) + 2 * kjp + 4 * c] + obase;
-                *(u32x4 *)kd = rawk[c][0];
-                *(u32x4 *)(kd + 1024) = rawk[c][1];
+                if (does_k) {
+                    uint8_t *kd = t.h[ku4 >> 1].k[KG * (ku4 & 1) + 2 * kjp + 4 * c] + obase;
+                    *(u32x4 *)kd = rawk[c][0];
+                    *(u32x4 *)(kd + 1024) = rawk[c][1];
+                }
+                if (does_v) {
 #pragma unroll
-                for (int bb = 0; bb < 8; ++bb)
-                    *(uint32_t *)(t.h[vhh].v[8 * c + bb] + vdst) = pick_halves(rawv[c][0][bb >> 1], rawv[c][1][bb >> 1], bb & 1);
+                    for (int bb = 0; bb < 8; ++bb)
+                        *(uint32_t *)(t.h[vhh].v[VBG * c + bb % VBG] + vdst + 16 * (bb / VBG)) = pick_halves(rawv[c][0][bb >> 1], rawv[c][1][bb >> 1], bb & 1);
+                }
             }
         };
         float4v s[kNB][4];
@@ -650,7 +680,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             return step * kNStep + 32 > wv_qlast ? 1 : 2;
         };
         constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
-        bf16x8 kop[KU * KG], vop[8], ones;
+        bf16x8 kop[KU * KG], vop[VBG], ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
         auto scores = [&](const HistTile &t, int nh) {
@@ -676,17 +706,17 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         auto load_v = [&](const HistTile &t, int hh, int c = 0) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[8 * c + i] + obase);
+            for (int i = 0; i < VBG; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[VBG * c + i] + obase);
         };
         auto output = [&](const HistTile &t, int hh) {
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 if (c > 0) load_v(t, hh, c);
 #pragma unroll
-                for (int bb = 0; bb < 8; ++bb)
+                for (int bb = 0; bb < VBG; ++bb)
 #pragma unroll
                     for (int nb = 0; nb < kNB; ++nb)
-                        acc[nb][8 * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb][hh], acc[nb][8 * c + bb], 0, 0, 0);
+                        acc[nb][VBG * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb][hh], acc[nb][VBG * c + bb], 0, 0, 0);
             }
         };
         auto softmax = [&](int step, int nh) {
@@ -773,17 +803,17 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     for (int nb = 0; nb < kNB; ++nb) {
         const float l = l_run[nb][0];
         if (qi[nb] >= S || hg * a.HG + (kNB * wave + nb) % a.HG >= a.G) continue;  // padding columns write nothing
-        if (kRow < kPD && 32 * lq >= kRow) continue;                                  // nor do padding rows of d
         const float inv = 1.0f / l;
-        uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kRow + 32 * lq;
+        uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kRow + 4 * VBG * lq;
 #pragma unroll
         for (int c = 0; c < NC; ++c)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {  // acc[8c + bb][r] is d = 128 c + 32 lq + 8 r + bb
-                u32x4 w;
+            for (int r = 0; r < 4; ++r) {  // acc[VBG c + bb][r] is d = DW c + 4 VBG lq + VBG r + bb
+                uint32_t w[VBG / 2];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(acc[nb][8 * c + 2 * e][r] * inv, acc[nb][8 * c + 2 * e + 1][r] * inv);
-                *(u32x4 *)(op + 128 * c + 8 * r) = w;
+                for (int e = 0; e < VBG / 2; ++e) w[e] = pack_bf16x2(acc[nb][VBG * c + 2 * e][r] * inv, acc[nb][VBG * c + 2 * e + 1][r] * inv);
+                if constexpr (VBG == 8) *(u32x4 *)(op + DW * c + VBG * r) = (u32x4){w[0], w[1], w[2], w[3]};
+                else *(u32x2 *)(op + DW * c + VBG * r) = (u32x2){w[0], w[1]};
             }
     }
 
@@ -923,7 +953,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.window = layout->prefill_window;
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
-    int q_per_wg = 16 * ((256 / (D == 64 ? 128 : D)) * kPWaves / a.HG);  // head_dim 64 runs in the 128 layout
+    int q_per_wg = 16 * ((D == 256 ? 1 : 2) * kPWaves / a.HG);  // PShape<D>::kNB column blocks per wavefront
     dim3 grid((S + q_per_wg - 1) / q_per_wg, Hkv * ((G + a.HG - 1) / a.HG), B);
     // A small problem (one short sequence, a chunk of a single prompt) would occupy a fraction of the CUs with 256
     // columns per workgroup: with half the columns there are twice the workgroups, each with half the matrix work
@@ -941,20 +971,20 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
 #define HS_PREFILL_LAUNCH(WIN)                                                                              \
     do {                                                                                                    \
         if (D == 64 && narrow) {                                                                            \
-            if (fp8) prefill_attn_kernel<128, true, 64, 1, WIN><<<grid, 512, 0, st>>>(a);                   \
-            else prefill_attn_kernel<128, false, 64, 1, WIN><<<grid, 512, 0, st>>>(a);                      \
+            if (fp8) prefill_attn_kernel<64, true, 1, WIN><<<grid, 512, 0, st>>>(a);                    \
+            else prefill_attn_kernel<64, false, 1, WIN><<<grid, 512, 0, st>>>(a);                       \
         } else if (D == 64) {                                                                               \
-            if (fp8) prefill_attn_kernel<128, true, 64, 0, WIN><<<grid, 512, 0, st>>>(a);                   \
-            else prefill_attn_kernel<128, false, 64, 0, WIN><<<grid, 512, 0, st>>>(a);                      \
+            if (fp8) prefill_attn_kernel<64, true, 0, WIN><<<grid, 512, 0, st>>>(a);                    \
+            else prefill_attn_kernel<64, false, 0, WIN><<<grid, 512, 0, st>>>(a);                       \
         } else if (D == 128 && narrow) {                                                                    \
-            if (fp8) prefill_attn_kernel<128, true, 128, 1, WIN><<<grid, 512, 0, st>>>(a);                  \
-            else prefill_attn_kernel<128, false, 128, 1, WIN><<<grid, 512, 0, st>>>(a);                     \
+            if (fp8) prefill_attn_kernel<128, true, 1, WIN><<<grid, 512, 0, st>>>(a);                  \
+            else prefill_attn_kernel<128, false, 1, WIN><<<grid, 512, 0, st>>>(a);                     \
         } else if (D == 128) {                                                                              \
-            if (fp8) prefill_attn_kernel<128, true, 128, 0, WIN><<<grid, 512, 0, st>>>(a);                  \
-            else prefill_attn_kernel<128, false, 128, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
+            if (fp8) prefill_attn_kernel<128, true, 0, WIN><<<grid, 512, 0, st>>>(a);                  \
+            else prefill_attn_kernel<128, false, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
         } else {                                                                                            \
-            if (fp8) prefill_attn_kernel<256, true, 256, 0, WIN><<<grid, 512, 0, st>>>(a);                  \
-            else prefill_attn_kernel<256, false, 256, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
+            if (fp8) prefill_attn_kernel<256, true, 0, WIN><<<grid, 512, 0, st>>>(a);                  \
+            else prefill_attn_kernel<256, false, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
         }                                                                                                   \
     } while (0)
     if (a.window > 0) HS_PREFILL_LAUNCH(true);

@@ -291,7 +291,7 @@ HS_API int hs_decode_attn_phases(int fmt_fp8, int phases, const void *q, const v
  * hist_len tokens per sequence are already in the int8 cache; query row i attends the whole
  * history (dequantized) and new tokens 0..=i (exact bf16).  With quantize_on_write != 0 the S
  * new tokens are also written to the cache at positions hist_len .. hist_len+S-1.
- * D is 64, 128 or 256 (64 runs in the layout of 128 with half of the matrix work as padding); Hq a multiple of Hkv (groups of 1, 2 or 4k query heads fill the workgroups, any
+ * D is 64, 128 or 256; Hq a multiple of Hkv (groups of 1, 2 or 4k query heads fill the workgroups, any
  * other group size pads its last group of four).  A paged layout needs capacity_tokens (tokens per block)
  * to be a multiple of 64 here.
  * Magnitudes: the cached history enters the matrix products as fp16(code * scale * 2^-E), E a power-of-two reference
