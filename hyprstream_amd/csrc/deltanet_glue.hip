@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void deltanet_conv8_kernel(PrepArgs a) {
         const int t = t0 - 3 + i;
         fr[i] = (u32x4){0u, 0u, 0u, 0u};
         if (t >= 0) {
-            if (i < nt + 3) fr[i] = *(const u32x4 *)(a.x + ((int64_t)b * a.S + t) * a.C + c);
+            if (i < nt + 3) fr[i] = __builtin_nontemporal_load((const u32x4 *)(a.x + ((int64_t)b * a.S + t) * a.C + c));
         } else if (a.state_in) {  // carried state [B, C, 3]: frame -3 + j of channel c + e is element 3*e + j
             const uint16_t *sp = a.state_in + ((int64_t)b * a.C + c) * 3 + (3 + t);
             uint32_t h[8];
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void deltanet_conv8_kernel(PrepArgs a) {
             const bf16x2 p = {(__bf16)y[2 * e], (__bf16)y[2 * e + 1]};
             o[e] = __builtin_bit_cast(uint32_t, p);
         }
-        *(u32x4 *)(dst + ((int64_t)b * a.S + t0 + i) * stride + off) = (u32x4){o[0], o[1], o[2], o[3]};
+        __builtin_nontemporal_store((u32x4){o[0], o[1], o[2], o[3]}, (u32x4 *)(dst + ((int64_t)b * a.S + t0 + i) * stride + off));
     }
     if (t0 + nt == a.S) {  // this thread saw the end of the sequence: the last three frames are the new state
         uint16_t *so = a.state_out + ((int64_t)b * a.C + c) * 3;
@@ -189,12 +189,14 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_rows_kernel(const float *x,
     const bool live = row < rows;  // lanes past the end still take part in the shuffles
     if (!live) row = rows - 1;
     const int64_t e0 = row * D + sub * 8;
-    const float4 xa = *(const float4 *)(x + e0), xb = *(const float4 *)(x + e0 + 4);
-    const uint4 zz = *(const uint4 *)(z + e0);
+    typedef float f4v __attribute__((ext_vector_type(4)));
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    const f4v xa = __builtin_nontemporal_load((const f4v *)(x + e0)), xb = __builtin_nontemporal_load((const f4v *)(x + e0 + 4));
+    const u32x4 zz = __builtin_nontemporal_load((const u32x4 *)(z + e0));
     const float4 wa = *(const float4 *)(w + sub * 8), wb = *(const float4 *)(w + sub * 8 + 4);
     const float xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
     const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
-    const uint32_t zw[4] = {zz.x, zz.y, zz.z, zz.w};
+    const uint32_t zw[4] = {zz[0], zz[1], zz[2], zz[3]};
     float ss = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) ss += xv[e] * xv[e];
@@ -210,7 +212,7 @@ __global__ __launch_bounds__(256) void gated_rmsnorm_rows_kernel(const float *x,
                           (__bf16)(xv[2 * i + 1] * rrms * wv[2 * i + 1] * silu_fast(z1))};
         o4[i] = __builtin_bit_cast(uint32_t, p);
     }
-    if (live) *(uint4 *)(out + e0) = make_uint4(o4[0], o4[1], o4[2], o4[3]);
+    if (live) __builtin_nontemporal_store((u32x4){o4[0], o4[1], o4[2], o4[3]}, (u32x4 *)(out + e0));
 }
 
 }  // namespace hs
