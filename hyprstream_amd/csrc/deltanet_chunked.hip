@@ -236,7 +236,7 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
             // masked q k^T: row = key j, col = query i, kept for j <= i
             m[r] = (_Float16)(row <= col ? qk[x][r] * __builtin_amdgcn_exp2f((gcol - Gs[row]) * kLog2eC) : 0.0f);
         }
-        __builtin_nontemporal_store(m, (half4v *)(wsu + kOffQK + ((nt * 2 + (mt >> 1)) * 64 + lane) * 16 + 8 * (mt & 1)));
+        *(half4v *)(wsu + kOffQK + ((nt * 2 + (mt >> 1)) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
     }
     // q as the A operand of q S: block (token tile, dk slab), lane (token li, group lq); the scan applies e^G
     if (first_of_head) {
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
                 o[e] = lo[e];
                 o[4 + e] = hi[e];
             }
-            __builtin_nontemporal_store(o, (half8 *)(wsh + kOffQh + (blk * 64 + ln) * 16));
+            *(half8 *)(wsh + kOffQh + (blk * 64 + ln) * 16) = o;
         }
     }
     if (tid < 64) {
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
                 o[e] = lo[e];
                 o[4 + e] = hi[e];
             }
-            __builtin_nontemporal_store(o, (half8 *)(wsh + kOffKt + (blk * 64 + ln) * 16));
+            *(half8 *)(wsh + kOffKt + (blk * 64 + ln) * 16) = o;
         }
     }
     __syncthreads();  // the transposed k tile has been read for the output above: its rows may be reused below
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
                 const half4v na = f4h(*(const float4v *)&Nm[(16 * ra + li) * kPitchF + 16 * ra + 4 * lq]);
                 const float4v xa = __builtin_amdgcn_mfma_f32_16x16x16f16(na, f4h(acc), (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 xh[x][ra] = f4h(xa);
-                if (!is_w) __builtin_nontemporal_store(xh[x][ra], (half4v *)(wsu + kOffU + ((ra * 8 + tile0 + x) * 64 + lane) * 8));
+                if (!is_w) *(half4v *)(wsu + kOffU + ((ra * 8 + tile0 + x) * 64 + lane) * 8) = xh[x][ra];
             }
         }
         if (is_w) {
@@ -366,7 +366,7 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
             __builtin_amdgcn_wave_barrier();  // LDS operations of one wavefront complete in order
 #pragma unroll
             for (int ra = 0; ra < 4; ++ra)
-                __builtin_nontemporal_store(*(const u32x4 *)(stg + (ra * 64 + lane) * 16), (u32x4 *)(wsu + kOffWn + ((ra * 4 + (wave & 3)) * 64 + lane) * 16));
+                *(u32x4 *)(wsu + kOffWn + ((ra * 4 + (wave & 3)) * 64 + lane) * 16) = *(const u32x4 *)(stg + (ra * 64 + lane) * 16);
         }
     }
 }
@@ -414,7 +414,8 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
 
     if (wave >= 8) {  // ---- the two loader wavefronts
         // (Plain loads: these operands are shared with the other column half through L2, and the non-temporal hint
-        // that helps U and every store of this file cost 3 % here.)
+        // that helps the U loads and the output stores (scan 165 -> 152 us) cost 3 % here.  The prepare kernel's
+        // workspace stores are plain too: with the hint it took the same time and wrote 5 % more.)
         // Region A of `ops` (-W, q and the decay vectors: 32.5 KB) is read between the two barriers of a chunk, region
         // B (k^T and the masked q k^T: 24 KB) after the second one.  So A of the next chunk is written after the second barrier, B of a chunk
         // after its first barrier -- neither write holds anybody up -- and each is fetched a whole chunk earlier.
