@@ -82,22 +82,27 @@ __device__ __forceinline__ half8 f32x8_to_half8(const float4v &a, const float4v 
 // ------------------------------------------------------------------------------------------------ prepare
 constexpr int kPitchH = 136;  // halves per row of the row-major k / q tiles
 constexpr int kPitchT = 72;   // halves per row of the transposed k / v tiles
-constexpr int kPitchF = 68;   // floats per row of the 64x64 fp32 matrices
-// 71 KB, two workgroups per CU.  The transposed tiles are written after the inverse, over what is dead by then
-// (the row-major tiles, their scratch aliases and L).
-constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsL = 34816, kLdsN = 52224, kLdsF = 69632, kLdsBytes = 71168;
-constexpr int kLdsKT = 0, kLdsVT = 18432;  // 2 x 18432 <= 52224
+constexpr int kPitchL = 68;   // halves per row of the 64x64 matrix L (fp16: it is only ever an MFMA operand)
+constexpr int kPitchD = 20;   // floats per row of a 16x16 fp32 block (diagonal blocks of L / of the inverse, and their scratch)
+constexpr int kBlockD = 16 * kPitchD;
+// 51 KB, three workgroups per CU.  Region A holds the row-major k / q tiles, then the scratch blocks of the four
+// inverses, then the transposed tiles; L (below its diagonal blocks) and the diagonal blocks live beside it.
+constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsKT = 0, kLdsVT = 18432;                   // region A: 36,864 B
+constexpr int kLdsS = 0;                                                                // scratch blocks, 3 per wavefront 0-3
+constexpr int kLdsL = 36864, kLdsD = kLdsL + 64 * kPitchL * 2, kLdsF = kLdsD + 4 * kBlockD * 4, kLdsBytes = kLdsF + 1536;
+static_assert(kLdsBytes <= 54528, "three workgroups of the prepare kernel per CU");
 
 // Transposed tiles [feature d][token]: the eight-token (16-byte) pieces of a row are permuted by d / 16, so that the
 // threads of a wavefront, which write one token each for features 16 apart, hit different banks.
 __device__ __forceinline__ int tpos(int d, int tok) { return d * kPitchT + ((((tok >> 3) ^ (d >> 4)) & 7) << 3) + (tok & 7); }
 
-__global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
+__global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
     _Float16 *kh = (_Float16 *)(lds + kLdsKh), *qh = (_Float16 *)(lds + kLdsQh);
     _Float16 *KT = (_Float16 *)(lds + kLdsKT), *VT = (_Float16 *)(lds + kLdsVT);
-    float *Lm = (float *)(lds + kLdsL), *Nm = (float *)(lds + kLdsN);
-    float *P0 = (float *)(lds + kLdsKh), *P1 = (float *)(lds + kLdsQh);  // scratch once k / q row tiles are dead
+    _Float16 *Lh = (_Float16 *)(lds + kLdsL);  // L, strictly below its diagonal blocks
+    float *Dm = (float *)(lds + kLdsD);        // the four diagonal blocks of L, later of N = (I - L)^-1
+    float *Sm = (float *)(lds + kLdsS);        // scratch blocks of the inverses, once the k / q row tiles are dead
     float *gs = (float *)(lds + kLdsF), *bs = gs + 64, *Gs = gs + 128, *eG = gs + 192, *eGl = gs + 256, *be = gs + 320;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -231,8 +236,10 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = 16 * mt + 4 * lq + r;
-            // L[i = row][j = col]
-            Lm[row * kPitchF + col] = col < row ? -bs[row] * kk[x][r] * __builtin_amdgcn_exp2f((Gs[row] - gcol) * kLog2eC) : 0.0f;
+            // L[i = row][j = col]: the diagonal blocks in fp32 for the inverse, the rest as the fp16 operand it will be
+            const float lv = col < row ? -bs[row] * kk[x][r] * __builtin_amdgcn_exp2f((Gs[row] - gcol) * kLog2eC) : 0.0f;
+            if (nt == mt) Dm[mt * kBlockD + (4 * lq + r) * kPitchD + li] = lv;
+            else Lh[row * kPitchL + col] = (_Float16)lv;
             // masked q k^T: row = key j, col = query i, kept for j <= i
             m[r] = (_Float16)(row <= col ? qk[x][r] * __builtin_amdgcn_exp2f((gcol - Gs[row]) * kLog2eC) : 0.0f);
         }
@@ -265,34 +272,31 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
     //         accumulation), the matrices passing through its own LDS blocks between products (the operations of
     //         one wavefront on LDS complete in order, so no workgroup barrier is needed until all four are done).
     if (wave < 4) {
-        auto at = [&](float *m, int blk) { return m + (16 * blk) * kPitchF + 16 * blk; };
         auto f4h = [](const float4v &x) { return (half4v){(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]}; };
         // dst = (add ? add : 0) + X Y; lane (li, lq) holds rows 4 lq + r of column li of the result
         auto mm = [&](float *dst, const float *X, const float *Y, const float *add) {
-            const half4v xa = f4h(*(const float4v *)&X[li * kPitchF + 4 * lq]);
+            const half4v xa = f4h(*(const float4v *)&X[li * kPitchD + 4 * lq]);
             float4v yb, c;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                yb[r] = Y[(4 * lq + r) * kPitchF + li];
-                c[r] = add ? add[(4 * lq + r) * kPitchF + li] : 0.0f;
+                yb[r] = Y[(4 * lq + r) * kPitchD + li];
+                c[r] = add ? add[(4 * lq + r) * kPitchD + li] : 0.0f;
             }
             c = __builtin_amdgcn_mfma_f32_16x16x16f16(xa, f4h(yb), c, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) dst[(4 * lq + r) * kPitchF + li] = c[r];
+            for (int r = 0; r < 4; ++r) dst[(4 * lq + r) * kPitchD + li] = c[r];
             __builtin_amdgcn_wave_barrier();
         };
-        float *Lb = at(Lm, wave), *Nb = at(Nm, wave), *Pb = at(P0, wave), *Qb = at(P1, wave);
+        float *Lb = Dm + wave * kBlockD, *Nb = Sm + (3 * wave) * kBlockD, *Pb = Nb + kBlockD, *Qb = Pb + kBlockD;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchF + li] = Lb[(4 * lq + r) * kPitchF + li] + (4 * lq + r == li ? 1.0f : 0.0f);
+        for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchD + li] = Lb[(4 * lq + r) * kPitchD + li] + (4 * lq + r == li ? 1.0f : 0.0f);
         __builtin_amdgcn_wave_barrier();
         mm(Qb, Lb, Lb, nullptr);  // L^2
         mm(Lb, Nb, Qb, Nb);       // (I + L)(I + L^2), into L's block (L itself is not needed any more)
         mm(Pb, Qb, Qb, nullptr);  // L^4
         mm(Nb, Lb, Pb, Lb);       // ... (I + L^4)
         mm(Qb, Pb, Pb, nullptr);  // L^8
-        mm(Lb, Nb, Qb, Nb);       // ... (I + L^8): the inverse, in L's diagonal block
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchF + li] = Lb[(4 * lq + r) * kPitchF + li];
+        mm(Lb, Nb, Qb, Nb);       // ... (I + L^8): the inverse, where the diagonal block of L was
     }
     __syncthreads();
 
@@ -342,10 +346,10 @@ __global__ __launch_bounds__(512, 2) void deltanet_chunk_prepare_kernel(ChunkArg
                 for (int r = 0; r < 4; ++r) acc[r] = (float)rr[r] * fac[16 * ra + 4 * lq + r];
 #pragma unroll
                 for (int m = 0; m < ra; ++m) {
-                    const half4v la = f4h(*(const float4v *)&Lm[(16 * ra + li) * kPitchF + 16 * m + 4 * lq]);
+                    const half4v la = *(const half4v *)&Lh[(16 * ra + li) * kPitchL + 16 * m + 4 * lq];
                     acc = __builtin_amdgcn_mfma_f32_16x16x16f16(la, xh[x][m], acc, 0, 0, 0);
                 }
-                const half4v na = f4h(*(const float4v *)&Nm[(16 * ra + li) * kPitchF + 16 * ra + 4 * lq]);
+                const half4v na = f4h(*(const float4v *)&Dm[ra * kBlockD + li * kPitchD + 4 * lq]);
                 const float4v xa = __builtin_amdgcn_mfma_f32_16x16x16f16(na, f4h(acc), (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                 xh[x][ra] = f4h(xa);
                 if (!is_w) *(half4v *)(wsu + kOffU + ((ra * 8 + tile0 + x) * 64 + lane) * 8) = xh[x][ra];
