@@ -399,11 +399,18 @@ __global__ __launch_bounds__(kScanThreads) void deltanet_chunk_scan_kernel(Chunk
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
-    // the two column halves of a (sequence, head) read the same operands: linear ids congruent mod 8 put them on
-    // the same XCD, where the second reader finds them in L2
-    const int p = blockIdx.x, pairs = a.B * a.nv;
+    // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The two column halves of a
+    // (sequence, v-head) read the same -W / masked q k^T, and all v-heads of a k-head (both halves of each) the same q and
+    // k^T: the 2 * rep workgroups of a (sequence, k-head) get linear ids congruent mod 8, consecutive in that XCD's
+    // order, so that each of those operands comes from HBM once and the other readers find it in L2.
+    const int p = blockIdx.x, pairs = a.B * a.nv, rep = a.nv / a.nk;
     int pair, half;
-    if ((pairs & 7) == 0) {
+    if (((a.B * a.nk) & 7) == 0) {
+        const int i = p >> 3, per = 2 * rep;                   // position in the XCD's order; workgroups per k-head
+        const int ku = (p & 7) + 8 * (i / per), sub = i % per;  // (sequence, k-head) unit; member of its group
+        pair = ku * rep + (sub >> 1);
+        half = sub & 1;
+    } else if ((pairs & 7) == 0) {
         pair = (p & 7) + 8 * (p >> 4);
         half = (p >> 3) & 1;
     } else {
