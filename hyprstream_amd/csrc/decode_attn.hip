@@ -231,9 +231,11 @@ __device__ __forceinline__ uint32_t fp8x2_to_f16x2(uint32_t t) {
 }
 
 template <int kD, bool FP8, bool ROPE, bool BAL>
-__global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
+__global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a_in) {
+    const DecodeArgs &a = a_in;
     constexpr int kStep = Shape<kD>::kStep, NT = Shape<kD>::NT, NJ = Shape<kD>::NJ, NC = Shape<kD>::NC;
     constexpr int VW = Shape<kD>::VW, NBB = Shape<kD>::NBB, CW = Shape<kD>::CW, NS = Shape<kD>::NS;
+    constexpr bool kPreloadNext = BAL;
     const int h = blockIdx.y;
     const int G = a.G;
     // the wavefront index as a scalar: everything derived from it (the steps this wavefront walks, block-table lookups,
@@ -244,10 +246,31 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     __shared__ float sm_m[kWavesPerWg][16], sm_l[kWavesPerWg][16];
     __shared__ float sm_o[kWavesPerWg][16][CW + 4];  // one column group of O at a time
     // One work item: tokens [t_begin, t_end) of sequence b (L cached tokens), partial slot `chunk`.
-    auto run_item = [&](const int b, const int L, const int t_begin, const int t_end, const int chunk) {
+    struct Item {
+        int b, L, t_begin, t_end, chunk;
+    };
+    // The two stages of the load pipeline and the location of the step this wavefront loads next live outside an
+    // item: a workgroup that walks several items (balanced mode) issues the first loads of the next item before it
+    // merges and writes out the current one, so that the pipeline does not run empty at every sequence end.
+    Stage<kD> sa, sb;
+    int64_t nku = 0, nvu = 0;
+    int nks = 0, nvs = 0;
+    // `preloaded`: the first stage of this item is already in flight (issued at the end of the previous item);
+    // `next`: the item whose first loads this one issues before it merges (has_next), else ignored.
+    auto run_item = [&](const Item it, const bool preloaded, const Item next, const bool has_next) {
+    const int b = it.b, L = it.L, chunk = it.chunk;
+    // Balanced mode runs this body in a loop over items.  Read through the kernel's own parameter, every argument an
+    // item needs anywhere (new-token sources, Q, outputs, tables: far more than the scalar register file holds) is
+    // loaded once ahead of that loop and stays live across it, and the loop over the steps runs on spilled scalars.
+    // Each item therefore reads its arguments anew from the kernel-argument segment, through a pointer the compiler
+    // cannot see through: they are loaded where they are used and die there, as in the one-item instances.
+    uintptr_t seg = (uintptr_t)__builtin_amdgcn_kernarg_segment_ptr();  // DecodeArgs is the kernel's only parameter
+    if constexpr (BAL) asm volatile("" : "+s"(seg));
+    const DecodeArgs &a = BAL ? *(const DecodeArgs *)(const __attribute__((address_space(4))) DecodeArgs *)seg : a_in;
     // This workgroup reads the newest token if it owns the end of the sequence: it then writes it first (K by
     // wavefront 0, V by wavefront 1).  With five or more steps the token sits beyond every wavefront's first tile,
     // so those first loads are issued ahead of the write and its barrier instead of behind them.
+    const int t_begin = it.t_begin, t_end = it.t_end;
     const bool writes_new = a.nt.src[0] != nullptr && t_end == L;
     auto write_new_token = [&]() {
         if (wave < 2) quantize_row<kD / 64, FP8>(a.nt, wave, (int64_t)b * a.Hkv + h, lane);
@@ -269,21 +292,19 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     // Where the step this wavefront loads next lives (sequence or block, slot).  With block tables the lookup is a
     // dependent (scalar) load in front of every address, so it is issued one stage ahead: load_stage() uses the
     // location found while the previous stage was loaded and starts the lookup for the one after.
-    int64_t nku = 0, nvu = 0;
-    int nks = 0, nvs = 0;
-    auto locate = [&](int step) {
-        const int t0 = t_begin + step * kStep;
-        if (t0 < t_end) {
-            resolve(a.ka, b, t0, nku, nks);
-            resolve(a.va, b, t0, nvu, nvs);
+    auto locate = [&](const Item &w, int step) {
+        const int t0 = w.t_begin + step * kStep;
+        if (t0 < w.t_end) {
+            resolve(a.ka, w.b, t0, nku, nks);
+            resolve(a.va, w.b, t0, nvu, nvs);
         }
     };
-    auto load_stage = [&](Stage<kD> &st, int step) {
-        const int t0 = t_begin + step * kStep;
+    auto load_stage = [&](Stage<kD> &st, const Item &w, int step) {
+        const int t0 = w.t_begin + step * kStep;
         const int64_t ku = nku, vu = nvu;
         const int kslot = nks, vslot = nvs;
-        locate(step + kWavesPerWg);
-        const int last = L - 1 - t0;  // last valid row offset inside this step (>= 0)
+        locate(w, step + kWavesPerWg);
+        const int last = w.L - 1 - t0;  // last valid row offset inside this step (>= 0)
         const uint8_t *kb = a.kc + ku * a.ka.code_stride_seq + (int64_t)h * a.ka.code_stride_head + (int64_t)kslot * kD;
         const uint8_t *vb = a.vc + vu * a.va.code_stride_seq + (int64_t)h * a.va.code_stride_head + (int64_t)vslot * kD;
 #pragma unroll
@@ -432,12 +453,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     };
 
     // ---- software pipeline over this wavefront's steps (wave, wave+4, ...)
-    Stage<kD> sa, sb;
     int step = wave;
-    const bool early_loads = nsteps >= kWavesPerWg + 1;
+    const bool early_loads = nsteps >= kWavesPerWg + 1;  // a preloaded item always has them
     if (writes_new && !early_loads) write_new_token();
-    locate(step);
-    if (step < nsteps) load_stage(sa, step);
+    if (!preloaded) {
+        locate(it, step);
+        if (step < nsteps) load_stage(sa, it, step);
+    }
     if (writes_new && early_loads) write_new_token();
     // ---- Q operand (prepared while the first K/V tiles are in flight): lane (head li, quarter lq) holds
     //      Q[head][64*(j/2) + 16*lq + 8*(j%2) + e] for MFMA j.
@@ -498,15 +520,20 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
     }
     while (step < nsteps) {
         const int n1 = step + kWavesPerWg;
-        if (n1 < nsteps) load_stage(sb, n1);
+        if (n1 < nsteps) load_stage(sb, it, n1);
         compute_stage(sa, step);
         if (n1 >= nsteps) break;
         const int n2 = n1 + kWavesPerWg;
-        if (n2 < nsteps) load_stage(sa, n2);
+        if (n2 < nsteps) load_stage(sa, it, n2);
         compute_stage(sb, n1);
         step = n2;
     }
 
+    // ---- the next item's first tiles travel while this one is merged and written out
+    if (kPreloadNext && has_next) {
+        locate(next, wave);
+        if (wave * kStep < next.t_end - next.t_begin) load_stage(sa, next, wave);
+    }
     // ---- merge the four wavefronts through LDS
     l_run += __shfl_xor(l_run, 16, 64);
     l_run += __shfl_xor(l_run, 32, 64);
@@ -584,7 +611,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
                 for (int i = threadIdx.x; i < G * kD; i += 256) a.out[((int64_t)b * a.Hq + h * G) * kD + i] = 0;
             return;
         }
-        run_item(b, L, t_begin, min(L, t_begin + a.chunk_tokens), slot);
+        const Item it = {b, L, t_begin, min(L, t_begin + a.chunk_tokens), slot};
+        run_item(it, false, it, false);
     } else {
         __shared__ int sm_pref[kMaxBalancedB + 1];  // granules before sequence b
         if (wave == 0) {
@@ -615,15 +643,32 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a) {
             const int mid = (lo + hi) >> 1;
             if (uni(sm_pref[mid + 1]) > g_lo) hi = mid; else lo = mid + 1;
         }
-        bool first = true;
-        for (int b = lo; b < a.B; ++b) {
-            const int pb = uni(sm_pref[b]);
-            if (pb >= g_hi) break;
-            if (uni(sm_pref[b + 1]) == pb) continue;  // an empty sequence: the merge kernel writes its zeros
-            const int L = min(a.seq_lens[b], a.max_seq_len);
-            if (!first) __syncthreads();  // the previous item's merge buffers have been read
-            first = false;
-            run_item(b, L, max(g_lo - pb, 0) * 64, min(L, (g_hi - pb) * 64), (int)blockIdx.x - pb / W);
+        // the item of the first non-empty sequence at or after b that reaches into the range (returns B: none); an
+        // empty sequence is skipped, the merge kernel writes its zeros
+        auto item_from = [&](int b, Item &it) {
+            for (; b < a.B; ++b) {
+                const int pb = uni(sm_pref[b]);
+                if (pb >= g_hi) return a.B;
+                if (uni(sm_pref[b + 1]) == pb) continue;
+                const int L = min(a.seq_lens[b], a.max_seq_len);
+                it = {b, L, max(g_lo - pb, 0) * 64, min(L, (g_hi - pb) * 64), (int)blockIdx.x - pb / W};
+                return b;
+            }
+            return a.B;
+        };
+        Item cur = {0, 0, 0, 0, 0}, nxt = cur;
+        int b = item_from(lo, cur);
+        bool preloaded = false;
+        while (b < a.B) {
+            const int nb = item_from(b + 1, nxt);
+            // the next item's first loads may go out early unless they could cover a token it has yet to write
+            const bool ahead = kPreloadNext && nb < a.B &&
+                               (a.nt.src[0] == nullptr || nxt.t_end != nxt.L || nxt.t_end - nxt.t_begin > kWavesPerWg * kStep);
+            run_item(cur, preloaded, nxt, ahead);
+            if (nb < a.B) __syncthreads();  // this item's merge buffers have been read
+            preloaded = ahead;
+            cur = nxt;
+            b = nb;
         }
     }
 }
