@@ -205,7 +205,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         "tokens_per_s": B * T / (ms * 1e-3),
         "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel (%d chunk launches)" % len(chunks), "achieved": flops / (kms * 1e-3) / 1e12,
                      "peak": peak, "unit": "TFLOP/s", "frac": flops / (kms * 1e-3) / 1e12 / peak, "traffic": None,
-                     "avg_us_8_launches": kms * 1e3},
+                     "avg_us_all_launches": kms * 1e3},
     }
     print(json.dumps(res))
 
@@ -289,6 +289,8 @@ def main():
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
     ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 128, 256],
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
+    ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
+                    help="prefill workloads: tokens per chunk call (0 = the workload's own: 512, c3-prompt 4096)")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
@@ -318,7 +320,7 @@ def main():
         print(json.dumps({"calibrate_copy_bytes": 1 << 30, "launches": max(1, args.steps)}))
         return
     if args.workload.startswith("c3"):
-        return bench_prefill(args, torch, hb, wl, C=4096 if args.workload == "c3-prompt" else 512,
+        return bench_prefill(args, torch, hb, wl, C=args.chunk_tokens or (4096 if args.workload == "c3-prompt" else 512),
                              fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload == "c3-b1", prologue=args.workload == "c3-prologue")
     if args.workload.startswith("c5"):
         return bench_deltanet(args, torch, hb, wl, "prefill" in args.workload, recurrent=args.workload.endswith("recurrent"))
