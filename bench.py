@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-prefill|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -278,12 +278,81 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False):
     print(json.dumps(res))
 
 
+def bench_deltanet_layer(args, torch, hb, wl, fused):
+    """The decode branch of a gated-DeltaNet layer between its two projections (Config 5's shape, B = 64 unless --batch):
+    conv1d + SiLU + gates for the new token, the recurrent step, the gated RMSNorm.  c5-decode-layer: one launch
+    (hs_deltanet_decode_layer); c5-decode-layer-3calls: hs_deltanet_prepare + hs_deltanet_forward + hs_deltanet_gated_norm
+    (four launches), the same results bit for bit.  Bytes: the fp32 state read and written once plus the step's
+    activations, conv state and weights."""
+    dev = "cuda:0"
+    nk, nv, d = 16, 32, 128
+    B = args.batch or 64
+    C = 2 * nk * d + nv * d
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(wl.SEED)
+    rn = lambda *s: torch.randn(*s, generator=gen, device=dev)
+    x, w = rn(B, 1, C).to(torch.bfloat16), (0.5 * rn(C, 4)).to(torch.bfloat16)
+    cs = [rn(B, C, 3).to(torch.bfloat16), torch.empty(B, C, 3, dtype=torch.bfloat16, device=dev)]
+    a_in, b_in = (2 * rn(B, 1, nv)).to(torch.bfloat16), (2 * rn(B, 1, nv)).to(torch.bfloat16)
+    nae, dtb = -rn(nv).exp(), rn(nv)
+    z, nw = rn(B, 1, nv, d).to(torch.bfloat16), rn(d)
+    ncopies = max(1, args.copies)
+    states = [rn(B, nv, d, d) * 0.1 for _ in range(ncopies)]
+    out = torch.empty(B, 1, nv, d, dtype=torch.bfloat16, device=dev)
+    o32 = torch.empty(B, 1, nv, d, dtype=torch.float32, device=dev)
+    qs = 1.0 / float(np.sqrt(d))
+
+    def step(i):
+        src, dst = cs[i & 1], cs[(i + 1) & 1]
+        if fused:
+            hb.deltanet_decode_layer(x, w, src, a_in, b_in, nae, dtb, z, nw, 1e-6, states[i % ncopies], nk, nv, d, d, qs, True,
+                                     out=out, conv_state_out=dst)
+        else:
+            q, k, v, g, beta, _ = hb.deltanet_prepare(x, w, src, a_in, b_in, nae, dtb, nk, nv, d, d)
+            hb.deltanet_forward(q, k, v, g, beta, states[i % ncopies], o32, qs, True)
+            hb.deltanet_gated_norm(o32, z, nw, 1e-6)
+
+    settle(torch, step, window=20, min_launches=300, max_launches=2000)
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / args.steps * 1e3
+    n_ev = 100
+    e0 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
+    e1 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
+    for i in range(n_ev):
+        e0[i].record()
+        step(i)
+        e1[i].record()
+    torch.cuda.synchronize()
+    kms = float(np.mean([a_.elapsed_time(b_) for a_, b_ in zip(e0, e1)]))
+    nbytes = 2 * B * nv * d * d * 4 + B * (C * 2 + 2 * C * 3 * 2 + 2 * nv * 2 + 2 * nv * d * 2) + C * 4 * 2
+    res = {
+        "metric": "deltanet decode layer (conv + gates + step + gated norm) HBM GB/s + tokens/s, nk=16 nv=32 dk=dv=128",
+        "value": nbytes / (ms * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32 state and arithmetic, bf16 activations", "data": "synthetic (seeded, generated on device)",
+        "config": {"workload": "c5-decode-layer%s: gated-DeltaNet layer decode step B=%d nk=16 nv=32 dk=dv=128, %s"
+                               % ("" if fused else "-3calls", B, "one launch" if fused else "prepare + step + gated norm (four launches)"),
+                   "algorithmic_bytes_per_step": int(nbytes)},
+        "tokens_per_s": B / (ms * 1e-3),
+        "roofline": {"bound": "hbm", "kernel": "deltanet_decode_kernel<true>" if fused else "deltanet_conv8 + gates + deltanet_decode_kernel<false> + gated_rmsnorm_rows",
+                     "achieved": nbytes / (kms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "avg_kernel_us": kms * 1e3},
+    }
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-prefill", "c5-prefill-recurrent"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
@@ -291,6 +360,7 @@ def main():
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
     ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
                     help="prefill workloads: tokens per chunk call (0 = the workload's own: 512, c3-prompt 4096)")
+    ap.add_argument("--batch", type=int, default=0, help="c5-decode-layer workloads: sequences in the batch (0 = 64)")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
@@ -322,6 +392,8 @@ def main():
     if args.workload.startswith("c3"):
         return bench_prefill(args, torch, hb, wl, C=args.chunk_tokens or (4096 if args.workload == "c3-prompt" else 512),
                              fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload == "c3-b1", prologue=args.workload == "c3-prologue")
+    if args.workload.startswith("c5-decode-layer"):
+        return bench_deltanet_layer(args, torch, hb, wl, fused=args.workload == "c5-decode-layer")
     if args.workload.startswith("c5"):
         return bench_deltanet(args, torch, hb, wl, "prefill" in args.workload, recurrent=args.workload.endswith("recurrent"))
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]

@@ -188,6 +188,22 @@ pub unsafe fn deltanet_forward_gpu(q: *const c_void, k: *const c_void, v: *const
     check(bindings::hs_deltanet_forward(q, k, v, g, beta, state, out, b, t, nk, nv, dk, dv, q_scale, l2norm as c_int, stream))
 }
 
+/// One decode step of a gated-DeltaNet layer between its projections in a single launch (conv1d + SiLU + gates,
+/// the recurrent step, RMSNormGated: GatedDeltaNetLayer::forward, qwen3_5.rs:629-786 with seq == 1).
+///
+/// # Safety
+/// As above; `conv_state_out` must not alias `conv_state_in`.
+#[allow(clippy::too_many_arguments)]
+pub unsafe fn deltanet_decode_layer_gpu(mixed_qkv: *const c_void, conv_weight: *const c_void, conv_state_in: *const c_void,
+                                        conv_state_out: *mut c_void, a_in: *const c_void, b_in: *const c_void,
+                                        neg_a_exp: *const f32, dt_bias: *const f32, z: *const c_void, norm_weight: *const f32,
+                                        norm_eps: f32, state: *mut f32, out: *mut c_void, b: i32, nk: i32, nv: i32, dk: i32,
+                                        dv: i32, q_scale: f32, l2norm: bool, stream: hs_stream_t) -> Result<()> {
+    check(bindings::hs_deltanet_decode_layer(mixed_qkv, conv_weight, conv_state_in, conv_state_out, a_in, b_in, neg_a_exp,
+                                             dt_bias, z, norm_weight, norm_eps, state, out, b, nk, nv, dk, dv, q_scale,
+                                             l2norm as c_int, stream))
+}
+
 /// Bytes of split-K workspace a decode call of this shape may need.
 pub fn decode_workspace_bytes(shape: AttnShape, max_seq_len: i32) -> usize {
     unsafe { bindings::hs_decode_attn_workspace_bytes(shape.b, shape.hq, shape.hkv, shape.d, max_seq_len) }

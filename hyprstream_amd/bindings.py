@@ -26,7 +26,7 @@ EXPORTS = [
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
     "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue",
-    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_forward_chunked", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
+    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
 
@@ -361,6 +361,25 @@ def deltanet_prepare(mixed_qkv, conv_weight, conv_state_in, a_in, b_in, neg_a_ex
                                     _ptr(a_in.contiguous()), _ptr(b_in.contiguous()), _ptr(neg_a_exp), _ptr(dt_bias),
                                     _ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), B, S, nk, nv, dk, dv, _stream()))
     return q, k, v, g, beta, state_out
+
+
+def deltanet_decode_layer(mixed_qkv, conv_weight, conv_state_in, a_in, b_in, neg_a_exp, dt_bias, z, norm_weight, eps,
+                          state, nk, nv, dk, dv, q_scale, l2norm=True, out=None, conv_state_out=None):
+    """One decode step of a gated-DeltaNet layer between its projections, one launch.  mixed_qkv [B, 1, C];
+    `state` is updated in place.  Returns (out bf16 [B, 1, nv, dv], new_conv_state)."""
+    import torch
+    B, S, C = mixed_qkv.shape
+    assert S == 1 and C == 2 * nk * dk + nv * dv and mixed_qkv.is_contiguous() and conv_weight.is_contiguous()
+    dev = mixed_qkv.device
+    if out is None:
+        out = torch.empty(B, 1, nv, dv, dtype=torch.bfloat16, device=dev)
+    if conv_state_out is None:
+        conv_state_out = torch.empty(B, C, 3, dtype=torch.bfloat16, device=dev)
+    check(lib().hs_deltanet_decode_layer(_ptr(mixed_qkv), _ptr(conv_weight), _ptr(conv_state_in), _ptr(conv_state_out),
+                                         _ptr(a_in), _ptr(b_in), _ptr(neg_a_exp), _ptr(dt_bias), _ptr(z), _ptr(norm_weight),
+                                         ctypes.c_float(eps), _ptr(state), _ptr(out), B, nk, nv, dk, dv,
+                                         ctypes.c_float(q_scale), int(bool(l2norm)), _stream()))
+    return out, conv_state_out
 
 
 def deltanet_gated_norm(x, z, weight, eps):

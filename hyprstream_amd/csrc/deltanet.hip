@@ -204,40 +204,134 @@ __global__ __launch_bounds__(512) void deltanet_prefill_kernel(DeltaArgs a) {
 // through LDS (32 floats each way).  With 16 KB per wavefront (all 128 rows, no exchange) the step took 47.9 us at
 // B = 64 x 32 heads; a plain read-scale-write kernel of the same shape takes 46.2 us with 16 KB per wavefront and
 // 43.1 us with 8 KB (more wavefronts in flight, shorter ones).
-__global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
+//
+// LAYER: the whole decode branch of GatedDeltaNetLayer::forward between the two projections in one launch
+// (qwen3_5.rs:629-686 conv1d + SiLU + gates, :725-751 the step, :305-313 RMSNormGated).  A 512-thread workgroup owns
+// all 128 columns of its (sequence, v-head) -- the norm runs over them -- as two such 64-column halves.  While the
+// state loads travel, 384 threads compute the head's q, k and v channels from the mixed projection (depthwise causal
+// conv over [3 carried frames | the new one], SiLU, each rounded to bf16 as the separate kernels store them) into
+// LDS and thread 384 the two gates; the step then reads them from there, and its output row goes through the gated
+// norm instead of to memory.  Every value is computed with the expressions of deltanet_conv8_kernel,
+// deltanet_gates_kernel, the plain instance of this kernel and gated_rmsnorm_rows_kernel, in their order.
+struct LayerArgs {
+    const uint16_t *x;         // [B, 1, C] bf16 mixed q|k|v projection, C = 2*key_dim + val_dim
+    const uint16_t *w;         // [C, 4] bf16 conv taps, tap 3 multiplies the new frame
+    const uint16_t *state_in;  // [B, C, 3] bf16 or nullptr (= zeros)
+    uint16_t *state_out;       // [B, C, 3]
+    const uint16_t *a_in, *b_in;          // [B, 1, nv] bf16
+    const float *neg_a_exp, *dt_bias;     // [nv]
+    const uint16_t *z;         // [B, 1, nv, dv] bf16 gate of the norm
+    const float *norm_w;       // [dv]
+    uint16_t *out;             // [B, 1, nv, dv] bf16
+    float eps;
+    int32_t C, key_dim;
+};
+
+// SiLU through v_exp_f32 and v_rcp_f32, as deltanet_glue.hip computes it
+__device__ __forceinline__ float silu_fast_layer(float x) {
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.4426950408889634f));
+}
+
+template <bool LAYER>
+__global__ __launch_bounds__(LAYER ? 512 : 256) void deltanet_decode_kernel(DeltaArgs a, LayerArgs la) {
     typedef float f4 __attribute__((ext_vector_type(4)));
-    __shared__ f4 sm_m[4][8], sm_o[4][8];  // [wavefront][column quad]
+    constexpr int NH = LAYER ? 2 : 1;             // column halves in this workgroup
+    __shared__ f4 sm_m[NH][4][8], sm_o[NH][4][8];  // [half][wavefront of the half][column quad]
+    __shared__ __attribute__((aligned(16))) float sm_in[LAYER ? 3 * 128 + 4 : 4];  // q | k | v of the head, then g and beta
+    __shared__ __attribute__((aligned(16))) float sm_row[LAYER ? 128 : 4];        // the step's output row
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int sl = wave & 1, rh = wave >> 1;
-    const int chalf = (int)(blockIdx.x & 1);
-    const int j = (int)((blockIdx.x >> 1) % a.nv);
-    const int b = (int)((blockIdx.x >> 1) / a.nv);
+    const int w4 = wave & 3, sl = wave & 1, rh = (wave >> 1) & 1;
+    const int unit = LAYER ? (int)blockIdx.x : (int)(blockIdx.x >> 1);
+    const int chalf = LAYER ? wave >> 2 : (int)(blockIdx.x & 1), hx = LAYER ? chalf : 0;
+    const int j = unit % a.nv;
+    const int b = unit / a.nv;
     const int hk = j / (a.nv / a.nk);
     const int c4 = lane & 7, rg = lane >> 3;
     const int col = chalf * 64 + sl * 32 + 4 * c4;
     const int row0 = rh * 64 + rg * 8;
     float *sp = a.state + (((int64_t)b * a.nv + j) * kDK + row0) * kDV + col;
+    const int64_t bt = b;  // T == 1
+    // LAYER: the small loads of the prologue are issued ahead of the state's (loads return in order: behind the 8 KB
+    // of state they would arrive last, and the arithmetic that hides under the state loads would wait).  The norm's
+    // own inputs are loaded where they are used: held from here they cost 14 registers and a resident workgroup
+    // (51.5 against 50.6 us per step at B = 64).
+    const int pt = threadIdx.x, ppart = pt >> 7;  // 0: q, 1: k (channels of k-head hk), 2: v (of v-head j)
+    const int pc = ppart == 2 ? 2 * la.key_dim + j * kDV + (pt & 127) : ppart * la.key_dim + hk * kDK + (pt & 127);
+    uint32_t ps0 = 0u, ps1 = 0u, ps2 = 0u, pxn = 0u, pw01 = 0u, pw23 = 0u, pab = 0u;
+    if constexpr (LAYER) {
+        if (pt < 3 * 128) {
+            if (la.state_in) {
+                const uint16_t *sin = la.state_in + ((int64_t)b * la.C + pc) * 3;
+                ps0 = sin[0]; ps1 = sin[1]; ps2 = sin[2];
+            }
+            pxn = la.x[(int64_t)b * la.C + pc];
+            pw01 = *(const uint32_t *)(la.w + (int64_t)pc * 4);
+            pw23 = *(const uint32_t *)(la.w + (int64_t)pc * 4 + 2);
+        } else if (pt == 3 * 128) {
+            pab = (uint32_t)la.a_in[bt * a.nv + j] | ((uint32_t)la.b_in[bt * a.nv + j] << 16);
+        }
+    }
     f4 S[8];
 #pragma unroll
     for (int r = 0; r < 8; ++r) S[r] = __builtin_nontemporal_load((const f4 *)(sp + (int64_t)r * kDV));  // read once
 
-    const int64_t bt = b;  // T == 1
-    const uint16_t *kfull = a.k + (bt * a.nk + hk) * kDK, *qfull = a.q + (bt * a.nk + hk) * kDK;
-    const u32x4 kw = *(const u32x4 *)(kfull + row0), qw = *(const u32x4 *)(qfull + row0);
     float kf[8], qf[8];
+    f4 v;
+    float g, beta;
+    if constexpr (LAYER) {
+        {
+#pragma clang fp contract(off)
+            const int t = pt;
+            if (t < 3 * 128) {
+                const int part = ppart, c = pc;
+                const uint32_t s0 = ps0, s1 = ps1, s2 = ps2, xn = pxn;
+                float acc = bf16_bits_to_f32(pw01 & 0xffffu) * bf16_bits_to_f32(s0);
+                acc += bf16_bits_to_f32(pw01 >> 16) * bf16_bits_to_f32(s1);
+                acc += bf16_bits_to_f32(pw23 & 0xffffu) * bf16_bits_to_f32(s2);
+                acc += bf16_bits_to_f32(pw23 >> 16) * bf16_bits_to_f32(xn);
+                const float y = silu_fast_layer((float)(__bf16)acc);  // the conv output is a bf16 tensor before the SiLU
+                sm_in[t] = (float)(__bf16)y;
+                // the carried frames move up by one; the k-head's channels are written by its first v-head only
+                if (part == 2 || j % (a.nv / a.nk) == 0) {
+                    uint16_t *so = la.state_out + ((int64_t)b * la.C + c) * 3;
+                    so[0] = (uint16_t)s1;
+                    so[1] = (uint16_t)s2;
+                    so[2] = (uint16_t)xn;
+                }
+            } else if (t == 3 * 128) {
+                const float xa = bf16_bits_to_f32(pab & 0xffffu) + la.dt_bias[j];
+                const float spl = xa > 20.0f ? xa : log1pf(expf(xa));  // softplus with libtorch's linear threshold
+                sm_in[3 * 128] = la.neg_a_exp[j] * spl;
+                sm_in[3 * 128 + 1] = 1.0f / (1.0f + expf(-bf16_bits_to_f32(pab >> 16)));
+            }
+        }
+        __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        kf[2 * i] = __uint_as_float(kw[i] << 16);
-        kf[2 * i + 1] = __uint_as_float(kw[i] & 0xffff0000u);
-        qf[2 * i] = __uint_as_float(qw[i] << 16);
-        qf[2 * i + 1] = __uint_as_float(qw[i] & 0xffff0000u);
+        for (int r = 0; r < 8; ++r) {
+            qf[r] = sm_in[row0 + r];
+            kf[r] = sm_in[128 + row0 + r];
+        }
+        v = *(const f4 *)&sm_in[256 + col];
+        g = sm_in[3 * 128];
+        beta = sm_in[3 * 128 + 1];
+    } else {
+        const uint16_t *kfull = a.k + (bt * a.nk + hk) * kDK, *qfull = a.q + (bt * a.nk + hk) * kDK;
+        const u32x4 kw = *(const u32x4 *)(kfull + row0), qw = *(const u32x4 *)(qfull + row0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            kf[2 * i] = __uint_as_float(kw[i] << 16);
+            kf[2 * i + 1] = __uint_as_float(kw[i] & 0xffff0000u);
+            qf[2 * i] = __uint_as_float(qw[i] << 16);
+            qf[2 * i + 1] = __uint_as_float(qw[i] & 0xffff0000u);
+        }
+        const uint32_t v01 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col);
+        const uint32_t v23 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col + 2);
+        v = (f4){__uint_as_float(v01 << 16), __uint_as_float(v01 & 0xffff0000u), __uint_as_float(v23 << 16),
+                 __uint_as_float(v23 & 0xffff0000u)};
+        g = a.g[bt * a.nv + j];
+        beta = a.beta[bt * a.nv + j];
     }
-    const uint32_t v01 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col);
-    const uint32_t v23 = *(const uint32_t *)(a.v + (bt * a.nv + j) * kDV + col + 2);
-    const f4 v = {__uint_as_float(v01 << 16), __uint_as_float(v01 & 0xffff0000u), __uint_as_float(v23 << 16),
-                  __uint_as_float(v23 & 0xffff0000u)};
-    const float g = a.g[bt * a.nv + j], beta = a.beta[bt * a.nv + j];
     auto rows_sum = [](float x) {  // over the 8 row groups: lanes with equal l % 8
         x += __shfl_xor(x, 8, 64);
         x += __shfl_xor(x, 16, 64);
@@ -246,9 +340,16 @@ __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
     };
     float kmul = 1.0f, qmul = a.q_scale;
     if (a.l2norm) {  // the norms run over all 128 elements: lane l takes elements 2l and 2l + 1 of each vector
-        const uint32_t k2 = ((const uint32_t *)kfull)[lane], q2 = ((const uint32_t *)qfull)[lane];
-        const float k0 = __uint_as_float(k2 << 16), k1 = __uint_as_float(k2 & 0xffff0000u);
-        const float q0 = __uint_as_float(q2 << 16), q1 = __uint_as_float(q2 & 0xffff0000u);
+        float k0, k1, q0, q1;
+        if constexpr (LAYER) {
+            k0 = sm_in[128 + 2 * lane]; k1 = sm_in[128 + 2 * lane + 1];
+            q0 = sm_in[2 * lane]; q1 = sm_in[2 * lane + 1];
+        } else {
+            const uint16_t *kfull = a.k + (bt * a.nk + hk) * kDK, *qfull = a.q + (bt * a.nk + hk) * kDK;
+            const uint32_t k2 = ((const uint32_t *)kfull)[lane], q2 = ((const uint32_t *)qfull)[lane];
+            k0 = __uint_as_float(k2 << 16); k1 = __uint_as_float(k2 & 0xffff0000u);
+            q0 = __uint_as_float(q2 << 16); q1 = __uint_as_float(q2 & 0xffff0000u);
+        }
         float sk = k0 * k0 + k1 * k1, sq = q0 * q0 + q1 * q1;
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
@@ -267,9 +368,9 @@ __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) m[e] = rows_sum(m[e]);
-    if (rg == 0) sm_m[wave][c4] = m;
+    if (rg == 0) sm_m[hx][w4][c4] = m;
     __syncthreads();
-    m = (sm_m[sl][c4] + sm_m[sl + 2][c4]) * decay;  // both row halves form the same sum in the same order
+    m = (sm_m[hx][sl][c4] + sm_m[hx][sl + 2][c4]) * decay;  // both row halves form the same sum in the same order
     const f4 delta = (v - m) * beta;
     f4 o = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -280,9 +381,39 @@ __global__ __launch_bounds__(256) void deltanet_decode_kernel(DeltaArgs a) {
     }
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = rows_sum(o[e]);
-    if (rg == 0) sm_o[wave][c4] = o;
+    if (rg == 0) sm_o[hx][w4][c4] = o;
     __syncthreads();
-    if (rh == 0 && rg == 0) *(f4 *)(a.out + (bt * a.nv + j) * kDV + col) = (sm_o[sl][c4] + sm_o[sl + 2][c4]) * qmul;
+    if constexpr (!LAYER) {
+        if (rh == 0 && rg == 0) *(f4 *)(a.out + (bt * a.nv + j) * kDV + col) = (sm_o[0][sl][c4] + sm_o[0][sl + 2][c4]) * qmul;
+    } else {
+        if (rh == 0 && rg == 0) *(f4 *)&sm_row[col] = (sm_o[hx][sl][c4] + sm_o[hx][sl + 2][c4]) * qmul;
+        __syncthreads();
+        if (wave == 0 && lane < 16) {  // RMSNormGated over the 128 columns: 16 lanes x 8 elements, as gated_rmsnorm_rows_kernel<16>
+            const int sub = lane;
+            const f4 xa = *(const f4 *)&sm_row[8 * sub], xb = *(const f4 *)&sm_row[8 * sub + 4];
+            const int64_t e0 = (bt * a.nv + j) * kDV + 8 * sub;
+            const u32x4 zz = *(const u32x4 *)(la.z + e0);
+            const f4 wa = *(const f4 *)(la.norm_w + 8 * sub), wb = *(const f4 *)(la.norm_w + 8 * sub + 4);
+            const float xv[8] = {xa[0], xa[1], xa[2], xa[3], xb[0], xb[1], xb[2], xb[3]};
+            const float wv[8] = {wa[0], wa[1], wa[2], wa[3], wb[0], wb[1], wb[2], wb[3]};
+            float ss = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss += xv[e] * xv[e];
+#pragma unroll
+            for (int o2 = 1; o2 < 16; o2 <<= 1) ss += __shfl_xor(ss, o2, 64);
+            const float rrms = 1.0f / sqrtf(ss / (float)kDV + la.eps);
+            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+            uint32_t o4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float z0 = __uint_as_float(zz[i] << 16), z1 = __uint_as_float(zz[i] & 0xffff0000u);
+                const bf16x2 pr = {(__bf16)(xv[2 * i] * rrms * wv[2 * i] * silu_fast_layer(z0)),
+                                   (__bf16)(xv[2 * i + 1] * rrms * wv[2 * i + 1] * silu_fast_layer(z1))};
+                o4[i] = __builtin_bit_cast(uint32_t, pr);
+            }
+            *(u32x4 *)(la.out + e0) = (u32x4){o4[0], o4[1], o4[2], o4[3]};
+        }
+    }
 }
 
 }  // namespace hs
@@ -302,9 +433,40 @@ extern "C" int hs_deltanet_forward(const void *q, const void *k, const void *v, 
     a.B = B; a.T = T; a.nk = nk; a.nv = nv; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
     hipStream_t st = (hipStream_t)stream;
     if (T == 1) {
-        deltanet_decode_kernel<<<(unsigned)((int64_t)B * nv * 2), 256, 0, st>>>(a);
+        deltanet_decode_kernel<false><<<(unsigned)((int64_t)B * nv * 2), 256, 0, st>>>(a, LayerArgs{});
     } else {
         deltanet_prefill_kernel<<<(unsigned)((int64_t)B * nv * 2), 512, 0, st>>>(a);
     }
     return check_launch("deltanet");
+}
+
+extern "C" int hs_deltanet_decode_layer(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in,
+                                        void *conv_state_out, const void *a_in, const void *b_in, const float *neg_a_exp,
+                                        const float *dt_bias, const void *z, const float *norm_weight, float norm_eps,
+                                        float *state, void *out, int32_t B, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
+                                        float q_scale, int l2norm, hs_stream_t stream) {
+    using namespace hs;
+    if (B > 0 && (!mixed_qkv || !conv_weight || !conv_state_out || !a_in || !b_in || !neg_a_exp || !dt_bias || !z ||
+                  !norm_weight || !state || !out))
+        return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (conv_state_out && conv_state_in == conv_state_out)
+        return fail(HS_ERR_INVALID_ARGUMENT, "conv_state_out must not alias conv_state_in");
+    if (dk != kDK || dv != kDV) return fail(HS_ERR_INVALID_ARGUMENT, "deltanet is built for dk = dv = 128, got %d x %d", dk, dv);
+    if (B < 0 || nk <= 0 || nv <= 0 || nv % nk != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d nk=%d nv=%d (need nv %% nk == 0)", B, nk, nv);
+    if ((((uintptr_t)z | (uintptr_t)norm_weight | (uintptr_t)out) & 15) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "z, norm_weight and out must be 16-byte aligned");
+    if (B == 0) return HS_OK;
+    DeltaArgs a{};
+    a.state = state;
+    a.B = B; a.T = 1; a.nk = nk; a.nv = nv; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
+    LayerArgs la;
+    la.x = (const uint16_t *)mixed_qkv; la.w = (const uint16_t *)conv_weight;
+    la.state_in = (const uint16_t *)conv_state_in; la.state_out = (uint16_t *)conv_state_out;
+    la.a_in = (const uint16_t *)a_in; la.b_in = (const uint16_t *)b_in;
+    la.neg_a_exp = neg_a_exp; la.dt_bias = dt_bias;
+    la.z = (const uint16_t *)z; la.norm_w = norm_weight; la.out = (uint16_t *)out; la.eps = norm_eps;
+    la.key_dim = nk * dk; la.C = 2 * nk * dk + nv * dv;
+    deltanet_decode_kernel<true><<<(unsigned)((int64_t)B * nv), 512, 0, (hipStream_t)stream>>>(a, la);
+    return check_launch("deltanet_decode_layer");
 }

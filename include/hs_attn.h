@@ -377,6 +377,19 @@ HS_API int hs_deltanet_prepare(const void *mixed_qkv, const void *conv_weight, c
                                int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv, hs_stream_t stream);
 HS_API int hs_deltanet_gated_norm(const float *x, const void *z, const float *weight, float eps, void *out,
                                   int64_t rows, int32_t D, hs_stream_t stream);
+/* The decode branch of GatedDeltaNetLayer::forward between the two projections as ONE launch (qwen3_5.rs:629-686 conv1d
+ * + SiLU + gates for the new token, :725-751 the recurrent step with L2-normalised q and k, :305-313 RMSNormGated):
+ * hs_deltanet_prepare (S = 1) + hs_deltanet_forward (T = 1) + hs_deltanet_gated_norm, with the arguments of those
+ * calls and their results bit for bit (conv_state_out, state, out; for 16-byte aligned buffers, the case those calls
+ * serve with their wide kernels), but q, k, v, g, beta and the fp32 output row never leave the chip.
+ *   mixed_qkv [B, 1, 2*nk*dk + nv*dv] bf16;  conv_state_in [B, C, 3] bf16 or NULL;  conv_state_out a different buffer;
+ *   a_in, b_in [B, 1, nv] bf16;  z [B, 1, nv, dv] bf16;  norm_weight [dv] fp32;  state [B, nv, dk, dv] fp32 in place;
+ *   out [B, 1, nv, dv] bf16.  dk = dv = 128. */
+HS_API int hs_deltanet_decode_layer(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in,
+                                    void *conv_state_out, const void *a_in, const void *b_in, const float *neg_a_exp,
+                                    const float *dt_bias, const void *z, const float *norm_weight, float norm_eps,
+                                    float *state, void *out, int32_t B, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
+                                    float q_scale, int l2norm, hs_stream_t stream);
 
 #ifdef __cplusplus
 }
