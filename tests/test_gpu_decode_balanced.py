@@ -175,3 +175,60 @@ def test_paged_cache_with_the_hint():
         d = np.abs(got - want)
         assert d.max() < TOL_MAX and d.mean() < TOL_MEAN
     assert np.abs(outs[0] - outs[1]).max() < 1e-2
+
+
+@pytest.mark.parametrize("D,rd", [(128, 128), (64, 64), (256, 64)])
+def test_decode_step_with_the_prologue_inside_a_hinted_launch(D, rd):
+    """QK-norm + rotation of q and k_new inside the launch (hs_decode_step_int8_prologue) on a ragged batch with the
+    hint: the cache rows written equal those of the unhinted launch bit for bit (the prologue's arithmetic does not
+    depend on the split), the outputs agree like any two splits, and both equal the separate pre-pass
+    (hs_qk_prologue_apply) followed by the plain step."""
+    B, Hq, Hkv, T = 9, 8, 2, 1700
+    case = wl.decode_case(83 + D, B, Hq, Hkv, D, T, ragged=True, min_len=2)
+    case["seq_lens"][1] = T
+    lens_np = case["seq_lens"]
+    lens = torch.from_numpy(lens_np).to(DEV)
+    r = wl.philox(900 + D)
+    q = torch.from_numpy(r.standard_normal((B, Hq, D)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    nk = torch.from_numpy(r.standard_normal((B, 1, Hkv, D)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    nv = torch.from_numpy(r.standard_normal((B, 1, Hkv, D)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    qw = torch.from_numpy(1.0 + 0.1 * r.standard_normal(D).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    kw = torch.from_numpy(1.0 + 0.1 * r.standard_normal(D).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    ang = torch.arange(T, dtype=torch.float32)[:, None] / (10000.0 ** (torch.arange(0, rd, 2, dtype=torch.float32) / rd))[None, :]
+    sin, cos = ang.sin().to(torch.bfloat16).to(DEV).contiguous(), ang.cos().to(torch.bfloat16).to(DEV).contiguous()
+    pro = hb.qk_prologue(hb.QKNORM_LLAMA, 1e-6, qw, kw, sin, cos, rotary_dim=rd)
+    scale = 1.0 / np.sqrt(D)
+
+    def fresh():
+        c = build_cache(case, Hkv, D)
+        for b in range(B):  # the step has to write the last token
+            c.k_codes[b, :, lens_np[b] - 1] = 0
+            c.v_codes[b, :, lens_np[b] - 1] = 0
+            c.k_scales[b, :, lens_np[b] - 1] = 0
+            c.v_scales[b, :, lens_np[b] - 1] = 0
+        return c
+
+    res = []
+    for hint in (0, int(lens_np.sum())):
+        c = fresh()
+        out = torch.full((B, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+        hb.decode_step_prologue(q, nk, nv, pro, c.k_codes, c.v_codes, c.k_scales, c.v_scales, hinted_layout(c, D, hint), lens,
+                                out, ws, Hkv, T, scale)
+        torch.cuda.synchronize()
+        res.append((out.float().cpu().numpy(), c))
+    (o0, c0), (o1, c1) = res
+    assert torch.equal(c0.k_codes, c1.k_codes) and torch.equal(c0.v_codes, c1.v_codes)
+    assert torch.equal(c0.k_scales, c1.k_scales) and torch.equal(c0.v_scales, c1.v_scales)
+    assert np.isfinite(o1).all() and np.abs(o0 - o1).max() < 1e-2
+    # the pre-pass + the plain hinted step: the same rows in the cache, outputs bit for bit (same split, same q)
+    c2 = fresh()
+    q_rot, k_rot = torch.empty(B, 1, Hq, D, dtype=torch.bfloat16, device=DEV), torch.empty_like(nk)
+    hb.qk_prologue_apply(q.view(B, 1, Hq, D), nk, pro, q_rot, k_rot, (lens - 1).to(torch.int32).contiguous(), 0)
+    out2 = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_step(q_rot.view(B, Hq, D).contiguous(), k_rot, nv, c2.k_codes, c2.v_codes, c2.k_scales, c2.v_scales,
+                   hinted_layout(c2, D, int(lens_np.sum())), lens, out2, ws, Hkv, T, scale)
+    torch.cuda.synchronize()
+    assert torch.equal(c2.k_codes, c1.k_codes) and torch.equal(c2.k_scales, c1.k_scales)
+    assert np.array_equal(out2.float().cpu().numpy(), o1)
