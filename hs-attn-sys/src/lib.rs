@@ -188,6 +188,23 @@ pub unsafe fn deltanet_forward_gpu(q: *const c_void, k: *const c_void, v: *const
     check(bindings::hs_deltanet_forward(q, k, v, g, beta, state, out, b, t, nk, nv, dk, dv, q_scale, l2norm as c_int, stream))
 }
 
+/// chunked_delta_rule (qwen3_5.rs:342-498) followed by RMSNormGated (qwen3_5.rs:305-313) without the fp32 tensor
+/// between them: `out` is the bf16 normed tensor.  The scan is a cooperative launch (not capturable in a HIP graph).
+///
+/// # Safety
+/// As above; `workspace` holds at least `hs_deltanet_chunked_workspace_bytes(b, t, nk, nv)` bytes.
+#[allow(clippy::too_many_arguments)]
+pub unsafe fn deltanet_forward_chunked_gated_norm_gpu(q: *const c_void, k: *const c_void, v: *const c_void, g: *const f32,
+                                                      beta: *const f32, state: *mut f32, z: *const c_void,
+                                                      norm_weight: *const f32, norm_eps: f32, out: *mut c_void, b: i32, t: i32,
+                                                      nk: i32, nv: i32, dk: i32, dv: i32, q_scale: f32, l2norm: bool,
+                                                      workspace: *mut c_void, workspace_bytes: usize,
+                                                      stream: hs_stream_t) -> Result<()> {
+    check(bindings::hs_deltanet_forward_chunked_gated_norm(q, k, v, g, beta, state, z, norm_weight, norm_eps, out, b, t, nk, nv,
+                                                           dk, dv, q_scale, l2norm as c_int, workspace, workspace_bytes,
+                                                           stream))
+}
+
 /// One decode step of a gated-DeltaNet layer between its projections in a single launch (conv1d + SiLU + gates,
 /// the recurrent step, RMSNormGated: GatedDeltaNetLayer::forward, qwen3_5.rs:629-786 with seq == 1).
 ///

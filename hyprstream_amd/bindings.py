@@ -26,7 +26,7 @@ EXPORTS = [
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
     "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue",
-    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
+    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_deltanet_forward_chunked_gated_norm", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
 
@@ -342,6 +342,24 @@ def deltanet_forward_chunked(q, k, v, g, beta, state, out, q_scale, l2norm=False
     check(lib().hs_deltanet_forward_chunked(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(out),
                                             B, T, nk, nv, dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)),
                                             _ptr(workspace), ctypes.c_size_t(workspace.numel()), _stream()))
+    return workspace
+
+
+def deltanet_forward_chunked_gated_norm(q, k, v, g, beta, state, z, norm_weight, eps, out, q_scale, l2norm=False, workspace=None):
+    """deltanet_forward_chunked with the gated RMSNorm in the epilogue: out bf16 [B, T, nv, dv]."""
+    import torch
+    B, T, nk, dk = q.shape
+    nv, dv = v.shape[2], v.shape[3]
+    for t in (q, k, v, g, beta, state, z, out):
+        assert t.is_contiguous()
+    lib().hs_deltanet_chunked_workspace_bytes.restype = ctypes.c_size_t
+    need = lib().hs_deltanet_chunked_workspace_bytes(B, T, nk, nv)
+    if workspace is None:
+        workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
+    check(lib().hs_deltanet_forward_chunked_gated_norm(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(z),
+                                                       _ptr(norm_weight), ctypes.c_float(eps), _ptr(out), B, T, nk, nv, dk, dv,
+                                                       ctypes.c_float(q_scale), int(bool(l2norm)), _ptr(workspace),
+                                                       ctypes.c_size_t(workspace.numel()), _stream()))
     return workspace
 
 

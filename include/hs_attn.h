@@ -348,13 +348,25 @@ HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, cons
  * everything else is fp16-operand / fp32-accumulate MFMA.  Mathematically identical to hs_deltanet_forward; outputs
  * and the final state differ from it by rounding (about 1e-3 relative).  Arguments as hs_deltanet_forward, plus a
  * device workspace of hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) bytes (per 64-token chunk: 32,768 per
- * (sequence, k-head) and 41,728 per (sequence, v-head)), 16-byte aligned, owned by the caller; q, k, v must be
+ * (sequence, k-head) and 42,240 per (sequence, v-head)), 16-byte aligned, owned by the caller; q, k, v must be
  * 16-byte aligned.  A prompt split into calls of a multiple
  * of 64 tokens (state carried through `state`) gives the bits of one call. */
 HS_API size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv);
 HS_API int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, const float *g, const float *beta,
                         float *state, float *out,
                         int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
+                        float q_scale, int l2norm, void *workspace, size_t workspace_bytes, hs_stream_t stream);
+/* hs_deltanet_forward_chunked with the layer's gated RMSNorm (RMSNormGated::forward, qwen3_5.rs:305-313; what
+ * hs_deltanet_gated_norm computes) in the epilogue: out [B, T, nv, dv] bf16 = bf16(o * rsqrt(mean(o^2) + eps) * weight *
+ * silu(z)) with z [B, T, nv, dv] bf16 and weight [dv] fp32; the fp32 rows o are never written.  Same workspace.  Equal
+ * to the two calls up to the order in which a row's squares are added (one bf16 ulp, rarely).  The two workgroups that
+ * share a row exchange their sums through the workspace, so the scan is a cooperative launch (all its workgroups
+ * resident; several launches when the batch needs more than the device holds): not capturable in a HIP graph, and
+ * HS_ERR_LAUNCH where the device has no cooperative launches, HS_ERR_INVALID_ARGUMENT when 2 * nv workgroups do not
+ * fit the device at once -- run the two calls then. */
+HS_API int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const void *v, const float *g,
+                        const float *beta, float *state, const void *z, const float *norm_weight, float norm_eps,
+                        void *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
                         float q_scale, int l2norm, void *workspace, size_t workspace_bytes, hs_stream_t stream);
 
 /* ---- the elementwise steps of a gated-DeltaNet layer around the delta rule ("next" of hs_deltanet_forward) ----
