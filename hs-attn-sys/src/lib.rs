@@ -205,6 +205,23 @@ pub unsafe fn deltanet_forward_chunked_gated_norm_gpu(q: *const c_void, k: *cons
                                                            stream))
 }
 
+/// The prompt branch of a gated-DeltaNet layer between its projections in one call (conv1d + SiLU + gates, the chunked
+/// delta rule, RMSNormGated: GatedDeltaNetLayer::forward, qwen3_5.rs:629-786 with seq > 1).
+///
+/// # Safety
+/// As above; `workspace` holds at least `hs_deltanet_prefill_layer_workspace_bytes(..)` bytes, 256-byte aligned.
+#[allow(clippy::too_many_arguments)]
+pub unsafe fn deltanet_prefill_layer_gpu(mixed_qkv: *const c_void, conv_weight: *const c_void, conv_state_in: *const c_void,
+                                         conv_state_out: *mut c_void, a_in: *const c_void, b_in: *const c_void,
+                                         neg_a_exp: *const f32, dt_bias: *const f32, z: *const c_void, norm_weight: *const f32,
+                                         norm_eps: f32, state: *mut f32, out: *mut c_void, b: i32, s: i32, nk: i32, nv: i32,
+                                         dk: i32, dv: i32, q_scale: f32, l2norm: bool, workspace: *mut c_void,
+                                         workspace_bytes: usize, stream: hs_stream_t) -> Result<()> {
+    check(bindings::hs_deltanet_prefill_layer(mixed_qkv, conv_weight, conv_state_in, conv_state_out, a_in, b_in, neg_a_exp,
+                                              dt_bias, z, norm_weight, norm_eps, state, out, b, s, nk, nv, dk, dv, q_scale,
+                                              l2norm as c_int, workspace, workspace_bytes, stream))
+}
+
 /// One decode step of a gated-DeltaNet layer between its projections in a single launch (conv1d + SiLU + gates,
 /// the recurrent step, RMSNormGated: GatedDeltaNetLayer::forward, qwen3_5.rs:629-786 with seq == 1).
 ///

@@ -26,7 +26,7 @@ EXPORTS = [
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
     "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue",
-    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_deltanet_forward_chunked_gated_norm", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
+    "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_deltanet_forward_chunked_gated_norm", "hs_deltanet_prefill_layer", "hs_deltanet_prefill_layer_workspace_bytes", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
 
@@ -398,6 +398,28 @@ def deltanet_decode_layer(mixed_qkv, conv_weight, conv_state_in, a_in, b_in, neg
                                          ctypes.c_float(eps), _ptr(state), _ptr(out), B, nk, nv, dk, dv,
                                          ctypes.c_float(q_scale), int(bool(l2norm)), _stream()))
     return out, conv_state_out
+
+
+def deltanet_prefill_layer(mixed_qkv, conv_weight, conv_state_in, a_in, b_in, neg_a_exp, dt_bias, z, norm_weight, eps,
+                           state, nk, nv, dk, dv, q_scale, l2norm=True, workspace=None):
+    """The prompt branch of a gated-DeltaNet layer between its projections in one call.  `state` is updated in place.
+    Returns (out bf16 [B, S, nv, dv], new_conv_state, workspace)."""
+    import torch
+    B, S, C = mixed_qkv.shape
+    assert C == 2 * nk * dk + nv * dv and mixed_qkv.is_contiguous() and conv_weight.is_contiguous() and z.is_contiguous()
+    dev = mixed_qkv.device
+    lib().hs_deltanet_prefill_layer_workspace_bytes.restype = ctypes.c_size_t
+    need = lib().hs_deltanet_prefill_layer_workspace_bytes(B, S, nk, nv, dk, dv)
+    if workspace is None:
+        workspace = torch.empty(max(need, 256), dtype=torch.uint8, device=dev)
+    out = torch.empty(B, S, nv, dv, dtype=torch.bfloat16, device=dev)
+    conv_state_out = torch.empty(B, C, 3, dtype=torch.bfloat16, device=dev)
+    check(lib().hs_deltanet_prefill_layer(_ptr(mixed_qkv), _ptr(conv_weight), _ptr(conv_state_in), _ptr(conv_state_out),
+                                          _ptr(a_in.contiguous()), _ptr(b_in.contiguous()), _ptr(neg_a_exp), _ptr(dt_bias),
+                                          _ptr(z), _ptr(norm_weight), ctypes.c_float(eps), _ptr(state), _ptr(out), B, S, nk, nv,
+                                          dk, dv, ctypes.c_float(q_scale), int(bool(l2norm)), _ptr(workspace),
+                                          ctypes.c_size_t(workspace.numel()), _stream()))
+    return out, conv_state_out, workspace
 
 
 def deltanet_gated_norm(x, z, weight, eps):

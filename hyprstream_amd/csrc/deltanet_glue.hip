@@ -275,4 +275,43 @@ int hs_deltanet_gated_norm(const float *x, const void *z, const float *weight, f
     return check_launch("gated_rmsnorm");
 }
 
+// The prompt branch of the layer as one call: three launches in a row, the intermediate tensors in the workspace.
+static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+size_t hs_deltanet_prefill_layer_workspace_bytes(int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv) {
+    if (B <= 0 || S <= 0 || nk <= 0 || nv <= 0 || dk <= 0 || dv <= 0) return 0;
+    const size_t bs = (size_t)B * S;
+    return align256(hs_deltanet_chunked_workspace_bytes(B, S, nk, nv)) + 2 * align256(bs * nk * dk * 2) + align256(bs * nv * dv * 2) +
+           2 * align256(bs * nv * 4);
+}
+
+int hs_deltanet_prefill_layer(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in, void *conv_state_out,
+                              const void *a_in, const void *b_in, const float *neg_a_exp, const float *dt_bias, const void *z,
+                              const float *norm_weight, float norm_eps, float *state, void *out, int32_t B, int32_t S,
+                              int32_t nk, int32_t nv, int32_t dk, int32_t dv, float q_scale, int l2norm, void *workspace,
+                              size_t workspace_bytes, hs_stream_t stream) {
+    using namespace hs;
+    if (B < 0 || S < 0 || nk <= 0 || nv <= 0 || dk <= 0 || dv <= 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d S=%d nk=%d nv=%d dk=%d dv=%d", B, S, nk, nv, dk, dv);
+    if (B == 0 || S == 0) return HS_OK;
+    const size_t need = hs_deltanet_prefill_layer_workspace_bytes(B, S, nk, nv, dk, dv);
+    if (!workspace || workspace_bytes < need) return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
+    if (((uintptr_t)workspace & 255) != 0) return fail(HS_ERR_INVALID_ARGUMENT, "workspace must be 256-byte aligned");
+    const size_t bs = (size_t)B * S;
+    uint8_t *p = (uint8_t *)workspace;
+    void *chunk_ws = p;
+    const size_t chunk_bytes = hs_deltanet_chunked_workspace_bytes(B, S, nk, nv);
+    p += align256(chunk_bytes);
+    void *q = p; p += align256(bs * nk * dk * 2);
+    void *k = p; p += align256(bs * nk * dk * 2);
+    void *v = p; p += align256(bs * nv * dv * 2);
+    float *g = (float *)p; p += align256(bs * nv * 4);
+    float *beta = (float *)p;
+    if (int rc = hs_deltanet_prepare(mixed_qkv, conv_weight, conv_state_in, conv_state_out, a_in, b_in, neg_a_exp, dt_bias, q, k, v,
+                                     g, beta, B, S, nk, nv, dk, dv, stream))
+        return rc;
+    return hs_deltanet_forward_chunked_gated_norm(q, k, v, g, beta, state, z, norm_weight, norm_eps, out, B, S, nk, nv, dk, dv,
+                                                  q_scale, l2norm, chunk_ws, chunk_bytes, stream);
+}
+
 }  // extern "C"

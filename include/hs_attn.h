@@ -403,6 +403,19 @@ HS_API int hs_deltanet_decode_layer(const void *mixed_qkv, const void *conv_weig
                                     float *state, void *out, int32_t B, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
                                     float q_scale, int l2norm, hs_stream_t stream);
 
+/* The prompt branch of GatedDeltaNetLayer::forward between the two projections as ONE call (qwen3_5.rs:629-686, :753-769,
+ * :771-786): hs_deltanet_prepare + hs_deltanet_forward_chunked_gated_norm, three launches in a row with q, k, v, g, beta
+ * and the chunk operands in the workspace (hs_deltanet_prefill_layer_workspace_bytes, 256-byte aligned); arguments and
+ * results as those calls (mixed_qkv [B, S, C], z and out [B, S, nv, dv] bf16), limits as
+ * hs_deltanet_forward_chunked_gated_norm.  The counterpart of hs_deltanet_decode_layer for seq > 1. */
+HS_API size_t hs_deltanet_prefill_layer_workspace_bytes(int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv);
+HS_API int hs_deltanet_prefill_layer(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in,
+                                     void *conv_state_out, const void *a_in, const void *b_in, const float *neg_a_exp,
+                                     const float *dt_bias, const void *z, const float *norm_weight, float norm_eps,
+                                     float *state, void *out, int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk,
+                                     int32_t dv, float q_scale, int l2norm, void *workspace, size_t workspace_bytes,
+                                     hs_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -2,6 +2,8 @@
 (chunked_delta_rule qwen3_5.rs:342-498 + RMSNormGated :305-313), against the two calls it replaces
 (hs_deltanet_forward_chunked + hs_deltanet_gated_norm: same state bit for bit, rows within one bf16 ulp -- only the
 order in which a row's squares are added differs) and against the CPU oracle (fp64 recurrence, then the norm)."""
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -82,3 +84,69 @@ def test_against_the_oracle():
     # the rows are O(1) after the norm; the chunked form's 1e-3 relative error in o carries over, plus bf16 rounding
     assert (err - 2.0 ** -7 * np.abs(want)).max() < 2e-2 and err.mean() < 2e-3
     assert np.abs(st_b.cpu().numpy() - ws).max() <= 3e-3 * np.abs(ws).max()
+
+
+def test_prefill_layer_is_prepare_plus_the_fused_scan_and_carries_state_across_calls():
+    """hs_deltanet_prefill_layer (one call for the prompt branch of the layer) against hs_deltanet_prepare +
+    hs_deltanet_forward_chunked_gated_norm, bit for bit, for a prompt given in two calls of 128 and 70 tokens with the
+    conv state and the recurrent state carried; and against the reference's op sequence for the whole run."""
+    from oracle import reference_path as ref
+    B, nk, nv, dk, dv, S = 2, 2, 4, 128, 128, 198
+    r = wl.philox(9400)
+    C = 2 * nk * dk + nv * dv
+    t = lambda *s, scale=1.0: torch.from_numpy((r.standard_normal(s) * scale).astype(np.float32))
+    p = dict(x=t(B, S, C).to(torch.bfloat16), w=t(C, 4, scale=0.5).to(torch.bfloat16), st=t(B, C, 3).to(torch.bfloat16),
+             a=t(B, S, nv, scale=2).to(torch.bfloat16), b=t(B, S, nv, scale=2).to(torch.bfloat16), nae=-t(nv).exp(), dtb=t(nv),
+             z=t(B, S, nv, dv).to(torch.bfloat16), nw=t(dv))
+    d = {k_: v_.to(DEV) for k_, v_ in p.items()}
+    qs = 1.0 / np.sqrt(dk)
+    state_a, state_b = torch.zeros(B, nv, dk, dv, device=DEV), torch.zeros(B, nv, dk, dv, device=DEV)
+    cs_a = cs_b = d["st"]
+    outs_a, outs_b = [], []
+    for lo, hi in ((0, 128), (128, S)):
+        sl = slice(lo, hi)
+        x, a_in, b_in, z = (d[n][:, sl].contiguous() for n in ("x", "a", "b", "z"))
+        y, cs_a, _ = hb.deltanet_prefill_layer(x, d["w"], cs_a, a_in, b_in, d["nae"], d["dtb"], z, d["nw"], 1e-6, state_a,
+                                               nk, nv, dk, dv, qs, True)
+        outs_a.append(y)
+        q, k, v, g, beta, cs_b = hb.deltanet_prepare(x, d["w"], cs_b, a_in, b_in, d["nae"], d["dtb"], nk, nv, dk, dv)
+        y2 = torch.empty(B, hi - lo, nv, dv, dtype=torch.bfloat16, device=DEV)
+        hb.deltanet_forward_chunked_gated_norm(q, k, v, g, beta, state_b, z, d["nw"], 1e-6, y2, qs, True)
+        outs_b.append(y2)
+    torch.cuda.synchronize()
+    ya, yb = torch.cat(outs_a, 1), torch.cat(outs_b, 1)
+    assert torch.equal(ya.view(torch.int16), yb.view(torch.int16)) and torch.equal(state_a, state_b)
+    assert torch.equal(cs_a.view(torch.int16), cs_b.view(torch.int16))
+    # the reference's ops over the whole run (GatedDeltaNetLayer::forward, qwen3_5.rs:629-786, recurrence iterated)
+    conv, ref_cs, rg, rb = ref.deltanet_prepare(p["x"], p["w"].unsqueeze(1), p["st"], p["a"], p["b"], p["nae"], p["dtb"])
+    kd = nk * dk
+    l2 = lambda t_: t_ / t_.norm(dim=-1, keepdim=True).clamp_min(1e-3)
+    rq = l2(conv[..., :kd].reshape(B, S, nk, dk).float()) * qs
+    rk = l2(conv[..., kd:2 * kd].reshape(B, S, nk, dk).float())
+    rv = conv[..., 2 * kd:].reshape(B, S, nv, dv).float()
+    rq, rk = rq.repeat_interleave(nv // nk, 2), rk.repeat_interleave(nv // nk, 2)
+    st = torch.zeros(B, nv, dk, dv)
+    rows = []
+    for i in range(S):
+        ot, st = ref.deltanet_decode_step(rq[:, i], rk[:, i], rv[:, i], rg[:, i], rb[:, i], st)
+        rows.append(ot)
+    want = ref.gated_rmsnorm(torch.stack(rows, 1), p["z"], p["nw"], 1e-6)
+    err = (ya.float().cpu() - want.float()).abs()
+    assert (err - 2.0 ** -7 * want.float().abs()).max() < 3e-2 and err.mean() < 2e-3
+    assert (state_a.cpu() - st).abs().max() < 3e-3 * float(st.abs().max())
+    assert torch.equal(cs_a.cpu().view(torch.int16), ref_cs.contiguous().view(torch.int16))
+
+
+def test_prefill_layer_workspace_is_checked():
+    L = hb.lib()
+    L.hs_deltanet_prefill_layer_workspace_bytes.restype = ctypes.c_size_t
+    need = L.hs_deltanet_prefill_layer_workspace_bytes(1, 64, 1, 1, 128, 128)
+    assert need >= hb.deltanet_chunked_workspace_bytes(1, 64, 1, 1) + 64 * (3 * 128 * 2 + 2 * 4) and need % 256 == 0
+    x = torch.zeros(1, 64, 384, dtype=torch.bfloat16, device=DEV)
+    f = torch.zeros(128 * 128, device=DEV)
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    p = hb._ptr
+    st = torch.zeros(1, 384, 3, dtype=torch.bfloat16, device=DEV)
+    rc = L.hs_deltanet_prefill_layer(p(x), p(x), None, p(st), p(x), p(x), p(f), p(f), p(x), p(f), ctypes.c_float(1e-6), p(f), p(x),
+                                     1, 64, 1, 1, 128, 128, ctypes.c_float(1.0), 1, p(ws), ctypes.c_size_t(need - 1), None)
+    assert rc == hb.HS_ERR_WORKSPACE
