@@ -64,6 +64,7 @@ pub fn contiguous_layout(hkv: i32, capacity_tokens: i32, d: i32) -> hs_kv_layout
         total_tokens_hint: 0,
         prefill_columns_hint: 0,
         prefill_window: 0,
+        out_gate: std::ptr::null(),
     }
 }
 

@@ -44,6 +44,7 @@ class KvLayout(ctypes.Structure):
         ("total_tokens_hint", ctypes.c_int64),
         ("prefill_columns_hint", ctypes.c_int32),
         ("prefill_window", ctypes.c_int32),
+        ("out_gate", ctypes.c_void_p),
     ]
 
 

@@ -68,6 +68,15 @@ __device__ __forceinline__ bool resolve(const KvAddr &a, int b, int t, int64_t &
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f);
+// The attention output as bf16, times the output gate when there is one (Qwen3.5 full-attention layers,
+// qwen3_5.rs:1056-1059: ctx * gate.sigmoid() on bf16 tensors -- the sigmoid is rounded to bf16, then the product).
+__device__ __forceinline__ uint32_t gated_bf16_bits(float attn, const uint16_t *gate, int64_t i) {
+    const uint32_t o = f32_to_bf16_bits(attn);
+    if (gate == nullptr) return o;
+    const float sg = bf16_bits_to_f32(f32_to_bf16_bits(1.0f / (1.0f + expf(-bf16_bits_to_f32(gate[i])))));
+    return f32_to_bf16_bits(bf16_bits_to_f32(o) * sg);
+}
 
 // fp32 -> bf16 bits, round-to-nearest-even (NaN stays a quiet NaN): gfx950's conversion instruction.  Compared on the
 // device with the integer formulation ((u + 0x7fff + ((u >> 16) & 1)) >> 16, NaN -> (u >> 16) | 0x40, which is what

@@ -103,6 +103,7 @@ struct DecodeArgs {
     float *part_o;   // [B, Hq, nchunks, D]
     float *part_ml;  // [B, Hq, nchunks, 2]   (m in log2 units, l)
     uint16_t *out;       // [B, Hq, D] bf16
+    const uint16_t *out_gate;  // optional [B, Hq, D] bf16: out = bf16(bf16(attention) * bf16(sigmoid(gate)))
     QuantArgs nt;        // the step's new token (nt.src[0] == nullptr: none); position = seq_len - 1
     int32_t direct;      // 1: single chunk, write `out` directly; 0: leave partials in the workspace
     int32_t B, Hq, Hkv, G, chunk_tokens, nchunks, max_seq_len;
@@ -569,7 +570,8 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a_in) {
                     o += sm_o[w][g][d];
                     l += sm_m[w][g] == -INFINITY ? 0.0f : sm_l[w][g] * __builtin_amdgcn_exp2f(sm_m[w][g] - Mg);
                 }
-                a.out[((int64_t)b * a.Hq + h * G + g) * kD + CW * c + d] = (uint16_t)f32_to_bf16_bits(o * out_scale / l);
+                const int64_t oi = ((int64_t)b * a.Hq + h * G + g) * kD + CW * c + d;
+                a.out[oi] = (uint16_t)gated_bf16_bits(o * out_scale / l, a.out_gate, oi);
             }
         } else {
             for (int idx = threadIdx.x; idx < G * CW; idx += 256) {
@@ -680,7 +682,7 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a_in) {
 // sequence (up to 128 chunks) are read by many lanes at once instead of one after the other; the chunk lanes meet
 // in LDS.  D is 64, 128 or 256.
 __global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, const float *part_ml,
-                                                          const int32_t *seq_lens, uint16_t *out, int Hq, int nchunks,
+                                                          const int32_t *seq_lens, uint16_t *out, const uint16_t *out_gate, int Hq, int nchunks,
                                                           int chunk_tokens, int max_seq_len, int kD, int B, int pieces,
                                                           int min_granules) {
     const int hq = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
@@ -744,7 +746,8 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, 
             os += sm_o[y * kD + tid];
             ls += sm_l[y];
         }
-        out[((int64_t)b * Hq + hq) * kD + tid] = (uint16_t)f32_to_bf16_bits(n > 0 ? os / ls : 0.0f);
+        const int64_t oi = ((int64_t)b * Hq + hq) * kD + tid;
+        out[oi] = (uint16_t)gated_bf16_bits(n > 0 ? os / ls : 0.0f, out_gate, oi);
     }
 }
 
@@ -864,6 +867,7 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.part_o = (float *)ws;
     a.part_ml = a.part_o + (size_t)B * Hq * a.nchunks * D;
     a.out = (uint16_t *)out;
+    a.out_gate = (const uint16_t *)l->out_gate;
     a.scale_log2e = softmax_scale * kLog2e;
     a.direct = (phases == 3 && a.nchunks == 1) ? 1 : 0;
     a.nt.src[0] = nt.k_src; a.nt.src[1] = nt.v_src;
@@ -911,7 +915,7 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
         if (int rc = check_launch("decode_attn")) return rc;
     }
     if ((phases & 2) && !a.direct) {
-        decode_merge_kernel<<<dim3(Hq, B), 256, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, Hq,
+        decode_merge_kernel<<<dim3(Hq, B), 256, 0, stream>>>(a.part_o, a.part_ml, seq_lens, (uint16_t *)out, a.out_gate, Hq,
                                                                a.nchunks, a.chunk_tokens, max_seq_len, D, B,
                                                                a.balanced ? a.pieces : 0, a.min_granules);
         return check_launch("decode_merge");

@@ -61,6 +61,7 @@ struct PrefillArgs {
     const float *ks, *vs;
     KvAddr ka, va;
     uint16_t *out;  // [B,S,Hq,D] bf16
+    const uint16_t *out_gate;  // optional [B,S,Hq,D] bf16: out = bf16(bf16(attention) * bf16(sigmoid(gate)))
     int32_t B, S, Hq, Hkv, G, HG, hist_len;
     const int32_t *hist_lens;  // optional, device [B]: cached tokens per sequence (then hist_len is their upper bound)
     int32_t heavy_first;  // the grid outnumbers the CUs: order the query tiles by decreasing work
@@ -805,6 +806,14 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         if (qi[nb] >= S || hg * a.HG + (kNB * wave + nb) % a.HG >= a.G) continue;  // padding columns write nothing
         const float inv = 1.0f / l;
         uint16_t *op = a.out + (((int64_t)b * S + qi[nb]) * a.Hq + head[nb]) * kRow + 4 * VBG * lq;
+        const uint16_t *gp = a.out_gate ? a.out_gate + (op - a.out) : nullptr;  // the output gate's elements of this lane
+        auto gate2 = [](uint32_t o2, uint32_t g2) {  // two bf16 outputs times the bf16-rounded sigmoid of two bf16 gates
+            auto one = [](uint32_t o, uint32_t g) {
+                const float sg = bf16_bits_to_f32(f32_to_bf16_bits(1.0f / (1.0f + expf(-bf16_bits_to_f32(g)))));
+                return f32_to_bf16_bits(bf16_bits_to_f32(o) * sg);
+            };
+            return one(o2 & 0xffffu, g2 & 0xffffu) | (one(o2 >> 16, g2 >> 16) << 16);
+        };
 #pragma unroll
         for (int c = 0; c < NC; ++c)
 #pragma unroll
@@ -812,6 +821,10 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 uint32_t w[VBG / 2];
 #pragma unroll
                 for (int e = 0; e < VBG / 2; ++e) w[e] = pack_bf16x2(acc[nb][VBG * c + 2 * e][r] * inv, acc[nb][VBG * c + 2 * e + 1][r] * inv);
+                if (gp != nullptr) {
+#pragma unroll
+                    for (int e = 0; e < VBG / 2; ++e) w[e] = gate2(w[e], *(const uint32_t *)(gp + DW * c + VBG * r + 2 * e));
+                }
                 if constexpr (VBG == 8) *(u32x4 *)(op + DW * c + VBG * r) = (u32x4){w[0], w[1], w[2], w[3]};
                 else *(u32x2 *)(op + DW * c + VBG * r) = (u32x2){w[0], w[1]};
             }
@@ -947,6 +960,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.ks = k_scales; a.vs = v_scales;
     a.ka = make_addr(*layout, 0); a.va = make_addr(*layout, 1);
     a.out = (uint16_t *)out;
+    a.out_gate = (const uint16_t *)layout->out_gate;
     a.B = B; a.S = S; a.Hq = Hq; a.Hkv = Hkv; a.G = G; a.hist_len = hist_len;
     a.hist_lens = hist_lens;
     a.write_new = quantize_on_write ? 1 : 0;

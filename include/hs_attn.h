@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define HS_ATTN_ABI_VERSION 4
+#define HS_ATTN_ABI_VERSION 5
 
 typedef void *hs_stream_t; /* hipStream_t */
 
@@ -89,6 +89,10 @@ typedef struct hs_kv_layout {
                                    empty cache this is the reference's mask; with history it is the same rule on
                                    absolute positions (the reference's [q_len, q_len] mask has no meaning there).
                                    Decode entry points ignore it, as the reference applies no window at q_len == 1. */
+    const void *out_gate;       /* attention calls, optional: bf16, device, the shape of `out`.  The output gate of the
+                                   Qwen3.5 full-attention layers (qwen3_5.rs:1056-1059: ctx * sigmoid(gate) in the model
+                                   dtype): out = bf16(bf16(attention) * bf16(sigmoid(gate))) written by the same launch.
+                                   NULL = none. */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */

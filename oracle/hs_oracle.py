@@ -257,3 +257,16 @@ def gated_rmsnorm(x, z_bits, w, eps):
     lib().orc_gated_rmsnorm(_p(x), _p(z), _p(_c(w, np.float32)), ctypes.c_float(eps), ctypes.c_int64(x.size // D), D, _p(out))
     return out
 
+
+
+def output_gate_bf16(attn, gate_bits):
+    """The output gate of the Qwen3.5 full-attention layers (qwen3_5.rs:1056-1059: ctx_flat * gate.sigmoid() on tensors
+    of the model dtype): the attention output rounded to bf16, the sigmoid of the bf16 gate computed in fp32 and
+    rounded to bf16, their product rounded to bf16.  attn fp32 (any shape), gate_bits uint16 of the same shape;
+    returns bf16 bits."""
+    o = bf16_to_f32(f32_to_bf16(np.asarray(attn, np.float32)))
+    g = bf16_to_f32(np.asarray(gate_bits, np.uint16))
+    with np.errstate(over="ignore"):
+        sg = (np.float32(1.0) / (np.float32(1.0) + np.exp(-g, dtype=np.float32))).astype(np.float32)
+    sg = bf16_to_f32(f32_to_bf16(sg))
+    return f32_to_bf16((o * sg).astype(np.float32))

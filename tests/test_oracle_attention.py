@@ -199,3 +199,25 @@ def test_window_with_history_is_attention_over_the_last_window_keys():
         want = oracle.prefill_attn(q[:, i:i + 1], k[:, lo:p + 1], v[:, lo:p + 1], None, None, oracle.FMT_DENSE,
                                    np.array([p + 1 - lo], np.int32), 0.125)
         assert np.abs(got[:, i] - want[:, 0]).max() < 1e-6
+
+
+def test_output_gate_matches_the_libtorch_ops_of_the_qwen35_layer():
+    """ctx * gate.sigmoid() on bf16 tensors (qwen3_5.rs:1056-1059), live: the oracle's restatement gives libtorch's bits
+    except where libm's and libtorch's exp differ in the last fp32 bit and that flips a bf16 rounding (rare, one ulp);
+    closed forms: gate 0 halves the output exactly, a large gate leaves it, a very negative one gives a signed zero."""
+    r = np.random.Generator(np.random.Philox(4242))
+    ctx = (r.standard_normal((7, 5, 128)) * 2).astype(np.float32)
+    gate = torch.from_numpy((r.standard_normal((7, 5, 128)) * 3).astype(np.float32)).to(torch.bfloat16)
+    gate_bits = gate.view(torch.int16).numpy().view(np.uint16)
+    got = oracle.output_gate_bf16(ctx, gate_bits)
+    want = (torch.from_numpy(ctx).to(torch.bfloat16) * gate.sigmoid()).view(torch.int16).numpy().view(np.uint16)
+    key = lambda u: np.where(u.astype(np.int32) & 0x8000, -(u.astype(np.int32) & 0x7fff), u.astype(np.int32) & 0x7fff)
+    d = np.abs(key(got) - key(want))
+    assert d.max() <= 1 and (d != 0).mean() < 2e-3
+    o = np.array([1.5, -3.0, 0.25], np.float32)
+    z = np.zeros(3, np.uint16)
+    assert np.array_equal(oracle.bf16_to_f32(oracle.output_gate_bf16(o, z)), o * 0.5)
+    big = oracle.f32_to_bf16(np.full(3, 40.0, np.float32))
+    assert np.array_equal(oracle.bf16_to_f32(oracle.output_gate_bf16(o, big)), o)
+    neg = oracle.f32_to_bf16(np.full(3, -200.0, np.float32))
+    assert np.all(oracle.bf16_to_f32(oracle.output_gate_bf16(o, neg)) == 0.0)
