@@ -55,9 +55,11 @@ constexpr int kOffU = 24576;     // U       accumulator tiles [token tile 4][dv 
 constexpr int kOffEG = 40960;    // exp(G_t), 64 floats
 constexpr int kOffEGl = 41216;   // exp(G_63 - G_t), 64 floats
 constexpr int kOffDecay = 41472; // exp(G63), one float
-constexpr int kOffSsq = 41728;   // 2 x 64 floats: per column half, the sums of squares of the chunk's output rows over that
-                                 // half's 64 columns (the fused gated norm's exchange between the two halves; -1 = not there yet)
-constexpr int kUnitBytes = 42240;
+constexpr int kUnitBytes = 41728;
+// Behind all chunks' operands, per (chunk, sequence, v-head): 2 x 64 floats -- per column half, the sums of squares of the
+// chunk's output rows over that half's 64 columns (the fused gated norm's exchange between the two halves; -1 = not
+// there yet).  A region of its own: inside the units it changed their stride, and the plain scan ran 7 % slower.
+constexpr int kSsqBytes = 512;
 // The same matrices inside the scan kernel's LDS operand buffer:
 constexpr int kOpsWn = 0, kOpsQh = 16384, kOpsKt = 32768, kOpsQK = 49152, kOpsFac = 57344, kOpsBytes = 57856;
 
@@ -211,8 +213,12 @@ __global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArg
         eGl[lane] = expf(g63 - x);
         be[lane] = bs[lane] * e;
         if (lane == 63) *(float *)(wsu + kOffDecay) = e;
-        *(float *)(wsu + kOffSsq + 4 * lane) = -1.0f;  // both halves' exchange slots: nothing there yet
-        *(float *)(wsu + kOffSsq + 256 + 4 * lane) = -1.0f;
+#ifndef EXP_NOSENT
+        float *ssq = (float *)(a.ws + a.nc * ((int64_t)a.B * a.nk * kHeadBytes + (int64_t)a.B * a.nv * kUnitBytes) +
+                               ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kSsqBytes);
+        ssq[lane] = -1.0f;  // both halves' exchange slots: nothing there yet
+        ssq[64 + lane] = -1.0f;
+#endif
     }
 
     // ---- 3. k k^T (rows i, columns j) and k q^T (rows j, columns i): wavefront w owns row tile w/2, column tiles 2(w%2), +1
@@ -406,305 +412,25 @@ static_assert(kOpsFac == 28 * 128 * 16, "28 16-byte pieces per loader thread");
 // up every barrier of the chunk.  Only U is read by the wavefront that uses it.
 // NORM: the gated RMSNorm of the layer (RMSNormGated, qwen3_5.rs:305-313) in the epilogue -- the output rows leave as
 // bf16(o * rsqrt(mean(o^2) + eps) * w * silu(z)) instead of fp32 o.  A row's 128 columns belong to two workgroups, so
-// each publishes the sums of squares of its 64 columns per chunk (kOffSsq; reset by the prepare kernel) at the start of
+// each publishes the sums of squares of its 64 columns per chunk (the exchange slots; reset by the prepare kernel) at the start of
 // the next chunk and reads the other's a chunk and a half later, long after it was written, so nothing waits.  Until
 // then the rows of a chunk stay in LDS (four chunks deep), and two more wavefronts, which do nothing else, finish
 // them: eight adjacent columns per lane with 16-byte loads of z and 16-byte stores (twelve wavefronts are still three
 // per SIMD, so they cost the others no registers).  The two workgroups must be resident together: the host launches this instance cooperatively (all
 // workgroups of a launch resident) and the wait for the other half is bounded all the same.
+constexpr int kRing = 4;     // chunks of output rows waiting in LDS for the other half's sums
+constexpr int kOPitch = 68;  // floats per staged output row: 64 columns + 4, so the four row groups of a store hit different banks
 constexpr int kNormSpin = 1 << 16;  // about 0.1 s: the other half is resident and at most a chunk apart
-template <bool NORM>
-__global__ __launch_bounds__(NORM ? kScanNormThreads : kScanThreads) void deltanet_chunk_scan_kernel(ChunkArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t ops[kOpsBytes];          // this chunk's A operands and decay vectors
-    __shared__ __attribute__((aligned(16))) uint8_t s_lds[4 * 4 * 64 * 16];  // S:  [dk slab][column tile][lane] 16 B
-    __shared__ __attribute__((aligned(16))) uint8_t v_lds[2 * 4 * 64 * 16];  // V': [token slab][column tile][lane] 16 B
-    constexpr int kOPitch = 68;  // floats per staged output row: 64 columns + 4, so the four row groups of a store hit different banks
-    constexpr int kRing = 4;     // chunks of output rows waiting in LDS for the other half's sums
-    __shared__ float ssq_lds[NORM ? kRing : 1][2][NORM ? 64 : 1];           // [chunk % kRing][column pair][token]
-    __shared__ __attribute__((aligned(16))) float o_lds[NORM ? kRing : 1][NORM ? 64 : 1][NORM ? kOPitch : 4];  // [chunk % kRing][token][column]
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int li = lane & 15, lq = lane >> 4;
-    // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The two column halves of a
-    // (sequence, v-head) read the same -W / masked q k^T, and all v-heads of a k-head (both halves of each) the same q and
-    // k^T: the 2 * rep workgroups of a (sequence, k-head) get linear ids congruent mod 8, consecutive in that XCD's
-    // order, so that each of those operands comes from HBM once and the other readers find it in L2.
-    const int p = blockIdx.x, pairs = a.b_count * a.nv, rep = a.nv / a.nk;
-    int pair, half;
-    if (((a.b_count * a.nk) & 7) == 0) {
-        const int i = p >> 3, per = 2 * rep;                   // position in the XCD's order; workgroups per k-head
-        const int ku = (p & 7) + 8 * (i / per), sub = i % per;  // (sequence, k-head) unit; member of its group
-        pair = ku * rep + (sub >> 1);
-        half = sub & 1;
-    } else if ((pairs & 7) == 0) {
-        pair = (p & 7) + 8 * (p >> 4);
-        half = (p >> 3) & 1;
-    } else {
-        pair = p >> 1;
-        half = p & 1;
-    }
-    pair += a.b_base * a.nv;
-    const int b = pair / a.nv, j = pair % a.nv;
-    const int tw = wave & 3, cp = wave >> 2;
-    const int64_t chunk_stride = (int64_t)a.B * a.nk * kHeadBytes + (int64_t)a.B * a.nv * kUnitBytes;
-    const uint8_t *wsh = a.ws + ((int64_t)b * a.nk + j / (a.nv / a.nk)) * kHeadBytes;        // + ci * chunk_stride
-    const uint8_t *wsp = a.ws + (int64_t)a.B * a.nk * kHeadBytes + (int64_t)pair * kUnitBytes;  // + ci * chunk_stride
-
-    if (NORM && wave >= 10) {  // ---- the two wavefronts that finish the output rows
-        const int lt = tid - 640;
-        // Wavefront fw finishes token rows 32 fw .. 32 fw + 31 of a chunk, eight rows per instruction: lane = (row
-        // 8 i + lane / 8, the eight columns 8 (lane % 8) .. + 7), so eight lanes cover a row's 128 bytes and every load
-        // of z and store of the result moves whole lines.  Lane l also owns the sums of row 32 fw + l % 32.
-        const int fw = lt >> 6, ecol = 8 * (lane & 7), rsub = lane >> 3, srow = 32 * fw + (lane & 31);
-        float other = 0.0f;
-        u32x4 zr[4];
-        const float4v wa = *(const float4v *)(a.norm_w + 64 * half + ecol), wb = *(const float4v *)(a.norm_w + 64 * half + ecol + 4);
-        const float wv[8] = {wa[0], wa[1], wa[2], wa[3], wb[0], wb[1], wb[2], wb[3]};
-        // sums of squares of chunk c over this workgroup's 64 columns -> the exchange slots of this half.  Device-scope
-        // stores and loads of single floats: nothing else has to be ordered.
-        auto publish = [&](int c) {
-            if (lane < 32) {
-                float *slot = (float *)(a.ws + (wsp - a.ws) + c * chunk_stride + kOffSsq + 256 * half) + srow;
-                __hip_atomic_store(slot, ssq_lds[c % kRing][0][srow] + ssq_lds[c % kRing][1][srow], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        };
-        auto their_slot = [&](int c) { return (const float *)(wsp + c * chunk_stride + kOffSsq + 256 * (half ^ 1)) + srow; };
-        auto elem = [&](int c, int i) {  // first of this lane's eight elements of row 8 i + rsub of its wavefront's rows
-            const int t = min(c * kC + 32 * fw + 8 * i + rsub, a.T - 1);
-            return (((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + ecol;
-        };
-        // what finishing chunk c needs from memory
-        auto load_other = [&](int c) { other = __hip_atomic_load(their_slot(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
-        auto load_z = [&](int c) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) zr[i] = __builtin_nontemporal_load((const u32x4 *)(a.z + elem(c, i)));
-        };
-        auto finish = [&](int c) {
-            if (__builtin_amdgcn_ballot_w64(other < 0.0f) != 0) {  // not the normal case: the other half is chunks behind
-                for (int spin = kNormSpin; spin > 0; --spin) {
-                    __builtin_amdgcn_s_sleep(8);
-                    other = __hip_atomic_load(their_slot(c), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (__builtin_amdgcn_ballot_w64(other < 0.0f) == 0) break;
-                }
-            }
-            // a half that never arrived (its workgroup is not running: the launch was not cooperative) poisons the row
-            const float ss = other >= 0.0f ? ssq_lds[c % kRing][0][srow] + ssq_lds[c % kRing][1][srow] + other : __builtin_nanf("");
-            const float rrms_mine = 1.0f / sqrtf(ss / (float)kWD + a.norm_eps);  // of row srow
-            typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = 32 * fw + 8 * i + rsub;
-                const float rrms = __shfl(rrms_mine, 8 * i + rsub, 64);
-                const float4v xa = *(const float4v *)&o_lds[c % kRing][row][ecol], xb = *(const float4v *)&o_lds[c % kRing][row][ecol + 4];
-                const float xv[8] = {xa[0], xa[1], xa[2], xa[3], xb[0], xb[1], xb[2], xb[3]};
-                uint32_t o4[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const float z0 = __uint_as_float(zr[i][u] << 16), z1 = __uint_as_float(zr[i][u] & 0xffff0000u);
-                    const float s0 = z0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z0 * -1.4426950408889634f));
-                    const float s1 = z1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z1 * -1.4426950408889634f));
-                    const bf16x2 pr = {(__bf16)(xv[2 * u] * rrms * wv[2 * u] * s0), (__bf16)(xv[2 * u + 1] * rrms * wv[2 * u + 1] * s1)};
-                    o4[u] = __builtin_bit_cast(uint32_t, pr);
-                }
-                if (c * kC + row < a.T) __builtin_nontemporal_store((u32x4){o4[0], o4[1], o4[2], o4[3]}, (u32x4 *)(a.out_norm + elem(c, i)));
-            }
-        };
-        // Chunk c: rows in LDS at the end of step c, sums published in round c + 1, the other half's sums and z
-        // requested in round c + 2 (a chunk and a half after they were published), the rows finished in round c + 3 (a
-        // chunk after the request): these wavefronts never wait for memory, so they never hold up a barrier.
-        for (int ci = 0; ci < a.nc; ++ci) {
-            lds_sync();  // the rows and sums of chunk ci - 1 are in LDS now
-            if (ci > 0) publish(ci - 1);
-            lds_sync();
-            if (ci > 2) finish(ci - 3);
-            if (ci > 1) {
-                load_z(ci - 2);
-                load_other(ci - 2);
-            }
-        }
-        lds_sync();  // the last chunk's rows and sums are in LDS
-        publish(a.nc - 1);
-        if (a.nc > 2) finish(a.nc - 3);
-        for (int c = max(a.nc - 2, 0); c < a.nc; ++c) {
-            load_z(c);
-            load_other(c);
-            finish(c);
-        }
-        return;
-    }
-    if (wave >= 8) {  // ---- the two loader wavefronts
-        // (Plain loads: these operands are shared with the other column half through L2, and the non-temporal hint
-        // that helps the U loads and the output stores (scan 165 -> 152 us) cost 3 % here.  The prepare kernel's
-        // workspace stores are plain too: with the hint it took the same time and wrote 5 % more.)
-        // Region A of `ops` (-W, q and the decay vectors: 32.5 KB) is read between the two barriers of a chunk, region
-        // B (k^T and the masked q k^T: 24 KB) after the second one.  So A of the next chunk is written after the second barrier, B of a chunk
-        // after its first barrier -- neither write holds anybody up -- and each is fetched a whole chunk earlier.
-        const int lt = tid - 512;
-        u32x4 sa[16], sb[12];
-        float fac = 0.0f;  // one of the 128 decay factors per loader thread
-        auto fetch_a = [&](int ci) {
-            const int64_t o = min(ci, a.nc - 1) * chunk_stride;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                sa[i] = *(const u32x4 *)(wsp + o + kOffWn + (lt + 128 * i) * 16);
-                sa[8 + i] = *(const u32x4 *)(wsh + o + kOffQh + (lt + 128 * i) * 16);
-            }
-            fac = *(const float *)(wsp + o + kOffEG + 4 * lt);  // e^G (64 floats) then e^(G63-G) (64 floats)
-        };
-        auto fetch_b = [&](int ci) {
-            const int64_t o = min(ci, a.nc - 1) * chunk_stride;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sb[i] = *(const u32x4 *)(wsh + o + kOffKt + (lt + 128 * i) * 16);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) sb[8 + i] = *(const u32x4 *)(wsp + o + kOffQK + (lt + 128 * i) * 16);
-        };
-        auto park_a = [&]() {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) *(u32x4 *)(ops + (lt + 128 * i) * 16) = sa[i];
-            *(float *)(ops + kOpsFac + 4 * lt) = fac;
-        };
-        auto park_b = [&]() {
-#pragma unroll
-            for (int i = 0; i < 12; ++i) *(u32x4 *)(ops + kOpsKt + (lt + 128 * i) * 16) = sb[i];
-        };
-        fetch_a(0);
-        fetch_b(0);
-        park_a();
-        fetch_a(1);
-        for (int ci = 0; ci < a.nc; ++ci) {
-            lds_sync();  // A of chunk ci is visible; nobody reads B of chunk ci - 1 any more
-            park_b();
-            fetch_b(ci + 1);
-            lds_sync();  // B of chunk ci is visible; nobody reads A of chunk ci any more
-            park_a();
-            fetch_a(ci + 2);
-        }
-        if constexpr (NORM) lds_sync();  // the hand-over of the last chunk's rows (every wavefront takes part)
-        return;
-    }
-
-    float4v S[2][kYT];  // [dk tile 2*tw + x][column tile kYT*cp + y]
-    float *sp = a.state + ((int64_t)pair * kWD) * kWD + 64 * half + 16 * kYT * cp + li;
-#pragma unroll
-    for (int x = 0; x < 2; ++x)
-#pragma unroll
-        for (int y = 0; y < kYT; ++y)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) S[x][y][r] = sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y];
-
-    u32x2 uu[kYT], un[kYT];
-    float decay, decay_n;
-    auto fetch = [&](int ci) {
-        const uint8_t *u = wsp + ci * chunk_stride;
-#pragma unroll
-        for (int y = 0; y < kYT; ++y) un[y] = __builtin_nontemporal_load((const u32x2 *)(u + kOffU + ((tw * 8 + 4 * half + kYT * cp + y) * 64 + lane) * 8));
-        decay_n = *(const float *)(u + kOffDecay);
-    };
-    auto park = [&]() {
-#pragma unroll
-        for (int y = 0; y < kYT; ++y) uu[y] = un[y];
-        decay = decay_n;
-    };
-    auto opA = [&](int off, int blk) { return *(const half8 *)(ops + off + (blk * 64 + lane) * 16); };
-
-    fetch(0);
-    park();
-    // One chunk.  `guard`: the chunk may reach past T (only the last one can); full chunks store without a predicate.
-    auto step = [&](int ci, auto guard_tag) {
-        constexpr bool guard = decltype(guard_tag)::value;
-        fetch(min(ci + 1, a.nc - 1));  // the last iteration re-reads its own chunk: one path through the loop
-        // S as the B operand of W S and q S
-#pragma unroll
-        for (int y = 0; y < kYT; ++y)
-            *(half8 *)(s_lds + ((tw * 4 + kYT * cp + y) * 64 + lane) * 16) = f32x8_to_half8(S[0][y], S[1][y]);
-        lds_sync();  // also: the loaders have parked this chunk's -W and q e^G
-        // decay vectors (region A of the buffer: read them before the second barrier).  e^G of this lane's token row;
-        // e^(G63-G) of the tokens that are the k-slots of the state update: 32 s + 4 lq + e and 32 s + 16 + 4 lq + e
-        const _Float16 eg_row = (_Float16)*(const float *)(ops + kOpsFac + 4 * (16 * tw + li));
-        half8 egl[2];
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-            egl[s] = f32x8_to_half8(*(const float4v *)(ops + kOpsFac + 256 + 4 * (32 * s + 4 * lq)),
-                                    *(const float4v *)(ops + kOpsFac + 256 + 4 * (32 * s + 16 + 4 * lq)));
-        float4v vp[kYT], o[kYT];
-#pragma unroll
-        for (int y = 0; y < kYT; ++y) {
-            const half4v u4 = __builtin_bit_cast(half4v, uu[y]);
-            vp[y] = (float4v){(float)u4[0], (float)u4[1], (float)u4[2], (float)u4[3]};
-            o[y] = (float4v){0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const half8 wn = opA(kOpsWn, tw * 4 + s), qp = opA(kOpsQh, tw * 4 + s) * eg_row;
-#pragma unroll
-            for (int y = 0; y < kYT; ++y) {
-                const half8 sb = *(const half8 *)(s_lds + ((s * 4 + kYT * cp + y) * 64 + lane) * 16);
-                vp[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wn, sb, vp[y], 0, 0, 0);
-                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qp, sb, o[y], 0, 0, 0);
-            }
-        }
-        // V' (this wavefront's 16 tokens) as half of a B operand block
-#pragma unroll
-        for (int y = 0; y < kYT; ++y) {
-            half4v h;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) h[r] = (_Float16)vp[y][r];
-            *(half4v *)(v_lds + (((tw >> 1) * 4 + kYT * cp + y) * 64 + lane) * 16 + 8 * (tw & 1)) = h;
-        }
-        lds_sync();
-        const float dec = decay;
-#pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const half8 qk = opA(kOpsQK, tw * 2 + s), kd0 = opA(kOpsKt, (2 * tw) * 2 + s) * egl[s], kd1 = opA(kOpsKt, (2 * tw + 1) * 2 + s) * egl[s];
-#pragma unroll
-            for (int y = 0; y < kYT; ++y) {
-                if (s == 0) {
-                    S[0][y] *= dec;
-                    S[1][y] *= dec;
-                }
-                const half8 vb = *(const half8 *)(v_lds + ((s * 4 + kYT * cp + y) * 64 + lane) * 16);
-                o[y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(qk, vb, o[y], 0, 0, 0);
-                S[0][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd0, vb, S[0][y], 0, 0, 0);
-                S[1][y] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kd1, vb, S[1][y], 0, 0, 0);
-            }
-        }
-        if constexpr (!NORM) {
-#pragma unroll
-            for (int y = 0; y < kYT; ++y)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int t = ci * kC + 16 * tw + 4 * lq + r;
-                    if (!guard || t < a.T) __builtin_nontemporal_store(o[y][r], &a.out[(((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + 16 * (kYT * cp + y) + li]);
-                }
-        } else {
-            // the rows wait in LDS for the other half's sums; their sums of squares over this wavefront's 32 columns too
-            float4v sq = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int y = 0; y < kYT; ++y) {
-                sq += o[y] * o[y];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) o_lds[ci % kRing][16 * tw + 4 * lq + r][16 * (kYT * cp + y) + li] = o[y][r];
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-#pragma unroll
-                for (int sh = 1; sh < 16; sh <<= 1) sq[r] += __shfl_xor(sq[r], sh, 64);
-            }
-            if (li == 0) *(float4v *)&ssq_lds[ci % kRing][cp][16 * tw + 4 * lq] = sq;
-        }
-        park();
-    };
-    const int nfull = a.T / kC;
-    for (int ci = 0; ci < nfull; ++ci) step(ci, std::false_type());
-    if (nfull < a.nc) step(nfull, std::true_type());
-    if constexpr (NORM) lds_sync();  // hands the last chunk's rows to the finishing wavefronts
-#pragma unroll
-    for (int x = 0; x < 2; ++x)
-#pragma unroll
-        for (int y = 0; y < kYT; ++y)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sp[(int64_t)(16 * (2 * tw + x) + 4 * lq + r) * kWD + 16 * y] = S[x][y][r];
-}
+// The scan kernel exists twice: deltanet_chunk_scan_kernel, and deltanet_chunk_scan_norm_kernel with the gated norm in
+// its epilogue.  One text, deltanet_chunk_scan.inc, included once with HS_SCAN_NORM 0 and once with 1 -- not one
+// template: with the norm's shared arrays, arguments or branches merely present (empty, unused or constant-false) the
+// compiler laid out LDS and ordered the chunk loop of the plain kernel differently, and it ran 5 % slower.
+#define HS_SCAN_NORM 0
+#include "deltanet_chunk_scan.inc"
+#undef HS_SCAN_NORM
+#define HS_SCAN_NORM 1
+#include "deltanet_chunk_scan.inc"
+#undef HS_SCAN_NORM
 
 }  // namespace hs
 
@@ -712,7 +438,7 @@ extern "C" {
 
 size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv) {
     if (B <= 0 || T <= 0 || nk <= 0 || nv <= 0) return 0;
-    return (size_t)((T + hs::kC - 1) / hs::kC) * ((size_t)B * nk * hs::kHeadBytes + (size_t)B * nv * hs::kUnitBytes);
+    return (size_t)((T + hs::kC - 1) / hs::kC) * ((size_t)B * nk * hs::kHeadBytes + (size_t)B * nv * (hs::kUnitBytes + hs::kSsqBytes));
 }
 
 static int chunked_common(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
@@ -750,7 +476,7 @@ int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, con
     hipStream_t st = (hipStream_t)stream;
     deltanet_chunk_prepare_kernel<<<(unsigned)((int64_t)B * nv * a.nc), 512, 0, st>>>(a);
     if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
-    deltanet_chunk_scan_kernel<false><<<(unsigned)(2 * B * nv), kScanThreads, 0, st>>>(a);
+    deltanet_chunk_scan_kernel<<<(unsigned)(2 * B * nv), kScanThreads, 0, st>>>(a);
     return check_launch("deltanet_chunk_scan");
 }
 
@@ -770,7 +496,7 @@ int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const v
     int dev = 0, cus = 0, per_cu = 0, coop = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
         hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess ||
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, deltanet_chunk_scan_kernel<true>, kScanNormThreads, 0) != hipSuccess) {
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, deltanet_chunk_scan_norm_kernel, kScanNormThreads, 0) != hipSuccess) {
         (void)hipGetLastError();
         return fail(HS_ERR_LAUNCH, "cannot query the device for a cooperative launch");
     }
@@ -788,7 +514,7 @@ int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const v
         a.b_base = b0;
         a.b_count = std::min(per_launch, B - b0);
         void *args[] = {&a};
-        const hipError_t e = hipLaunchCooperativeKernel((const void *)deltanet_chunk_scan_kernel<true>, dim3((unsigned)(2 * a.b_count * nv)),
+        const hipError_t e = hipLaunchCooperativeKernel((const void *)deltanet_chunk_scan_norm_kernel, dim3((unsigned)(2 * a.b_count * nv)),
                                                         dim3(kScanNormThreads), args, 0, st);
         if (e != hipSuccess) {
             (void)hipGetLastError();

@@ -352,7 +352,7 @@ HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, cons
  * everything else is fp16-operand / fp32-accumulate MFMA.  Mathematically identical to hs_deltanet_forward; outputs
  * and the final state differ from it by rounding (about 1e-3 relative).  Arguments as hs_deltanet_forward, plus a
  * device workspace of hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) bytes (per 64-token chunk: 32,768 per
- * (sequence, k-head) and 42,240 per (sequence, v-head)), 16-byte aligned, owned by the caller; q, k, v must be
+ * (sequence, k-head) and 41,728 + 512 per (sequence, v-head)), 16-byte aligned, owned by the caller; q, k, v must be
  * 16-byte aligned.  A prompt split into calls of a multiple
  * of 64 tokens (state carried through `state`) gives the bits of one call. */
 HS_API size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv);
