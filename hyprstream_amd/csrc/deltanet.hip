@@ -454,8 +454,8 @@ extern "C" int hs_deltanet_decode_layer(const void *mixed_qkv, const void *conv_
     if (dk != kDK || dv != kDV) return fail(HS_ERR_INVALID_ARGUMENT, "deltanet is built for dk = dv = 128, got %d x %d", dk, dv);
     if (B < 0 || nk <= 0 || nv <= 0 || nv % nk != 0)
         return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d nk=%d nv=%d (need nv %% nk == 0)", B, nk, nv);
-    if ((((uintptr_t)z | (uintptr_t)norm_weight | (uintptr_t)out) & 15) != 0)
-        return fail(HS_ERR_INVALID_ARGUMENT, "z, norm_weight and out must be 16-byte aligned");
+    if ((((uintptr_t)z | (uintptr_t)norm_weight | (uintptr_t)out) & 15) != 0 || ((uintptr_t)conv_weight & 7) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "z, norm_weight and out must be 16-byte aligned, conv_weight 8-byte");
     if (B == 0) return HS_OK;
     DeltaArgs a{};
     a.state = state;

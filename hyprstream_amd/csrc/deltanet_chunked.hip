@@ -490,18 +490,32 @@ int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const v
     ChunkArgs a;
     if (int rc = chunked_common(q, k, v, g, beta, state, B, T, nk, nv, dk, dv, q_scale, l2norm, workspace, workspace_bytes, a); rc >= 0)
         return rc;
+    if ((((uintptr_t)z | (uintptr_t)norm_weight | (uintptr_t)out) & 15) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "z, norm_weight and out must be 16-byte aligned");
     a.z = (const uint16_t *)z; a.norm_w = norm_weight; a.norm_eps = norm_eps; a.out_norm = (uint16_t *)out;
     // The two workgroups of a (sequence, v-head) wait for each other once per chunk, so every workgroup of a scan
     // launch has to be resident: a cooperative launch, over as many whole sequences as the device holds at a time.
-    int dev = 0, cus = 0, per_cu = 0, coop = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess ||
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, deltanet_chunk_scan_norm_kernel, kScanNormThreads, 0) != hipSuccess) {
+    // (what the device holds is looked up once per device; a second thread doing the same stores the same values)
+    constexpr int kMaxDevices = 64;
+    static int resident_of[kMaxDevices];  // 0: not asked yet, -1: no cooperative launches, else workgroups resident at once
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
         (void)hipGetLastError();
         return fail(HS_ERR_LAUNCH, "cannot query the device for a cooperative launch");
     }
-    if (!coop) return fail(HS_ERR_LAUNCH, "the device does not support cooperative launches: run hs_deltanet_forward_chunked and hs_deltanet_gated_norm");
-    const int64_t resident = (int64_t)cus * per_cu;
+    if (resident_of[dev] == 0) {
+        int cus = 0, per_cu = 0, coop = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, deltanet_chunk_scan_norm_kernel, kScanNormThreads, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(HS_ERR_LAUNCH, "cannot query the device for a cooperative launch");
+        }
+        resident_of[dev] = coop ? std::max(1, cus * per_cu) : -1;
+    }
+    if (resident_of[dev] < 0)
+        return fail(HS_ERR_LAUNCH, "the device does not support cooperative launches: run hs_deltanet_forward_chunked and hs_deltanet_gated_norm");
+    const int64_t resident = resident_of[dev];
     if (resident < 2 * (int64_t)nv)
         return fail(HS_ERR_INVALID_ARGUMENT,
                     "%d v-heads need %d workgroups resident at once, the device holds %lld: run hs_deltanet_forward_chunked "

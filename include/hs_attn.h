@@ -362,7 +362,8 @@ HS_API int hs_deltanet_forward_chunked(const void *q, const void *k, const void 
                         float q_scale, int l2norm, void *workspace, size_t workspace_bytes, hs_stream_t stream);
 /* hs_deltanet_forward_chunked with the layer's gated RMSNorm (RMSNormGated::forward, qwen3_5.rs:305-313; what
  * hs_deltanet_gated_norm computes) in the epilogue: out [B, T, nv, dv] bf16 = bf16(o * rsqrt(mean(o^2) + eps) * weight *
- * silu(z)) with z [B, T, nv, dv] bf16 and weight [dv] fp32; the fp32 rows o are never written.  Same workspace.  Equal
+ * silu(z)) with z [B, T, nv, dv] bf16 and weight [dv] fp32 (both, and out, 16-byte aligned); the fp32 rows o are never
+ * written.  Same workspace.  Equal
  * to the two calls up to the order in which a row's squares are added (one bf16 ulp, rarely).  The two workgroups that
  * share a row exchange their sums through the workspace, so the scan is a cooperative launch (all its workgroups
  * resident; several launches when the batch needs more than the device holds): not capturable in a HIP graph, and
@@ -400,7 +401,7 @@ HS_API int hs_deltanet_gated_norm(const float *x, const void *z, const float *we
  * serve with their wide kernels), but q, k, v, g, beta and the fp32 output row never leave the chip.
  *   mixed_qkv [B, 1, 2*nk*dk + nv*dv] bf16;  conv_state_in [B, C, 3] bf16 or NULL;  conv_state_out a different buffer;
  *   a_in, b_in [B, 1, nv] bf16;  z [B, 1, nv, dv] bf16;  norm_weight [dv] fp32;  state [B, nv, dk, dv] fp32 in place;
- *   out [B, 1, nv, dv] bf16.  dk = dv = 128. */
+ *   out [B, 1, nv, dv] bf16.  dk = dv = 128; z, norm_weight and out 16-byte aligned, conv_weight 8-byte. */
 HS_API int hs_deltanet_decode_layer(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in,
                                     void *conv_state_out, const void *a_in, const void *b_in, const float *neg_a_exp,
                                     const float *dt_bias, const void *z, const float *norm_weight, float norm_eps,
