@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-norm-2calls|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-norm-2calls|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -72,6 +72,8 @@ WORKLOADS = {
     # c2 with q and the new K row arriving as projected: per-head QK-norm (Llama flavour) and the rotary embedding run
     # inside the decode-step launch (hs_decode_step_int8_prologue)
     "c2-prologue": (64, 32, 8, 128, 8192, False, False, 1.0, True),
+    # c4 the same way over the FP8 cache (hs_decode_step_fp8_prologue): the step a Qwen3-style layer runs
+    "c4-prologue": (32, 64, 8, 128, 32768, False, True, 0.5, False),
 }
 
 
@@ -482,7 +484,7 @@ def main():
     quant = hb.kv_quantize_fp8 if fp8 else hb.kv_quantize_int8
 
     pro = None
-    if args.workload == "c2-prologue":
+    if args.workload in ("c2-prologue", "c4-prologue"):
         inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
         ang = torch.arange(T, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
         rope = (ang.sin().to(torch.bfloat16).contiguous(), ang.cos().to(torch.bfloat16).contiguous())
@@ -493,7 +495,7 @@ def main():
     def step(i):
         kc, vc, ks, vs = caches[i % ncopies]
         if pro is not None:
-            hb.decode_step_prologue(q, k_new, v_new, pro, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale)
+            hb.decode_step_prologue(q, k_new, v_new, pro, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8)
         else:
             hb.decode_step(q, k_new, v_new, kc, vc, ks, vs, layout, lens, out, ws, Hkv, max_len, scale, fp8=fp8)
 

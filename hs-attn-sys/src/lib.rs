@@ -151,6 +151,23 @@ pub unsafe fn decode_step_fp8_gpu(q: *const c_void, k_new: *const c_void, v_new:
                                        softmax_scale, stream))
 }
 
+/// `decode_step_fp8_gpu` with QK-norm and rotary embedding of q and k_new inside the launch (qwen3_5.rs:1077-1091,
+/// rope.rs:206-248).
+///
+/// # Safety
+/// As `decode_step_int8_prologue_gpu`.
+#[allow(clippy::too_many_arguments)]
+pub unsafe fn decode_step_fp8_prologue_gpu(q: *const c_void, k_new: *const c_void, v_new: *const c_void,
+                                           prologue: &hs_qk_prologue, k_codes: *mut u8, v_codes: *mut u8,
+                                           k_scales: *const f32, v_scales: *const f32, layout: &hs_kv_layout,
+                                           seq_lens: *const i32, out: *mut c_void, workspace: *mut c_void,
+                                           workspace_bytes: usize, shape: AttnShape, max_seq_len: i32,
+                                           softmax_scale: f32, stream: hs_stream_t) -> Result<()> {
+    check(bindings::hs_decode_step_fp8_prologue(q, k_new, v_new, prologue, k_codes, v_codes, k_scales, v_scales, layout,
+                                                seq_lens, out, workspace, workspace_bytes, shape.b, shape.hq, shape.hkv,
+                                                shape.d, max_seq_len, softmax_scale, stream))
+}
+
 /// Causal prefill of `s` new tokens over [int8 history | their own bf16 K/V], caching them (q_len > 1 branch,
 /// llama.rs:1066-1112).  q and k_new arrive rotated (`qk_prologue_apply_gpu` is the one-launch pre-pass).
 ///

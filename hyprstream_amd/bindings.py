@@ -25,7 +25,7 @@ EXPORTS = [
     "hs_decode_attn_workspace_bytes", "hs_decode_attn_int8", "hs_decode_attn_fp8", "hs_decode_attn_phases",
     "hs_decode_step_int8", "hs_decode_step_fp8", "hs_prefill_attn_int8", "hs_prefill_attn_fp8", "hs_deltanet_forward",
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
-    "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue",
+    "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue", "hs_decode_step_fp8_prologue",
     "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_deltanet_forward_chunked_gated_norm", "hs_deltanet_prefill_layer", "hs_deltanet_prefill_layer_workspace_bytes", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
 ]
 
@@ -199,15 +199,16 @@ def kv_quantize_int8_prologue(k_src, v_src, prologue, k_codes, v_codes, k_scales
 
 
 def decode_step_prologue(q, k_new, v_new, prologue, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out,
-                         workspace, Hkv, max_seq_len, softmax_scale):
-    """decode_step (int8) with the QK-norm and the rotation of q and k_new inside the launch."""
+                         workspace, Hkv, max_seq_len, softmax_scale, fp8=False):
+    """decode_step (int8, or fp8 with calibrated scales) with the QK-norm and the rotation of q and k_new inside the
+    launch."""
     B, Hq, D = q.shape
     assert k_new.shape == (B, 1, Hkv, D) and k_new.is_contiguous() and v_new.is_contiguous()
-    check(lib().hs_decode_step_int8_prologue(_ptr(q), _ptr(k_new), _ptr(v_new), ctypes.byref(prologue), _ptr(k_codes),
-                                             _ptr(v_codes), _ptr(k_scales), _ptr(v_scales), ctypes.byref(layout),
-                                             _ptr(seq_lens), _ptr(out), _ptr(workspace),
-                                             ctypes.c_size_t(workspace.numel() * workspace.element_size()), B, Hq, Hkv,
-                                             D, ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
+    fn = lib().hs_decode_step_fp8_prologue if fp8 else lib().hs_decode_step_int8_prologue
+    check(fn(_ptr(q), _ptr(k_new), _ptr(v_new), ctypes.byref(prologue), _ptr(k_codes), _ptr(v_codes), _ptr(k_scales),
+             _ptr(v_scales), ctypes.byref(layout), _ptr(seq_lens), _ptr(out), _ptr(workspace),
+             ctypes.c_size_t(workspace.numel() * workspace.element_size()), B, Hq, Hkv, D,
+             ctypes.c_int32(max_seq_len), ctypes.c_float(softmax_scale), _stream()))
 
 
 def kv_fp8_calibrate(k_src, v_src, k_scales, v_scales):

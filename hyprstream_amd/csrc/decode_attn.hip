@@ -898,7 +898,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
         const dim3 grid = a.balanced ? dim3(a.pieces, Hkv, 1) : dim3(a.nchunks, Hkv, B);
 #define HS_DECODE_LAUNCH(DD, BAL)                                                                      \
     do {                                                                                               \
-        if (fp8) decode_attn_kernel<DD, true, false, BAL><<<grid, 256, 0, stream>>>(a);                \
+        if (fp8 && pro) decode_attn_kernel<DD, true, true, BAL><<<grid, 256, 0, stream>>>(a);          \
+        else if (fp8) decode_attn_kernel<DD, true, false, BAL><<<grid, 256, 0, stream>>>(a);           \
         else if (pro) decode_attn_kernel<DD, false, true, BAL><<<grid, 256, 0, stream>>>(a);           \
         else decode_attn_kernel<DD, false, false, BAL><<<grid, 256, 0, stream>>>(a);                   \
     } while (0)
@@ -1007,6 +1008,23 @@ int hs_decode_step_int8_prologue(const void *q, const void *k_new, const void *v
     nt.prologue = true;
     return hs::launch_decode(false, 3, nt, q, k_codes, v_codes, k_scales, v_scales, layout, seq_lens, out, workspace,
                              workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
+}
+
+int hs_decode_step_fp8_prologue(const void *q, const void *k_new, const void *v_new, const hs_qk_prologue *prologue,
+                                uint8_t *k_codes, uint8_t *v_codes, const float *k_scales, const float *v_scales,
+                                const hs_kv_layout *layout, const int32_t *seq_lens, void *out, void *workspace,
+                                size_t workspace_bytes, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
+                                int32_t max_seq_len, float softmax_scale, hs_stream_t stream) {
+    if (!k_new || !v_new) return hs::fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (int rc = hs::check_prologue(prologue, HS_BF16, D, true, true)) return rc;
+    hs::NewToken nt;
+    nt.k_src = k_new; nt.v_src = v_new; nt.dtype = HS_BF16;
+    nt.rope_sin = prologue->rope_sin; nt.rope_cos = prologue->rope_cos; nt.rope_len = prologue->rope_len;
+    nt.rotary_dim = prologue->rotary_dim;
+    nt.qnorm = hs::norm_spec(prologue, 0); nt.knorm = hs::norm_spec(prologue, 1);
+    nt.prologue = true;
+    return hs::launch_decode(true, 3, nt, q, k_codes, v_codes, (float *)k_scales, (float *)v_scales, layout, seq_lens, out,
+                             workspace, workspace_bytes, B, Hq, Hkv, D, max_seq_len, softmax_scale, (hipStream_t)stream);
 }
 
 int hs_decode_step_fp8(const void *q, const void *k_new, const void *v_new, int src_dtype, uint8_t *k_codes,

@@ -275,6 +275,16 @@ HS_API int hs_decode_step_fp8(const void *q, const void *k_new, const void *v_ne
                               void *workspace, size_t workspace_bytes,
                               int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
                               float softmax_scale, hs_stream_t stream);
+/* hs_decode_step_int8_prologue for the FP8 cache (qwen3_5.rs:1077-1091 + rope.rs:206-248 in front of
+ * kv_cache.rs:459-497 with an FP8 cache): k_new is normalised and rotated, then encoded with the sequence's calibrated
+ * scale; q is normalised and rotated on its way into the attention.  Same argument rules and served rotary_dim values as
+ * the int8 call; results equal hs_qk_prologue_apply + hs_decode_step_fp8 bit for bit. */
+HS_API int hs_decode_step_fp8_prologue(const void *q, const void *k_new, const void *v_new, const hs_qk_prologue *prologue,
+                              uint8_t *k_codes, uint8_t *v_codes, const float *k_scales, const float *v_scales,
+                              const hs_kv_layout *layout, const int32_t *seq_lens, void *out,
+                              void *workspace, size_t workspace_bytes,
+                              int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
+                              float softmax_scale, hs_stream_t stream);
 
 /* The two phases of split-K decode attention on their own: phases = 1 runs only the attention kernel
  * and leaves per-chunk partials (m, l, o) in the workspace, 2 only the merge of those partials into

@@ -5,6 +5,7 @@
   hs_qk_prologue_apply            bit-exact with the oracle's norm followed by its op-by-op rounded rotation
   hs_kv_quantize_int8_prologue    codes / scales of quantizing the oracle's normalised and rotated K
   hs_decode_step_int8_prologue    = hs_qk_prologue_apply + hs_decode_step_int8 bit for bit, and the oracle
+  hs_decode_step_fp8_prologue     = hs_qk_prologue_apply + hs_decode_step_fp8 bit for bit, and the oracle
   prologue -> prefill -> cache    rope(q), rope(k) -> hs_prefill_attn_int8(quantize_on_write) against the oracle's
                                   rotation + causal attention; the cache holds the codes of hs_kv_quantize_int8_rope
 """
@@ -216,6 +217,64 @@ def test_decode_step_with_prologue_matches_unfused_and_oracle(lens, kind, D, rd)
     for b, n in enumerate(lens):
         assert np.array_equal(kc[b, n - 1], wkc[b]) and np.array_equal(ks[b, n - 1].view(np.uint32), wks[b].view(np.uint32))
     want = oracle.decode_attn(oracle.bf16_to_f32(q_fin), kc, vc, ks, vs, oracle.FMT_INT8, np.array(lens, np.int32), scale)
+    err = np.abs(out1.float().cpu().numpy() - want)
+    assert err.max() < TOL_MAX and err.mean() < TOL_MEAN
+
+
+@pytest.mark.parametrize("kind,D,rd", [(hb.QKNORM_LLAMA, 128, 128), (hb.QKNORM_QWEN35, 256, 64), (hb.QKNORM_LLAMA, 64, 64),
+                                       (hb.QKNORM_NONE, 128, 32), (hb.QKNORM_QWEN35, 128, 0)])
+@pytest.mark.parametrize("lens", [[260, 260, 260], [1, 129, 700]])
+def test_fp8_decode_step_with_prologue_matches_unfused_and_oracle(lens, kind, D, rd):
+    """The FP8 cache (per-(sequence, head) scales calibrated on the history): hs_decode_step_fp8_prologue against
+    hs_qk_prologue_apply + hs_decode_step_fp8 bit for bit, the new token's codes against the oracle's e4m3 encoder
+    applied to the oracle's normalised and rotated k_new, the output against the oracle's attention."""
+    r = wl.philox(1400 + len(set(lens)) + D + rd + kind)
+    B, Hq, Hkv, L = len(lens), 16, 4, 1024
+    T = max(lens)
+    rope = rd > 0
+    sin, cos = _tables(rd, 1000000.0, L) if rope else (None, None)
+    hist_k = _bf(r.standard_normal((B, T, Hkv, D)) * 0.8).to(DEV)
+    hist_v = _bf(r.standard_normal((B, T, Hkv, D)) * 0.8).to(DEV)
+    q = _bf(r.standard_normal((B, Hq, D)) * 1.7).to(DEV)
+    k_new = _bf(r.standard_normal((B, 1, Hkv, D)) * 0.6).to(DEV)
+    v_new = _bf(r.standard_normal((B, 1, Hkv, D)) * 0.8).to(DEV)
+    wq = _weights(r, kind, Hq, D, per_head=False) if kind else None
+    wk = _weights(r, kind, Hkv, D, per_head=True) if kind else None
+    pro = hb.qk_prologue(kind, 1e-6, wq.to(DEV) if kind else None, wk.to(DEV) if kind else None,
+                         sin.to(DEV) if rope else None, cos.to(DEV) if rope else None, rd)
+    lens_d = torch.tensor(lens, dtype=torch.int32, device=DEV)
+    scale = 1.0 / np.sqrt(D)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+
+    def fresh():
+        c = DeviceCache(B, Hkv, T, D, fp8=True)
+        hb.kv_fp8_calibrate(hist_k, hist_v, c.k_scales, c.v_scales)
+        c.write(hist_k, hist_v)
+        return c
+
+    c1 = fresh()
+    out1 = torch.empty(B, Hq, D, dtype=torch.bfloat16, device=DEV)
+    hb.decode_step_prologue(q, k_new, v_new, pro, c1.k_codes, c1.v_codes, c1.k_scales, c1.v_scales, c1.layout, lens_d,
+                            out1, ws, Hkv, T, scale, fp8=True)
+    c2 = fresh()
+    q2 = torch.empty(B, 1, Hq, D, dtype=torch.bfloat16, device=DEV)
+    k2 = torch.empty(B, 1, Hkv, D, dtype=torch.bfloat16, device=DEV)
+    hb.qk_prologue_apply(q.view(B, 1, Hq, D), k_new, pro, q2, k2, lens_d - 1, 0)
+    out2 = torch.empty_like(out1)
+    hb.decode_step(q2.view(B, Hq, D), k2, v_new, c2.k_codes, c2.v_codes, c2.k_scales, c2.v_scales, c2.layout, lens_d,
+                   out2, ws, Hkv, T, scale, fp8=True)
+    torch.cuda.synchronize()
+    assert bool(torch.equal(c1.k_codes, c2.k_codes)) and bool(torch.equal(c1.v_codes, c2.v_codes))
+    assert bool(torch.equal(out1, out2))
+    pos = np.array(lens, np.int32) - 1
+    q_fin = oracle_prologue(_bits(q).reshape(B, Hq, D), kind, wq, 1e-6, sin, cos, pos, rd)
+    k_fin = oracle_prologue(_bits(k_new).reshape(B, Hkv, D), kind, wk, 1e-6, sin, cos, pos, rd)
+    kc, vc, ks, vs = c1.canonical(T)
+    wkc = oracle.quant_fp8(oracle.bf16_to_f32(k_fin).reshape(B, 1, Hkv, D), ks)
+    wvc = oracle.quant_fp8(v_new.float().cpu().numpy(), vs)
+    for b, n in enumerate(lens):
+        assert np.array_equal(kc[b, n - 1], wkc[b, 0]) and np.array_equal(vc[b, n - 1], wvc[b, 0])
+    want = oracle.decode_attn(oracle.bf16_to_f32(q_fin), kc, vc, ks, vs, oracle.FMT_FP8, np.array(lens, np.int32), scale)
     err = np.abs(out1.float().cpu().numpy() - want)
     assert err.max() < TOL_MAX and err.mean() < TOL_MEAN
 
