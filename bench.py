@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-norm-2calls|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -215,9 +215,8 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
 def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
     """Config 5: gated DeltaNet, nk 16 / nv 32, dk = dv = 128.  Decode: B = 64, one token, fp32 state read and
     written once (HBM bound).  Prefill: B = 4 x 4096 tokens in chunks of 64 on the matrix pipe (c5-prefill), or
-    through the token-by-token fp32 recurrence (c5-prefill-recurrent).  norm = "fused" / "2calls": the chunked prefill
-    followed by the layer's gated RMSNorm, inside the scan's epilogue (hs_deltanet_forward_chunked_gated_norm,
-    c5-prefill-norm) or as a second call over the fp32 rows (c5-prefill-norm-2calls)."""
+    through the token-by-token fp32 recurrence (c5-prefill-recurrent).  norm: the chunked prefill followed by the layer's
+    gated RMSNorm as one call (hs_deltanet_forward_chunked_gated_norm, c5-prefill-norm)."""
     dev = "cuda:0"
     nk, nv, d = 16, 32, 128
     B, T = (4, 4096) if prefill else (64, 1)
@@ -235,7 +234,8 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
     qs = 1.0 / float(np.sqrt(d))
 
     chunked = prefill and not recurrent
-    ws = torch.empty(hb.deltanet_chunked_workspace_bytes(B, T, nk, nv), dtype=torch.uint8, device=dev) if chunked else None
+    ws_bytes = (hb.deltanet_chunked_gated_norm_workspace_bytes if norm else hb.deltanet_chunked_workspace_bytes)(B, T, nk, nv)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if chunked else None
 
     if norm:
         z = torch.randn(B, T, nv, d, generator=gen, device=dev).to(torch.bfloat16)
@@ -243,11 +243,8 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
         out_n = torch.empty(B, T, nv, d, dtype=torch.bfloat16, device=dev)
 
     def step(i):
-        if norm == "fused":
+        if norm:
             hb.deltanet_forward_chunked_gated_norm(q, k, v, g, beta, states[i % ncopies], z, nw, 1e-6, out_n, qs, False, workspace=ws)
-        elif norm:
-            hb.deltanet_forward_chunked(q, k, v, g, beta, states[i % ncopies], out, qs, False, workspace=ws)
-            hb.deltanet_gated_norm(out, z, nw, 1e-6)
         elif chunked:
             hb.deltanet_forward_chunked(q, k, v, g, beta, states[i % ncopies], out, qs, False, workspace=ws)
         else:
@@ -281,12 +278,12 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
         "dtype": "f16 MFMA operands, f32 accumulation, triangular solve and state; bf16 q/k/v" if chunked else "f32 state and arithmetic, bf16 q/k/v",
         "data": "synthetic (seeded, generated on device)",
         "config": {"workload": "c5-%s: gated delta rule B=%d T=%d nk=16 nv=32 dk=dv=128, fp32 state [B,32,128,128]%s%s"
-                               % (("prefill-norm" + ("" if norm == "fused" else "-2calls") if norm else "prefill") if prefill else "decode", B, T,
+                               % (("prefill-norm" if norm else "prefill") if prefill else "decode", B, T,
                                   ", chunk size 64" if chunked else (", token recurrence" if prefill else ""),
-                                  (", gated RMSNorm in the scan's epilogue" if norm == "fused" else ", gated RMSNorm as a second call") if norm else ""),
+                                  ", then the gated RMSNorm (same call)" if norm else ""),
                    "algorithmic_bytes_per_step": int(nbytes)},
         "tokens_per_s": B * T / (ms * 1e-3),
-        "roofline": {"bound": "hbm", "kernel": ("deltanet_chunk_prepare_kernel + deltanet_chunk_scan_kernel" if chunked else "deltanet_prefill_kernel") if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": ("deltanet_chunk_factor_kernel + deltanet_chunk_walk_kernel" + (" + gated_rmsnorm_rows_kernel" if norm else "") if chunked else "deltanet_prefill_kernel") if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "avg_kernel_us": kms * 1e3},
     }
@@ -367,7 +364,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-norm-2calls", "c5-prefill-recurrent"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
@@ -411,7 +408,7 @@ def main():
         return bench_deltanet_layer(args, torch, hb, wl, fused=args.workload == "c5-decode-layer")
     if args.workload.startswith("c5"):
         return bench_deltanet(args, torch, hb, wl, "prefill" in args.workload, recurrent=args.workload.endswith("recurrent"),
-                              norm="fused" if args.workload == "c5-prefill-norm" else "2calls" if args.workload == "c5-prefill-norm-2calls" else None)
+                              norm=args.workload == "c5-prefill-norm")
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)

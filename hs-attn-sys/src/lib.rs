@@ -206,11 +206,11 @@ pub unsafe fn deltanet_forward_gpu(q: *const c_void, k: *const c_void, v: *const
     check(bindings::hs_deltanet_forward(q, k, v, g, beta, state, out, b, t, nk, nv, dk, dv, q_scale, l2norm as c_int, stream))
 }
 
-/// chunked_delta_rule (qwen3_5.rs:342-498) followed by RMSNormGated (qwen3_5.rs:305-313) without the fp32 tensor
-/// between them: `out` is the bf16 normed tensor.  The scan is a cooperative launch (not capturable in a HIP graph).
+/// chunked_delta_rule (qwen3_5.rs:342-498) followed by RMSNormGated (qwen3_5.rs:305-313) in one call: `out` is the
+/// bf16 normed tensor, the fp32 rows between the two pass through the workspace.
 ///
 /// # Safety
-/// As above; `workspace` holds at least `hs_deltanet_chunked_workspace_bytes(b, t, nk, nv)` bytes.
+/// As above; `workspace` holds at least `hs_deltanet_chunked_gated_norm_workspace_bytes(b, t, nk, nv)` bytes.
 #[allow(clippy::too_many_arguments)]
 pub unsafe fn deltanet_forward_chunked_gated_norm_gpu(q: *const c_void, k: *const c_void, v: *const c_void, g: *const f32,
                                                       beta: *const f32, state: *mut f32, z: *const c_void,

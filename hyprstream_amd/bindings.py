@@ -27,6 +27,7 @@ EXPORTS = [
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
     "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue", "hs_decode_step_fp8_prologue",
     "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_deltanet_forward_chunked_gated_norm", "hs_deltanet_prefill_layer", "hs_deltanet_prefill_layer_workspace_bytes", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
+    "hs_deltanet_chunked_gated_norm_workspace_bytes",
 ]
 
 
@@ -330,6 +331,11 @@ def deltanet_chunked_workspace_bytes(B, T, nk, nv):
     return int(lib().hs_deltanet_chunked_workspace_bytes(B, T, nk, nv))
 
 
+def deltanet_chunked_gated_norm_workspace_bytes(B, T, nk, nv):
+    lib().hs_deltanet_chunked_gated_norm_workspace_bytes.restype = ctypes.c_size_t
+    return int(lib().hs_deltanet_chunked_gated_norm_workspace_bytes(B, T, nk, nv))
+
+
 def deltanet_forward_chunked(q, k, v, g, beta, state, out, q_scale, l2norm=False, workspace=None):
     """The same over a prompt in 64-token chunks on the matrix pipe (fp16 operands, fp32 accumulation and state)."""
     import torch
@@ -348,14 +354,14 @@ def deltanet_forward_chunked(q, k, v, g, beta, state, out, q_scale, l2norm=False
 
 
 def deltanet_forward_chunked_gated_norm(q, k, v, g, beta, state, z, norm_weight, eps, out, q_scale, l2norm=False, workspace=None):
-    """deltanet_forward_chunked with the gated RMSNorm in the epilogue: out bf16 [B, T, nv, dv]."""
+    """deltanet_forward_chunked + the gated RMSNorm, one call: out bf16 [B, T, nv, dv]."""
     import torch
     B, T, nk, dk = q.shape
     nv, dv = v.shape[2], v.shape[3]
     for t in (q, k, v, g, beta, state, z, out):
         assert t.is_contiguous()
-    lib().hs_deltanet_chunked_workspace_bytes.restype = ctypes.c_size_t
-    need = lib().hs_deltanet_chunked_workspace_bytes(B, T, nk, nv)
+    lib().hs_deltanet_chunked_gated_norm_workspace_bytes.restype = ctypes.c_size_t
+    need = lib().hs_deltanet_chunked_gated_norm_workspace_bytes(B, T, nk, nv)
     if workspace is None:
         workspace = torch.empty(max(need, 16), dtype=torch.uint8, device=q.device)
     check(lib().hs_deltanet_forward_chunked_gated_norm(_ptr(q), _ptr(k), _ptr(v), _ptr(g), _ptr(beta), _ptr(state), _ptr(z),

@@ -26,9 +26,6 @@ COMMON = [
 # the quantizers must do exactly the fp32 operations written (bit-exact with the CPU oracle)
 PER_FILE = {
     "kv_quantize.hip": ["-ffp-contract=off"],
-    # the two chunk kernels of the delta rule run 1.5 % faster with loads clustered by the scheduler (0.315 -> 0.310 ms at
-    # 4 x 4096 tokens); on the attention kernels the default strategy is the best of those tried
-    "deltanet_chunked.hip": ["-mllvm", "-amdgpu-sched-strategy=max-memory-clause"],
 }
 
 

@@ -1,34 +1,31 @@
-// Gated delta rule over a prompt in chunks of 64 tokens on the MFMA pipe (gfx950, wave64).
+// Gated delta rule over a prompt in chunks of 64 tokens on the MFMA pipe (gfx950, wave64): the reference's own prefill
+// formulation (chunked_delta_rule, qwen3_5.rs:342-498; chunk size 64), regrouped so that little has to pass through
+// memory between the part that is parallel over chunks and the part that walks them in order.
 //
-// The reference's own prefill formulation (chunked_delta_rule, qwen3_5.rs:342-498; chunk size 64): with
-// G_t the running sum of the log-decays g inside a chunk, k and q L2-normalised (q also scaled), and
-//   L[i][j] = -beta_i (k_i . k_j) exp(G_i - G_j)  for j < i (0 otherwise),      N = (I - L)^-1,
-//   U = N (v * beta),     W = N (k * beta * exp(G)),
+// With G_t the running sum of the log-decays inside a chunk, k and q L2-normalised (q also scaled) and
+//   L[i][j] = -beta_i (k_i . k_j) exp(G_i - G_j)  (j < i),      N = (I - L)^-1,      N' = N diag(beta),
+//   M[i][j] = (q_i . k_j) exp(G_i - G_j)          (j <= i),
 // a chunk that starts from the state S (dk x dv) gives
-//   V' = U - W S
-//   O  = (q * exp(G)) S + tril(q k^T * exp(G_i - G_j)) V'
-//   S <- exp(G_63) S + (k * exp(G_63 - G))^T V'.
-// It is the token recurrence S <- S e^g; S += k (v - k^T S) beta; o = q^T S regrouped, so the results differ
-// from the recurrent kernel only by rounding.
+//   X  = v - (k e^G) S
+//   V' = N' X                                  (= N (v beta) - N (k beta e^G) S, the U - W S of the reference)
+//   O  = (q e^G) S + M V'
+//   S <- e^(G_63) S + (k e^(G_63 - G))^T V'.
+// Only N' and M (two 64 x 64 triangles per chunk and v-head) do not follow from one row of the inputs at a time, so
+// only they go through memory: deltanet_chunk_factor_kernel makes them for all chunks in parallel, and
+// deltanet_chunk_walk_kernel walks the chunks of one (sequence, v-head, half of the state columns) in order, reading
+// q, k and v as they were given.  Against a workspace that also carries W, U and the normalised q and k in operand
+// order (deltanet_chunked.hip) this moves 17 KB instead of 58 KB per chunk and v-head through HBM twice.
 //
-// Two kernels.  deltanet_chunk_prepare_kernel does everything that does not involve S, for all chunks of all
-// (sequence, v-head) pairs in parallel (one 512-thread workgroup per chunk): normalisation, the two 64x64
-// products on MFMA, the inverses of the four diagonal 16x16 blocks of I - L (repeated squaring, one wavefront per block), then
-// [U | W] = N [v beta | k beta e^G] by block forward substitution on MFMA (the rest of N is never formed), and
-// writes every matrix the second kernel needs into the workspace ALREADY in MFMA operand order (fp16).
-// deltanet_chunk_scan_kernel walks the chunks of one (sequence, v-head, half of the state columns) in order with
-// the state in accumulator registers: 28 MFMAs per computing wavefront and chunk, S and V' exchanged between the wavefronts through LDS
-// in operand order, the chunk's operands brought in by two wavefronts that do nothing else.
+// The walk: four wavefronts each own 16 state columns -- all 128 rows, in accumulator registers -- for the whole
+// prompt.  Nothing passes between them: the accumulator layout of S, X and V' (lane (li, lq): column li, rows
+// 4 lq + r) is the B operand layout of the next product once the k-slots of the A operand are taken in that
+// order (slots 0-3: rows 4 lq + r of the even 16-row tile of a 32-row slab, slots 4-7: of the odd tile), so a
+// chunk is 62 MFMAs and three conversions in registers per wavefront, and one workgroup barrier (the hand-over of
+// the operand buffer).  Four more wavefronts do nothing but bring in the next chunk: they read k, q, v rows and the
+// two triangles a chunk ahead, normalise, fold the decay factors in and write everything as fp16 A operands into
+// the other half of a two-chunk LDS buffer.
 //
-// Operands are fp16 (11-bit significands; every decay factor is <= 1, so nothing overflows and what underflows
-// is negligible in absolute terms), accumulation and the state are fp32.  Against the fp32 recurrence the
-// outputs differ by about 1e-3 relative.
-//
-// MFMA layouts (v_mfma_f32_16x16x32_f16, lane l: li = l % 16, lq = l / 16): A row li / B column li hold eight
-// k-slots of group lq; C/D column li holds rows 4*lq + r.  Where one operand of a product is the accumulator
-// of an earlier one (S, V', the masked q k^T), the k-slots stand for the rows that accumulator layout
-// holds -- slots 0-3: row 4*lq + r of the even 16-row tile of a 32-row slab, slots 4-7: the same rows of the
-// odd tile -- and the other operand is read in the same order.
+// Operands are fp16, accumulation and the state fp32 (every decay factor is <= 1: nothing overflows).
 #include <algorithm>
 #include <climits>
 #include <type_traits>
@@ -37,33 +34,24 @@
 
 namespace hs {
 
-constexpr int kC = 64;               // tokens per chunk
-constexpr int kWD = 128;             // dk = dv = 128
-constexpr float kLog2eC = 1.4426950408889634f;
+constexpr int kC = 64;    // tokens per chunk
+constexpr int kWD = 128;  // dk = dv = 128
+constexpr float kLog2e = 1.4426950408889634f;
 typedef _Float16 half4v __attribute__((ext_vector_type(4)));
 
-// Workspace, chunk-major; every matrix is a list of 64-lane blocks in MFMA operand order.
-// Per (sequence, k-head, chunk) -- the normalised q and k do not depend on the v-head, so the v-heads of a k-head
-// share them and the decays that make them "q e^G" and "(k e^(G63-G))^T" travel as two vectors per v-head:
-constexpr int kOffQh = 0;        // q (normalised, scaled)  A operand [token tile 4][dk slab 4][lane] 16 B
-constexpr int kOffKt = 16384;    // k^T (normalised)        A operand [dk tile 8][token slab 2][lane] 16 B
-constexpr int kHeadBytes = 32768;
-// Per (sequence, v-head, chunk):
-constexpr int kOffWn = 0;        // -W      A operand [token tile 4][dk slab 4][lane] 16 B
-constexpr int kOffQK = 16384;    // masked q k^T     A operand [token tile 4][token slab 2][lane] 16 B
-constexpr int kOffU = 24576;     // U       accumulator tiles [token tile 4][dv tile 8][lane] 8 B
-constexpr int kOffEG = 40960;    // exp(G_t), 64 floats
-constexpr int kOffEGl = 41216;   // exp(G_63 - G_t), 64 floats
-constexpr int kOffDecay = 41472; // exp(G63), one float
-constexpr int kUnitBytes = 41728;
-// Behind all chunks' operands, per (chunk, sequence, v-head): 2 x 64 floats -- per column half, the sums of squares of the
-// chunk's output rows over that half's 64 columns (the fused gated norm's exchange between the two halves; -1 = not
-// there yet).  A region of its own: inside the units it changed their stride, and the plain scan ran 7 % slower.
-constexpr int kSsqBytes = 512;
-// The same matrices inside the scan kernel's LDS operand buffer:
-constexpr int kOpsWn = 0, kOpsQh = 16384, kOpsKt = 32768, kOpsQK = 49152, kOpsFac = 57344, kOpsBytes = 57856;
+// Workspace, chunk-major: per (chunk, sequence, v-head)
+// The triangles as A operands, 64-lane blocks of 16 B: block (token tile tt, token slab s) for the six pairs with
+// 32 s <= 16 tt + 15 (the other two are zero and are neither stored nor multiplied), at index tri_block(tt, s).
+constexpr int kOffNt = 0;         // N' (A operand of N' X), 6 KB
+constexpr int kOffQK = 6144;      // M  (A operand of M V'), 6 KB
+constexpr int kOffFn = 12288;     // -exp(G_t) / |k_t|            (what turns a row of k into a row of -k-hat e^G), 64 floats
+constexpr int kOffFq = 12544;     // exp(G_t) q_scale / |q_t|
+constexpr int kOffFt = 12800;     // exp(G_63 - G_t) / |k_t|
+constexpr int kOffDecay = 13056;  // exp(G_63)
+constexpr int kUnitBytes = 13312;
+__host__ __device__ constexpr int tri_block(int tt, int s) { return tt < 2 ? tt : 2 * tt - 2 + s; }
 
-struct ChunkArgs {
+struct WalkArgs {
     const uint16_t *q, *k, *v;  // bf16 [B,T,nk,128], [B,T,nk,128], [B,T,nv,128]
     const float *g, *beta;      // [B,T,nv]
     float *state;               // [B,nv,128,128]
@@ -72,12 +60,6 @@ struct ChunkArgs {
     int32_t B, T, nk, nv, nc;
     float q_scale;
     int32_t l2norm;
-    // scan with the gated RMSNorm in its epilogue (out is then unused): z [B,T,nv,128] bf16, weight [128], bf16 result
-    const uint16_t *z;
-    const float *norm_w;
-    uint16_t *out_norm;
-    float norm_eps;
-    int32_t b_base, b_count;  // the sequences this scan launch covers (all of them unless the launch is cooperative)
 };
 
 __device__ __forceinline__ half8 f32x8_to_half8(const float4v &a, const float4v &b) {
@@ -89,32 +71,41 @@ __device__ __forceinline__ half8 f32x8_to_half8(const float4v &a, const float4v 
     }
     return h;
 }
+__device__ __forceinline__ half4v f32x4_to_half4(const float4v &x) {
+    return (half4v){(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+}
 
-// ------------------------------------------------------------------------------------------------ prepare
+// Sixteen bf16 (two 16-byte pieces) -> fp32
+__device__ __forceinline__ void unpack16(const u32x4 &a, const u32x4 &b, float *f) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        f[2 * e] = __uint_as_float(a[e] << 16);
+        f[2 * e + 1] = __uint_as_float(a[e] & 0xffff0000u);
+        f[8 + 2 * e] = __uint_as_float(b[e] << 16);
+        f[8 + 2 * e + 1] = __uint_as_float(b[e] & 0xffff0000u);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------- factors
 constexpr int kPitchH = 136;  // halves per row of the row-major k / q tiles
-constexpr int kPitchT = 72;   // halves per row of the transposed k / v tiles
-constexpr int kPitchL = 68;   // halves per row of the 64x64 matrix L (fp16: it is only ever an MFMA operand)
-constexpr int kPitchD = 20;   // floats per row of a 16x16 fp32 block (diagonal blocks of L / of the inverse, and their scratch)
+constexpr int kPitchL = 68;   // halves per row of the 64 x 64 matrix P = L^T
+constexpr int kPitchD = 20;   // floats per row of a 16 x 16 fp32 block
 constexpr int kBlockD = 16 * kPitchD;
-// 51 KB, three workgroups per CU.  Region A holds the row-major k / q tiles, then the scratch blocks of the four
-// inverses, then the transposed tiles; L (below its diagonal blocks) and the diagonal blocks live beside it.
-constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsKT = 0, kLdsVT = 18432;                   // region A: 36,864 B
-constexpr int kLdsS = 0;                                                                // scratch blocks, 3 per wavefront 0-3
-constexpr int kLdsL = 36864, kLdsD = kLdsL + 64 * kPitchL * 2, kLdsF = kLdsD + 4 * kBlockD * 4, kLdsBytes = kLdsF + 1536;
-static_assert(kLdsBytes <= 54528, "three workgroups of the prepare kernel per CU");
+// Region A: the row-major k / q tiles, later the scratch blocks of the four inverses.
+constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsS = 0;
+constexpr int kLdsP = 34816, kLdsD = kLdsP + 64 * kPitchL * 2, kLdsF = kLdsD + 4 * kBlockD * 4, kLdsBytes = kLdsF + 1536;
+static_assert(kLdsBytes <= 54528, "three workgroups of the factor kernel per CU");
 
-// Transposed tiles [feature d][token]: the eight-token (16-byte) pieces of a row are permuted by d / 16, so that the
-// threads of a wavefront, which write one token each for features 16 apart, hit different banks.
-__device__ __forceinline__ int tpos(int d, int tok) { return d * kPitchT + ((((tok >> 3) ^ (d >> 4)) & 7) << 3) + (tok & 7); }
-
-__global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArgs a) {
+// One 512-thread workgroup per (sequence, v-head, chunk).  Everything is built transposed -- P = L^T, the diagonal
+// blocks of (I - P)^-1 = N^T, then N^T by block back substitution -- because the accumulator layout of a tile of
+// N^T (lane: column i, rows j = 4 lq + r) is the A operand layout the walk needs for N (row i, k-slots j).
+__global__ __launch_bounds__(512, 6) void deltanet_chunk_factor_kernel(WalkArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
     _Float16 *kh = (_Float16 *)(lds + kLdsKh), *qh = (_Float16 *)(lds + kLdsQh);
-    _Float16 *KT = (_Float16 *)(lds + kLdsKT), *VT = (_Float16 *)(lds + kLdsVT);
-    _Float16 *Lh = (_Float16 *)(lds + kLdsL);  // L, strictly below its diagonal blocks
-    float *Dm = (float *)(lds + kLdsD);        // the four diagonal blocks of L, later of N = (I - L)^-1
-    float *Sm = (float *)(lds + kLdsS);        // scratch blocks of the inverses, once the k / q row tiles are dead
-    float *gs = (float *)(lds + kLdsF), *bs = gs + 64, *Gs = gs + 128, *eG = gs + 192, *eGl = gs + 256, *be = gs + 320;
+    _Float16 *Ph = (_Float16 *)(lds + kLdsP);  // P[j][i] = L[i][j], outside the diagonal blocks
+    float *Dm = (float *)(lds + kLdsD);        // the four diagonal blocks of P, later of (I - P)^-1
+    float *Sm = (float *)(lds + kLdsS);        // scratch blocks of the inverses, once the k / q tiles are dead
+    float *gs = (float *)(lds + kLdsF), *bs = gs + 64, *Gs = gs + 128, *km = gs + 192;  // km: 64 x (kmul, qmul)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -124,42 +115,22 @@ __global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArg
     const int j = (int)((unit / a.nc) % a.nv);
     const int b = (int)(unit / ((int64_t)a.nc * a.nv));
     const int hk = j / (a.nv / a.nk);
-    // chunk-major workspace: the workgroups of the scan kernel walk the chunks in step, so what they read at one
-    // moment is one contiguous region spread over all memory channels (sequence-major, they would all sit at the
-    // same offset of regions a fixed stride apart and queue up on a few channels)
-    const int rep = a.nv / a.nk;
-    uint8_t *wsc = a.ws + (int64_t)c * ((int64_t)a.B * a.nk * kHeadBytes + (int64_t)a.B * a.nv * kUnitBytes);
-    uint8_t *wsh = wsc + ((int64_t)b * a.nk + hk) * kHeadBytes;  // written by the first v-head of the k-head
-    uint8_t *wsu = wsc + (int64_t)a.B * a.nk * kHeadBytes + ((int64_t)b * a.nv + j) * kUnitBytes;
-    const bool first_of_head = j % rep == 0;
+    uint8_t *wsu = a.ws + ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kUnitBytes;
 
-    // ---- 1. load 64 tokens, normalise, stage: thread = (token tt, 16 consecutive elements)
-    half8 kreg[2], vreg[2];  // this thread's k-hat and v, written transposed once the inverse is done
+    // ---- 1. 64 tokens of k and q, normalised, row-major in LDS: thread = (token tt, 16 consecutive elements)
     const int tt = tid >> 3, part = tid & 7;
     {
         const int t = c * kC + tt;
         const bool valid = t < a.T;
-        float kf[16], qf[16], vf[16];
+        float kf[16], qf[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) kf[e] = qf[e] = vf[e] = 0.0f;
+        for (int e = 0; e < 16; ++e) kf[e] = qf[e] = 0.0f;
         if (valid) {
             const int64_t bt = (int64_t)b * a.T + t;
             const uint16_t *kp = a.k + (bt * a.nk + hk) * kWD + 16 * part;
             const uint16_t *qp = a.q + (bt * a.nk + hk) * kWD + 16 * part;
-            const uint16_t *vp = a.v + (bt * a.nv + j) * kWD + 16 * part;
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const u32x4 kw = *(const u32x4 *)(kp + 8 * i), qw = *(const u32x4 *)(qp + 8 * i), vw = *(const u32x4 *)(vp + 8 * i);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    kf[8 * i + 2 * e] = __uint_as_float(kw[e] << 16);
-                    kf[8 * i + 2 * e + 1] = __uint_as_float(kw[e] & 0xffff0000u);
-                    qf[8 * i + 2 * e] = __uint_as_float(qw[e] << 16);
-                    qf[8 * i + 2 * e + 1] = __uint_as_float(qw[e] & 0xffff0000u);
-                    vf[8 * i + 2 * e] = __uint_as_float(vw[e] << 16);
-                    vf[8 * i + 2 * e + 1] = __uint_as_float(vw[e] & 0xffff0000u);
-                }
-            }
+            unpack16(*(const u32x4 *)kp, *(const u32x4 *)(kp + 8), kf);
+            unpack16(*(const u32x4 *)qp, *(const u32x4 *)(qp + 8), qf);
         }
         float kmul = 1.0f, qmul = a.q_scale;
         if (a.l2norm) {
@@ -180,13 +151,9 @@ __global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArg
         half8 k8[2], q8[2];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const _Float16 kk = (_Float16)(kf[e] * kmul);
-            k8[e >> 3][e & 7] = kk;
+            k8[e >> 3][e & 7] = (_Float16)(kf[e] * kmul);
             q8[e >> 3][e & 7] = (_Float16)(qf[e] * qmul);
-            vreg[e >> 3][e & 7] = (_Float16)vf[e];
         }
-        kreg[0] = k8[0];
-        kreg[1] = k8[1];
         *(half8 *)&kh[tt * kPitchH + 16 * part] = k8[0];
         *(half8 *)&kh[tt * kPitchH + 16 * part + 8] = k8[1];
         *(half8 *)&qh[tt * kPitchH + 16 * part] = q8[0];
@@ -194,6 +161,8 @@ __global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArg
         if (part == 0) {
             gs[tt] = valid ? a.g[((int64_t)b * a.T + t) * a.nv + j] : 0.0f;
             bs[tt] = valid ? a.beta[((int64_t)b * a.T + t) * a.nv + j] : 0.0f;
+            km[2 * tt] = valid ? kmul : 0.0f;  // rows past T are zero
+            km[2 * tt + 1] = valid ? qmul : 0.0f;
         }
     }
     __syncthreads();
@@ -209,228 +178,512 @@ __global__ __launch_bounds__(512, 6) void deltanet_chunk_prepare_kernel(ChunkArg
         const float g63 = __shfl(x, 63, 64);
         const float e = expf(x);
         Gs[lane] = x;
-        eG[lane] = e;
-        eGl[lane] = expf(g63 - x);
-        be[lane] = bs[lane] * e;
+        *(float *)(wsu + kOffFn + 4 * lane) = -e * km[2 * lane];
+        *(float *)(wsu + kOffFq + 4 * lane) = e * km[2 * lane + 1];
+        *(float *)(wsu + kOffFt + 4 * lane) = expf(g63 - x) * km[2 * lane];
         if (lane == 63) *(float *)(wsu + kOffDecay) = e;
-#ifndef EXP_NOSENT
-        float *ssq = (float *)(a.ws + a.nc * ((int64_t)a.B * a.nk * kHeadBytes + (int64_t)a.B * a.nv * kUnitBytes) +
-                               ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kSsqBytes);
-        ssq[lane] = -1.0f;  // both halves' exchange slots: nothing there yet
-        ssq[64 + lane] = -1.0f;
-#endif
     }
 
     // ---- 3. k k^T (rows i, columns j) and k q^T (rows j, columns i): wavefront w owns row tile w/2, column tiles 2(w%2), +1
     float4v kk[2], qk[2];
     const int mt = wave >> 1;
-    {
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        kk[x] = (float4v){0.f, 0.f, 0.f, 0.f};
+        qk[x] = (float4v){0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        const half8 ar = *(const half8 *)&kh[(16 * mt + li) * kPitchH + 32 * s + 8 * lq];
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
-            kk[x] = (float4v){0.f, 0.f, 0.f, 0.f};
-            qk[x] = (float4v){0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const half8 ar = *(const half8 *)&kh[(16 * mt + li) * kPitchH + 32 * s + 8 * lq];
-#pragma unroll
-            for (int x = 0; x < 2; ++x) {
-                const int nt = 2 * (wave & 1) + x;
-                const half8 bk = *(const half8 *)&kh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
-                const half8 bq = *(const half8 *)&qh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
-                kk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bk, kk[x], 0, 0, 0);
-                qk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bq, qk[x], 0, 0, 0);
-            }
+            const int nt = 2 * (wave & 1) + x;
+            const half8 bk = *(const half8 *)&kh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
+            const half8 bq = *(const half8 *)&qh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
+            kk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bk, kk[x], 0, 0, 0);
+            qk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bq, qk[x], 0, 0, 0);
         }
     }
-    __syncthreads();  // G and the factors are visible
+    __syncthreads();  // G and beta are visible
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
         const int nt = 2 * (wave & 1) + x;
         const int col = 16 * nt + li;
         const float gcol = Gs[col];
+        float4v lv;
         half4v m;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = 16 * mt + 4 * lq + r;
-            // L[i = row][j = col]: the diagonal blocks in fp32 for the inverse, the rest as the fp16 operand it will be
-            const float lv = col < row ? -bs[row] * kk[x][r] * __builtin_amdgcn_exp2f((Gs[row] - gcol) * kLog2eC) : 0.0f;
-            if (nt == mt) Dm[mt * kBlockD + (4 * lq + r) * kPitchD + li] = lv;
-            else Lh[row * kPitchL + col] = (_Float16)lv;
+            lv[r] = col < row ? -bs[row] * kk[x][r] * __builtin_amdgcn_exp2f((Gs[row] - gcol) * kLog2e) : 0.0f;  // L[row][col]
             // masked q k^T: row = key j, col = query i, kept for j <= i
-            m[r] = (_Float16)(row <= col ? qk[x][r] * __builtin_amdgcn_exp2f((gcol - Gs[row]) * kLog2eC) : 0.0f);
+            m[r] = (_Float16)(row <= col ? qk[x][r] * __builtin_amdgcn_exp2f((gcol - Gs[row]) * kLog2e) : 0.0f);
         }
-        *(half4v *)(wsu + kOffQK + ((nt * 2 + (mt >> 1)) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
+        // P[col][row]: the diagonal blocks in fp32 for the inverse, the rest as the fp16 operand it will be
+        if (nt == mt) *(float4v *)&Dm[mt * kBlockD + li * kPitchD + 4 * lq] = lv;
+        else *(half4v *)&Ph[col * kPitchL + 16 * mt + 4 * lq] = f32x4_to_half4(lv);
+        if (nt >= 2 || mt < 2) *(half4v *)(wsu + kOffQK + (tri_block(nt, mt >> 1) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
     }
-    // q as the A operand of q S: block (token tile, dk slab), lane (token li, group lq); the scan applies e^G
-    if (first_of_head) {
-#pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
-            const int tok = 16 * (blk >> 2) + (ln & 15), d0 = 32 * (blk & 3) + 4 * (ln >> 4);
-            const half4v lo = *(const half4v *)&qh[tok * kPitchH + d0], hi = *(const half4v *)&qh[tok * kPitchH + d0 + 16];
-            half8 o;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                o[e] = lo[e];
-                o[4 + e] = hi[e];
-            }
-            *(half8 *)(wsh + kOffQh + (blk * 64 + ln) * 16) = o;
-        }
-    }
-    if (tid < 64) {
-        *(float *)(wsu + kOffEG + 4 * tid) = eG[tid];
-        *(float *)(wsu + kOffEGl + 4 * tid) = eGl[tid];
-    }
-    __syncthreads();  // L complete; the row-major k / q tiles are dead from here on
+    __syncthreads();  // P complete; the row-major k / q tiles are dead from here on
 
-    // ---- 4. the diagonal 16x16 blocks of N = (I - L)^-1: N_aa = (I + L)(I + L^2)(I + L^4)(I + L^8) with L = L_aa.
-    //         Wavefront a < 4 does block a by itself -- six 16x16x16 products on MFMA (fp16 operands, fp32
-    //         accumulation), the matrices passing through its own LDS blocks between products (the operations of
-    //         one wavefront on LDS complete in order, so no workgroup barrier is needed until all four are done).
+    // ---- 4. the diagonal 16 x 16 blocks of (I - P)^-1: (I + D)(I + D^2)(I + D^4)(I + D^8) with D the (nilpotent) block.
+    //         Wavefront a < 4 does block a by itself -- six 16x16x16 products on MFMA, the matrices passing through
+    //         its own LDS blocks between products (the LDS operations of one wavefront complete in order).
     if (wave < 4) {
-        auto f4h = [](const float4v &x) { return (half4v){(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]}; };
-        // dst = (add ? add : 0) + X Y; lane (li, lq) holds rows 4 lq + r of column li of the result
         auto mm = [&](float *dst, const float *X, const float *Y, const float *add) {
-            const half4v xa = f4h(*(const float4v *)&X[li * kPitchD + 4 * lq]);
-            float4v yb, c;
+            const half4v xa = f32x4_to_half4(*(const float4v *)&X[li * kPitchD + 4 * lq]);
+            float4v yb, cc;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 yb[r] = Y[(4 * lq + r) * kPitchD + li];
-                c[r] = add ? add[(4 * lq + r) * kPitchD + li] : 0.0f;
+                cc[r] = add ? add[(4 * lq + r) * kPitchD + li] : 0.0f;
             }
-            c = __builtin_amdgcn_mfma_f32_16x16x16f16(xa, f4h(yb), c, 0, 0, 0);
+            cc = __builtin_amdgcn_mfma_f32_16x16x16f16(xa, f32x4_to_half4(yb), cc, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) dst[(4 * lq + r) * kPitchD + li] = c[r];
+            for (int r = 0; r < 4; ++r) dst[(4 * lq + r) * kPitchD + li] = cc[r];
             __builtin_amdgcn_wave_barrier();
         };
         float *Lb = Dm + wave * kBlockD, *Nb = Sm + (3 * wave) * kBlockD, *Pb = Nb + kBlockD, *Qb = Pb + kBlockD;
 #pragma unroll
         for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchD + li] = Lb[(4 * lq + r) * kPitchD + li] + (4 * lq + r == li ? 1.0f : 0.0f);
         __builtin_amdgcn_wave_barrier();
-        mm(Qb, Lb, Lb, nullptr);  // L^2
-        mm(Lb, Nb, Qb, Nb);       // (I + L)(I + L^2), into L's block (L itself is not needed any more)
-        mm(Pb, Qb, Qb, nullptr);  // L^4
-        mm(Nb, Lb, Pb, Lb);       // ... (I + L^4)
-        mm(Qb, Pb, Pb, nullptr);  // L^8
-        mm(Lb, Nb, Qb, Nb);       // ... (I + L^8): the inverse, where the diagonal block of L was
+        mm(Qb, Lb, Lb, nullptr);  // D^2
+        mm(Lb, Nb, Qb, Nb);       // (I + D)(I + D^2), into D's block (D itself is not needed any more)
+        mm(Pb, Qb, Qb, nullptr);  // D^4
+        mm(Nb, Lb, Pb, Lb);       // ... (I + D^4)
+        mm(Qb, Pb, Pb, nullptr);  // D^8
+        mm(Lb, Nb, Qb, Nb);       // ... (I + D^8): the inverse, where the diagonal block was
     }
     __syncthreads();
 
-    // ---- 5. X = N [v beta | k beta e^G] by block forward substitution, X_a = N_aa (R_a + sum_{m<a} L_am X_m), on
-    //         v_mfma_f32_16x16x16_f16.  A wavefront owns 32 columns (wavefronts 0-3: U, two dv tiles each; 4-7: W, the
-    //         two dk tiles of one slab) and walks the four row blocks with X_m in registers: the accumulator layout
-    //         of X_m (column li, rows 4 lq + r) is the B operand layout of the next level, so nothing is exchanged.
+    // ---- 5. Y = (I - P)^-1 = N^T by block back substitution, Y_b = Y_bb (I_b + sum_{m>b} P_bm Y_m), on
+    //         v_mfma_f32_16x16x16_f16: wavefront w < 4 owns the 16 columns i of block w and walks the row blocks
+    //         upwards with Y_m in registers (the accumulator layout of Y_m is the B operand layout of the next level).
+    //         Rows are then scaled by beta_j (N' = N diag(beta)) and stored as the A operand of N' X.
+    if (wave < 4) {
+        half4v yh[4];
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        KT[tpos(16 * part + e, tt)] = kreg[e >> 3][e & 7];
-        VT[tpos(16 * part + e, tt)] = vreg[e >> 3][e & 7];
-    }
-    __syncthreads();
-    // k^T as the A operand of the state update: block (dk tile, token slab), lane (dk li, group lq); the scan
-    // applies e^(G63 - G)
-    if (first_of_head) {
+        for (int m = 0; m < 4; ++m) yh[m] = (half4v){(_Float16)0.f, (_Float16)0.f, (_Float16)0.f, (_Float16)0.f};
 #pragma unroll
-        for (int it = 0; it < 2; ++it) {
-            const int item = tid + 512 * it, blk = item >> 6, ln = item & 63;
-            const int dk = 16 * (blk >> 1) + (ln & 15), t0 = 32 * (blk & 1) + 4 * (ln >> 4);
-            const half4v lo = *(const half4v *)&KT[tpos(dk, t0)], hi = *(const half4v *)&KT[tpos(dk, t0 + 16)];
-            half8 o;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                o[e] = lo[e];
-                o[4 + e] = hi[e];
-            }
-            *(half8 *)(wsh + kOffKt + (blk * 64 + ln) * 16) = o;
-        }
-    }
-    __syncthreads();  // the transposed k tile has been read for the output above: its rows may be reused below
-    {
-        const bool is_w = wave >= 4;
-        const _Float16 *T = is_w ? KT : VT;
-        const float *fac = is_w ? be : bs;
-        const int tile0 = 2 * (wave & 3);
-        auto f4h = [](const float4v &x) { return (half4v){(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]}; };
-        half4v xh[2][4];
-#pragma unroll
-        for (int ra = 0; ra < 4; ++ra) {
-#pragma unroll
-            for (int x = 0; x < 2; ++x) {
-                const int col = 16 * (tile0 + x) + li;
-                const half4v rr = *(const half4v *)&T[tpos(col, 16 * ra + 4 * lq)];
+        for (int bb = 0; bb < 4; ++bb) {
+            const int bl = 3 - bb;
+            float4v ya = {0.f, 0.f, 0.f, 0.f};
+            if (bl <= wave) {
                 float4v acc;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) acc[r] = (float)rr[r] * fac[16 * ra + 4 * lq + r];
+                for (int r = 0; r < 4; ++r) acc[r] = (bl == wave && 4 * lq + r == li) ? 1.0f : 0.0f;
 #pragma unroll
-                for (int m = 0; m < ra; ++m) {
-                    const half4v la = *(const half4v *)&Lh[(16 * ra + li) * kPitchL + 16 * m + 4 * lq];
-                    acc = __builtin_amdgcn_mfma_f32_16x16x16f16(la, xh[x][m], acc, 0, 0, 0);
+                for (int m = bl + 1; m < 4; ++m) {
+                    if (m <= wave) {
+                        const half4v pa = *(const half4v *)&Ph[(16 * bl + li) * kPitchL + 16 * m + 4 * lq];
+                        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(pa, yh[m], acc, 0, 0, 0);
+                    }
                 }
-                const half4v na = f4h(*(const float4v *)&Dm[ra * kBlockD + li * kPitchD + 4 * lq]);
-                const float4v xa = __builtin_amdgcn_mfma_f32_16x16x16f16(na, f4h(acc), (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
-                xh[x][ra] = f4h(xa);
-                if (!is_w) *(half4v *)(wsu + kOffU + ((ra * 8 + tile0 + x) * 64 + lane) * 8) = xh[x][ra];
+                const half4v da = f32x4_to_half4(*(const float4v *)&Dm[bl * kBlockD + li * kPitchD + 4 * lq]);
+                ya = __builtin_amdgcn_mfma_f32_16x16x16f16(da, f32x4_to_half4(acc), (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                yh[bl] = f32x4_to_half4(ya);
             }
-        }
-        if (is_w) {
-            // -W as the A operand of the scan (row = token, k-slots = the slab's dk in accumulator order): element
-            // (token 4 lq + r, dk li of tile x) belongs to lane (4 lq + r) + 16 (li / 4), slot li % 4 + 4 x.  Shuffled
-            // through this wavefront's own 32 rows of the transposed k tile, which nobody reads any more.
-            uint8_t *stg = (uint8_t *)(KT + (32 * (wave & 3)) * kPitchT);
+            half4v o;
 #pragma unroll
-            for (int ra = 0; ra < 4; ++ra)
-#pragma unroll
-                for (int x = 0; x < 2; ++x)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        *(_Float16 *)(stg + (ra * 64 + 4 * lq + r + 16 * (li >> 2)) * 16 + 2 * ((li & 3) + 4 * x)) = -xh[x][ra][r];
-            __builtin_amdgcn_wave_barrier();  // LDS operations of one wavefront complete in order
-#pragma unroll
-            for (int ra = 0; ra < 4; ++ra)
-                *(u32x4 *)(wsu + kOffWn + ((ra * 4 + (wave & 3)) * 64 + lane) * 16) = *(const u32x4 *)(stg + (ra * 64 + lane) * 16);
+            for (int r = 0; r < 4; ++r) o[r] = (_Float16)(ya[r] * bs[16 * bl + 4 * lq + r]);
+            if (wave >= 2 || bl < 2) *(half4v *)(wsu + kOffNt + (tri_block(wave, bl >> 1) * 64 + lane) * 16 + 8 * (bl & 1)) = o;
         }
     }
 }
 
-// --------------------------------------------------------------------------------------------------- scan
-// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for the operand prefetch of the
-// next chunk, which is issued at the top of the loop and not needed before the next iteration.
+// ---------------------------------------------------------------------------------------------------- walk
+// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for the loaders' global prefetch.
 __device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-constexpr int kYT = 2;  // 16-column tiles of the state per wavefront (a workgroup owns 64 of the 128 columns)
-constexpr int kScanThreads = 640;      // eight computing wavefronts and two that only move operands
-constexpr int kScanNormThreads = 768;  // ... and two that finish the output rows (NORM)
-static_assert(kOpsFac == 28 * 128 * 16, "28 16-byte pieces per loader thread");
+// One chunk's operands in LDS; A operand blocks are 64 lanes x 16 B.
+constexpr int kPitchT = 72;  // halves per row of the transposed k tile [dk][token]
+constexpr int oKn = 0;                        // -k e^G        [token tile 4][dk slab 4]
+constexpr int oQg = oKn + 16384;              // q e^G         [token tile 4][dk slab 4]
+constexpr int oKt = oQg + 16384;              // k e^(G63-G), transposed [dk 128][token 64], eight-token pieces permuted
+constexpr int oNt = oKt + kWD * kPitchT * 2;  // N'            six blocks, tri_block order
+constexpr int oQK = oNt + 6144;               // M             six blocks
+constexpr int oV = oQK + 6144;                // v, this half's 64 columns: [token tile 4][column slab 2], natural k order
+constexpr int oDec = oV + 8192;               // e^(G63)
+constexpr int kBufBytes = oDec + 16;
+// Behind the two operand buffers: the finished output rows of a chunk on their way out, and who has fetched them.
+constexpr int kOutPitch = 68;  // floats per staged row: 64 columns + 4, so the four rows of a 16-byte read hit different banks
+constexpr int oOut = 2 * kBufBytes, oFlag = oOut + kC * kOutPitch * 4, kLdsWalk = oFlag + 16;
+static_assert(kLdsWalk <= 163840, "two chunks of operands and one of output rows in the CU's LDS");
 
-// Two workgroups per (sequence, v-head), 64 of the 128 state columns each (with one, half the CUs stay idle at
-// B x nv = 128; the second reader of the common operands finds them in the L2 it shares with the first).
-// Wavefront w < 8: token tile w % 4 (also the 32-row dk slab of the state it owns) x column tiles 2*(w / 4), +1.
-// The A operands are common to the
-// wavefronts of a token tile, so they are fetched once per workgroup, one chunk ahead, and handed round through
-// LDS -- by wavefronts 8 and 9, which do nothing else: a wavefront that issues 1-KB loads waits behind the CU's
-// address unit (measured: ~2500 cycles per chunk for the 72 KB), and a computing wavefront that waits there holds
-// up every barrier of the chunk.  Only U is read by the wavefront that uses it.
-// NORM: the gated RMSNorm of the layer (RMSNormGated, qwen3_5.rs:305-313) in the epilogue -- the output rows leave as
-// bf16(o * rsqrt(mean(o^2) + eps) * w * silu(z)) instead of fp32 o.  A row's 128 columns belong to two workgroups, so
-// each publishes the sums of squares of its 64 columns per chunk (the exchange slots; reset by the prepare kernel) at the start of
-// the next chunk and reads the other's a chunk and a half later, long after it was written, so nothing waits.  Until
-// then the rows of a chunk stay in LDS (four chunks deep), and two more wavefronts, which do nothing else, finish
-// them: eight adjacent columns per lane with 16-byte loads of z and 16-byte stores (twelve wavefronts are still three
-// per SIMD, so they cost the others no registers).  The two workgroups must be resident together: the host launches this instance cooperatively (all
-// workgroups of a launch resident) and the wait for the other half is bounded all the same.
-constexpr int kRing = 4;     // chunks of output rows waiting in LDS for the other half's sums
-constexpr int kOPitch = 68;  // floats per staged output row: 64 columns + 4, so the four row groups of a store hit different banks
-constexpr int kNormSpin = 1 << 16;  // about 0.1 s: the other half is resident and at most a chunk apart
-// The scan kernel exists twice: deltanet_chunk_scan_kernel, and deltanet_chunk_scan_norm_kernel with the gated norm in
-// its epilogue.  One text, deltanet_chunk_scan.inc, included once with HS_SCAN_NORM 0 and once with 1 -- not one
-// template: with the norm's shared arrays, arguments or branches merely present (empty, unused or constant-false) the
-// compiler laid out LDS and ordered the chunk loop of the plain kernel differently, and it ran 5 % slower.
-#define HS_SCAN_NORM 0
-#include "deltanet_chunk_scan.inc"
-#undef HS_SCAN_NORM
-#define HS_SCAN_NORM 1
-#include "deltanet_chunk_scan.inc"
-#undef HS_SCAN_NORM
+// Transposed tile [feature d][token]: the eight-token (16-byte) pieces of a row are permuted by d / 16, so that the
+// threads of a wavefront, which write one token each for features 16 apart, hit different banks.
+__device__ __forceinline__ int tpos(int d, int tok) { return d * kPitchT + ((((tok >> 3) ^ (d >> 4)) & 7) << 3) + (tok & 7); }
+
+constexpr int kWalkThreads = 512;
+
+__global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsWalk];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int li = lane & 15, lq = lane >> 4;
+    // Workgroups go to the 8 XCDs round-robin by linear id, and each XCD has its own L2.  The two column halves of a
+    // (sequence, v-head) read the same triangles, and all v-heads of a k-head (both halves of each) the same q and k
+    // rows: the 2 * rep workgroups of a (sequence, k-head) get linear ids congruent mod 8, consecutive in that XCD's
+    // order, so that each of those comes from HBM once and the other readers find it in L2.
+    const int p = blockIdx.x, pairs = a.B * a.nv, rep = a.nv / a.nk;
+    int pair, half;
+    if (((a.B * a.nk) & 7) == 0) {
+        const int i = p >> 3, per = 2 * rep;
+        const int ku = (p & 7) + 8 * (i / per), sub = i % per;
+        pair = ku * rep + (sub >> 1);
+        half = sub & 1;
+    } else if ((pairs & 7) == 0) {
+        pair = (p & 7) + 8 * (p >> 4);
+        half = (p >> 3) & 1;
+    } else {
+        pair = p >> 1;
+        half = p & 1;
+    }
+    const int b = pair / a.nv, j = pair % a.nv, hk = j / rep;
+    const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
+    const uint8_t *wsp = a.ws + (int64_t)pair * kUnitBytes;  // + ci * chunk_stride
+    volatile int *flag = (volatile int *)(lds + oFlag);      // [0], [1]: the last chunk + 1 whose staged rows wavefront 2 / 3 has fetched
+
+    // Roles by wavefront (wavefront w runs on SIMD w % 4): 0 and 1 compute, one per SIMD; 2, 3, 6 and 7 bring in the k
+    // and q rows (the vector work of the loaders, on the two SIMDs without a computing wavefront) and 2 and 3 also carry
+    // the finished output rows from LDS to memory; 4 and 5 copy the triangles and v.  A computing wavefront issues no
+    // global access inside the walk: 32 four-byte stores per chunk cost it 2200 cycles of issue (a third of the chunk).
+    if (wave == 4 || wave == 5) {  // ---- N', M, v, e^(G63): thread ct of 128; plain copies, no arithmetic
+        const int ct = tid - 256;
+        struct Stage {
+            u32x4 nm[6], vr[4];
+            float dec;
+        };
+        auto fetch = [&](Stage &st, int ci) {
+            ci = min(ci, a.nc - 1);
+            const uint8_t *u = wsp + ci * chunk_stride;
+#pragma unroll
+            for (int i = 0; i < 6; ++i) st.nm[i] = *(const u32x4 *)(u + (ct + 128 * i) * 16);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // item = (token, eight columns of this half)
+                const int item = ct + 128 * i, tok = item >> 3, pc = item & 7;
+                const int64_t bt = (int64_t)b * a.T + min(ci * kC + tok, a.T - 1);
+                st.vr[i] = __builtin_nontemporal_load((const u32x4 *)(a.v + (bt * a.nv + j) * kWD + 64 * half + 8 * pc));
+            }
+            st.dec = *(const float *)(u + kOffDecay);
+        };
+        auto put = [&](const Stage &st, int ci, uint8_t *buf) {
+#pragma unroll
+            for (int i = 0; i < 6; ++i) *(u32x4 *)(buf + oNt + (ct + 128 * i) * 16) = st.nm[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int item = ct + 128 * i, tok = item >> 3, pc = item & 7;
+                const bool valid = ci * kC + tok < a.T;  // rows past T are zero
+                // eight bf16 as they are: one 16-byte piece of an A operand block of the bf16 MFMA (row = token, k-slots =
+                // columns, natural order); the piece of lane (li, lq) sits at 4 li + lq, so that the eight tokens x four
+                // pieces a wavefront writes are contiguous
+                *(u32x4 *)(buf + oV + (((tok >> 4) * 2 + (pc >> 2)) * 64 + (tok & 15) * 4 + (pc & 3)) * 16) =
+                    valid ? st.vr[i] : (u32x4){0u, 0u, 0u, 0u};
+            }
+            if (ct == 0) *(float *)(buf + oDec) = st.dec;
+        };
+        // Round c (after the barrier that publishes chunk c): chunk c + 1 goes into the other operand buffer, chunk c + 3
+        // is requested.
+        auto round = [&](Stage &st, int c) {
+            lds_sync();
+            if (c + 1 < a.nc) {
+                put(st, c + 1, lds + ((c + 1) & 1) * kBufBytes);
+                fetch(st, c + 3);
+            }
+        };
+        Stage sa, sb;
+        fetch(sa, 0);
+        fetch(sb, 1);
+        put(sa, 0, lds);
+        fetch(sa, 2);
+        for (int c = 0; c <= a.nc; c += 2) {  // chunk c + 1 comes from sb in even rounds, from sa in odd ones
+            round(sb, c);
+            if (c + 1 <= a.nc) round(sa, c + 1);
+        }
+        return;
+    }
+    if (wave >= 2) {
+        // ---- k and q rows: thread = (token tl and tl + 32, dk 8 part .. + 7 and 64 + 8 part .. + 7: the eight threads
+        //      of a token read whole 128-byte lines)
+        const int lt = ((wave & 1) | ((wave >> 2) << 1)) * 64 + lane, tl = lt >> 3, part = lt & 7;
+        if (lt == 0) { flag[0] = 0; flag[1] = 0; }  // visible to the computing wavefronts after the first barrier
+        struct Stage {
+            u32x4 kr[2][2], qr[2][2];
+            float fn[2], fq[2], ft[2];
+        };
+        auto fetch = [&](Stage &st, int ci) {
+            ci = min(ci, a.nc - 1);
+            const uint8_t *u = wsp + ci * chunk_stride;
+#pragma unroll
+            for (int ps = 0; ps < 2; ++ps) {
+                const int tok = tl + 32 * ps;
+                const int64_t bt = (int64_t)b * a.T + min(ci * kC + tok, a.T - 1);
+                const uint16_t *kp = a.k + (bt * a.nk + hk) * kWD + 8 * part;
+                const uint16_t *qp = a.q + (bt * a.nk + hk) * kWD + 8 * part;
+                st.kr[ps][0] = *(const u32x4 *)kp;
+                st.kr[ps][1] = *(const u32x4 *)(kp + 64);
+                st.qr[ps][0] = *(const u32x4 *)qp;
+                st.qr[ps][1] = *(const u32x4 *)(qp + 64);
+                st.fn[ps] = *(const float *)(u + kOffFn + 4 * tok);  // zero for rows past T
+                st.fq[ps] = *(const float *)(u + kOffFq + 4 * tok);
+                st.ft[ps] = *(const float *)(u + kOffFt + 4 * tok);
+            }
+        };
+        auto put = [&](const Stage &st, uint8_t *buf) {
+            _Float16 *KT = (_Float16 *)(buf + oKt);
+#pragma unroll
+            for (int ps = 0; ps < 2; ++ps) {
+                const int tok = tl + 32 * ps;
+                float kf[16], qf[16];  // elements 0-7: dk 8 part + e, 8-15: dk 64 + 8 part + e
+                unpack16(st.kr[ps][0], st.kr[ps][1], kf);
+                unpack16(st.qr[ps][0], st.qr[ps][1], qf);
+                const float fn = st.fn[ps], fq = st.fq[ps], ft = st.ft[ps];
+#pragma unroll
+                for (int h8 = 0; h8 < 2; ++h8) {
+                    // dk 64 h8 + 8 part + e: slab 2 h8 + part / 4; inside the slab at 8 (part % 4) + e, i.e. the tile of
+                    // the slab (slots 0-3 or 4-7) is (part / 2) % 2 and the row groups are lq = 2 (part % 2), + 1
+                    const int blk = (tok >> 4) * 4 + 2 * h8 + (part >> 2);
+                    const int o = blk * 1024 + (2 * (part & 1) * 16 + (tok & 15)) * 16 + 8 * ((part >> 1) & 1);
+#pragma unroll
+                    for (int g4 = 0; g4 < 2; ++g4) {
+                        half4v hn, hq;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int i = 8 * h8 + 4 * g4 + e;
+                            hn[e] = (_Float16)(kf[i] * fn);
+                            hq[e] = (_Float16)(qf[i] * fq);
+                            KT[tpos(64 * h8 + 8 * part + 4 * g4 + e, tok)] = (_Float16)(kf[i] * ft);
+                        }
+                        *(half4v *)(buf + oKn + o + g4 * 256) = hn;
+                        *(half4v *)(buf + oQg + o + g4 * 256) = hq;
+                    }
+                }
+            }
+        };
+        // Two chunks of rows are in flight in registers: what is written into LDS for chunk c + 1 was requested while
+        // chunk c - 1 was being computed.
+        // Round c (after the barrier that publishes chunk c).  Wavefronts 2 and 3 (thread lt of 128) first take the
+        // staged rows of chunk c - 1 into registers and release the staging area.  Then chunk c + 1 goes into the other
+        // operand buffer; the rows leave for memory, 16 B per lane (16 lanes cover the 256 bytes this half owns of a
+        // token's row); chunk c + 3 is requested.
+        auto round = [&](Stage &st, int c) {
+            lds_sync();
+            u32x4 orow[8];
+            const bool carry = wave < 4 && c >= 1;
+            if (carry) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int pc = lt + 128 * i;
+                    orow[i] = *(const u32x4 *)(lds + oOut + ((pc >> 4) * kOutPitch + 4 * (pc & 15)) * 4);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (lane == 0) flag[wave - 2] = c;
+            }
+            if (c + 1 < a.nc) put(st, lds + ((c + 1) & 1) * kBufBytes);
+            if (carry) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int pc = lt + 128 * i, t = (c - 1) * kC + (pc >> 4);
+                    if (t < a.T) __builtin_nontemporal_store(orow[i], (u32x4 *)(a.out + (((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + 4 * (pc & 15)));
+                }
+            }
+            if (c + 1 < a.nc) fetch(st, c + 3);
+        };
+        Stage sa, sb;
+        fetch(sa, 0);
+        fetch(sb, 1);
+        put(sa, lds);
+        fetch(sa, 2);
+        for (int c = 0; c <= a.nc; c += 2) {
+            round(sb, c);
+            if (c + 1 <= a.nc) round(sa, c + 1);
+        }
+        return;
+    }
+
+    // ---- the two computing wavefronts: wavefront w owns state columns 64 half + 32 w .. + 31 (two 16-column tiles c)
+    const int col = 64 * half + 32 * wave + li;
+    float4v S[8][2];  // dk tile x: rows 16 x + 4 lq + r
+    float *sp = a.state + ((int64_t)pair * kWD) * kWD + col;
+#pragma unroll
+    for (int x = 0; x < 8; ++x)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) S[x][c][r] = sp[(int64_t)(16 * x + 4 * lq + r) * kWD + 16 * c];
+    // the B operands (bf16, like v itself) that pick column tile c out of this wavefront's 32-column slab of v
+    bf16x8 pick[2];
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pick[c][e] = (__bf16)(8 * lq + e == 16 * c + li ? 1.0f : 0.0f);
+    const float4v zero = {0.f, 0.f, 0.f, 0.f};
+    float *stage = (float *)(lds + oOut) + (4 * lq) * kOutPitch + 32 * wave + li;  // + (16 tt + r) * kOutPitch + 16 c
+
+#define HS_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, C, 0, 0, 0)
+    // One chunk.  Every A operand read from LDS feeds two products (the two column tiles), and the reads of a group of
+    // eight products are issued one group ahead (the scheduling barriers keep the compiler from sinking each read to
+    // its use, which would serialise read latency and MFMA).
+    for (int ci = 0; ci < a.nc; ++ci) {
+        lds_sync();
+        const uint8_t *buf = lds + (ci & 1) * kBufBytes;
+        auto opA = [&](int off, int blk) { return *(const half8 *)(buf + off + blk * 1024 + lane * 16); };
+        const _Float16 *KT = (const _Float16 *)(buf + oKt);
+        auto opKt = [&](int x, int s) {  // (k e^(G63-G))^T: row dk 16 x + li, k-slots = tokens of slab s in accumulator order
+            const half4v lo = *(const half4v *)&KT[tpos(16 * x + li, 32 * s + 4 * lq)];
+            const half4v hi = *(const half4v *)&KT[tpos(16 * x + li, 32 * s + 16 + 4 * lq)];
+            return (half8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        };
+        float4v X[4][2], V[4][2];
+        half8 an[2][4], nt[6], sh[2];
+        bf16x8 va[4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            va[tt] = *(const bf16x8 *)(buf + oV + (tt * 2 + wave) * 1024 + (li * 4 + lq) * 16);
+            an[0][tt] = opA(oKn, tt * 4);
+        }
+        const float dec = *(const float *)(buf + oDec);
+        __builtin_amdgcn_sched_barrier(0);
+        // X = v - (k e^G) S
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) X[tt][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[tt], pick[c], zero, 0, 0, 0);
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {  // dk slab sl
+            if (sl < 3) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) an[(sl + 1) & 1][tt] = opA(oKn, tt * 4 + sl + 1);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 6; ++i) nt[i] = opA(oNt, i);
+            }
+#pragma unroll
+            for (int c = 0; c < 2; ++c) sh[c] = f32x8_to_half8(S[2 * sl][c], S[2 * sl + 1][c]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) X[tt][c] = HS_MFMA(an[sl & 1][tt], sh[c], X[tt][c]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        half8 aq[2][4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) aq[0][tt] = opA(oQg, tt * 4);
+        half8 Xh[2][2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            Xh[0][c] = f32x8_to_half8(X[0][c], X[1][c]);
+            Xh[1][c] = f32x8_to_half8(X[2][c], X[3][c]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // V' = N' X (N' is lower triangular: token tiles 0 and 1 see only the first slab)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            V[0][c] = HS_MFMA(nt[tri_block(0, 0)], Xh[0][c], zero);
+            V[1][c] = HS_MFMA(nt[tri_block(1, 0)], Xh[0][c], zero);
+            V[2][c] = HS_MFMA(nt[tri_block(2, 0)], Xh[0][c], zero);
+            V[3][c] = HS_MFMA(nt[tri_block(3, 0)], Xh[0][c], zero);
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            V[2][c] = HS_MFMA(nt[tri_block(2, 1)], Xh[1][c], V[2][c]);
+            V[3][c] = HS_MFMA(nt[tri_block(3, 1)], Xh[1][c], V[3][c]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // O = (q e^G) S + M V'
+        float4v O[4][2];
+        half8 qm[6], kt[2][4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) O[tt][c] = zero;
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            if (sl < 3) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt) aq[(sl + 1) & 1][tt] = opA(oQg, tt * 4 + sl + 1);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 6; ++i) qm[i] = opA(oQK, i);
+            }
+#pragma unroll
+            for (int c = 0; c < 2; ++c) sh[c] = f32x8_to_half8(S[2 * sl][c], S[2 * sl + 1][c]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int c = 0; c < 2; ++c) O[tt][c] = HS_MFMA(aq[sl & 1][tt], sh[c], O[tt][c]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kt[0][i] = opKt(i >> 1, i & 1);
+        half8 Vh[2][2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            Vh[0][c] = f32x8_to_half8(V[0][c], V[1][c]);
+            Vh[1][c] = f32x8_to_half8(V[2][c], V[3][c]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            O[0][c] = HS_MFMA(qm[tri_block(0, 0)], Vh[0][c], O[0][c]);
+            O[1][c] = HS_MFMA(qm[tri_block(1, 0)], Vh[0][c], O[1][c]);
+            O[2][c] = HS_MFMA(qm[tri_block(2, 0)], Vh[0][c], O[2][c]);
+            O[3][c] = HS_MFMA(qm[tri_block(3, 0)], Vh[0][c], O[3][c]);
+        }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            O[2][c] = HS_MFMA(qm[tri_block(2, 1)], Vh[1][c], O[2][c]);
+            O[3][c] = HS_MFMA(qm[tri_block(3, 1)], Vh[1][c], O[3][c]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) kt[1][i] = opKt(2 + (i >> 1), i & 1);
+#pragma unroll
+        for (int x = 0; x < 8; ++x)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) S[x][c] *= dec;
+        __builtin_amdgcn_sched_barrier(0);
+        // S <- e^(G63) S + (k e^(G63-G))^T V', two dk tiles at a time
+#pragma unroll
+        for (int xp = 0; xp < 4; ++xp) {
+#pragma unroll
+            for (int sl = 0; sl < 2; ++sl)
+#pragma unroll
+                for (int xo = 0; xo < 2; ++xo)
+#pragma unroll
+                    for (int c = 0; c < 2; ++c)
+                        S[2 * xp + xo][c] = HS_MFMA(kt[xp & 1][2 * xo + sl], Vh[sl][c], S[2 * xp + xo][c]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (xp < 2) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) kt[xp & 1][i] = opKt(2 * (xp + 2) + (i >> 1), i & 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // The finished rows go to the staging area once the rows of the chunk before have been taken out of it (they
+        // were, right after this chunk's barrier: the wait is there for the guarantee, not for the time).
+        if (ci > 0)
+            while (flag[0] < ci || flag[1] < ci) __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int c = 0; c < 2; ++c)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) stage[(16 * tt + r) * kOutPitch + 16 * c] = O[tt][c][r];
+    }
+#undef HS_MFMA
+    lds_sync();  // the last chunk's rows are staged: wavefronts 4 and 5 take them from here
+    float *sq = sp;  // opaque to the compiler: it would otherwise keep the 64 addresses of the first loads alive (spilled) across the walk
+    asm volatile("" : "+v"(sq));
+#pragma unroll
+    for (int x = 0; x < 8; ++x)
+#pragma unroll
+        for (int c = 0; c < 2; ++c)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sq[(int64_t)(16 * x + 4 * lq + r) * kWD + 16 * c] = S[x][c][r];
+}
 
 }  // namespace hs
 
@@ -438,46 +691,54 @@ extern "C" {
 
 size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv) {
     if (B <= 0 || T <= 0 || nk <= 0 || nv <= 0) return 0;
-    return (size_t)((T + hs::kC - 1) / hs::kC) * ((size_t)B * nk * hs::kHeadBytes + (size_t)B * nv * (hs::kUnitBytes + hs::kSsqBytes));
+    return (size_t)((T + hs::kC - 1) / hs::kC) * (size_t)B * nv * hs::kUnitBytes;
 }
 
-static int chunked_common(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
-                          int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv, float q_scale, int l2norm,
-                          void *workspace, size_t workspace_bytes, hs::ChunkArgs &a) {
+// ... plus the fp32 output rows between the walk and the norm
+size_t hs_deltanet_chunked_gated_norm_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv) {
+    if (B <= 0 || T <= 0 || nk <= 0 || nv <= 0) return 0;
+    return ((hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) + 255) & ~(size_t)255) + (size_t)B * T * nv * hs::kWD * sizeof(float);
+}
+
+static int chunked_launch(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
+                          float *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv, float q_scale,
+                          int l2norm, void *workspace, hipStream_t st) {
     using namespace hs;
-    if (B > 0 && T > 0 && (!q || !k || !v || !g || !beta || !state)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    WalkArgs a{};
+    a.q = (const uint16_t *)q; a.k = (const uint16_t *)k; a.v = (const uint16_t *)v;
+    a.g = g; a.beta = beta; a.state = state; a.out = out; a.ws = (uint8_t *)workspace;
+    a.B = B; a.T = T; a.nk = nk; a.nv = nv; a.nc = (T + kC - 1) / kC; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
+    deltanet_chunk_factor_kernel<<<(unsigned)((int64_t)B * nv * a.nc), 512, 0, st>>>(a);
+    if (int rc = check_launch("deltanet_chunk_factor")) return rc;
+    deltanet_chunk_walk_kernel<<<(unsigned)(2 * B * nv), kWalkThreads, 0, st>>>(a);
+    return check_launch("deltanet_chunk_walk");
+}
+
+// Argument checks common to both entry points; -1 = go on.
+static int chunked_check(const void *q, const void *k, const void *v, const float *g, const float *beta, const float *state,
+                         const void *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
+                         const void *workspace, size_t workspace_bytes, size_t need) {
+    using namespace hs;
+    if (B > 0 && T > 0 && (!q || !k || !v || !g || !beta || !state || !out)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
     if (dk != kWD || dv != kWD) return fail(HS_ERR_INVALID_ARGUMENT, "deltanet is built for dk = dv = 128, got %d x %d", dk, dv);
     if (B < 0 || T < 0 || nk <= 0 || nv <= 0 || nv % nk != 0)
         return fail(HS_ERR_INVALID_ARGUMENT, "bad shape B=%d T=%d nk=%d nv=%d (need nv %% nk == 0)", B, T, nk, nv);
     if (B == 0 || T == 0) return HS_OK;
     const int64_t units = (int64_t)B * nv * ((T + kC - 1) / kC);
     if (units > INT32_MAX || (int64_t)B * nv > (1 << 29)) return fail(HS_ERR_INVALID_ARGUMENT, "too many chunks (%lld)", (long long)units);
-    const size_t need = hs_deltanet_chunked_workspace_bytes(B, T, nk, nv);
     if (!workspace || workspace_bytes < need) return fail(HS_ERR_WORKSPACE, "workspace of %zu bytes given, %zu needed", workspace_bytes, need);
-    if ((((uintptr_t)workspace | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) != 0)
-        return fail(HS_ERR_INVALID_ARGUMENT, "q, k, v and the workspace must be 16-byte aligned");
-    a = ChunkArgs{};
-    a.q = (const uint16_t *)q; a.k = (const uint16_t *)k; a.v = (const uint16_t *)v;
-    a.g = g; a.beta = beta; a.state = state; a.ws = (uint8_t *)workspace;
-    a.B = B; a.T = T; a.nk = nk; a.nv = nv; a.nc = (T + kC - 1) / kC; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
-    a.b_base = 0; a.b_count = B;
-    return -1;  // go on
+    if ((((uintptr_t)workspace | (uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "q, k, v, out and the workspace must be 16-byte aligned");
+    return -1;
 }
 
 int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
                                 float *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
                                 float q_scale, int l2norm, void *workspace, size_t workspace_bytes, hs_stream_t stream) {
-    using namespace hs;
-    if (B > 0 && T > 0 && !out) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
-    ChunkArgs a;
-    if (int rc = chunked_common(q, k, v, g, beta, state, B, T, nk, nv, dk, dv, q_scale, l2norm, workspace, workspace_bytes, a); rc >= 0)
+    if (int rc = chunked_check(q, k, v, g, beta, state, out, B, T, nk, nv, dk, dv, workspace, workspace_bytes,
+                               hs_deltanet_chunked_workspace_bytes(B, T, nk, nv)); rc >= 0)
         return rc;
-    a.out = out;
-    hipStream_t st = (hipStream_t)stream;
-    deltanet_chunk_prepare_kernel<<<(unsigned)((int64_t)B * nv * a.nc), 512, 0, st>>>(a);
-    if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
-    deltanet_chunk_scan_kernel<<<(unsigned)(2 * B * nv), kScanThreads, 0, st>>>(a);
-    return check_launch("deltanet_chunk_scan");
+    return chunked_launch(q, k, v, g, beta, state, out, B, T, nk, nv, dk, dv, q_scale, l2norm, workspace, (hipStream_t)stream);
 }
 
 int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const void *v, const float *g, const float *beta,
@@ -486,56 +747,16 @@ int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const v
                                            float q_scale, int l2norm, void *workspace, size_t workspace_bytes,
                                            hs_stream_t stream) {
     using namespace hs;
-    if (B > 0 && T > 0 && (!out || !z || !norm_weight)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
-    ChunkArgs a;
-    if (int rc = chunked_common(q, k, v, g, beta, state, B, T, nk, nv, dk, dv, q_scale, l2norm, workspace, workspace_bytes, a); rc >= 0)
+    if (B > 0 && T > 0 && (!z || !norm_weight)) return fail(HS_ERR_INVALID_ARGUMENT, "null buffer");
+    if (int rc = chunked_check(q, k, v, g, beta, state, out, B, T, nk, nv, dk, dv, workspace, workspace_bytes,
+                               hs_deltanet_chunked_gated_norm_workspace_bytes(B, T, nk, nv)); rc >= 0)
         return rc;
-    if ((((uintptr_t)z | (uintptr_t)norm_weight | (uintptr_t)out) & 15) != 0)
-        return fail(HS_ERR_INVALID_ARGUMENT, "z, norm_weight and out must be 16-byte aligned");
-    a.z = (const uint16_t *)z; a.norm_w = norm_weight; a.norm_eps = norm_eps; a.out_norm = (uint16_t *)out;
-    // The two workgroups of a (sequence, v-head) wait for each other once per chunk, so every workgroup of a scan
-    // launch has to be resident: a cooperative launch, over as many whole sequences as the device holds at a time.
-    // (what the device holds is looked up once per device; a second thread doing the same stores the same values)
-    constexpr int kMaxDevices = 64;
-    static int resident_of[kMaxDevices];  // 0: not asked yet, -1: no cooperative launches, else workgroups resident at once
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-        (void)hipGetLastError();
-        return fail(HS_ERR_LAUNCH, "cannot query the device for a cooperative launch");
-    }
-    if (resident_of[dev] == 0) {
-        int cus = 0, per_cu = 0, coop = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-            hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev) != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, deltanet_chunk_scan_norm_kernel, kScanNormThreads, 0) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(HS_ERR_LAUNCH, "cannot query the device for a cooperative launch");
-        }
-        resident_of[dev] = coop ? std::max(1, cus * per_cu) : -1;
-    }
-    if (resident_of[dev] < 0)
-        return fail(HS_ERR_LAUNCH, "the device does not support cooperative launches: run hs_deltanet_forward_chunked and hs_deltanet_gated_norm");
-    const int64_t resident = resident_of[dev];
-    if (resident < 2 * (int64_t)nv)
-        return fail(HS_ERR_INVALID_ARGUMENT,
-                    "%d v-heads need %d workgroups resident at once, the device holds %lld: run hs_deltanet_forward_chunked "
-                    "and hs_deltanet_gated_norm", nv, 2 * nv, (long long)resident);
-    hipStream_t st = (hipStream_t)stream;
-    deltanet_chunk_prepare_kernel<<<(unsigned)((int64_t)B * nv * a.nc), 512, 0, st>>>(a);
-    if (int rc = check_launch("deltanet_chunk_prepare")) return rc;
-    const int per_launch = (int)std::min<int64_t>(B, resident / (2 * nv));
-    for (int b0 = 0; b0 < B; b0 += per_launch) {
-        a.b_base = b0;
-        a.b_count = std::min(per_launch, B - b0);
-        void *args[] = {&a};
-        const hipError_t e = hipLaunchCooperativeKernel((const void *)deltanet_chunk_scan_norm_kernel, dim3((unsigned)(2 * a.b_count * nv)),
-                                                        dim3(kScanNormThreads), args, 0, st);
-        if (e != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(HS_ERR_LAUNCH, "deltanet_chunk_scan (cooperative): %s", hipGetErrorString(e));
-        }
-    }
-    return HS_OK;
+    if ((((uintptr_t)z | (uintptr_t)norm_weight) & 15) != 0)
+        return fail(HS_ERR_INVALID_ARGUMENT, "z and norm_weight must be 16-byte aligned");
+    float *rows = (float *)((uint8_t *)workspace + ((hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) + 255) & ~(size_t)255));
+    if (int rc = chunked_launch(q, k, v, g, beta, state, rows, B, T, nk, nv, dk, dv, q_scale, l2norm, workspace, (hipStream_t)stream))
+        return rc;
+    return hs_deltanet_gated_norm(rows, z, norm_weight, norm_eps, out, (int64_t)B * T * nv, dv, stream);
 }
 
 }  // extern "C"

@@ -275,13 +275,14 @@ int hs_deltanet_gated_norm(const float *x, const void *z, const float *weight, f
     return check_launch("gated_rmsnorm");
 }
 
-// The prompt branch of the layer as one call: three launches in a row, the intermediate tensors in the workspace.
+// The prompt branch of the layer as one call: the launches of the three steps in a row, the intermediate tensors in the
+// workspace.
 static size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
 size_t hs_deltanet_prefill_layer_workspace_bytes(int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv) {
     if (B <= 0 || S <= 0 || nk <= 0 || nv <= 0 || dk <= 0 || dv <= 0) return 0;
     const size_t bs = (size_t)B * S;
-    return align256(hs_deltanet_chunked_workspace_bytes(B, S, nk, nv)) + 2 * align256(bs * nk * dk * 2) + align256(bs * nv * dv * 2) +
+    return align256(hs_deltanet_chunked_gated_norm_workspace_bytes(B, S, nk, nv)) + 2 * align256(bs * nk * dk * 2) + align256(bs * nv * dv * 2) +
            2 * align256(bs * nv * 4);
 }
 
@@ -300,7 +301,7 @@ int hs_deltanet_prefill_layer(const void *mixed_qkv, const void *conv_weight, co
     const size_t bs = (size_t)B * S;
     uint8_t *p = (uint8_t *)workspace;
     void *chunk_ws = p;
-    const size_t chunk_bytes = hs_deltanet_chunked_workspace_bytes(B, S, nk, nv);
+    const size_t chunk_bytes = hs_deltanet_chunked_gated_norm_workspace_bytes(B, S, nk, nv);
     p += align256(chunk_bytes);
     void *q = p; p += align256(bs * nk * dk * 2);
     void *k = p; p += align256(bs * nk * dk * 2);

@@ -358,27 +358,25 @@ HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, cons
                         float q_scale, int l2norm, hs_stream_t stream);
 
 /* The same function over a prompt in the reference's chunked form (chunked_delta_rule, qwen3_5.rs:342-498, chunk
- * size 64) on the matrix pipe: per chunk the triangular system (I + tril(beta k k^T decay))^-1 is solved in fp32,
- * everything else is fp16-operand / fp32-accumulate MFMA.  Mathematically identical to hs_deltanet_forward; outputs
- * and the final state differ from it by rounding (about 1e-3 relative).  Arguments as hs_deltanet_forward, plus a
- * device workspace of hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) bytes (per 64-token chunk: 32,768 per
- * (sequence, k-head) and 41,728 + 512 per (sequence, v-head)), 16-byte aligned, owned by the caller; q, k, v must be
- * 16-byte aligned.  A prompt split into calls of a multiple
- * of 64 tokens (state carried through `state`) gives the bits of one call. */
+ * size 64) on the matrix pipe: per chunk the triangular system (I + tril(beta k k^T decay))^-1 is inverted (diagonal
+ * blocks with fp32 accumulation, the rest by block substitution), everything else is fp16-operand / fp32-accumulate
+ * MFMA.  Mathematically identical to hs_deltanet_forward; outputs and the final state differ from it by rounding
+ * (about 1e-3 relative).  Arguments as hs_deltanet_forward, plus a device workspace of
+ * hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) bytes (13,312 per 64-token chunk and (sequence, v-head): the two
+ * triangular factors of the chunk and three vectors), 16-byte aligned, owned by the caller; q, k, v and out must be
+ * 16-byte aligned.  A prompt split into calls of a multiple of 64 tokens (state carried through `state`) gives the
+ * bits of one call. */
 HS_API size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv);
 HS_API int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, const float *g, const float *beta,
                         float *state, float *out,
                         int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
                         float q_scale, int l2norm, void *workspace, size_t workspace_bytes, hs_stream_t stream);
-/* hs_deltanet_forward_chunked with the layer's gated RMSNorm (RMSNormGated::forward, qwen3_5.rs:305-313; what
- * hs_deltanet_gated_norm computes) in the epilogue: out [B, T, nv, dv] bf16 = bf16(o * rsqrt(mean(o^2) + eps) * weight *
- * silu(z)) with z [B, T, nv, dv] bf16 and weight [dv] fp32 (both, and out, 16-byte aligned); the fp32 rows o are never
- * written.  Same workspace.  Equal
- * to the two calls up to the order in which a row's squares are added (one bf16 ulp, rarely).  The two workgroups that
- * share a row exchange their sums through the workspace, so the scan is a cooperative launch (all its workgroups
- * resident; several launches when the batch needs more than the device holds): not capturable in a HIP graph, and
- * HS_ERR_LAUNCH where the device has no cooperative launches, HS_ERR_INVALID_ARGUMENT when 2 * nv workgroups do not
- * fit the device at once -- run the two calls then. */
+/* hs_deltanet_forward_chunked followed by the layer's gated RMSNorm (RMSNormGated::forward, qwen3_5.rs:305-313; what
+ * hs_deltanet_gated_norm computes) as one call: out [B, T, nv, dv] bf16 = bf16(o * rsqrt(mean(o^2) + eps) * weight *
+ * silu(z)) with z [B, T, nv, dv] bf16 and weight [dv] fp32 (both, and out, 16-byte aligned).  The fp32 rows o pass
+ * through the workspace, which is therefore larger: hs_deltanet_chunked_gated_norm_workspace_bytes.  Results are those
+ * of the two calls bit for bit; three ordinary launches (capturable in a HIP graph). */
+HS_API size_t hs_deltanet_chunked_gated_norm_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv);
 HS_API int hs_deltanet_forward_chunked_gated_norm(const void *q, const void *k, const void *v, const float *g,
                         const float *beta, float *state, const void *z, const float *norm_weight, float norm_eps,
                         void *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv,
@@ -419,10 +417,10 @@ HS_API int hs_deltanet_decode_layer(const void *mixed_qkv, const void *conv_weig
                                     float q_scale, int l2norm, hs_stream_t stream);
 
 /* The prompt branch of GatedDeltaNetLayer::forward between the two projections as ONE call (qwen3_5.rs:629-686, :753-769,
- * :771-786): hs_deltanet_prepare + hs_deltanet_forward_chunked_gated_norm, three launches in a row with q, k, v, g, beta
- * and the chunk operands in the workspace (hs_deltanet_prefill_layer_workspace_bytes, 256-byte aligned); arguments and
- * results as those calls (mixed_qkv [B, S, C], z and out [B, S, nv, dv] bf16), limits as
- * hs_deltanet_forward_chunked_gated_norm.  The counterpart of hs_deltanet_decode_layer for seq > 1. */
+ * :771-786): hs_deltanet_prepare + hs_deltanet_forward_chunked_gated_norm, five launches in a row with q, k, v, g, beta,
+ * the chunk factors and the fp32 output rows in the workspace (hs_deltanet_prefill_layer_workspace_bytes, 256-byte
+ * aligned); arguments and results as those calls (mixed_qkv [B, S, C], z and out [B, S, nv, dv] bf16).  The
+ * counterpart of hs_deltanet_decode_layer for seq > 1. */
 HS_API size_t hs_deltanet_prefill_layer_workspace_bytes(int32_t B, int32_t S, int32_t nk, int32_t nv, int32_t dk, int32_t dv);
 HS_API int hs_deltanet_prefill_layer(const void *mixed_qkv, const void *conv_weight, const void *conv_state_in,
                                      void *conv_state_out, const void *a_in, const void *b_in, const float *neg_a_exp,

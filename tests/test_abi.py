@@ -187,10 +187,13 @@ def test_format_names_are_distinct_and_stable():
 def test_workspace_sizes_are_host_arithmetic():
     """The workspace functions need no GPU: sizes a caller can plan with."""
     # chunked delta rule: per 64-token chunk 32,768 B per (sequence, k-head) and 42,240 B per (sequence, v-head)
-    assert hb.deltanet_chunked_workspace_bytes(4, 4096, 16, 32) == 64 * (4 * 16 * 32768 + 4 * 32 * 42240)
-    assert hb.deltanet_chunked_workspace_bytes(1, 1, 1, 1) == 32768 + 42240
-    assert hb.deltanet_chunked_workspace_bytes(1, 65, 2, 4) == 2 * (2 * 32768 + 4 * 42240)
+    assert hb.deltanet_chunked_workspace_bytes(4, 4096, 16, 32) == 64 * 4 * 32 * 13312  # per chunk and (sequence, v-head)
+    assert hb.deltanet_chunked_workspace_bytes(1, 1, 1, 1) == 13312
+    assert hb.deltanet_chunked_workspace_bytes(1, 65, 2, 4) == 2 * 4 * 13312
     assert hb.deltanet_chunked_workspace_bytes(0, 64, 1, 1) == 0
+    # with the norm: the fp32 output rows behind the factors (256-byte aligned)
+    assert hb.deltanet_chunked_gated_norm_workspace_bytes(1, 65, 2, 4) == 2 * 4 * 13312 + 65 * 4 * 128 * 4
+    assert hb.deltanet_chunked_gated_norm_workspace_bytes(0, 64, 1, 1) == 0
     # decode: room for (D + 2) floats per (sequence, query head, chunk), a multiple of 256 bytes, growing with head_dim
     small, big = hb.decode_workspace_bytes(64, 32, 8, 128, 8192), hb.decode_workspace_bytes(64, 32, 8, 256, 8192)
     assert small % 256 == 0 and big % 256 == 0 and big > small >= 64 * 32 * 130 * 4

@@ -116,7 +116,7 @@ def test_workspace_and_shape_errors():
     st = torch.zeros(1, 2, 128, 128, device=DEV)
     out = torch.empty(1, 70, 2, 128, device=DEV)
     need = hb.deltanet_chunked_workspace_bytes(1, 70, 1, 2)
-    assert need == 2 * (1 * 32768 + 2 * 42240)  # per chunk: one k-head block and two v-head blocks
+    assert need == 2 * 2 * 13312  # per chunk and v-head: the two triangular factors and three vectors
     small = torch.empty(need - 1, dtype=torch.uint8, device=DEV)
     with pytest.raises(hb.HsError) as e:
         hb.deltanet_forward_chunked(q, k, v, g, beta, st, out, 1.0, True, workspace=small)
