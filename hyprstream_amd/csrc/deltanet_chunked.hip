@@ -307,8 +307,8 @@ constexpr int oDec = oV + 8192;               // e^(G63)
 constexpr int kBufBytes = oDec + 16;
 // Behind the two operand buffers: the finished output rows of a chunk on their way out, and who has fetched them.
 constexpr int kOutPitch = 68;  // floats per staged row: 64 columns + 4, so the four rows of a 16-byte read hit different banks
-constexpr int oOut = 2 * kBufBytes, oFlag = oOut + kC * kOutPitch * 4, kLdsWalk = oFlag + 16;
-static_assert(kLdsWalk <= 163840, "two chunks of operands and one of output rows in the CU's LDS");
+constexpr int oOut = 2 * kBufBytes, kLdsWalk = oOut + kC * kOutPitch * 4;
+static_assert(kLdsWalk + 16 <= 163840, "two chunks of operands and one of output rows in the CU's LDS");
 
 // Transposed tile [feature d][token]: the eight-token (16-byte) pieces of a row are permuted by d / 16, so that the
 // threads of a wavefront, which write one token each for features 16 apart, hit different banks.
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
     const int b = pair / a.nv, j = pair % a.nv, hk = j / rep;
     const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
     const uint8_t *wsp = a.ws + (int64_t)pair * kUnitBytes;  // + ci * chunk_stride
-    volatile int *flag = (volatile int *)(lds + oFlag);      // [0], [1]: the last chunk + 1 whose staged rows wavefront 2 / 3 has fetched
+    __shared__ int flag[2];  // the last chunk + 1 whose staged rows wavefront 2 / 3 has fetched
 
     // Roles by wavefront (wavefront w runs on SIMD w % 4): 0 and 1 compute, one per SIMD; 2, 3, 6 and 7 bring in the k
     // and q rows (the vector work of the loaders, on the two SIMDs without a computing wavefront) and 2 and 3 also carry
@@ -406,7 +406,10 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         // ---- k and q rows: thread = (token tl and tl + 32, dk 8 part .. + 7 and 64 + 8 part .. + 7: the eight threads
         //      of a token read whole 128-byte lines)
         const int lt = ((wave & 1) | ((wave >> 2) << 1)) * 64 + lane, tl = lt >> 3, part = lt & 7;
-        if (lt == 0) { flag[0] = 0; flag[1] = 0; }  // visible to the computing wavefronts after the first barrier
+        if (lt == 0) {  // visible to the computing wavefronts after the first barrier
+            flag[0] = 0;
+            flag[1] = 0;
+        }
         struct Stage {
             u32x4 kr[2][2], qr[2][2];
             float fn[2], fq[2], ft[2];
@@ -477,7 +480,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
                     orow[i] = *(const u32x4 *)(lds + oOut + ((pc >> 4) * kOutPitch + 4 * (pc & 15)) * 4);
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (lane == 0) flag[wave - 2] = c;
+                if (lane == 0) __hip_atomic_store(&flag[wave - 2], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             }
             if (c + 1 < a.nc) put(st, lds + ((c + 1) & 1) * kBufBytes);
             if (carry) {
@@ -665,7 +668,9 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         // The finished rows go to the staging area once the rows of the chunk before have been taken out of it (they
         // were, right after this chunk's barrier: the wait is there for the guarantee, not for the time).
         if (ci > 0)
-            while (flag[0] < ci || flag[1] < ci) __builtin_amdgcn_s_sleep(1);
+            while (__hip_atomic_load(&flag[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < ci ||
+                   __hip_atomic_load(&flag[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < ci)
+                __builtin_amdgcn_s_sleep(1);
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
