@@ -91,15 +91,18 @@ constexpr int kPitchH = 136;  // halves per row of the row-major k / q tiles
 constexpr int kPitchL = 68;   // halves per row of the 64 x 64 matrix P = L^T
 constexpr int kPitchD = 20;   // floats per row of a 16 x 16 fp32 block
 constexpr int kBlockD = 16 * kPitchD;
-// Region A: the row-major k / q tiles, later the scratch blocks of the four inverses.
+// Region A: the row-major k / q tiles; once the two products are done, the scratch blocks of the four inverses, P and
+// its diagonal blocks.
 constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsS = 0;
-constexpr int kLdsP = 34816, kLdsD = kLdsP + 64 * kPitchL * 2, kLdsF = kLdsD + 4 * kBlockD * 4, kLdsBytes = kLdsF + 1536;
-static_assert(kLdsBytes <= 54528, "three workgroups of the factor kernel per CU");
+constexpr int kLdsP = 12 * kBlockD * 4, kLdsD = kLdsP + 64 * kPitchL * 2;
+static_assert(kLdsD + 4 * kBlockD * 4 <= 34816, "scratch, P and the diagonal blocks inside the dead k / q tiles");
+constexpr int kLdsF = 34816, kLdsBytes = kLdsF + 1536;
+static_assert(4 * kLdsBytes <= 163840, "four workgroups of the factor kernel per CU");
 
-// One 512-thread workgroup per (sequence, v-head, chunk).  Everything is built transposed -- P = L^T, the diagonal
+// One 512-thread workgroup per (sequence, v-head, chunk), four to a CU.  Everything is built transposed -- P = L^T, the diagonal
 // blocks of (I - P)^-1 = N^T, then N^T by block back substitution -- because the accumulator layout of a tile of
 // N^T (lane: column i, rows j = 4 lq + r) is the A operand layout the walk needs for N (row i, k-slots j).
-__global__ __launch_bounds__(512, 6) void deltanet_chunk_factor_kernel(WalkArgs a) {
+__global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsBytes];
     _Float16 *kh = (_Float16 *)(lds + kLdsKh), *qh = (_Float16 *)(lds + kLdsQh);
     _Float16 *Ph = (_Float16 *)(lds + kLdsP);  // P[j][i] = L[i][j], outside the diagonal blocks
