@@ -13,19 +13,19 @@
 // Only N' and M (two 64 x 64 triangles per chunk and v-head) do not follow from one row of the inputs at a time, so
 // only they go through memory: deltanet_chunk_factor_kernel makes them for all chunks in parallel, and
 // deltanet_chunk_walk_kernel walks the chunks of one (sequence, v-head, half of the state columns) in order, reading
-// q, k and v as they were given.  Against a workspace that also carries W, U and the normalised q and k in operand
-// order (deltanet_chunked.hip) this moves 17 KB instead of 58 KB per chunk and v-head through HBM twice.
+// q, k and v as they were given.  A workspace that also carried W, U and the normalised q and k in operand order
+// would move 58 KB instead of 13 KB per chunk and v-head through HBM twice.
 //
-// The walk: four wavefronts each own 16 state columns -- all 128 rows, in accumulator registers -- for the whole
-// prompt.  Nothing passes between them: the accumulator layout of S, X and V' (lane (li, lq): column li, rows
-// 4 lq + r) is the B operand layout of the next product once the k-slots of the A operand are taken in that
-// order (slots 0-3: rows 4 lq + r of the even 16-row tile of a 32-row slab, slots 4-7: of the odd tile), so a
-// chunk is 62 MFMAs and three conversions in registers per wavefront, and one workgroup barrier (the hand-over of
-// the operand buffer).  Four more wavefronts do nothing but bring in the next chunk: they read k, q, v rows and the
-// two triangles a chunk ahead, normalise, fold the decay factors in and write everything as fp16 A operands into
-// the other half of a two-chunk LDS buffer.
+// The walk: two wavefronts, each alone on its SIMD, own 32 state columns each -- all 128 rows, in accumulator
+// registers -- for the whole prompt.  Nothing passes between them: the accumulator layout of S, X and V' (lane
+// (li, lq): column li, rows 4 lq + r) is the B operand layout of the next product once the k-slots of the A operand
+// are taken in that order (slots 0-3: rows 4 lq + r of the even 16-row tile of a 32-row slab, slots 4-7: of the odd
+// tile), so a chunk is 128 MFMAs and three conversions in registers per wavefront, and one workgroup barrier (the
+// hand-over of the operand buffer).  Six more wavefronts do the moving: they read k, q, v rows and the two triangles
+// two chunks ahead, fold normalisation and decay factors in, write everything as A operands into the other half of a
+// two-chunk LDS buffer, and carry the finished output rows from LDS to memory.
 //
-// Operands are fp16, accumulation and the state fp32 (every decay factor is <= 1: nothing overflows).
+// Operands are fp16 (v: bf16 as given), accumulation and the state fp32 (every decay factor is <= 1: nothing overflows).
 #include <algorithm>
 #include <climits>
 #include <type_traits>
