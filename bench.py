@@ -287,6 +287,16 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "avg_kernel_us": kms * 1e3},
     }
+    tpath = os.path.join(ROOT, "profiles", "deltanet_traffic.json")
+    wname = ("c5-prefill-norm" if norm else "c5-prefill") if chunked else None
+    if wname and os.path.exists(tpath):  # both kernels' FETCH_SIZE + WRITE_SIZE per step, recorded under rocprofv3
+        try:
+            t = json.load(open(tpath)).get(wname)
+        except (OSError, ValueError):
+            t = None
+        if t is not None:
+            res["roofline"]["traffic"] = t
+            res["roofline"]["traffic_source"] = "recorded rocprofv3 counters: profiles/deltanet_traffic.json (not measured in this run)"
     print(json.dumps(res))
 
 
