@@ -73,6 +73,37 @@ def test_chunked_prefill_in_a_graph():
         assert bool(torch.equal(out, want)) and bool(torch.equal(c.k_codes, want_codes)), "replay %d" % i
 
 
+def test_chunked_deltanet_with_its_norm_in_a_graph():
+    """hs_deltanet_forward_chunked_gated_norm is three ordinary launches (factor, walk, norm): recorded once, replayed
+    with the state put back before every replay, it gives the eager bits each time."""
+    B, T, nk, nv = 2, 200, 2, 4
+    case = wl.deltanet_case(1530, B, T, nk, nv, 128, 128)
+    from gpu_util import bf16_from_bits
+    q, k, v = (bf16_from_bits(case[n]).to(DEV) for n in ("q_bits", "k_bits", "v_bits"))
+    g, beta = torch.from_numpy(case["g"]).to(DEV), torch.from_numpy(case["beta"]).to(DEV)
+    r = wl.philox(1531)
+    z = torch.from_numpy(r.standard_normal((B, T, nv, 128)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    w = torch.from_numpy((1.0 + 0.2 * r.standard_normal(128)).astype(np.float32)).to(DEV)
+    s0 = torch.from_numpy((r.standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)).to(DEV)
+    st = s0.clone()
+    out = torch.empty(B, T, nv, 128, dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.deltanet_chunked_gated_norm_workspace_bytes(B, T, nk, nv), dtype=torch.uint8, device=DEV)
+    call = lambda: hb.deltanet_forward_chunked_gated_norm(q, k, v, g, beta, st, z, w, 1e-6, out, 0.0884, True, workspace=ws)
+    call()
+    torch.cuda.synchronize()
+    want, want_state = out.clone(), st.clone()
+    st.copy_(s0)
+    gr = _capture(call)
+    for i in range(3):
+        out.zero_()
+        st.copy_(s0)
+        ws.zero_()
+        torch.cuda.synchronize()
+        gr.replay()
+        torch.cuda.synchronize()
+        assert bool(torch.equal(out, want)) and bool(torch.equal(st, want_state)), "replay %d" % i
+
+
 def _cache_with_history(B, T0, cap, Hkv, D, seed, quant):
     from hyprstream_amd import kv_cache as kc
     r = wl.philox(seed)
