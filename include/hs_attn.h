@@ -365,7 +365,8 @@ HS_API int hs_deltanet_forward(const void *q, const void *k, const void *v, cons
  * hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) bytes (13,312 per 64-token chunk and (sequence, v-head): the two
  * triangular factors of the chunk and three vectors), 16-byte aligned, owned by the caller; q, k, v and out must be
  * 16-byte aligned.  A prompt split into calls of a multiple of 64 tokens (state carried through `state`) gives the
- * bits of one call. */
+ * bits of one call.  Operands are fp16: with l2norm = 0 the caller's q and k (times q_scale) and their dot products
+ * inside a chunk must stay inside the fp16 range (65,504); with l2norm != 0, the reference's setting, they are <= 1. */
 HS_API size_t hs_deltanet_chunked_workspace_bytes(int32_t B, int32_t T, int32_t nk, int32_t nv);
 HS_API int hs_deltanet_forward_chunked(const void *q, const void *k, const void *v, const float *g, const float *beta,
                         float *state, float *out,
