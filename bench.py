@@ -378,6 +378,7 @@ def main():
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
+    ap.add_argument("--cap-pad", type=int, default=0, help="decode workloads: cache capacity = context length + this many tokens")
     ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 128, 256],
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
     ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
@@ -424,12 +425,13 @@ def main():
     gen.manual_seed(wl.SEED)
 
     ncopies = max(1, args.copies)
-    layout = hb.contiguous_layout(Hkv, T, D)
+    cap = T + args.cap_pad  # tokens the cache has room for (the reference allocates max_seq_len, not the current length)
+    layout = hb.contiguous_layout(Hkv, cap, D)
     cdt = torch.uint8 if fp8 else torch.int8
     caches = []
     for c in range(ncopies):
-        kc = torch.empty(B, Hkv, T, D, dtype=cdt, device=dev)
-        vc = torch.empty(B, Hkv, T, D, dtype=cdt, device=dev)
+        kc = torch.empty(B, Hkv, cap, D, dtype=cdt, device=dev)
+        vc = torch.empty(B, Hkv, cap, D, dtype=cdt, device=dev)
         if fp8:
             ks = torch.empty(B, Hkv, dtype=torch.float32, device=dev)
             vs = torch.empty(B, Hkv, dtype=torch.float32, device=dev)
@@ -439,7 +441,7 @@ def main():
         caches.append((kc, vc, ks, vs))
     # fill copy 0 through the library's own quantize-on-write path (a prefill-sized write), sequence by sequence
     kc0, vc0, ks0, vs0 = caches[0]
-    one = hb.contiguous_layout(Hkv, T, D)
+    one = hb.contiguous_layout(Hkv, cap, D)
     tchunk = min(T, 8192)
     for b in range(B):
         for t0 in range(0, T, tchunk):
@@ -455,6 +457,8 @@ def main():
         for dst, src in zip(caches[c], caches[0]):
             dst.copy_(src)
     paged = args.workload == "c2-paged"
+    if paged and args.cap_pad:
+        sys.exit("--cap-pad is for the contiguous cache layouts")
     if paged:
         # every cache copy becomes a pool of 256-token blocks in a random order; K and V blocks of a sequence come from
         # one pool (ids 0..n-1 for K, n..2n-1 for V before the shuffle), as PagedLayerKVCache takes them
