@@ -98,7 +98,7 @@ def test_against_the_oracle():
     assert np.abs(st_b.cpu().numpy() - ws).max() <= 3e-3 * np.abs(ws).max()
 
 
-def test_prefill_layer_is_prepare_plus_the_fused_scan_and_carries_state_across_calls():
+def test_prefill_layer_is_prepare_plus_the_chunked_call_and_carries_state_across_calls():
     """hs_deltanet_prefill_layer (one call for the prompt branch of the layer) against hs_deltanet_prepare +
     hs_deltanet_forward_chunked_gated_norm, bit for bit, for a prompt given in two calls of 128 and 70 tokens with the
     conv state and the recurrent state carried; and against the reference's op sequence for the whole run."""
