@@ -260,3 +260,20 @@ pub unsafe fn deltanet_decode_layer_gpu(mixed_qkv: *const c_void, conv_weight: *
 pub fn decode_workspace_bytes(shape: AttnShape, max_seq_len: i32) -> usize {
     unsafe { bindings::hs_decode_attn_workspace_bytes(shape.b, shape.hq, shape.hkv, shape.d, max_seq_len) }
 }
+
+/// Bytes of workspace of the chunked delta rule (`deltanet_forward_chunked*`): the per-chunk factors, and with
+/// `with_gated_norm` also the fp32 rows between the walk and the norm.
+pub fn deltanet_chunked_workspace_bytes(b: i32, t: i32, nk: i32, nv: i32, with_gated_norm: bool) -> usize {
+    unsafe {
+        if with_gated_norm {
+            bindings::hs_deltanet_chunked_gated_norm_workspace_bytes(b, t, nk, nv)
+        } else {
+            bindings::hs_deltanet_chunked_workspace_bytes(b, t, nk, nv)
+        }
+    }
+}
+
+/// Bytes of workspace of `deltanet_prefill_layer_gpu` (256-byte aligned).
+pub fn deltanet_prefill_layer_workspace_bytes(b: i32, s: i32, nk: i32, nv: i32, dk: i32, dv: i32) -> usize {
+    unsafe { bindings::hs_deltanet_prefill_layer_workspace_bytes(b, s, nk, nv, dk, dv) }
+}
