@@ -124,6 +124,10 @@ def test_workspace_and_shape_errors():
     with pytest.raises(hb.HsError) as e:  # nv must be a multiple of nk
         hb.deltanet_forward_chunked(q.repeat(1, 1, 3, 1), k.repeat(1, 1, 3, 1), v, g, beta, st, out, 1.0, True)
     assert e.value.code == hb.HS_ERR_INVALID_ARGUMENT
+    flat = torch.empty(out.numel() + 4, device=DEV)  # the rows leave in 16-byte stores: out must be aligned like q, k, v
+    with pytest.raises(hb.HsError) as e:
+        hb.deltanet_forward_chunked(q, k, v, g, beta, st, flat[1:1 + out.numel()].view(out.shape), 1.0, True)
+    assert e.value.code == hb.HS_ERR_INVALID_ARGUMENT and "aligned" in str(e.value)
     torch.cuda.synchronize()
 
 
