@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-layer|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -216,7 +216,8 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
     """Config 5: gated DeltaNet, nk 16 / nv 32, dk = dv = 128.  Decode: B = 64, one token, fp32 state read and
     written once (HBM bound).  Prefill: B = 4 x 4096 tokens in chunks of 64 on the matrix pipe (c5-prefill), or
     through the token-by-token fp32 recurrence (c5-prefill-recurrent).  norm: the chunked prefill followed by the layer's
-    gated RMSNorm as one call (hs_deltanet_forward_chunked_gated_norm, c5-prefill-norm)."""
+    gated RMSNorm as one call (hs_deltanet_forward_chunked_gated_norm, c5-prefill-norm); norm = "layer": the prompt branch
+    of the whole layer between its projections, conv1d + SiLU + gates included (hs_deltanet_prefill_layer, c5-prefill-layer)."""
     dev = "cuda:0"
     nk, nv, d = 16, 32, 128
     B, T = (4, 4096) if prefill else (64, 1)
@@ -241,9 +242,20 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
         z = torch.randn(B, T, nv, d, generator=gen, device=dev).to(torch.bfloat16)
         nw = torch.rand(d, generator=gen, device=dev) + 0.5
         out_n = torch.empty(B, T, nv, d, dtype=torch.bfloat16, device=dev)
+    if norm == "layer":
+        C = 2 * nk * d + nv * d
+        rn = lambda *sh: torch.randn(*sh, generator=gen, device=dev)
+        lx, lw, lcs = rn(B, T, C).to(torch.bfloat16), (0.5 * rn(C, 4)).to(torch.bfloat16), rn(B, C, 3).to(torch.bfloat16)
+        la, lb = (2 * rn(B, T, nv)).to(torch.bfloat16), (2 * rn(B, T, nv)).to(torch.bfloat16)
+        lnae, ldtb = -rn(nv).exp(), rn(nv)
+        lws = None
 
     def step(i):
-        if norm:
+        if norm == "layer":
+            nonlocal lws
+            lws = hb.deltanet_prefill_layer(lx, lw, lcs, la, lb, lnae, ldtb, z, nw, 1e-6, states[i % ncopies], nk, nv, d, d, qs, True,
+                                            workspace=lws)[2]
+        elif norm:
             hb.deltanet_forward_chunked_gated_norm(q, k, v, g, beta, states[i % ncopies], z, nw, 1e-6, out_n, qs, False, workspace=ws)
         elif chunked:
             hb.deltanet_forward_chunked(q, k, v, g, beta, states[i % ncopies], out, qs, False, workspace=ws)
@@ -270,6 +282,8 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
     kms = float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
     state_bytes = 2 * B * nv * d * d * 4
     io_bytes = B * T * (2 * nk * d * 2 + nv * d * 2 + 2 * nv * 4 + (nv * d * 2 * 2 if norm else nv * d * 4))
+    if norm == "layer":  # mixed q|k|v in, z in, bf16 rows out, the gate inputs, the conv state both ways
+        io_bytes = B * T * ((2 * nk * d + nv * d) * 2 + 2 * nv * d * 2 + 2 * nv * 2) + 2 * B * (2 * nk * d + nv * d) * 3 * 2
     nbytes = state_bytes + io_bytes
     res = {
         "metric": "deltanet %s HBM GB/s + tokens/s, nk=16 nv=32 dk=dv=128" % ("prefill" if prefill else "decode"),
@@ -278,17 +292,18 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
         "dtype": "f16 MFMA operands, f32 accumulation, triangular solve and state; bf16 q/k/v" if chunked else "f32 state and arithmetic, bf16 q/k/v",
         "data": "synthetic (seeded, generated on device)",
         "config": {"workload": "c5-%s: gated delta rule B=%d T=%d nk=16 nv=32 dk=dv=128, fp32 state [B,32,128,128]%s%s"
-                               % (("prefill-norm" if norm else "prefill") if prefill else "decode", B, T,
+                               % (("prefill-layer" if norm == "layer" else "prefill-norm" if norm else "prefill") if prefill else "decode", B, T,
                                   ", chunk size 64" if chunked else (", token recurrence" if prefill else ""),
+                                  ", between conv1d + SiLU + gates and the gated RMSNorm (one call)" if norm == "layer" else
                                   ", then the gated RMSNorm (same call)" if norm else ""),
                    "algorithmic_bytes_per_step": int(nbytes)},
         "tokens_per_s": B * T / (ms * 1e-3),
-        "roofline": {"bound": "hbm", "kernel": ("deltanet_chunk_factor_kernel + deltanet_chunk_walk_kernel" + (" + gated_rmsnorm_rows_kernel" if norm else "") if chunked else "deltanet_prefill_kernel") if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
+        "roofline": {"bound": "hbm", "kernel": (("deltanet_conv8 + gates + " if norm == "layer" else "") + "deltanet_chunk_factor_kernel + deltanet_chunk_walk_kernel" + (" + gated_rmsnorm_rows_kernel" if norm else "") if chunked else "deltanet_prefill_kernel") if prefill else "deltanet_decode_kernel", "achieved": nbytes / (kms * 1e-3) / 1e9,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": nbytes / (kms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                      "traffic": None, "avg_kernel_us": kms * 1e3},
     }
     tpath = os.path.join(ROOT, "profiles", "deltanet_traffic.json")
-    wname = ("c5-prefill-norm" if norm else "c5-prefill") if chunked else None
+    wname = ("c5-prefill-layer" if norm == "layer" else "c5-prefill-norm" if norm else "c5-prefill") if chunked else None
     if wname and os.path.exists(tpath):  # both kernels' FETCH_SIZE + WRITE_SIZE per step, recorded under rocprofv3
         try:
             t = json.load(open(tpath)).get(wname)
@@ -374,7 +389,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-recurrent"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-layer", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
@@ -419,7 +434,7 @@ def main():
         return bench_deltanet_layer(args, torch, hb, wl, fused=args.workload == "c5-decode-layer")
     if args.workload.startswith("c5"):
         return bench_deltanet(args, torch, hb, wl, "prefill" in args.workload, recurrent=args.workload.endswith("recurrent"),
-                              norm=args.workload == "c5-prefill-norm")
+                              norm="layer" if args.workload == "c5-prefill-layer" else args.workload == "c5-prefill-norm")
     B, Hq, Hkv, D, T, ragged, fp8, sigma, outliers = WORKLOADS[args.workload]
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)
