@@ -148,12 +148,14 @@ def test_against_the_numpy_restatement_of_the_reference_chunked_form():
     check(o, s, np.asarray(wo, np.float32).transpose(0, 2, 1, 3), np.asarray(ws, np.float32), "numpy chunked form")
 
 
-@pytest.mark.parametrize("nk,nv", [(2, 2), (1, 4), (3, 3)])
-def test_head_groupings(nk, nv):
-    """One, several or all v-heads per k-head (the normalised q / k operands are written once per k-head)."""
-    B, T = 3, 130
+@pytest.mark.parametrize("B,nk,nv", [(3, 2, 2), (3, 1, 4), (3, 3, 3), (8, 1, 4), (2, 1, 4), (4, 2, 8)])
+def test_head_groupings(B, nk, nv):
+    """One, several or all v-heads per k-head, and the three ways the walk places its workgroups on the XCDs (B * nk a
+    multiple of 8: the workgroups of a k-head together; B * nv a multiple of 8: the two halves of a v-head together;
+    otherwise in grid order)."""
+    T = 130
     case = wl.deltanet_case(80 + nk + nv, B, T, nk, nv, 128, 128)
     s0 = (wl.philox(81).standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)
     o, s = run(case, s0, 1 / np.sqrt(128.0), True)
     wo, ws = want(case, s0, 1 / np.sqrt(128.0), True)
-    check(o, s, wo, ws, "nk=%d nv=%d" % (nk, nv))
+    check(o, s, wo, ws, "B=%d nk=%d nv=%d" % (B, nk, nv))
