@@ -220,7 +220,7 @@ def bench_deltanet(args, torch, hb, wl, prefill, recurrent=False, norm=None):
     of the whole layer between its projections, conv1d + SiLU + gates included (hs_deltanet_prefill_layer, c5-prefill-layer)."""
     dev = "cuda:0"
     nk, nv, d = 16, 32, 128
-    B, T = (4, 4096) if prefill else (64, 1)
+    B, T = (args.batch or 4, 4096) if prefill else (args.batch or 64, 1)
     gen = torch.Generator(device=dev)
     gen.manual_seed(wl.SEED)
     nrm = lambda x: (x / x.norm(dim=-1, keepdim=True).clamp_min(1e-3)).to(torch.bfloat16)
@@ -398,7 +398,7 @@ def main():
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
     ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
                     help="prefill workloads: tokens per chunk call (0 = the workload's own: 512, c3-prompt 4096)")
-    ap.add_argument("--batch", type=int, default=0, help="c5-decode-layer workloads: sequences in the batch (0 = 64)")
+    ap.add_argument("--batch", type=int, default=0, help="c5 workloads: sequences in the batch (0 = the configuration's 64 for decode, 4 for prefill)")
     ap.add_argument("--graph", action="store_true", help="replay the decode steps from a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain 1 GiB device-to-device copy, the reference point for scaling "
