@@ -12,11 +12,12 @@
 //   S <- e^(G_63) S + (k e^(G_63 - G))^T V'.
 // Only N' and M (two 64 x 64 triangles per chunk and v-head) do not follow from one row of the inputs at a time, so
 // only they go through memory: deltanet_chunk_factor_kernel makes them for all chunks in parallel, and
-// deltanet_chunk_walk_kernel walks the chunks of one (sequence, v-head, half of the state columns) in order, reading
-// q, k and v as they were given.  A workspace that also carried W, U and the normalised q and k in operand order
+// deltanet_chunk_walk_kernel walks the chunks of one (sequence, v-head, half or quarter of the state columns) in
+// order, reading q, k and v as they were given.  A workspace that also carried W, U and the normalised q and k in operand order
 // would move 58 KB instead of 13 KB per chunk and v-head through HBM twice.
 //
-// The walk: two wavefronts, each alone on its SIMD, own 32 state columns each -- all 128 rows, in accumulator
+// The walk: two wavefronts, each alone on its SIMD, own 32 state columns each (16 in the instance for batches that
+// leave the device part empty otherwise: half the products of a chunk step) -- all 128 rows, in accumulator
 // registers -- for the whole prompt.  Nothing passes between them: the accumulator layout of S, X and V' (lane
 // (li, lq): column li, rows 4 lq + r) is the B operand layout of the next product once the k-slots of the A operand
 // are taken in that order (slots 0-3: rows 4 lq + r of the even 16-row tile of a 32-row slab, slots 4-7: of the odd
@@ -305,7 +306,7 @@ constexpr int oQg = oKn + 16384;              // q e^G         [token tile 4][dk
 constexpr int oKt = oQg + 16384;              // k e^(G63-G), transposed [dk 128][token 64], eight-token pieces permuted
 constexpr int oNt = oKt + kWD * kPitchT * 2;  // N'            six blocks, tri_block order
 constexpr int oQK = oNt + 6144;               // M             six blocks
-constexpr int oV = oQK + 6144;                // v, this half's 64 columns: [token tile 4][column slab 2], natural k order
+constexpr int oV = oQK + 6144;                // v, the workgroup's columns: [token tile 4][32-column slab], natural k order
 constexpr int oDec = oV + 8192;               // e^(G63)
 constexpr int kBufBytes = oDec + 16;
 // Behind the two operand buffers: the finished output rows of a chunk on their way out, and who has fetched them.
@@ -319,7 +320,15 @@ __device__ __forceinline__ int tpos(int d, int tok) { return d * kPitchT + ((((t
 
 constexpr int kWalkThreads = 512;
 
+// kCT: 16-column tiles per computing wavefront.  2: a workgroup owns 64 state columns, two workgroups per (sequence,
+// v-head).  1: 32 columns, four workgroups -- half the products per chunk step for the same loading work, for batches
+// whose walk would otherwise leave most of the chip idle (the chunk steps of a sequence are a chain).
+template <int kCT>
 __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkArgs a) {
+    constexpr int kW = 32 * kCT;           // state columns of a workgroup
+    constexpr int NP = kWD / kW;           // workgroups per (sequence, v-head)
+    constexpr int kPitchO = kW + 4;        // floats per staged output row: the rows of a 16-byte read hit different banks
+    static_assert(kPitchO <= kOutPitch, "the staging area is sized for 64 columns");
     __shared__ __attribute__((aligned(16))) uint8_t lds[kLdsWalk];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -329,18 +338,18 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
     // rows: the 2 * rep workgroups of a (sequence, k-head) get linear ids congruent mod 8, consecutive in that XCD's
     // order, so that each of those comes from HBM once and the other readers find it in L2.
     const int p = blockIdx.x, pairs = a.B * a.nv, rep = a.nv / a.nk;
-    int pair, half;
+    int pair, part;  // part: which kW columns of the v-head
     if (((a.B * a.nk) & 7) == 0) {
-        const int i = p >> 3, per = 2 * rep;
+        const int i = p >> 3, per = NP * rep;
         const int ku = (p & 7) + 8 * (i / per), sub = i % per;
-        pair = ku * rep + (sub >> 1);
-        half = sub & 1;
+        pair = ku * rep + sub / NP;
+        part = sub % NP;
     } else if ((pairs & 7) == 0) {
-        pair = (p & 7) + 8 * (p >> 4);
-        half = (p >> 3) & 1;
+        pair = (p & 7) + 8 * (p / (8 * NP));
+        part = (p >> 3) % NP;
     } else {
-        pair = p >> 1;
-        half = p & 1;
+        pair = p / NP;
+        part = p % NP;
     }
     const int b = pair / a.nv, j = pair % a.nv, hk = j / rep;
     const int64_t chunk_stride = (int64_t)a.B * a.nv * kUnitBytes;
@@ -354,7 +363,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
     if (wave == 4 || wave == 5) {  // ---- N', M, v, e^(G63): thread ct of 128; plain copies, no arithmetic
         const int ct = tid - 256;
         struct Stage {
-            u32x4 nm[6], vr[4];
+            u32x4 nm[6], vr[2 * kCT];
             float dec;
         };
         auto fetch = [&](Stage &st, int ci) {
@@ -363,10 +372,10 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
             for (int i = 0; i < 6; ++i) st.nm[i] = *(const u32x4 *)(u + (ct + 128 * i) * 16);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {  // item = (token, eight columns of this half)
-                const int item = ct + 128 * i, tok = item >> 3, pc = item & 7;
+            for (int i = 0; i < 2 * kCT; ++i) {  // item = (token, eight of this workgroup's columns)
+                const int item = ct + 128 * i, tok = item / (kW / 8), pc = item % (kW / 8);
                 const int64_t bt = (int64_t)b * a.T + min(ci * kC + tok, a.T - 1);
-                st.vr[i] = __builtin_nontemporal_load((const u32x4 *)(a.v + (bt * a.nv + j) * kWD + 64 * half + 8 * pc));
+                st.vr[i] = __builtin_nontemporal_load((const u32x4 *)(a.v + (bt * a.nv + j) * kWD + kW * part + 8 * pc));
             }
             st.dec = *(const float *)(u + kOffDecay);
         };
@@ -374,13 +383,13 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
             for (int i = 0; i < 6; ++i) *(u32x4 *)(buf + oNt + (ct + 128 * i) * 16) = st.nm[i];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int item = ct + 128 * i, tok = item >> 3, pc = item & 7;
+            for (int i = 0; i < 2 * kCT; ++i) {
+                const int item = ct + 128 * i, tok = item / (kW / 8), pc = item % (kW / 8);
                 const bool valid = ci * kC + tok < a.T;  // rows past T are zero
                 // eight bf16 as they are: one 16-byte piece of an A operand block of the bf16 MFMA (row = token, k-slots =
                 // columns, natural order); the piece of lane (li, lq) sits at 4 li + lq, so that the eight tokens x four
                 // pieces a wavefront writes are contiguous
-                *(u32x4 *)(buf + oV + (((tok >> 4) * 2 + (pc >> 2)) * 64 + (tok & 15) * 4 + (pc & 3)) * 16) =
+                *(u32x4 *)(buf + oV + (((tok >> 4) * kCT + (pc >> 2)) * 64 + (tok & 15) * 4 + (pc & 3)) * 16) =
                     valid ? st.vr[i] : (u32x4){0u, 0u, 0u, 0u};
             }
             if (ct == 0) *(float *)(buf + oDec) = st.dec;
@@ -406,9 +415,9 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         return;
     }
     if (wave >= 2) {
-        // ---- k and q rows: thread = (token tl and tl + 32, dk 8 part .. + 7 and 64 + 8 part .. + 7: the eight threads
+        // ---- k and q rows: thread = (token tl and tl + 32, dk 8 dp .. + 7 and 64 + 8 dp .. + 7: the eight threads
         //      of a token read whole 128-byte lines)
-        const int lt = ((wave & 1) | ((wave >> 2) << 1)) * 64 + lane, tl = lt >> 3, part = lt & 7;
+        const int lt = ((wave & 1) | ((wave >> 2) << 1)) * 64 + lane, tl = lt >> 3, dp = lt & 7;
         if (lt == 0) {  // visible to the computing wavefronts after the first barrier
             flag[0] = 0;
             flag[1] = 0;
@@ -424,8 +433,8 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
             for (int ps = 0; ps < 2; ++ps) {
                 const int tok = tl + 32 * ps;
                 const int64_t bt = (int64_t)b * a.T + min(ci * kC + tok, a.T - 1);
-                const uint16_t *kp = a.k + (bt * a.nk + hk) * kWD + 8 * part;
-                const uint16_t *qp = a.q + (bt * a.nk + hk) * kWD + 8 * part;
+                const uint16_t *kp = a.k + (bt * a.nk + hk) * kWD + 8 * dp;
+                const uint16_t *qp = a.q + (bt * a.nk + hk) * kWD + 8 * dp;
                 st.kr[ps][0] = *(const u32x4 *)kp;
                 st.kr[ps][1] = *(const u32x4 *)(kp + 64);
                 st.qr[ps][0] = *(const u32x4 *)qp;
@@ -440,16 +449,16 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
             for (int ps = 0; ps < 2; ++ps) {
                 const int tok = tl + 32 * ps;
-                float kf[16], qf[16];  // elements 0-7: dk 8 part + e, 8-15: dk 64 + 8 part + e
+                float kf[16], qf[16];  // elements 0-7: dk 8 dp + e, 8-15: dk 64 + 8 dp + e
                 unpack16(st.kr[ps][0], st.kr[ps][1], kf);
                 unpack16(st.qr[ps][0], st.qr[ps][1], qf);
                 const float fn = st.fn[ps], fq = st.fq[ps], ft = st.ft[ps];
 #pragma unroll
                 for (int h8 = 0; h8 < 2; ++h8) {
-                    // dk 64 h8 + 8 part + e: slab 2 h8 + part / 4; inside the slab at 8 (part % 4) + e, i.e. the tile of
-                    // the slab (slots 0-3 or 4-7) is (part / 2) % 2 and the row groups are lq = 2 (part % 2), + 1
-                    const int blk = (tok >> 4) * 4 + 2 * h8 + (part >> 2);
-                    const int o = blk * 1024 + (2 * (part & 1) * 16 + (tok & 15)) * 16 + 8 * ((part >> 1) & 1);
+                    // dk 64 h8 + 8 dp + e: slab 2 h8 + dp / 4; inside the slab at 8 (dp % 4) + e, i.e. the tile of
+                    // the slab (slots 0-3 or 4-7) is (dp / 2) % 2 and the row groups are lq = 2 (dp % 2), + 1
+                    const int blk = (tok >> 4) * 4 + 2 * h8 + (dp >> 2);
+                    const int o = blk * 1024 + (2 * (dp & 1) * 16 + (tok & 15)) * 16 + 8 * ((dp >> 1) & 1);
 #pragma unroll
                     for (int g4 = 0; g4 < 2; ++g4) {
                         half4v hn, hq;
@@ -458,7 +467,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
                             const int i = 8 * h8 + 4 * g4 + e;
                             hn[e] = (_Float16)(kf[i] * fn);
                             hq[e] = (_Float16)(qf[i] * fq);
-                            KT[tpos(64 * h8 + 8 * part + 4 * g4 + e, tok)] = (_Float16)(kf[i] * ft);
+                            KT[tpos(64 * h8 + 8 * dp + 4 * g4 + e, tok)] = (_Float16)(kf[i] * ft);
                         }
                         *(half4v *)(buf + oKn + o + g4 * 256) = hn;
                         *(half4v *)(buf + oQg + o + g4 * 256) = hq;
@@ -470,17 +479,17 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         // chunk c - 1 was being computed.
         // Round c (after the barrier that publishes chunk c).  Wavefronts 2 and 3 (thread lt of 128) first take the
         // staged rows of chunk c - 1 into registers and release the staging area.  Then chunk c + 1 goes into the other
-        // operand buffer; the rows leave for memory, 16 B per lane (16 lanes cover the 256 bytes this half owns of a
+        // operand buffer; the rows leave for memory, 16 B per lane (kW / 4 lanes cover the bytes this workgroup owns of a
         // token's row); chunk c + 3 is requested.
         auto round = [&](Stage &st, int c) {
             lds_sync();
-            u32x4 orow[8];
+            u32x4 orow[4 * kCT];
             const bool carry = wave < 4 && c >= 1;
             if (carry) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
+                for (int i = 0; i < 4 * kCT; ++i) {  // piece = (row, four columns)
                     const int pc = lt + 128 * i;
-                    orow[i] = *(const u32x4 *)(lds + oOut + ((pc >> 4) * kOutPitch + 4 * (pc & 15)) * 4);
+                    orow[i] = *(const u32x4 *)(lds + oOut + ((pc / (kW / 4)) * kPitchO + 4 * (pc % (kW / 4))) * 4);
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 if (lane == 0) __hip_atomic_store(&flag[wave - 2], c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -488,9 +497,9 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
             if (c + 1 < a.nc) put(st, lds + ((c + 1) & 1) * kBufBytes);
             if (carry) {
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    const int pc = lt + 128 * i, t = (c - 1) * kC + (pc >> 4);
-                    if (t < a.T) __builtin_nontemporal_store(orow[i], (u32x4 *)(a.out + (((int64_t)b * a.T + t) * a.nv + j) * kWD + 64 * half + 4 * (pc & 15)));
+                for (int i = 0; i < 4 * kCT; ++i) {
+                    const int pc = lt + 128 * i, t = (c - 1) * kC + pc / (kW / 4);
+                    if (t < a.T) __builtin_nontemporal_store(orow[i], (u32x4 *)(a.out + (((int64_t)b * a.T + t) * a.nv + j) * kWD + kW * part + 4 * (pc % (kW / 4))));
                 }
             }
             if (c + 1 < a.nc) fetch(st, c + 3);
@@ -507,24 +516,24 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         return;
     }
 
-    // ---- the two computing wavefronts: wavefront w owns state columns 64 half + 32 w .. + 31 (two 16-column tiles c)
-    const int col = 64 * half + 32 * wave + li;
-    float4v S[8][2];  // dk tile x: rows 16 x + 4 lq + r
+    // ---- the two computing wavefronts: wavefront w owns state columns kW part + 16 kCT w .. (kCT 16-column tiles c)
+    const int col = kW * part + 16 * kCT * wave + li;
+    float4v S[8][kCT];  // dk tile x: rows 16 x + 4 lq + r
     float *sp = a.state + ((int64_t)pair * kWD) * kWD + col;
 #pragma unroll
     for (int x = 0; x < 8; ++x)
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < kCT; ++c)
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[x][c][r] = sp[(int64_t)(16 * x + 4 * lq + r) * kWD + 16 * c];
-    // the B operands (bf16, like v itself) that pick column tile c out of this wavefront's 32-column slab of v
-    bf16x8 pick[2];
+    // the B operands (bf16, like v itself) that pick column tile c of this wavefront out of a 32-column slab of v
+    bf16x8 pick[kCT];
 #pragma unroll
-    for (int c = 0; c < 2; ++c)
+    for (int c = 0; c < kCT; ++c)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pick[c][e] = (__bf16)(8 * lq + e == 16 * c + li ? 1.0f : 0.0f);
+        for (int e = 0; e < 8; ++e) pick[c][e] = (__bf16)(8 * lq + e == (16 * (kCT * wave + c)) % 32 + li ? 1.0f : 0.0f);
     const float4v zero = {0.f, 0.f, 0.f, 0.f};
-    float *stage = (float *)(lds + oOut) + (4 * lq) * kOutPitch + 32 * wave + li;  // + (16 tt + r) * kOutPitch + 16 c
+    float *stage = (float *)(lds + oOut) + (4 * lq) * kPitchO + 16 * kCT * wave + li;  // + (16 tt + r) * kPitchO + 16 c
 
 #define HS_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16(A, B, C, 0, 0, 0)
     // One chunk.  Every A operand read from LDS feeds two products (the two column tiles), and the reads of a group of
@@ -540,12 +549,12 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
             const half4v hi = *(const half4v *)&KT[tpos(16 * x + li, 32 * s + 16 + 4 * lq)];
             return (half8){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
         };
-        float4v X[4][2], V[4][2];
-        half8 an[2][4], nt[6], sh[2];
+        float4v X[4][kCT], V[4][kCT];
+        half8 an[2][4], nt[6], sh[kCT];
         bf16x8 va[4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            va[tt] = *(const bf16x8 *)(buf + oV + (tt * 2 + wave) * 1024 + (li * 4 + lq) * 16);
+            va[tt] = *(const bf16x8 *)(buf + oV + (tt * kCT + (kCT * wave) / 2) * 1024 + (li * 4 + lq) * 16);
             an[0][tt] = opA(oKn, tt * 4);
         }
         const float dec = *(const float *)(buf + oDec);
@@ -554,7 +563,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-            for (int c = 0; c < 2; ++c) X[tt][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[tt], pick[c], zero, 0, 0, 0);
+            for (int c = 0; c < kCT; ++c) X[tt][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[tt], pick[c], zero, 0, 0, 0);
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {  // dk slab sl
             if (sl < 3) {
@@ -565,45 +574,45 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
                 for (int i = 0; i < 6; ++i) nt[i] = opA(oNt, i);
             }
 #pragma unroll
-            for (int c = 0; c < 2; ++c) sh[c] = f32x8_to_half8(S[2 * sl][c], S[2 * sl + 1][c]);
+            for (int c = 0; c < kCT; ++c) sh[c] = f32x8_to_half8(S[2 * sl][c], S[2 * sl + 1][c]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-                for (int c = 0; c < 2; ++c) X[tt][c] = HS_MFMA(an[sl & 1][tt], sh[c], X[tt][c]);
+                for (int c = 0; c < kCT; ++c) X[tt][c] = HS_MFMA(an[sl & 1][tt], sh[c], X[tt][c]);
             __builtin_amdgcn_sched_barrier(0);
         }
         half8 aq[2][4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) aq[0][tt] = opA(oQg, tt * 4);
-        half8 Xh[2][2];
+        half8 Xh[2][kCT];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < kCT; ++c) {
             Xh[0][c] = f32x8_to_half8(X[0][c], X[1][c]);
             Xh[1][c] = f32x8_to_half8(X[2][c], X[3][c]);
         }
         __builtin_amdgcn_sched_barrier(0);
         // V' = N' X (N' is lower triangular: token tiles 0 and 1 see only the first slab)
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < kCT; ++c) {
             V[0][c] = HS_MFMA(nt[tri_block(0, 0)], Xh[0][c], zero);
             V[1][c] = HS_MFMA(nt[tri_block(1, 0)], Xh[0][c], zero);
             V[2][c] = HS_MFMA(nt[tri_block(2, 0)], Xh[0][c], zero);
             V[3][c] = HS_MFMA(nt[tri_block(3, 0)], Xh[0][c], zero);
         }
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < kCT; ++c) {
             V[2][c] = HS_MFMA(nt[tri_block(2, 1)], Xh[1][c], V[2][c]);
             V[3][c] = HS_MFMA(nt[tri_block(3, 1)], Xh[1][c], V[3][c]);
         }
         __builtin_amdgcn_sched_barrier(0);
         // O = (q e^G) S + M V'
-        float4v O[4][2];
+        float4v O[4][kCT];
         half8 qm[6], kt[2][4];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-            for (int c = 0; c < 2; ++c) O[tt][c] = zero;
+            for (int c = 0; c < kCT; ++c) O[tt][c] = zero;
 #pragma unroll
         for (int sl = 0; sl < 4; ++sl) {
             if (sl < 3) {
@@ -614,32 +623,32 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
                 for (int i = 0; i < 6; ++i) qm[i] = opA(oQK, i);
             }
 #pragma unroll
-            for (int c = 0; c < 2; ++c) sh[c] = f32x8_to_half8(S[2 * sl][c], S[2 * sl + 1][c]);
+            for (int c = 0; c < kCT; ++c) sh[c] = f32x8_to_half8(S[2 * sl][c], S[2 * sl + 1][c]);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-                for (int c = 0; c < 2; ++c) O[tt][c] = HS_MFMA(aq[sl & 1][tt], sh[c], O[tt][c]);
+                for (int c = 0; c < kCT; ++c) O[tt][c] = HS_MFMA(aq[sl & 1][tt], sh[c], O[tt][c]);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) kt[0][i] = opKt(i >> 1, i & 1);
-        half8 Vh[2][2];
+        half8 Vh[2][kCT];
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < kCT; ++c) {
             Vh[0][c] = f32x8_to_half8(V[0][c], V[1][c]);
             Vh[1][c] = f32x8_to_half8(V[2][c], V[3][c]);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < kCT; ++c) {
             O[0][c] = HS_MFMA(qm[tri_block(0, 0)], Vh[0][c], O[0][c]);
             O[1][c] = HS_MFMA(qm[tri_block(1, 0)], Vh[0][c], O[1][c]);
             O[2][c] = HS_MFMA(qm[tri_block(2, 0)], Vh[0][c], O[2][c]);
             O[3][c] = HS_MFMA(qm[tri_block(3, 0)], Vh[0][c], O[3][c]);
         }
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < kCT; ++c) {
             O[2][c] = HS_MFMA(qm[tri_block(2, 1)], Vh[1][c], O[2][c]);
             O[3][c] = HS_MFMA(qm[tri_block(3, 1)], Vh[1][c], O[3][c]);
         }
@@ -649,7 +658,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
         for (int x = 0; x < 8; ++x)
 #pragma unroll
-            for (int c = 0; c < 2; ++c) S[x][c] *= dec;
+            for (int c = 0; c < kCT; ++c) S[x][c] *= dec;
         __builtin_amdgcn_sched_barrier(0);
         // S <- e^(G63) S + (k e^(G63-G))^T V', two dk tiles at a time
 #pragma unroll
@@ -659,7 +668,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
                 for (int xo = 0; xo < 2; ++xo)
 #pragma unroll
-                    for (int c = 0; c < 2; ++c)
+                    for (int c = 0; c < kCT; ++c)
                         S[2 * xp + xo][c] = HS_MFMA(kt[xp & 1][2 * xo + sl], Vh[sl][c], S[2 * xp + xo][c]);
             __builtin_amdgcn_sched_barrier(0);
             if (xp < 2) {
@@ -677,18 +686,18 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
-            for (int c = 0; c < 2; ++c)
+            for (int c = 0; c < kCT; ++c)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) stage[(16 * tt + r) * kOutPitch + 16 * c] = O[tt][c][r];
+                for (int r = 0; r < 4; ++r) stage[(16 * tt + r) * kPitchO + 16 * c] = O[tt][c][r];
     }
 #undef HS_MFMA
-    lds_sync();  // the last chunk's rows are staged: wavefronts 4 and 5 take them from here
+    lds_sync();  // the last chunk's rows are staged: wavefronts 2 and 3 take them from here
     float *sq = sp;  // opaque to the compiler: it would otherwise keep the 64 addresses of the first loads alive (spilled) across the walk
     asm volatile("" : "+v"(sq));
 #pragma unroll
     for (int x = 0; x < 8; ++x)
 #pragma unroll
-        for (int c = 0; c < 2; ++c)
+        for (int c = 0; c < kCT; ++c)
 #pragma unroll
             for (int r = 0; r < 4; ++r) sq[(int64_t)(16 * x + 4 * lq + r) * kWD + 16 * c] = S[x][c][r];
 }
@@ -708,6 +717,25 @@ size_t hs_deltanet_chunked_gated_norm_workspace_bytes(int32_t B, int32_t T, int3
     return ((hs_deltanet_chunked_workspace_bytes(B, T, nk, nv) + 255) & ~(size_t)255) + (size_t)B * T * nv * hs::kWD * sizeof(float);
 }
 
+// Workgroups of the walk the current device runs at once: one per CU (its LDS), looked up once per device.
+static int walk_slots() {
+    constexpr int kMaxDevices = 64;
+    static int slots[kMaxDevices];  // 0: not asked yet (a second thread asking at the same time stores the same value)
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    if (slots[dev] == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0;
+        }
+        slots[dev] = cus > 0 ? cus : -1;
+    }
+    return slots[dev] > 0 ? slots[dev] : 0;
+}
+
 static int chunked_launch(const void *q, const void *k, const void *v, const float *g, const float *beta, float *state,
                           float *out, int32_t B, int32_t T, int32_t nk, int32_t nv, int32_t dk, int32_t dv, float q_scale,
                           int l2norm, void *workspace, hipStream_t st) {
@@ -718,7 +746,9 @@ static int chunked_launch(const void *q, const void *k, const void *v, const flo
     a.B = B; a.T = T; a.nk = nk; a.nv = nv; a.nc = (T + kC - 1) / kC; a.q_scale = q_scale; a.l2norm = l2norm ? 1 : 0;
     deltanet_chunk_factor_kernel<<<(unsigned)((int64_t)B * nv * a.nc), 512, 0, st>>>(a);
     if (int rc = check_launch("deltanet_chunk_factor")) return rc;
-    deltanet_chunk_walk_kernel<<<(unsigned)(2 * B * nv), kWalkThreads, 0, st>>>(a);
+    // 32-column workgroups while four of them per (sequence, v-head) still fit the device in one round
+    if (4 * (int64_t)B * nv <= walk_slots()) deltanet_chunk_walk_kernel<1><<<(unsigned)(4 * B * nv), kWalkThreads, 0, st>>>(a);
+    else deltanet_chunk_walk_kernel<2><<<(unsigned)(2 * B * nv), kWalkThreads, 0, st>>>(a);
     return check_launch("deltanet_chunk_walk");
 }
 

@@ -148,14 +148,28 @@ def test_against_the_numpy_restatement_of_the_reference_chunked_form():
     check(o, s, np.asarray(wo, np.float32).transpose(0, 2, 1, 3), np.asarray(ws, np.float32), "numpy chunked form")
 
 
-@pytest.mark.parametrize("B,nk,nv", [(3, 2, 2), (3, 1, 4), (3, 3, 3), (8, 1, 4), (2, 1, 4), (4, 2, 8)])
+@pytest.mark.parametrize("B,nk,nv", [(3, 2, 2), (3, 1, 4), (3, 3, 3), (8, 1, 4), (2, 1, 4), (4, 2, 8),
+                                     (40, 2, 4), (17, 1, 4), (24, 4, 4)])
 def test_head_groupings(B, nk, nv):
-    """One, several or all v-heads per k-head, and the three ways the walk places its workgroups on the XCDs (B * nk a
-    multiple of 8: the workgroups of a k-head together; B * nv a multiple of 8: the two halves of a v-head together;
-    otherwise in grid order)."""
-    T = 130
+    """One, several or all v-heads per k-head; the three ways the walk places its workgroups on the XCDs (B * nk a
+    multiple of 8: the workgroups of a k-head together; B * nv a multiple of 8: the parts of a v-head together; otherwise
+    in grid order); and both widths of its workgroups (32 state columns while 4 B nv workgroups fit the device in one
+    round -- the first six cases --, 64 columns beyond)."""
+    T = 130 if B < 10 else 70
     case = wl.deltanet_case(80 + nk + nv, B, T, nk, nv, 128, 128)
     s0 = (wl.philox(81).standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)
     o, s = run(case, s0, 1 / np.sqrt(128.0), True)
     wo, ws = want(case, s0, 1 / np.sqrt(128.0), True)
     check(o, s, wo, ws, "B=%d nk=%d nv=%d" % (B, nk, nv))
+
+
+def test_both_workgroup_widths_give_the_same_bits():
+    """The first two sequences of a batch of 40 (64-column workgroups) against the same two alone (32-column
+    workgroups): a state column's sums do not depend on which wavefront owns it."""
+    B, T, nk, nv = 40, 130, 2, 4
+    case = wl.deltanet_case(90, B, T, nk, nv, 128, 128)
+    s0 = (wl.philox(91).standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)
+    o, s = run(case, s0, 1 / np.sqrt(128.0), True)
+    two = {n: np.ascontiguousarray(a[:2]) for n, a in case.items() if isinstance(a, np.ndarray) and a.shape[:1] == (B,)}
+    o2, s2 = run(two, np.ascontiguousarray(s0[:2]), 1 / np.sqrt(128.0), True)
+    assert np.array_equal(o[:2], o2) and np.array_equal(s[:2], s2)
