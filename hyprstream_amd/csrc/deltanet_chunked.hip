@@ -87,16 +87,26 @@ __device__ __forceinline__ void unpack16(const u32x4 &a, const u32x4 &b, float *
     }
 }
 
+// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for global accesses in flight (the
+// walk's prefetch, the factor kernel's stores into the workspace, which nothing in the same launch reads).
+__device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// v of the lane a DPP control selects (0x110 + n: n lanes down inside a row of 16; 0x142 / 0x143: lane 15 / 31 of the
+// preceding rows), 0 for a lane without a source or in a row that kRows masks out.
+template <int kCtrl, int kRows>
+__device__ __forceinline__ float dpp_or_zero(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, kRows, 0xf, false));
+}
+
 // ------------------------------------------------------------------------------------------------- factors
 constexpr int kPitchH = 136;  // halves per row of the row-major k / q tiles
 constexpr int kPitchL = 68;   // halves per row of the 64 x 64 matrix P = L^T
 constexpr int kPitchD = 20;   // floats per row of a 16 x 16 fp32 block
 constexpr int kBlockD = 16 * kPitchD;
-// Region A: the row-major k / q tiles; once the two products are done, the scratch blocks of the four inverses, P and
-// its diagonal blocks.
-constexpr int kLdsKh = 0, kLdsQh = 17408, kLdsS = 0;
-constexpr int kLdsP = 12 * kBlockD * 4, kLdsD = kLdsP + 64 * kPitchL * 2;
-static_assert(kLdsD + 4 * kBlockD * 4 <= 34816, "scratch, P and the diagonal blocks inside the dead k / q tiles");
+// Region A: the row-major k / q tiles; once the two products are done, P and its diagonal blocks.
+constexpr int kLdsKh = 0, kLdsQh = 17408;
+constexpr int kLdsP = 0, kLdsD = kLdsP + 64 * kPitchL * 2;
+static_assert(kLdsD + 4 * kBlockD * 4 <= 34816, "P and the diagonal blocks inside the dead k / q tiles");
 constexpr int kLdsF = 34816, kLdsBytes = kLdsF + 1536;
 static_assert(4 * kLdsBytes <= 163840, "four workgroups of the factor kernel per CU");
 
@@ -108,16 +118,14 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
     _Float16 *kh = (_Float16 *)(lds + kLdsKh), *qh = (_Float16 *)(lds + kLdsQh);
     _Float16 *Ph = (_Float16 *)(lds + kLdsP);  // P[j][i] = L[i][j], outside the diagonal blocks
     float *Dm = (float *)(lds + kLdsD);        // the four diagonal blocks of P, later of (I - P)^-1
-    float *Sm = (float *)(lds + kLdsS);        // scratch blocks of the inverses, once the k / q tiles are dead
     float *gs = (float *)(lds + kLdsF), *bs = gs + 64, *Gs = gs + 128, *km = gs + 192;  // km: 64 x (kmul, qmul)
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15, lq = lane >> 4;
-    const int64_t unit = blockIdx.x;
-    const int c = (int)(unit % a.nc);
-    const int j = (int)((unit / a.nc) % a.nv);
-    const int b = (int)(unit / ((int64_t)a.nc * a.nv));
+    const uint32_t unit = blockIdx.x, uv = unit / (uint32_t)a.nc;  // 32-bit: the grid is one
+    const int c = (int)(unit - uv * (uint32_t)a.nc);
+    const int b = (int)(uv / (uint32_t)a.nv), j = (int)(uv - (uint32_t)b * (uint32_t)a.nv);
     const int hk = j / (a.nv / a.nk);
     uint8_t *wsu = a.ws + ((int64_t)c * a.B * a.nv + (int64_t)b * a.nv + j) * kUnitBytes;
 
@@ -125,12 +133,14 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
     const int tt = tid >> 3, part = tid & 7;
     {
         const int t = c * kC + tt;
-        const bool valid = t < a.T;
-        float kf[16], qf[16];
-#pragma unroll
-        for (int e = 0; e < 16; ++e) kf[e] = qf[e] = 0.0f;
-        if (valid) {
-            const int64_t bt = (int64_t)b * a.T + t;
+        const bool valid = t < a.T;  // a row past T reads the last row and gets the factor zero
+        float kf[16], qf[16], gt = 0.0f, bt_ = 0.0f;
+        {
+            const int64_t bt = (int64_t)b * a.T + min(t, a.T - 1);
+            if (part == 0) {  // requested with the rows, not where they are used
+                gt = a.g[bt * a.nv + j];
+                bt_ = a.beta[bt * a.nv + j];
+            }
             const uint16_t *kp = a.k + (bt * a.nk + hk) * kWD + 16 * part;
             const uint16_t *qp = a.q + (bt * a.nk + hk) * kWD + 16 * part;
             unpack16(*(const u32x4 *)kp, *(const u32x4 *)(kp + 8), kf);
@@ -144,14 +154,20 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
                 sk += kf[e] * kf[e];
                 sq += qf[e] * qf[e];
             }
-#pragma unroll
-            for (int o = 1; o < 8; o <<= 1) {  // the eight threads of a token are eight consecutive lanes
-                sk += __shfl_xor(sk, o, 64);
-                sq += __shfl_xor(sq, o, 64);
-            }
-            kmul = 1.0f / fmaxf(sqrtf(sk), 1e-3f);
-            qmul = a.q_scale / fmaxf(sqrtf(sq), 1e-3f);
+            // the eight threads of a token are eight consecutive lanes: neighbours in a quad, the other pair of the quad
+            // (quad_perm [1,0,3,2], [2,3,0,1]), then the mirrored lane of the other quad (row_half_mirror); every
+            // lane adds the same two numbers at each step, so all eight hold the same sum
+            sk += dpp_or_zero<0xb1, 0xf>(sk);
+            sq += dpp_or_zero<0xb1, 0xf>(sq);
+            sk += dpp_or_zero<0x4e, 0xf>(sk);
+            sq += dpp_or_zero<0x4e, 0xf>(sq);
+            sk += dpp_or_zero<0x141, 0xf>(sk);
+            sq += dpp_or_zero<0x141, 0xf>(sq);
+            // 1 / max(|x|, 1e-3) as min(rsq(|x|^2), 1e3): one instruction (1 ulp) instead of a rounded sqrt and divide
+            kmul = fminf(__builtin_amdgcn_rsqf(sk), 1e3f);
+            qmul = a.q_scale * fminf(__builtin_amdgcn_rsqf(sq), 1e3f);
         }
+        if (!valid) kmul = qmul = 0.0f;
         half8 k8[2], q8[2];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
@@ -163,23 +179,27 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
         *(half8 *)&qh[tt * kPitchH + 16 * part] = q8[0];
         *(half8 *)&qh[tt * kPitchH + 16 * part + 8] = q8[1];
         if (part == 0) {
-            gs[tt] = valid ? a.g[((int64_t)b * a.T + t) * a.nv + j] : 0.0f;
-            bs[tt] = valid ? a.beta[((int64_t)b * a.T + t) * a.nv + j] : 0.0f;
-            km[2 * tt] = valid ? kmul : 0.0f;  // rows past T are zero
-            km[2 * tt + 1] = valid ? qmul : 0.0f;
+            gs[tt] = valid ? gt : 0.0f;
+            bs[tt] = valid ? bt_ : 0.0f;
+            km[2 * tt] = kmul;
+            km[2 * tt + 1] = qmul;
         }
     }
-    __syncthreads();
+    lds_sync();
 
     // ---- 2. running sum of g and the decay factors (wavefront 0)
     if (wave == 0) {
+        // inclusive scan over the 64 lanes with DPP moves (no trip through the LDS pipe per step): inside each row of
+        // 16 lanes by shifts of 1, 2, 4, 8 (a lane with no source gets 0), then lane 15 of a row into the next row
+        // (rows 1 and 3) and lane 31 into rows 2 and 3
         float x = gs[lane];
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const float y = __shfl_up(x, o, 64);
-            if (lane >= o) x += y;
-        }
-        const float g63 = __shfl(x, 63, 64);
+        x += dpp_or_zero<0x111, 0xf>(x);
+        x += dpp_or_zero<0x112, 0xf>(x);
+        x += dpp_or_zero<0x114, 0xf>(x);
+        x += dpp_or_zero<0x118, 0xf>(x);
+        x += dpp_or_zero<0x142, 0xa>(x);
+        x += dpp_or_zero<0x143, 0xc>(x);
+        const float g63 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
         const float e = expf(x);
         Gs[lane] = x;
         *(float *)(wsu + kOffFn + 4 * lane) = -e * km[2 * lane];
@@ -208,7 +228,7 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
             qk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bq, qk[x], 0, 0, 0);
         }
     }
-    __syncthreads();  // G and beta are visible
+    lds_sync();  // G and beta are visible
 #pragma unroll
     for (int x = 0; x < 2; ++x) {
         const int nt = 2 * (wave & 1) + x;
@@ -228,37 +248,33 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
         else *(half4v *)&Ph[col * kPitchL + 16 * mt + 4 * lq] = f32x4_to_half4(lv);
         if (nt >= 2 || mt < 2) *(half4v *)(wsu + kOffQK + (tri_block(nt, mt >> 1) * 64 + lane) * 16 + 8 * (mt & 1)) = m;
     }
-    __syncthreads();  // P complete; the row-major k / q tiles are dead from here on
+    lds_sync();  // P complete; the row-major k / q tiles are dead from here on
 
     // ---- 4. the diagonal 16 x 16 blocks of (I - P)^-1: (I + D)(I + D^2)(I + D^4)(I + D^8) with D the (nilpotent) block.
-    //         Wavefront a < 4 does block a by itself -- six 16x16x16 products on MFMA, the matrices passing through
-    //         its own LDS blocks between products (the LDS operations of one wavefront complete in order).
+    //         Wavefront a < 4 does block a by itself, in registers, on v_mfma_f32_16x16x16_f16.  With c(W) the
+    //         accumulator layout of a matrix W (lane (li, lq): W[4 lq + r][li]), the B operand of W is c(W) and its A
+    //         operand c(W^T) (both rounded to fp16), so a matrix kept as the pair c(W), c(W^T) multiplies without
+    //         leaving the registers: eight products in a chain of four, where a trip through LDS per product was 2,200
+    //         cycles.  The result is wanted as an A operand (step 5), i.e. as c of its transpose.
     if (wave < 4) {
-        auto mm = [&](float *dst, const float *X, const float *Y, const float *add) {
-            const half4v xa = f32x4_to_half4(*(const float4v *)&X[li * kPitchD + 4 * lq]);
-            float4v yb, cc;
+        auto mm = [](const half4v &xa, const half4v &yb, const float4v &add) { return __builtin_amdgcn_mfma_f32_16x16x16f16(xa, yb, add, 0, 0, 0); };
+        const float4v zero = {0.f, 0.f, 0.f, 0.f};
+        float *Lb = Dm + wave * kBlockD;
+        float4v d, it = *(const float4v *)&Lb[li * kPitchD + 4 * lq];  // c(D), c(D^T)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                yb[r] = Y[(4 * lq + r) * kPitchD + li];
-                cc[r] = add ? add[(4 * lq + r) * kPitchD + li] : 0.0f;
-            }
-            cc = __builtin_amdgcn_mfma_f32_16x16x16f16(xa, f32x4_to_half4(yb), cc, 0, 0, 0);
+        for (int r = 0; r < 4; ++r) d[r] = Lb[(4 * lq + r) * kPitchD + li];
+        const half4v hd = f32x4_to_half4(d), hdt = f32x4_to_half4(it);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) dst[(4 * lq + r) * kPitchD + li] = cc[r];
-            __builtin_amdgcn_wave_barrier();
-        };
-        float *Lb = Dm + wave * kBlockD, *Nb = Sm + (3 * wave) * kBlockD, *Pb = Nb + kBlockD, *Qb = Pb + kBlockD;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Nb[(4 * lq + r) * kPitchD + li] = Lb[(4 * lq + r) * kPitchD + li] + (4 * lq + r == li ? 1.0f : 0.0f);
-        __builtin_amdgcn_wave_barrier();
-        mm(Qb, Lb, Lb, nullptr);  // D^2
-        mm(Lb, Nb, Qb, Nb);       // (I + D)(I + D^2), into D's block (D itself is not needed any more)
-        mm(Pb, Qb, Qb, nullptr);  // D^4
-        mm(Nb, Lb, Pb, Lb);       // ... (I + D^4)
-        mm(Qb, Pb, Pb, nullptr);  // D^8
-        mm(Lb, Nb, Qb, Nb);       // ... (I + D^8): the inverse, where the diagonal block was
+        for (int r = 0; r < 4; ++r) it[r] += 4 * lq + r == li ? 1.0f : 0.0f;            // c((I + D)^T)
+        const half4v hq = f32x4_to_half4(mm(hdt, hd, zero)), hqt = f32x4_to_half4(mm(hd, hdt, zero));  // D^2 and its transpose
+        const float4v a1t = mm(hq, f32x4_to_half4(it), it);                             // ((I + D)(I + D^2))^T
+        const half4v hp = f32x4_to_half4(mm(hqt, hq, zero)), hpt = f32x4_to_half4(mm(hq, hqt, zero));  // D^4
+        const float4v a2t = mm(hp, f32x4_to_half4(a1t), a1t);                           // (... (I + D^4))^T
+        const half4v hr = f32x4_to_half4(mm(hpt, hp, zero));                            // D^8
+        const float4v a3t = mm(hr, f32x4_to_half4(a2t), a2t);                           // the inverse, transposed
+        *(float4v *)&Lb[li * kPitchD + 4 * lq] = a3t;  // row li, columns 4 lq + r: where the diagonal block was
     }
-    __syncthreads();
+    lds_sync();
 
     // ---- 5. Y = (I - P)^-1 = N^T by block back substitution, Y_b = Y_bb (I_b + sum_{m>b} P_bm Y_m), on
     //         v_mfma_f32_16x16x16_f16: wavefront w < 4 owns the 16 columns i of block w and walks the row blocks
@@ -296,8 +312,6 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
 }
 
 // ---------------------------------------------------------------------------------------------------- walk
-// Workgroup barrier that orders LDS traffic only: __syncthreads() would also wait for the loaders' global prefetch.
-__device__ __forceinline__ void lds_sync() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // One chunk's operands in LDS; A operand blocks are 64 lanes x 16 B.
 constexpr int kPitchT = 72;  // halves per row of the transposed k tile [dk][token]
