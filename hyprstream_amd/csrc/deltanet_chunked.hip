@@ -222,10 +222,14 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
 #pragma unroll
         for (int x = 0; x < 2; ++x) {
             const int nt = 2 * (wave & 1) + x;
-            const half8 bk = *(const half8 *)&kh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
-            const half8 bq = *(const half8 *)&qh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
-            kk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bk, kk[x], 0, 0, 0);
-            qk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bq, qk[x], 0, 0, 0);
+            if (nt <= mt) {  // L is kept below the diagonal only, M on and above it: 20 of the 32 tile products
+                const half8 bk = *(const half8 *)&kh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
+                kk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bk, kk[x], 0, 0, 0);
+            }
+            if (nt >= mt) {
+                const half8 bq = *(const half8 *)&qh[(16 * nt + li) * kPitchH + 32 * s + 8 * lq];
+                qk[x] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ar, bq, qk[x], 0, 0, 0);
+            }
         }
     }
     lds_sync();  // G and beta are visible
