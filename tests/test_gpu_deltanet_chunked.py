@@ -173,3 +173,20 @@ def test_both_workgroup_widths_give_the_same_bits():
     two = {n: np.ascontiguousarray(a[:2]) for n, a in case.items() if isinstance(a, np.ndarray) and a.shape[:1] == (B,)}
     o2, s2 = run(two, np.ascontiguousarray(s0[:2]), 1 / np.sqrt(128.0), True)
     assert np.array_equal(o[:2], o2) and np.array_equal(s[:2], s2)
+
+
+def test_rows_below_the_norm_floor():
+    """l2_normalize divides by max(|x|, 1e-3) (qwen3_5.rs:331-335): rows of k and q with a norm of about 1e-4 are scaled
+    by 1e3 and stay small, all-zero rows stay zero (no 0 * inf)."""
+    B, T, nk, nv = 1, 150, 2, 4
+    case = wl.deltanet_case(92, B, T, nk, nv, 128, 128)
+    f, tb = wl.bf16_bits_to_f32, wl.to_bf16_bits
+    for name in ("k_bits", "q_bits"):
+        x = f(case[name]).copy()
+        x[:, 3::7] *= 2.0 ** -17  # exact in bf16
+        x[:, 5::11] = 0.0
+        case[name] = tb(x)
+    s0 = (wl.philox(93).standard_normal((B, nv, 128, 128)) * 0.2).astype(np.float32)
+    o, s = run(case, s0, 1 / np.sqrt(128.0), True)
+    wo, ws = want(case, s0, 1 / np.sqrt(128.0), True)
+    check(o, s, wo, ws, "rows below the norm floor")
