@@ -17,6 +17,7 @@ HS_ERR_OVERFLOW = 2
 HS_ERR_WORKSPACE = 3
 HS_ERR_LAUNCH = 4
 HS_ERR_POOL_EXHAUSTED = 5
+HS_ERR_BUSY = 6
 HS_BF16, HS_F32, HS_F16 = 0, 1, 2
 
 EXPORTS = [

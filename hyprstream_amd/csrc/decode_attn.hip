@@ -34,6 +34,7 @@
 //
 // HBM bytes per cached token and kv-head: 2*D codes + 8 B of scales (int8) -- 264 B at D = 128.
 #include <atomic>
+#include <mutex>
 
 #include "quant_device.hpp"
 
@@ -63,6 +64,59 @@ static int scratch_of_current_device(void **out) {
         g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing first calls store the same address
     }
     *out = p;
+    return HS_OK;
+}
+
+// Calls that use the array must not overlap on a GPU.  Calls on one stream follow each other; a call on another
+// stream is refused while the stream of the previous call still has work pending.  No event is created or recorded
+// (the entry point allocates nothing and may run under graph capture): the test is hipStreamQuery on the previous
+// stream, which is conservative (any pending work there counts).
+struct ScratchUse {
+    std::mutex mu;
+    hipStream_t last = nullptr;
+    bool valid = false;
+};
+static ScratchUse g_scratch_use[kMaxDevices];
+
+static bool stream_blocks_with_default(hipStream_t s) {
+    if (!s) return true;
+    unsigned flags = 0;
+    if (hipStreamGetFlags(s, &flags) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+    }
+    return (flags & hipStreamNonBlocking) == 0;
+}
+
+static int claim_scratch(hipStream_t stream) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return fail(HS_ERR_LAUNCH, "hipGetDevice failed");
+    ScratchUse &u = g_scratch_use[dev];
+    std::lock_guard<std::mutex> lock(u.mu);
+    if (u.valid && u.last != stream) {
+        // the legacy default stream and a blocking stream wait for each other's work: ordered like one stream
+        const bool ordered = (!stream && stream_blocks_with_default(u.last)) || (!u.last && stream_blocks_with_default(stream));
+        if (!ordered) {
+            hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+            if (u.last && hipStreamIsCapturing(u.last, &cs) != hipSuccess) {
+                (void)hipGetLastError();  // the stream no longer exists: nothing of it is pending
+                cs = hipStreamCaptureStatusNone;
+                u.valid = false;
+            }
+            if (cs != hipStreamCaptureStatusNone)
+                return fail(HS_ERR_BUSY, "the built-in split-K scratch of this GPU is being captured on another stream");
+            if (u.valid) {
+                const hipError_t q = hipStreamQuery(u.last);
+                if (q == hipErrorNotReady)
+                    return fail(HS_ERR_BUSY,
+                                "the built-in split-K scratch of this GPU is in use on another stream: call on that "
+                                "stream, wait for it, or use hs_decode_attn_int8 with a workspace per stream");
+                if (q != hipSuccess) (void)hipGetLastError();
+            }
+        }
+    }
+    u.last = stream;
+    u.valid = true;
     return HS_OK;
 }
 
@@ -751,6 +805,13 @@ __global__ __launch_bounds__(256) void decode_merge_kernel(const float *part_o, 
     }
 }
 
+// The balanced instances read their arguments anew from the kernel-argument segment, reinterpreted as DecodeArgs:
+// that is only right while DecodeArgs is the kernel's sole parameter (it then starts at offset 0 of the segment) and
+// is passed by value as plain bytes.
+static_assert(std::is_trivially_copyable<DecodeArgs>::value, "DecodeArgs is read back as raw kernel-argument bytes");
+static_assert(std::is_same<decltype(&decode_attn_kernel<128, false, false, true>), void (*)(DecodeArgs)>::value,
+              "decode_attn_kernel must take DecodeArgs and nothing else");
+
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
 int check_prologue(const hs_qk_prologue *p, int dtype, int D, bool need_q, bool need_k);
 NormSpec norm_spec(const hs_qk_prologue *p, int which);
@@ -800,11 +861,19 @@ static Split pick_split(int B, int Hkv, int max_seq_len, int64_t total_tokens_hi
     return s;
 }
 
-// most partial slots per sequence any call can use, for sizing a workspace without knowing the hint
+// Most partial slots per sequence that a call with THIS max_seq_len or any smaller one can use, whatever its hint:
+// a caller sizes its workspace once, for the capacity of its cache, and then calls with the length it has reached.
+// pick_split's own slot count is not monotone in max_seq_len (chunks are rounded up to 128 tokens, so
+// ceil(L / chunk_tokens) drops when L passes certain multiples), hence a bound and not pick_split's value:
+// fixed chunks never exceed want_chunks nor ceil(L / 256) (a chunk is at least 256 tokens); balanced ranges never
+// exceed ceil(g / 8) + 1 while a range is 8 granules (g <= 128 granules of 64 tokens) and 17 beyond.
 static int max_slots(int B, int Hkv, int max_seq_len) {
+    const int64_t units = (int64_t)B * Hkv;
+    const int64_t want_chunks = units >= 512 ? 1 : (512 + units - 1) / units;
+    const int64_t fixed = std::min<int64_t>(want_chunks, ((int64_t)max_seq_len + 255) / 256);
     const int gmax = (max_seq_len + 63) / 64;
-    const int mg = std::max(8, (gmax + 15) / 16);
-    return std::max(pick_split(B, Hkv, max_seq_len, 0).nchunks, (gmax + mg - 1) / mg + 1);
+    const int64_t balanced = B <= kMaxBalancedB ? (gmax <= 128 ? (gmax + 7) / 8 + 1 : 17) : 1;
+    return (int)std::max<int64_t>(1, std::max(fixed, balanced));
 }
 
 struct NewToken {  // optional quantize-on-write of one token per sequence inside the same call
@@ -852,6 +921,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
                         "this shape needs %zu bytes of split-K scratch (%d chunks per sequence), the built-in scratch "
                         "holds %zu: use hs_decode_attn_int8 with a caller workspace", need, a.nchunks, kScratchBytes);
         if (int rc = scratch_of_current_device(&ws)) return rc;
+        if (need > 0)
+            if (int rc = claim_scratch(stream)) return rc;
     } else {
         const size_t need = hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, max_seq_len);
         if (!ws || ws_bytes < need)
@@ -894,6 +965,13 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
     a.rotary_dim = rd;
     a.qnorm = nt.qnorm;
     const bool pro = nt.prologue || a.rope_sin != nullptr;
+    // the fused prologue reads the norm weights and the rotary tables with 16-byte loads
+    for (const void *p : {(const void *)a.rope_sin, (const void *)a.rope_cos, (const void *)nt.qnorm.weight,
+                          (const void *)nt.knorm.weight})
+        if (((uintptr_t)p & 15) != 0)
+            return fail(HS_ERR_INVALID_ARGUMENT,
+                        "the fused decode step needs 16-byte aligned norm weights and rotary tables: run "
+                        "hs_qk_prologue_apply (which takes any alignment) and hs_decode_step_* instead");
     if (phases & 1) {
         const dim3 grid = a.balanced ? dim3(a.pieces, Hkv, 1) : dim3(a.nchunks, Hkv, B);
 #define HS_DECODE_LAUNCH(DD, BAL)                                                                      \

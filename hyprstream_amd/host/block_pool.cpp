@@ -130,6 +130,8 @@ PagedLayerKVCache::~PagedLayerKVCache() {
     clear();
     for (void *p : {(void *)table_dev_, (void *)len_dev_, (void *)head_scales_dev_, workspace_})
         if (p) (void)hipFree(p);
+    if (table_host_) (void)hipHostFree(table_host_);
+    if (table_copied_) (void)hipEventDestroy(table_copied_);
 }
 
 Status PagedLayerKVCache::reserve(size_t end_pos) {
@@ -149,27 +151,44 @@ Status PagedLayerKVCache::reserve(size_t end_pos) {
 }
 
 // New table entries (a block pair every 256 tokens) go to the device with a copy ordered on the caller's stream, so
-// a kernel of an earlier step on that stream never sees a table that changes under it.
+// a kernel of an earlier step on that stream never sees a table that changes under it.  The copy's source is a
+// pinned mirror of the table (a copy from pageable std::vector storage is staged by the runtime, blocks the host and
+// cannot be recorded under stream capture).  Appending never touches mirror entries an earlier copy may still be
+// reading; only after blocks were returned (clear / truncate_to) are entries rewritten, and then the last copy's
+// event is waited for first.
 Status PagedLayerKVCache::sync_table(hs_stream_t stream) {
-    const size_t max_blocks = (max_seq_len + kBlockSize - 1) / kBlockSize;
+    const size_t max_blocks = std::max<size_t>((max_seq_len + kBlockSize - 1) / kBlockSize, 1);
     hipError_t e;
     if (!table_dev_) {
-        if ((e = hipMalloc((void **)&table_dev_, 2 * std::max<size_t>(max_blocks, 1) * sizeof(int32_t))) != hipSuccess)
+        if ((e = hipMalloc((void **)&table_dev_, 2 * max_blocks * sizeof(int32_t))) != hipSuccess)
             return hip_err(e, "allocating the block table");
+        if ((e = hipHostMalloc((void **)&table_host_, 2 * max_blocks * sizeof(int32_t), hipHostMallocDefault)) != hipSuccess)
+            return hip_err(e, "allocating the pinned block table");
+        if ((e = hipEventCreateWithFlags(&table_copied_, hipEventDisableTiming)) != hipSuccess) return hip_err(e, "creating an event");
         if ((e = hipMalloc((void **)&len_dev_, sizeof(int32_t))) != hipSuccess) return hip_err(e, "allocating the length");
         if (pool_->fp8() && (e = hipMalloc((void **)&head_scales_dev_, 2 * sizeof(float) * pool_->num_kv_heads())) != hipSuccess)
             return hip_err(e, "allocating the head scales");
         table_synced_ = 0;
+        mirror_high_ = 0;
     }
     if (table_synced_ > key_blocks_.size()) table_synced_ = 0;  // blocks were returned: rewrite what is left
     const size_t n = key_blocks_.size() - table_synced_;
     if (n) {
-        if ((e = hipMemcpyAsync(table_dev_ + table_synced_, key_blocks_.data() + table_synced_, n * sizeof(int32_t),
-                                hipMemcpyHostToDevice, (hipStream_t)stream)) != hipSuccess ||
-            (e = hipMemcpyAsync(table_dev_ + max_blocks + table_synced_, value_blocks_.data() + table_synced_,
-                                n * sizeof(int32_t), hipMemcpyHostToDevice, (hipStream_t)stream)) != hipSuccess)
+        if (table_synced_ < mirror_high_) {  // entries an earlier copy read are about to change
+            if ((e = hipEventSynchronize(table_copied_)) != hipSuccess) return hip_err(e, "waiting for the last table upload");
+            mirror_high_ = table_synced_;
+        }
+        int32_t *hk = table_host_ + table_synced_, *hv = table_host_ + max_blocks + table_synced_;
+        std::copy(key_blocks_.begin() + table_synced_, key_blocks_.end(), hk);
+        std::copy(value_blocks_.begin() + table_synced_, value_blocks_.end(), hv);
+        if ((e = hipMemcpyAsync(table_dev_ + table_synced_, hk, n * sizeof(int32_t), hipMemcpyHostToDevice,
+                                (hipStream_t)stream)) != hipSuccess ||
+            (e = hipMemcpyAsync(table_dev_ + max_blocks + table_synced_, hv, n * sizeof(int32_t), hipMemcpyHostToDevice,
+                                (hipStream_t)stream)) != hipSuccess)
             return hip_err(e, "uploading the block table");
+        if ((e = hipEventRecord(table_copied_, (hipStream_t)stream)) != hipSuccess) return hip_err(e, "recording the table upload");
         table_synced_ = key_blocks_.size();
+        mirror_high_ = std::max(mirror_high_, table_synced_);
     }
     return {};
 }

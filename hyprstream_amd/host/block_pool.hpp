@@ -124,7 +124,10 @@ class PagedLayerKVCache {
     int32_t *table_dev_ = nullptr;  // [2][max_blocks]: row 0 = K blocks, row 1 = V blocks
     int32_t *len_dev_ = nullptr;
     float *head_scales_dev_ = nullptr;  // fp8 pools: [2][Hkv], K then V, calibrated by the update at start_pos 0
+    int32_t *table_host_ = nullptr; // pinned mirror of the table, the source of the uploads
+    hipEvent_t table_copied_ = nullptr;  // recorded behind the last upload
     size_t table_synced_ = 0;       // number of blocks the device table already holds
+    size_t mirror_high_ = 0;        // mirror entries below this index may still be read by an upload in flight
     void *workspace_ = nullptr;
     size_t workspace_bytes_ = 0;
 };

@@ -62,7 +62,8 @@ enum hs_status {
     HS_ERR_OVERFLOW = 2,         /* write past capacity_tokens (kv_cache.rs:1288-1294 "Cache overflow") */
     HS_ERR_WORKSPACE = 3,        /* workspace too small */
     HS_ERR_LAUNCH = 4,           /* hipGetLastError() after the launch */
-    HS_ERR_POOL_EXHAUSTED = 5    /* host-side block pool has no free block (fail-soft, hs_kv_cache.h) */
+    HS_ERR_POOL_EXHAUSTED = 5,   /* host-side block pool has no free block (fail-soft, hs_kv_cache.h) */
+    HS_ERR_BUSY = 6              /* hs_decode_attn_int8_static: the GPU's built-in scratch is in use on another stream */
 };
 
 enum hs_dtype { HS_BF16 = 0, HS_F32 = 1, HS_F16 = 2 };
@@ -222,9 +223,14 @@ HS_API int hs_decode_attn_int8(const void *q, const int8_t *k_codes, const int8_
  * hs_decode_attn_int8.  A shape whose split needs more than 32 MiB of partials
  * (B * Hq * chunks * (D + 2) * 4 bytes, chunks = hs_decode_attn_num_chunks(...); nothing when chunks == 1) is refused
  * with HS_ERR_WORKSPACE.  The array keeps the previous call's partials; nothing in it has to start at zero, because the
- * merge reads only what the same call wrote.  All calls on one GPU share that GPU's array: calls that overlap on one
- * GPU (different streams or threads) race.  The array's address is looked up on the first call on each device
- * (hipGetSymbolAddress, no allocation); make that first call outside graph capture. */
+ * merge reads only what the same call wrote.  All calls on one GPU share that GPU's array, so calls that could overlap
+ * on one GPU are refused: a call whose split uses the array, on a stream other than the one the previous such call on
+ * this GPU was given, returns HS_ERR_BUSY (nothing launched) while that previous stream still has work pending
+ * (hipStreamQuery; the legacy default stream and a blocking stream order each other and count as one).  Calls on one
+ * stream follow each other and are always accepted.  What the guard cannot see: launches recorded under graph capture
+ * run when the graph is replayed, so keep replays of graphs that hold this call and other users of the array on one
+ * stream.  The array's address is looked up on the first call on each device (hipGetSymbolAddress, no allocation);
+ * make that first call outside graph capture. */
 HS_API int hs_decode_attn_int8_static(const void *q, const int8_t *k_codes, const int8_t *v_codes,
                         const float *k_scales, const float *v_scales, const hs_kv_layout *layout,
                         const int32_t *seq_lens, void *out,
@@ -262,7 +268,9 @@ HS_API int hs_decode_step_int8_rope(const void *q, const void *k_new, const void
 /* The step with the whole prologue inside the launch: QK-norm of q and k_new, then their rotation (hs_qk_prologue above;
  * q [B, Hq, D], k_new [B, 1, Hkv, D], v_new in bf16 as projected; table row = seq_lens[b] - 1).  Rotated parts the
  * kernel serves: rotary_dim = head_dim, or 128, 64, 32 leading elements (Qwen3.5: 64 of 256); anything else is
- * HS_ERR_INVALID_ARGUMENT (run hs_qk_prologue_apply + hs_decode_step_int8).  Results equal those calls' bit for bit. */
+ * HS_ERR_INVALID_ARGUMENT (run hs_qk_prologue_apply + hs_decode_step_int8).  The norm weights and the rotary tables
+ * must be 16-byte aligned here (the launch reads them 16 bytes at a time; hs_qk_prologue_apply takes any alignment),
+ * else HS_ERR_INVALID_ARGUMENT.  Results equal those calls' bit for bit. */
 HS_API int hs_decode_step_int8_prologue(const void *q, const void *k_new, const void *v_new, const hs_qk_prologue *prologue,
                                int8_t *k_codes, int8_t *v_codes, float *k_scales, float *v_scales,
                                const hs_kv_layout *layout, const int32_t *seq_lens, void *out,

@@ -172,6 +172,28 @@ def test_chunk_policy_unsplit_for_uniform_and_split_for_ragged_hint():
     assert hb.decode_workspace_bytes(B, Hq, Hkv, D, T) >= 17 * per_chunk >= n * per_chunk
 
 
+@pytest.mark.parametrize("cap", [2508, 10000, 20000, 40960, 100000, 128000])
+def test_workspace_sized_for_the_capacity_covers_every_shorter_call(cap):
+    """A cache object sizes its workspace once, for its capacity, and then calls with the length it has reached
+    (LayerKVCache::decode_step passes seq_pos).  The split's slot count is not monotone in the length (chunks are
+    rounded up to 128 tokens), so the size the library asks for must bound every shorter call, with any hint."""
+    L = hb.lib()
+    Hq, D = 32, 128
+    for B, Hkv in ((1, 8), (1, 4), (2, 2), (4, 8), (64, 8)):
+        have = L.hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, cap)
+        per_slot = B * Hq * (D + 2) * 4
+        step = 1 if cap <= 20000 else 7
+        worst = 0
+        for n in list(range(1, cap + 1, step)) + [cap]:
+            worst = max(worst, L.hs_decode_attn_num_chunks(B, Hkv, n, 0),
+                        L.hs_decode_attn_num_chunks(B, Hkv, n, ctypes.c_int64(max(1, B * n // 2))))
+            # the check launch_decode itself makes is against the size for THIS call's length: it must not ask for
+            # more than the capacity's size
+            if n % 97 == 0 or n == cap:
+                assert L.hs_decode_attn_workspace_bytes(B, Hq, Hkv, D, n) <= have, (B, Hkv, n)
+        assert worst * per_slot <= have, (B, Hkv, worst, have // per_slot)
+
+
 def test_format_names_are_distinct_and_stable():
     """The names feed the reference's compatibility fingerprint (kv_compat.rs:215-237): the device formats must
     not collide with each other or with the reference's own "int8" / "nf4" / "fp4"."""

@@ -133,3 +133,35 @@ def test_chunked_prefill_then_decode_through_the_cache_object(fmt, D):
         assert d.max() < 2e-2 and d.mean() < 2e-3
     with pytest.raises(kc.CacheError, match="past the cached tokens"):
         cache.prefill(q[:, :C], k[:, :C], v[:, :C], 300, 1 / np.sqrt(D))
+
+
+def test_decode_step_where_the_split_has_more_chunks_than_at_capacity():
+    """The workspace of a cache object is sized once for its capacity, the step is launched with the length reached.
+    Capacity 20000 with one sequence of 8 KV heads: chunks of 384 tokens = 53 slots at the capacity, but a sequence
+    of 13569..16384 tokens is cut into 256-token chunks, up to 64 of them.  The step must run there (it returned a
+    workspace error when the size was taken from the split at the capacity) and match the oracle."""
+    from hyprstream_amd import bindings as hb
+    B, T, Hq, Hkv, D = 1, 14000, 32, 8, 128
+    assert hb.decode_num_chunks(B, Hkv, T) > hb.decode_num_chunks(B, Hkv, 20000)
+    k, v = randn(21, B, T, Hkv, D), randn(22, B, T, Hkv, D)
+    q = randn(23, B, Hq, D)
+    cache = kc.LayerKVCache(20000, kc.INT8)
+    cache.update(k[:, :T - 1], v[:, :T - 1], 0)
+    out = cache.decode_step(q, k[:, T - 1:], v[:, T - 1:], 1 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert cache.seq_pos == T
+    kf, vf = k.float().cpu().numpy(), v.float().cpu().numpy()
+    kc_, ks_ = oracle.quant_int8(kf)
+    vc_, vs_ = oracle.quant_int8(vf)
+    want = oracle.decode_attn(q.float().cpu().numpy(), kc_, vc_, ks_, vs_, oracle.FMT_INT8, np.full(B, T, np.int32),
+                              1 / np.sqrt(D))
+    d = np.abs(out.float().cpu().numpy() - want)
+    assert d.max() < 2e-2 and d.mean() < 2e-3
+    # the same through a paged cache of that capacity
+    pool = kc.BlockPool(64, Hkv, D)
+    paged = kc.PagedLayerKVCache(20000, pool, 1)
+    paged.update(k, v, 0)
+    got = paged.decode_attention(q, 1 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert torch.equal(got, out)
+    paged.close()

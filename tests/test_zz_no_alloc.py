@@ -69,6 +69,67 @@ def test_two_calls_in_a_row_second_smaller():
     assert torch.equal(got3.view(torch.int16), want1.view(torch.int16))
 
 
+def test_balanced_split_through_the_scratch_then_a_smaller_unhinted_call():
+    """The ragged-batch split (token ranges over the whole batch, up to 17 partial slots per sequence, counted from a
+    sequence's first range) through the built-in scratch: bits of hs_decode_attn_int8 under the same hint, and no stale
+    balanced partial leaks into a smaller fixed-chunk call that follows."""
+    Hq, Hkv, D, T = 32, 8, 128, 4096
+    B = 24
+    case = wl.decode_case(15, B, Hq, Hkv, D, T, ragged=True, outliers=True, min_len=64)
+    case["seq_lens"][0] = T          # the longest sequence fixes max_seq_len; most are far shorter
+    case["seq_lens"][1:] = np.minimum(case["seq_lens"][1:], T // 3)
+    cache = gu.DeviceCache(B, Hkv, T, D)
+    cache.write(torch.from_numpy(case["k"]).to(gu.DEV).bfloat16(), torch.from_numpy(case["v"]).to(gu.DEV).bfloat16())
+    hint = int(case["seq_lens"].sum())
+    assert hb.decode_num_chunks(B, Hkv, T, hint) > 1 and hb.decode_num_chunks(B, Hkv, T, hint) != hb.decode_num_chunks(B, Hkv, T)
+    got, want = _both(case, cache, Hq, T, hint=hint)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    _check_oracle(case, cache, got, T)
+    case2, cache2 = _case(16, 2, Hq, Hkv, D, 1024, ragged=True)
+    got2, want2 = _both(case2, cache2, Hq, 1024)
+    assert torch.equal(got2.view(torch.int16), want2.view(torch.int16))
+    _check_oracle(case2, cache2, got2, 1024)
+
+
+def test_a_call_on_another_stream_is_refused_while_the_first_stream_is_busy():
+    """All calls on a GPU share one scratch array.  A call on a second (non-blocking) stream while the first stream
+    still has work pending returns HS_ERR_BUSY and launches nothing; once the first stream has drained it is accepted
+    and gives the same bits."""
+    Hq, Hkv, D, T = 32, 8, 128, 2048
+    case, cache = _case(17, 2, Hq, Hkv, D, T, ragged=True)
+    assert hb.decode_num_chunks(2, Hkv, T) > 1
+    want, _ = _both(case, cache, Hq, T)
+    q = gu.bf16_from_bits(case["q_bits"]).to(gu.DEV)
+    lens = torch.from_numpy(case["seq_lens"]).to(gu.DEV)
+    lay = hb.contiguous_layout(Hkv, T, D)
+    scale = 1.0 / float(np.sqrt(D))
+    args = (q, cache.k_codes, cache.v_codes, cache.k_scales, cache.v_scales, lay, lens)
+    out1 = torch.zeros(2, Hq, D, dtype=torch.bfloat16, device=gu.DEV)
+    out2 = torch.full((2, Hq, D), 7.0, dtype=torch.bfloat16, device=gu.DEV)
+    big = torch.randn(8192, 8192, device=gu.DEV)
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()   # non-blocking streams, default priority
+    with torch.cuda.stream(s1):
+        for _ in range(20):
+            big = big @ big * 1e-4                       # a few hundred ms of work ahead of the call
+        hb.decode_attn_static(*args, out1, Hkv, T, scale)
+    with torch.cuda.stream(s2):
+        with pytest.raises(hb.HsError) as e:
+            hb.decode_attn_static(*args, out2, Hkv, T, scale)
+        assert e.value.code == hb.HS_ERR_BUSY and "another stream" in str(e.value)
+    s1.synchronize()
+    assert torch.all(out2 == 7.0)                        # the refused call launched nothing
+    with torch.cuda.stream(s2):
+        hb.decode_attn_static(*args, out2, Hkv, T, scale)  # the first stream has drained: accepted
+    s2.synchronize()
+    assert torch.equal(out1.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(out2.view(torch.int16), want.view(torch.int16))
+    # back on the stream the rest of the suite uses
+    torch.cuda.synchronize()
+    got, _ = _both(case, cache, Hq, T)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
 def test_no_allocation_during_the_call():
     Hq, Hkv, D, T = 16, 4, 256, 2048
     case, cache = _case(13, 2, Hq, Hkv, D, T, ragged=False)
