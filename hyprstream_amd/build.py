@@ -14,7 +14,7 @@ OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(LIBDIR, "libhs_attn.so")
 HOST_LIB = os.path.join(LIBDIR, "libhs_kv_cache.so")
 
-SOURCES = ["api.hip", "kv_quantize.hip", "decode_attn.hip", "prefill_attn.hip", "deltanet.hip", "deltanet_chunked.hip", "deltanet_glue.hip"]
+SOURCES = ["api.hip", "kv_quantize.hip", "decode_attn.hip", "prefill_attn.hip", "prefill_attn_wide.hip", "deltanet.hip", "deltanet_chunked.hip", "deltanet_glue.hip"]
 
 COMMON = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

@@ -33,12 +33,10 @@
 #include <climits>
 #include <type_traits>
 
-#include "mfma_common.hpp"
-#include "quant_device.hpp"
+#include "prefill_common.hpp"
 
 namespace hs {
 
-constexpr int kPWaves = 8;
 // head_dim 128 or 256.  What a wavefront holds is the same for both: its output tile is (16 kNB columns) x D, so
 // D = 256 halves the columns of a wavefront (and of a workgroup: 128 instead of 256) and doubles the operand
 // blocks of a key step.
@@ -50,26 +48,6 @@ template <int D> struct PShape {
     static constexpr int NC = D / DW;             // groups of d
     static constexpr int VBG = DW / 16;           // V^T operand blocks of a group: block bb holds rows d = VBG * li + bb
 };
-constexpr float kPLog2e = 1.4426950408889634f;
-constexpr float kPShift = 6.0f;  // weights are carried as 2^6 * exp2(s - m_run): keeps small ones out of the fp16 subnormals
-constexpr float kMaxScale = 512.0f;  // 127 * scale stays finite in fp16; larger magnitudes saturate instead of overflowing
-constexpr float kSlack = 4.0f;  // log2 units by which the softmax reference value overshoots a new maximum
-
-struct PrefillArgs {
-    const uint16_t *q, *kn, *vn;  // [B,S,Hq,D], [B,S,Hkv,D], [B,S,Hkv,D] bf16
-    const uint8_t *kc, *vc;
-    const float *ks, *vs;
-    KvAddr ka, va;
-    uint16_t *out;  // [B,S,Hq,D] bf16
-    const uint16_t *out_gate;  // optional [B,S,Hq,D] bf16: out = bf16(bf16(attention) * bf16(sigmoid(gate)))
-    int32_t B, S, Hq, Hkv, G, HG, hist_len;
-    const int32_t *hist_lens;  // optional, device [B]: cached tokens per sequence (then hist_len is their upper bound)
-    int32_t heavy_first;  // the grid outnumbers the CUs: order the query tiles by decreasing work
-    int32_t write_new;    // quantize-on-write of the call's K/V rows by the workgroups that finish early
-    int32_t window;       // sliding window of local layers: a query at position p attends keys in (p - window, p]; 0 = none
-    float scale_log2e;
-};
-
 template <int D> struct alignas(16) StepTile {
     uint8_t k[2 * PShape<D>::KG][1024];  // block KG*u + j: K tile u (16 keys), k-group j; 64 lanes x 16 B in MFMA lane order
     uint8_t v[PShape<D>::VB][1024];      // block 8*c + bb: V^T rows d = 128*c + 8*li + bb, 32 keys
@@ -78,10 +56,6 @@ template <int D> struct alignas(16) StepTile {
 template <int D> struct alignas(16) HistTile {
     StepTile<D> h[2];  // keys 0..31 and 32..63 of a 64-key step (history or new tokens)
 };
-
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
-// load, i.e. for the tile prefetch that was issued a moment earlier and is not needed before the next step.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // A step of one wavefront (64 keys, as two 32-key tiles) is
 //   scores  : S^T = K Q^T                     -- MFMA, operands from LDS
@@ -830,91 +804,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             }
     }
 
-    // =============================== quantize-on-write of the call's own K/V ===============================
-    // The query tiles at the front of the prompt walk the fewest keys and finish first: the first half of them
-    // (head group 0 of each kv-head) write the rows of two tiles each into the cache while the late tiles still
-    // compute.  Nothing in this launch reads those rows (the history ends below them).  D/8 lanes own a row, as in
-    // the stand-alone bulk writer, and the arithmetic per element is the same: the same codes and scales.
-    if (a.write_new && hg == 0) {
-#pragma clang fp contract(off)
-        constexpr int LPR = kRow / 8, RPW = 64 / LPR;
-        const int tile = q0 / q_per_wg, tiles = (S + q_per_wg - 1) / q_per_wg;
-        if (tile < (tiles + 1) / 2) {
-            const int t_lo = 2 * tile * q_per_wg, t_hi = min(S, t_lo + 2 * q_per_wg);
-            const int sub = lane % LPR;
-#pragma unroll 2
-            for (int tb = t_lo + wave * RPW; tb < t_hi; tb += kPWaves * RPW) {
-                const int t = tb + lane / LPR;
-                const bool live = t < t_hi;  // lanes of rows past the end still take part in the shuffles
-                const int tt = live ? t : t_hi - 1;
-                const int64_t e0 = (((int64_t)b * S + tt) * a.Hkv + kvh) * kRow + sub * 8;
-                const u32x4 wk = *(const u32x4 *)(a.kn + e0), wv = *(const u32x4 *)(a.vn + e0);
-#pragma unroll
-                for (int which = 0; which < 2; ++which) {
-                    const KvAddr &ad = which ? a.va : a.ka;
-                    const u32x4 w = which ? wv : wk;
-                    float *scales = const_cast<float *>(which ? a.vs : a.ks);
-                    int64_t unit;
-                    int slot;
-                    const bool ok = resolve(ad, b, H + tt, unit, slot) && live;
-                    float x[8];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        x[2 * i] = __uint_as_float(w[i] << 16);
-                        x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-                    }
-                    float sc = 0.0f;
-                    uint32_t packed[2] = {0u, 0u};
-                    if (FP8) {
-                        sc = scales[(int64_t)b * a.Hkv + kvh];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            float y = 0.0f;
-                            if (sc > 0.0f) {
-                                y = x[e] / sc;
-                                if (y > 448.0f) y = 448.0f;
-                                if (y < -448.0f) y = -448.0f;
-                            }
-                            packed[e >> 2] |= f32_to_e4m3fn_bits(y) << (8 * (e & 3));
-                        }
-                    } else {
-                        float m = 0.0f;
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            const float v = fabsf(x[e]);
-                            m = v > m ? v : m;
-                        }
-#pragma unroll
-                        for (int o = LPR / 2; o > 0; o >>= 1) {
-                            const float w2 = __shfl_xor(m, o, 64);
-                            m = m > w2 ? m : w2;
-                        }
-                        if (m > 0.0f) {
-                            sc = m / 127.0f;
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) {
-                                float qv = rintf(x[e] / sc);
-                                qv = qv > 127.0f ? 127.0f : qv;
-                                qv = qv < -127.0f ? -127.0f : qv;
-                                if (qv != qv) qv = 0.0f;
-                                packed[e >> 2] |= ((uint32_t)(int)qv & 0xffu) << (8 * (e & 3));
-                            }
-                        }
-                    }
-                    if (ok) {
-                        uint8_t *dst = const_cast<uint8_t *>(which ? a.vc : a.kc) + unit * ad.code_stride_seq +
-                                       (int64_t)kvh * ad.code_stride_head + (int64_t)slot * kRow + sub * 8;
-                        *(u32x2 *)dst = (u32x2){packed[0], packed[1]};
-                        if (!FP8 && sub == 0)
-                            scales[unit * ad.scale_stride_seq + (int64_t)kvh * ad.scale_stride_head + slot] = sc;
-                    }
-                }
-            }
-        }
-    }
+    if (a.write_new && hg == 0) write_new_rows<kRow, FP8>(a, b, kvh, H, q0, q_per_wg, wave, lane);
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
+void launch_prefill_wide(bool fp8, const PrefillArgs &a, dim3 grid, hipStream_t st);  // prefill_attn_wide.hip
 
 // CUs of the current device (looked up once per device; 256 if the query fails).
 static int compute_units() {
@@ -973,8 +867,12 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     // columns per workgroup: with half the columns there are twice the workgroups, each with half the matrix work
     // per step and the same conversion work.
     bool narrow = D <= 128 && q_per_wg >= 32 && 2 * (int64_t)grid.x * grid.y * grid.z <= compute_units();
-    if (layout->prefill_columns_hint == 256 || layout->prefill_columns_hint == 128)  // the caller fixes the width
-        narrow = D <= 128 && q_per_wg >= 32 && layout->prefill_columns_hint == 128;
+    const int hint = layout->prefill_columns_hint;
+    if (hint == 256 || hint == 128 || hint == 32)  // the caller fixes the width
+        narrow = D <= 128 && q_per_wg >= 32 && hint == 128;
+    // head_dim 128 at full width without a window runs on 32x32x16 MFMA tiles (prefill_attn_wide.hip) unless the caller
+    // asks for the 16x16x32 instance (256); 32 asks for it by name and is the same as 0 where it applies.
+    const bool wide32 = D == 128 && !narrow && a.window == 0 && hint != 256;
     if (narrow) {
         q_per_wg /= 2;
         grid.x = (S + q_per_wg - 1) / q_per_wg;
@@ -1001,7 +899,8 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
             else prefill_attn_kernel<256, false, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
         }                                                                                                   \
     } while (0)
-    if (a.window > 0) HS_PREFILL_LAUNCH(true);
+    if (wide32) launch_prefill_wide(fp8, a, grid, st);
+    else if (a.window > 0) HS_PREFILL_LAUNCH(true);
     else HS_PREFILL_LAUNCH(false);
 #undef HS_PREFILL_LAUNCH
     if (int rc = check_launch("prefill_attn")) return rc;

@@ -158,7 +158,7 @@ def test_decode_step_where_the_split_has_more_chunks_than_at_capacity():
     d = np.abs(out.float().cpu().numpy() - want)
     assert d.max() < 2e-2 and d.mean() < 2e-3
     # the same through a paged cache of that capacity
-    pool = kc.BlockPool(64, Hkv, D)
+    pool = kc.BlockPool(128, Hkv, D)   # 55 K blocks + 55 V blocks of 256 tokens
     paged = kc.PagedLayerKVCache(20000, pool, 1)
     paged.update(k, v, 0)
     got = paged.decode_attention(q, 1 / np.sqrt(D))
