@@ -870,9 +870,10 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     const int hint = layout->prefill_columns_hint;
     if (hint == 256 || hint == 128 || hint == 32)  // the caller fixes the width
         narrow = D <= 128 && q_per_wg >= 32 && hint == 128;
-    // head_dim 128 at full width without a window runs on 32x32x16 MFMA tiles (prefill_attn_wide.hip) unless the caller
-    // asks for the 16x16x32 instance (256); 32 asks for it by name and is the same as 0 where it applies.
-    const bool wide32 = D == 128 && !narrow && a.window == 0 && hint != 256;
+    // 32: head_dim 128 at full width without a window on 32x32x16 MFMA tiles (prefill_attn_wide.hip).  Measured slower
+    // than the 16x16x32 instance at 4 x 4096 tokens in 512-token chunks (0.77 against 0.65 ms), so the library never
+    // picks it by itself; elsewhere 32 is the same as 256.
+    const bool wide32 = D == 128 && !narrow && a.window == 0 && hint == 32;
     if (narrow) {
         q_per_wg /= 2;
         grid.x = (S + q_per_wg - 1) / q_per_wg;

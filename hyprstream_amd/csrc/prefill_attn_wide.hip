@@ -75,7 +75,7 @@ template <bool FP8>
 __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a) {
     constexpr int kRow = 128;
     constexpr int kStep = 64;  // keys per step, history and new tokens alike
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kWStepBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[4 * kWStepBytes];  // a ring of four step buffers
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int n = lane & 31, hf = lane >> 5;
@@ -153,34 +153,36 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
     const int vkey = 32 * vt + 16 * vm + 8 * (vac >> 1) + 4 * vhh + 2 * (vac & 1);
     const uint32_t vdst = kWKBytes + (vt * 2 + vm) * 4096 + (vx + 32 * vhh) * 16 + 4 * vac;
 
-    // One step of a wavefront: 64 keys whose operands are in `buf`.
-    //   scores:  16 MFMAs (tile t = i/8, d-group j = i%8); piece(i) is producer work for the next step, issued behind
-    //            MFMA i
-    //   check:   the largest score of the step against the reference (rarely: new reference, rescale)
-    //   output:  4 groups (tile g/2, key half g%2) of 4 MFMAs + the row-sum MFMA; the weights of group g + 1, two per
-    //            MFMA, are issued behind the MFMAs of group g
-    // A weight is exp2(score - sref), sref = m_run - kPShift.  Two ways to take the reference off (kSeed):
-    //   seeded     the score accumulators start from -sref (a 16-register tuple of copies) and the MFMA result is the
-    //              exponent itself: 32 vector instructions less per step, for the history walk, whose steps are full of
-    //              conversion work;
-    //   unseeded   accumulators start from zero and the subtraction (with the factor cq of a rescaled Q) is an fma in
-    //              front of every exponential: for the new tokens, whose raw rows need the registers, and for the rare
-    //              history walk with cq != 1.
+    // A step of a wavefront (64 keys) is four phases, each closed by a workgroup barrier:
+    //   M1  scores: 16 MFMAs (tile t = i/8, d-group j = i%8), operands read from LDS four MFMAs ahead
+    //   V1  softmax: the largest score against the reference (rarely: new reference, rescale), then the step's 32
+    //       weights exp2(score - sref), rounded and packed as the B operands of M2
+    //   M2  output: 4 groups (tile g/2, key half g%2) of 4 MFMAs (+ the row-sum MFMA in the history walk)
+    //   V2  producer work: this wavefront's share of the tile two steps ahead goes into LDS, the rows of the tile three
+    //       steps ahead are requested
+    // Wavefronts 4-7 run ONE PHASE BEHIND wavefronts 0-3 (w and w + 4 share a SIMD): while one wavefront of a SIMD is
+    // in a matrix phase the other is in a vector phase, so the vector work of a step runs in the shadow of the other
+    // wavefront's MFMAs without any instruction-level interleaving, and a matrix phase has the pipe to itself (one
+    // wavefront issuing 32x32x16 MFMAs back to back keeps it busy).  The tiles are therefore converted two steps ahead
+    // and live in a ring of four LDS buffers.
+    // A weight is exp2(score - sref), sref = m_run - kPShift.  Seeded (the history walk unless Q was rescaled): the score
+    // accumulators start from -sref, a 16-register tuple of copies, and the MFMA result is the exponent itself.
+    // Unseeded: accumulators start from zero and an fma (with the factor cq of a rescaled Q) precedes every exponential.
     float16v s[2];
     float sref = 0.0f;
     float16v sinit = splat16(0.0f);
+    uint32_t pk[16];  // the step's weights: four B operands of M2
+    const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;
 
-    // Operand reads are issued RN/2 MFMAs ahead of their use into a ring of RN operand registers.
-    auto scores_phase = [&](auto tag, const uint8_t *buf, const u32x4 (&qop)[8], auto &ring, const float16v &init, auto &&piece) {
+    auto scores_phase = [&](auto tag, const uint8_t *buf, const u32x4 (&qop)[8], const float16v &init) {
         typedef WideOp<decltype(tag)::value> Op;
-        constexpr int RN = sizeof(ring) / sizeof(ring[0]), RD = RN / 2;
+        u32x4 ring[8];
 #pragma unroll
-        for (int i = 0; i < RD; ++i) ring[i] = *(const u32x4 *)(buf + i * 1024);
+        for (int i = 0; i < 4; ++i) ring[i] = *(const u32x4 *)(buf + i * 1024);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            if (i + RD < 16) ring[(i + RD) % RN] = *(const u32x4 *)(buf + (i + RD) * 1024);
-            s[i >> 3] = Op::mfma(ring[i % RN], qop[i & 7], (i & 7) == 0 ? init : s[i >> 3]);
-            piece(i);
+            if (i + 4 < 16) ring[(i + 4) & 7] = *(const u32x4 *)(buf + (i + 4) * 1024);
+            s[i >> 3] = Op::mfma(ring[i & 7], qop[i & 7], (i & 7) == 0 ? init : s[i >> 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -191,9 +193,11 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
         for (int r = 1; r < 16; ++r) m = fmaxf(m, fmaxf(s[0][r], s[1][r]));
         return m;
     };
-    // In (almost) every step no score passes the reference and nothing happens here.
-    auto update_reference = [&](auto seed_tag, float cq) {
+    // In (almost) every step no score passes the reference and nothing happens in the branch.
+    auto softmax_phase = [&](auto tag, auto seed_tag, float cq) {
+        typedef WideOp<decltype(tag)::value> Op;
         constexpr bool kSeed = decltype(seed_tag)::value;
+        constexpr bool kOnesMfma = !decltype(tag)::value;  // history (f16 operands): row sums by MFMA
         const float m = kSeed ? step_max() + sref : step_max() * cq;  // the largest score, log2 units
         const float thr = (m_run == -INFINITY) ? -INFINITY : sref + kPShift;
         if (__builtin_amdgcn_ballot_w64(m > thr) != 0) {
@@ -209,43 +213,39 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
             }
             sref = nref;
         }
-    };
-    // (the first RN/2 operands of vbuf are already on their way into ring[0 .. RN/2))
-    auto output_phase = [&](auto tag, auto seed_tag, const uint8_t *vbuf, auto &ring, float cq, int ngroups) {
-        typedef WideOp<decltype(tag)::value> Op;
-        constexpr bool kSeed = decltype(seed_tag)::value;
-        constexpr bool kOnesMfma = !decltype(tag)::value;  // history (f16 operands): row sums by MFMA
-        constexpr int RN = sizeof(ring) / sizeof(ring[0]), RD = RN / 2;
-        const u32x4 ones = {Op::kOnes, Op::kOnes, Op::kOnes, Op::kOnes};
-        auto weight = [&](float x) { return __builtin_amdgcn_exp2f(kSeed ? x : fmaf(x, cq, -sref)); };
-        auto weight2 = [&](int g, int k) {  // k-slots 2k, 2k + 1 of group g
-            const int t = g >> 1, r = 8 * (g & 1) + 2 * k;
-            const float p0 = weight(s[t][r]), p1 = weight(s[t][r + 1]);
-            if (!kOnesMfma) lrow += p0 + p1;
-            return Op::pack2(p0, p1);
-        };
-        uint32_t pk[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) pk[k] = weight2(0, k);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {  // k-slots 2k, 2k + 1 of group g
+                const int t = g >> 1, r = 8 * (g & 1) + 2 * k;
+                const float p0 = __builtin_amdgcn_exp2f(kSeed ? s[t][r] : fmaf(s[t][r], cq, -sref));
+                const float p1 = __builtin_amdgcn_exp2f(kSeed ? s[t][r + 1] : fmaf(s[t][r + 1], cq, -sref));
+                if (!kOnesMfma) lrow += p0 + p1;
+                pk[4 * g + k] = Op::pack2(p0, p1);
+            }
+    };
+    auto output_phase = [&](auto tag, const uint8_t *vbuf, int ngroups) {
+        typedef WideOp<decltype(tag)::value> Op;
+        constexpr bool kOnesMfma = !decltype(tag)::value;
+        const u32x4 ones = {Op::kOnes, Op::kOnes, Op::kOnes, Op::kOnes};
+        u32x4 ring[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ring[i] = *(const u32x4 *)(vbuf + i * 1024);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if (g >= ngroups) break;
-            const u32x4 pop = {pk[0], pk[1], pk[2], pk[3]};
+            const u32x4 pop = {pk[4 * g], pk[4 * g + 1], pk[4 * g + 2], pk[4 * g + 3]};
 #pragma unroll
             for (int blk = 0; blk < 4; ++blk) {
                 const int i = 4 * g + blk;
-                if (i + RD < 16) ring[(i + RD) % RN] = *(const u32x4 *)(vbuf + (i + RD) * 1024);
-                acc[blk] = Op::mfma(ring[i % RN], pop, acc[blk]);
-                if (g < 3) pk[blk] = weight2(g + 1, blk);
+                if (i + 4 < 16) ring[(i + 4) & 7] = *(const u32x4 *)(vbuf + (i + 4) * 1024);
+                acc[blk] = Op::mfma(ring[i & 7], pop, acc[blk]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (kOnesMfma) {
-                lsum = Op::mfma(ones, pop, lsum);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            if (kOnesMfma) lsum = Op::mfma(ones, pop, lsum);
         }
     };
+    auto tile_buf = [&](int tile) { return lds + (tile & 3) * kWStepBytes; };
 
     // ------------------------------------------------------------------------------------------ history
     if (H > 0) {
@@ -310,7 +310,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
         }
 
         const int nsteps = (H + kStep - 1) / kStep;
-        // ---- producer state: raw codes and scales of the step that is converted next
+        // ---- producer state: raw codes and scales of the tile that is converted next
         u32x4 rawk = {0u, 0u, 0u, 0u};
         u32x2 rawv[2] = {{0u, 0u}, {0u, 0u}};
         float rawsk = 0.0f, rawsv[2] = {0.0f, 0.0f};
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
         const uint8_t *kb = a.kc, *vb = a.vc;
         const float *ksp = a.ks, *vsp = a.vs;
         int kleft = 0, vleft = 0;
-        // issue() is called for steps 0, 1, 2, ... in order, so the (scalar) addresses advance by a constant; a block
+        // issue() is called for tiles 0, 1, 2, ... in order, so the (scalar) addresses advance by a constant; a block
         // table is consulted only when a cursor leaves its block.
         auto issue = [&](int step) {
             const int t0 = step * kStep;
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
             }
             uint32_t ko = koff, vo0 = voff, vo1 = voff + kRow, sk = 4u * krow, sv = 4u * vkey;
             uint32_t sv1 = sv + 4u;
-            if (last < kStep - 1) {  // the last, partial step: rows past the end repeat the last one (and convert to zero)
+            if (last < kStep - 1) {  // the last, partial tile: rows past the end repeat the last one (and convert to zero)
                 ko = min(krow, last) * kRow + 32 * plq + 16 * kjp;
                 vo0 = min(vkey, last) * kRow + 8 * vx;
                 vo1 = min(vkey + 1, last) * kRow + 8 * vx;
@@ -365,32 +365,29 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
             ksp += kStep; vsp += kStep;
             kleft -= kStep; vleft -= kStep;
         };
-        // The conversion of step `step` into `dst`, in pieces (piece i is issued behind score MFMA i).  The token scales
-        // are applied here, once per workgroup: operands are fp16(code * scale * 2^-E), zero rows past the end, rows far
-        // above the head's reference saturated (prefill_attn.hip).
-        _Float16 csk = (_Float16)0.0f;
-        half2v csv = {(_Float16)0.0f, (_Float16)0.0f};
-        half8 kconv;
-        const _Float16 bias = (_Float16)1152.0f;
-        auto commit_piece = [&](uint8_t *dst, int step, int i) {
-            if (i == 0) {
-                const int last = H - 1 - step * kStep;
-                float fk = rawsk * kdown, fv0 = rawsv[0] * vdown, fv1 = rawsv[1] * vdown;
-                if (last < kStep - 1) {
-                    if (krow > last) fk = 0.0f;
-                    if (vkey > last) fv0 = 0.0f;
-                    if (vkey + 1 > last) fv1 = 0.0f;
-                }
-                const float smax = FP8 ? 64.0f * kMaxScale : kMaxScale;
-                csk = (_Float16)fminf(fk, smax);
-                csv = (half2v){(_Float16)fminf(fv0, smax), (_Float16)fminf(fv1, smax)};
-            } else if (i == 1 || i == 3) {  // K codes 0-7 / 8-15 of the lane's sixteen
-                const uint32_t w0 = rawk[i - 1], w1 = rawk[i];
-                kconv = FP8 ? e4m3x8_to_f16_div256(w0, w1) : int8x8_to_f16_biased(w0, w1) - bias;
-            } else if (i == 2 || i == 4) {
-                *(half8 *)(dst + kdst + (i == 4 ? 512 : 0)) = kconv * csk;
-            } else if (i >= 5 && i < 13) {  // V: pair bb = i - 5 of the lane's eight
-                const int bb = i - 5;
+        // The conversion of tile `step` into `dst`.  The token scales are applied here, once per workgroup: operands are
+        // fp16(code * scale * 2^-E), zero rows past the end, rows far above the head's reference saturated
+        // (prefill_attn.hip).
+        auto commit = [&](uint8_t *dst, int step) {
+            const int last = H - 1 - step * kStep;
+            float fk = rawsk * kdown, fv0 = rawsv[0] * vdown, fv1 = rawsv[1] * vdown;
+            if (last < kStep - 1) {
+                if (krow > last) fk = 0.0f;
+                if (vkey > last) fv0 = 0.0f;
+                if (vkey + 1 > last) fv1 = 0.0f;
+            }
+            const float smax = FP8 ? 64.0f * kMaxScale : kMaxScale;
+            const _Float16 csk = (_Float16)fminf(fk, smax);
+            const half2v csv = {(_Float16)fminf(fv0, smax), (_Float16)fminf(fv1, smax)};
+            const _Float16 bias = (_Float16)1152.0f;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {  // K codes 0-7 / 8-15 of the lane's sixteen
+                const uint32_t w0 = rawk[2 * i], w1 = rawk[2 * i + 1];
+                const half8 kconv = FP8 ? e4m3x8_to_f16_div256(w0, w1) : int8x8_to_f16_biased(w0, w1) - bias;
+                *(half8 *)(dst + kdst + 512 * i) = kconv * csk;
+            }
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb) {  // V: the lane's eight (key, key + 1) pairs
                 const uint32_t pair = FP8 ? e4m3_pair_to_f16_div256(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3)
                                           : int8_pair_to_f16(rawv[0][bb >> 2], rawv[1][bb >> 2], bb & 3);
                 const half2v hv = __builtin_bit_cast(half2v, pair) * csv;
@@ -398,26 +395,22 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
             }
         };
 
-        // prologue: step 0 converted, step 1 requested
+        // prologue: tiles 0 and 1 converted, tile 2 requested
         issue(0);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) commit_piece(lds, 0, i);
+        commit(tile_buf(0), 0);
         if (1 < nsteps) issue(1);
+        commit(tile_buf(1), 1);
+        if (2 < nsteps) issue(2);
         lds_barrier();
         auto walk = [&](auto seed_tag) {
+            constexpr bool kSeed = decltype(seed_tag)::value;
+            if (late) lds_barrier();  // one phase behind
             for (int st = 0; st < nsteps; ++st) {
-                const uint8_t *buf = lds + (st & 1) * kWStepBytes + lane16;
-                uint8_t *nxt = lds + ((st + 1) & 1) * kWStepBytes;
-                u32x4 ring[8];
-                // pieces 0-12 convert step st + 1 (past the last step: zero rows into the buffer nobody reads); piece 13
-                // requests the rows of step st + 2 into the registers piece 12 has just emptied
-                scores_phase(std::false_type{}, buf, qop, ring, decltype(seed_tag)::value ? sinit : splat16(0.0f), [&](int i) {
-                    if (i < 13) commit_piece(nxt, st + 1, i);
-                    else if (i == 13 && st + 2 < nsteps) issue(st + 2);
-                });
-                // V operands of the first output group, on their way while the check runs
-#pragma unroll
-                for (int i = 0; i < 4; ++i) ring[i] = *(const u32x4 *)(buf + kWKBytes + i * 1024);
+                const uint8_t *buf = tile_buf(st) + lane16;
+                __builtin_amdgcn_s_setprio(1);
+                scores_phase(std::false_type{}, buf, qop, kSeed ? sinit : splat16(0.0f));
+                __builtin_amdgcn_s_setprio(0);
+                lds_barrier();
                 const int lim = H - st * kStep;
                 if (lim < kStep) {  // the last, partial step
 #pragma unroll
@@ -426,10 +419,17 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
                         for (int r = 0; r < 16; ++r)
                             if (32 * t + 8 * (r >> 2) + 4 * hf + (r & 3) >= lim) s[t][r] = -INFINITY;
                 }
-                update_reference(seed_tag, cq);
-                output_phase(std::false_type{}, seed_tag, buf + kWKBytes, ring, cq, 4);
+                softmax_phase(std::false_type{}, seed_tag, cq);
+                lds_barrier();
+                __builtin_amdgcn_s_setprio(1);
+                output_phase(std::false_type{}, buf + kWKBytes, 4);
+                __builtin_amdgcn_s_setprio(0);
+                lds_barrier();
+                commit(tile_buf(st + 2), st + 2);  // past the last tile: zero rows into a buffer nobody reads
+                if (st + 3 < nsteps) issue(st + 3);
                 lds_barrier();
             }
+            if (!late) lds_barrier();
         };
         if (__builtin_amdgcn_ballot_w64(cq != 1.0f) != 0)
             walk(std::false_type{});
@@ -469,7 +469,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
         const uint32_t voff = vkey * (uint32_t)rstride + 8 * vx;
         u32x4 rawv[2];
         rawv[0] = rawv[1] = (u32x4){0u, 0u, 0u, 0u};
-        auto issue_k = [&](int step, uint8_t *dst) {
+        auto issue_k = [&](int step) {
+            uint8_t *dst = tile_buf(step);
             const int row = min(step * kStep + 32 * kt + n, S - 1);  // rows past the last token repeat it (masked)
             const uint16_t *kp = knb + (int64_t)row * rstride + 16 * kj + 8 * hf;
             typedef __attribute__((address_space(3))) void *lds_ptr;
@@ -489,57 +490,66 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_wide_kernel(PrefillArgs a
             rawv[0] = *(const u32x4 *)vp0;
             rawv[1] = *(const u32x4 *)vp1;
         };
-        auto commit_piece = [&](uint8_t *dst, int i) {
-            if (i >= 2 && i < 10) {
-                const int bb = i - 2;
+        auto commit_v = [&](int step) {
+            uint8_t *dst = tile_buf(step);
+#pragma unroll
+            for (int bb = 0; bb < 8; ++bb)
                 *(uint32_t *)(dst + vdst + (bb >> 1) * 1024 + (bb & 1) * 256) = pick_halves(rawv[0][bb >> 1], rawv[1][bb >> 1], bb & 1);
-            }
         };
-        // The direct loads write LDS behind the compiler's back: every one of them has landed (vmcnt) before the barrier
-        // that publishes the buffer.
-        auto publish = [&]() {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            lds_barrier();
-        };
-        issue_k(0, lds);
+        // The direct loads write LDS behind the compiler's back.  Every V2 phase starts by waiting for all of this
+        // wavefront's loads (the V rows it is about to commit were requested after the K loads of the V2 phase before),
+        // and its closing barrier publishes them: the K blocks of tile st + 3, requested in V2 of step st, are published
+        // by the barrier that closes V2 of step st + 1, two steps before their first reader.
+        // prologue: K tiles 0, 1, 2 requested; V tiles 0 and 1 committed, V tile 2 requested
+        issue_k(0);
+        if (1 < nsteps) issue_k(1);
+        if (2 < nsteps) issue_k(2);
         issue_v(0);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) commit_piece(lds, i);
+        commit_v(0);
         if (1 < nsteps) issue_v(1);
-        publish();
+        commit_v(1);
+        if (2 < nsteps) issue_v(2);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        lds_barrier();
+        if (late) lds_barrier();  // one phase behind
         for (int st = 0; st < nsteps; ++st) {
-            const uint8_t *buf = lds + (st & 1) * kWStepBytes + lane16;
-            uint8_t *nxt = lds + ((st + 1) & 1) * kWStepBytes;
+            const uint8_t *buf = tile_buf(st) + lane16;
             const int t0 = st * kStep;
-            if (st + 1 < nsteps) issue_k(st + 1, nxt);
             // a step none of whose keys a query of this wavefront may see leaves only the producer work
-            if (!wv_active || t0 > wv_qlast) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) commit_piece(nxt, i);
-                if (st + 2 < nsteps) issue_v(st + 2);
-                publish();
-                continue;
+            const bool active = wv_active && t0 <= wv_qlast;
+            if (active) {
+                __builtin_amdgcn_s_setprio(1);
+                scores_phase(std::true_type{}, buf, qop, splat16(0.0f));
+                __builtin_amdgcn_s_setprio(0);
             }
-            u32x4 ring[4];  // the raw bf16 rows of the next step take the registers of half a ring
-            // past the last step the pieces copy the last rows again into the buffer nobody reads
-            scores_phase(std::true_type{}, buf, qop, ring, splat16(0.0f), [&](int i) {
-                if (i < 12) commit_piece(nxt, i);
-                else if (i == 12 && st + 2 < nsteps) issue_v(st + 2);
-            });
+            lds_barrier();
+            if (active) {
+                if (t0 + kStep - 1 > wv_q0) {  // some (key, query) pair of this step is in the future
+                    const int qrel = min(qi, S - 1) - t0 - 4 * hf;  // key offsets 32t + 8(r/4) + r%4 beyond this are masked
 #pragma unroll
-            for (int i = 0; i < 2; ++i) ring[i] = *(const u32x4 *)(buf + kWKBytes + i * 1024);
-            if (t0 + kStep - 1 > wv_q0) {  // some (key, query) pair of this step is in the future
-                const int qrel = min(qi, S - 1) - t0 - 4 * hf;  // key offsets 32t + 8(r/4) + r%4 beyond this are masked
+                    for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        if (32 * t + 8 * (r >> 2) + (r & 3) > qrel) s[t][r] = -INFINITY;
+                        for (int r = 0; r < 16; ++r)
+                            if (32 * t + 8 * (r >> 2) + (r & 3) > qrel) s[t][r] = -INFINITY;
+                }
+                softmax_phase(std::true_type{}, std::false_type{}, 1.0f);
             }
-            update_reference(std::false_type{}, 1.0f);
-            output_phase(std::true_type{}, std::false_type{}, buf + kWKBytes, ring, 1.0f, t0 + 32 > wv_qlast ? 2 : 4);
-            publish();
+            lds_barrier();
+            if (active) {
+                __builtin_amdgcn_s_setprio(1);
+                output_phase(std::true_type{}, buf + kWKBytes, t0 + 32 > wv_qlast ? 2 : 4);
+                __builtin_amdgcn_s_setprio(0);
+            }
+            lds_barrier();
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            commit_v(st + 2);  // past the last tile: the last rows again, into a buffer nobody reads
+            if (st + 3 < nsteps) {
+                issue_k(st + 3);
+                issue_v(st + 3);
+            }
+            lds_barrier();
         }
+        if (!late) lds_barrier();
     }
 
     // ------------------------------------------------------------------------------------------ normalise and store
