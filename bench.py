@@ -394,7 +394,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
     ap.add_argument("--cap-pad", type=int, default=0, help="decode workloads: cache capacity = context length + this many tokens")
-    ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 32, 128, 256],
+    ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 16, 32, 128, 256],
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
     ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
                     help="prefill workloads: tokens per chunk call (0 = the workload's own: 512, c3-prompt 4096)")

@@ -76,8 +76,11 @@ template <int D> struct alignas(16) HistTile {
 // that would leave most CUs without a workgroup).
 // kWin: the instance with a sliding window (the checks it adds to every step cost the plain instance 2 % at 4 x 4096
 // tokens, so they are compiled in only where a window is asked for).
-template <int kPD, bool FP8, int kCols = 0, bool kWin = false>
-__global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
+// kWaves: 8, or 16 wavefronts of one 16-column block each (kCols = 1, head_dim 128): the same 256 columns per workgroup
+// on four wavefronts per SIMD with at most 128 registers; wavefronts 0-7 then convert K, wavefronts 8-15 V.
+template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8>
+__global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_attn_kernel(PrefillArgs a) {
+    static_assert(kWaves == 8 || (kWaves == 16 && kCols == 1 && kPD == 128), "sixteen wavefronts: one column block each, head_dim 128");
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
     constexpr int DW = PShape<kPD>::DW, VBG = PShape<kPD>::VBG;
     constexpr int kRow = kPD;  // elements per row of q, k, v, out and of the cache
@@ -110,7 +113,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     const int groups = (a.G + a.HG - 1) / a.HG;  // the last group of a kv-head may be partly padding (G = 3, 5, 6, 7 ...)
     const int kvh = by / groups, hg = by % groups;
     const int S = a.S, H = a.hist_lens ? min(max(a.hist_lens[b], 0), a.hist_len) : a.hist_len;
-    const int q_per_wg = 16 * (kNB * kPWaves / a.HG);
+    const int q_per_wg = 16 * (kNB * kWaves / a.HG);
     const int q0 = bx * q_per_wg;
     if (q0 >= S) return;
     const int wg_qlast = min(S - 1, q0 + q_per_wg - 1);
@@ -178,7 +181,8 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
     };
     const int obase = lane * 16;  // this lane's 16 bytes inside an operand block
     const float qscale = a.scale_log2e;
-    const bool late = __builtin_amdgcn_readfirstlane(wave >> 2) != 0;  // wavefronts w and w+4 share a SIMD
+    const bool late = __builtin_amdgcn_readfirstlane((wave >> 2) & 1) != 0;  // wavefronts w and w+4 share a SIMD
+    const int pw = kWaves == 16 ? wave & 7 : wave;  // index among the wavefronts of this one's producer role
     float vup = 1.0f;  // 2^E of the history's V operands, folded back into the accumulators when the history ends
 
     // =============================== history: int8 cache, f16 MFMA ===============================
@@ -274,12 +278,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // (head_dim 64: eight d-octets per row, so a wavefront covers eight key pairs and wavefronts 4-7 the 32 of a
         //  step; d = 8x + bb lives in block bb % 4 at operand lane 2x + bb / 4.  K: wavefront w < 4 takes tile w whole.)
         const int vx = kSplitRoles ? lane & 7 : lane & 15;
-        const int vpp = kSplitRoles ? 8 * (wave & 3) + (lane >> 3) : 4 * wave + (lane >> 4);
+        const int vpp = kSplitRoles ? 8 * (wave & 3) + (lane >> 3) : 4 * pw + (lane >> 4);
         const int vhh = vpp >> 4, vg = (vpp >> 2) & 3, vpe = vpp & 3;
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
         const int vdst = ((kSplitRoles ? 2 * vx : vx) + 16 * vg) * 16 + 4 * vpe;
-        const int ku4 = kSplitRoles ? wave & 3 : wave >> 1, kjp = kSplitRoles ? 0 : wave & 1;
-        const bool does_k = !kSplitRoles || wave < 4, does_v = !kSplitRoles || wave >= 4;
+        const int ku4 = kSplitRoles ? wave & 3 : pw >> 1, kjp = kSplitRoles ? 0 : pw & 1;
+        const bool does_k = kWaves == 16 ? wave < 8 : (!kSplitRoles || wave < 4), does_v = kWaves == 16 ? wave >= 8 : (!kSplitRoles || wave >= 4);
         const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp, vcol = 8 * vx;
         const uint32_t koff = krow * kRow + kcol, voff = vkey * kRow + vcol;
         // head_dim 256: the same lane also takes the d-halves jp + 2 (32 codes further) and the d-octet x + 16
@@ -390,7 +394,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         float4v s[kNB][4];    // scores of the step: key block u4 = 2*half + u
         half8 pop[kNB][2];    // P^T operands per half
-        constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
+        constexpr int KU = kPD == 128 && kWaves == 8 ? 2 : 1;  // 16-key tiles whose K operands are read at once
         half8 kop[KU * KG], vop[VBG];
         half8 ones;
 #pragma unroll
@@ -425,11 +429,24 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         };
         // V^T operands of half hh, 128-wide group c of d; output() consumes them and, for head_dim 256, goes on to
         // the second group by itself
+        // (sixteen wavefronts: the operands are read four at a time where they are used, to stay within 128 registers)
         auto load_v = [&](const HistTile &t, int hh, int c = 0) {
+            if constexpr (kWaves == 16) return;
 #pragma unroll
             for (int i = 0; i < VBG; ++i) vop[i] = *(const half8 *)(t.h[hh].v[VBG * c + i] + obase);
         };
         auto output = [&](const HistTile &t, int hh) {
+            if constexpr (kWaves == 16) {
+#pragma unroll
+                for (int q4 = 0; q4 < VBG; q4 += 4) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vop[i] = *(const half8 *)(t.h[hh].v[q4 + i] + obase);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[0][q4 + i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop[i], pop[0][hh], acc[0][q4 + i], 0, 0, 0);
+                }
+                return;
+            }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 if (c > 0) load_v(t, hh, c);
@@ -596,12 +613,12 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
         // (head_dim 64: eight d-octets per row, so a wavefront covers eight key pairs and wavefronts 4-7 the 32 of a
         //  step; d = 8x + bb lives in block bb % 4 at operand lane 2x + bb / 4.  K: wavefront w < 4 takes tile w whole.)
         const int vx = kSplitRoles ? lane & 7 : lane & 15;
-        const int vpp = kSplitRoles ? 8 * (wave & 3) + (lane >> 3) : 4 * wave + (lane >> 4);
+        const int vpp = kSplitRoles ? 8 * (wave & 3) + (lane >> 3) : 4 * pw + (lane >> 4);
         const int vhh = vpp >> 4, vg = (vpp >> 2) & 3, vpe = vpp & 3;
         const int vkey = 32 * vhh + 16 * (vpe >> 1) + 4 * vg + 2 * (vpe & 1);
         const int vdst = ((kSplitRoles ? 2 * vx : vx) + 16 * vg) * 16 + 4 * vpe;
-        const int ku4 = kSplitRoles ? wave & 3 : wave >> 1, kjp = kSplitRoles ? 0 : wave & 1;
-        const bool does_k = !kSplitRoles || wave < 4, does_v = !kSplitRoles || wave >= 4;
+        const int ku4 = kSplitRoles ? wave & 3 : pw >> 1, kjp = kSplitRoles ? 0 : pw & 1;
+        const bool does_k = kWaves == 16 ? wave < 8 : (!kSplitRoles || wave < 4), does_v = kWaves == 16 ? wave >= 8 : (!kSplitRoles || wave >= 4);
         const int krow = 16 * ku4 + li, kcol = 8 * KG * lq + 16 * kjp, vcol = 8 * vx;
         const uint32_t koff = krow * (uint32_t)rstride + kcol, voff = vkey * (uint32_t)rstride + vcol;  // elements
         u32x4 rawk[NC][2], rawv[NC][2];  // head_dim 256: also the d-halves jp + 2 (32 elements on) and the d-octet x + 16
@@ -654,7 +671,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             if (!wv_active || step * kNStep > wv_qlast || (kWin && step * kNStep + kNStep <= wv_lo)) return 0;
             return step * kNStep + 32 > wv_qlast ? 1 : 2;
         };
-        constexpr int KU = kPD == 128 ? 2 : 1;  // 16-key tiles whose K operands are read at once
+        constexpr int KU = kPD == 128 && kWaves == 8 ? 2 : 1;  // 16-key tiles whose K operands are read at once
         bf16x8 kop[KU * KG], vop[VBG], ones;
 #pragma unroll
         for (int e = 0; e < 8; ++e) ones[e] = (__bf16)1.0f;
@@ -679,11 +696,24 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
                 }
             }
         };
+        // (sixteen wavefronts: the operands are read four at a time where they are used, to stay within 128 registers)
         auto load_v = [&](const HistTile &t, int hh, int c = 0) {
+            if constexpr (kWaves == 16) return;
 #pragma unroll
             for (int i = 0; i < VBG; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[VBG * c + i] + obase);
         };
         auto output = [&](const HistTile &t, int hh) {
+            if constexpr (kWaves == 16) {
+#pragma unroll
+                for (int q4 = 0; q4 < VBG; q4 += 4) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) vop[i] = *(const bf16x8 *)(t.h[hh].v[q4 + i] + obase);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[0][q4 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[i], pop[0][hh], acc[0][q4 + i], 0, 0, 0);
+                }
+                return;
+            }
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 if (c > 0) load_v(t, hh, c);
@@ -804,7 +834,7 @@ __global__ __launch_bounds__(512, 2) void prefill_attn_kernel(PrefillArgs a) {
             }
     }
 
-    if (a.write_new && hg == 0) write_new_rows<kRow, FP8>(a, b, kvh, H, q0, q_per_wg, wave, lane);
+    if (a.write_new && hg == 0) write_new_rows<kRow, FP8, kWaves>(a, b, kvh, H, q0, q_per_wg, wave, lane);
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
@@ -868,12 +898,15 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     // per step and the same conversion work.
     bool narrow = D <= 128 && q_per_wg >= 32 && 2 * (int64_t)grid.x * grid.y * grid.z <= compute_units();
     const int hint = layout->prefill_columns_hint;
-    if (hint == 256 || hint == 128 || hint == 32)  // the caller fixes the width
+    if (hint == 256 || hint == 128 || hint == 32 || hint == 16)  // the caller fixes the width
         narrow = D <= 128 && q_per_wg >= 32 && hint == 128;
     // 32: head_dim 128 at full width without a window on 32x32x16 MFMA tiles (prefill_attn_wide.hip).  Measured slower
     // than the 16x16x32 instance at 4 x 4096 tokens in 512-token chunks (0.77 against 0.65 ms), so the library never
     // picks it by itself; elsewhere 32 is the same as 256.
     const bool wide32 = D == 128 && !narrow && a.window == 0 && hint == 32;
+    // 16: the same 256 columns per workgroup on sixteen wavefronts of one 16-column block each (four per SIMD, at most
+    // 128 registers), head_dim 128 without a window; elsewhere the same as 256.
+    const bool waves16 = D == 128 && !narrow && a.window == 0 && hint == 16;
     if (narrow) {
         q_per_wg /= 2;
         grid.x = (S + q_per_wg - 1) / q_per_wg;
@@ -900,7 +933,10 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
             else prefill_attn_kernel<256, false, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
         }                                                                                                   \
     } while (0)
-    if (wide32) launch_prefill_wide(fp8, a, grid, st);
+    if (waves16) {
+        if (fp8) prefill_attn_kernel<128, true, 1, false, 16><<<grid, 1024, 0, st>>>(a);
+        else prefill_attn_kernel<128, false, 1, false, 16><<<grid, 1024, 0, st>>>(a);
+    } else if (wide32) launch_prefill_wide(fp8, a, grid, st);
     else if (a.window > 0) HS_PREFILL_LAUNCH(true);
     else HS_PREFILL_LAUNCH(false);
 #undef HS_PREFILL_LAUNCH

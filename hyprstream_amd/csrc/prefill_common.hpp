@@ -39,7 +39,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 // (head group 0 of each kv-head) write the rows of two tiles each into the cache while the late tiles still
 // compute.  Nothing in this launch reads those rows (the history ends below them).  D/8 lanes own a row, as in
 // the stand-alone bulk writer, and the arithmetic per element is the same: the same codes and scales.
-template <int kRow, bool FP8>
+template <int kRow, bool FP8, int kWaves = kPWaves>
 __device__ __forceinline__ void write_new_rows(const PrefillArgs &a, int b, int kvh, int H, int q0, int q_per_wg, int wave, int lane) {
 #pragma clang fp contract(off)
     const int S = a.S;
@@ -49,7 +49,7 @@ __device__ __forceinline__ void write_new_rows(const PrefillArgs &a, int b, int 
         const int t_lo = 2 * tile * q_per_wg, t_hi = min(S, t_lo + 2 * q_per_wg);
         const int sub = lane % LPR;
 #pragma unroll 2
-        for (int tb = t_lo + wave * RPW; tb < t_hi; tb += kPWaves * RPW) {
+        for (int tb = t_lo + wave * RPW; tb < t_hi; tb += kWaves * RPW) {
             const int t = tb + lane / LPR;
             const bool live = t < t_hi;  // lanes of rows past the end still take part in the shuffles
             const int tt = live ? t : t_hi - 1;

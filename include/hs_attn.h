@@ -83,8 +83,9 @@ typedef struct hs_kv_layout {
                                    sequences do not set the time of the launch. */
     int32_t prefill_columns_hint; /* prefill only, optional: 0 = the library picks the (query, head) columns a
                                    workgroup owns from the size of the grid; 256 or 128 fixes them, 32 asks for 256
-                                   columns on 32x32 MFMA tiles (head_dim 128 without a window; elsewhere the same as
-                                   256; a measured variant the library never picks by itself).  Results are the same
+                                   columns on 32x32 MFMA tiles, 16 for 256 columns on sixteen wavefronts of at most
+                                   128 registers (both: head_dim 128 without a window; elsewhere the same as 256;
+                                   measured variants the library never picks by itself).  Results are the same
                                    within rounding every way; head_dim 256 always uses its one width. */
     int32_t prefill_window;     /* prefill only, optional: sliding window of local-attention layers (Gemma3 / Mistral;
                                    apply_sliding_window_mask, llama.rs:1086-1091, 1123-1155): a query at absolute

@@ -13,11 +13,12 @@ from gpu_util import DEV, DeviceCache, bf16_from_bits, run_decode
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["auto", "256", "128", "32"])
+@pytest.fixture(autouse=True, params=["auto", "256", "128", "32", "16"])
 def columns_per_workgroup(request, monkeypatch):
     """Every test runs with the library's own choice of workgroup width (half-width workgroups for small grids) and
-    with each instance forced -- 256 columns on 16x16x32 MFMA tiles, 128 columns, 256 columns on 32x32x16 tiles
-    (head_dim 128 without a window; elsewhere 32 is the same as 256) -- so that small shapes exercise every kernel."""
+    with each instance forced -- 256 columns on 16x16x32 MFMA tiles, 128 columns, 256 columns on 32x32x16 tiles, 256
+    columns on sixteen wavefronts (the last two: head_dim 128 without a window; elsewhere the same as 256) -- so that
+    small shapes exercise every kernel."""
     monkeypatch.setattr(hb, "PREFILL_COLUMNS", 0 if request.param == "auto" else int(request.param))
 
 TOL_MAX, TOL_MEAN = 2e-2, 2e-3
