@@ -119,8 +119,18 @@ def cpu_baseline(torch, name, caches, q, lens, Hq, fp8, seconds_budget=20.0):
     from hyprstream_amd import workloads as wl
     Hkv, D = kc.shape[1], kc.shape[3]
     nbytes = (wl.decode_bytes_fp8 if fp8 else wl.decode_bytes_int8)(np.array(lens_h), Hq, Hkv, D)
+    cpu_model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    cpu_model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {
         "value": nbytes / med / 1e9, "unit": "GB/s", "cores": int(torch.get_num_threads()), "kind": "port",
+        "nproc": int(os.cpu_count() or 0), "intra_op_threads": int(torch.get_num_threads()), "cpu_model": cpu_model,
         "sample": "first %d of %d sequences of workload %s (T=%d): libtorch CPU dequantize + GQA expand + fp32 "
                   "matmul/softmax/matmul, median of %d runs, %.1f ms per call, %.1f tokens/s"
                   % (bs, B, name, T, len(times), med * 1e3, bs / med),
@@ -163,14 +173,36 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         qw = (1.0 + 0.1 * torch.randn(D, generator=gen, device=dev)).to(torch.bfloat16)
         kw = (1.0 + 0.1 * torch.randn(D, generator=gen, device=dev)).to(torch.bfloat16)
         pro = hb.qk_prologue(hb.QKNORM_LLAMA, 1e-6, qw, kw, sin, cos)
-        q_rot, k_rot = torch.empty_like(chunks[0][0]), torch.empty_like(chunks[0][1])
+        # The projections of a prompt give q and k for all of its tokens at once (llama.rs:560-611 runs norm and rotation
+        # on the whole [B, T, H, D] tensors before cache.update), so the pre-pass is ONE launch over the prompt: the eight
+        # chunks' rows laid end to end as 8 B "sequences" of C tokens whose first positions are 0, C, 2C, ...; the chunk
+        # calls read their slices of its output.  --prologue-fused-q sends only k through the pre-pass and lets the
+        # chunk launches normalise and rotate q themselves (hs_kv_layout.prefill_q_prologue); --prologue-per-chunk runs
+        # the q + k pre-pass in front of every chunk call instead of once (eight launches of an eighth of the rows).
+        nch = len(chunks)
+        q_all = torch.cat([c[0] for c in chunks], 0).contiguous()   # [nch * B, C, Hq, D]
+        k_all = torch.cat([c[1] for c in chunks], 0).contiguous()
+        q_rot, k_rot = torch.empty_like(q_all), torch.empty_like(k_all)
+        first_pos = (torch.arange(nch * B, device=dev, dtype=torch.int32) // B * C).contiguous()
+    q_prepass = not args.prologue_fused_q or args.prologue_per_chunk
 
     def step(write=True, with_prologue=True):
+        if prologue and with_prologue and not args.prologue_per_chunk:
+            if q_prepass:
+                hb.qk_prologue_apply(q_all, k_all, pro, q_rot, k_rot, first_pos, 0)
+            else:
+                hb.qk_prologue_apply(None, k_all, pro, None, k_rot, first_pos, 0)
         for i, (qc, kcn, vcn) in enumerate(chunks):
+            fused = None
             if prologue and with_prologue:
-                hb.qk_prologue_apply(qc, kcn, pro, q_rot, k_rot, None, i * C)
-                qc, kcn = q_rot, k_rot
-            hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8)
+                kcn = k_rot[i * B:(i + 1) * B]
+                if q_prepass:
+                    qc = q_rot[i * B:(i + 1) * B]
+                    if args.prologue_per_chunk:
+                        hb.qk_prologue_apply(chunks[i][0], chunks[i][1], pro, qc, kcn, None, i * C)
+                else:
+                    fused = pro
+            hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8, q_prologue=fused)
 
     settle(torch, lambda i: step(), window=10, min_launches=100, max_launches=1000)
     for _ in range(args.warmup):
@@ -396,6 +428,10 @@ def main():
     ap.add_argument("--cap-pad", type=int, default=0, help="decode workloads: cache capacity = context length + this many tokens")
     ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 16, 32, 128, 256],
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
+    ap.add_argument("--prologue-fused-q", action="store_true",
+                    help="c3-prologue: only k goes through the pre-pass, the chunk launches normalise and rotate q themselves")
+    ap.add_argument("--prologue-per-chunk", action="store_true",
+                    help="c3-prologue: run the QK-norm + rotary pre-pass in front of every chunk call instead of once over the prompt")
     ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
                     help="prefill workloads: tokens per chunk call (0 = the workload's own: 512, c3-prompt 4096)")
     ap.add_argument("--batch", type=int, default=0, help="c5 workloads: sequences in the batch (0 = the configuration's 64 for decode, 4 for prefill)")

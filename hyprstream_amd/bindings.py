@@ -47,6 +47,7 @@ class KvLayout(ctypes.Structure):
         ("prefill_columns_hint", ctypes.c_int32),
         ("prefill_window", ctypes.c_int32),
         ("out_gate", ctypes.c_void_p),
+        ("prefill_q_prologue", ctypes.c_void_p),
     ]
 
 
@@ -292,14 +293,17 @@ PREFILL_COLUMNS = 0  # default for prefill_attn's `columns` (tests set it to run
 
 
 def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, hist_len, out, softmax_scale,
-                 quantize_on_write=True, fp8=False, hist_lens=None, columns=None, window=0):
+                 quantize_on_write=True, fp8=False, hist_lens=None, columns=None, window=0, q_prologue=None):
     """Causal attention of S new tokens over [int8 or fp8 history | their own bf16 K/V]; optionally caches them.
     hist_lens (int32 device tensor [B]): rows at different positions; hist_len is then their upper bound.
     columns: 0 = the library's choice of workgroup width, 256 or 128 fixes it (layout.prefill_columns_hint).
-    window: sliding window of local layers (layout.prefill_window), 0 = none."""
+    window: sliding window of local layers (layout.prefill_window), 0 = none.
+    q_prologue (QkPrologue): q arrives as projected and the launch normalises and rotates it
+    (layout.prefill_q_prologue); k_new arrives normalised and rotated either way."""
     B, S, Hq, D = q.shape
     layout.prefill_columns_hint = PREFILL_COLUMNS if columns is None else columns
     layout.prefill_window = window
+    layout.prefill_q_prologue = ctypes.addressof(q_prologue) if q_prologue is not None else None
     Hkv = k_new.shape[2]
     assert q.is_contiguous() and k_new.is_contiguous() and v_new.is_contiguous() and out.is_contiguous()
     if hist_lens is not None:

@@ -7,6 +7,7 @@
 //
 // Arithmetic is written to be bit-identical to the CPU oracle: IEEE fp32 division
 // (-fhip-fp32-correctly-rounded-divide-sqrt), round-half-even (v_rndne_f32), no fast-math.
+#include "prologue_rows.hpp"
 #include "quant_device.hpp"
 
 namespace hs {
@@ -303,6 +304,49 @@ __global__ __launch_bounds__(256) void qk_prologue_rows_kernel(PrologueArgs a) {
         res[i] = r2[0] | (r2[1] << 16);
     }
     *(uint4 *)((uint16_t *)a.out[which] + row * a.D + d0) = make_uint4(res[0], res[1], res[2], res[3]);
+}
+
+// qk_prologue_rows_kernel for bf16 with longer pieces: a lane owns E = 32 consecutive elements of a row (16 at head_dim
+// 64), D/E adjacent lanes a row (prologue_row_part).  What comes once per lane whatever its share -- row and position
+// arithmetic, the reciprocal root's chain of roundings, the reduction steps, the exchange's addressing -- is spread over
+// four times as many elements, which is what bounds this launch (its arithmetic, not its bytes).
+// Serves the rotary_dim values of prologue_parts_serve(rd, E).
+template <int D>
+__global__ __launch_bounds__(256) void qk_prologue_parts_kernel(PrologueArgs a) {
+    constexpr int E = D == 64 ? 16 : 32, P = D / E, kRowsPerWave = 64 / P;
+    const int lane = threadIdx.x & 63, part = lane % P;
+    const int HH = a.H[0] + a.H[1];
+    const int total = a.B * a.S * HH;
+    const int wave_row = (blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6)) * kRowsPerWave;
+    const int r_raw = wave_row + lane / P;
+    const bool live = r_raw < total;  // lanes of rows past the end still take part in the shuffles
+    const int first = min(wave_row, total - 1);
+    int bs = first / HH, hh = first - bs * HH + (min(r_raw, total - 1) - first);
+    while (hh >= HH) {
+        hh -= HH;
+        ++bs;
+    }
+    const int bs0 = first / HH;
+    int b = bs0 / a.S, s = bs0 - b * a.S + (bs - bs0);
+    while (s >= a.S) {
+        s -= a.S;
+        ++b;
+    }
+    const int which = hh >= a.H[0] ? 1 : 0, h = which ? hh - a.H[0] : hh;
+    const int pos = (a.positions ? a.positions[b] : 0) + a.start_pos + s;
+    const int64_t row = (int64_t)bs * a.H[which] + h;
+    RowPrologue p;
+    p.norm = a.norm[which];
+    p.sin_t = a.sin_t;
+    p.cos_t = a.cos_t;
+    p.rope_len = a.rope_len;
+    p.rd = a.rd;
+    u32x4 res[E / 8];
+    prologue_row_part<D, E>(p, (const uint16_t *)a.x[which] + row * D, h, pos, part, 1, lane, res);
+    if (!live) return;
+    uint16_t *dst = (uint16_t *)a.out[which] + row * D + E * part;
+#pragma unroll
+    for (int i = 0; i < E / 8; ++i) *(u32x4 *)(dst + 8 * i) = res[i];
 }
 
 // The same for many rows of a 16-bit tensor: D/8 lanes own a row, eight consecutive elements each (16-byte loads
@@ -696,6 +740,14 @@ int hs_qk_prologue_apply(const void *q, const void *k, int dtype, const hs_qk_pr
     a.rd = prologue->rotary_dim > 0 ? prologue->rotary_dim : D;
     uintptr_t bits = (uintptr_t)q | (uintptr_t)k | (uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)a.sin_t | (uintptr_t)a.cos_t;
     if (prologue->norm_kind != HS_QKNORM_NONE) bits |= (uintptr_t)a.norm[0].weight | (uintptr_t)a.norm[1].weight;
+    if (dtype == HS_BF16 && (bits & 15) == 0 && rows < (1ll << 30) && (!a.sin_t || prologue_parts_serve(a.rd, D == 64 ? 16 : 32))) {
+        const int rows_per_wg = 4 * (64 / (D / (D == 64 ? 16 : 32)));  // bf16, 16-byte accesses, 32 elements per lane
+        dim3 g((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));
+        if (D == 64) qk_prologue_parts_kernel<64><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else if (D == 128) qk_prologue_parts_kernel<128><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        else qk_prologue_parts_kernel<256><<<g, 256, 0, (hipStream_t)stream>>>(a);
+        return check_launch("qk_prologue");
+    }
     if (dtype != HS_F32 && (bits & 15) == 0 && rows < (1ll << 30)) {  // 16-bit tensors, 16-byte accesses: several rows per wavefront
         const int rows_per_wg = 4 * (64 / (D / 8));
         dim3 g((unsigned)((rows + rows_per_wg - 1) / rows_per_wg));

@@ -136,6 +136,26 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     auto qlo = [&](int nb) { return min(qi[nb], S - 1) - W + 1; };
     const int wg_lo = q0 - W + 1, wv_lo = wv_q0 - W + 1, wv_lo_last = wv_qlast - W + 1;
 
+    // q arrives as projected: its QK-norm and rotation run here, once per workgroup.  A lane's piece of the row is the
+    // piece its Q operands are made of, so the history phase takes it from registers; the row also goes to the
+    // workgroup's own rows of `out` (which nobody else touches before the final store), where the new-token phase reads
+    // it back -- each lane exactly what it wrote.  (Measured at 4 x 512 tokens per launch, Llama-flavour norm and
+    // whole-head rotation: 10 us per launch, half of it arithmetic; the same code as loops over 8-element groups, which
+    // is a fifth of the instructions, took 15 us: every iteration waits for its own loads.)
+    const uint16_t *qsrc = a.q;
+    u32x4 qpre[kNB][KG];
+    if (a.qpro.on) {
+#pragma unroll
+        for (int nb = 0; nb < kNB; ++nb) {
+            const int qrow = min(qi[nb], S - 1);
+            const int64_t row = (((int64_t)b * S + qrow) * a.Hq + head[nb]) * kRow;
+            prologue_row_part<kPD, 8 * KG>(a.qpro, a.q + row, head[nb], H + qrow, lq, 16, lane, qpre[nb]);
+#pragma unroll
+            for (int j = 0; j < KG; ++j) *(u32x4 *)(a.out + row + 8 * KG * lq + 8 * j) = qpre[nb][j];
+        }
+        qsrc = a.out;
+    }
+
     float4v acc[kNB][VB];
     float m_run[kNB];
     float4v l_run[kNB];  // row sums, kept on the matrix pipe: ones(16x32) x P^T, every register holds the column's sum
@@ -234,11 +254,11 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         bool scaled = false;
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
+            const uint16_t *qp = qsrc + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
             float qf[8 * KG], amax = 0.0f;
 #pragma unroll
             for (int i = 0; i < KG; ++i) {
-                const u32x4 w = *(const u32x4 *)(qp + 8 * i);
+                const u32x4 w = a.qpro.on ? qpre[nb][i] : *(const u32x4 *)(qp + 8 * i);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     qf[8 * i + 2 * e] = __uint_as_float(w[e] << 16) * qscale * kup;
@@ -583,9 +603,10 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         float sref[kNB];
         float4v sinit[kNB];
         int force = pending();  // columns that have seen nothing yet: their first step sets the reference
+        if (a.qpro.on) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the finished q rows this lane stored to `out`
 #pragma unroll
         for (int nb = 0; nb < kNB; ++nb) {
-            const uint16_t *qp = a.q + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
+            const uint16_t *qp = qsrc + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
 #pragma unroll
             for (int j = 0; j < KG; ++j) {
                 const u32x4 w = *(const u32x4 *)(qp + 8 * j);
@@ -838,6 +859,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
+int check_prologue(const hs_qk_prologue *p, int dtype, int D, bool need_q, bool need_k);
+NormSpec norm_spec(const hs_qk_prologue *p, int which);
 void launch_prefill_wide(bool fp8, const PrefillArgs &a, dim3 grid, hipStream_t st);  // prefill_attn_wide.hip
 
 // CUs of the current device (looked up once per device; 256 if the query fails).
@@ -889,6 +912,25 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     a.hist_lens = hist_lens;
     a.write_new = quantize_on_write ? 1 : 0;
     a.window = layout->prefill_window;
+    if (const hs_qk_prologue *qp = layout->prefill_q_prologue) {
+        if (int rc = check_prologue(qp, HS_BF16, D, true, false)) return rc;
+        const int rd = qp->rotary_dim > 0 ? qp->rotary_dim : D;
+        if (qp->rope_sin && !prologue_parts_serve(rd, D / 4))
+            return fail(HS_ERR_INVALID_ARGUMENT,
+                        "the prefill launch rotates head_dim, head_dim/2 or head_dim/4 leading elements of q, not %d: run "
+                        "hs_qk_prologue_apply on q as well", rd);
+        if (qp->rope_sin && (int64_t)hist_len + S > qp->rope_len)
+            return fail(HS_ERR_INVALID_ARGUMENT, "positions %d..%d exceed the rotary tables (%d rows)", hist_len,
+                        hist_len + S - 1, qp->rope_len);
+        for (const void *p : {qp->rope_sin, qp->rope_cos, qp->norm_kind != HS_QKNORM_NONE ? qp->q_norm_weight : nullptr})
+            if (((uintptr_t)p & 15) != 0)
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_q_prologue needs 16-byte aligned norm weights and rotary tables");
+        if (q == out) return fail(HS_ERR_INVALID_ARGUMENT, "prefill_q_prologue: q and out must be different buffers");
+        a.qpro.norm = norm_spec(qp, 0);
+        a.qpro.sin_t = qp->rope_sin; a.qpro.cos_t = qp->rope_cos;
+        a.qpro.rope_len = qp->rope_len; a.qpro.rd = rd;
+        a.qpro.on = 1;
+    }
     a.HG = G >= 3 ? 4 : G;  // query heads per workgroup; a group size that is not 1, 2 or 4k pads its last group
     a.scale_log2e = softmax_scale * kPLog2e;
     int q_per_wg = 16 * ((D == 256 ? 1 : 2) * kPWaves / a.HG);  // PShape<D>::kNB column blocks per wavefront
@@ -903,7 +945,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     // 32: head_dim 128 at full width without a window on 32x32x16 MFMA tiles (prefill_attn_wide.hip).  Measured slower
     // than the 16x16x32 instance at 4 x 4096 tokens in 512-token chunks (0.77 against 0.65 ms), so the library never
     // picks it by itself; elsewhere 32 is the same as 256.
-    const bool wide32 = D == 128 && !narrow && a.window == 0 && hint == 32;
+    const bool wide32 = D == 128 && !narrow && a.window == 0 && hint == 32 && !a.qpro.on;  // (its Q layout has no prologue)
     // 16: the same 256 columns per workgroup on sixteen wavefronts of one 16-column block each (four per SIMD, at most
     // 128 registers), head_dim 128 without a window; elsewhere the same as 256.
     const bool waves16 = D == 128 && !narrow && a.window == 0 && hint == 16;

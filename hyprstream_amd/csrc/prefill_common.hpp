@@ -5,6 +5,7 @@
 #include <type_traits>
 
 #include "mfma_common.hpp"
+#include "prologue_rows.hpp"
 #include "quant_device.hpp"
 
 namespace hs {
@@ -28,7 +29,9 @@ struct PrefillArgs {
     int32_t write_new;    // quantize-on-write of the call's K/V rows by the workgroups that finish early
     int32_t window;       // sliding window of local layers: a query at position p attends keys in (p - window, p]; 0 = none
     float scale_log2e;
+    RowPrologue qpro;     // the q side of the layer's prologue run inside the launch (hs_kv_layout.prefill_q_prologue)
 };
+
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
 // load, i.e. for the tile prefetch that was issued a moment earlier and is not needed before the next step.

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define HS_ATTN_ABI_VERSION 5
+#define HS_ATTN_ABI_VERSION 6
 
 typedef void *hs_stream_t; /* hipStream_t */
 
@@ -67,6 +67,8 @@ enum hs_status {
 };
 
 enum hs_dtype { HS_BF16 = 0, HS_F32 = 1, HS_F16 = 2 };
+
+struct hs_qk_prologue;
 
 typedef struct hs_kv_layout {
     int64_t code_stride_seq;    /* bytes between sequences (or blocks when paged) */
@@ -97,6 +99,14 @@ typedef struct hs_kv_layout {
                                    Qwen3.5 full-attention layers (qwen3_5.rs:1056-1059: ctx * sigmoid(gate) in the model
                                    dtype): out = bf16(bf16(attention) * bf16(sigmoid(gate))) written by the same launch.
                                    NULL = none. */
+    const struct hs_qk_prologue *prefill_q_prologue;
+                                /* prefill only, optional: q arrives AS PROJECTED and the launch runs the q side of the
+                                   prologue below on it (QK-norm with q_norm_weight, then the rotary embedding at
+                                   position hist_len + s), the bits hs_qk_prologue_apply writes; only q: k_new must
+                                   arrive normalised and rotated (hs_qk_prologue_apply with q = NULL over the prompt's
+                                   K).  Rotated parts served: rotary_dim = head_dim, head_dim / 2 or head_dim / 4,
+                                   anything else is HS_ERR_INVALID_ARGUMENT (run the pre-pass on q as well); weights and
+                                   tables 16-byte aligned.  NULL = q arrives ready. */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */

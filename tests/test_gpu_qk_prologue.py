@@ -336,3 +336,98 @@ def test_rope_then_prefill_then_cache(D):
     want2 = oracle.prefill_attn(q_rot[:, C:], kd, vd, None, None, oracle.FMT_DENSE, np.full(B, S, np.int32), 1.0 / np.sqrt(D))
     err = np.abs(out - np.concatenate([want1, want2], 1))
     assert err.max() < TOL_MAX and err.mean() < TOL_MEAN, (err.max(), err.mean())
+
+
+@pytest.mark.parametrize("columns", [0, 128, 16])
+@pytest.mark.parametrize("kind", [hb.QKNORM_NONE, hb.QKNORM_LLAMA, hb.QKNORM_QWEN35])
+@pytest.mark.parametrize("D,rd,Hq,Hkv", [(64, 64, 8, 2), (128, 128, 8, 2), (128, 64, 6, 2), (128, 32, 4, 4),
+                                         (256, 256, 8, 1), (256, 64, 4, 2), (64, 16, 4, 1)])
+def test_prefill_with_the_q_prologue_inside_the_launch(D, rd, Hq, Hkv, kind, columns):
+    """hs_kv_layout.prefill_q_prologue: q arrives as projected, the prefill launch runs its QK-norm and rotation.
+    Outputs and cache equal, bit for bit, those of hs_qk_prologue_apply on q followed by the plain launch -- a prompt in
+    two ragged chunks (S not a multiple of the tile; the second chunk over an int8 history), per-head weights, the
+    hinted widths (16 = the sixteen-wavefront instance, head_dim 128 only)."""
+    if columns == 16 and D != 128:
+        pytest.skip("the sixteen-wavefront instance serves head_dim 128")
+    r = wl.philox(9100 + D + rd + 7 * kind + columns)
+    B, L = 2, 512
+    chunks = [(0, 150), (150, 333)]
+    T = 333
+    sin, cos = _tables(rd, 10000.0, L)
+    wq, wk = _weights(r, kind, Hq, D, True), _weights(r, kind, Hkv, D, False)
+    pro = hb.qk_prologue(kind, 1e-6, wq.to(DEV) if kind else None, wk.to(DEV) if kind else None, sin.to(DEV), cos.to(DEV), rd)
+    q, k, v = (_bf(r.standard_normal((B, T, H, D))) for H in (Hq, Hkv, Hkv))
+    fused, plain = DeviceCache(B, Hkv, T, D), DeviceCache(B, Hkv, T, D)
+    for lo, hi in chunks:
+        qc, kc_, vc_ = (t[:, lo:hi].contiguous().to(DEV) for t in (q, k, v))
+        q_fin, k_fin = torch.empty_like(qc), torch.empty_like(kc_)
+        hb.qk_prologue_apply(qc, kc_, pro, q_fin, k_fin, None, lo)
+        want = torch.full_like(qc, float("nan"))
+        hb.prefill_attn(q_fin, k_fin, vc_, plain.k_codes, plain.v_codes, plain.k_scales, plain.v_scales, plain.layout, lo,
+                        want, 1.0 / np.sqrt(D), True, columns=columns)
+        got = torch.full_like(qc, float("nan"))
+        q_before = qc.clone()
+        hb.prefill_attn(qc, k_fin, vc_, fused.k_codes, fused.v_codes, fused.k_scales, fused.v_scales, fused.layout, lo,
+                        got, 1.0 / np.sqrt(D), True, columns=columns, q_prologue=pro)
+        torch.cuda.synchronize()
+        assert torch.equal(qc, q_before)  # q is read, never written
+        assert not torch.isnan(want.float()).any()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16)), (lo, hi)
+    assert torch.equal(fused.k_codes, plain.k_codes) and torch.equal(fused.v_codes, plain.v_codes)
+    assert torch.equal(fused.k_scales, plain.k_scales) and torch.equal(fused.v_scales, plain.v_scales)
+
+
+def test_prefill_q_prologue_on_ragged_rows_and_fp8():
+    """Rows at different positions (hist_lens) rotate their q at their own positions; fp8 history."""
+    r = wl.philox(9200)
+    B, Hq, Hkv, D, Hmax, S, L = 3, 8, 2, 128, 200, 96, 512
+    hist = np.array([200, 0, 77], np.int32)
+    sin, cos = _tables(D, 10000.0, L)
+    wq = _weights(r, hb.QKNORM_LLAMA, Hq, D, False)
+    pro = hb.qk_prologue(hb.QKNORM_LLAMA, 1e-6, wq.to(DEV), wq.to(DEV), sin.to(DEV), cos.to(DEV), 0)
+    q, k, v = (_bf(r.standard_normal((B, S, H, D))).to(DEV) for H in (Hq, Hkv, Hkv))
+    hk, hv = (_bf(r.standard_normal((B, Hmax, Hkv, D))).to(DEV) for _ in range(2))
+    hl = torch.from_numpy(hist).to(DEV)
+    outs = []
+    for fused in (False, True):
+        c = DeviceCache(B, Hkv, Hmax + S, D, fp8=True)
+        hb.kv_fp8_calibrate(hk, hv, c.k_scales, c.v_scales)
+        hb.kv_quantize_fp8(hk, hv, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, None, 0)
+        o = torch.full_like(q, float("nan"))
+        if fused:
+            hb.prefill_attn(q, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, Hmax, o, 0.088, True, fp8=True,
+                            hist_lens=hl, q_prologue=pro)
+        else:
+            q_fin = torch.empty_like(q)
+            hb.qk_prologue_apply(q, None, pro, q_fin, None, hl, 0)  # positions: each row's first position
+            hb.prefill_attn(q_fin, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, Hmax, o, 0.088, True,
+                            fp8=True, hist_lens=hl)
+        torch.cuda.synchronize()
+        outs.append((o, c.k_codes.clone()))
+    assert not torch.isnan(outs[0][0].float()).any()
+    assert torch.equal(outs[0][0].view(torch.int16), outs[1][0].view(torch.int16))
+    assert torch.equal(outs[0][1], outs[1][1])
+
+
+def test_prefill_q_prologue_rejections():
+    B, S, Hq, Hkv, D = 1, 64, 4, 1, 128
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    c = DeviceCache(B, Hkv, S, D)
+    q, k, o = z(B, S, Hq, D), z(B, S, Hkv, D), z(B, S, Hq, D)
+    run = lambda pro, q_=q, o_=o, hist=0: hb.prefill_attn(q_, k, k, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout,
+                                                           hist, o_, 0.1, False, q_prologue=pro)
+    sin = z(64, 48)
+    with pytest.raises(hb.HsError) as e:  # 96 of 128 rotated: not one of the served fractions
+        run(hb.qk_prologue(hb.QKNORM_NONE, 0.0, None, None, sin, sin, 96))
+    assert e.value.code == 1 and "hs_qk_prologue_apply" in str(e.value)
+    full = z(32, 64)
+    with pytest.raises(hb.HsError) as e:  # tables shorter than the positions
+        run(hb.qk_prologue(hb.QKNORM_NONE, 0.0, None, None, full, full, 0))
+    assert e.value.code == 1 and "rotary tables" in str(e.value)
+    ok = z(64, 64)
+    with pytest.raises(hb.HsError) as e:  # the launch stages the finished q in `out`
+        run(hb.qk_prologue(hb.QKNORM_NONE, 0.0, None, None, ok, ok, 0), o_=q)
+    assert e.value.code == 1 and "different buffers" in str(e.value)
+    with pytest.raises(hb.HsError) as e:  # norm asked for, no weight
+        run(hb.qk_prologue(hb.QKNORM_LLAMA, 1e-6, None, None, ok, ok, 0))
+    assert e.value.code == 1
