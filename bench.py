@@ -166,6 +166,8 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         vs = torch.zeros_like(ks)
     outs = [torch.empty(B, C, Hq, D, dtype=torch.bfloat16, device=dev) for _ in chunks]
     scale = 1.0 / float(np.sqrt(D))
+    # scratch for the key split of calls with few query tiles (the library decides per call; --key-splits 1 = never)
+    split_ws = hb.prefill_split_workspace(B, C, Hq, Hkv, D)
     if prologue:
         inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
         ang = torch.arange(T, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
@@ -202,7 +204,8 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
                         hb.qk_prologue_apply(chunks[i][0], chunks[i][1], pro, qc, kcn, None, i * C)
                 else:
                     fused = pro
-            hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8, q_prologue=fused)
+            hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8, q_prologue=fused,
+                            split_workspace=split_ws, key_splits=args.key_splits)
 
     settle(torch, lambda i: step(), window=10, min_launches=100, max_launches=1000)
     for _ in range(args.warmup):
@@ -428,6 +431,8 @@ def main():
     ap.add_argument("--cap-pad", type=int, default=0, help="decode workloads: cache capacity = context length + this many tokens")
     ap.add_argument("--prefill-columns", type=int, default=0, choices=[0, 16, 32, 128, 256],
                     help="prefill workloads: fix the (query, head) columns a workgroup owns (0 = the library's choice)")
+    ap.add_argument("--key-splits", type=int, default=0,
+                    help="prefill workloads: runs the keys of a query tile are cut into (0 = the library decides, 1 = never)")
     ap.add_argument("--prologue-fused-q", action="store_true",
                     help="c3-prologue: only k goes through the pre-pass, the chunk launches normalise and rotate q themselves")
     ap.add_argument("--prologue-per-chunk", action="store_true",

@@ -65,6 +65,11 @@ pub fn contiguous_layout(hkv: i32, capacity_tokens: i32, d: i32) -> hs_kv_layout
         prefill_columns_hint: 0,
         prefill_window: 0,
         out_gate: std::ptr::null(),
+        prefill_q_prologue: std::ptr::null(),
+        prefill_split_workspace: std::ptr::null_mut(),
+        prefill_split_workspace_bytes: 0,
+        prefill_key_splits: 0,
+        reserved0: 0,
     }
 }
 

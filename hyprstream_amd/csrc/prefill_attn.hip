@@ -78,9 +78,15 @@ template <int D> struct alignas(16) HistTile {
 // tokens, so they are compiled in only where a window is asked for).
 // kWaves: 8, or 16 wavefronts of one 16-column block each (kCols = 1, head_dim 128): the same 256 columns per workgroup
 // on four wavefronts per SIMD with at most 128 registers; wavefronts 0-7 then convert K, wavefronts 8-15 V.
-template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8>
+// kSplit: the 64-key steps of a query tile (history, then the call's own tokens) are cut into a.nsplit equal runs, one
+// workgroup each (blockIdx.x = tile * nsplit + part).  Every part writes its unnormalised accumulators, softmax
+// reference and row sums to the workspace and counts itself in at the tile's counter; the part that finds all others
+// already there adds their partials to its registers, normalises and stores.  Nobody waits for anybody.  For calls
+// whose tiles are too few to occupy the CUs (a chunk of one sequence).
+template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8, bool kSplit = false>
 __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_attn_kernel(PrefillArgs a) {
     static_assert(kWaves == 8 || (kWaves == 16 && kCols == 1 && kPD == 128), "sixteen wavefronts: one column block each, head_dim 128");
+    static_assert(!kSplit || (!kWin && kWaves == 8), "key split: eight wavefronts, no window");
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
     constexpr int DW = PShape<kPD>::DW, VBG = PShape<kPD>::VBG;
     constexpr int kRow = kPD;  // elements per row of q, k, v, out and of the cache
@@ -109,6 +115,11 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
             bz = grp / gridDim.y;
         }
     }
+    int part = 0;
+    if constexpr (kSplit) {
+        part = bx % a.nsplit;
+        bx /= a.nsplit;
+    }
     const int b = bz;
     const int groups = (a.G + a.HG - 1) / a.HG;  // the last group of a kv-head may be partly padding (G = 3, 5, 6, 7 ...)
     const int kvh = by / groups, hg = by % groups;
@@ -117,6 +128,16 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     const int q0 = bx * q_per_wg;
     if (q0 >= S) return;
     const int wg_qlast = min(S - 1, q0 + q_per_wg - 1);
+    // key split: this part's run of the tile's history steps [h_lo, h_hi) and new-token steps [n_lo, n_hi)
+    int h_lo = 0, h_hi = 0, n_lo = 0, n_hi = 0;
+    if constexpr (kSplit) {
+        const int hn = (H + 63) / 64, total = hn + wg_qlast / 64 + 1;
+        const int g0 = total * part / a.nsplit, g1 = total * (part + 1) / a.nsplit;
+        h_lo = min(g0, hn);
+        h_hi = min(g1, hn);
+        n_lo = max(g0 - hn, 0);
+        n_hi = max(g1 - hn, 0);
+    }
 
     int head[kNB], qi[kNB];
 #pragma unroll
@@ -206,7 +227,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     float vup = 1.0f;  // 2^E of the history's V operands, folded back into the accumulators when the history ends
 
     // =============================== history: int8 cache, f16 MFMA ===============================
-    if (H > 0) {
+    if (H > 0 && (!kSplit || h_lo < h_hi)) {
         // The history operands are fp16(code * scale), and fp16 spans 2^-14 .. 65504 only.  Each (sequence, kv-head)
         // therefore gets a power-of-two reference for K and one for V, taken from the largest scale among its first
         // cached tokens (int8; up to 64 of them, inside one block) or from its head scale (fp8): operands are
@@ -283,8 +304,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         // once per step whatever its size -- barrier, loop and address bookkeeping, the overflow check, waits --
         // is shared by twice as many MFMAs as in a 32-key step.
         constexpr int kHStep = 64;
-        const int nsteps = (H + kHStep - 1) / kHStep;
-        const int st0 = kWin ? min(max(H + wg_lo, 0) / kHStep, nsteps) : 0;  // first step that holds a key some query of the workgroup sees
+        const int nsteps = kSplit ? h_hi : (H + kHStep - 1) / kHStep;
+        const int st0 = kSplit ? h_lo : kWin ? min(max(H + wg_lo, 0) / kHStep, nsteps) : 0;  // first step that holds a key some query of the workgroup sees
         HistTile *htiles = (HistTile *)lds;
         // ---- producers: every wavefront converts one eighth of the step's K tiles and of its V tiles.
         //      K: wavefront w takes 16-key block u4 = w/2 and the d-halves jp = w%2 of every 32-d group: lane
@@ -595,7 +616,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     }
 
     // =============================== new tokens: bf16, causal ===============================
-    {
+    if (!kSplit || n_lo < n_hi) {
         // Q operands carry the softmax scale and log2(e), rounded back to bf16 (2^-9 relative, the precision the
         // weights are rounded to anyway), so that the MFMA result needs no multiplication; as in the history
         // phase the score accumulators start from -sref and the common step only checks for an overflow.
@@ -621,8 +642,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         }
         // 64 keys per step, as two 32-key tiles in the layout of the history phase.
         constexpr int kNStep = 64;
-        const int nsteps = wg_qlast / kNStep + 1;
-        const int st0 = kWin ? max(wg_lo, 0) / kNStep : 0;  // first step with a key inside the window of the workgroup's first query
+        const int nsteps = kSplit ? n_hi : wg_qlast / kNStep + 1;
+        const int st0 = kSplit ? n_lo : kWin ? max(wg_lo, 0) / kNStep : 0;  // first step with a key inside the window of the workgroup's first query
         HistTile *ntiles = (HistTile *)lds;
         const uint16_t *knb = a.kn + ((int64_t)b * S * a.Hkv + kvh) * kRow;
         const uint16_t *vnb = a.vn + ((int64_t)b * S * a.Hkv + kvh) * kRow;
@@ -824,6 +845,73 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         }
     }
 
+    // =============================== key split: hand over or merge ===============================
+    if constexpr (kSplit) {
+        static_assert(kNB <= 2, "softmax reference and row sum of a thread's columns in one 16-byte slot");
+        constexpr int kThreads = 64 * kWaves, kSlots = kNB * VB + 1;  // 16-byte slots per thread
+        const int tiles_x = gridDim.x / a.nsplit;
+        const int tile_id = (bz * gridDim.y + by) * tiles_x + bx;
+        const auto word = [&](int prt, int i) {  // word i of this thread's record in run prt: a wavefront's 256 bytes are contiguous
+            return a.split_ws + (((int64_t)tile_id * a.nsplit + prt) * (4 * kSlots) + i) * kThreads + threadIdx.x;
+        };
+        // The partials travel between workgroups that may sit on different XCDs, whose L2s do not see each other's
+        // lines.  They are written and read with device-scope accesses (relaxed atomics: written through to, and read
+        // from, the memory side), a few hundred per thread; the alternative -- ordinary accesses between a device-scope
+        // release and acquire fence -- writes back and invalidates whole L2s once per workgroup and measured 24 us per
+        // launch at four runs per tile (15 us per run with a fence in every thread).
+        const auto put = [](float *p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+        const auto get = [](const float *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+#pragma unroll
+        for (int nb = 0; nb < kNB; ++nb)
+#pragma unroll
+            for (int i = 0; i < VB; ++i)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) put(word(part, 4 * (nb * VB + i) + c), acc[nb][i][c]);
+#pragma unroll
+        for (int nb = 0; nb < kNB; ++nb) {
+            put(word(part, 4 * kNB * VB + 2 * nb), m_run[nb]);
+            put(word(part, 4 * kNB * VB + 2 * nb + 1), l_run[nb][0]);
+        }
+        if (a.write_new && hg == 0 && part == 0) write_new_rows<kRow, FP8, kWaves>(a, b, kvh, H, q0, q_per_wg, wave, lane);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this thread's partial has reached the memory side
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            const uint32_t before = atomicAdd(a.split_cnt + tile_id, 1u);  // device scope
+            const bool last_in = before == (uint32_t)a.nsplit - 1;
+            if (last_in) __hip_atomic_store(a.split_cnt + tile_id, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+            *(volatile int *)lds = last_in;
+        }
+        __syncthreads();
+        if (*(volatile int *)lds == 0) return;
+        // The runs are added in their order, this one's own read back like the others, so that the result does not
+        // depend on which workgroup happened to finish last.
+#pragma unroll
+        for (int nb = 0; nb < kNB; ++nb) {
+            m_run[nb] = -INFINITY;
+            l_run[nb] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < VB; ++i) acc[nb][i] = (float4v){0.f, 0.f, 0.f, 0.f};
+        }
+        for (int prt = 0; prt < a.nsplit; ++prt) {
+#pragma unroll
+            for (int nb = 0; nb < kNB; ++nb) {
+                const float mo = get(word(prt, 4 * kNB * VB + 2 * nb)), lo = get(word(prt, 4 * kNB * VB + 2 * nb + 1));
+                float4v other[VB];
+#pragma unroll
+                for (int i = 0; i < VB; ++i)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) other[i][c] = get(word(prt, 4 * (nb * VB + i) + c));
+                const float m_new = fmaxf(m_run[nb], mo);
+                const float mine = m_run[nb] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m_run[nb] - m_new);
+                const float theirs = mo == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(mo - m_new);
+                l_run[nb] = l_run[nb] * mine + lo * theirs;
+#pragma unroll
+                for (int i = 0; i < VB; ++i) acc[nb][i] = acc[nb][i] * mine + other[i] * theirs;
+                m_run[nb] = m_new;
+            }
+        }
+    }
+
     // =============================== normalise and store ===============================
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
@@ -855,13 +943,24 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
             }
     }
 
-    if (a.write_new && hg == 0) write_new_rows<kRow, FP8, kWaves>(a, b, kvh, H, q0, q_per_wg, wave, lane);
+    if (!kSplit && a.write_new && hg == 0) write_new_rows<kRow, FP8, kWaves>(a, b, kvh, H, q0, q_per_wg, wave, lane);
 }
 
 int validate_layout(const hs_kv_layout *l, int B, int S, int Hkv, int D, bool need_scales);
 int check_prologue(const hs_qk_prologue *p, int dtype, int D, bool need_q, bool need_k);
 NormSpec norm_spec(const hs_qk_prologue *p, int which);
 void launch_prefill_wide(bool fp8, const PrefillArgs &a, dim3 grid, hipStream_t st);  // prefill_attn_wide.hip
+
+// Key split of small calls: at most this many runs per query tile; per (tile, run) a workgroup's 512 threads store
+// their accumulators (64 registers at every head_dim) and one slot of softmax state, 16 bytes each.
+constexpr int kMaxKeySplits = 8;
+static size_t split_tile_bytes(int D, bool narrow) { return (size_t)512 * 16 * ((D == 64 ? 8 : 16) / (narrow ? 2 : 1) + 1); }
+static size_t split_counter_bytes(int64_t tiles) { return ((size_t)tiles * 4 + 255) / 256 * 256; }
+
+__global__ void zero_words_kernel(uint32_t *p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
 
 // CUs of the current device (looked up once per device; 256 if the query fails).
 static int compute_units() {
@@ -949,10 +1048,47 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     // 16: the same 256 columns per workgroup on sixteen wavefronts of one 16-column block each (four per SIMD, at most
     // 128 registers), head_dim 128 without a window; elsewhere the same as 256.
     const bool waves16 = D == 128 && !narrow && a.window == 0 && hint == 16;
+    // Key split: every query tile cut into runs of 64-key steps for several workgroups, when the tiles alone would leave
+    // most CUs idle and every run still has a few steps to amortise the merge (the caller gives scratch).  Half-width
+    // tiles in two runs move half the partial bytes of full-width tiles in four and merge them on twice the CUs.
+    if (layout->prefill_split_workspace != nullptr && layout->prefill_key_splits != 1 && a.window == 0 &&
+        (hint == 0 || hint == 256 || hint == 128)) {
+        int64_t tiles = (int64_t)grid.x * grid.y * grid.z;  // full width
+        const int max_steps = (hist_len + 63) / 64 + (S + 63) / 64;
+        const bool can_narrow = D <= 128 && q_per_wg >= 32;
+        int P = layout->prefill_key_splits;
+        bool split_narrow = can_narrow && hint == 128;
+        if (P == 0) {
+            P = (int)std::min<int64_t>(kMaxKeySplits, compute_units() / tiles);
+            P = std::min(P, max_steps / 4);  // at least four steps to a run
+            if (P < 3) P = 1;                // two runs of full-width tiles: the half-width workgroups do as well without a merge
+            if (P >= 4 && can_narrow && hint == 0) {
+                split_narrow = true;
+                P /= 2;
+            }
+        }
+        if (P < 1 || P > kMaxKeySplits)
+            return fail(HS_ERR_INVALID_ARGUMENT, "prefill_key_splits %d not in [0, %d]", P, kMaxKeySplits);
+        if (P > 1) {
+            if (split_narrow) tiles = (int64_t)((S + q_per_wg / 2 - 1) / (q_per_wg / 2)) * grid.y * grid.z;
+            const size_t cnt_bytes = split_counter_bytes(tiles);
+            const size_t need = cnt_bytes + (size_t)tiles * P * split_tile_bytes(D, split_narrow);
+            if (layout->prefill_split_workspace_bytes < 0 || (size_t)layout->prefill_split_workspace_bytes < need)
+                return fail(HS_ERR_WORKSPACE, "prefill split workspace of %lld bytes, %zu needed",
+                            (long long)layout->prefill_split_workspace_bytes, need);
+            if (((uintptr_t)layout->prefill_split_workspace & 255) != 0)
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill split workspace must be 256-byte aligned");
+            a.nsplit = P;
+            a.split_cnt = (uint32_t *)layout->prefill_split_workspace;
+            a.split_ws = (float *)((uint8_t *)layout->prefill_split_workspace + cnt_bytes);
+            narrow = split_narrow;
+        }
+    }
     if (narrow) {
         q_per_wg /= 2;
         grid.x = (S + q_per_wg - 1) / q_per_wg;
     }
+    grid.x *= a.nsplit;
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
@@ -975,7 +1111,19 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
             else prefill_attn_kernel<256, false, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
         }                                                                                                   \
     } while (0)
-    if (waves16) {
+    if (a.nsplit > 1) {
+#define HS_PREFILL_SPLIT(DD, CC)                                                                     \
+    do {                                                                                             \
+        if (fp8) prefill_attn_kernel<DD, true, CC, false, 8, true><<<grid, 512, 0, st>>>(a);         \
+        else prefill_attn_kernel<DD, false, CC, false, 8, true><<<grid, 512, 0, st>>>(a);            \
+    } while (0)
+        if (D == 64 && narrow) HS_PREFILL_SPLIT(64, 1);
+        else if (D == 64) HS_PREFILL_SPLIT(64, 0);
+        else if (D == 128 && narrow) HS_PREFILL_SPLIT(128, 1);
+        else if (D == 128) HS_PREFILL_SPLIT(128, 0);
+        else HS_PREFILL_SPLIT(256, 0);
+#undef HS_PREFILL_SPLIT
+    } else if (waves16) {
         if (fp8) prefill_attn_kernel<128, true, 1, false, 16><<<grid, 1024, 0, st>>>(a);
         else prefill_attn_kernel<128, false, 1, false, 16><<<grid, 1024, 0, st>>>(a);
     } else if (wide32) launch_prefill_wide(fp8, a, grid, st);
@@ -989,6 +1137,24 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
 }  // namespace hs
 
 extern "C" {
+
+size_t hs_prefill_attn_split_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D) {
+    if (B <= 0 || S <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || (D != 64 && D != 128 && D != 256)) return 0;
+    const int G = Hq / Hkv, HG = G >= 3 ? 4 : G;
+    const int q_per_wg = 16 * ((D == 256 ? 1 : 2) * hs::kPWaves / HG);
+    const int64_t tiles = (int64_t)((S + q_per_wg - 1) / q_per_wg) * Hkv * ((G + HG - 1) / HG) * B;
+    return hs::split_counter_bytes(tiles) + (size_t)tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, false);  // (half-width tiles: twice the counters, fewer bytes)
+}
+
+int hs_prefill_attn_split_workspace_init(void *workspace, size_t bytes, hs_stream_t stream) {
+    if (!workspace || ((uintptr_t)workspace & 255) != 0)
+        return hs::fail(HS_ERR_INVALID_ARGUMENT, "prefill split workspace must be a 256-byte aligned device buffer");
+    // the arrival counters sit in front of the partials; their number depends on the call, so all of it is cleared
+    const size_t words = bytes / 4;
+    if (words == 0) return HS_OK;
+    hs::zero_words_kernel<<<dim3((unsigned)((words + 255) / 256)), 256, 0, (hipStream_t)stream>>>((uint32_t *)workspace, words);
+    return hs::check_launch("prefill_split_workspace_init");
+}
 
 int hs_prefill_attn_int8(const void *q, const void *k_new, const void *v_new, int8_t *k_codes, int8_t *v_codes,
                          float *k_scales, float *v_scales, const hs_kv_layout *layout, int32_t hist_len, void *out,

@@ -29,6 +29,11 @@ struct PrefillArgs {
     int32_t write_new;    // quantize-on-write of the call's K/V rows by the workgroups that finish early
     int32_t window;       // sliding window of local layers: a query at position p attends keys in (p - window, p]; 0 = none
     float scale_log2e;
+    // keys of a query tile split over nsplit workgroups (prefill_attn_kernel<..., kSplit>): partial accumulators and an
+    // arrival counter per tile in the caller's workspace; the workgroup that arrives last merges and stores
+    int32_t nsplit = 1;
+    float *split_ws = nullptr;
+    uint32_t *split_cnt = nullptr;
     RowPrologue qpro;     // the q side of the layer's prologue run inside the launch (hs_kv_layout.prefill_q_prologue)
 };
 

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define HS_ATTN_ABI_VERSION 6
+#define HS_ATTN_ABI_VERSION 7
 
 typedef void *hs_stream_t; /* hipStream_t */
 
@@ -107,6 +107,21 @@ typedef struct hs_kv_layout {
                                    K).  Rotated parts served: rotary_dim = head_dim, head_dim / 2 or head_dim / 4,
                                    anything else is HS_ERR_INVALID_ARGUMENT (run the pre-pass on q as well); weights and
                                    tables 16-byte aligned.  NULL = q arrives ready. */
+    void *prefill_split_workspace;
+    int64_t prefill_split_workspace_bytes;
+    int32_t prefill_key_splits;
+    int32_t reserved0;          /* prefill only, optional: device scratch that lets a call whose query tiles are too few
+                                   to occupy the GPU (a chunk of ONE sequence: 64 tiles on 256 compute units) cut the
+                                   keys of every tile into runs for several workgroups, the last of which to finish
+                                   merges the partial results.  At least hs_prefill_attn_split_workspace_bytes(...)
+                                   bytes, 256-byte aligned, prepared once by hs_prefill_attn_split_workspace_init and
+                                   left ready by every call; calls that overlap in time need workspaces of their own.
+                                   NULL = never split.  prefill_key_splits: 0 = the library decides whether and how
+                                   far to split, 1 = never, 2..8 = this many runs (tests, measurements).  A workspace
+                                   that is too small for the call is HS_ERR_WORKSPACE.  Outputs agree with the unsplit
+                                   launch within the rounding of a different summation order; the cache rows written
+                                   are the same bits.  Not combined with a window or a width hint of 128, 32 or 16
+                                   (those calls run unsplit). */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */
@@ -363,6 +378,13 @@ HS_API int hs_prefill_attn_fp8_ragged(const void *q, const void *k_new, const vo
                                const hs_kv_layout *layout, const int32_t *hist_lens, int32_t max_hist_len,
                                void *out, int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
                                float softmax_scale, int quantize_on_write, hs_stream_t stream);
+
+/* Scratch for the key split of small prefill calls (hs_kv_layout.prefill_split_workspace): bytes needed for calls of
+ * at most B x S new tokens, whatever their history; _init zeroes the arrival counters (a small fill launch on
+ * `stream`) and is needed once per allocation.  No counterpart in the reference, whose attention is one libtorch
+ * matmul per call (llama.rs:1066-1112). */
+HS_API size_t hs_prefill_attn_split_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D);
+HS_API int hs_prefill_attn_split_workspace_init(void *workspace, size_t bytes, hs_stream_t stream);
 
 /* ---- gated delta rule (replaces the decode branch qwen3_5.rs:725-751 and
  * chunked_delta_rule qwen3_5.rs:342-498) -------------------------------------------------------

@@ -13,13 +13,19 @@ from gpu_util import DEV, DeviceCache, bf16_from_bits, run_decode
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["auto", "256", "128", "32", "16"])
+@pytest.fixture(autouse=True, params=["auto", "256", "128", "32", "16", "split3", "split8", "split2x128"])
 def columns_per_workgroup(request, monkeypatch):
     """Every test runs with the library's own choice of workgroup width (half-width workgroups for small grids) and
     with each instance forced -- 256 columns on 16x16x32 MFMA tiles, 128 columns, 256 columns on 32x32x16 tiles, 256
     columns on sixteen wavefronts (the last two: head_dim 128 without a window; elsewhere the same as 256) -- so that
-    small shapes exercise every kernel."""
-    monkeypatch.setattr(hb, "PREFILL_COLUMNS", 0 if request.param == "auto" else int(request.param))
+    small shapes exercise every kernel; and with the keys of every query tile split into runs whose partial results the
+    last workgroup to finish merges: 3 and 8 runs of full-width tiles, 2 of half-width ones (runs may be empty: most
+    of these shapes have fewer steps than 8)."""
+    name = request.param
+    split = int(name[5]) if name.startswith("split") else 0
+    cols = int(name.split("x")[1]) if "x" in name else 0 if split or name == "auto" else int(name)
+    monkeypatch.setattr(hb, "PREFILL_COLUMNS", cols)
+    monkeypatch.setattr(hb, "PREFILL_KEY_SPLITS", split)
 
 TOL_MAX, TOL_MEAN = 2e-2, 2e-3
 
@@ -516,7 +522,7 @@ def test_windowed_prompt_without_history(D, Hq, Hkv, W):
     compare(got, want, "window %d D=%d" % (W, D))
     if W >= S:  # a window that covers the prompt changes nothing
         plain = gpu_prefill(DeviceCache(B, Hkv, S, D), q, k, v, 0)
-        if D == 128 and hb.PREFILL_COLUMNS == 32:
+        if (D == 128 and hb.PREFILL_COLUMNS == 32) or hb.PREFILL_KEY_SPLITS > 1:  # the unwindowed launch is another kernel
             # the unwindowed call runs on the 32x32 MFMA instance here, the windowed one never does: the same values
             # summed in another order, then rounded to bf16
             assert np.abs(got - plain).max() <= 2.0 ** -7 * max(1.0, np.abs(plain).max())
@@ -580,3 +586,59 @@ def test_negative_window_is_refused():
     with pytest.raises(hb.HsError):
         gpu_prefill_window(c, q, k, v, 0, -1)
     c.layout.prefill_window = 0
+
+
+@pytest.mark.parametrize("D,fp8", [(128, False), (128, True), (64, False), (256, False)])
+def test_key_split_the_library_picks_for_a_chunk_of_one_sequence(D, fp8):
+    """One sequence, a 512-token chunk over 1536 cached tokens (llama.rs:492-668 runs prompts one sequence at a time): 64
+    full-width query tiles on 256 compute units, so with a workspace the library cuts every tile's 24 + up to 8 steps
+    into runs.  Outputs agree with the unsplit launch within the rounding of another summation order and with the
+    oracle; the cache rows are the same bits; the workspace is left ready for the next call (second call, same
+    answer)."""
+    B, S, H, Hq, Hkv = 1, 512, 1536, (32 if D != 256 else 16), (8 if D != 256 else 4)
+    r = wl.philox(7300 + D + fp8)
+    sigma = 0.5 if fp8 else 1.0
+    q, k, v = make(7400 + D, B, S, Hq, Hkv, D, sigma)
+    hk = bf16r((sigma * r.standard_normal((B, H, Hkv, D))).astype(np.float32))
+    hv = bf16r((sigma * r.standard_normal((B, H, Hkv, D))).astype(np.float32))
+    dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
+    ws = hb.prefill_split_workspace(B, S, Hq, Hkv, D)
+    caches, outs = [], []
+    for use_ws in (None, ws, ws):
+        c = DeviceCache(B, Hkv, H + S, D, fp8=fp8)
+        if fp8:
+            hb.kv_fp8_calibrate(dev(hk), dev(hv), c.k_scales, c.v_scales)
+        c.write(dev(hk), dev(hv))
+        out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+        hb.prefill_attn(dev(q), dev(k), dev(v), c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, H, out,
+                        1.0 / np.sqrt(D), True, fp8=fp8, columns=0, split_workspace=use_ws, key_splits=0 if use_ws is not None else 1)
+        torch.cuda.synchronize()
+        caches.append(c)
+        outs.append(out.float().cpu().numpy())
+    assert np.isfinite(outs[1]).all()
+    assert np.abs(outs[1] - outs[0]).max() <= 2.0 ** -7 * max(1.0, np.abs(outs[0]).max())
+    assert np.array_equal(outs[1], outs[2])
+    for c in caches[1:]:
+        assert torch.equal(c.k_codes, caches[0].k_codes) and torch.equal(c.v_codes, caches[0].v_codes)
+        assert torch.equal(c.k_scales, caches[0].k_scales) and torch.equal(c.v_scales, caches[0].v_scales)
+    if not fp8:
+        kc, vc, ks, vs = caches[0].canonical(H)
+        want = oracle_prefill(q, oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k, v)
+        compare(outs[1], want, "key split D=%d" % D)
+
+
+def test_key_split_workspace_errors():
+    B, S, Hq, Hkv, D = 1, 128, 8, 2, 128
+    q, k, v = (torch.zeros(B, S, H, D, dtype=torch.bfloat16, device=DEV) for H in (Hq, Hkv, Hkv))
+    c = DeviceCache(B, Hkv, S, D)
+    out = torch.empty_like(q)
+    small = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    with pytest.raises(hb.HsError) as e:
+        hb.prefill_attn(q, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, 0, out, 0.1, False,
+                        columns=0, split_workspace=small, key_splits=4)
+    assert e.value.code == hb.HS_ERR_WORKSPACE
+    ws = hb.prefill_split_workspace(B, S, Hq, Hkv, D)
+    with pytest.raises(hb.HsError) as e:
+        hb.prefill_attn(q, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, 0, out, 0.1, False,
+                        columns=0, split_workspace=ws, key_splits=9)
+    assert e.value.code == 1

@@ -338,7 +338,7 @@ def test_rope_then_prefill_then_cache(D):
     assert err.max() < TOL_MAX and err.mean() < TOL_MEAN, (err.max(), err.mean())
 
 
-@pytest.mark.parametrize("columns", [0, 128, 16])
+@pytest.mark.parametrize("columns", [0, 128, 16, "split3"])
 @pytest.mark.parametrize("kind", [hb.QKNORM_NONE, hb.QKNORM_LLAMA, hb.QKNORM_QWEN35])
 @pytest.mark.parametrize("D,rd,Hq,Hkv", [(64, 64, 8, 2), (128, 128, 8, 2), (128, 64, 6, 2), (128, 32, 4, 4),
                                          (256, 256, 8, 1), (256, 64, 4, 2), (64, 16, 4, 1)])
@@ -346,10 +346,13 @@ def test_prefill_with_the_q_prologue_inside_the_launch(D, rd, Hq, Hkv, kind, col
     """hs_kv_layout.prefill_q_prologue: q arrives as projected, the prefill launch runs its QK-norm and rotation.
     Outputs and cache equal, bit for bit, those of hs_qk_prologue_apply on q followed by the plain launch -- a prompt in
     two ragged chunks (S not a multiple of the tile; the second chunk over an int8 history), per-head weights, the
-    hinted widths (16 = the sixteen-wavefront instance, head_dim 128 only)."""
+    hinted widths (16 = the sixteen-wavefront instance, head_dim 128 only), and with every query tile's keys split into
+    three runs (all of which stage the same finished q rows in `out`)."""
     if columns == 16 and D != 128:
         pytest.skip("the sixteen-wavefront instance serves head_dim 128")
-    r = wl.philox(9100 + D + rd + 7 * kind + columns)
+    splits = 3 if columns == "split3" else 0
+    columns = 0 if splits else columns
+    r = wl.philox(9100 + D + rd + 7 * kind + columns + splits)
     B, L = 2, 512
     chunks = [(0, 150), (150, 333)]
     T = 333
@@ -358,17 +361,20 @@ def test_prefill_with_the_q_prologue_inside_the_launch(D, rd, Hq, Hkv, kind, col
     pro = hb.qk_prologue(kind, 1e-6, wq.to(DEV) if kind else None, wk.to(DEV) if kind else None, sin.to(DEV), cos.to(DEV), rd)
     q, k, v = (_bf(r.standard_normal((B, T, H, D))) for H in (Hq, Hkv, Hkv))
     fused, plain = DeviceCache(B, Hkv, T, D), DeviceCache(B, Hkv, T, D)
+    extra = {}
     for lo, hi in chunks:
+        if splits:
+            extra = dict(split_workspace=hb.prefill_split_workspace(B, hi - lo, Hq, Hkv, D), key_splits=splits)
         qc, kc_, vc_ = (t[:, lo:hi].contiguous().to(DEV) for t in (q, k, v))
         q_fin, k_fin = torch.empty_like(qc), torch.empty_like(kc_)
         hb.qk_prologue_apply(qc, kc_, pro, q_fin, k_fin, None, lo)
         want = torch.full_like(qc, float("nan"))
         hb.prefill_attn(q_fin, k_fin, vc_, plain.k_codes, plain.v_codes, plain.k_scales, plain.v_scales, plain.layout, lo,
-                        want, 1.0 / np.sqrt(D), True, columns=columns)
+                        want, 1.0 / np.sqrt(D), True, columns=columns, **extra)
         got = torch.full_like(qc, float("nan"))
         q_before = qc.clone()
         hb.prefill_attn(qc, k_fin, vc_, fused.k_codes, fused.v_codes, fused.k_scales, fused.v_scales, fused.layout, lo,
-                        got, 1.0 / np.sqrt(D), True, columns=columns, q_prologue=pro)
+                        got, 1.0 / np.sqrt(D), True, columns=columns, q_prologue=pro, **extra)
         torch.cuda.synchronize()
         assert torch.equal(qc, q_before)  # q is read, never written
         assert not torch.isnan(want.float()).any()
