@@ -318,7 +318,9 @@ __global__ __launch_bounds__(512, 8) void deltanet_chunk_factor_kernel(WalkArgs 
 // ---------------------------------------------------------------------------------------------------- walk
 
 // One chunk's operands in LDS; A operand blocks are 64 lanes x 16 B.
-constexpr int kPitchT = 72;  // halves per row of the transposed k tile [dk][token]
+constexpr int kPitchT = 68;  // halves per row of the transposed k tile [dk][token]: 34 words, so the 16 rows an 8-byte read of a
+                             // wavefront's quarter touches, and the rows 8 apart that its 2-byte writes touch, fall on different banks
+                             // (72 gave two-way conflicts on both)
 constexpr int oKn = 0;                        // -k e^G        [token tile 4][dk slab 4]
 constexpr int oQg = oKn + 16384;              // q e^G         [token tile 4][dk slab 4]
 constexpr int oKt = oQg + 16384;              // k e^(G63-G), transposed [dk 128][token 64], eight-token pieces permuted
@@ -331,6 +333,11 @@ constexpr int kBufBytes = oDec + 16;
 constexpr int kOutPitch = 68;  // floats per staged row: 64 columns + 4, so the four rows of a 16-byte read hit different banks
 constexpr int oOut = 2 * kBufBytes, kLdsWalk = oOut + kC * kOutPitch * 4;
 static_assert(kLdsWalk + 16 <= 163840, "two chunks of operands and one of output rows in the CU's LDS");
+
+// Permutation of the 16-byte pieces inside a (-k e^G) / (q e^G) operand block: bits 1 and 2 of the piece index are
+// flipped by the piece's row group (lq / 2) and by the parity of the block.  Readers (a lane per piece, 16 bytes) stay
+// conflict-free: eight consecutive lanes still cover an aligned 128 bytes.
+__device__ __forceinline__ int kq_swizzle(int lq, int blk) { return 2 * (lq >> 1) + 4 * (blk & 1); }
 
 // Transposed tile [feature d][token]: the eight-token (16-byte) pieces of a row are permuted by d / 16, so that the
 // threads of a wavefront, which write one token each for features 16 apart, hit different banks.
@@ -475,8 +482,10 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
                 for (int h8 = 0; h8 < 2; ++h8) {
                     // dk 64 h8 + 8 dp + e: slab 2 h8 + dp / 4; inside the slab at 8 (dp % 4) + e, i.e. the tile of
                     // the slab (slots 0-3 or 4-7) is (dp / 2) % 2 and the row groups are lq = 2 (dp % 2), + 1
+                    // The 16-byte pieces of a block are permuted: piece index (= reader lane) ^ kq_swizzle.  Unpermuted, the
+                    // 16 lanes an 8-byte write handles per cycle (two tokens x eight dp) met in four bank pairs, four deep.
                     const int blk = (tok >> 4) * 4 + 2 * h8 + (dp >> 2);
-                    const int o = blk * 1024 + (2 * (dp & 1) * 16 + (tok & 15)) * 16 + 8 * ((dp >> 1) & 1);
+                    const int o = blk * 1024 + (((2 * (dp & 1) * 16 + (tok & 15)) ^ kq_swizzle(2 * (dp & 1), blk)) * 16) + 8 * ((dp >> 1) & 1);
 #pragma unroll
                     for (int g4 = 0; g4 < 2; ++g4) {
                         half4v hn, hq;
@@ -561,6 +570,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         lds_sync();
         const uint8_t *buf = lds + (ci & 1) * kBufBytes;
         auto opA = [&](int off, int blk) { return *(const half8 *)(buf + off + blk * 1024 + lane * 16); };
+        auto opKQ = [&](int off, int blk) { return *(const half8 *)(buf + off + blk * 1024 + (lane ^ kq_swizzle(lq, blk)) * 16); };
         const _Float16 *KT = (const _Float16 *)(buf + oKt);
         auto opKt = [&](int x, int s) {  // (k e^(G63-G))^T: row dk 16 x + li, k-slots = tokens of slab s in accumulator order
             const half4v lo = *(const half4v *)&KT[tpos(16 * x + li, 32 * s + 4 * lq)];
@@ -573,7 +583,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
             va[tt] = *(const bf16x8 *)(buf + oV + (tt * kCT + (kCT * wave) / 2) * 1024 + (li * 4 + lq) * 16);
-            an[0][tt] = opA(oKn, tt * 4);
+            an[0][tt] = opKQ(oKn, tt * 4);
         }
         const float dec = *(const float *)(buf + oDec);
         __builtin_amdgcn_sched_barrier(0);
@@ -586,7 +596,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         for (int sl = 0; sl < 4; ++sl) {  // dk slab sl
             if (sl < 3) {
 #pragma unroll
-                for (int tt = 0; tt < 4; ++tt) an[(sl + 1) & 1][tt] = opA(oKn, tt * 4 + sl + 1);
+                for (int tt = 0; tt < 4; ++tt) an[(sl + 1) & 1][tt] = opKQ(oKn, tt * 4 + sl + 1);
             } else {
 #pragma unroll
                 for (int i = 0; i < 6; ++i) nt[i] = opA(oNt, i);
@@ -602,7 +612,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         }
         half8 aq[2][4];
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) aq[0][tt] = opA(oQg, tt * 4);
+        for (int tt = 0; tt < 4; ++tt) aq[0][tt] = opKQ(oQg, tt * 4);
         half8 Xh[2][kCT];
 #pragma unroll
         for (int c = 0; c < kCT; ++c) {
@@ -635,7 +645,7 @@ __global__ __launch_bounds__(kWalkThreads) void deltanet_chunk_walk_kernel(WalkA
         for (int sl = 0; sl < 4; ++sl) {
             if (sl < 3) {
 #pragma unroll
-                for (int tt = 0; tt < 4; ++tt) aq[(sl + 1) & 1][tt] = opA(oQg, tt * 4 + sl + 1);
+                for (int tt = 0; tt < 4; ++tt) aq[(sl + 1) & 1][tt] = opKQ(oQg, tt * 4 + sl + 1);
             } else {
 #pragma unroll
                 for (int i = 0; i < 6; ++i) qm[i] = opA(oQK, i);
