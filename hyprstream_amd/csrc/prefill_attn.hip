@@ -163,6 +163,16 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     // it back -- each lane exactly what it wrote.  (Measured at 4 x 512 tokens per launch, Llama-flavour norm and
     // whole-head rotation: 10 us per launch, half of it arithmetic; the same code as loops over 8-element groups, which
     // is a fifth of the instructions, took 15 us: every iteration waits for its own loads.)
+    // (Key split: several workgroups, possibly on different XCDs, share the tile's rows of `out`, and a staged row left
+    // dirty in one XCD's L2 could be written back over the final output stored from another.  The runs therefore stage
+    // their q pieces in their own record of the workspace and `out` is touched by the merging workgroup alone.)
+    constexpr int kSplitThreads = 64 * kWaves, kSplitSlots = kNB * VB + 1 + kNB * KG;  // 16-byte slots per thread and run
+    int tile_id = 0;
+    u32x4 *qstage = nullptr;
+    if constexpr (kSplit) {
+        tile_id = (bz * gridDim.y + by) * (gridDim.x / a.nsplit) + bx;
+        qstage = (u32x4 *)a.split_ws + (((int64_t)tile_id * a.nsplit + part) * kSplitSlots + kNB * VB + 1) * kSplitThreads + threadIdx.x;
+    }
     const uint16_t *qsrc = a.q;
     u32x4 qpre[kNB][KG];
     if (a.qpro.on) {
@@ -172,7 +182,10 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
             const int64_t row = (((int64_t)b * S + qrow) * a.Hq + head[nb]) * kRow;
             prologue_row_part<kPD, 8 * KG>(a.qpro, a.q + row, head[nb], H + qrow, lq, 16, lane, qpre[nb]);
 #pragma unroll
-            for (int j = 0; j < KG; ++j) *(u32x4 *)(a.out + row + 8 * KG * lq + 8 * j) = qpre[nb][j];
+            for (int j = 0; j < KG; ++j) {
+                if constexpr (kSplit) qstage[(nb * KG + j) * kSplitThreads] = qpre[nb][j];
+                else *(u32x4 *)(a.out + row + 8 * KG * lq + 8 * j) = qpre[nb][j];
+            }
         }
         qsrc = a.out;
     }
@@ -630,7 +643,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
             const uint16_t *qp = qsrc + (((int64_t)b * S + min(qi[nb], S - 1)) * a.Hq + head[nb]) * kRow + 8 * KG * lq;
 #pragma unroll
             for (int j = 0; j < KG; ++j) {
-                const u32x4 w = *(const u32x4 *)(qp + 8 * j);
+                const u32x4 w = kSplit && a.qpro.on ? qstage[(nb * KG + j) * kSplitThreads] : *(const u32x4 *)(qp + 8 * j);
                 uint32_t o[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
@@ -848,9 +861,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     // =============================== key split: hand over or merge ===============================
     if constexpr (kSplit) {
         static_assert(kNB <= 2, "softmax reference and row sum of a thread's columns in one 16-byte slot");
-        constexpr int kThreads = 64 * kWaves, kSlots = kNB * VB + 1;  // 16-byte slots per thread
-        const int tiles_x = gridDim.x / a.nsplit;
-        const int tile_id = (bz * gridDim.y + by) * tiles_x + bx;
+        constexpr int kThreads = kSplitThreads, kSlots = kSplitSlots;  // accumulators, softmax state, staged q pieces
         const auto word = [&](int prt, int i) {  // word i of this thread's record in run prt: a wavefront's 256 bytes are contiguous
             return a.split_ws + (((int64_t)tile_id * a.nsplit + prt) * (4 * kSlots) + i) * kThreads + threadIdx.x;
         };
@@ -952,9 +963,12 @@ NormSpec norm_spec(const hs_qk_prologue *p, int which);
 void launch_prefill_wide(bool fp8, const PrefillArgs &a, dim3 grid, hipStream_t st);  // prefill_attn_wide.hip
 
 // Key split of small calls: at most this many runs per query tile; per (tile, run) a workgroup's 512 threads store
-// their accumulators (64 registers at every head_dim) and one slot of softmax state, 16 bytes each.
+// their accumulators (64 registers at every head_dim), one slot of softmax state and, when the launch runs q's
+// prologue, their pieces of the finished q rows, 16 bytes each.
 constexpr int kMaxKeySplits = 8;
-static size_t split_tile_bytes(int D, bool narrow) { return (size_t)512 * 16 * ((D == 64 ? 8 : 16) / (narrow ? 2 : 1) + 1); }
+static size_t split_tile_bytes(int D, bool narrow) {  // accumulator slots + one of softmax state + the staged q pieces
+    return (size_t)512 * 16 * ((D == 64 ? 8 : 16) / (narrow ? 2 : 1) + 1 + (D == 64 ? 4 : 8) / (narrow ? 2 : 1));
+}
 static size_t split_counter_bytes(int64_t tiles) { return ((size_t)tiles * 4 + 255) / 256 * 256; }
 
 __global__ void zero_words_kernel(uint32_t *p, size_t n) {
@@ -1143,7 +1157,12 @@ size_t hs_prefill_attn_split_workspace_bytes(int32_t B, int32_t S, int32_t Hq, i
     const int G = Hq / Hkv, HG = G >= 3 ? 4 : G;
     const int q_per_wg = 16 * ((D == 256 ? 1 : 2) * hs::kPWaves / HG);
     const int64_t tiles = (int64_t)((S + q_per_wg - 1) / q_per_wg) * Hkv * ((G + HG - 1) / HG) * B;
-    return hs::split_counter_bytes(tiles) + (size_t)tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, false);  // (half-width tiles: twice the counters, fewer bytes)
+    // full-width tiles, or (head_dim <= 128) twice as many half-width ones: whichever record layout is larger
+    const size_t wide = hs::split_counter_bytes(tiles) + (size_t)tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, false);
+    const size_t half = D <= 128 && q_per_wg >= 32
+                            ? hs::split_counter_bytes(2 * tiles) + (size_t)2 * tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, true)
+                            : 0;
+    return wide > half ? wide : half;
 }
 
 int hs_prefill_attn_split_workspace_init(void *workspace, size_t bytes, hs_stream_t stream) {

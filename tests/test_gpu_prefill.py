@@ -13,14 +13,14 @@ from gpu_util import DEV, DeviceCache, bf16_from_bits, run_decode
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(autouse=True, params=["auto", "256", "128", "32", "16", "split3", "split8", "split2x128"])
+@pytest.fixture(autouse=True, params=["auto", "256", "128", "32", "16", "split8", "split2x128"])
 def columns_per_workgroup(request, monkeypatch):
     """Every test runs with the library's own choice of workgroup width (half-width workgroups for small grids) and
     with each instance forced -- 256 columns on 16x16x32 MFMA tiles, 128 columns, 256 columns on 32x32x16 tiles, 256
     columns on sixteen wavefronts (the last two: head_dim 128 without a window; elsewhere the same as 256) -- so that
     small shapes exercise every kernel; and with the keys of every query tile split into runs whose partial results the
-    last workgroup to finish merges: 3 and 8 runs of full-width tiles, 2 of half-width ones (runs may be empty: most
-    of these shapes have fewer steps than 8)."""
+    last workgroup to finish merges: 8 runs of full-width tiles, 2 of half-width ones (runs may be empty: most of these
+    shapes have fewer steps than 8)."""
     name = request.param
     split = int(name[5]) if name.startswith("split") else 0
     cols = int(name.split("x")[1]) if "x" in name else 0 if split or name == "auto" else int(name)
