@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-layer|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-prologue|c3-shadow|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-layer|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -138,13 +138,15 @@ def cpu_baseline(torch, name, caches, q, lens, Hq, fp8, seconds_budget=20.0):
     }, out
 
 
-def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, b1=False, prologue=False):
+def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, b1=False, prologue=False, shadow=False):
     """Config 3: chunked causal prefill, B=4 x 4096 tokens in 512-token chunks, Hq 32 / Hkv 8, D 128.
     One step = all eight chunk calls of one layer (attention + quantize-on-write of every chunk).
     Variants: C = 4096 (the whole prompt in one call), fp8 = an e4m3fn cache with per-head scales, d256 = the head
     shape of Qwen3.5's full-attention layers (Hq 16 / Hkv 4, D 256: the same flops and bytes), prologue = q and k arrive
     as projected and every chunk call is preceded by the QK-norm + rotary pre-pass (hs_qk_prologue_apply, Llama-flavour
-    norm, whole-head rotation); the pre-pass is inside the timed step, the roofline figure stays the attention kernel's."""
+    norm, whole-head rotation); the pre-pass is inside the timed step, the roofline figure stays the attention kernel's;
+    shadow = the calls also keep a bf16 operand-order copy of the prompt's dequantized K/V (hs_kv_layout.prefill_shadow,
+    2 x the int8 bytes, for the duration of the prompt) and read the history from it instead of converting codes."""
     dev = "cuda:0"
     B, T, Hq, Hkv, D = (4, 4096, 16, 4, 256) if d256 else (4, 4096, 32, 8, 64) if d64 else (1 if b1 else 4, 4096, 32, 8, 128)
     gen = torch.Generator(device=dev)
@@ -168,6 +170,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
     scale = 1.0 / float(np.sqrt(D))
     # scratch for the key split of calls with few query tiles (the library decides per call; --key-splits 1 = never)
     split_ws = hb.prefill_split_workspace(B, C, Hq, Hkv, D)
+    shadow_buf = hb.prefill_shadow(B, Hkv, D, T) if shadow else None
     if prologue:
         inv = 1.0 / (10000.0 ** (torch.arange(0, D, 2, device=dev, dtype=torch.float32) / D))
         ang = torch.arange(T, device=dev, dtype=torch.float32)[:, None] * inv[None, :]
@@ -205,7 +208,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
                 else:
                     fused = pro
             hb.prefill_attn(qc, kcn, vcn, kc, vc, ks, vs, lay, i * C, outs[i], scale, write, fp8=fp8, q_prologue=fused,
-                            split_workspace=split_ws, key_splits=args.key_splits)
+                            split_workspace=split_ws, key_splits=args.key_splits, shadow=shadow_buf)
 
     settle(torch, lambda i: step(), window=10, min_launches=100, max_launches=1000)
     for _ in range(args.warmup):
@@ -223,7 +226,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
     e1 = [torch.cuda.Event(enable_timing=True) for _ in range(n_ev)]
     for i in range(n_ev):
         e0[i].record()
-        step(write=False, with_prologue=False)
+        step(write=shadow, with_prologue=False)  # (the copy is appended by the cache write: with it the write stays in)
         e1[i].record()
     torch.cuda.synchronize()
     kms = float(np.mean([a.elapsed_time(b) for a, b in zip(e0, e1)]))
@@ -236,7 +239,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         "data": "synthetic (seeded, generated on device)",
         "config": {"workload": "c3%s: chunked causal prefill B=%d T=4096 chunk=%d Hq=%d Hkv=%d D=%d, %s cache of earlier "
                                "chunks + own bf16 K/V, quantize-on-write, one layer"
-                               % ("-prologue" if prologue else "-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
+                               % ("-shadow" if shadow else "-prologue" if prologue else "-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
                                   "fp8 e4m3fn" if fp8 else "int8"),
                    "algorithmic_flops_per_step": int(flops)},
         "tokens_per_s": B * T / (ms * 1e-3),
@@ -424,7 +427,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-layer", "c5-prefill-recurrent"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-prologue", "c3-shadow", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-layer", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
@@ -470,7 +473,7 @@ def main():
         return
     if args.workload.startswith("c3"):
         return bench_prefill(args, torch, hb, wl, C=args.chunk_tokens or (4096 if args.workload == "c3-prompt" else 512),
-                             fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload == "c3-b1", prologue=args.workload == "c3-prologue")
+                             fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload == "c3-b1", prologue=args.workload == "c3-prologue", shadow=args.workload == "c3-shadow")
     if args.workload.startswith("c5-decode-layer"):
         return bench_deltanet_layer(args, torch, hb, wl, fused=args.workload == "c5-decode-layer")
     if args.workload.startswith("c5"):

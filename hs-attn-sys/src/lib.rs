@@ -70,6 +70,10 @@ pub fn contiguous_layout(hkv: i32, capacity_tokens: i32, d: i32) -> hs_kv_layout
         prefill_split_workspace_bytes: 0,
         prefill_key_splits: 0,
         reserved0: 0,
+        prefill_shadow: std::ptr::null_mut(),
+        prefill_shadow_bytes: 0,
+        prefill_shadow_tokens: 0,
+        reserved1: 0,
     }
 }
 

@@ -28,7 +28,7 @@ EXPORTS = [
     "hs_kv_quantize_int8_rope", "hs_rope_apply", "hs_rope_apply_partial", "hs_decode_step_int8_rope", "hs_decode_attn_num_chunks",
     "hs_decode_attn_int8_static", "hs_qk_prologue_apply", "hs_kv_quantize_int8_prologue", "hs_decode_step_int8_prologue", "hs_decode_step_fp8_prologue",
     "hs_deltanet_prepare", "hs_deltanet_gated_norm", "hs_deltanet_decode_layer", "hs_deltanet_forward_chunked", "hs_deltanet_forward_chunked_gated_norm", "hs_deltanet_prefill_layer", "hs_deltanet_prefill_layer_workspace_bytes", "hs_prefill_attn_int8_ragged", "hs_prefill_attn_fp8_ragged", "hs_deltanet_chunked_workspace_bytes",
-    "hs_deltanet_chunked_gated_norm_workspace_bytes", "hs_prefill_attn_split_workspace_bytes", "hs_prefill_attn_split_workspace_init",
+    "hs_deltanet_chunked_gated_norm_workspace_bytes", "hs_prefill_attn_split_workspace_bytes", "hs_prefill_attn_split_workspace_init", "hs_prefill_shadow_bytes", "hs_prefill_shadow_init",
 ]
 
 
@@ -52,6 +52,10 @@ class KvLayout(ctypes.Structure):
         ("prefill_split_workspace_bytes", ctypes.c_int64),
         ("prefill_key_splits", ctypes.c_int32),
         ("reserved0", ctypes.c_int32),
+        ("prefill_shadow", ctypes.c_void_p),
+        ("prefill_shadow_bytes", ctypes.c_int64),
+        ("prefill_shadow_tokens", ctypes.c_int32),
+        ("reserved1", ctypes.c_int32),
     ]
 
 
@@ -112,6 +116,8 @@ def lib():
         L.hs_attn_last_error.restype = ctypes.c_char_p
         L.hs_decode_attn_workspace_bytes.restype = ctypes.c_size_t
         L.hs_decode_attn_workspace_bytes.argtypes = [ctypes.c_int32] * 5
+        L.hs_prefill_shadow_bytes.restype = ctypes.c_size_t
+        L.hs_prefill_shadow_bytes.argtypes = [ctypes.c_int32] * 4
         L.hs_prefill_attn_split_workspace_bytes.restype = ctypes.c_size_t
         L.hs_prefill_attn_split_workspace_bytes.argtypes = [ctypes.c_int32] * 5
         _lib = L
@@ -304,6 +310,16 @@ def prefill_split_workspace(B, S, Hq, Hkv, D, device="cuda:0"):
     return ws
 
 
+def prefill_shadow(B, Hkv, D, max_tokens, device="cuda:0"):
+    """(buffer, tokens) for prefill_attn's `shadow`: the cleared bf16 copy for prompts of at most max_tokens tokens."""
+    import torch
+    tokens = (max_tokens + 63) // 64 * 64
+    n = lib().hs_prefill_shadow_bytes(B, Hkv, D, tokens)
+    buf = torch.empty(n, dtype=torch.uint8, device=device)
+    check(lib().hs_prefill_shadow_init(_ptr(buf), ctypes.c_size_t(n), _stream()))
+    return buf, tokens
+
+
 PREFILL_KEY_SPLITS = 0  # tests: force this many key runs per query tile on every prefill_attn call (with a scratch of their own)
 _split_scratch = {}
 
@@ -313,7 +329,7 @@ PREFILL_COLUMNS = 0  # default for prefill_attn's `columns` (tests set it to run
 
 def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, hist_len, out, softmax_scale,
                  quantize_on_write=True, fp8=False, hist_lens=None, columns=None, window=0, q_prologue=None,
-                 split_workspace=None, key_splits=0):
+                 split_workspace=None, key_splits=0, shadow=None):
     """Causal attention of S new tokens over [int8 or fp8 history | their own bf16 K/V]; optionally caches them.
     hist_lens (int32 device tensor [B]): rows at different positions; hist_len is then their upper bound.
     columns: 0 = the library's choice of workgroup width, 256 or 128 fixes it (layout.prefill_columns_hint).
@@ -321,7 +337,9 @@ def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, 
     q_prologue (QkPrologue): q arrives as projected and the launch normalises and rotates it
     (layout.prefill_q_prologue); k_new arrives normalised and rotated either way.
     split_workspace (uint8 device tensor from prefill_split_workspace()): lets a call with few query tiles split their
-    keys over several workgroups; key_splits 0 = the library decides, 1 = never, 2..8 = forced."""
+    keys over several workgroups; key_splits 0 = the library decides, 1 = never, 2..8 = forced.
+    shadow ((uint8 device tensor, tokens) from prefill_shadow()): the bf16 operand-order copy of the prompt's K/V that
+    every call appends to and calls with history read instead of the codes (layout.prefill_shadow)."""
     B, S, Hq, D = q.shape
     layout.prefill_columns_hint = PREFILL_COLUMNS if columns is None else columns
     layout.prefill_window = window
@@ -334,6 +352,9 @@ def prefill_attn(q, k_new, v_new, k_codes, v_codes, k_scales, v_scales, layout, 
     layout.prefill_split_workspace = split_workspace.data_ptr() if split_workspace is not None else None
     layout.prefill_split_workspace_bytes = split_workspace.numel() if split_workspace is not None else 0
     layout.prefill_key_splits = key_splits
+    layout.prefill_shadow = shadow[0].data_ptr() if shadow is not None else None
+    layout.prefill_shadow_bytes = shadow[0].numel() if shadow is not None else 0
+    layout.prefill_shadow_tokens = shadow[1] if shadow is not None else 0
     Hkv = k_new.shape[2]
     assert q.is_contiguous() and k_new.is_contiguous() and v_new.is_contiguous() and out.is_contiguous()
     if hist_lens is not None:

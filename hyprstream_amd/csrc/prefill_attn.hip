@@ -83,8 +83,12 @@ template <int D> struct alignas(16) HistTile {
 // reference and row sums to the workspace and counts itself in at the tile's counter; the part that finds all others
 // already there adds their partials to its registers, normalises and stores.  Nobody waits for anybody.  For calls
 // whose tiles are too few to occupy the CUs (a chunk of one sequence).
-template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8, bool kSplit = false>
+// kShadow: the history comes from the bf16 operand-order copy of the prompt's dequantized K/V (PrefillArgs::shadow)
+// instead of the codes: whole 32 KB step images go global -> LDS (no registers, no conversion) into a ring of four
+// buffers, three steps ahead, and are consumed by the bf16 products of the new-token phase.  head_dim 128, full width.
+template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8, bool kSplit = false, bool kShadow = false>
 __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_attn_kernel(PrefillArgs a) {
+    static_assert(!kShadow || (kPD == 128 && kCols == 0 && !kWin && kWaves == 8 && !kSplit && !FP8), "shadow history: head_dim 128, full width, int8 cache");
     static_assert(kWaves == 8 || (kWaves == 16 && kCols == 1 && kPD == 128), "sixteen wavefronts: one column block each, head_dim 128");
     static_assert(!kSplit || (!kWin && kWaves == 8), "key split: eight wavefronts, no window");
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
@@ -95,7 +99,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     // converts an eighth of both.
     constexpr bool kSplitRoles = kPD == 64;
     typedef HistTile<kPD> HistTile;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * sizeof(HistTile)];  // two step buffers
+    __shared__ __attribute__((aligned(16))) uint8_t lds[(kShadow ? 4 : 2) * sizeof(HistTile)];  // two step buffers (shadow history: a ring of four)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // scalar: wavefront-dependent branches stay uniform
     const int li = lane & 15, lq = lane >> 4;
@@ -240,7 +244,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     float vup = 1.0f;  // 2^E of the history's V operands, folded back into the accumulators when the history ends
 
     // =============================== history: int8 cache, f16 MFMA ===============================
-    if (H > 0 && (!kSplit || h_lo < h_hi)) {
+    if (!kShadow && H > 0 && (!kSplit || h_lo < h_hi)) {
         // The history operands are fp16(code * scale), and fp16 spans 2^-14 .. 65504 only.  Each (sequence, kv-head)
         // therefore gets a power-of-two reference for K and one for V, taken from the largest scale among its first
         // cached tokens (int8; up to 64 of them, inside one block) or from its head scale (fp8): operands are
@@ -779,10 +783,12 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                         acc[nb][VBG * c + bb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[bb], pop[nb][hh], acc[nb][VBG * c + bb], 0, 0, 0);
             }
         };
-        auto softmax = [&](int step, int nh) {
+        // hist_lim: -1 for a step of the call's own tokens; for a step of the shadow history, the number of its keys that
+        // exist (all 64 but in the last step): every query sees those and nothing else of the step.
+        auto softmax = [&](int step, int nh, int hist_lim = -1) {
             const int t0 = step * kNStep;
             // some (key, query) pair of this step is in the future, or out of the query's window
-            const bool diag = t0 + kNStep - 1 > wv_q0 || (kWin && t0 < wv_lo_last);
+            const bool diag = hist_lim >= 0 ? hist_lim < kNStep : (t0 + kNStep - 1 > wv_q0 || (kWin && t0 < wv_lo_last));
             float e[kNB][16];
             int over = force;
 #pragma unroll
@@ -792,7 +798,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
 #pragma unroll
                     for (int r = 0; r < 4; ++r) e[nb][4 * u4 + r] = (u4 < 2 * nh) ? s[nb][u4][r] : -INFINITY;
                 if (diag) {
-                    const int qrel = min(qi[nb], S - 1) - t0 - 4 * lq;  // key offsets 16u4 + r beyond this are in the future
+                    const int qrel = (hist_lim >= 0 ? hist_lim - 1 : min(qi[nb], S - 1) - t0) - 4 * lq;  // key offsets 16u4 + r beyond this are in the future
 #pragma unroll
                     for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
@@ -835,6 +841,42 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                     l_run[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pop[nb][hh], l_run[nb], 0, 0, 0);
                 }
         };
+        if constexpr (kShadow) {
+            if (H > 0) {
+                // wavefront w moves bytes [4096 w, 4096 w + 4096) of a step image: four 1 KB pieces, lane i its 16 bytes
+                const int hsteps = (H + 63) / 64;
+                const uint8_t *img = (const uint8_t *)a.shadow + ((int64_t)b * a.Hkv + kvh) * a.shadow_steps * (int64_t)kShadowStepBytes + 4096 * wave + 16 * lane;
+                typedef __attribute__((address_space(3))) void *lds_ptr;
+                auto fetch = [&](int hs) {
+                    const uint8_t *src = img + (int64_t)hs * kShadowStepBytes;
+                    uint8_t *dst = lds + (hs & 3) * kShadowStepBytes + 4096 * wave;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) __builtin_amdgcn_global_load_lds(src + 1024 * i, (lds_ptr)(dst + 1024 * i), 16, 0, 0);
+                };
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the Q rows above: the counts below are of step pieces only)
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    if (i < hsteps) fetch(i);
+                for (int hs = 0; hs < hsteps; ++hs) {
+                    // this wavefront's pieces of step hs have landed once at most the pieces of the later steps are pending
+                    if (hs + 2 < hsteps) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+                    else if (hs + 1 < hsteps) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    lds_barrier();  // everybody's pieces of step hs are in; everybody is done with step hs - 1
+                    if (hs + 3 < hsteps) fetch(hs + 3);  // into the buffer of step hs - 1
+                    if (wv_active) {
+                        const HistTile &t = ntiles[hs & 3];
+                        scores(t, 2);
+                        load_v(t, 0);
+                        softmax(0, 2, min(H - hs * 64, 64));
+                        output(t, 0);
+                        load_v(t, 1);
+                        output(t, 1);
+                    }
+                }
+                lds_barrier();  // the ring is free for the tiles of the call's own tokens
+            }
+        }
         issue(st0);
         commit(ntiles[st0 & 1]);
         if (st0 + 1 < nsteps) issue(st0 + 1);
@@ -1103,6 +1145,35 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
         grid.x = (S + q_per_wg - 1) / q_per_wg;
     }
     grid.x *= a.nsplit;
+    // The bf16 copy of the prompt's K/V: every instance that writes the cache appends to it; the full-width instance
+    // reads the history from it.
+    bool shadow_read = false;
+    if (layout->prefill_shadow != nullptr) {
+        const int tokens = layout->prefill_shadow_tokens;
+        const bool can_append = D == 128 && !fp8;
+        if (!can_append) {
+            if (hist_len > 0)
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow serves head_dim 128 over an int8 cache; this call could not append to it");
+        } else {
+            if (tokens <= 0 || (tokens & 63) != 0 || (int64_t)hist_len + S > tokens)
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow_tokens %d must be a multiple of 64 and hold hist_len + S = %lld tokens",
+                            tokens, (long long)hist_len + S);
+            const size_t need = (size_t)B * Hkv * (tokens / 64) * kShadowStepBytes;
+            if (layout->prefill_shadow_bytes < 0 || (size_t)layout->prefill_shadow_bytes < need)
+                return fail(HS_ERR_WORKSPACE, "prefill shadow of %lld bytes, %zu needed", (long long)layout->prefill_shadow_bytes, need);
+            if (((uintptr_t)layout->prefill_shadow & 255) != 0)
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow must be 256-byte aligned");
+            if (!quantize_on_write && hist_len == 0) {
+                // nothing to read and nothing appended: the copy plays no part in this call
+            } else {
+                if (!quantize_on_write)
+                    return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow needs quantize_on_write: a call that caches nothing leaves a hole in the copy");
+                a.shadow = (uint16_t *)layout->prefill_shadow;
+                a.shadow_steps = tokens / 64;
+                shadow_read = hist_len > 0 && a.window == 0 && !narrow && a.nsplit == 1 && !wide32 && !waves16 && hist_lens == nullptr;  // (rows at different positions append, and read the codes)
+            }
+        }
+    }
     // One workgroup fills a CU.  When the grid takes several rounds, the query tiles with the most keys go first so
     // that the launch does not end on them; a single round keeps the plain order.
     a.heavy_first = (int64_t)grid.x * grid.y * grid.z > compute_units();
@@ -1125,7 +1196,9 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
             else prefill_attn_kernel<256, false, 0, WIN><<<grid, 512, 0, st>>>(a);                     \
         }                                                                                                   \
     } while (0)
-    if (a.nsplit > 1) {
+    if (shadow_read) {
+        prefill_attn_kernel<128, false, 0, false, 8, false, true><<<grid, 512, 0, st>>>(a);
+    } else if (a.nsplit > 1) {
 #define HS_PREFILL_SPLIT(DD, CC)                                                                     \
     do {                                                                                             \
         if (fp8) prefill_attn_kernel<DD, true, CC, false, 8, true><<<grid, 512, 0, st>>>(a);         \
@@ -1163,6 +1236,15 @@ size_t hs_prefill_attn_split_workspace_bytes(int32_t B, int32_t S, int32_t Hq, i
                             ? hs::split_counter_bytes(2 * tiles) + (size_t)2 * tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, true)
                             : 0;
     return wide > half ? wide : half;
+}
+
+size_t hs_prefill_shadow_bytes(int32_t B, int32_t Hkv, int32_t D, int32_t max_tokens) {
+    if (B <= 0 || Hkv <= 0 || max_tokens <= 0 || D != 128) return 0;
+    return (size_t)B * Hkv * (((size_t)max_tokens + 63) / 64) * hs::kShadowStepBytes;
+}
+
+int hs_prefill_shadow_init(void *shadow, size_t bytes, hs_stream_t stream) {
+    return hs_prefill_attn_split_workspace_init(shadow, bytes, stream);  // the same clearing launch
 }
 
 int hs_prefill_attn_split_workspace_init(void *workspace, size_t bytes, hs_stream_t stream) {

@@ -34,9 +34,17 @@ struct PrefillArgs {
     int32_t nsplit = 1;
     float *split_ws = nullptr;
     uint32_t *split_cnt = nullptr;
+    // bf16 copy of the prompt's dequantized K/V in MFMA operand order (hs_kv_layout.prefill_shadow): one 64-key step is a
+    // HistTile<128> image, shadow_steps of them per (sequence, kv-head).  Every launch appends its tokens; the instance
+    // that can read it copies whole steps into LDS instead of converting codes.
+    uint16_t *shadow = nullptr;
+    int32_t shadow_steps = 0;
     RowPrologue qpro;     // the q side of the layer's prologue run inside the launch (hs_kv_layout.prefill_q_prologue)
 };
 
+
+// Bytes of one 64-key step of the shadow at head_dim 128 (= sizeof(HistTile<128>): two halves of 8 K + 8 V^T blocks).
+constexpr int kShadowStepBytes = 32768;
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() would also wait for every outstanding global
 // load, i.e. for the tile prefetch that was issued a moment earlier and is not needed before the next step.
@@ -112,6 +120,29 @@ __device__ __forceinline__ void write_new_rows(const PrefillArgs &a, int b, int 
                             qv = qv < -127.0f ? -127.0f : qv;
                             if (qv != qv) qv = 0.0f;
                             packed[e >> 2] |= ((uint32_t)(int)qv & 0xffu) << (8 * (e & 3));
+                        }
+                    }
+                }
+                if constexpr (!FP8 && kRow == 128) {
+                    if (a.shadow != nullptr && live) {
+                        // the dequantized row (code * scale, rounded to bf16: what the reference's get() hands to its
+                        // attention) into the step image of its position; `packed` holds the codes
+                        const int pos = H + tt, kk = pos & 31;
+                        uint16_t *img = a.shadow + (((int64_t)b * a.Hkv + kvh) * a.shadow_steps + (pos >> 6)) * (kShadowStepBytes / 2) +
+                                        ((pos >> 5) & 1) * (kShadowStepBytes / 4);  // this half: K blocks [2 KG][512 el], then V^T blocks [VB][512 el]
+                        float dq[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) dq[e] = (float)(int8_t)(packed[e >> 2] >> (8 * (e & 3))) * sc;
+                        if (which == 0) {
+                            // K block (tile u = kk / 16, d-group j): lane (li = key, lq) holds d = 32 lq + 8 j ..; this lane has d = 8 sub ..
+                            const int blk = 4 * (kk >> 4) + (sub & 3), ln = (sub >> 2) * 16 + (kk & 15);
+                            *(u32x4 *)(img + blk * 512 + ln * 8) = (u32x4){pack_bf16x2(dq[0], dq[1]), pack_bf16x2(dq[2], dq[3]),
+                                                                           pack_bf16x2(dq[4], dq[5]), pack_bf16x2(dq[6], dq[7])};
+                        } else {
+                            // V^T block bb: lane (li = d / 8, lq = (kk % 16) / 4), slot 4 (kk / 16) + kk % 4, row d = 8 li + bb
+                            uint16_t *vp = img + 8 * 512 + (((kk & 15) >> 2) * 16 + sub) * 8 + 4 * (kk >> 4) + (kk & 3);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) vp[e * 512] = (uint16_t)f32_to_bf16_bits(dq[e]);
                         }
                     }
                 }

@@ -72,12 +72,12 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_abi_version_and_empty_error():
-    assert hb.lib().hs_attn_abi_version() == 7
+    assert hb.lib().hs_attn_abi_version() == 8
 
 
 def test_layout_struct_matches_header_size():
-    # 4 x int64 + 2 x int32 + 2 pointers + int64 + 2 x int32 + 3 pointers + int64 + 2 x int32
-    assert ctypes.sizeof(hb.KvLayout) == 4 * 8 + 2 * 4 + 2 * 8 + 8 + 2 * 4 + 3 * 8 + 8 + 2 * 4
+    # 4 x int64 + 2 x int32 + 2 pointers + int64 + 2 x int32 + 3 pointers + int64 + 2 x int32 + pointer + int64 + 2 x int32
+    assert ctypes.sizeof(hb.KvLayout) == 4 * 8 + 2 * 4 + 2 * 8 + 8 + 2 * 4 + 3 * 8 + 8 + 2 * 4 + 8 + 8 + 2 * 4
 
 
 def _call_quant(layout, B=1, S=1, Hkv=2, D=128, start_pos=0, fake=0x1000):

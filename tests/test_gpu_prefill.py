@@ -642,3 +642,59 @@ def test_key_split_workspace_errors():
         hb.prefill_attn(q, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, 0, out, 0.1, False,
                         columns=0, split_workspace=ws, key_splits=9)
     assert e.value.code == 1
+
+
+@pytest.mark.parametrize("chunks", [(64, 64, 64), (100, 37, 200, 91), (512, 512), (1, 63, 64, 300)])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (6, 2), (4, 4)])
+def test_history_from_the_bf16_shadow(chunks, Hq, Hkv):
+    """hs_kv_layout.prefill_shadow: every call appends its dequantized rows to a bf16 operand-order copy and calls with
+    history read that copy instead of the codes.  A prompt in uneven chunks (history lengths that are not multiples of
+    the 64-key step, a partial last step whose remaining rows the same launch is writing) against the same calls
+    without the copy and against the oracle; the int8 cache is the same bits either way."""
+    B, D = 2, 128
+    T = sum(chunks)
+    q, k, v = make(8100 + T + Hq, B, T, Hq, Hkv, D)
+    dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
+    shadow = hb.prefill_shadow(B, Hkv, D, T)
+    with_copy, without = DeviceCache(B, Hkv, T, D), DeviceCache(B, Hkv, T, D)
+    lo = 0
+    for n in chunks:
+        hi = lo + n
+        outs = []
+        for c, sh in ((without, None), (with_copy, shadow)):
+            out = torch.full((B, n, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+            hb.prefill_attn(dev(q[:, lo:hi]), dev(k[:, lo:hi]), dev(v[:, lo:hi]), c.k_codes, c.v_codes, c.k_scales, c.v_scales,
+                            c.layout, lo, out, 1.0 / np.sqrt(D), True, columns=256, key_splits=1, shadow=sh)
+            torch.cuda.synchronize()
+            outs.append(out.float().cpu().numpy())
+        assert np.isfinite(outs[1]).all(), (lo, hi)
+        # the copy holds bf16(code * scale) where the other path uses fp16(code * scale): both within the oracle's bar
+        assert np.abs(outs[1] - outs[0]).max() <= 2.0 ** -6 * max(1.0, np.abs(outs[0]).max()), (lo, hi)
+        if lo > 0:
+            kc, vc, ks, vs = without.canonical(lo)
+            want = oracle_prefill(q[:, lo:hi], oracle.dequant_int8(kc, ks), oracle.dequant_int8(vc, vs), k[:, lo:hi], v[:, lo:hi])
+            compare(outs[1], want, "shadow history %d..%d" % (lo, hi))
+        lo = hi
+    assert torch.equal(with_copy.k_codes, without.k_codes) and torch.equal(with_copy.v_codes, without.v_codes)
+    assert torch.equal(with_copy.k_scales, without.k_scales) and torch.equal(with_copy.v_scales, without.v_scales)
+
+
+def test_shadow_contract_errors():
+    B, S, Hq, Hkv, D = 1, 64, 4, 1, 128
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
+    c = DeviceCache(B, Hkv, 256, D)
+    q, k, o = z(B, S, Hq, D), z(B, S, Hkv, D), z(B, S, Hq, D)
+    run = lambda sh, hist=0, write=True: hb.prefill_attn(q, k, k, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, hist, o,
+                                                          0.1, write, columns=0, key_splits=1, shadow=sh)
+    buf, tokens = hb.prefill_shadow(B, Hkv, D, 128)
+    run((buf, tokens))                                   # fits
+    with pytest.raises(hb.HsError) as e:                 # 128 + 64 tokens do not
+        run((buf, tokens), hist=128)
+    assert e.value.code == 1 and "prefill_shadow_tokens" in str(e.value)
+    with pytest.raises(hb.HsError) as e:                 # a buffer shorter than its token count says
+        run((buf[: buf.numel() // 2], tokens), hist=64)
+    assert e.value.code == hb.HS_ERR_WORKSPACE
+    with pytest.raises(hb.HsError) as e:                 # history but no cache write: would leave a hole
+        run((buf, tokens), hist=64, write=False)
+    assert e.value.code == 1 and "quantize_on_write" in str(e.value)
+    assert hb.lib().hs_prefill_shadow_bytes(1, 1, 256, 128) == 0
