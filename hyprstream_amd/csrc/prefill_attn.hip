@@ -1118,9 +1118,11 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
             P = (int)std::min<int64_t>(kMaxKeySplits, compute_units() / tiles);
             P = std::min(P, max_steps / 4);  // at least four steps to a run
             if (P < 3) P = 1;                // two runs of full-width tiles: the half-width workgroups do as well without a merge
-            if (P >= 4 && can_narrow && hint == 0) {
+            if (P >= 4 && can_narrow && hint != 256) {  // half-width tiles (the library's choice, or asked for): half the runs
                 split_narrow = true;
                 P /= 2;
+            } else if (split_narrow) {
+                P = 1;  // half-width asked for, too few steps to split those: the plain half-width launch
             }
         }
         if (P < 1 || P > kMaxKeySplits)
