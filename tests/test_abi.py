@@ -255,3 +255,43 @@ def test_prefill_rejects_bad_arguments_before_launching():
     rc = L.hs_prefill_attn_int8_ragged(p, p, p, p, p, p, p, ctypes.byref(lay), p, 60, p, 2, 8, 8, 2, 128, f, 1, None)
     assert rc == hb.HS_ERR_OVERFLOW                                   # the bound, not the array, is what the host checks
     assert call(lay, 0, B=0) == hb.HS_OK and call(lay, 0, S=0) == hb.HS_OK  # empty problems are not an error
+
+
+def _call_prefill(layout, hist_len=0, B=1, S=64, Hq=4, Hkv=1, D=128, write=1, fake=0x1000):
+    p = ctypes.c_void_p(fake)
+    out = ctypes.c_void_p(fake + 0x100000)
+    return hb.lib().hs_prefill_attn_int8(p, p, p, p, p, p, p, ctypes.byref(layout), ctypes.c_int32(hist_len), out, B, S, Hq,
+                                         Hkv, D, ctypes.c_float(0.1), write, None)
+
+
+def test_prefill_scratch_sizes_and_contracts_without_a_gpu():
+    """The two optional prefill buffers: their size functions, and the checks that refuse a bad one before any launch."""
+    L = hb.lib()
+    # key-split workspace: grows with the tokens of a call, zero for shapes the kernels do not serve
+    small = L.hs_prefill_attn_split_workspace_bytes(1, 512, 32, 8, 128)
+    assert small > 0 and small % 256 == 0
+    assert L.hs_prefill_attn_split_workspace_bytes(1, 1024, 32, 8, 128) > small
+    assert L.hs_prefill_attn_split_workspace_bytes(1, 512, 32, 8, 96) == 0
+    assert L.hs_prefill_attn_split_workspace_bytes(1, 512, 30, 8, 128) == 0
+    # bf16 copy: 512 bytes per token and kv-head at head_dim 128, whole 64-token steps
+    assert L.hs_prefill_shadow_bytes(4, 8, 128, 4096) == 4 * 8 * 4096 * 512
+    assert L.hs_prefill_shadow_bytes(1, 1, 128, 65) == 128 * 512
+    assert L.hs_prefill_shadow_bytes(1, 1, 64, 64) == 0
+    lay = hb.contiguous_layout(1, 256, 128)
+    lay.prefill_shadow, lay.prefill_shadow_bytes, lay.prefill_shadow_tokens = 0x200000, 128 * 512, 100
+    assert _call_prefill(lay) == hb.HS_ERR_INVALID_ARGUMENT            # tokens not a multiple of 64
+    assert b"prefill_shadow_tokens" in L.hs_attn_last_error()
+    lay.prefill_shadow_tokens = 128
+    assert _call_prefill(lay, hist_len=128) == hb.HS_ERR_INVALID_ARGUMENT  # 128 + 64 tokens do not fit
+    lay.prefill_shadow_bytes = 64 * 512
+    assert _call_prefill(lay, hist_len=64) == hb.HS_ERR_WORKSPACE
+    lay.prefill_shadow_bytes = 128 * 512
+    assert _call_prefill(lay, hist_len=64, write=0) == hb.HS_ERR_INVALID_ARGUMENT  # history, nothing cached
+    lay.prefill_shadow = 0x200010
+    assert _call_prefill(lay, hist_len=64) == hb.HS_ERR_INVALID_ARGUMENT   # alignment
+    # key split: too small a workspace, a count out of range
+    lay = hb.contiguous_layout(1, 256, 128)
+    lay.prefill_split_workspace, lay.prefill_split_workspace_bytes, lay.prefill_key_splits = 0x300000, 4096, 4
+    assert _call_prefill(lay, hist_len=128) == hb.HS_ERR_WORKSPACE
+    lay.prefill_key_splits = 9
+    assert _call_prefill(lay, hist_len=128) == hb.HS_ERR_INVALID_ARGUMENT
