@@ -698,3 +698,46 @@ def test_shadow_contract_errors():
         run((buf, tokens), hist=64, write=False)
     assert e.value.code == 1 and "quantize_on_write" in str(e.value)
     assert hb.lib().hs_prefill_shadow_bytes(1, 1, 256, 128) == 0
+
+
+def test_shadow_over_a_paged_pool_and_random_chunkings():
+    """The copy is indexed by the call's sequences, not by the cache's storage: the same prompt prefilled into a paged pool
+    (64-token blocks scattered, K and V interleaved) with the copy gives the outputs of the contiguous cache with the
+    copy, bit for bit, and the same pool contents as without it; chunk boundaries drawn at random."""
+    B, Hq, Hkv, D, BT = 2, 8, 2, 128, 64
+    r = wl.philox(8300)
+    for trial in range(3):
+        cuts = sorted(set(int(x) for x in r.integers(1, 700, size=4)))
+        T = cuts[-1]
+        q, k, v = make(8310 + trial, B, T, Hq, Hkv, D)
+        dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
+        nblk = (T + BT - 1) // BT
+        ids = r.permutation(2 * B * nblk + 3).astype(np.int32)
+        k_tab = torch.from_numpy(ids[:B * nblk].reshape(B, nblk)).to(DEV)
+        v_tab = torch.from_numpy(ids[B * nblk:2 * B * nblk].reshape(B, nblk)).to(DEV)
+        pools = []
+        outs = {}
+        for name in ("contiguous+copy", "paged+copy", "paged"):
+            if name.startswith("paged"):
+                codes = torch.zeros(len(ids), Hkv, BT, D, dtype=torch.int8, device=DEV)
+                scales = torch.zeros(len(ids), Hkv, BT, dtype=torch.float32, device=DEV)
+                bufs, lay = (codes, codes, scales, scales), hb.paged_layout(Hkv, BT, D, k_tab, v_tab)
+                pools.append((codes, scales))
+            else:
+                c = DeviceCache(B, Hkv, T, D)
+                bufs, lay = (c.k_codes, c.v_codes, c.k_scales, c.v_scales), c.layout
+            sh = hb.prefill_shadow(B, Hkv, D, T) if name.endswith("copy") else None
+            got, lo = [], 0
+            for hi in cuts:
+                out = torch.full((B, hi - lo, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+                hb.prefill_attn(dev(q[:, lo:hi]), dev(k[:, lo:hi]), dev(v[:, lo:hi]), *bufs, lay, lo, out, 1.0 / np.sqrt(D), True,
+                                columns=256, key_splits=1, shadow=sh)
+                got.append(out)
+                lo = hi
+            torch.cuda.synchronize()
+            outs[name] = torch.cat(got, 1)
+        assert not torch.isnan(outs["paged+copy"].float()).any()
+        assert torch.equal(outs["paged+copy"].view(torch.int16), outs["contiguous+copy"].view(torch.int16)), cuts
+        assert torch.equal(pools[0][0], pools[1][0]) and torch.equal(pools[0][1], pools[1][1])
+        d = (outs["paged+copy"].float() - outs["paged"].float()).abs().max().item()
+        assert d <= 2.0 ** -6 * max(1.0, outs["paged"].float().abs().max().item()), (cuts, d)
