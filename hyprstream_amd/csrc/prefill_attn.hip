@@ -785,10 +785,14 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         };
         // hist_lim: -1 for a step of the call's own tokens; for a step of the shadow history, the number of its keys that
         // exist (all 64 but in the last step): every query sees those and nothing else of the step.
-        auto softmax = [&](int step, int nh, int hist_lim = -1) {
+        // kind 0: a step of the call's own tokens.  Shadow history: 1 = a whole step (every query sees every key: no
+        // mask code at all -- as a run-time flag the compiler turned the masks into 64 selects per step), 2 = the last,
+        // partial step, of which hist_lim keys exist.
+        auto softmax = [&](int step, int nh, auto kind_tag, int hist_lim = -1) {
+            constexpr int kKind = decltype(kind_tag)::value;
             const int t0 = step * kNStep;
             // some (key, query) pair of this step is in the future, or out of the query's window
-            const bool diag = hist_lim >= 0 ? hist_lim < kNStep : (t0 + kNStep - 1 > wv_q0 || (kWin && t0 < wv_lo_last));
+            const bool diag = kKind == 1 ? false : kKind == 2 ? true : (t0 + kNStep - 1 > wv_q0 || (kWin && t0 < wv_lo_last));
             float e[kNB][16];
             int over = force;
 #pragma unroll
@@ -797,8 +801,8 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                 for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) e[nb][4 * u4 + r] = (u4 < 2 * nh) ? s[nb][u4][r] : -INFINITY;
-                if (diag) {
-                    const int qrel = (hist_lim >= 0 ? hist_lim - 1 : min(qi[nb], S - 1) - t0) - 4 * lq;  // key offsets 16u4 + r beyond this are in the future
+                if (kKind != 1 && diag) {
+                    const int qrel = (kKind == 2 ? hist_lim - 1 : min(qi[nb], S - 1) - t0) - 4 * lq;  // key offsets 16u4 + r beyond this are in the future
 #pragma unroll
                     for (int u4 = 0; u4 < 4; ++u4)
 #pragma unroll
@@ -857,7 +861,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
 #pragma unroll
                 for (int i = 0; i < 3; ++i)
                     if (i < hsteps) fetch(i);
-                for (int hs = 0; hs < hsteps; ++hs) {
+                auto hist_step = [&](int hs, auto kind_tag) {
                     // this wavefront's pieces of step hs have landed once at most the pieces of the later steps are pending
                     if (hs + 2 < hsteps) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
                     else if (hs + 1 < hsteps) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
@@ -868,12 +872,15 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                         const HistTile &t = ntiles[hs & 3];
                         scores(t, 2);
                         load_v(t, 0);
-                        softmax(0, 2, min(H - hs * 64, 64));
+                        softmax(0, 2, kind_tag, H - hs * 64);
                         output(t, 0);
                         load_v(t, 1);
                         output(t, 1);
                     }
-                }
+                };
+                const int whole = H / 64;  // the steps every key of which exists; a last, partial one has its own code
+                for (int hs = 0; hs < whole; ++hs) hist_step(hs, std::integral_constant<int, 1>{});
+                if (whole < hsteps) hist_step(whole, std::integral_constant<int, 2>{});
                 lds_barrier();  // the ring is free for the tiles of the call's own tokens
             }
         }
@@ -889,7 +896,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                 const HistTile &t = ntiles[st & 1];
                 scores(t, nh);
                 load_v(t, 0);
-                softmax(st, nh);
+                softmax(st, nh, std::integral_constant<int, 0>{});
                 output(t, 0);
                 if (nh > 1) {
                     load_v(t, 1);
