@@ -131,7 +131,7 @@ typedef struct hs_kv_layout {
                                    kept by the caller for as long as one prompt is being prefilled into one layer's
                                    cache.  Every prefill call with quantize_on_write = 1 appends its tokens to it; a
                                    call with history reads the history from it instead of converting the cached codes
-                                   in every workgroup that needs them (-21 % per history step at 4 x 512 queries).  The
+                                   in every workgroup that needs them (-15 % per history step at 4 x 512 queries).  The
                                    int8 cache is written as always and stays the cache; the copy may be dropped after
                                    the prompt.  Contract: hs_prefill_shadow_bytes(B, Hkv, D, prefill_shadow_tokens)
                                    bytes, 256-byte aligned, cleared once by hs_prefill_shadow_init; prefill_shadow_tokens
