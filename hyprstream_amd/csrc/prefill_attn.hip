@@ -593,34 +593,37 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
         // the other buffer and starts the global loads of tile s+2.  The second wavefront of each SIMD does its
         // conversion at the end of the step instead of the beginning, so that its matrix phases tend to meet
         // the other one's vector phases.
-        // head_dim 128, eight wavefronts: operand reads run kAhead blocks ahead of the products that use them, through a
-        // ring of eight registers, in a pinned order (see the copy-fed walk of the new-token phase for what that is worth).
-        constexpr bool kRing = kPD == 128 && kWaves == 8;
-        constexpr int kAhead = 6;
+        // Eight wavefronts: operand reads run kAhead blocks ahead of the products that use them, through a ring of eight
+        // registers, in a pinned order (see the copy-fed walk of the new-token phase for what that is worth).  A half of a
+        // step holds NKB = 2 KG blocks of K (tile-major) and NVB = VB blocks of V^T.
+        constexpr bool kRing = kWaves == 8;
+        constexpr int kAhead = 6, NKB = 2 * KG, NVB = VB;
         half8 ring[8];
-        auto kblk = [&](const HistTile &t, int k) { return *(const half8 *)(t.h[k >> 3].k[k & 7] + obase); };
-        auto vblk = [&](const HistTile &t, int k) { return *(const half8 *)(t.h[k >> 3].v[k & 7] + obase); };
-        auto scores_ahead = [&](const HistTile &t) {  // K block k = 8 half + 4 tile-of-half + d-group; leaves the first V blocks in the ring
+        auto kblk = [&](const HistTile &t, int k) { return *(const half8 *)(t.h[k / NKB].k[k % NKB] + obase); };
+        auto vblk = [&](const HistTile &t, int k) { return *(const half8 *)(t.h[k / NVB].v[k % NVB] + obase); };
+        auto scores_ahead = [&](const HistTile &t) {  // leaves the first V blocks in the ring
 #pragma unroll
             for (int k = 0; k < kAhead; ++k) ring[k] = kblk(t, k);
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
-                ring[(k + kAhead) & 7] = k + kAhead < 16 ? kblk(t, k + kAhead) : vblk(t, k + kAhead - 16);
+            for (int k = 0; k < 2 * NKB; ++k) {
+                if (k + kAhead < 2 * NKB) ring[(k + kAhead) & 7] = kblk(t, k + kAhead);
+                else if (k + kAhead - 2 * NKB < 2 * NVB) ring[(k + kAhead) & 7] = vblk(t, k + kAhead - 2 * NKB);
                 __builtin_amdgcn_sched_barrier(0);
+                const int tile = 2 * (k / NKB) + (k % NKB) / KG, j = k % KG;
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb)
-                    s[nb][k >> 2] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[k & 7], qop[nb][k & 3], (k & 3) == 0 ? sinit[nb] : s[nb][k >> 2], 0, 0, 0);
+                    s[nb][tile] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[k & 7], qop[nb][j], j == 0 ? sinit[nb] : s[nb][tile], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        auto output_ahead = [&](const HistTile &t) {  // V^T block k = 8 half + row block
+        auto output_ahead = [&](const HistTile &t) {  // V^T block k of the step sits in ring slot (2 NKB + k) % 8
 #pragma unroll
-            for (int k = 0; k < 16; ++k) {
-                if (k + kAhead < 16) ring[(k + kAhead) & 7] = vblk(t, k + kAhead);
+            for (int k = 0; k < 2 * NVB; ++k) {
+                if (k + kAhead < 2 * NVB) ring[(2 * NKB + k + kAhead) & 7] = vblk(t, k + kAhead);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int nb = 0; nb < kNB; ++nb)
-                    acc[nb][k & 7] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[k & 7], pop[nb][k >> 3], acc[nb][k & 7], 0, 0, 0);
+                    acc[nb][k % NVB] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[(2 * NKB + k) & 7], pop[nb][k / NVB], acc[nb][k % NVB], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
