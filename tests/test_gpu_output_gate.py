@@ -64,9 +64,20 @@ def test_decode(B, T, hint, D, fp8):
     _check(outs[1], outs[0], gate)
 
 
+@pytest.mark.parametrize("mode", ["plain", "key-split", "bf16-copy"])
 @pytest.mark.parametrize("D,Hq,Hkv,hist,S", [(128, 8, 2, 0, 70), (128, 32, 8, 200, 130), (256, 8, 2, 64, 64), (64, 6, 2, 33, 100)])
-def test_prefill(D, Hq, Hkv, hist, S):
+def test_prefill(D, Hq, Hkv, hist, S, mode):
+    """The gate is applied by whichever workgroup stores the output: the tile's own, the one that merges a key split's
+    runs, or the instance that reads the history from the bf16 copy."""
+    if mode == "bf16-copy" and D != 128:
+        pytest.skip("the copy serves head_dim 128")
     B, T = 2, hist + S
+    extra = lambda: {}
+    if mode == "key-split":
+        extra = lambda: dict(columns=0, key_splits=3, split_workspace=hb.prefill_split_workspace(B, max(S, hist, 1), Hq, Hkv, D))
+    elif mode == "bf16-copy":
+        extra = lambda: dict(columns=256, key_splits=1, shadow=shadows[-1])
+    shadows = []
     r = wl.philox(5200 + D)
     t = lambda *s: torch.from_numpy(r.standard_normal(s).astype(np.float32)).to(torch.bfloat16).to(DEV)
     q, k, v = t(B, T, Hq, D), t(B, T, Hkv, D), t(B, T, Hkv, D)
@@ -78,13 +89,15 @@ def test_prefill(D, Hq, Hkv, hist, S):
         vc = torch.zeros_like(kc)
         ks = torch.zeros(B, Hkv, lay.scale_stride_head, dtype=torch.float32, device=DEV)
         vs = torch.zeros_like(ks)
+        if mode == "bf16-copy":
+            shadows.append(hb.prefill_shadow(B, Hkv, D, T))
         if hist:
             o0 = torch.empty(B, hist, Hq, D, dtype=torch.bfloat16, device=DEV)
             hb.prefill_attn(q[:, :hist].contiguous(), k[:, :hist].contiguous(), v[:, :hist].contiguous(), kc, vc, ks, vs, lay, 0, o0,
-                            1.0 / np.sqrt(D), True)
+                            1.0 / np.sqrt(D), True, **extra())
         out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
         hb.prefill_attn(q[:, hist:].contiguous(), k[:, hist:].contiguous(), v[:, hist:].contiguous(), kc, vc, ks, vs,
-                        _with_gate(lay, gate) if use_gate else lay, hist, out, 1.0 / np.sqrt(D), True)
+                        _with_gate(lay, gate) if use_gate else lay, hist, out, 1.0 / np.sqrt(D), True, **extra())
         torch.cuda.synchronize()
         outs.append((out, kc.clone(), ks.clone()))
     _check(outs[1][0], outs[0][0], gate)
