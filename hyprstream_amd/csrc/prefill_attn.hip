@@ -88,7 +88,7 @@ template <int D> struct alignas(16) HistTile {
 // buffers, three steps ahead, and are consumed by the bf16 products of the new-token phase.  head_dim 128, full width.
 template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8, bool kSplit = false, bool kShadow = false>
 __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_attn_kernel(PrefillArgs a) {
-    static_assert(!kShadow || (kPD == 128 && kCols == 0 && !kWin && kWaves == 8 && !kSplit && !FP8), "shadow history: head_dim 128, full width, int8 cache");
+    static_assert(!kShadow || (kPD == 128 && !kWin && kWaves == 8 && !FP8), "shadow history: head_dim 128, eight wavefronts, int8 cache, no window");
     static_assert(kWaves == 8 || (kWaves == 16 && kCols == 1 && kPD == 128), "sixteen wavefronts: one column block each, head_dim 128");
     static_assert(!kSplit || (!kWin && kWaves == 8), "key split: eight wavefronts, no window");
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
@@ -673,7 +673,9 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
     }
 
     // =============================== new tokens: bf16, causal ===============================
-    if (!kSplit || n_lo < n_hi) {
+    // (with the bf16 copy, the history steps of this workgroup run in here too, ahead of the call's own tokens)
+    const bool hist_here = kShadow && H > 0 && (!kSplit || h_lo < h_hi), new_here = !kSplit || n_lo < n_hi;
+    if (hist_here || new_here) {
         // Q operands carry the softmax scale and log2(e), rounded back to bf16 (2^-9 relative, the precision the
         // weights are rounded to anyway), so that the MFMA result needs no multiplication; as in the history
         // phase the score accumulators start from -sref and the common step only checks for an overflow.
@@ -886,9 +888,9 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                 }
         };
         if constexpr (kShadow) {
-            if (H > 0) {
+            if (hist_here) {
                 // wavefront w moves bytes [4096 w, 4096 w + 4096) of a step image: four 1 KB pieces, lane i its 16 bytes
-                const int hsteps = (H + 63) / 64;
+                const int hs0 = kSplit ? h_lo : 0, hsteps = kSplit ? h_hi : (H + 63) / 64;  // this workgroup's run of history steps
                 const uint8_t *img = (const uint8_t *)a.shadow + ((int64_t)b * a.Hkv + kvh) * a.shadow_steps * (int64_t)kShadowStepBytes + 4096 * wave + 16 * lane;
                 typedef __attribute__((address_space(3))) void *lds_ptr;
                 auto fetch = [&](int hs) {
@@ -900,7 +902,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the Q rows above: the counts below are of step pieces only)
 #pragma unroll
                 for (int i = 0; i < 3; ++i)
-                    if (i < hsteps) fetch(i);
+                    if (hs0 + i < hsteps) fetch(hs0 + i);
                 // Operand reads run kAhead blocks ahead of the products that use them, through a ring of eight registers,
                 // in a pinned order: a wavefront that first issues its sixteen products of a tile and only then asks for
                 // the next operands leaves the matrix pipe idle for an LDS round trip per tile, and its SIMD partner is
@@ -948,11 +950,12 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                     }
                 };
                 const int whole = H / 64;  // the steps every key of which exists; a last, partial one has its own code
-                for (int hs = 0; hs < whole; ++hs) hist_step(hs, std::integral_constant<int, 1>{});
+                for (int hs = hs0; hs < min(whole, hsteps); ++hs) hist_step(hs, std::integral_constant<int, 1>{});
                 if (whole < hsteps) hist_step(whole, std::integral_constant<int, 2>{});
                 lds_barrier();  // the ring is free for the tiles of the call's own tokens
             }
         }
+        if (new_here) {
         issue(st0);
         commit(ntiles[st0 & 1]);
         if (st0 + 1 < nsteps) issue(st0 + 1);
@@ -973,6 +976,7 @@ __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_att
                 }
             }
             lds_barrier();
+        }
         }
     }
 
@@ -1248,7 +1252,7 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
                     return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow needs quantize_on_write: a call that caches nothing leaves a hole in the copy");
                 a.shadow = (uint16_t *)layout->prefill_shadow;
                 a.shadow_steps = tokens / 64;
-                shadow_read = hist_len > 0 && a.window == 0 && !narrow && a.nsplit == 1 && !wide32 && !waves16 && hist_lens == nullptr;  // (rows at different positions append, and read the codes)
+                shadow_read = hist_len > 0 && a.window == 0 && !wide32 && !waves16 && hist_lens == nullptr;  // (rows at different positions append, and read the codes)
             }
         }
     }
@@ -1275,7 +1279,13 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
         }                                                                                                   \
     } while (0)
     if (shadow_read) {
-        prefill_attn_kernel<128, false, 0, false, 8, false, true><<<grid, 512, 0, st>>>(a);
+        if (a.nsplit > 1) {
+            if (narrow) prefill_attn_kernel<128, false, 1, false, 8, true, true><<<grid, 512, 0, st>>>(a);
+            else prefill_attn_kernel<128, false, 0, false, 8, true, true><<<grid, 512, 0, st>>>(a);
+        } else {
+            if (narrow) prefill_attn_kernel<128, false, 1, false, 8, false, true><<<grid, 512, 0, st>>>(a);
+            else prefill_attn_kernel<128, false, 0, false, 8, false, true><<<grid, 512, 0, st>>>(a);
+        }
     } else if (a.nsplit > 1) {
 #define HS_PREFILL_SPLIT(DD, CC)                                                                     \
     do {                                                                                             \

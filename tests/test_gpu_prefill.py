@@ -644,14 +644,18 @@ def test_key_split_workspace_errors():
     assert e.value.code == 1
 
 
+@pytest.mark.parametrize("variant", ["full", "half", "split3", "split2-half"])
 @pytest.mark.parametrize("chunks", [(64, 64, 64), (100, 37, 200, 91), (512, 512), (1, 63, 64, 300)])
 @pytest.mark.parametrize("Hq,Hkv", [(8, 2), (6, 2), (4, 4)])
-def test_history_from_the_bf16_shadow(chunks, Hq, Hkv):
+def test_history_from_the_bf16_shadow(chunks, Hq, Hkv, variant):
     """hs_kv_layout.prefill_shadow: every call appends its dequantized rows to a bf16 operand-order copy and calls with
     history read that copy instead of the codes.  A prompt in uneven chunks (history lengths that are not multiples of
     the 64-key step, a partial last step whose remaining rows the same launch is writing) against the same calls
-    without the copy and against the oracle; the int8 cache is the same bits either way."""
+    without the copy and against the oracle; the int8 cache is the same bits either way.  At full and at half width,
+    and with every tile's steps split into runs (a run may hold history steps only, new-token steps only, or both)."""
     B, D = 2, 128
+    cols = 128 if variant.endswith("half") else 256
+    runs = int(variant[5]) if variant.startswith("split") else 1
     T = sum(chunks)
     q, k, v = make(8100 + T + Hq, B, T, Hq, Hkv, D)
     dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
@@ -663,8 +667,9 @@ def test_history_from_the_bf16_shadow(chunks, Hq, Hkv):
         outs = []
         for c, sh in ((without, None), (with_copy, shadow)):
             out = torch.full((B, n, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ws = hb.prefill_split_workspace(B, n, Hq, Hkv, D) if runs > 1 else None
             hb.prefill_attn(dev(q[:, lo:hi]), dev(k[:, lo:hi]), dev(v[:, lo:hi]), c.k_codes, c.v_codes, c.k_scales, c.v_scales,
-                            c.layout, lo, out, 1.0 / np.sqrt(D), True, columns=256, key_splits=1, shadow=sh)
+                            c.layout, lo, out, 1.0 / np.sqrt(D), True, columns=cols, key_splits=runs, split_workspace=ws, shadow=sh)
             torch.cuda.synchronize()
             outs.append(out.float().cpu().numpy())
         assert np.isfinite(outs[1]).all(), (lo, hi)
