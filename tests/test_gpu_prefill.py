@@ -30,6 +30,12 @@ def columns_per_workgroup(request, monkeypatch):
 TOL_MAX, TOL_MEAN = 2e-2, 2e-3
 
 
+def _fixes_its_own_instance():
+    """For tests that pass the width and the split themselves: run them once, not once per value of the fixture."""
+    if hb.PREFILL_COLUMNS != 0 or hb.PREFILL_KEY_SPLITS != 0:
+        pytest.skip("chooses its own instance: run under the fixture's first value only")
+
+
 def bf16r(x):
     return wl.bf16_bits_to_f32(wl.to_bf16_bits(x))
 
@@ -595,6 +601,7 @@ def test_key_split_the_library_picks_for_a_chunk_of_one_sequence(D, fp8):
     into runs.  Outputs agree with the unsplit launch within the rounding of another summation order and with the
     oracle; the cache rows are the same bits; the workspace is left ready for the next call (second call, same
     answer)."""
+    _fixes_its_own_instance()
     B, S, H, Hq, Hkv = 1, 512, 1536, (32 if D != 256 else 16), (8 if D != 256 else 4)
     r = wl.philox(7300 + D + fp8)
     sigma = 0.5 if fp8 else 1.0
@@ -628,6 +635,7 @@ def test_key_split_the_library_picks_for_a_chunk_of_one_sequence(D, fp8):
 
 
 def test_key_split_workspace_errors():
+    _fixes_its_own_instance()
     B, S, Hq, Hkv, D = 1, 128, 8, 2, 128
     q, k, v = (torch.zeros(B, S, H, D, dtype=torch.bfloat16, device=DEV) for H in (Hq, Hkv, Hkv))
     c = DeviceCache(B, Hkv, S, D)
@@ -653,6 +661,7 @@ def test_history_from_the_bf16_shadow(chunks, Hq, Hkv, variant):
     the 64-key step, a partial last step whose remaining rows the same launch is writing) against the same calls
     without the copy and against the oracle; the int8 cache is the same bits either way.  At full and at half width,
     and with every tile's steps split into runs (a run may hold history steps only, new-token steps only, or both)."""
+    _fixes_its_own_instance()
     B, D = 2, 128
     cols = 128 if variant.endswith("half") else 256
     runs = int(variant[5]) if variant.startswith("split") else 1
@@ -685,6 +694,7 @@ def test_history_from_the_bf16_shadow(chunks, Hq, Hkv, variant):
 
 
 def test_shadow_contract_errors():
+    _fixes_its_own_instance()
     B, S, Hq, Hkv, D = 1, 64, 4, 1, 128
     z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
     c = DeviceCache(B, Hkv, 256, D)
@@ -709,6 +719,7 @@ def test_shadow_over_a_paged_pool_and_random_chunkings():
     """The copy is indexed by the call's sequences, not by the cache's storage: the same prompt prefilled into a paged pool
     (64-token blocks scattered, K and V interleaved) with the copy gives the outputs of the contiguous cache with the
     copy, bit for bit, and the same pool contents as without it; chunk boundaries drawn at random."""
+    _fixes_its_own_instance()
     B, Hq, Hkv, D, BT = 2, 8, 2, 128, 64
     r = wl.philox(8300)
     for trial in range(3):
