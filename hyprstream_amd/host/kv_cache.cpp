@@ -2,6 +2,8 @@
 // memory with hipMalloc and calls the C ABI of libhs_attn for every kernel.
 #include "kv_cache.hpp"
 
+#include <algorithm>
+
 #include <hip/hip_runtime_api.h>
 
 #include "device_fill.hpp"
@@ -23,7 +25,17 @@ LayerKVCache::LayerKVCache(size_t max_len, KVQuantType qt) : max_seq_len(max_len
 
 LayerKVCache::~LayerKVCache() { release(); }
 
+void LayerKVCache::drop_prompt_scratch() {
+    for (void *p : {split_ws_, copy_})
+        if (p) (void)hipFree(p);
+    split_ws_ = copy_ = nullptr;
+    split_ws_bytes_ = copy_bytes_ = 0;
+    split_tokens_ = copy_tokens_ = 0;
+    copy_upto_ = -1;
+}
+
 void LayerKVCache::release() {
+    drop_prompt_scratch();
     for (void *p : {k_codes_, v_codes_, (void *)k_scales_, (void *)v_scales_, (void *)seq_lens_dev_, workspace_})
         if (p) (void)hipFree(p);
     k_codes_ = v_codes_ = workspace_ = nullptr;
@@ -101,6 +113,7 @@ Status LayerKVCache::update(const void *new_keys, const void *new_values, int dt
         return err(HS_ERR_OVERFLOW, buf);
     }
     if (Status s = ensure_storage(batch, heads, dim); !s.ok()) return s;
+    copy_upto_ = -1;  // tokens written here are not in the prompt copy
     int rc;
     if (quant_type_ == KVQuantType::Fp8) {
         if (start_pos == 0) {  // fresh prompt: calibrate the per-(sequence, head) scales on it
@@ -159,6 +172,7 @@ Status LayerKVCache::decode_step(const void *q, const void *k_new, const void *v
         snprintf(buf, sizeof(buf), "Cache overflow: trying to cache 1 tokens starting at position %zu, but max_seq_len is %zu", seq_pos, max_seq_len);
         return err(HS_ERR_OVERFLOW, buf);
     }
+    copy_upto_ = -1;  // the new token is not in the prompt copy
     seq_pos += 1;  // the entry point writes the new token at seq_pos - 1 and attends seq_pos tokens
     Status s = ensure_scratch(hq, batch_, stream);
     int rc = HS_OK;
@@ -196,9 +210,48 @@ Status LayerKVCache::prefill(const void *q, const void *new_keys, const void *ne
         }
         rc = hs_prefill_attn_fp8(q, new_keys, new_values, (uint8_t *)k_codes_, (uint8_t *)v_codes_, k_scales_, v_scales_,
                                  &layout_, (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
+        copy_upto_ = -1;
     } else {
-        rc = hs_prefill_attn_int8(q, new_keys, new_values, (int8_t *)k_codes_, (int8_t *)v_codes_, k_scales_, v_scales_,
-                                  &layout_, (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
+        hs_kv_layout lay = layout_;
+        bool with_copy = false;
+        if (prompt_tokens_ > 0) {
+            // key-split workspace: sized for the longest chunk seen (grows like the decode workspace)
+            if (seq_len > split_tokens_) {
+                if (split_ws_) {
+                    if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) return hip_err(e, "waiting before the split workspace grows");
+                    (void)hipFree(split_ws_);
+                    split_ws_ = nullptr;
+                }
+                split_ws_bytes_ = hs_prefill_attn_split_workspace_bytes(batch, seq_len, hq, heads, dim);
+                split_tokens_ = 0;
+                if (split_ws_bytes_ > 0) {
+                    if (hipError_t e = hipMalloc(&split_ws_, split_ws_bytes_); e != hipSuccess) return hip_err(e, "allocating the split workspace");
+                    if (int rc2 = hs_prefill_attn_split_workspace_init(split_ws_, split_ws_bytes_, stream); rc2 != HS_OK) return from_abi(rc2);
+                    split_tokens_ = seq_len;
+                }
+            }
+            if (split_ws_) {
+                lay.prefill_split_workspace = split_ws_;
+                lay.prefill_split_workspace_bytes = (int64_t)split_ws_bytes_;
+            }
+            // the bf16 copy: begun by a chunk at position 0, extended by a chunk that starts where the copy ends
+            const size_t want = std::min(prompt_tokens_, max_seq_len);
+            if (dim == 128 && end_pos <= want && (start_pos == 0 || (copy_upto_ >= 0 && (size_t)copy_upto_ == start_pos))) {
+                if (!copy_) {
+                    copy_tokens_ = (int32_t)((want + 63) / 64 * 64);
+                    copy_bytes_ = hs_prefill_shadow_bytes(batch, heads, dim, copy_tokens_);
+                    if (hipError_t e = hipMalloc(&copy_, copy_bytes_); e != hipSuccess) return hip_err(e, "allocating the prompt copy");
+                    if (int rc2 = hs_prefill_shadow_init(copy_, copy_bytes_, stream); rc2 != HS_OK) return from_abi(rc2);
+                }
+                lay.prefill_shadow = copy_;
+                lay.prefill_shadow_bytes = (int64_t)copy_bytes_;
+                lay.prefill_shadow_tokens = copy_tokens_;
+                with_copy = true;
+            }
+        }
+        rc = hs_prefill_attn_int8(q, new_keys, new_values, (int8_t *)k_codes_, (int8_t *)v_codes_, k_scales_, v_scales_, &lay,
+                                  (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
+        copy_upto_ = rc == HS_OK && with_copy ? (int64_t)end_pos : -1;
     }
     if (rc != HS_OK) return from_abi(rc);
     seq_pos = end_pos;
@@ -215,6 +268,7 @@ void LayerKVCache::clear() {
 void LayerKVCache::truncate_to(size_t pos) {
     if (pos >= seq_pos) return;
     seq_pos = pos;
+    copy_upto_ = -1;  // (a prompt that continues from here starts its copy again at position 0 only)
 }
 
 size_t LayerKVCache::memory_usage() const { return k_codes_ ? bytes_ : 0; }

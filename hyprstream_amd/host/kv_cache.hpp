@@ -71,6 +71,17 @@ class LayerKVCache {
                    int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, size_t start_pos,
                    float softmax_scale, hs_stream_t stream = nullptr);
 
+    // Opt in to faster prompts: prefill() then offers the library a key-split workspace (calls with few query tiles,
+    // i.e. one sequence) and, for an int8 cache at head_dim 128, keeps a bf16 operand-order copy of the prompt's K/V
+    // that later chunks read instead of converting the codes (2 x the int8 bytes of the prompt, allocated at the
+    // first prefill after this call for max_prompt_tokens tokens, dropped by drop_prompt_scratch(), clear() and the
+    // destructor).  The copy follows the prompt: a chunk at start_pos 0 begins it, a chunk that starts where the
+    // last one ended extends it, and anything else written into the cache (update, decode_step) or taken out of it
+    // (truncate_to) retires it until the next prompt.  Results are those of prefill() without it within rounding.
+    void enable_prompt_scratch(size_t max_prompt_tokens) { prompt_tokens_ = max_prompt_tokens; }
+    void drop_prompt_scratch();
+    bool prompt_copy_active() const { return copy_upto_ >= 0; }  // for tests: the next chunk would read the copy
+
     void clear();
     void truncate_to(size_t pos);
     bool is_initialized() const { return k_codes_ != nullptr && seq_pos > 0; }
@@ -94,6 +105,12 @@ class LayerKVCache {
     hs_kv_layout layout_{};
     int32_t batch_ = 0, heads_ = 0, dim_ = 0;
     size_t bytes_ = 0;
+    // prompt scratch (enable_prompt_scratch)
+    size_t prompt_tokens_ = 0;       // 0 = not enabled
+    void *split_ws_ = nullptr, *copy_ = nullptr;
+    size_t split_ws_bytes_ = 0, copy_bytes_ = 0;
+    int32_t split_tokens_ = 0, copy_tokens_ = 0;
+    int64_t copy_upto_ = -1;         // tokens 0 .. copy_upto_ - 1 of the cache are in the copy; -1: it is not in step with the cache
 };
 
 }  // namespace hs

@@ -80,4 +80,12 @@ int hs_cache_prefill(hs_cache *c, const void *q, const void *k, const void *v, v
     return c->done(c->cache.prefill(q, k, v, out, batch, seq_len, hq, heads, dim, (size_t)start_pos, scale, stream));
 }
 
+void hs_cache_enable_prompt_scratch(hs_cache *c, int64_t max_prompt_tokens) {
+    if (c && max_prompt_tokens >= 0) c->cache.enable_prompt_scratch((size_t)max_prompt_tokens);
+}
+void hs_cache_drop_prompt_scratch(hs_cache *c) {
+    if (c) c->cache.drop_prompt_scratch();
+}
+int hs_cache_prompt_copy_active(const hs_cache *c) { return c && c->cache.prompt_copy_active() ? 1 : 0; }
+
 }  // extern "C"

@@ -16,7 +16,8 @@ EXPORTS = [
     "hs_cache_create", "hs_cache_destroy", "hs_cache_last_error", "hs_cache_update", "hs_cache_get_dense",
     "hs_cache_get_view", "hs_cache_seq_pos", "hs_cache_max_seq_len", "hs_cache_clear", "hs_cache_truncate_to",
     "hs_cache_is_initialized", "hs_cache_memory_usage", "hs_cache_quant_type", "hs_cache_decode_attention",
-    "hs_cache_decode_step", "hs_cache_prefill", "hs_paged_cache_prefill", "hs_kv_quant_canonical_str",
+    "hs_cache_decode_step", "hs_cache_prefill", "hs_cache_enable_prompt_scratch", "hs_cache_drop_prompt_scratch",
+    "hs_cache_prompt_copy_active", "hs_paged_cache_prefill", "hs_kv_quant_canonical_str",
     "hs_pool_create", "hs_pool_create_format", "hs_pool_quant_type", "hs_pool_destroy", "hs_pool_last_error", "hs_pool_allocate", "hs_pool_free", "hs_pool_owner_of",
     "hs_pool_used_blocks", "hs_pool_free_block_count", "hs_pool_total_blocks", "hs_pool_used_memory",
     "hs_paged_cache_create", "hs_paged_cache_destroy", "hs_paged_cache_last_error", "hs_paged_cache_update",
@@ -169,6 +170,17 @@ class LayerKVCache:
                                            k.shape[2], D, ctypes.c_int64(start_pos), ctypes.c_float(softmax_scale),
                                            hb._stream()))
         return out
+
+    def enable_prompt_scratch(self, max_prompt_tokens):
+        """Opt in to the key split of small prefill calls and to the bf16 copy of the prompt (hs_cache_enable_prompt_scratch)."""
+        lib().hs_cache_enable_prompt_scratch(self._h, ctypes.c_int64(max_prompt_tokens))
+
+    def drop_prompt_scratch(self):
+        lib().hs_cache_drop_prompt_scratch(self._h)
+
+    @property
+    def prompt_copy_active(self):
+        return bool(lib().hs_cache_prompt_copy_active(self._h))
 
 
 # ------------------------------------------------------------------------------------------- paged mode

@@ -100,6 +100,20 @@ HS_API int hs_cache_prefill(hs_cache *c, const void *q, const void *new_keys, co
                             int32_t batch, int32_t seq_len, int32_t num_q_heads, int32_t num_kv_heads,
                             int32_t head_dim, int64_t start_pos, float softmax_scale, hs_stream_t stream);
 
+/* Opt in to faster prompts through hs_cache_prefill (no counterpart in the reference, whose get() dequantizes the whole
+ * cache on every call, kv_cache.rs:1493-1560).  After this call prefill offers the library a key-split workspace (a
+ * chunk of ONE sequence is too few query tiles for the GPU: the keys of a tile are then split over workgroups) and,
+ * for an int8 cache at head_dim 128, keeps a bf16 copy of the prompt's dequantized K/V in the order the matrix
+ * instructions take it, which later chunks of the same prompt read instead of converting the codes in every
+ * workgroup.  The copy holds 2 x the int8 bytes of max_prompt_tokens tokens, is allocated by the first prefill after
+ * this call and freed by hs_cache_drop_prompt_scratch, hs_cache_clear and hs_cache_destroy.  It follows the prompt by
+ * itself: a chunk at start_pos 0 begins it, a chunk that starts where the last one ended extends it, anything else
+ * written into or cut from the cache (update, decode_step, truncate_to) retires it until the next prompt
+ * (hs_cache_prompt_copy_active reports which).  max_prompt_tokens = 0 turns it off again. */
+HS_API void hs_cache_enable_prompt_scratch(hs_cache *c, int64_t max_prompt_tokens);
+HS_API void hs_cache_drop_prompt_scratch(hs_cache *c);
+HS_API int hs_cache_prompt_copy_active(const hs_cache *c);
+
 /* ---- paged mode: shared block pool, per-sequence paged caches, ragged-batch decode step -----------------
  * BlockPool (kv_cache.rs:508-676): 256-token blocks, LIFO free list, every block tagged with its owner.
  * An owner is (kind, id, name) as CacheOwner (kv_cache.rs:49-82): kind 0 = Stateless(id), 1 = Session(name),

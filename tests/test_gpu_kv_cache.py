@@ -165,3 +165,57 @@ def test_decode_step_where_the_split_has_more_chunks_than_at_capacity():
     torch.cuda.synchronize()
     assert torch.equal(got, out)
     paged.close()
+
+
+def test_prompt_scratch_of_the_cache_object():
+    """hs_cache_enable_prompt_scratch: one sequence prefilled in 512-token chunks through the cache object with the
+    key-split workspace and the bf16 copy of the prompt.  Outputs agree with a cache object that has neither (within
+    the rounding of another summation order and operand format) and with the oracle; the codes and scales are the same
+    bits; the copy follows the prompt (active after each chunk in sequence), retires at a decode step, and a new
+    prompt at position 0 begins it again; the decode step after the prompt is the same either way."""
+    B, Hq, Hkv, D, C, T = 1, 32, 8, 128, 512, 2048
+    q, k, v = randn(31, B, T, Hq, D), randn(32, B, T, Hkv, D), randn(33, B, T, Hkv, D)
+    plain, fast = kc.LayerKVCache(T + 64, kc.INT8), kc.LayerKVCache(T + 64, kc.INT8)
+    fast.enable_prompt_scratch(T)
+    assert not fast.prompt_copy_active
+    outs = []
+    for lo in range(0, T, C):
+        o_plain = plain.prefill(q[:, lo:lo + C], k[:, lo:lo + C], v[:, lo:lo + C], lo, 1 / np.sqrt(D))
+        o_fast = fast.prefill(q[:, lo:lo + C], k[:, lo:lo + C], v[:, lo:lo + C], lo, 1 / np.sqrt(D))
+        torch.cuda.synchronize()
+        assert fast.prompt_copy_active and not plain.prompt_copy_active
+        d = (o_fast.float() - o_plain.float()).abs().max().item()
+        assert d <= 2.0 ** -6 * max(1.0, o_plain.float().abs().max().item()), (lo, d)
+        outs.append(o_fast)
+    kp, vp = plain.get(torch.float32)
+    kf, vf = fast.get(torch.float32)
+    assert torch.equal(kp, kf) and torch.equal(vp, vf)  # dequantized views of identical codes and scales
+    # last chunk against the oracle over the dequantized history
+    lo = T - C
+    kn, vn = k.float().cpu().numpy(), v.float().cpu().numpy()
+    k1 = np.concatenate([kp[:, :lo].cpu().numpy(), kn[:, lo:]], 1)
+    v1 = np.concatenate([vp[:, :lo].cpu().numpy(), vn[:, lo:]], 1)
+    want = oracle.prefill_attn(q[:, lo:].float().cpu().numpy(), k1, v1, None, None, oracle.FMT_DENSE, np.array([T], np.int32),
+                               1 / np.sqrt(D))
+    d = np.abs(outs[-1].float().cpu().numpy() - want)
+    assert d.max() < 2e-2 and d.mean() < 2e-3
+    # a decode step retires the copy; the step itself does not depend on it
+    qd, kd, vd = randn(34, B, Hq, D), randn(35, B, 1, Hkv, D), randn(36, B, 1, Hkv, D)
+    s_plain = plain.decode_step(qd, kd, vd, 1 / np.sqrt(D))
+    s_fast = fast.decode_step(qd, kd, vd, 1 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert torch.equal(s_plain, s_fast) and not fast.prompt_copy_active
+    # a chunk that does not start at 0 now reads the codes (and is then the plain call, bit for bit, split aside)
+    fast.truncate_to(C)
+    plain.truncate_to(C)
+    o_plain = plain.prefill(q[:, C:2 * C], k[:, C:2 * C], v[:, C:2 * C], C, 1 / np.sqrt(D))
+    o_fast = fast.prefill(q[:, C:2 * C], k[:, C:2 * C], v[:, C:2 * C], C, 1 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert not fast.prompt_copy_active
+    assert (o_fast.float() - o_plain.float()).abs().max().item() <= 2.0 ** -7 * max(1.0, o_plain.float().abs().max().item())
+    # a new prompt begins the copy again
+    fast.prefill(q[:, :C], k[:, :C], v[:, :C], 0, 1 / np.sqrt(D))
+    torch.cuda.synchronize()
+    assert fast.prompt_copy_active
+    fast.drop_prompt_scratch()
+    assert not fast.prompt_copy_active
