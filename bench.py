@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-KV decode-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-b1-shadow|c3-prologue|c3-shadow|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-layer|c5-prefill-recurrent]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c2-paged|c2-prologue|c2-ragged|c1|c4|c4-prologue|b1-32k|b4-16k|d256-int8|d256-fp8|d64-int8|c3|c3-prompt|c3-fp8|c3-d256|c3-d64|c3-b1|c3-b1-shadow|c3-prologue|c3-shadow|c3-fp8-shadow|c5-decode|c5-decode-layer|c5-decode-layer-3calls|c5-prefill|c5-prefill-norm|c5-prefill-layer|c5-prefill-recurrent]
 
 One "step" is one pass of the hot path over one batch: quantize-on-write of one new token per
 sequence into the int8 cache, then dequant-fused GQA decode attention over the whole context
@@ -239,7 +239,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         "data": "synthetic (seeded, generated on device)",
         "config": {"workload": "c3%s: chunked causal prefill B=%d T=4096 chunk=%d Hq=%d Hkv=%d D=%d, %s cache of earlier "
                                "chunks + own bf16 K/V, quantize-on-write, one layer"
-                               % ("-b1-shadow" if shadow and b1 else "-shadow" if shadow else "-prologue" if prologue else "-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
+                               % ("-b1-shadow" if shadow and b1 else "-fp8-shadow" if shadow and fp8 else "-shadow" if shadow else "-prologue" if prologue else "-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
                                   "fp8 e4m3fn" if fp8 else "int8"),
                    "algorithmic_flops_per_step": int(flops)},
         "tokens_per_s": B * T / (ms * 1e-3),
@@ -427,7 +427,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=200)  # the first launches after set-up run a few % slower (clocks settle)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-b1-shadow", "c3-prologue", "c3-shadow", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-layer", "c5-prefill-recurrent"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c3", "c3-prompt", "c3-fp8", "c3-d256", "c3-d64", "c3-b1", "c3-b1-shadow", "c3-prologue", "c3-shadow", "c3-fp8-shadow", "c5-decode", "c5-decode-layer", "c5-decode-layer-3calls", "c5-prefill", "c5-prefill-norm", "c5-prefill-layer", "c5-prefill-recurrent"])
     ap.add_argument("--copies", type=int, default=4, help="cache copies rotated through (defeats the last-level cache)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--block-tokens", type=int, default=256, help="tokens per pool block of the c2-paged workload")
@@ -473,7 +473,7 @@ def main():
         return
     if args.workload.startswith("c3"):
         return bench_prefill(args, torch, hb, wl, C=args.chunk_tokens or (4096 if args.workload == "c3-prompt" else 512),
-                             fp8=args.workload == "c3-fp8", d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload.startswith("c3-b1"), prologue=args.workload == "c3-prologue", shadow=args.workload.endswith("-shadow"))
+                             fp8=args.workload.startswith("c3-fp8"), d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload.startswith("c3-b1"), prologue=args.workload == "c3-prologue", shadow=args.workload.endswith("-shadow"))
     if args.workload.startswith("c5-decode-layer"):
         return bench_deltanet_layer(args, torch, hb, wl, fused=args.workload == "c5-decode-layer")
     if args.workload.startswith("c5"):

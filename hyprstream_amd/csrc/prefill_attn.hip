@@ -88,7 +88,7 @@ template <int D> struct alignas(16) HistTile {
 // buffers, three steps ahead, and are consumed by the bf16 products of the new-token phase.  head_dim 128, full width.
 template <int kPD, bool FP8, int kCols = 0, bool kWin = false, int kWaves = 8, bool kSplit = false, bool kShadow = false>
 __global__ __launch_bounds__(64 * kWaves, kWaves == 16 ? 4 : 2) void prefill_attn_kernel(PrefillArgs a) {
-    static_assert(!kShadow || (kPD == 128 && !kWin && kWaves == 8 && !FP8), "shadow history: head_dim 128, eight wavefronts, int8 cache, no window");
+    static_assert(!kShadow || (kPD == 128 && !kWin && kWaves == 8), "shadow history: head_dim 128, eight wavefronts, no window");
     static_assert(kWaves == 8 || (kWaves == 16 && kCols == 1 && kPD == 128), "sixteen wavefronts: one column block each, head_dim 128");
     static_assert(!kSplit || (!kWin && kWaves == 8), "key split: eight wavefronts, no window");
     constexpr int kNB = kCols ? kCols : PShape<kPD>::kNB, KG = PShape<kPD>::KG, VB = PShape<kPD>::VB, NC = PShape<kPD>::NC;
@@ -1232,10 +1232,10 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
     bool shadow_read = false;
     if (layout->prefill_shadow != nullptr) {
         const int tokens = layout->prefill_shadow_tokens;
-        const bool can_append = D == 128 && !fp8;
+        const bool can_append = D == 128;
         if (!can_append) {
             if (hist_len > 0)
-                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow serves head_dim 128 over an int8 cache; this call could not append to it");
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow serves head_dim 128; this call could not append to it");
         } else {
             if (tokens <= 0 || (tokens & 63) != 0 || (int64_t)hist_len + S > tokens)
                 return fail(HS_ERR_INVALID_ARGUMENT, "prefill_shadow_tokens %d must be a multiple of 64 and hold hist_len + S = %lld tokens",
@@ -1279,13 +1279,19 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
         }                                                                                                   \
     } while (0)
     if (shadow_read) {
-        if (a.nsplit > 1) {
-            if (narrow) prefill_attn_kernel<128, false, 1, false, 8, true, true><<<grid, 512, 0, st>>>(a);
-            else prefill_attn_kernel<128, false, 0, false, 8, true, true><<<grid, 512, 0, st>>>(a);
-        } else {
-            if (narrow) prefill_attn_kernel<128, false, 1, false, 8, false, true><<<grid, 512, 0, st>>>(a);
-            else prefill_attn_kernel<128, false, 0, false, 8, false, true><<<grid, 512, 0, st>>>(a);
-        }
+#define HS_PREFILL_COPY(F8)                                                                                  \
+    do {                                                                                                     \
+        if (a.nsplit > 1) {                                                                                  \
+            if (narrow) prefill_attn_kernel<128, F8, 1, false, 8, true, true><<<grid, 512, 0, st>>>(a);       \
+            else prefill_attn_kernel<128, F8, 0, false, 8, true, true><<<grid, 512, 0, st>>>(a);              \
+        } else {                                                                                             \
+            if (narrow) prefill_attn_kernel<128, F8, 1, false, 8, false, true><<<grid, 512, 0, st>>>(a);      \
+            else prefill_attn_kernel<128, F8, 0, false, 8, false, true><<<grid, 512, 0, st>>>(a);             \
+        }                                                                                                    \
+    } while (0)
+        if (fp8) HS_PREFILL_COPY(true);
+        else HS_PREFILL_COPY(false);
+#undef HS_PREFILL_COPY
     } else if (a.nsplit > 1) {
 #define HS_PREFILL_SPLIT(DD, CC)                                                                     \
     do {                                                                                             \

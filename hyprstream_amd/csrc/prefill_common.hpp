@@ -123,7 +123,7 @@ __device__ __forceinline__ void write_new_rows(const PrefillArgs &a, int b, int 
                         }
                     }
                 }
-                if constexpr (!FP8 && kRow == 128) {
+                if constexpr (kRow == 128) {
                     if (a.shadow != nullptr && live) {
                         // the dequantized row (code * scale, rounded to bf16: what the reference's get() hands to its
                         // attention) into the step image of its position; `packed` holds the codes
@@ -131,8 +131,14 @@ __device__ __forceinline__ void write_new_rows(const PrefillArgs &a, int b, int 
                         uint16_t *img = a.shadow + (((int64_t)b * a.Hkv + kvh) * a.shadow_steps + (pos >> 6)) * (kShadowStepBytes / 2) +
                                         ((pos >> 5) & 1) * (kShadowStepBytes / 4);  // this half: K blocks [2 KG][512 el], then V^T blocks [VB][512 el]
                         float dq[8];
+                        if constexpr (FP8) {
+                            const half8 hv = e4m3x8_to_f16_div256(packed[0], packed[1]);  // exact: the codes' values / 256
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) dq[e] = (float)(int8_t)(packed[e >> 2] >> (8 * (e & 3))) * sc;
+                            for (int e = 0; e < 8; ++e) dq[e] = (float)hv[e] * 256.0f * sc;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) dq[e] = (float)(int8_t)(packed[e >> 2] >> (8 * (e & 3))) * sc;
+                        }
                         if (which == 0) {
                             // K block (tile u = kk / 16, d-group j): lane (li = key, lq) holds d = 32 lq + 8 j ..; this lane has d = 8 sub ..
                             const int blk = 4 * (kk >> 4) + (sub & 3), ln = (sub >> 2) * 16 + (kk & 15);

@@ -125,7 +125,7 @@ typedef struct hs_kv_layout {
     void *prefill_shadow;
     int64_t prefill_shadow_bytes;
     int32_t prefill_shadow_tokens;
-    int32_t reserved1;          /* prefill only, optional, head_dim 128 over an int8 cache: a bf16 copy of the prompt's
+    int32_t reserved1;          /* prefill only, optional, head_dim 128 (int8 or fp8 cache): a bf16 copy of the prompt's
                                    DEQUANTIZED K/V (code * scale, the values the reference's get() hands to its
                                    attention, kv_cache.rs:1493-1560) in the order the matrix instructions take them,
                                    kept by the caller for as long as one prompt is being prefilled into one layer's
@@ -138,10 +138,9 @@ typedef struct hs_kv_layout {
                                    a multiple of 64 and >= hist_len + S; every token below hist_len must have been
                                    appended by earlier prefill calls with the same copy and the same B, Hkv (tokens
                                    written by decode steps or by hs_kv_quantize_* are not in it: leave the field NULL
-                                   for such calls).  NULL = none.  Calls that cannot use it (fp8, other head_dim, a
-                                   window, the hinted or split instances) still append when they can and otherwise
-                                   ignore it -- except that a call WITH history that cannot append (fp8, head_dim
-                                   != 128) is refused rather than leaving a hole. */
+                                   for such calls).  NULL = none.  Calls that cannot read it (a window, rows at different
+                                   positions, the 32 and 16 width hints) still append; a call WITH history at another
+                                   head_dim is refused rather than leaving a hole. */
 } hs_kv_layout;
 
 /* Message of the last failing call on this thread ("" if none). */

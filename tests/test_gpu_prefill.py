@@ -757,3 +757,42 @@ def test_shadow_over_a_paged_pool_and_random_chunkings():
         assert torch.equal(pools[0][0], pools[1][0]) and torch.equal(pools[0][1], pools[1][1])
         d = (outs["paged+copy"].float() - outs["paged"].float()).abs().max().item()
         assert d <= 2.0 ** -6 * max(1.0, outs["paged"].float().abs().max().item()), (cuts, d)
+
+
+@pytest.mark.parametrize("variant", ["full", "split2-half"])
+def test_bf16_shadow_over_an_fp8_cache(variant):
+    """The copy holds the dequantized e4m3fn codes (code value x head scale, rounded to bf16): a prompt in uneven chunks
+    over an FP8 cache with and without the copy -- outputs within the operand rounding of each other and inside the
+    oracle's bar, the cache the same bits."""
+    _fixes_its_own_instance()
+    B, Hq, Hkv, D = 2, 8, 2, 128
+    chunks = (150, 70, 200, 64)
+    T = sum(chunks)
+    q, k, v = make(8500, B, T, Hq, Hkv, D, 0.5)
+    dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
+    cols = 128 if variant.endswith("half") else 256
+    runs = int(variant[5]) if variant.startswith("split") else 1
+    shadow = hb.prefill_shadow(B, Hkv, D, T)
+    with_copy, without = DeviceCache(B, Hkv, T, D, fp8=True), DeviceCache(B, Hkv, T, D, fp8=True)
+    for c in (with_copy, without):
+        hb.kv_fp8_calibrate(dev(k[:, :chunks[0]]), dev(v[:, :chunks[0]]), c.k_scales, c.v_scales)
+    lo = 0
+    for n in chunks:
+        hi = lo + n
+        outs = []
+        for c, sh in ((without, None), (with_copy, shadow)):
+            out = torch.full((B, n, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+            ws = hb.prefill_split_workspace(B, n, Hq, Hkv, D) if runs > 1 else None
+            hb.prefill_attn(dev(q[:, lo:hi]), dev(k[:, lo:hi]), dev(v[:, lo:hi]), c.k_codes, c.v_codes, c.k_scales, c.v_scales,
+                            c.layout, lo, out, 1.0 / np.sqrt(D), True, fp8=True, columns=cols, key_splits=runs,
+                            split_workspace=ws, shadow=sh)
+            torch.cuda.synchronize()
+            outs.append(out.float().cpu().numpy())
+        assert np.isfinite(outs[1]).all(), (lo, hi)
+        assert np.abs(outs[1] - outs[0]).max() <= 2.0 ** -6 * max(1.0, np.abs(outs[0]).max()), (lo, hi)
+        if lo > 0:
+            kc, vc, ks, vs = without.canonical(lo)
+            want = oracle_prefill(q[:, lo:hi], oracle.dequant_fp8(kc, ks), oracle.dequant_fp8(vc, vs), k[:, lo:hi], v[:, lo:hi])
+            compare(outs[1], want, "fp8 shadow history %d..%d" % (lo, hi))
+        lo = hi
+    assert torch.equal(with_copy.k_codes, without.k_codes) and torch.equal(with_copy.v_codes, without.v_codes)
