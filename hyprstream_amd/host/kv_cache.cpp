@@ -203,56 +203,55 @@ Status LayerKVCache::prefill(const void *q, const void *new_keys, const void *ne
     if (start_pos > seq_pos) return err(HS_ERR_INVALID_ARGUMENT, "start_pos is past the cached tokens");
     if (Status s = ensure_storage(batch, heads, dim); !s.ok()) return s;
     int rc;
+    hs_kv_layout lay = layout_;
+    bool with_copy = false;
+    if (prompt_tokens_ > 0) {
+        // key-split workspace: sized for the longest chunk seen (grows like the decode workspace)
+        if (seq_len > split_tokens_) {
+            if (split_ws_) {
+                if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) return hip_err(e, "waiting before the split workspace grows");
+                (void)hipFree(split_ws_);
+                split_ws_ = nullptr;
+            }
+            split_ws_bytes_ = hs_prefill_attn_split_workspace_bytes(batch, seq_len, hq, heads, dim);
+            split_tokens_ = 0;
+            if (split_ws_bytes_ > 0) {
+                if (hipError_t e = hipMalloc(&split_ws_, split_ws_bytes_); e != hipSuccess) return hip_err(e, "allocating the split workspace");
+                if (int rc2 = hs_prefill_attn_split_workspace_init(split_ws_, split_ws_bytes_, stream); rc2 != HS_OK) return from_abi(rc2);
+                split_tokens_ = seq_len;
+            }
+        }
+        if (split_ws_) {
+            lay.prefill_split_workspace = split_ws_;
+            lay.prefill_split_workspace_bytes = (int64_t)split_ws_bytes_;
+        }
+        // the bf16 copy: begun by a chunk at position 0, extended by a chunk that starts where the copy ends
+        const size_t want = std::min(prompt_tokens_, max_seq_len);
+        if (dim == 128 && end_pos <= want && (start_pos == 0 || (copy_upto_ >= 0 && (size_t)copy_upto_ == start_pos))) {
+            if (!copy_) {
+                copy_tokens_ = (int32_t)((want + 63) / 64 * 64);
+                copy_bytes_ = hs_prefill_shadow_bytes(batch, heads, dim, copy_tokens_);
+                if (hipError_t e = hipMalloc(&copy_, copy_bytes_); e != hipSuccess) return hip_err(e, "allocating the prompt copy");
+                if (int rc2 = hs_prefill_shadow_init(copy_, copy_bytes_, stream); rc2 != HS_OK) return from_abi(rc2);
+            }
+            lay.prefill_shadow = copy_;
+            lay.prefill_shadow_bytes = (int64_t)copy_bytes_;
+            lay.prefill_shadow_tokens = copy_tokens_;
+            with_copy = true;
+        }
+    }
     if (quant_type_ == KVQuantType::Fp8) {
         if (start_pos == 0) {  // fresh prompt: calibrate the per-(sequence, head) scales on it, as update() does
             rc = hs_kv_fp8_calibrate(new_keys, new_values, HS_BF16, k_scales_, v_scales_, batch, seq_len, heads, dim, stream);
             if (rc != HS_OK) return from_abi(rc);
         }
-        rc = hs_prefill_attn_fp8(q, new_keys, new_values, (uint8_t *)k_codes_, (uint8_t *)v_codes_, k_scales_, v_scales_,
-                                 &layout_, (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
-        copy_upto_ = -1;
+        rc = hs_prefill_attn_fp8(q, new_keys, new_values, (uint8_t *)k_codes_, (uint8_t *)v_codes_, k_scales_, v_scales_, &lay,
+                                 (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
     } else {
-        hs_kv_layout lay = layout_;
-        bool with_copy = false;
-        if (prompt_tokens_ > 0) {
-            // key-split workspace: sized for the longest chunk seen (grows like the decode workspace)
-            if (seq_len > split_tokens_) {
-                if (split_ws_) {
-                    if (hipError_t e = hipDeviceSynchronize(); e != hipSuccess) return hip_err(e, "waiting before the split workspace grows");
-                    (void)hipFree(split_ws_);
-                    split_ws_ = nullptr;
-                }
-                split_ws_bytes_ = hs_prefill_attn_split_workspace_bytes(batch, seq_len, hq, heads, dim);
-                split_tokens_ = 0;
-                if (split_ws_bytes_ > 0) {
-                    if (hipError_t e = hipMalloc(&split_ws_, split_ws_bytes_); e != hipSuccess) return hip_err(e, "allocating the split workspace");
-                    if (int rc2 = hs_prefill_attn_split_workspace_init(split_ws_, split_ws_bytes_, stream); rc2 != HS_OK) return from_abi(rc2);
-                    split_tokens_ = seq_len;
-                }
-            }
-            if (split_ws_) {
-                lay.prefill_split_workspace = split_ws_;
-                lay.prefill_split_workspace_bytes = (int64_t)split_ws_bytes_;
-            }
-            // the bf16 copy: begun by a chunk at position 0, extended by a chunk that starts where the copy ends
-            const size_t want = std::min(prompt_tokens_, max_seq_len);
-            if (dim == 128 && end_pos <= want && (start_pos == 0 || (copy_upto_ >= 0 && (size_t)copy_upto_ == start_pos))) {
-                if (!copy_) {
-                    copy_tokens_ = (int32_t)((want + 63) / 64 * 64);
-                    copy_bytes_ = hs_prefill_shadow_bytes(batch, heads, dim, copy_tokens_);
-                    if (hipError_t e = hipMalloc(&copy_, copy_bytes_); e != hipSuccess) return hip_err(e, "allocating the prompt copy");
-                    if (int rc2 = hs_prefill_shadow_init(copy_, copy_bytes_, stream); rc2 != HS_OK) return from_abi(rc2);
-                }
-                lay.prefill_shadow = copy_;
-                lay.prefill_shadow_bytes = (int64_t)copy_bytes_;
-                lay.prefill_shadow_tokens = copy_tokens_;
-                with_copy = true;
-            }
-        }
         rc = hs_prefill_attn_int8(q, new_keys, new_values, (int8_t *)k_codes_, (int8_t *)v_codes_, k_scales_, v_scales_, &lay,
                                   (int32_t)start_pos, out, batch, seq_len, hq, heads, dim, scale, 1, stream);
-        copy_upto_ = rc == HS_OK && with_copy ? (int64_t)end_pos : -1;
     }
+    copy_upto_ = rc == HS_OK && with_copy ? (int64_t)end_pos : -1;
     if (rc != HS_OK) return from_abi(rc);
     seq_pos = end_pos;
     return {};

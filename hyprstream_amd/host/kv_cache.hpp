@@ -72,7 +72,7 @@ class LayerKVCache {
                    float softmax_scale, hs_stream_t stream = nullptr);
 
     // Opt in to faster prompts: prefill() then offers the library a key-split workspace (calls with few query tiles,
-    // i.e. one sequence) and, for an int8 cache at head_dim 128, keeps a bf16 operand-order copy of the prompt's K/V
+    // i.e. one sequence) and, at head_dim 128, keeps a bf16 operand-order copy of the prompt's K/V
     // that later chunks read instead of converting the codes (2 x the int8 bytes of the prompt, allocated at the
     // first prefill after this call for max_prompt_tokens tokens, dropped by drop_prompt_scratch(), clear() and the
     // destructor).  The copy follows the prompt: a chunk at start_pos 0 begins it, a chunk that starts where the

@@ -103,7 +103,7 @@ HS_API int hs_cache_prefill(hs_cache *c, const void *q, const void *new_keys, co
 /* Opt in to faster prompts through hs_cache_prefill (no counterpart in the reference, whose get() dequantizes the whole
  * cache on every call, kv_cache.rs:1493-1560).  After this call prefill offers the library a key-split workspace (a
  * chunk of ONE sequence is too few query tiles for the GPU: the keys of a tile are then split over workgroups) and,
- * for an int8 cache at head_dim 128 (the mirror's FP8 caches take the plain path), keeps a bf16 copy of the prompt's dequantized K/V in the order the matrix
+ * at head_dim 128, keeps a bf16 copy of the prompt's dequantized K/V in the order the matrix
  * instructions take it, which later chunks of the same prompt read instead of converting the codes in every
  * workgroup.  The copy holds 2 x the int8 bytes of max_prompt_tokens tokens, is allocated by the first prefill after
  * this call and freed by hs_cache_drop_prompt_scratch, hs_cache_clear and hs_cache_destroy.  It follows the prompt by

@@ -167,7 +167,8 @@ def test_decode_step_where_the_split_has_more_chunks_than_at_capacity():
     paged.close()
 
 
-def test_prompt_scratch_of_the_cache_object():
+@pytest.mark.parametrize("fmt", ["int8", "fp8"])
+def test_prompt_scratch_of_the_cache_object(fmt):
     """hs_cache_enable_prompt_scratch: one sequence prefilled in 512-token chunks through the cache object with the
     key-split workspace and the bf16 copy of the prompt.  Outputs agree with a cache object that has neither (within
     the rounding of another summation order and operand format) and with the oracle; the codes and scales are the same
@@ -175,7 +176,8 @@ def test_prompt_scratch_of_the_cache_object():
     prompt at position 0 begins it again; the decode step after the prompt is the same either way."""
     B, Hq, Hkv, D, C, T = 1, 32, 8, 128, 512, 2048
     q, k, v = randn(31, B, T, Hq, D), randn(32, B, T, Hkv, D), randn(33, B, T, Hkv, D)
-    plain, fast = kc.LayerKVCache(T + 64, kc.INT8), kc.LayerKVCache(T + 64, kc.INT8)
+    qt = kc.INT8 if fmt == "int8" else kc.FP8
+    plain, fast = kc.LayerKVCache(T + 64, qt), kc.LayerKVCache(T + 64, qt)
     fast.enable_prompt_scratch(T)
     assert not fast.prompt_copy_active
     outs = []
