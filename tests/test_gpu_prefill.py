@@ -796,3 +796,38 @@ def test_bf16_shadow_over_an_fp8_cache(variant):
             compare(outs[1], want, "fp8 shadow history %d..%d" % (lo, hi))
         lo = hi
     assert torch.equal(with_copy.k_codes, without.k_codes) and torch.equal(with_copy.v_codes, without.v_codes)
+
+
+@pytest.mark.parametrize("kmag,vmag", [(1e-5, 1e5), (1e5, 1e-5), (3e-7, 3e-7), (1.0, 1e9)])
+def test_shadow_history_magnitude_ranges(kmag, vmag):
+    """test_history_magnitude_ranges with the history read from the bf16 copy: bf16 has fp32's exponent range, so caches
+    that are tiny or huge as a whole need no reference scale there -- and a row far above its head's other rows, which
+    saturates the fp16 operands of the code path, does not saturate here."""
+    _fixes_its_own_instance()
+    B, Hq, Hkv, hist, S, D = 2, 8, 2, 150, 70, 128
+    qh, kh, vh = make(90, B, hist, Hq, Hkv)
+    q, k, v = make(91, B, S, Hq, Hkv)
+    mags = np.array([[kmag, vmag], [vmag, kmag]], np.float32)
+    kh, vh = bf16r(kh * mags[:, 0, None, None, None]), bf16r(vh * mags[:, 1, None, None, None])
+    vh[0, 100] *= 2.0 ** 13  # one cached row 2^13 above its head's first tokens: beyond the fp16 window of the code path
+    vh = bf16r(vh)
+    k, v = bf16r(k * mags[:, 0, None, None, None]), bf16r(v * mags[:, 1, None, None, None])
+    q = bf16r(q / np.maximum(mags[:, 0, None, None, None], 1e-3))
+    dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
+    c = DeviceCache(B, Hkv, hist + S, D)
+    shadow = hb.prefill_shadow(B, Hkv, D, hist + S)
+    o0 = torch.empty(B, hist, Hq, D, dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(dev(qh), dev(kh), dev(vh), c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, 0, o0, 1.0 / np.sqrt(D), True,
+                    columns=256, key_splits=1, shadow=shadow)
+    out = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(dev(q), dev(k), dev(v), c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, hist, out, 1.0 / np.sqrt(D), True,
+                    columns=256, key_splits=1, shadow=shadow)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    kc, vc, ks, vs = c.canonical(hist)
+    want = oracle_prefill(q, bf16r(oracle.dequant_int8(kc, ks)), bf16r(oracle.dequant_int8(vc, vs)), k, v)  # the copy's values
+    assert np.isfinite(got).all()
+    for b in range(B):
+        top = np.abs(want[b]).max()
+        d = np.abs(got[b] - want[b])
+        assert d.max() < 2e-2 * top and d.mean() < 2e-3 * top, (b, d.max() / top, d.mean() / top)
