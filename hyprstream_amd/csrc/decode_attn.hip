@@ -217,22 +217,34 @@ __device__ __forceinline__ void rope_q_crosslane(float (&qf)[8 * NJ], const uint
         }
     }
 }
-template <int NJ>
-__device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq, int rd) {
-    if constexpr (NJ >= 4) {
-        if (rd == 32 * NJ) return rope_q_inlane<NJ, NJ>(qf, sin_row, cos_row, lq);
+// Normalises the 8 elements d0 .. d0 + 7 of a head's row in place, given the row's reciprocal root.
+__device__ __forceinline__ void norm_q_group(float (&x)[8], const NormSpec &n, int head, int d0, float rrms) {
+#pragma clang fp contract(off)
+    float w[8];
+    if (n.kind == 1) {
+        const u32x4 ww = *(const u32x4 *)((const uint16_t *)n.weight + (int64_t)head * n.head_stride + d0);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            w[2 * e] = __uint_as_float(ww[e] << 16);
+            w[2 * e + 1] = __uint_as_float(ww[e] & 0xffff0000u);
+        }
+    } else {
+        const float *wp = (const float *)n.weight + (int64_t)head * n.head_stride + d0;
+        const float4v w0 = *(const float4v *)wp, w1 = *(const float4v *)(wp + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            w[e] = w0[e];
+            w[4 + e] = w1[e];
+        }
     }
-    if constexpr (NJ == 8) {
-        if (rd == 128) return rope_q_inlane<NJ, 4>(qf, sin_row, cos_row, lq);
-    }
-    if (rd == 64) return rope_q_crosslane<NJ, 32>(qf, sin_row, cos_row, lq);
-    if (rd == 32) return rope_q_crosslane<NJ, 16>(qf, sin_row, cos_row, lq);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = norm_apply(x[e], w[e], rrms, HS_BF16, n.kind);
 }
 
 // Per-head QK-norm of the query elements a lane holds (bf16 tensor; NormSpec in quant_device.hpp).  The four lanes
-// lq = 0..3 of a head share its sum of squares.
+// lq = 0..3 of a head share its sum of squares.  Returns the row's reciprocal root.
 template <int NJ>
-__device__ __forceinline__ void norm_q(float (&qf)[8 * NJ], const NormSpec &n, int head, int lq, int D) {
+__device__ __forceinline__ float norm_q(float (&qf)[8 * NJ], const NormSpec &n, int head, int lq, int D) {
 #pragma clang fp contract(off)
     double ss = 0.0;
 #pragma unroll
@@ -243,26 +255,62 @@ __device__ __forceinline__ void norm_q(float (&qf)[8 * NJ], const NormSpec &n, i
 #pragma unroll
     for (int i = 0; i < NJ; ++i) {
         const int d0 = NJ == 2 ? 16 * lq + 8 * i : 64 * (i >> 1) + 16 * lq + 8 * (i & 1);
-        float w[8];
-        if (n.kind == 1) {
-            const u32x4 ww = *(const u32x4 *)((const uint16_t *)n.weight + (int64_t)head * n.head_stride + d0);
+        float x[8];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                w[2 * e] = __uint_as_float(ww[e] << 16);
-                w[2 * e + 1] = __uint_as_float(ww[e] & 0xffff0000u);
-            }
-        } else {
-            const float *wp = (const float *)n.weight + (int64_t)head * n.head_stride + d0;
-            const float4v w0 = *(const float4v *)wp, w1 = *(const float4v *)(wp + 4);
+        for (int e = 0; e < 8; ++e) x[e] = qf[8 * i + e];
+        norm_q_group(x, n, head, d0, rrms);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                w[e] = w0[e];
-                w[4 + e] = w1[e];
-            }
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) qf[8 * i + e] = norm_apply(qf[8 * i + e], w[e], rrms, HS_BF16, n.kind);
+        for (int e = 0; e < 8; ++e) qf[8 * i + e] = x[e];
     }
+    return rrms;
+}
+
+// Any other rotated length (a multiple of 16): the 8 partners of a lane's 8 elements are 8 consecutive elements of the
+// row, which the lane reads from the q tensor and normalises itself (the norm is elementwise once the row's reciprocal
+// root is known) instead of finding the lane and register that hold them.
+template <int NJ>
+__device__ __forceinline__ void rope_q_general(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq, int rd,
+                                               const uint16_t *q_row, const NormSpec &n, int head, float rrms) {
+#pragma clang fp contract(off)
+    auto rb = [](float v) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); };
+    const int half = rd / 2;
+#pragma unroll
+    for (int i = 0; i < NJ; ++i) {
+        const int d0 = NJ == 2 ? 16 * lq + 8 * i : 64 * (i >> 1) + 16 * lq + 8 * (i & 1);
+        if (d0 >= rd) continue;
+        const bool upper = d0 >= half;  // this lane holds x2 of its pairs
+        const int pd0 = upper ? d0 - half : d0 + half, j0 = upper ? pd0 : d0;
+        const u32x4 pw = *(const u32x4 *)(q_row + pd0);
+        float other[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            other[2 * e] = __uint_as_float(pw[e] << 16);
+            other[2 * e + 1] = __uint_as_float(pw[e] & 0xffff0000u);
+        }
+        if (n.kind != 0) norm_q_group(other, n, head, pd0, rrms);
+        const u32x4 sw = *(const u32x4 *)(sin_row + j0), cw = *(const u32x4 *)(cos_row + j0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float sn = (e & 1) ? __uint_as_float(sw[e >> 1] & 0xffff0000u) : __uint_as_float(sw[e >> 1] << 16);
+            const float cs = (e & 1) ? __uint_as_float(cw[e >> 1] & 0xffff0000u) : __uint_as_float(cw[e >> 1] << 16);
+            const float mine = qf[8 * i + e];
+            qf[8 * i + e] = upper ? rb(rb(other[e] * sn) + rb(mine * cs)) : rb(rb(mine * cs) - rb(other[e] * sn));
+        }
+    }
+}
+
+template <int NJ>
+__device__ __forceinline__ void rope_rotate_q(float (&qf)[8 * NJ], const uint16_t *sin_row, const uint16_t *cos_row, int lq, int rd,
+                                              const uint16_t *q_row, const NormSpec &n, int head, float rrms) {
+    if constexpr (NJ >= 4) {
+        if (rd == 32 * NJ) return rope_q_inlane<NJ, NJ>(qf, sin_row, cos_row, lq);
+    }
+    if constexpr (NJ == 8) {
+        if (rd == 128) return rope_q_inlane<NJ, 4>(qf, sin_row, cos_row, lq);
+    }
+    if (rd == 64) return rope_q_crosslane<NJ, 32>(qf, sin_row, cos_row, lq);
+    if (rd == 32) return rope_q_crosslane<NJ, 16>(qf, sin_row, cos_row, lq);
+    rope_q_general<NJ>(qf, sin_row, cos_row, lq, rd, q_row, n, head, rrms);
 }
 
 template <int D>
@@ -533,11 +581,13 @@ __global__ __launch_bounds__(256, 2) void decode_attn_kernel(DecodeArgs a_in) {
                 }
             }
             if (ROPE) {  // the step's prologue on q: QK-norm, then the rotation
-                if (a.qnorm.kind != 0) norm_q<NJ>(qf, a.qnorm, h * G + li, lq, kD);
+                float rrms = 0.0f;
+                if (a.qnorm.kind != 0) rrms = norm_q<NJ>(qf, a.qnorm, h * G + li, lq, kD);
                 if (a.rope_sin != nullptr) {
                     const int p = min(max(a.seq_lens[b] - 1, 0), a.rope_len - 1);  // the query is the newest token
                     const int half = a.rotary_dim / 2;
-                    rope_rotate_q<NJ>(qf, a.rope_sin + (int64_t)p * half, a.rope_cos + (int64_t)p * half, lq, a.rotary_dim);
+                    rope_rotate_q<NJ>(qf, a.rope_sin + (int64_t)p * half, a.rope_cos + (int64_t)p * half, lq, a.rotary_dim,
+                                      qp - 16 * lq, a.qnorm, h * G + li, rrms);
                 }
             }
 #pragma unroll
@@ -953,10 +1003,8 @@ static int launch_decode(bool fp8, int phases, const NewToken &nt, const void *q
             return fail(HS_ERR_INVALID_ARGUMENT, "the rotary decode step takes a bf16 new token");
     }
     const int rd = nt.rotary_dim > 0 ? nt.rotary_dim : D;
-    if (nt.rope_sin && !(rd == D || ((rd == 32 || rd == 64 || rd == 128) && rd < D)))
-        return fail(HS_ERR_INVALID_ARGUMENT,
-                    "the fused decode step rotates head_dim, 128, 64 or 32 leading elements, not %d: run "
-                    "hs_qk_prologue_apply and hs_decode_step_int8 instead", rd);
+    if (nt.rope_sin && (rd <= 0 || rd > D || (rd % 16) != 0))
+        return fail(HS_ERR_INVALID_ARGUMENT, "rotary_dim %d must be a multiple of 16 in (0, head_dim %d]", rd, D);
     if ((nt.qnorm.kind != 0 || nt.knorm.kind != 0) && (!nt.k_src || nt.dtype != HS_BF16))
         return fail(HS_ERR_INVALID_ARGUMENT, "the decode step with a QK-norm takes a bf16 new token");
     a.nt.rope_sin = nt.rope_sin; a.nt.rope_cos = nt.rope_cos; a.nt.rope_len = nt.rope_len; a.nt.rotary_dim = rd;

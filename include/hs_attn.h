@@ -313,9 +313,9 @@ HS_API int hs_decode_step_int8_rope(const void *q, const void *k_new, const void
                                int32_t B, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_seq_len,
                                float softmax_scale, hs_stream_t stream);
 /* The step with the whole prologue inside the launch: QK-norm of q and k_new, then their rotation (hs_qk_prologue above;
- * q [B, Hq, D], k_new [B, 1, Hkv, D], v_new in bf16 as projected; table row = seq_lens[b] - 1).  Rotated parts the
- * kernel serves: rotary_dim = head_dim, or 128, 64, 32 leading elements (Qwen3.5: 64 of 256); anything else is
- * HS_ERR_INVALID_ARGUMENT (run hs_qk_prologue_apply + hs_decode_step_int8).  The norm weights and the rotary tables
+ * q [B, Hq, D], k_new [B, 1, Hkv, D], v_new in bf16 as projected; table row = seq_lens[b] - 1).  rotary_dim is any
+ * multiple of 16 up to head_dim, as for hs_qk_prologue_apply (head_dim, 128, 64 and 32 pair their elements between the
+ * lanes that hold them; other lengths read the partners from q again).  The norm weights and the rotary tables
  * must be 16-byte aligned here (the launch reads them 16 bytes at a time; hs_qk_prologue_apply takes any alignment),
  * else HS_ERR_INVALID_ARGUMENT.  Results equal those calls' bit for bit. */
 HS_API int hs_decode_step_int8_prologue(const void *q, const void *k_new, const void *v_new, const hs_qk_prologue *prologue,

@@ -163,7 +163,11 @@ def test_quantize_with_prologue_bit_exact(kind, D, rd):
 
 @pytest.mark.parametrize("kind,D,rd", [(hb.QKNORM_LLAMA, 128, 128), (hb.QKNORM_QWEN35, 256, 64), (hb.QKNORM_QWEN35, 256, 128),
                                        (hb.QKNORM_LLAMA, 64, 64), (hb.QKNORM_NONE, 128, 32), (hb.QKNORM_LLAMA, 256, 256),
-                                       (hb.QKNORM_QWEN35, 128, 0)])
+                                       (hb.QKNORM_QWEN35, 128, 0),
+                                       # lengths with no lane pattern of their own: partners re-read from the q tensor
+                                       (hb.QKNORM_LLAMA, 128, 96), (hb.QKNORM_QWEN35, 128, 16), (hb.QKNORM_NONE, 128, 48),
+                                       (hb.QKNORM_QWEN35, 256, 192), (hb.QKNORM_LLAMA, 256, 80), (hb.QKNORM_LLAMA, 64, 48),
+                                       (hb.QKNORM_NONE, 64, 16), (hb.QKNORM_QWEN35, 64, 32)])
 @pytest.mark.parametrize("lens", [[260, 260, 260], [1, 129, 700]])
 def test_decode_step_with_prologue_matches_unfused_and_oracle(lens, kind, D, rd):
     """rd = 0 here means no rotation at all (norm only)."""
@@ -222,7 +226,8 @@ def test_decode_step_with_prologue_matches_unfused_and_oracle(lens, kind, D, rd)
 
 
 @pytest.mark.parametrize("kind,D,rd", [(hb.QKNORM_LLAMA, 128, 128), (hb.QKNORM_QWEN35, 256, 64), (hb.QKNORM_LLAMA, 64, 64),
-                                       (hb.QKNORM_NONE, 128, 32), (hb.QKNORM_QWEN35, 128, 0)])
+                                       (hb.QKNORM_NONE, 128, 32), (hb.QKNORM_QWEN35, 128, 0), (hb.QKNORM_LLAMA, 128, 96),
+                                       (hb.QKNORM_QWEN35, 256, 112)])
 @pytest.mark.parametrize("lens", [[260, 260, 260], [1, 129, 700]])
 def test_fp8_decode_step_with_prologue_matches_unfused_and_oracle(lens, kind, D, rd):
     """The FP8 cache (per-(sequence, head) scales calibrated on the history): hs_decode_step_fp8_prologue against
@@ -279,18 +284,20 @@ def test_fp8_decode_step_with_prologue_matches_unfused_and_oracle(lens, kind, D,
     assert err.max() < TOL_MAX and err.mean() < TOL_MEAN
 
 
-def test_decode_step_prologue_rejects_unserved_rotary_dim():
+@pytest.mark.parametrize("rd", [24, 136, 8])
+def test_decode_step_prologue_rejects_bad_rotary_dim(rd):
+    """The rotated length is a multiple of 16 within the head, as for hs_rope_apply_partial and hs_qk_prologue_apply."""
     B, Hq, Hkv, D, T = 1, 4, 1, 128, 64
     z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16, device=DEV)
-    sin = z(8, 48)
-    pro = hb.qk_prologue(hb.QKNORM_NONE, 0.0, None, None, sin, sin, 96)
+    sin = z(8, 128)
+    pro = hb.qk_prologue(hb.QKNORM_NONE, 0.0, None, None, sin, sin, rd)
     c = DeviceCache(B, Hkv, T, D)
     ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
     with pytest.raises(hb.HsError) as e:
         hb.decode_step_prologue(z(B, Hq, D), z(B, 1, Hkv, D), z(B, 1, Hkv, D), pro, c.k_codes, c.v_codes, c.k_scales,
                                 c.v_scales, c.layout, torch.ones(B, dtype=torch.int32, device=DEV), z(B, Hq, D), ws, Hkv,
                                 T, 0.1)
-    assert e.value.code == 1 and "hs_qk_prologue_apply" in str(e.value)
+    assert e.value.code == 1 and "rotary_dim" in str(e.value)
 
 
 @pytest.mark.parametrize("D", [64, 128, 256])
