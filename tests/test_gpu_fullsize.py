@@ -246,6 +246,69 @@ def test_config3_shape_with_fp8_history():
     assert np.array_equal(kc[2, 3].cpu().numpy(), wk)
 
 
+@pytest.mark.parametrize("B,copy,fp8", [(4, True, False), (4, True, True), (1, False, False), (1, True, False)])
+def test_config3_full_size_prompt_copy_and_single_sequence(B, copy, fp8):
+    """The launches the other prefill workloads time, at their size: 4096-token prompts in 512-token chunks with the
+    history read from the bf16 copy of the prompt (int8 and FP8 caches), and one sequence alone, where the library
+    splits the keys of a query tile over several workgroups (with the codes and with the copy).  Sampled query rows of
+    every part of the prompt against the oracle over [dequantized cache of earlier chunks | own bf16 K/V]; the cache
+    ends up as the oracle's codes; a second run gives the same bits (the merge order of the key runs is fixed)."""
+    T, C, Hq, Hkv, D = 4096, 512, 32, 8, 128
+    g = gen(wl.SEED + 11 + B + 2 * copy + 4 * fp8)
+    sg = 0.5 if fp8 else 1.0
+    q, k, v = source(g, (B, T, Hq, D)), source(g, (B, T, Hkv, D), sg), source(g, (B, T, Hkv, D), sg)
+    lay = hb.contiguous_layout(Hkv, T, D)
+    split_ws = hb.prefill_split_workspace(B, C, Hq, Hkv, D)
+
+    def run():
+        kc = torch.zeros(B, Hkv, T, D, dtype=torch.uint8 if fp8 else torch.int8, device=DEV)
+        vc = torch.zeros_like(kc)
+        ks = torch.zeros((B, Hkv) if fp8 else (B, Hkv, lay.scale_stride_head), dtype=torch.float32, device=DEV)
+        vs = torch.zeros_like(ks)
+        if fp8:
+            hb.kv_fp8_calibrate(k[:, :C].contiguous(), v[:, :C].contiguous(), ks, vs)
+        shadow = hb.prefill_shadow(B, Hkv, D, T) if copy else None
+        outs = []
+        for i in range(0, T, C):
+            o = torch.full((B, C, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+            hb.prefill_attn(q[:, i:i + C].contiguous(), k[:, i:i + C].contiguous(), v[:, i:i + C].contiguous(), kc, vc, ks, vs,
+                            lay, i, o, 1.0 / np.sqrt(D), True, fp8=fp8, columns=0, split_workspace=split_ws, shadow=shadow)
+            outs.append(o)
+        torch.cuda.synchronize()
+        return torch.cat(outs, 1), kc, vc, ks, vs
+
+    out, kc, vc, ks, vs = run()
+    assert torch.isfinite(out.float()).all()
+    again = run()[0]
+    assert torch.equal(out.view(torch.int16), again.view(torch.int16))
+    ksn, vsn = ks.cpu().numpy(), vs.cpu().numpy()
+    r = wl.philox(41 + B + copy)
+    for i in range(8):
+        b, h = int(r.integers(B)), int(r.integers(Hkv))
+        pos = C * i + int(r.integers(C))  # one row of every chunk: every history length and key-run count
+        c0 = pos // C * C
+        if fp8:
+            kh = oracle.dequant_fp8(kc[b, h, :c0].cpu().numpy()[None, :, None], ksn[b:b + 1, h:h + 1])[0, :, 0]
+            vh = oracle.dequant_fp8(vc[b, h, :c0].cpu().numpy()[None, :, None], vsn[b:b + 1, h:h + 1])[0, :, 0]
+        else:
+            kh = (kc[b, h, :c0].float() * ks[b, h, :c0, None]).cpu().numpy()
+            vh = (vc[b, h, :c0].float() * vs[b, h, :c0, None]).cpu().numpy()
+        kd = np.concatenate([kh, k[b, c0:pos + 1, h].float().cpu().numpy()])
+        vd = np.concatenate([vh, v[b, c0:pos + 1, h].float().cpu().numpy()])
+        qb = q[b, pos, 4 * h:4 * h + 4].float().cpu().numpy()[None]
+        want = oracle.decode_attn(qb, kd[None, :, None], vd[None, :, None], None, None, oracle.FMT_DENSE,
+                                  np.array([pos + 1], np.int32), 1.0 / np.sqrt(D))[0]
+        d = np.abs(out[b, pos, 4 * h:4 * h + 4].float().cpu().numpy() - want)
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, pos, d.max(), d.mean())
+    b, h = B - 1, Hkv - 3
+    if fp8:
+        wk = oracle.quant_fp8(k[b, :, h].float().cpu().numpy()[None, :, None], ksn[b:b + 1, h:h + 1])[0, :, 0]
+        assert np.array_equal(kc[b, h].cpu().numpy(), wk)
+    else:
+        wk, wks = oracle.quant_int8(k[b, :, h].float().cpu().numpy())
+        assert np.array_equal(kc[b, h].cpu().numpy(), wk) and np.array_equal(ks[b, h, :T].cpu().numpy(), wks)
+
+
 def test_config5_full_size_deltanet():
     """Decode at B = 64 (whole batch against the oracle) and prefill at B = 4 x 4096 (two sampled heads against
     the oracle, and chunked calls with carried state against the single call)."""
