@@ -239,7 +239,7 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         "data": "synthetic (seeded, generated on device)",
         "config": {"workload": "c3%s: chunked causal prefill B=%d T=4096 chunk=%d Hq=%d Hkv=%d D=%d, %s cache of earlier "
                                "chunks + own bf16 K/V, quantize-on-write, one layer"
-                               % ("-b1-shadow" if shadow and b1 else "-fp8-shadow" if shadow and fp8 else "-shadow" if shadow else "-prologue" if prologue else "-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
+                               % ("-b1-shadow" if shadow and b1 else "-fp8-shadow" if shadow and fp8 else "-prologue with the prompt copy" if shadow and prologue else "-shadow" if shadow else "-prologue" if prologue else "-d256" if d256 else "-d64" if d64 else "-b1" if b1 else "-fp8" if fp8 else "-prompt" if C == T else "", B, C, Hq, Hkv, D,
                                   "fp8 e4m3fn" if fp8 else "int8"),
                    "algorithmic_flops_per_step": int(flops)},
         "tokens_per_s": B * T / (ms * 1e-3),
@@ -438,6 +438,8 @@ def main():
                     help="prefill workloads: runs the keys of a query tile are cut into (0 = the library decides, 1 = never)")
     ap.add_argument("--prologue-fused-q", action="store_true",
                     help="c3-prologue: only k goes through the pre-pass, the chunk launches normalise and rotate q themselves")
+    ap.add_argument("--prompt-copy", action="store_true",
+                    help="c3 workloads: keep the bf16 copy of the prompt's K/V and read the history from it (what the -shadow workloads do)")
     ap.add_argument("--prologue-per-chunk", action="store_true",
                     help="c3-prologue: run the QK-norm + rotary pre-pass in front of every chunk call instead of once over the prompt")
     ap.add_argument("--chunk-tokens", type=int, default=0, choices=[0, 256, 512, 1024, 2048, 4096],
@@ -473,7 +475,7 @@ def main():
         return
     if args.workload.startswith("c3"):
         return bench_prefill(args, torch, hb, wl, C=args.chunk_tokens or (4096 if args.workload == "c3-prompt" else 512),
-                             fp8=args.workload.startswith("c3-fp8"), d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload.startswith("c3-b1"), prologue=args.workload == "c3-prologue", shadow=args.workload.endswith("-shadow"))
+                             fp8=args.workload.startswith("c3-fp8"), d256=args.workload == "c3-d256", d64=args.workload == "c3-d64", b1=args.workload.startswith("c3-b1"), prologue=args.workload == "c3-prologue", shadow=args.workload.endswith("-shadow") or args.prompt_copy)
     if args.workload.startswith("c5-decode-layer"):
         return bench_deltanet_layer(args, torch, hb, wl, fused=args.workload == "c5-decode-layer")
     if args.workload.startswith("c5"):
