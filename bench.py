@@ -235,7 +235,8 @@ def bench_prefill(args, torch, hb, wl, C=512, fp8=False, d256=False, d64=False, 
         "metric": "prefill-attn TFLOP/s (%% bf16 MFMA peak) + tokens/s, B=%d x 4096 in %d-chunks, Llama-3-8B shape" % (B, C),
         "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 MFMA (new tokens) + f16 MFMA over %s codes (history), f32 accumulate" % ("fp8" if fp8 else "int8"),
+        "dtype": ("bf16 MFMA (new tokens; history from the bf16 copy of the dequantized %s cache), f32 accumulate" if shadow else
+                  "bf16 MFMA (new tokens) + f16 MFMA over %s codes (history), f32 accumulate") % ("fp8" if fp8 else "int8"),
         "data": "synthetic (seeded, generated on device)",
         "config": {"workload": "c3%s: chunked causal prefill B=%d T=4096 chunk=%d Hq=%d Hkv=%d D=%d, %s cache of earlier "
                                "chunks + own bf16 K/V, quantize-on-write, one layer"
