@@ -1091,7 +1091,11 @@ constexpr int kMaxKeySplits = 8;
 static size_t split_tile_bytes(int D, bool narrow) {  // accumulator slots + one of softmax state + the staged q pieces
     return (size_t)512 * 16 * ((D == 64 ? 8 : 16) / (narrow ? 2 : 1) + 1 + (D == 64 ? 4 : 8) / (narrow ? 2 : 1));
 }
-static size_t split_counter_bytes(int64_t tiles) { return ((size_t)tiles * 4 + 255) / 256 * 256; }
+// The arrival counters sit in front of the partials in a region of fixed size: every call finds them in the same place
+// whatever its tile count and width, so the partials of one call can never land where another call keeps a counter
+// (counters are zero between launches -- the last arriver of a tile clears its own -- and nothing else may write there).
+constexpr int64_t kMaxSplitTiles = 4096;
+constexpr size_t kSplitCounterBytes = (size_t)kMaxSplitTiles * 4;
 
 __global__ void zero_words_kernel(uint32_t *p, size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1209,7 +1213,10 @@ static int launch_prefill(bool fp8, const void *q, const void *k_new, const void
             return fail(HS_ERR_INVALID_ARGUMENT, "prefill_key_splits %d not in [0, %d]", P, kMaxKeySplits);
         if (P > 1) {
             if (split_narrow) tiles = (int64_t)((S + q_per_wg / 2 - 1) / (q_per_wg / 2)) * grid.y * grid.z;
-            const size_t cnt_bytes = split_counter_bytes(tiles);
+            if (tiles > kMaxSplitTiles)
+                return fail(HS_ERR_INVALID_ARGUMENT, "prefill_key_splits: %lld query tiles, at most %lld can be split (a call of this size fills the chip without)",
+                            (long long)tiles, (long long)kMaxSplitTiles);
+            const size_t cnt_bytes = kSplitCounterBytes;
             const size_t need = cnt_bytes + (size_t)tiles * P * split_tile_bytes(D, split_narrow);
             if (layout->prefill_split_workspace_bytes < 0 || (size_t)layout->prefill_split_workspace_bytes < need)
                 return fail(HS_ERR_WORKSPACE, "prefill split workspace of %lld bytes, %zu needed",
@@ -1325,9 +1332,9 @@ size_t hs_prefill_attn_split_workspace_bytes(int32_t B, int32_t S, int32_t Hq, i
     const int q_per_wg = 16 * ((D == 256 ? 1 : 2) * hs::kPWaves / HG);
     const int64_t tiles = (int64_t)((S + q_per_wg - 1) / q_per_wg) * Hkv * ((G + HG - 1) / HG) * B;
     // full-width tiles, or (head_dim <= 128) twice as many half-width ones: whichever record layout is larger
-    const size_t wide = hs::split_counter_bytes(tiles) + (size_t)tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, false);
+    const size_t wide = hs::kSplitCounterBytes + (size_t)tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, false);
     const size_t half = D <= 128 && q_per_wg >= 32
-                            ? hs::split_counter_bytes(2 * tiles) + (size_t)2 * tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, true)
+                            ? hs::kSplitCounterBytes + (size_t)2 * tiles * hs::kMaxKeySplits * hs::split_tile_bytes(D, true)
                             : 0;
     return wide > half ? wide : half;
 }
@@ -1344,7 +1351,7 @@ int hs_prefill_shadow_init(void *shadow, size_t bytes, hs_stream_t stream) {
 int hs_prefill_attn_split_workspace_init(void *workspace, size_t bytes, hs_stream_t stream) {
     if (!workspace || ((uintptr_t)workspace & 255) != 0)
         return hs::fail(HS_ERR_INVALID_ARGUMENT, "prefill split workspace must be a 256-byte aligned device buffer");
-    // the arrival counters sit in front of the partials; their number depends on the call, so all of it is cleared
+    // the arrival counters sit in front of the partials; the whole buffer is cleared
     const size_t words = bytes / 4;
     if (words == 0) return HS_OK;
     hs::zero_words_kernel<<<dim3((unsigned)((words + 255) / 256)), 256, 0, (hipStream_t)stream>>>((uint32_t *)workspace, words);

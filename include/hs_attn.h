@@ -117,11 +117,14 @@ typedef struct hs_kv_layout {
                                    bytes, 256-byte aligned, prepared once by hs_prefill_attn_split_workspace_init and
                                    left ready by every call; calls that overlap in time need workspaces of their own.
                                    NULL = never split.  prefill_key_splits: 0 = the library decides whether and how
-                                   far to split, 1 = never, 2..8 = this many runs (tests, measurements).  A workspace
-                                   that is too small for the call is HS_ERR_WORKSPACE.  Outputs agree with the unsplit
-                                   launch within the rounding of a different summation order; the cache rows written
-                                   are the same bits.  Not combined with a window or a width hint of 128, 32 or 16
-                                   (those calls run unsplit). */
+                                   far to split, 1 = never, 2..8 = this many runs (tests, measurements; a call of
+                                   more than 4096 query tiles has no counters to be split with and is
+                                   HS_ERR_INVALID_ARGUMENT).  A workspace that is too small for the call is
+                                   HS_ERR_WORKSPACE.  The first 16 KB of the workspace hold the tiles' arrival
+                                   counters, zero between calls; calls of any shape and width may share a workspace
+                                   one after the other.  Outputs agree with the unsplit launch within the rounding of
+                                   a different summation order; the cache rows written are the same bits.  Not
+                                   combined with a window or a width hint of 32 or 16 (those calls run unsplit). */
     void *prefill_shadow;
     int64_t prefill_shadow_bytes;
     int32_t prefill_shadow_tokens;

@@ -652,6 +652,53 @@ def test_key_split_workspace_errors():
     assert e.value.code == 1
 
 
+def test_one_split_workspace_for_calls_of_every_width_and_size():
+    """Calls that split at full width, at half width (twice the tiles), with other run counts and for other lengths take
+    turns on ONE workspace: the arrival counters have a fixed place in it, so the partial results of one call never
+    land where a later call, with more tiles, looks for a counter (they did once, when the counter region was sized by
+    the call: all rows of the later call's second sequence stayed unwritten).  Over a history, so that every run of
+    every tile, the first included, holds numbers."""
+    _fixes_its_own_instance()
+    B, H, S, Hq, Hkv, D = 2, 256, 844, 32, 8, 128
+    q, k, v = make(77, B, H + S, Hq, Hkv)
+    ws = hb.prefill_split_workspace(B, S, Hq, Hkv, D)
+    dev = lambda x: torch.from_numpy(x).to(DEV).bfloat16().contiguous()
+    qd, kd, vd = dev(q), dev(k), dev(v)
+
+    def run(n, cols, runs):
+        c = DeviceCache(B, Hkv, H + S, D)
+        o0 = torch.empty(B, H, Hq, D, dtype=torch.bfloat16, device=DEV)
+        hb.prefill_attn(qd[:, :H].contiguous(), kd[:, :H].contiguous(), vd[:, :H].contiguous(), c.k_codes, c.v_codes, c.k_scales,
+                        c.v_scales, c.layout, 0, o0, 1.0 / np.sqrt(D), True, columns=256, key_splits=1)
+        out = torch.full((B, n, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+        hb.prefill_attn(qd[:, H:H + n].contiguous(), kd[:, H:H + n].contiguous(), vd[:, H:H + n].contiguous(), c.k_codes, c.v_codes,
+                        c.k_scales, c.v_scales, c.layout, H, out, 1.0 / np.sqrt(D), True, columns=cols, split_workspace=ws,
+                        key_splits=runs)
+        torch.cuda.synchronize()
+        return out.float().cpu().numpy()
+
+    want = run(S, 256, 1)
+    assert np.isfinite(want).all()
+    for n, cols, runs in ((S, 256, 2), (S, 128, 3), (300, 256, 8), (S, 128, 4), (S, 256, 3), (700, 128, 2), (S, 128, 2)):
+        got = run(n, cols, runs)
+        assert np.isfinite(got).all(), (n, cols, runs)
+        d = np.abs(got - want[:, :n])
+        assert d.max() < 2e-2 and d.mean() < 2e-3, (n, cols, runs, d.max())
+
+
+def test_key_split_refuses_more_tiles_than_it_has_counters_for():
+    _fixes_its_own_instance()
+    B, S, Hq, Hkv, D = 8, 2048, 32, 8, 128  # 64 x 8 x 8 = 4096 tiles of half width... and twice that below
+    q, k, v = (torch.zeros(B, 2 * S, H, D, dtype=torch.bfloat16, device=DEV) for H in (Hq, Hkv, Hkv))
+    c = DeviceCache(B, Hkv, 2 * S, D)
+    out = torch.empty_like(q)
+    ws = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+    with pytest.raises(hb.HsError) as e:
+        hb.prefill_attn(q, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, 0, out, 0.1, False,
+                        columns=128, split_workspace=ws, key_splits=2)
+    assert e.value.code == 1 and "4096" in str(e.value)
+
+
 @pytest.mark.parametrize("variant", ["full", "half", "split3", "split2-half"])
 @pytest.mark.parametrize("chunks", [(64, 64, 64), (100, 37, 200, 91), (512, 512), (1, 63, 64, 300)])
 @pytest.mark.parametrize("Hq,Hkv", [(8, 2), (6, 2), (4, 4)])
