@@ -309,6 +309,78 @@ def test_config3_full_size_prompt_copy_and_single_sequence(B, copy, fp8):
         assert np.array_equal(kc[b, h].cpu().numpy(), wk) and np.array_equal(ks[b, h, :T].cpu().numpy(), wks)
 
 
+def test_cache_tensors_beyond_2_gib():
+    """Maximum sizes: K and V code tensors of 2.5 GiB each (80 sequences x 32768 tokens x 8 heads x 128), where a 32-bit
+    element or byte offset wraps (the reference's `n as i32` counts do at this scale, kv_cache.rs:832).  The bulk
+    writer, decode attention, the fused decode step and a prefill chunk over the longest history, each checked against
+    the oracle on sequences whose offsets lie beyond 2^31; then the same codes read through a block table whose entries
+    point beyond 2^31 bytes into the pool."""
+    B, Hq, Hkv, D, T = 80, 32, 8, 128, 32768
+    assert B * Hkv * T * D > 2 ** 31
+    g = gen(wl.SEED + 21)
+    lay, kc, vc, ks, vs, kept = fill_cache(g, B, Hkv, T, D, False, 1.0, True, keep=(79,))
+    k79, _ = kept[79]
+    wk, wks = oracle.quant_int8(k79[:, :, 6])
+    assert np.array_equal(kc[79, 6].cpu().numpy(), wk[0]) and np.array_equal(ks[79, 6, :T].cpu().numpy(), wks[0])
+    q = torch.randn(B, Hq, D, generator=g, device=DEV).to(torch.bfloat16)
+    lens = torch.full((B,), T - 64, dtype=torch.int32, device=DEV)
+    lens[70] = 20001
+    out = decode(q, kc, vc, ks, vs, lay, lens, Hkv, T, False)
+    assert torch.isfinite(out.float()).all()
+    sample_check(out, q, kc, vc, ks, vs, lens.cpu().numpy(), [(0, 0), (70, 3), (79, 7)], 4, False)
+    decode_step_check(g, q, kc, vc, ks, vs, lay, lens, Hkv, T, False, 1.0, True, [(66, 1), (79, 6)])
+    # a 64-token chunk on top of T - 64 cached tokens, rows of the last sequences against the oracle
+    S, H = 64, T - 64
+    qn, kn, vn = source(g, (B, S, Hq, D)), source(g, (B, S, Hkv, D)), source(g, (B, S, Hkv, D))
+    lens.fill_(H)  # (the decode step above moved nothing: it rewrote position len - 1)
+    o = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(qn, kn, vn, kc, vc, ks, vs, lay, H, o, 1.0 / np.sqrt(D), True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all()
+    for b, h, pos in ((79, 7, 63), (72, 0, 5)):
+        kd = torch.cat([kc[b, h, :H].float() * ks[b, h, :H, None], kn[b, :pos + 1, h].float()]).cpu().numpy()
+        vd = torch.cat([vc[b, h, :H].float() * vs[b, h, :H, None], vn[b, :pos + 1, h].float()]).cpu().numpy()
+        qb = qn[b, pos, 4 * h:4 * h + 4].float().cpu().numpy()[None]
+        want = oracle.decode_attn(qb, kd[None, :, None], vd[None, :, None], None, None, oracle.FMT_DENSE,
+                                  np.array([H + pos + 1], np.int32), 1.0 / np.sqrt(D))[0]
+        d = np.abs(o[b, pos, 4 * h:4 * h + 4].float().cpu().numpy() - want)
+        assert d.max() < TOL_MAX and d.mean() < TOL_MEAN, (b, h, pos, d.max(), d.mean())
+    wkn, wksn = oracle.quant_int8(kn[79].float().cpu().numpy()[None])
+    assert np.array_equal(kc[79, :, H:].cpu().numpy(), wkn[0].transpose(1, 0, 2))
+    assert np.array_equal(ks[79, :, H:T].cpu().numpy(), wksn[0].transpose(1, 0))
+    # the same memory as a pool of 256-token blocks [B * T / 256 blocks, Hkv, 256, D]: sequence b's blocks are
+    # b * 128 .. b * 128 + 127 of a layout in which a block is one (sequence, 256-token) slab -- which the contiguous
+    # [B, Hkv, T, D] tensor is not, so the pool is filled from it for three sequences at the far end
+    BT, nblk = 256, T // 256
+    pool_k = torch.zeros(B * nblk, Hkv, BT, D, dtype=torch.int8, device=DEV)
+    pool_v = torch.zeros_like(pool_k)
+    pool_ks = torch.zeros(B * nblk, Hkv, BT, dtype=torch.float32, device=DEV)
+    pool_vs = torch.zeros_like(pool_ks)
+    tab = torch.zeros(B, nblk, dtype=torch.int32, device=DEV)
+    perm = torch.randperm(B * nblk, generator=g, device=DEV).to(torch.int32).view(B, nblk)
+    tab.copy_(perm)
+    far = [b for b in range(B) if int(perm[b].max()) * Hkv * BT * D > 2 ** 31][:3]
+    assert len(far) == 3
+    for b in far:
+        idx = perm[b].long()
+        pool_k[idx] = kc[b].view(Hkv, nblk, BT, D).permute(1, 0, 2, 3)
+        pool_v[idx] = vc[b].view(Hkv, nblk, BT, D).permute(1, 0, 2, 3)
+        pool_ks[idx] = ks[b, :, :T].reshape(Hkv, nblk, BT).permute(1, 0, 2)
+        pool_vs[idx] = vs[b, :, :T].reshape(Hkv, nblk, BT).permute(1, 0, 2)
+    play = hb.paged_layout(Hkv, BT, D, tab, tab)
+    plens = torch.zeros(B, dtype=torch.int32, device=DEV)
+    for b in far:
+        plens[b] = T
+    pout = torch.full((B, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(hb.decode_workspace_bytes(B, Hq, Hkv, D, T), dtype=torch.uint8, device=DEV)
+    hb.decode_attn(q, pool_k, pool_v, pool_ks, pool_vs, play, plens, pout, ws, Hkv, T, 1.0 / np.sqrt(D))
+    full = torch.full((B,), T, dtype=torch.int32, device=DEV)
+    cout = decode(q, kc, vc, ks, vs, lay, full, Hkv, T, False)
+    torch.cuda.synchronize()
+    for b in far:  # the same codes, the same chunking: the same bits
+        assert torch.equal(pout[b].view(torch.int16), cout[b].view(torch.int16)), b
+
+
 def test_config5_full_size_deltanet():
     """Decode at B = 64 (whole batch against the oracle) and prefill at B = 4 x 4096 (two sampled heads against
     the oracle, and chunked calls with carried state against the single call)."""
