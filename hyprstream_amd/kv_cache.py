@@ -88,16 +88,27 @@ class CacheError(RuntimeError):
         self.code = code
 
 
-class LayerKVCache:
+class _Handle:
+    """Owner of a C handle.  The destroy function is taken at construction and kept on the object: at interpreter exit
+    this module's globals, lib() among them, may already be gone when the last objects are collected."""
+    _h = None
+    _destroy = None
+
+    def close(self):
+        h, destroy = self._h, self._destroy
+        if h and destroy:
+            destroy(h)
+            self._h = None
+
+    __del__ = close
+
+
+class LayerKVCache(_Handle):
     def __init__(self, max_seq_len, quant_type=INT8):
+        self._destroy = lib().hs_cache_destroy
         self._h = ctypes.c_void_p(lib().hs_cache_create(max_seq_len, quant_type))
         if not self._h:
             raise ValueError("bad max_seq_len / quant_type")
-
-    def __del__(self):
-        if getattr(self, "_h", None):
-            lib().hs_cache_destroy(self._h)
-            self._h = None
 
     def _check(self, rc):
         if rc != hb.HS_OK:
@@ -198,19 +209,15 @@ class BlockPoolExhausted(CacheError):
     """Fail-soft: the pool has no free block; retry once other sequences have released theirs."""
 
 
-class BlockPool:
+class BlockPool(_Handle):
     """BlockPool of the reference (kv_cache.rs:508-676) over int8 blocks; bookkeeping works without a GPU."""
 
     def __init__(self, num_blocks, num_kv_heads, head_dim, quant_type=INT8):
+        self._destroy = lib().hs_pool_destroy
         self._h = ctypes.c_void_p(lib().hs_pool_create_format(num_blocks, num_kv_heads, head_dim, quant_type))
         if not self._h:
             raise ValueError("bad pool shape")
         self.num_kv_heads, self.head_dim = num_kv_heads, head_dim
-
-    def __del__(self):
-        if getattr(self, "_h", None):
-            lib().hs_pool_destroy(self._h)
-            self._h = None
 
     def _check(self, rc):
         if rc != hb.HS_OK:
@@ -252,22 +259,16 @@ class BlockPool:
         return lib().hs_pool_used_memory(self._h)
 
 
-class PagedLayerKVCache:
+class PagedLayerKVCache(_Handle):
     """LayerKVCache::new_paged (kv_cache.rs:1100-1120): one sequence, int8 blocks from a shared pool."""
 
     def __init__(self, max_seq_len, pool, owner):
         kind, ident, name = _owner(owner)
         self.pool = pool  # keeps the Python pool object alive as long as the cache
+        self._destroy = lib().hs_paged_cache_destroy
         self._h = ctypes.c_void_p(lib().hs_paged_cache_create(max_seq_len, pool._h, kind, ident, name))
         if not self._h:
             raise ValueError("bad max_seq_len / pool")
-
-    def close(self):
-        if getattr(self, "_h", None):
-            lib().hs_paged_cache_destroy(self._h)
-            self._h = None
-
-    __del__ = close
 
     def _check(self, rc):
         if rc != hb.HS_OK:
@@ -344,17 +345,13 @@ def f32_bits(x):
     return struct.unpack("<I", struct.pack("<f", x))[0]
 
 
-class KvCompatDescriptor:
+class KvCompatDescriptor(_Handle):
     """ctypes handle on hs_compat; fields are set by the names of the reference's struct."""
 
     def __init__(self, **fields):
+        self._destroy = lib().hs_compat_destroy
         self._h = ctypes.c_void_p(lib().hs_compat_create())
         self.set(**fields)
-
-    def __del__(self):
-        if getattr(self, "_h", None):
-            lib().hs_compat_destroy(self._h)
-            self._h = None
 
     def set(self, **fields):
         L = lib()
