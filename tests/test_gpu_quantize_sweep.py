@@ -85,3 +85,62 @@ def test_codes_and_scales_bit_exact(seed):
                 assert np.array_equal(gks[b, lo:lo + S].view(np.uint32), wsk[b].view(np.uint32)), (cfg, b)
                 assert np.array_equal(gvs[b, lo:lo + S].view(np.uint32), wsv[b].view(np.uint32)), (cfg, b)
                 assert (gks[b, untouched] == -1.0).all(), (cfg, b)
+
+
+@pytest.mark.parametrize("seed", [73])
+def test_dense_view_of_random_caches(seed):
+    """hs_kv_dequantize (LayerKVCache::get): random codes and scales -- every code value, scales over many decades, zero
+    scales -- in a contiguous cache or behind a shuffled block table, read back in bf16, fp16 or fp32 for a prefix of
+    the capacity: the oracle's dequantisation, rounded once to the view's dtype."""
+    rng = np.random.default_rng(seed)
+    for t in range(60):
+        D, Hkv, B = int(rng.choice([64, 128, 256])), int(rng.choice([1, 2, 3, 8])), int(rng.integers(1, 4))
+        cap = int(rng.choice([1, 7, 64, 100, 300, 700]))
+        T = int(rng.integers(1, cap + 1))
+        fp8, paged = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+        cfg = dict(seed=seed, t=t, D=D, Hkv=Hkv, B=B, cap=cap, T=T, fp8=fp8, paged=paged, dtype=str(dtype))
+        span = 4 if dtype == torch.float16 else 20  # (fp16 views of huge values would just be infinities)
+        if fp8:
+            codes = rng.integers(0, 256, (B, cap, Hkv, D)).astype(np.uint8)
+            codes[(codes & 0x7f) == 0x7f] = 0x7e  # e4m3fn's NaN patterns never come out of the quantizer
+            scales = (10.0 ** rng.uniform(-span, span - 3, (B, Hkv))).astype(np.float32)
+            want = oracle.dequant_fp8(codes, scales)
+        else:
+            codes = rng.integers(-127, 128, (B, cap, Hkv, D)).astype(np.int8)
+            scales = (10.0 ** rng.uniform(-span, span - 3, (B, cap, Hkv))).astype(np.float32)
+            scales[rng.random(scales.shape) < 0.05] = 0.0
+            want = oracle.dequant_int8(codes, scales)
+        BT = 256
+        nblk = (cap + BT - 1) // BT
+        ct = torch.from_numpy(codes).to(DEV)
+        if paged:
+            tab = torch.from_numpy(rng.permutation(B * nblk + 2).astype(np.int32)[:B * nblk].reshape(B, nblk)).to(DEV)
+            pool = torch.zeros(B * nblk + 2, Hkv, BT, D, dtype=ct.dtype, device=DEV)
+            padded = torch.zeros(B, nblk * BT, Hkv, D, dtype=ct.dtype, device=DEV)
+            padded[:, :cap] = ct
+            pool[tab.long()] = padded.view(B, nblk, BT, Hkv, D).permute(0, 1, 3, 2, 4)
+            lay = hb.paged_layout(Hkv, BT, D, tab, tab)
+            if fp8:
+                sc = torch.from_numpy(scales).to(DEV)
+            else:
+                sp = torch.zeros(B, nblk * BT, Hkv, device=DEV)
+                sp[:, :cap] = torch.from_numpy(scales).to(DEV)
+                sc = torch.zeros(B * nblk + 2, Hkv, BT, device=DEV)
+                sc[tab.long()] = sp.view(B, nblk, BT, Hkv).permute(0, 1, 3, 2)
+            store = pool
+        else:
+            lay = hb.contiguous_layout(Hkv, cap, D)
+            store = ct.permute(0, 2, 1, 3).contiguous()
+            if fp8:
+                sc = torch.from_numpy(scales).to(DEV)
+            else:
+                sc = torch.zeros(B, Hkv, lay.scale_stride_head, device=DEV)
+                sc[:, :, :cap] = torch.from_numpy(scales).to(DEV).permute(0, 2, 1)
+        out = torch.full((B, T, Hkv, D), float("nan"), dtype=dtype, device=DEV)
+        hb.kv_dequantize(store, sc, fp8, lay, 0, out)
+        torch.cuda.synchronize()
+        w = torch.from_numpy(want[:, :T]).to(dtype)
+        got = out.cpu()
+        same = (got == w) | (torch.isnan(got) & torch.isnan(w))
+        assert bool(same.all()), (cfg, int((~same).sum()))
