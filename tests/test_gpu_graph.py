@@ -73,6 +73,38 @@ def test_chunked_prefill_in_a_graph():
         assert bool(torch.equal(out, want)) and bool(torch.equal(c.k_codes, want_codes)), "replay %d" % i
 
 
+@pytest.mark.parametrize("cols,runs,copy", [(0, 3, False), (128, 2, True), (0, 0, True)])
+def test_split_and_copy_fed_prefill_in_a_graph(cols, runs, copy):
+    """The key split keeps state between launches (arrival counters that every launch leaves at zero) and the prompt
+    copy is appended to by every call: a captured chunk call replays to the same bits, three times, with eager work
+    and synchronisations in between."""
+    B, S, Hq, Hkv, D, H = 1, 192, 8, 2, 128, 320
+    r = wl.philox(1520 + cols + runs)
+    rnd = lambda *s: torch.from_numpy(r.standard_normal(s).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    c = DeviceCache(B, Hkv, H + S, D)
+    ws = hb.prefill_split_workspace(B, S, Hq, Hkv, D)
+    sh = hb.prefill_shadow(B, Hkv, D, H + S) if copy else None
+    o0 = torch.empty(B, H, Hq, D, dtype=torch.bfloat16, device=DEV)
+    hb.prefill_attn(rnd(B, H, Hq, D), rnd(B, H, Hkv, D), rnd(B, H, Hkv, D), c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, 0,
+                    o0, 0.0884, True, columns=256, key_splits=1, shadow=sh)  # the history (and its part of the copy)
+    q, k, v = rnd(B, S, Hq, D), rnd(B, S, Hkv, D), rnd(B, S, Hkv, D)
+    out = torch.empty(B, S, Hq, D, dtype=torch.bfloat16, device=DEV)
+    call = lambda: hb.prefill_attn(q, k, v, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout, H, out, 0.0884, True,
+                                   columns=cols, split_workspace=ws, key_splits=runs, shadow=sh)
+    call()
+    torch.cuda.synchronize()
+    want, want_codes = out.clone(), c.k_codes.clone()
+    g = _capture(call)
+    for i in range(3):
+        out.zero_()
+        c.k_codes[:, :, H:].zero_()
+        (q.float().reshape(S, -1) @ q.float().reshape(S, -1).T).sum().item()  # unrelated eager work between replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert bool(torch.equal(out, want)) and bool(torch.equal(c.k_codes, want_codes)), "replay %d" % i
+
+
 def test_chunked_deltanet_with_its_norm_in_a_graph():
     """hs_deltanet_forward_chunked_gated_norm is three ordinary launches (factor, walk, norm): recorded once, replayed
     with the state put back before every replay, it gives the eager bits each time."""
