@@ -173,3 +173,55 @@ def test_paged_caches_the_output_gate_and_the_q_prologue(seed):
             kcA = kcA[idx].permute(0, 2, 1, 3, 4).reshape(B, Hkv, idx.shape[1] * BT, D)
             vcA = vcA[idx].permute(0, 2, 1, 3, 4).reshape(B, Hkv, idx.shape[1] * BT, D)
         assert torch.equal(kcA[:, :, :T], R[0][:, :, :T]) and torch.equal(vcA[:, :, :T], R[1][:, :, :T]), cfg
+
+
+@pytest.mark.parametrize("seed", [16])
+def test_rows_at_different_positions_against_one_sequence_at_a_time(seed):
+    """hs_prefill_attn_*_ragged (the reference's forward_batched with q_len > 1): sequences with DIFFERENT numbers of
+    cached tokens take S new tokens in one call.  Against the same sequences one at a time (B = 1 calls at their own
+    history length, the form the other tests pin to the oracle): outputs within rounding, caches bit for bit."""
+    rng = np.random.default_rng(seed)
+    ws = hb.prefill_split_workspace(4, 300, 64, 8, 128)
+    for t in range(60):
+        D, Hkv, G = int(rng.choice([64, 128, 128, 256])), int(rng.choice([1, 2, 8])), int(rng.choice([1, 2, 4, 6]))
+        Hq, B = G * Hkv, int(rng.integers(2, 5))
+        S = int(rng.choice([1, 5, 64, 100, 257, 300]))
+        hist = [int(rng.choice([0, 0, 1, 63, 64, 200, 513])) for _ in range(B)]
+        fp8 = bool(rng.integers(0, 2))
+        cols, runs = int(rng.choice([0, 0, 256, 128])), int(rng.choice([0, 0, 1, 3]))
+        cap = max(hist) + S
+        cfg = dict(seed=seed, t=t, D=D, Hq=Hq, Hkv=Hkv, B=B, S=S, hist=hist, fp8=fp8, cols=cols, runs=runs)
+        g = torch.Generator(device=DEV)
+        g.manual_seed(5000 * seed + t)
+        sg = 0.5 if fp8 else 1.0
+        mk = lambda *s: (sg * torch.randn(*s, generator=g, device=DEV)).bfloat16()
+        a, r = DeviceCache(B, Hkv, cap, D, fp8=fp8), DeviceCache(B, Hkv, cap, D, fp8=fp8)
+        one = lambda c, b: (c.k_codes[b:b + 1], c.v_codes[b:b + 1], c.k_scales[b:b + 1], c.v_scales[b:b + 1])
+        if fp8:
+            kcal, vcal = mk(B, 64, Hkv, D), mk(B, 64, Hkv, D)
+            for c in (a, r):
+                hb.kv_fp8_calibrate(kcal, vcal, c.k_scales, c.v_scales)
+        for b in range(B):  # each sequence's own history, the same in both caches
+            if hist[b]:
+                kh, vh = mk(1, hist[b], Hkv, D), mk(1, hist[b], Hkv, D)
+                for c in (a, r):
+                    (hb.kv_quantize_fp8 if fp8 else hb.kv_quantize_int8)(kh, vh, *one(c, b), c.layout, None, 0)
+        q, k, v = torch.randn(B, S, Hq, D, generator=g, device=DEV).bfloat16(), mk(B, S, Hkv, D), mk(B, S, Hkv, D)
+        got = torch.full((B, S, Hq, D), float("nan"), dtype=torch.bfloat16, device=DEV)
+        want = torch.full_like(got, float("nan"))
+        hl = torch.tensor(hist, dtype=torch.int32, device=DEV)
+        hb.prefill_attn(q, k, v, a.k_codes, a.v_codes, a.k_scales, a.v_scales, a.layout, max(hist), got, 1 / np.sqrt(D), True, fp8=fp8,
+                        hist_lens=hl, columns=cols, split_workspace=ws, key_splits=runs)
+        for b in range(B):
+            hb.prefill_attn(q[b:b + 1], k[b:b + 1], v[b:b + 1], *one(r, b), r.layout, hist[b], want[b:b + 1], 1 / np.sqrt(D), True, fp8=fp8,
+                            columns=256, key_splits=1)
+        torch.cuda.synchronize()
+        x, y = got.float(), want.float()
+        assert bool(torch.isfinite(x).all()) and bool(torch.isfinite(y).all()), cfg
+        d = (x - y).abs()
+        assert float(d.max()) < TOL_MAX and float(d.mean()) < TOL_MEAN, (cfg, float(d.max()))
+        for b in range(B):
+            n = hist[b] + S
+            assert torch.equal(a.k_codes[b, :, :n], r.k_codes[b, :, :n]) and torch.equal(a.v_codes[b, :, :n], r.v_codes[b, :, :n]), (cfg, b)
+            if not fp8:
+                assert torch.equal(a.k_scales[b, :, :n], r.k_scales[b, :, :n]), (cfg, b)
