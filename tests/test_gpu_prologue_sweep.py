@@ -78,3 +78,56 @@ def test_prepass_against_the_oracle_and_fused_step_against_the_prepass(seed):
         assert torch.equal(out1.view(torch.int16), out2.view(torch.int16)), (cfg, fp8, T)
         assert torch.equal(c1.k_codes, c2.k_codes) and torch.equal(c1.v_codes, c2.v_codes), (cfg, fp8, T)
         assert torch.equal(c1.k_scales, c2.k_scales) and torch.equal(c1.v_scales, c2.v_scales), (cfg, fp8, T)
+
+
+@pytest.mark.parametrize("seed", [63])
+def test_cache_write_with_the_prologue_and_the_stand_alone_rotation(seed):
+    """hs_kv_quantize_int8_prologue (K normalised and rotated inside the cache write, any rotated length that is a
+    multiple of 16, rows placed by a scalar start or per-sequence positions): codes and scales of the oracle's
+    quantizer applied to the oracle's normalised, rotated K; V as plain.  hs_rope_apply_partial on its own: the
+    oracle's rotation bit for bit, the unrotated tail copied."""
+    import oracle
+    from oracle import hs_oracle as orc
+    rng = np.random.default_rng(seed)
+    tables = {}
+    for t in range(60):
+        D = int(rng.choice([64, 128, 256]))
+        rd = int(rng.choice(np.arange(16, D + 1, 16)))
+        kind = int(rng.choice([hb.QKNORM_NONE, hb.QKNORM_LLAMA, hb.QKNORM_QWEN35]))
+        Hkv, B, S, L = int(rng.choice([1, 2, 3, 8])), int(rng.integers(1, 4)), int(rng.choice([1, 2, 21, 64, 130])), 1024
+        by_position = bool(rng.integers(0, 2))
+        cfg = dict(seed=seed, t=t, D=D, rd=rd, kind=kind, Hkv=Hkv, B=B, S=S, by_position=by_position)
+        if rd not in tables:
+            tables[rd] = _tables(rd, 10000.0, L)
+        sin, cos = tables[rd]
+        k = _bf(rng.standard_normal((B, S, Hkv, D)) * 2)
+        v = _bf(rng.standard_normal((B, S, Hkv, D)))
+        wk = _weights(rng, kind, Hkv, D, bool(rng.integers(0, 2))) if kind else None
+        pro = hb.qk_prologue(kind, 1e-6, None, wk.to(DEV) if kind else None, sin.to(DEV), cos.to(DEV), rd)
+        cap = int(rng.integers(S, S + 200))
+        starts = rng.integers(0, cap - S + 1, B).astype(np.int32) if by_position else np.full(B, int(rng.integers(0, cap - S + 1)), np.int32)
+        c = DeviceCache(B, Hkv, cap, D)
+        hb.kv_quantize_int8_prologue(k.to(DEV), v.to(DEV), pro, c.k_codes, c.v_codes, c.k_scales, c.v_scales, c.layout,
+                                     torch.from_numpy(starts).to(DEV) if by_position else None, 0 if by_position else int(starts[0]))
+        torch.cuda.synchronize()
+        kc, vc, ks, vs = c.canonical(cap)
+        pos = (starts[:, None] + np.arange(S, dtype=np.int32)[None]).reshape(-1)
+        k_fin = oracle_prologue(_bits(k).reshape(B * S, Hkv, D), kind, wk, 1e-6, sin, cos, pos, rd).reshape(B, S, Hkv, D)
+        wkc, wks = oracle.quant_int8(oracle.bf16_to_f32(k_fin))
+        wvc, wvs = oracle.quant_int8(v.float().numpy())
+        for b in range(B):
+            lo = int(starts[b])
+            assert np.array_equal(kc[b, lo:lo + S], wkc[b]) and np.array_equal(ks[b, lo:lo + S].view(np.uint32), wks[b].view(np.uint32)), (cfg, b)
+            assert np.array_equal(vc[b, lo:lo + S], wvc[b]) and np.array_equal(vs[b, lo:lo + S].view(np.uint32), wvs[b].view(np.uint32)), (cfg, b)
+            rest = np.ones(cap, bool)
+            rest[lo:lo + S] = False
+            assert not kc[b, rest].any() and not vc[b, rest].any(), (cfg, b)
+        # the rotation alone
+        x = k.to(DEV)
+        out = torch.full_like(x, float("nan"))
+        hb.rope_apply(x, sin.to(DEV), cos.to(DEV), out, torch.from_numpy(starts).to(DEV) if by_position else None,
+                      0 if by_position else int(starts[0]), rotary_dim=rd)
+        torch.cuda.synchronize()
+        want = _bits(k).reshape(B * S, Hkv, D).copy()
+        want[..., :rd] = orc.rope_apply_bf16(np.ascontiguousarray(want[..., :rd]), _bits(sin), _bits(cos), pos)
+        assert np.array_equal(_bits(out).reshape(B * S, Hkv, D), want), cfg
